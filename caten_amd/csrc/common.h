@@ -1,0 +1,140 @@
+// Internal helpers shared by the translation units of libcaten_hip.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string>
+
+#include "../../include/caten_hip.h"
+
+namespace cthip {
+
+// ---- process-wide state (one device, one in-order stream) ----
+struct State {
+  bool inited = false;
+  int device = -1;
+  hipStream_t stream = nullptr;
+  int compute_units = 0;
+  hipEvent_t ev0 = nullptr, ev1 = nullptr;
+};
+State &state();
+void set_error(const char *fmt, ...);
+int fail(int code, const char *fmt, ...);
+
+#define CTHIP_REQUIRE_INIT()                                                         \
+  do {                                                                               \
+    if (!cthip::state().inited) return cthip::fail(CTHIP_E_NOT_INIT, "%s: cthip_init has not been called", __func__); \
+  } while (0)
+
+#define CTHIP_CHECK(expr)                                                            \
+  do {                                                                               \
+    hipError_t _e = (expr);                                                          \
+    if (_e != hipSuccess)                                                            \
+      return cthip::fail((int)_e, "%s: %s -> %s", __func__, #expr, hipGetErrorString(_e)); \
+  } while (0)
+
+#define CTHIP_ARG(cond)                                                              \
+  do {                                                                               \
+    if (!(cond)) return cthip::fail(CTHIP_E_BAD_ARG, "%s: bad argument: %s", __func__, #cond); \
+  } while (0)
+
+// checks the launch that was just queued
+#define CTHIP_LAUNCH_CHECK() CTHIP_CHECK(hipGetLastError())
+
+// ---- packed weight matrix ----
+struct WMat {
+  int type;         // CTHIP_F32 / F16 / Q4_0 / Q8_0
+  int64_t rows, cols;
+  void *q;          // quant plane: Q8_0 int8[rows][cols]; Q4_0 u8[rows][cols/2]; F32 float; F16 half
+  void *d;          // scale plane: fp16[rows][cols/32] (quantised types), else NULL
+  int64_t q_bytes, d_bytes;
+};
+
+// Arguments of one fused Linear launch:
+//   y = act(prologue(x) . W^T + bias) + residual
+// Output rows >= split1 / split2 are routed to y1 / y2 (fused-qkv rows going straight
+// into the K / V cache), offset by (pos[0] + m) * pos_stride floats.
+struct GemvArgs {
+  float *y;
+  float *y1;
+  float *y2;
+  const int *pos;
+  int pos_stride;
+  int split1, split2;
+  const void *q;
+  const unsigned short *d;
+  const float *x;
+  const float *bias;
+  const float *residual;
+  const float *norm_g;
+  const float *norm_b;
+  float eps;
+  int rows, cols;
+  int act, pro;
+  int64_t x_stride, y_stride;  // between the m input / output vectors (blockIdx.y)
+};
+int launch_gemv(const WMat *w, GemvArgs a, int m);
+int wmat_create_impl(WMat **out, int type, const void *raw, int64_t rows, int64_t cols);
+// true when a register-resident GEMV variant covers the matrix (no temporary is allocated at launch)
+bool gemv_is_direct(const WMat *w);
+int launch_attn(float *out, const float *q, const float *kc, const float *vc, int S, int start_pos, const int *pos,
+                int max_T, int H, int Hkv, int Dh);
+int launch_embedding(float *out, const float *W, const float *idx_f, const int *idx_i, int ntok, int vocab, int dim,
+                     const float *W2, const int *pos, int max_pos);
+int launch_argmax(int64_t *out, const float *x, int64_t rows, int n, int *tok_out, int *pos, int64_t *history,
+                  int *hist_n);
+int launch_rope_append(float *kc, float *vc, const float *kv, int Hkv, int Dh, float base, const int *pos);
+int launch_rope(float *out, const float *x, int B, int S, int H, int Dh, float base, int start_pos, const int *pos);
+
+}  // namespace cthip
+
+// ---- device helpers ----
+#if defined(__HIPCC__)
+namespace cthip {
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+// sum over aligned groups of G lanes (G = 16, 32, 64); every lane gets the group's sum
+template <int G>
+__device__ __forceinline__ float group_sum(float v) {
+#pragma unroll
+  for (int o = G / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+__device__ __forceinline__ float half_bits_to_float(unsigned short h) {
+  return (float)__builtin_bit_cast(_Float16, h);
+}
+
+// Caten's decompositions (api/function.lisp:437-440, nn/activations.lisp:3-7,202-215,
+// api/high-level-ops.lisp:112-117): exp(x) = exp2(x * 1/ln2); sigmoid = recip(1 + exp2(-x/ln2));
+// tanh(y) = 2*sigmoid(2y) - 1.
+__device__ __forceinline__ float ct_exp(float x) { return exp2f(x * 1.442695f); }
+__device__ __forceinline__ float ct_sigmoid(float x) { return 1.0f / (1.0f + exp2f(x * -1.442695f)); }
+__device__ __forceinline__ float ct_tanh(float y) { return 2.0f * ct_sigmoid(2.0f * y) - 1.0f; }
+__device__ __forceinline__ float ct_gelu(float x) {
+  return 0.5f * x * (1.0f + ct_tanh(0.7978846f * (x + 0.044715f * (x * x * x))));
+}
+__device__ __forceinline__ float ct_silu(float x) { return x * ct_sigmoid(x); }
+__device__ __forceinline__ float apply_act(int act, float v) {
+  switch (act) {
+    case CTHIP_ACT_RELU: return fmaxf(v, 0.0f);
+    case CTHIP_ACT_GELU: return ct_gelu(v);
+    case CTHIP_ACT_SILU: return ct_silu(v);
+    case CTHIP_ACT_SIGMOID: return ct_sigmoid(v);
+    case CTHIP_ACT_TANH: return ct_tanh(v);
+    default: return v;
+  }
+}
+
+}  // namespace cthip
+#endif

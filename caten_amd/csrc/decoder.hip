@@ -1,0 +1,552 @@
+// Decoder session: Caten's Transformer (external/llm/layers.lisp:73-90) and the
+// gpt2-generate loop (apps/gpt2/gpt2.lisp:97-113) as a device-resident pipeline.
+//
+// One decode step is a fixed sequence of fused launches whose only varying
+// inputs -- the current token and the position -- live in device memory, so the
+// sequence is captured ONCE as a hipGraph and replayed for every step without a
+// host round trip: the argmax kernel writes the next token where the embedding
+// kernel reads it and advances the position.  Per GPT-2 layer:
+//   1. LayerNorm1 -> c_attn GEMV -> +bias, q to a buffer, k/v rows straight into
+//      the KV cache at `pos` (the !assign of layers.lisp:30-31)
+//   2. attention of the one query row over cache rows 0..pos (causal mask implicit)
+//   3. c_proj GEMV + bias + residual
+//   4. LayerNorm2 -> c_fc GEMV + bias -> GELU
+//   5. mlp c_proj GEMV + bias + residual
+// then ln_f -> lm_head GEMV and the argmax.  Llama-shaped models (not in the
+// reference) use RMSNorm prologues, a fused wq|wk|wv matrix, a RoPE + cache-append
+// kernel, GQA attention and a fused gate|up matrix whose SwiGLU is the prologue of
+// the down projection.
+//
+// The reference pushes a whole prompt through one forward (s > 1).  Here a prompt is
+// fed row by row through the same step (causal attention makes that the same
+// function); only the last row runs lm_head and argmax.
+#include <stdlib.h>
+#include <string.h>
+
+#include <map>
+#include <string>
+#include <vector>
+
+#include "common.h"
+
+namespace cthip {
+
+struct RawTensor {
+  void *dev = nullptr;  // GGUF bytes on the device
+  int type = 0;
+  int64_t rows = 0, cols = 0;
+  size_t nbytes = 0;
+};
+
+static size_t raw_nbytes(int type, int64_t n) {
+  switch (type) {
+    case CTHIP_F32: return (size_t)n * 4;
+    case CTHIP_F16: return (size_t)n * 2;
+    case CTHIP_Q8_0: return (size_t)((n + 31) / 32) * 34;
+    case CTHIP_Q4_0: return (size_t)(n / 32) * 18;
+    default: return 0;
+  }
+}
+
+struct Layer {
+  // GPT-2
+  float *ln1_g = nullptr, *ln1_b = nullptr, *ln2_g = nullptr, *ln2_b = nullptr;
+  WMat *attn = nullptr, *proj = nullptr, *fc = nullptr, *fc2 = nullptr;
+  float *attn_b = nullptr, *proj_b = nullptr, *fc_b = nullptr, *fc2_b = nullptr;
+  // Llama: attn = wq|wk|wv, proj = wo, fc = gate|up, fc2 = down, ln1_g/ln2_g = rms weights
+  float *k_cache = nullptr, *v_cache = nullptr;
+};
+
+struct Decoder {
+  cthip_decoder_config cfg;
+  std::map<std::string, RawTensor> raw;
+  std::vector<std::string> required;
+  bool finalized = false;
+  std::vector<Layer> layers;
+  float *wte = nullptr, *wpe = nullptr, *lnf_g = nullptr, *lnf_b = nullptr;
+  WMat *lm_head = nullptr;
+  // activations
+  float *x = nullptr, *q = nullptr, *kv_tmp = nullptr, *att = nullptr, *h = nullptr, *logits = nullptr;
+  // device-resident loop state: [0] = current token, [1] = position
+  int *tokpos = nullptr;
+  int64_t *token64 = nullptr;
+  int64_t *history = nullptr;
+  int *hist_n = nullptr;
+  int position = 0;
+  bool primed = false;  // a forward has left token/position on the device
+  bool use_graph = true;
+  hipGraphExec_t g_step = nullptr, g_body = nullptr;
+  int64_t weight_bytes = 0, vector_bytes = 0;
+  std::vector<void *> owned;  // device blocks to free
+};
+
+static int kv_dim(const cthip_decoder_config &c) { return c.dim / c.n_heads * c.n_kv_heads; }
+
+static void build_required(Decoder *d) {
+  const cthip_decoder_config &c = d->cfg;
+  char buf[128];
+  if (c.arch == CTHIP_ARCH_GPT2) {
+    // state-dict keys after remap-key (apps/gpt2/gpt2.lisp:52-70)
+    d->required = {"wte.weight", "wpe.weight", "ln_f.affine", "ln_f.bias", "lm_head.weight"};
+    static const char *per[] = {"ln_1.affine", "ln_1.bias", "attn.c_attn.weight", "attn.c_attn.bias",
+                                "attn.c_proj.weight", "attn.c_proj.bias", "ln_2.affine", "ln_2.bias",
+                                "mlp.c_fc.weight", "mlp.c_fc.bias", "mlp.c_proj.weight", "mlp.c_proj.bias"};
+    for (int l = 0; l < c.n_layers; l++)
+      for (const char *p : per) {
+        snprintf(buf, sizeof(buf), "h.%d.%s", l, p);
+        d->required.push_back(buf);
+      }
+  } else {
+    d->required = {"tok_embeddings.weight", "norm.weight", "output.weight"};
+    static const char *per[] = {"attention_norm.weight", "attention.wq.weight", "attention.wk.weight",
+                                "attention.wv.weight", "attention.wo.weight", "ffn_norm.weight",
+                                "feed_forward.w1.weight", "feed_forward.w2.weight", "feed_forward.w3.weight"};
+    for (int l = 0; l < c.n_layers; l++)
+      for (const char *p : per) {
+        snprintf(buf, sizeof(buf), "layers.%d.%s", l, p);
+        d->required.push_back(buf);
+      }
+  }
+}
+
+static int dev_alloc(Decoder *d, void **p, size_t bytes) {
+  int rc = cthip_alloc(p, bytes);
+  if (rc == 0) d->owned.push_back(*p);
+  return rc;
+}
+
+// dequantise a raw tensor to an fp32 device vector owned by the session
+static int to_f32(Decoder *d, const std::string &key, int64_t want_n, float **out) {
+  auto it = d->raw.find(key);
+  if (it == d->raw.end()) return fail(CTHIP_E_STATE, "decoder: tensor '%s' was not loaded", key.c_str());
+  RawTensor &r = it->second;
+  const int64_t n = r.rows * r.cols;
+  if (n != want_n)
+    return fail(CTHIP_E_BAD_ARG, "decoder: tensor '%s' has %lld elements, expected %lld", key.c_str(), (long long)n,
+                (long long)want_n);
+  int rc = dev_alloc(d, (void **)out, sizeof(float) * (size_t)n);
+  if (rc) return rc;
+  rc = cthip_dequant(r.type, r.dev, n, *out);
+  if (rc) return rc;
+  d->vector_bytes += 4 * n;
+  return 0;
+}
+
+// pack one or more raw tensors (row-concatenated) into a weight matrix
+static int to_wmat(Decoder *d, const std::vector<std::string> &keys, int64_t want_rows, int64_t want_cols, WMat **out) {
+  std::vector<RawTensor *> parts;
+  int64_t rows = 0;
+  for (const std::string &k : keys) {
+    auto it = d->raw.find(k);
+    if (it == d->raw.end()) return fail(CTHIP_E_STATE, "decoder: tensor '%s' was not loaded", k.c_str());
+    parts.push_back(&it->second);
+    rows += it->second.rows;
+    if (it->second.cols != want_cols || it->second.type != parts[0]->type)
+      return fail(CTHIP_E_BAD_ARG, "decoder: tensor '%s' is (%lld,%lld) type %d; expected %lld columns of type %d",
+                  k.c_str(), (long long)it->second.rows, (long long)it->second.cols, it->second.type,
+                  (long long)want_cols, parts[0]->type);
+  }
+  if (rows != want_rows)
+    return fail(CTHIP_E_BAD_ARG, "decoder: '%s' (+%zu) has %lld rows, expected %lld", keys[0].c_str(), keys.size() - 1,
+                (long long)rows, (long long)want_rows);
+  int rc;
+  if (parts.size() == 1) {
+    rc = wmat_create_impl(out, parts[0]->type, parts[0]->dev, rows, want_cols);
+  } else {
+    size_t total = 0;
+    for (RawTensor *p : parts) total += p->nbytes;
+    void *cat = nullptr;
+    if ((rc = cthip_alloc(&cat, total))) return rc;
+    size_t off = 0;
+    for (RawTensor *p : parts) {
+      if ((rc = cthip_d2d((char *)cat + off, p->dev, p->nbytes))) return rc;
+      off += p->nbytes;
+    }
+    rc = wmat_create_impl(out, parts[0]->type, cat, rows, want_cols);
+    cthip_free(cat);
+  }
+  if (rc) return rc;
+  d->weight_bytes += (*out)->q_bytes + (*out)->d_bytes;
+  if (!gemv_is_direct(*out)) d->use_graph = false;
+  return 0;
+}
+
+static int queue_step(Decoder *d, bool with_head);
+
+static int finalize(Decoder *d) {
+  if (d->finalized) return 0;
+  const cthip_decoder_config &c = d->cfg;
+  for (const std::string &k : d->required)
+    if (!d->raw.count(k)) return fail(CTHIP_E_STATE, "decoder: tensor '%s' has not been loaded", k.c_str());
+  const int D = c.dim, F = c.ffn, V = c.vocab, KD = kv_dim(c);
+  int rc;
+  char b[128];
+  d->layers.resize(c.n_layers);
+  auto key = [&](int l, const char *s) {
+    snprintf(b, sizeof(b), c.arch == CTHIP_ARCH_GPT2 ? "h.%d.%s" : "layers.%d.%s", l, s);
+    return std::string(b);
+  };
+#define TRY(e) \
+  if ((rc = (e))) return rc
+  if (c.arch == CTHIP_ARCH_GPT2) {
+    TRY(to_f32(d, "wte.weight", (int64_t)V * D, &d->wte));
+    TRY(to_f32(d, "wpe.weight", (int64_t)c.max_seq * D, &d->wpe));
+    TRY(to_f32(d, "ln_f.affine", D, &d->lnf_g));
+    TRY(to_f32(d, "ln_f.bias", D, &d->lnf_b));
+    TRY(to_wmat(d, {"lm_head.weight"}, V, D, &d->lm_head));
+    for (int l = 0; l < c.n_layers; l++) {
+      Layer &L = d->layers[l];
+      TRY(to_f32(d, key(l, "ln_1.affine"), D, &L.ln1_g));
+      TRY(to_f32(d, key(l, "ln_1.bias"), D, &L.ln1_b));
+      TRY(to_wmat(d, {key(l, "attn.c_attn.weight")}, 3 * D, D, &L.attn));
+      TRY(to_f32(d, key(l, "attn.c_attn.bias"), 3 * D, &L.attn_b));
+      TRY(to_wmat(d, {key(l, "attn.c_proj.weight")}, D, D, &L.proj));
+      TRY(to_f32(d, key(l, "attn.c_proj.bias"), D, &L.proj_b));
+      TRY(to_f32(d, key(l, "ln_2.affine"), D, &L.ln2_g));
+      TRY(to_f32(d, key(l, "ln_2.bias"), D, &L.ln2_b));
+      TRY(to_wmat(d, {key(l, "mlp.c_fc.weight")}, F, D, &L.fc));
+      TRY(to_f32(d, key(l, "mlp.c_fc.bias"), F, &L.fc_b));
+      TRY(to_wmat(d, {key(l, "mlp.c_proj.weight")}, D, F, &L.fc2));
+      TRY(to_f32(d, key(l, "mlp.c_proj.bias"), D, &L.fc2_b));
+    }
+  } else {
+    TRY(to_f32(d, "tok_embeddings.weight", (int64_t)V * D, &d->wte));
+    TRY(to_f32(d, "norm.weight", D, &d->lnf_g));
+    TRY(to_wmat(d, {"output.weight"}, V, D, &d->lm_head));
+    for (int l = 0; l < c.n_layers; l++) {
+      Layer &L = d->layers[l];
+      TRY(to_f32(d, key(l, "attention_norm.weight"), D, &L.ln1_g));
+      TRY(to_wmat(d, {key(l, "attention.wq.weight"), key(l, "attention.wk.weight"), key(l, "attention.wv.weight")},
+                  D + 2 * KD, D, &L.attn));
+      TRY(to_wmat(d, {key(l, "attention.wo.weight")}, D, D, &L.proj));
+      TRY(to_f32(d, key(l, "ffn_norm.weight"), D, &L.ln2_g));
+      TRY(to_wmat(d, {key(l, "feed_forward.w1.weight"), key(l, "feed_forward.w3.weight")}, 2 * F, D, &L.fc));
+      TRY(to_wmat(d, {key(l, "feed_forward.w2.weight")}, D, F, &L.fc2));
+    }
+  }
+  // raw GGUF bytes are no longer needed
+  for (auto &kv : d->raw) cthip_free(kv.second.dev);
+  d->raw.clear();
+  // embeddings are read one row per step; norms/biases were counted in to_f32, remove the tables
+  d->vector_bytes -= 4 * (int64_t)V * D;
+  if (c.arch == CTHIP_ARCH_GPT2) d->vector_bytes -= 4 * (int64_t)c.max_seq * D;
+
+  for (int l = 0; l < c.n_layers; l++) {
+    // merge-kv-cache creates (B, max_len, H, Dh) zeros once (layers.lisp:25-26)
+    TRY(dev_alloc(d, (void **)&d->layers[l].k_cache, sizeof(float) * (size_t)c.max_seq * KD));
+    TRY(dev_alloc(d, (void **)&d->layers[l].v_cache, sizeof(float) * (size_t)c.max_seq * KD));
+  }
+  const int hdim = c.arch == CTHIP_ARCH_GPT2 ? F : 2 * F;
+  TRY(dev_alloc(d, (void **)&d->x, sizeof(float) * D));
+  TRY(dev_alloc(d, (void **)&d->q, sizeof(float) * D));
+  TRY(dev_alloc(d, (void **)&d->kv_tmp, sizeof(float) * 2 * KD));
+  TRY(dev_alloc(d, (void **)&d->att, sizeof(float) * D));
+  TRY(dev_alloc(d, (void **)&d->h, sizeof(float) * hdim));
+  TRY(dev_alloc(d, (void **)&d->logits, sizeof(float) * V));
+  TRY(dev_alloc(d, (void **)&d->tokpos, 256));
+  TRY(dev_alloc(d, (void **)&d->token64, 256));
+  TRY(dev_alloc(d, (void **)&d->history, sizeof(int64_t) * (size_t)(c.max_seq + 1)));
+  TRY(dev_alloc(d, (void **)&d->hist_n, 256));
+
+  const char *ng = getenv("CTHIP_NO_GRAPH");
+  if (ng && *ng && *ng != '0') d->use_graph = false;
+  if (d->use_graph) {
+    hipStream_t st = state().stream;
+    for (int pass = 0; pass < 2; pass++) {
+      hipGraph_t g = nullptr;
+      CTHIP_CHECK(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
+      rc = queue_step(d, pass == 0);
+      hipError_t e = hipStreamEndCapture(st, &g);
+      if (rc) {
+        if (g) (void)hipGraphDestroy(g);
+        return rc;
+      }
+      if (e != hipSuccess) return fail((int)e, "decoder: hipStreamEndCapture -> %s", hipGetErrorString(e));
+      hipGraphExec_t ex = nullptr;
+      e = hipGraphInstantiate(&ex, g, nullptr, nullptr, 0);
+      (void)hipGraphDestroy(g);
+      if (e != hipSuccess) return fail((int)e, "decoder: hipGraphInstantiate -> %s", hipGetErrorString(e));
+      (pass == 0 ? d->g_step : d->g_body) = ex;
+    }
+  }
+#undef TRY
+  d->finalized = true;
+  return 0;
+}
+
+// queues one decode step on the stream; token and position are read from d->tokpos
+static int queue_step(Decoder *d, bool with_head) {
+  const cthip_decoder_config &c = d->cfg;
+  const int D = c.dim, F = c.ffn, V = c.vocab, KD = kv_dim(c), Dh = c.dim / c.n_heads;
+  const int *tok = d->tokpos, *pos = d->tokpos + 1;
+  int rc;
+#define TRY(e) \
+  if ((rc = (e))) return rc
+  const bool gpt2 = c.arch == CTHIP_ARCH_GPT2;
+  TRY(launch_embedding(d->x, d->wte, nullptr, tok, 1, V, D, gpt2 ? d->wpe : nullptr, pos, c.max_seq));
+  for (int l = 0; l < c.n_layers; l++) {
+    Layer &L = d->layers[l];
+    GemvArgs a = {};
+    a.x = d->x;
+    a.pro = gpt2 ? CTHIP_PRO_LAYERNORM : CTHIP_PRO_RMSNORM;
+    a.norm_g = L.ln1_g;
+    a.norm_b = L.ln1_b;
+    a.eps = c.eps;
+    a.bias = L.attn_b;
+    a.y = d->q;
+    a.split1 = D;
+    a.split2 = D + KD;
+    a.x_stride = D;
+    a.y_stride = D;
+    if (gpt2) {
+      a.y1 = L.k_cache;
+      a.y2 = L.v_cache;
+      a.pos = pos;
+      a.pos_stride = KD;
+    } else {
+      a.y1 = d->kv_tmp;
+      a.y2 = d->kv_tmp + KD;
+      a.pos = nullptr;
+      a.pos_stride = 0;
+    }
+    TRY(launch_gemv(L.attn, a, 1));
+    if (!gpt2) {
+      // rotate q in place and k into the cache at `pos`; v is copied beside it
+      TRY(launch_rope(d->q, d->q, 1, 1, c.n_heads, Dh, c.rope_base, 0, pos));
+      TRY(launch_rope_append(L.k_cache, L.v_cache, d->kv_tmp, c.n_kv_heads, Dh, c.rope_base, pos));
+    }
+    TRY(launch_attn(d->att, d->q, L.k_cache, L.v_cache, 1, 0, pos, c.max_seq, c.n_heads, c.n_kv_heads, Dh));
+    GemvArgs p = {};
+    p.x = d->att;
+    p.bias = L.proj_b;
+    p.residual = d->x;
+    p.y = d->x;
+    p.x_stride = D;
+    p.y_stride = D;
+    TRY(launch_gemv(L.proj, p, 1));
+    GemvArgs f = {};
+    f.x = d->x;
+    f.pro = gpt2 ? CTHIP_PRO_LAYERNORM : CTHIP_PRO_RMSNORM;
+    f.norm_g = L.ln2_g;
+    f.norm_b = L.ln2_b;
+    f.eps = c.eps;
+    f.bias = L.fc_b;
+    f.act = gpt2 ? CTHIP_ACT_GELU : CTHIP_ACT_NONE;
+    f.y = d->h;
+    f.x_stride = D;
+    f.y_stride = gpt2 ? F : 2 * F;
+    TRY(launch_gemv(L.fc, f, 1));
+    GemvArgs g = {};
+    g.x = d->h;
+    g.pro = gpt2 ? CTHIP_PRO_NONE : CTHIP_PRO_SWIGLU;
+    g.bias = L.fc2_b;
+    g.residual = d->x;
+    g.y = d->x;
+    g.x_stride = gpt2 ? F : 2 * F;
+    g.y_stride = D;
+    TRY(launch_gemv(L.fc2, g, 1));
+  }
+  if (with_head) {
+    GemvArgs o = {};
+    o.x = d->x;
+    o.pro = gpt2 ? CTHIP_PRO_LAYERNORM : CTHIP_PRO_RMSNORM;
+    o.norm_g = d->lnf_g;
+    o.norm_b = d->lnf_b;
+    o.eps = c.eps;
+    o.y = d->logits;
+    o.x_stride = D;
+    o.y_stride = V;
+    TRY(launch_gemv(d->lm_head, o, 1));
+    // greedy token -> next step's input; position advances (apps/gpt2/gpt2.lisp:105-107)
+    TRY(launch_argmax(d->token64, d->logits, 1, V, d->tokpos, d->tokpos + 1, d->history, d->hist_n));
+  }
+#undef TRY
+  return 0;
+}
+
+static int run_step(Decoder *d, bool with_head) {
+  if (d->use_graph) {
+    CTHIP_CHECK(hipGraphLaunch(with_head ? d->g_step : d->g_body, state().stream));
+    return 0;
+  }
+  return queue_step(d, with_head);
+}
+
+}  // namespace cthip
+
+using namespace cthip;
+
+extern "C" {
+
+int cthip_decoder_create(void **dec, const cthip_decoder_config *cfg) {
+  CTHIP_REQUIRE_INIT();
+  CTHIP_ARG(dec != nullptr && cfg != nullptr);
+  const cthip_decoder_config &c = *cfg;
+  CTHIP_ARG(c.arch == CTHIP_ARCH_GPT2 || c.arch == CTHIP_ARCH_LLAMA);
+  CTHIP_ARG(c.n_layers > 0 && c.dim > 0 && c.n_heads > 0 && c.ffn > 0 && c.vocab > 0 && c.max_seq > 0);
+  CTHIP_ARG(c.dim % c.n_heads == 0);
+  CTHIP_ARG(c.n_kv_heads > 0 && c.n_heads % c.n_kv_heads == 0);
+  if (c.arch == CTHIP_ARCH_GPT2 && c.n_kv_heads != c.n_heads)
+    return fail(CTHIP_E_BAD_ARG, "cthip_decoder_create: the GPT-2 shaped Transformer has n_kv_heads == n_heads");
+  const int Dh = c.dim / c.n_heads;
+  if (Dh != 32 && Dh != 64 && Dh != 128)
+    return fail(CTHIP_E_UNSUPPORTED, "cthip_decoder_create: head_dim %d (supported: 32, 64, 128)", Dh);
+  if (c.max_seq > 8192) return fail(CTHIP_E_UNSUPPORTED, "cthip_decoder_create: max_seq %d > 8192", c.max_seq);
+  Decoder *d = new Decoder();
+  d->cfg = c;
+  build_required(d);
+  *dec = d;
+  return 0;
+}
+
+int cthip_decoder_destroy(void *dec) {
+  if (!dec) return 0;
+  Decoder *d = (Decoder *)dec;
+  if (state().inited) (void)hipStreamSynchronize(state().stream);
+  if (d->g_step) (void)hipGraphExecDestroy(d->g_step);
+  if (d->g_body) (void)hipGraphExecDestroy(d->g_body);
+  for (auto &kv : d->raw) cthip_free(kv.second.dev);
+  for (void *p : d->owned) cthip_free(p);
+  for (Layer &L : d->layers) {
+    cthip_wmat_destroy(L.attn);
+    cthip_wmat_destroy(L.proj);
+    cthip_wmat_destroy(L.fc);
+    cthip_wmat_destroy(L.fc2);
+  }
+  cthip_wmat_destroy(d->lm_head);
+  delete d;
+  return 0;
+}
+
+int cthip_decoder_load(void *dec, const char *key, int ggml_type, const void *host_raw, int64_t rows, int64_t cols) {
+  CTHIP_REQUIRE_INIT();
+  CTHIP_ARG(dec != nullptr && key != nullptr && host_raw != nullptr && rows > 0 && cols > 0);
+  Decoder *d = (Decoder *)dec;
+  if (d->finalized) return fail(CTHIP_E_STATE, "cthip_decoder_load: the session has already run; weights are frozen");
+  bool known = false;
+  for (const std::string &k : d->required)
+    if (k == key) known = true;
+  if (!known) return fail(CTHIP_E_BAD_ARG, "cthip_decoder_load: '%s' is not a tensor of this model", key);
+  const size_t nbytes = raw_nbytes(ggml_type, rows * cols);
+  if (nbytes == 0) return fail(CTHIP_E_UNSUPPORTED, "cthip_decoder_load: ggml type %d is not supported", ggml_type);
+  if ((ggml_type == CTHIP_Q8_0 || ggml_type == CTHIP_Q4_0) && cols % 32)
+    return fail(CTHIP_E_BAD_ARG, "cthip_decoder_load: '%s': quantised rows need cols %% 32 == 0", key);
+  RawTensor r;
+  r.type = ggml_type;
+  r.rows = rows;
+  r.cols = cols;
+  r.nbytes = nbytes;
+  int rc = cthip_alloc(&r.dev, nbytes);
+  if (rc) return rc;
+  rc = cthip_h2d(r.dev, host_raw, nbytes);
+  if (rc) {
+    cthip_free(r.dev);
+    return rc;
+  }
+  auto it = d->raw.find(key);
+  if (it != d->raw.end()) cthip_free(it->second.dev);
+  d->raw[key] = r;
+  return 0;
+}
+
+int cthip_decoder_missing(const void *dec) {
+  const Decoder *d = (const Decoder *)dec;
+  if (!d) return -1;
+  if (d->finalized) return 0;
+  int n = 0;
+  for (const std::string &k : d->required)
+    if (!d->raw.count(k)) n++;
+  return n;
+}
+
+int cthip_decoder_forward(void *dec, const float *tokens, int s, int n, int64_t *token, float *logits_out) {
+  CTHIP_REQUIRE_INIT();
+  CTHIP_ARG(dec != nullptr && tokens != nullptr && token != nullptr);
+  Decoder *d = (Decoder *)dec;
+  const cthip_decoder_config &c = d->cfg;
+  if (s < 1) return fail(CTHIP_E_BAD_ARG, "cthip_decoder_forward: s = %d; a forward needs at least one token", s);
+  if (n < 0 || n + s > c.max_seq)
+    return fail(CTHIP_E_BAD_ARG, "cthip_decoder_forward: positions %d..%d fall outside the KV cache (max_seq %d)", n,
+                n + s - 1, c.max_seq);
+  int rc = finalize(d);
+  if (rc) return rc;
+  int zero = 0;
+  if ((rc = cthip_h2d(d->hist_n, &zero, sizeof(int)))) return rc;
+  for (int i = 0; i < s; i++) {
+    // ids arrive as floats (gpt2.lisp:95); one that equals no vocabulary index selects no row
+    const float tf = tokens[i];
+    int id = (tf >= 0.0f && tf < (float)c.vocab && (float)(int)tf == tf) ? (int)tf : -1;
+    int tp[2] = {id, n + i};
+    if ((rc = cthip_h2d(d->tokpos, tp, sizeof(tp)))) return rc;
+    if ((rc = run_step(d, i == s - 1))) return rc;
+  }
+  if (logits_out && (rc = cthip_d2h(logits_out, d->logits, sizeof(float) * (size_t)c.vocab))) return rc;
+  if ((rc = cthip_d2h(token, d->token64, sizeof(int64_t)))) return rc;
+  d->position = n + s;
+  d->primed = true;
+  return 0;
+}
+
+int cthip_decoder_generate(void *dec, int steps, int64_t *tokens_out) {
+  CTHIP_REQUIRE_INIT();
+  CTHIP_ARG(dec != nullptr && steps >= 0 && (steps == 0 || tokens_out != nullptr));
+  Decoder *d = (Decoder *)dec;
+  if (!d->primed)
+    return fail(CTHIP_E_STATE, "cthip_decoder_generate: run cthip_decoder_forward on a prompt first");
+  if (d->position + steps > d->cfg.max_seq)
+    return fail(CTHIP_E_BAD_ARG, "cthip_decoder_generate: %d more tokens from position %d overflow max_seq %d", steps,
+                d->position, d->cfg.max_seq);
+  if (steps == 0) return 0;
+  int rc, zero = 0;
+  if ((rc = cthip_h2d(d->hist_n, &zero, sizeof(int)))) return rc;
+  for (int i = 0; i < steps; i++)
+    if ((rc = run_step(d, true))) return rc;
+  if ((rc = cthip_d2h(tokens_out, d->history, sizeof(int64_t) * (size_t)steps))) return rc;
+  d->position += steps;
+  return 0;
+}
+
+int cthip_decoder_position(const void *dec) { return dec ? ((const Decoder *)dec)->position : -1; }
+
+int64_t cthip_decoder_step_bytes(const void *dec, int t) {
+  const Decoder *d = (const Decoder *)dec;
+  if (!d || !d->finalized) return -1;
+  const cthip_decoder_config &c = d->cfg;
+  const int64_t KD = kv_dim(c);
+  int64_t emb = 4LL * c.dim * (c.arch == CTHIP_ARCH_GPT2 ? 2 : 1);
+  int64_t kv_read = 2LL * c.n_layers * t * KD * 4;
+  int64_t kv_write = 2LL * c.n_layers * KD * 4;
+  return d->weight_bytes + d->vector_bytes + emb + kv_read + kv_write;
+}
+
+int cthip_decoder_peek(void *dec, const char *what, void **ptr, int64_t *n_floats) {
+  CTHIP_REQUIRE_INIT();
+  CTHIP_ARG(dec != nullptr && what != nullptr && ptr != nullptr);
+  Decoder *d = (Decoder *)dec;
+  int rc = finalize(d);
+  if (rc) return rc;
+  const cthip_decoder_config &c = d->cfg;
+  int64_t n = 0;
+  void *p = nullptr;
+  int l = -1;
+  if (!strcmp(what, "logits")) {
+    p = d->logits;
+    n = c.vocab;
+  } else if (!strcmp(what, "x")) {
+    p = d->x;
+    n = c.dim;
+  } else if (sscanf(what, "k_cache.%d", &l) == 1 && l >= 0 && l < c.n_layers) {
+    p = d->layers[l].k_cache;
+    n = (int64_t)c.max_seq * kv_dim(c);
+  } else if (sscanf(what, "v_cache.%d", &l) == 1 && l >= 0 && l < c.n_layers) {
+    p = d->layers[l].v_cache;
+    n = (int64_t)c.max_seq * kv_dim(c);
+  } else {
+    return fail(CTHIP_E_BAD_ARG, "cthip_decoder_peek: unknown buffer '%s'", what);
+  }
+  *ptr = p;
+  if (n_floats) *n_floats = n;
+  return 0;
+}
+
+}  // extern "C"

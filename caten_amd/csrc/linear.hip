@@ -1,0 +1,659 @@
+// GGUF block codecs, the packed weight matrix, and the dequant-in-register
+// GEMV that carries batch-1 decode (Linear, source/nn/linear.lisp:3-17, with
+// the LayerNorm/RMSNorm/SwiGLU prologue and bias/activation/residual epilogue
+// that Caten's scheduler fuses around a matmul, test-scheduler.lisp:140-163).
+//
+// HBM layout of a packed matrix (rows x cols):
+//   quant plane  Q8_0: int8  [rows][cols]      Q4_0: u8 [rows][cols/2]
+//                F32 : float [rows][cols]      F16 : half [rows][cols]
+//   scale plane  fp16 [rows][cols/32]          (quantised types only)
+// Q4_0 keeps ggml's nibble order inside each 16-byte block (low nibbles are
+// elements 0..15, high nibbles 16..31).  Total bytes equal the GGUF bytes, but
+// every lane can issue aligned 128-bit loads, which the 34/18-byte GGUF blocks
+// do not allow.
+//
+// GEMV work distribution: a row is owned by an aligned group of G lanes
+// (G = 16, 32 or 64; 64/G rows per wavefront), lane l of the group streams the
+// 16-byte chunks l, l+G, l+2G, ... (KC of them) of the row.  The slice of the
+// input vector that multiplies those chunks is loaded ONCE per wavefront into
+// registers (after applying the fused prologue) and reused for every row the
+// wavefront visits, so the steady state touches nothing but weights.  Partial
+// sums are combined with DPP/shuffle steps inside the group and the group's
+// first lane applies the epilogue.
+#include "common.h"
+
+namespace cthip {
+
+// ------------------------------------------------------------------ codecs
+__global__ void k_dequant_q8_0_raw(const uint8_t *__restrict__ raw, int64_t n, float *__restrict__ out) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  int64_t b = i >> 5;
+  int j = (int)(i & 31);
+  const uint8_t *p = raw + 34 * b;
+  float scale = half_bits_to_float((unsigned short)(p[0] | (p[1] << 8)));
+  out[i] = (float)(int8_t)p[2 + j] * scale;
+}
+
+__global__ void k_dequant_q4_0_raw(const uint8_t *__restrict__ raw, int64_t n, float *__restrict__ out) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  int64_t b = i >> 5;
+  int j = (int)(i & 31);
+  const uint8_t *p = raw + 18 * b;
+  float d = half_bits_to_float((unsigned short)(p[0] | (p[1] << 8)));
+  int byte = p[2 + (j & 15)];
+  int nib = (j < 16) ? (byte & 0x0f) : (byte >> 4);
+  out[i] = (float)(nib - 8) * d;
+}
+
+__global__ void k_dequant_f16_raw(const uint8_t *__restrict__ raw, int64_t n, float *__restrict__ out) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  out[i] = half_bits_to_float((unsigned short)(raw[2 * i] | (raw[2 * i + 1] << 8)));
+}
+
+__global__ void k_dequant_f32_raw(const uint8_t *__restrict__ raw, int64_t n, float *__restrict__ out) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  uint32_t u = (uint32_t)raw[4 * i] | ((uint32_t)raw[4 * i + 1] << 8) | ((uint32_t)raw[4 * i + 2] << 16) |
+               ((uint32_t)raw[4 * i + 3] << 24);
+  out[i] = __uint_as_float(u);
+}
+
+// GGUF blocks -> planes. One thread per block.
+__global__ void k_repack_q8_0(const uint8_t *__restrict__ raw, int64_t nblocks, uint32_t *__restrict__ q,
+                              unsigned short *__restrict__ d) {
+  int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (b >= nblocks) return;
+  const uint8_t *p = raw + 34 * b;
+  d[b] = (unsigned short)(p[0] | (p[1] << 8));
+#pragma unroll
+  for (int t = 0; t < 8; t++) {
+    const uint8_t *s = p + 2 + 4 * t;
+    q[8 * b + t] = (uint32_t)s[0] | ((uint32_t)s[1] << 8) | ((uint32_t)s[2] << 16) | ((uint32_t)s[3] << 24);
+  }
+}
+
+__global__ void k_repack_q4_0(const uint8_t *__restrict__ raw, int64_t nblocks, uint32_t *__restrict__ q,
+                              unsigned short *__restrict__ d) {
+  int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (b >= nblocks) return;
+  const uint8_t *p = raw + 18 * b;
+  d[b] = (unsigned short)(p[0] | (p[1] << 8));
+#pragma unroll
+  for (int t = 0; t < 4; t++) {
+    const uint8_t *s = p + 2 + 4 * t;
+    q[4 * b + t] = (uint32_t)s[0] | ((uint32_t)s[1] << 8) | ((uint32_t)s[2] << 16) | ((uint32_t)s[3] << 24);
+  }
+}
+
+// planes -> fp32, one thread per element
+__global__ void k_wmat_dequant(int type, const void *__restrict__ qp, const unsigned short *__restrict__ dp,
+                               int64_t n, float *__restrict__ out) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  if (type == CTHIP_Q8_0) {
+    out[i] = (float)((const int8_t *)qp)[i] * half_bits_to_float(dp[i >> 5]);
+  } else if (type == CTHIP_Q4_0) {
+    int64_t b = i >> 5;
+    int j = (int)(i & 31);
+    int byte = ((const uint8_t *)qp)[16 * b + (j & 15)];
+    int nib = (j < 16) ? (byte & 0x0f) : (byte >> 4);
+    out[i] = (float)(nib - 8) * half_bits_to_float(dp[b]);
+  } else if (type == CTHIP_F16) {
+    out[i] = half_bits_to_float(((const unsigned short *)qp)[i]);
+  } else {
+    out[i] = ((const float *)qp)[i];
+  }
+}
+
+// ------------------------------------------------------------------ GEMV
+template <int TYPE>
+struct Fmt;
+template <>
+struct Fmt<CTHIP_Q8_0> {
+  static constexpr int XPC = 16;  // input elements multiplied by one 16-byte chunk
+};
+template <>
+struct Fmt<CTHIP_Q4_0> {
+  static constexpr int XPC = 32;
+};
+template <>
+struct Fmt<CTHIP_F32> {
+  static constexpr int XPC = 4;
+};
+template <>
+struct Fmt<CTHIP_F16> {
+  static constexpr int XPC = 8;
+};
+
+template <int TYPE>
+__device__ __forceinline__ float chunk_dot(const uint4 w, float scale, const float *__restrict__ x, float xsum);
+
+template <>
+__device__ __forceinline__ float chunk_dot<CTHIP_Q8_0>(const uint4 w, float scale, const float *__restrict__ x, float) {
+  const uint32_t dw[4] = {w.x, w.y, w.z, w.w};
+  float s = 0.0f;
+#pragma unroll
+  for (int t = 0; t < 4; t++) {
+    int v = (int)dw[t];
+    s = fmaf((float)(int)(int8_t)(v), x[4 * t + 0], s);
+    s = fmaf((float)(int)(int8_t)(v >> 8), x[4 * t + 1], s);
+    s = fmaf((float)(int)(int8_t)(v >> 16), x[4 * t + 2], s);
+    s = fmaf((float)(v >> 24), x[4 * t + 3], s);
+  }
+  return s * scale;
+}
+
+template <>
+__device__ __forceinline__ float chunk_dot<CTHIP_Q4_0>(const uint4 w, float scale, const float *__restrict__ x, float xsum) {
+  const uint32_t dw[4] = {w.x, w.y, w.z, w.w};
+  float s = 0.0f;
+#pragma unroll
+  for (int t = 0; t < 4; t++) {
+    uint32_t lo = dw[t] & 0x0f0f0f0fu;
+    uint32_t hi = (dw[t] >> 4) & 0x0f0f0f0fu;
+    s = fmaf((float)(lo & 0xff), x[4 * t + 0], s);
+    s = fmaf((float)((lo >> 8) & 0xff), x[4 * t + 1], s);
+    s = fmaf((float)((lo >> 16) & 0xff), x[4 * t + 2], s);
+    s = fmaf((float)(lo >> 24), x[4 * t + 3], s);
+    s = fmaf((float)(hi & 0xff), x[16 + 4 * t + 0], s);
+    s = fmaf((float)((hi >> 8) & 0xff), x[16 + 4 * t + 1], s);
+    s = fmaf((float)((hi >> 16) & 0xff), x[16 + 4 * t + 2], s);
+    s = fmaf((float)(hi >> 24), x[16 + 4 * t + 3], s);
+  }
+  // sum (n-8) x = sum n x - 8 sum x
+  return (s - 8.0f * xsum) * scale;
+}
+
+template <>
+__device__ __forceinline__ float chunk_dot<CTHIP_F32>(const uint4 w, float, const float *__restrict__ x, float) {
+  float s = __uint_as_float(w.x) * x[0];
+  s = fmaf(__uint_as_float(w.y), x[1], s);
+  s = fmaf(__uint_as_float(w.z), x[2], s);
+  s = fmaf(__uint_as_float(w.w), x[3], s);
+  return s;
+}
+
+template <>
+__device__ __forceinline__ float chunk_dot<CTHIP_F16>(const uint4 w, float, const float *__restrict__ x, float) {
+  const uint32_t dw[4] = {w.x, w.y, w.z, w.w};
+  float s = 0.0f;
+#pragma unroll
+  for (int t = 0; t < 4; t++) {
+    s = fmaf(half_bits_to_float((unsigned short)(dw[t] & 0xffff)), x[2 * t], s);
+    s = fmaf(half_bits_to_float((unsigned short)(dw[t] >> 16)), x[2 * t + 1], s);
+  }
+  return s;
+}
+
+template <int TYPE, int G, int KC>
+__global__ __launch_bounds__(256) void k_gemv(GemvArgs a) {
+  constexpr int XPC = Fmt<TYPE>::XPC;
+  constexpr int RPW = 64 / G;  // rows per wavefront per iteration
+  constexpr bool QUANT = (TYPE == CTHIP_Q8_0 || TYPE == CTHIP_Q4_0);
+  const int lane = threadIdx.x & 63;
+  const int g = lane / G, l = lane % G;
+  const int waves_per_block = blockDim.x >> 6;
+  const int wave = blockIdx.x * waves_per_block + (threadIdx.x >> 6);
+  const int total_waves = gridDim.x * waves_per_block;
+  const int nchunks = a.cols / XPC;
+  const int m = blockIdx.y;
+  const float *__restrict__ x = a.x + (int64_t)m * a.x_stride;
+
+  // ---- input slice -> registers, with the fused prologue ----
+  float xr[KC][XPC];
+  float xs[KC];
+#pragma unroll
+  for (int j = 0; j < KC; j++) {
+    const int c = l + G * j;
+    const bool ok = c < nchunks;
+#pragma unroll
+    for (int t = 0; t < XPC / 4; t++) {
+      float4 v = ok ? *(const float4 *)(x + (int64_t)c * XPC + 4 * t) : make_float4(0.f, 0.f, 0.f, 0.f);
+      if (a.pro == CTHIP_PRO_SWIGLU && ok) {
+        float4 u = *(const float4 *)(x + a.cols + (int64_t)c * XPC + 4 * t);
+        v.x = ct_silu(v.x) * u.x;
+        v.y = ct_silu(v.y) * u.y;
+        v.z = ct_silu(v.z) * u.z;
+        v.w = ct_silu(v.w) * u.w;
+      }
+      xr[j][4 * t + 0] = v.x;
+      xr[j][4 * t + 1] = v.y;
+      xr[j][4 * t + 2] = v.z;
+      xr[j][4 * t + 3] = v.w;
+    }
+  }
+  if (a.pro == CTHIP_PRO_LAYERNORM || a.pro == CTHIP_PRO_RMSNORM) {
+    const float inv_n = 1.0f / (float)a.cols;
+    float mean = 0.0f;
+    if (a.pro == CTHIP_PRO_LAYERNORM) {
+      float s = 0.0f;
+#pragma unroll
+      for (int j = 0; j < KC; j++)
+#pragma unroll
+        for (int e = 0; e < XPC; e++) s += xr[j][e];
+      mean = group_sum<G>(s) * inv_n;
+    }
+    float v = 0.0f;
+#pragma unroll
+    for (int j = 0; j < KC; j++) {
+      const bool ok = (l + G * j) < nchunks;
+#pragma unroll
+      for (int e = 0; e < XPC; e++) {
+        float dlt = ok ? xr[j][e] - mean : 0.0f;
+        xr[j][e] = dlt;
+        v = fmaf(dlt, dlt, v);
+      }
+    }
+    const float rstd = 1.0f / sqrtf(group_sum<G>(v) * inv_n + a.eps);
+#pragma unroll
+    for (int j = 0; j < KC; j++) {
+      const int c = l + G * j;
+      if (c < nchunks) {
+#pragma unroll
+        for (int t = 0; t < XPC / 4; t++) {
+          float4 gm = a.norm_g ? *(const float4 *)(a.norm_g + (int64_t)c * XPC + 4 * t) : make_float4(1.f, 1.f, 1.f, 1.f);
+          float4 bt = a.norm_b ? *(const float4 *)(a.norm_b + (int64_t)c * XPC + 4 * t) : make_float4(0.f, 0.f, 0.f, 0.f);
+          xr[j][4 * t + 0] = xr[j][4 * t + 0] * rstd * gm.x + bt.x;
+          xr[j][4 * t + 1] = xr[j][4 * t + 1] * rstd * gm.y + bt.y;
+          xr[j][4 * t + 2] = xr[j][4 * t + 2] * rstd * gm.z + bt.z;
+          xr[j][4 * t + 3] = xr[j][4 * t + 3] * rstd * gm.w + bt.w;
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < KC; j++) {
+    float s = 0.0f;
+    if (TYPE == CTHIP_Q4_0) {
+#pragma unroll
+      for (int e = 0; e < XPC; e++) s += xr[j][e];
+    }
+    xs[j] = s;
+  }
+
+  // ---- stream the rows ----
+  const uint4 *__restrict__ qp = (const uint4 *)a.q;
+  const int64_t row_chunks = nchunks;            // 16-byte chunks per row in the quant plane
+  const int scales_per_row = a.cols >> 5;
+  const int nrq = (a.rows + RPW - 1) / RPW;
+
+  uint4 wc[KC];
+  unsigned short sc[KC];
+  auto load = [&](int rq, uint4 *w, unsigned short *s) {
+    const int row = rq * RPW + g;
+    const bool rok = row < a.rows;
+#pragma unroll
+    for (int j = 0; j < KC; j++) {
+      const int c = l + G * j;
+      const bool ok = rok && c < nchunks;
+      w[j] = ok ? qp[(int64_t)row * row_chunks + c] : make_uint4(0u, 0u, 0u, 0u);
+      if (QUANT) {
+        const int sidx = (TYPE == CTHIP_Q8_0) ? (c >> 1) : c;
+        s[j] = ok ? a.d[(int64_t)row * scales_per_row + sidx] : (unsigned short)0;
+      }
+    }
+  };
+
+  int rq = wave;
+  if (rq < nrq) load(rq, wc, sc);
+  while (rq < nrq) {
+    const int rqn = rq + total_waves;
+    uint4 wn[KC];
+    unsigned short sn[KC];
+    if (rqn < nrq) load(rqn, wn, sn);
+    float acc = 0.0f;
+#pragma unroll
+    for (int j = 0; j < KC; j++) {
+      const float scale = QUANT ? half_bits_to_float(sc[j]) : 1.0f;
+      acc += chunk_dot<TYPE>(wc[j], scale, xr[j], xs[j]);
+    }
+    acc = group_sum<G>(acc);
+    const int row = rq * RPW + g;
+    if (l == 0 && row < a.rows) {
+      float v = acc;
+      if (a.bias) v += a.bias[row];
+      v = apply_act(a.act, v);
+      if (a.residual) v += a.residual[(int64_t)m * a.y_stride + row];
+      float *dst;
+      if (row < a.split1) {
+        dst = a.y + (int64_t)m * a.y_stride + row;
+      } else {
+        const int64_t off = (int64_t)(a.pos ? a.pos[0] + m : m) * a.pos_stride;
+        dst = (row < a.split2) ? a.y1 + off + (row - a.split1) : a.y2 + off + (row - a.split2);
+      }
+      *dst = v;
+    }
+    if (rqn < nrq) {
+#pragma unroll
+      for (int j = 0; j < KC; j++) {
+        wc[j] = wn[j];
+        sc[j] = sn[j];
+      }
+    }
+    rq = rqn;
+  }
+}
+
+// Fallback for shapes no (G,KC) instantiation covers: one wavefront per row, the
+// input vector re-read through the cache hierarchy. `x` must already carry the prologue.
+template <int TYPE>
+__global__ __launch_bounds__(256) void k_gemv_generic(GemvArgs a) {
+  constexpr int XPC = Fmt<TYPE>::XPC;
+  constexpr bool QUANT = (TYPE == CTHIP_Q8_0 || TYPE == CTHIP_Q4_0);
+  const int lane = threadIdx.x & 63;
+  const int wave = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int total_waves = gridDim.x * (blockDim.x >> 6);
+  const int nchunks = a.cols / XPC;
+  const int m = blockIdx.y;
+  const float *__restrict__ x = a.x + (int64_t)m * a.x_stride;
+  const uint4 *__restrict__ qp = (const uint4 *)a.q;
+  for (int row = wave; row < a.rows; row += total_waves) {
+    float acc = 0.0f;
+    for (int c = lane; c < nchunks; c += 64) {
+      uint4 w = qp[(int64_t)row * nchunks + c];
+      float xl[XPC];
+      float xsum = 0.0f;
+#pragma unroll
+      for (int e = 0; e < XPC; e++) {
+        xl[e] = x[(int64_t)c * XPC + e];
+        xsum += xl[e];
+      }
+      float scale = 1.0f;
+      if (QUANT) {
+        const int sidx = (TYPE == CTHIP_Q8_0) ? (c >> 1) : c;
+        scale = half_bits_to_float(a.d[(int64_t)row * (a.cols >> 5) + sidx]);
+      }
+      acc += chunk_dot<TYPE>(w, scale, xl, xsum);
+    }
+    acc = wave_sum(acc);
+    if (lane == 0) {
+      float v = acc;
+      if (a.bias) v += a.bias[row];
+      v = apply_act(a.act, v);
+      if (a.residual) v += a.residual[(int64_t)m * a.y_stride + row];
+      float *dst;
+      if (row < a.split1) {
+        dst = a.y + (int64_t)m * a.y_stride + row;
+      } else {
+        const int64_t off = (int64_t)(a.pos ? a.pos[0] + m : m) * a.pos_stride;
+        dst = (row < a.split2) ? a.y1 + off + (row - a.split1) : a.y2 + off + (row - a.split2);
+      }
+      *dst = v;
+    }
+  }
+}
+
+// prologue as a kernel of its own, for the generic fallback: one block per input vector
+__global__ __launch_bounds__(256) void k_prologue(float *__restrict__ out, const float *__restrict__ x, int cols,
+                                                  int pro, const float *__restrict__ g,
+                                                  const float *__restrict__ b, float eps, int64_t x_stride) {
+  __shared__ float red[4];
+  const float *xi = x + (int64_t)blockIdx.x * x_stride;
+  float *o = out + (int64_t)blockIdx.x * cols;
+  const int tid = threadIdx.x;
+  auto block_sum = [&](float v) {
+    v = wave_sum(v);
+    __syncthreads();
+    if ((tid & 63) == 0) red[tid >> 6] = v;
+    __syncthreads();
+    return red[0] + red[1] + red[2] + red[3];
+  };
+  if (pro == CTHIP_PRO_SWIGLU) {
+    for (int i = tid; i < cols; i += 256) o[i] = ct_silu(xi[i]) * xi[cols + i];
+    return;
+  }
+  float mean = 0.0f;
+  if (pro == CTHIP_PRO_LAYERNORM) {
+    float s = 0.0f;
+    for (int i = tid; i < cols; i += 256) s += xi[i];
+    mean = block_sum(s) / (float)cols;
+  }
+  float v = 0.0f;
+  for (int i = tid; i < cols; i += 256) {
+    float dlt = xi[i] - mean;
+    v = fmaf(dlt, dlt, v);
+  }
+  const float rstd = 1.0f / sqrtf(block_sum(v) / (float)cols + eps);
+  for (int i = tid; i < cols; i += 256) {
+    float t = (xi[i] - mean) * rstd;
+    if (g) t *= g[i];
+    if (b) t += b[i];
+    o[i] = t;
+  }
+}
+
+// ------------------------------------------------------------------ dispatch
+typedef void (*gemv_fn)(GemvArgs);
+struct GemvVariant {
+  int type, G, KC;
+  gemv_fn fn;
+};
+#define V(T, G, KC) {T, G, KC, k_gemv<T, G, KC>}
+static const GemvVariant kVariants[] = {
+    V(CTHIP_Q8_0, 16, 1), V(CTHIP_Q8_0, 16, 2), V(CTHIP_Q8_0, 16, 3), V(CTHIP_Q8_0, 16, 4),
+    V(CTHIP_Q8_0, 32, 3), V(CTHIP_Q8_0, 32, 4), V(CTHIP_Q8_0, 64, 3), V(CTHIP_Q8_0, 64, 4),
+    V(CTHIP_Q8_0, 64, 6), V(CTHIP_Q8_0, 64, 8),
+    V(CTHIP_Q4_0, 16, 1), V(CTHIP_Q4_0, 16, 2), V(CTHIP_Q4_0, 32, 2), V(CTHIP_Q4_0, 64, 1),
+    V(CTHIP_Q4_0, 64, 2), V(CTHIP_Q4_0, 64, 3), V(CTHIP_Q4_0, 64, 4),
+    V(CTHIP_F32, 16, 4), V(CTHIP_F32, 64, 1), V(CTHIP_F32, 64, 2), V(CTHIP_F32, 64, 3), V(CTHIP_F32, 64, 4),
+    V(CTHIP_F32, 64, 6), V(CTHIP_F32, 64, 8), V(CTHIP_F32, 64, 12), V(CTHIP_F32, 64, 16), V(CTHIP_F32, 64, 24),
+    V(CTHIP_F16, 16, 2), V(CTHIP_F16, 64, 1), V(CTHIP_F16, 64, 2), V(CTHIP_F16, 64, 3), V(CTHIP_F16, 64, 4),
+    V(CTHIP_F16, 64, 6), V(CTHIP_F16, 64, 8), V(CTHIP_F16, 64, 12),
+};
+#undef V
+
+static int xpc_of(int type) {
+  switch (type) {
+    case CTHIP_Q8_0: return 16;
+    case CTHIP_Q4_0: return 32;
+    case CTHIP_F16: return 8;
+    default: return 4;
+  }
+}
+
+static const GemvVariant *pick_variant(int type, int cols) {
+  const int xpc = xpc_of(type);
+  if (cols % xpc) return nullptr;
+  const int nchunks = cols / xpc;
+  const GemvVariant *best = nullptr;
+  int best_waste = 1 << 30;
+  for (const GemvVariant &v : kVariants) {
+    if (v.type != type || v.G * v.KC < nchunks) continue;
+    int waste = v.G * v.KC - nchunks;
+    if (waste < best_waste || (waste == best_waste && best && v.G < best->G)) {
+      best = &v;
+      best_waste = waste;
+    }
+  }
+  return best;
+}
+
+bool gemv_is_direct(const WMat *w) { return pick_variant(w->type, (int)w->cols) != nullptr; }
+
+// Queues one fused Linear on the stream. Used by cthip_linear and by the decoder.
+int launch_gemv(const WMat *w, GemvArgs a, int m) {
+  State &s = state();
+  a.q = w->q;
+  a.d = (const unsigned short *)w->d;
+  a.rows = (int)w->rows;
+  a.cols = (int)w->cols;
+  if (a.split1 <= 0) a.split1 = a.split2 = a.rows;
+  const GemvVariant *v = pick_variant(w->type, a.cols);
+  if (v) {
+    const int rpw = 64 / v->G;
+    const int nrq = (a.rows + rpw - 1) / rpw;
+    dim3 grid, block;
+    if (nrq <= 2048) {
+      block = dim3(64);
+      grid = dim3(nrq, m);
+    } else {
+      block = dim3(256);
+      int blocks = (nrq + 3) / 4;
+      int cap = s.compute_units * 4;
+      grid = dim3(blocks < cap ? blocks : cap, m);
+    }
+    hipLaunchKernelGGL(v->fn, grid, block, 0, s.stream, a);
+    CTHIP_LAUNCH_CHECK();
+    return 0;
+  }
+  // generic path: prologue into a temporary, then wave-per-row
+  float *tmp = nullptr;
+  if (a.pro != CTHIP_PRO_NONE) {
+    int rc = cthip_alloc((void **)&tmp, sizeof(float) * (size_t)a.cols * m);
+    if (rc) return rc;
+    hipLaunchKernelGGL(k_prologue, dim3(m), dim3(256), 0, s.stream, tmp, a.x, a.cols, a.pro, a.norm_g, a.norm_b, a.eps,
+                       a.x_stride);
+    CTHIP_LAUNCH_CHECK();
+    a.x = tmp;
+    a.x_stride = a.cols;
+    a.pro = CTHIP_PRO_NONE;
+  }
+  int blocks = (a.rows + 3) / 4;
+  int cap = s.compute_units * 8;
+  dim3 grid(blocks < cap ? blocks : cap, m), block(256);
+  switch (w->type) {
+    case CTHIP_Q8_0: hipLaunchKernelGGL(k_gemv_generic<CTHIP_Q8_0>, grid, block, 0, s.stream, a); break;
+    case CTHIP_Q4_0: hipLaunchKernelGGL(k_gemv_generic<CTHIP_Q4_0>, grid, block, 0, s.stream, a); break;
+    case CTHIP_F16: hipLaunchKernelGGL(k_gemv_generic<CTHIP_F16>, grid, block, 0, s.stream, a); break;
+    default: hipLaunchKernelGGL(k_gemv_generic<CTHIP_F32>, grid, block, 0, s.stream, a); break;
+  }
+  CTHIP_LAUNCH_CHECK();
+  if (tmp) return cthip_free(tmp);
+  return 0;
+}
+
+int wmat_create_impl(WMat **out, int type, const void *raw, int64_t rows, int64_t cols) {
+  State &s = state();
+  WMat *w = new WMat();
+  w->type = type;
+  w->rows = rows;
+  w->cols = cols;
+  w->q = w->d = nullptr;
+  const int64_t n = rows * cols;
+  int rc = 0;
+  if (type == CTHIP_Q8_0 || type == CTHIP_Q4_0) {
+    const int64_t nblocks = n / 32;
+    w->q_bytes = (type == CTHIP_Q8_0) ? n : n / 2;
+    w->d_bytes = nblocks * 2;
+    if ((rc = cthip_alloc(&w->q, (size_t)w->q_bytes)) || (rc = cthip_alloc(&w->d, (size_t)w->d_bytes))) {
+      cthip_free(w->q);
+      delete w;
+      return rc;
+    }
+    unsigned blocks = (unsigned)((nblocks + 255) / 256);
+    if (type == CTHIP_Q8_0)
+      hipLaunchKernelGGL(k_repack_q8_0, dim3(blocks), dim3(256), 0, s.stream, (const uint8_t *)raw, nblocks,
+                         (uint32_t *)w->q, (unsigned short *)w->d);
+    else
+      hipLaunchKernelGGL(k_repack_q4_0, dim3(blocks), dim3(256), 0, s.stream, (const uint8_t *)raw, nblocks,
+                         (uint32_t *)w->q, (unsigned short *)w->d);
+    CTHIP_LAUNCH_CHECK();
+  } else {
+    w->q_bytes = n * (type == CTHIP_F32 ? 4 : 2);
+    w->d_bytes = 0;
+    if ((rc = cthip_alloc(&w->q, (size_t)w->q_bytes))) {
+      delete w;
+      return rc;
+    }
+    CTHIP_CHECK(hipMemcpyAsync(w->q, raw, (size_t)w->q_bytes, hipMemcpyDeviceToDevice, s.stream));
+  }
+  *out = w;
+  return 0;
+}
+
+}  // namespace cthip
+
+using namespace cthip;
+
+extern "C" {
+
+int cthip_dequant(int ggml_type, const void *raw, int64_t n, float *out) {
+  CTHIP_REQUIRE_INIT();
+  if (n == 0) return 0;
+  CTHIP_ARG(raw != nullptr && out != nullptr && n > 0);
+  dim3 grid((unsigned)((n + 255) / 256)), block(256);
+  hipStream_t st = state().stream;
+  switch (ggml_type) {
+    case CTHIP_Q8_0: hipLaunchKernelGGL(k_dequant_q8_0_raw, grid, block, 0, st, (const uint8_t *)raw, n, out); break;
+    case CTHIP_Q4_0:
+      if (n % 32) return fail(CTHIP_E_BAD_ARG, "cthip_dequant: Q4_0 needs n %% 32 == 0, got %lld", (long long)n);
+      hipLaunchKernelGGL(k_dequant_q4_0_raw, grid, block, 0, st, (const uint8_t *)raw, n, out);
+      break;
+    case CTHIP_F16: hipLaunchKernelGGL(k_dequant_f16_raw, grid, block, 0, st, (const uint8_t *)raw, n, out); break;
+    case CTHIP_F32: hipLaunchKernelGGL(k_dequant_f32_raw, grid, block, 0, st, (const uint8_t *)raw, n, out); break;
+    default:
+      // tensor-info.lisp:36-41 signals "Not ready" for every other ggml type
+      return fail(CTHIP_E_UNSUPPORTED, "cthip_dequant: ggml type %d is not supported", ggml_type);
+  }
+  CTHIP_LAUNCH_CHECK();
+  return 0;
+}
+
+int cthip_wmat_create(void **wmat, int ggml_type, const void *raw, int64_t rows, int64_t cols) {
+  CTHIP_REQUIRE_INIT();
+  CTHIP_ARG(wmat != nullptr && raw != nullptr && rows > 0 && cols > 0);
+  if (ggml_type != CTHIP_Q8_0 && ggml_type != CTHIP_Q4_0 && ggml_type != CTHIP_F32 && ggml_type != CTHIP_F16)
+    return fail(CTHIP_E_UNSUPPORTED, "cthip_wmat_create: ggml type %d is not supported", ggml_type);
+  if ((ggml_type == CTHIP_Q8_0 || ggml_type == CTHIP_Q4_0) && cols % 32)
+    return fail(CTHIP_E_BAD_ARG, "cthip_wmat_create: quantised rows need cols %% 32 == 0, got %lld", (long long)cols);
+  if (rows > 0x7fffffff || cols > 0x7fffffff) return fail(CTHIP_E_BAD_ARG, "cthip_wmat_create: dimension too large");
+  WMat *w = nullptr;
+  int rc = wmat_create_impl(&w, ggml_type, raw, rows, cols);
+  if (rc) return rc;
+  *wmat = w;
+  return 0;
+}
+
+int cthip_wmat_destroy(void *wmat) {
+  if (!wmat) return 0;
+  WMat *w = (WMat *)wmat;
+  cthip_free(w->q);
+  cthip_free(w->d);
+  delete w;
+  return 0;
+}
+
+int64_t cthip_wmat_nbytes(const void *wmat) {
+  const WMat *w = (const WMat *)wmat;
+  return w ? w->q_bytes + w->d_bytes : 0;
+}
+
+int cthip_wmat_dequant(const void *wmat, float *out) {
+  CTHIP_REQUIRE_INIT();
+  CTHIP_ARG(wmat != nullptr && out != nullptr);
+  const WMat *w = (const WMat *)wmat;
+  const int64_t n = w->rows * w->cols;
+  hipLaunchKernelGGL(k_wmat_dequant, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, state().stream, w->type, w->q,
+                     (const unsigned short *)w->d, n, out);
+  CTHIP_LAUNCH_CHECK();
+  return 0;
+}
+
+int cthip_linear(float *y, const void *wmat, const float *x, int m, const float *bias, const float *residual,
+                 int act, int prologue, const float *norm_g, const float *norm_b, float eps) {
+  CTHIP_REQUIRE_INIT();
+  CTHIP_ARG(y != nullptr && wmat != nullptr && x != nullptr && m >= 0);
+  CTHIP_ARG(prologue >= CTHIP_PRO_NONE && prologue <= CTHIP_PRO_SWIGLU);
+  CTHIP_ARG(act >= CTHIP_ACT_NONE && act <= CTHIP_ACT_TANH);
+  if (m == 0) return 0;
+  if (m > 65535) return fail(CTHIP_E_BAD_ARG, "cthip_linear: m = %d exceeds 65535", m);
+  const WMat *w = (const WMat *)wmat;
+  GemvArgs a = {};
+  a.y = y;
+  a.x = x;
+  a.bias = bias;
+  a.residual = residual;
+  a.act = act;
+  a.pro = prologue;
+  a.norm_g = norm_g;
+  a.norm_b = norm_b;
+  a.eps = eps;
+  a.x_stride = (prologue == CTHIP_PRO_SWIGLU) ? 2 * w->cols : w->cols;
+  a.y_stride = w->rows;
+  return launch_gemv(w, a, m);
+}
+
+}  // extern "C"

@@ -1,0 +1,527 @@
+// Memory-bound fused items over the last axis (softmax, LayerNorm, RMSNorm and
+// LayerNorm->softmax), elementwise activations, embedding gather, argmax, RoPE
+// and the KV-cached attention of batch-1 decode.
+//
+// Row ops: one wavefront owns one row and keeps it in registers (VPL float4 per
+// lane, 128-bit coalesced loads/stores), so every row is read once and written
+// once; the reductions are 64-lane shuffles, no LDS.  Rows longer than
+// 64*4*8 = 2048 floats fall back to one 256-thread block per row that re-reads
+// the row through L2.
+#include "common.h"
+
+namespace cthip {
+
+enum { ROW_SOFTMAX = 0, ROW_LAYERNORM = 1, ROW_RMSNORM = 2, ROW_LN_SOFTMAX = 3 };
+
+struct RowArgs {
+  float *y;
+  const float *x;
+  const float *g;
+  const float *b;
+  float eps;
+  int64_t rows;
+  int n;
+};
+
+template <int MODE, int VPL>
+__global__ __launch_bounds__(256) void k_rowop(RowArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (row >= a.rows) return;
+  const int n = a.n;
+  const int n4 = n >> 2;  // n % 4 == 0 on this path
+  const float4 *__restrict__ xp = (const float4 *)(a.x + row * n);
+  float4 *__restrict__ yp = (float4 *)(a.y + row * n);
+  float v[VPL][4];
+  bool ok[VPL];
+#pragma unroll
+  for (int j = 0; j < VPL; j++) {
+    const int c = lane + 64 * j;
+    ok[j] = c < n4;
+    float4 t = ok[j] ? xp[c] : make_float4(0.f, 0.f, 0.f, 0.f);
+    v[j][0] = t.x; v[j][1] = t.y; v[j][2] = t.z; v[j][3] = t.w;
+  }
+  if (MODE == ROW_LAYERNORM || MODE == ROW_RMSNORM || MODE == ROW_LN_SOFTMAX) {
+    const float inv_n = 1.0f / (float)n;
+    float mean = 0.0f;
+    if (MODE != ROW_RMSNORM) {
+      float s = 0.0f;
+#pragma unroll
+      for (int j = 0; j < VPL; j++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) s += v[j][e];
+      mean = wave_sum(s) * inv_n;
+    }
+    float q = 0.0f;
+#pragma unroll
+    for (int j = 0; j < VPL; j++)
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        float d = ok[j] ? v[j][e] - mean : 0.0f;
+        v[j][e] = d;
+        q = fmaf(d, d, q);
+      }
+    const float rstd = 1.0f / sqrtf(wave_sum(q) * inv_n + a.eps);
+#pragma unroll
+    for (int j = 0; j < VPL; j++) {
+      if (ok[j]) {
+        const int c = lane + 64 * j;
+        float4 gm = a.g ? ((const float4 *)a.g)[c] : make_float4(1.f, 1.f, 1.f, 1.f);
+        float4 bt = a.b ? ((const float4 *)a.b)[c] : make_float4(0.f, 0.f, 0.f, 0.f);
+        v[j][0] = v[j][0] * rstd * gm.x + bt.x;
+        v[j][1] = v[j][1] * rstd * gm.y + bt.y;
+        v[j][2] = v[j][2] * rstd * gm.z + bt.z;
+        v[j][3] = v[j][3] * rstd * gm.w + bt.w;
+      }
+    }
+  }
+  if (MODE == ROW_SOFTMAX || MODE == ROW_LN_SOFTMAX) {
+    float m = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < VPL; j++)
+#pragma unroll
+      for (int e = 0; e < 4; e++)
+        if (ok[j]) m = fmaxf(m, v[j][e]);
+    m = wave_max(m);
+    float s = 0.0f;
+#pragma unroll
+    for (int j = 0; j < VPL; j++)
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        float ex = ok[j] ? ct_exp(v[j][e] - m) : 0.0f;
+        v[j][e] = ex;
+        s += ex;
+      }
+    const float inv = 1.0f / wave_sum(s);
+#pragma unroll
+    for (int j = 0; j < VPL; j++)
+#pragma unroll
+      for (int e = 0; e < 4; e++) v[j][e] *= inv;
+  }
+#pragma unroll
+  for (int j = 0; j < VPL; j++)
+    if (ok[j]) yp[lane + 64 * j] = make_float4(v[j][0], v[j][1], v[j][2], v[j][3]);
+}
+
+// any n: one block per row, three passes through L2
+template <int MODE>
+__global__ __launch_bounds__(256) void k_rowop_generic(RowArgs a) {
+  __shared__ float red[4];
+  const int tid = threadIdx.x;
+  const int n = a.n;
+  const float *__restrict__ xr = a.x + (int64_t)blockIdx.x * n;
+  float *__restrict__ yr = a.y + (int64_t)blockIdx.x * n;
+  auto block_sum = [&](float v) {
+    v = wave_sum(v);
+    __syncthreads();
+    if ((tid & 63) == 0) red[tid >> 6] = v;
+    __syncthreads();
+    return red[0] + red[1] + red[2] + red[3];
+  };
+  auto block_max = [&](float v) {
+    v = wave_max(v);
+    __syncthreads();
+    if ((tid & 63) == 0) red[tid >> 6] = v;
+    __syncthreads();
+    return fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  };
+  float mean = 0.0f, rstd = 1.0f;
+  const bool norm = MODE != ROW_SOFTMAX;
+  if (norm) {
+    if (MODE != ROW_RMSNORM) {
+      float s = 0.0f;
+      for (int i = tid; i < n; i += 256) s += xr[i];
+      mean = block_sum(s) / (float)n;
+    }
+    float q = 0.0f;
+    for (int i = tid; i < n; i += 256) {
+      float d = xr[i] - mean;
+      q = fmaf(d, d, q);
+    }
+    rstd = 1.0f / sqrtf(block_sum(q) / (float)n + a.eps);
+  }
+  auto val = [&](int i) {
+    float t = xr[i];
+    if (norm) {
+      t = (t - mean) * rstd;
+      if (a.g) t *= a.g[i];
+      if (a.b) t += a.b[i];
+    }
+    return t;
+  };
+  if (MODE == ROW_LAYERNORM || MODE == ROW_RMSNORM) {
+    for (int i = tid; i < n; i += 256) yr[i] = val(i);
+    return;
+  }
+  float m = -INFINITY;
+  for (int i = tid; i < n; i += 256) m = fmaxf(m, val(i));
+  m = block_max(m);
+  float s = 0.0f;
+  for (int i = tid; i < n; i += 256) s += ct_exp(val(i) - m);
+  const float inv = 1.0f / block_sum(s);
+  for (int i = tid; i < n; i += 256) yr[i] = ct_exp(val(i) - m) * inv;
+}
+
+template <int MODE>
+static int launch_rowop(RowArgs a) {
+  if (a.rows == 0 || a.n == 0) return 0;
+  hipStream_t st = state().stream;
+  if (a.n % 4 == 0 && a.n <= 2048 && ((uintptr_t)a.x % 16 == 0) && ((uintptr_t)a.y % 16 == 0) &&
+      (!a.g || (uintptr_t)a.g % 16 == 0) && (!a.b || (uintptr_t)a.b % 16 == 0)) {
+    const int n4 = a.n / 4;
+    const int vpl = (n4 + 63) / 64;
+    if ((a.rows + 3) / 4 > 0x7fffffff) return fail(CTHIP_E_BAD_ARG, "row op: too many rows");
+    dim3 grid((unsigned)((a.rows + 3) / 4)), block(256);
+    switch (vpl) {
+      case 1: hipLaunchKernelGGL((k_rowop<MODE, 1>), grid, block, 0, st, a); break;
+      case 2: hipLaunchKernelGGL((k_rowop<MODE, 2>), grid, block, 0, st, a); break;
+      case 3: hipLaunchKernelGGL((k_rowop<MODE, 3>), grid, block, 0, st, a); break;
+      case 4: hipLaunchKernelGGL((k_rowop<MODE, 4>), grid, block, 0, st, a); break;
+      case 5: case 6: hipLaunchKernelGGL((k_rowop<MODE, 6>), grid, block, 0, st, a); break;
+      default: hipLaunchKernelGGL((k_rowop<MODE, 8>), grid, block, 0, st, a); break;
+    }
+  } else {
+    if (a.rows > 0x7fffffff) return fail(CTHIP_E_BAD_ARG, "row op: too many rows");
+    hipLaunchKernelGGL((k_rowop_generic<MODE>), dim3((unsigned)a.rows), dim3(256), 0, st, a);
+  }
+  CTHIP_LAUNCH_CHECK();
+  return 0;
+}
+
+// ------------------------------------------------------------------ elementwise
+__global__ __launch_bounds__(256) void k_unary(int kind, float *__restrict__ y, const float *__restrict__ x, int64_t n) {
+  const int64_t n4 = n >> 2;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const bool vec = ((uintptr_t)x % 16 == 0) && ((uintptr_t)y % 16 == 0);
+  if (vec) {
+    for (int64_t k = i; k < n4; k += stride) {
+      float4 v = ((const float4 *)x)[k];
+      v.x = apply_act(kind, v.x);
+      v.y = apply_act(kind, v.y);
+      v.z = apply_act(kind, v.z);
+      v.w = apply_act(kind, v.w);
+      ((float4 *)y)[k] = v;
+    }
+    for (int64_t k = n4 * 4 + i; k < n; k += stride) y[k] = apply_act(kind, x[k]);
+  } else {
+    for (int64_t k = i; k < n; k += stride) y[k] = apply_act(kind, x[k]);
+  }
+}
+
+// out[t,:] = W[idx[t],:]  (+ W2[pos0 + t,:] when W2 is given: wte + wpe of Transformer, layers.lisp:80-82)
+__global__ __launch_bounds__(256) void k_embedding(float *__restrict__ out, const float *__restrict__ W,
+                                                   const float *__restrict__ idx_f, const int *__restrict__ idx_i,
+                                                   int vocab, int dim, const float *__restrict__ W2,
+                                                   const int *__restrict__ pos, int max_pos) {
+  const int t = blockIdx.x;
+  int id = idx_f ? (int)idx_f[t] : idx_i[t];
+  const bool hit = id >= 0 && id < vocab && (!idx_f || (float)id == idx_f[t]);
+  int p = 0;
+  bool phit = false;
+  if (W2) {
+    p = pos[0] + t;
+    phit = p >= 0 && p < max_pos;
+  }
+  for (int d = threadIdx.x; d < dim; d += blockDim.x) {
+    // an index no vocabulary row equals selects nothing in the reference's one-hot sum: 0
+    float v = hit ? W[(int64_t)id * dim + d] : 0.0f;
+    if (W2) v += phit ? W2[(int64_t)p * dim + d] : 0.0f;
+    out[(int64_t)t * dim + d] = v;
+  }
+}
+
+// lowest index of the maximum of each row; one 1024-thread block per row.
+// tok_out/pos (optional) feed the device-resident decode loop: the token is also
+// stored as int32 and the position counter advanced.
+__global__ __launch_bounds__(1024) void k_argmax(int64_t *__restrict__ out, const float *__restrict__ x, int n,
+                                                 int *__restrict__ tok_out, int *__restrict__ pos,
+                                                 int64_t *__restrict__ history, int *__restrict__ hist_n) {
+  __shared__ float sm[16];
+  __shared__ int si[16];
+  const float *__restrict__ xr = x + (int64_t)blockIdx.x * n;
+  float best = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    float v = xr[i];
+    if (v > best || (v == best && i < bi)) {
+      best = v;
+      bi = i;
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    float ob = __shfl_xor(best, o, 64);
+    int oi = __shfl_xor(bi, o, 64);
+    if (ob > best || (ob == best && oi < bi)) {
+      best = ob;
+      bi = oi;
+    }
+  }
+  const int w = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  if ((threadIdx.x & 63) == 0) {
+    sm[w] = best;
+    si[w] = bi;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int k = 1; k < nw; k++)
+      if (sm[k] > best || (sm[k] == best && si[k] < bi)) {
+        best = sm[k];
+        bi = si[k];
+      }
+    if (bi == 0x7fffffff) bi = 0;  // all-NaN / empty row
+    out[blockIdx.x] = bi;
+    if (tok_out) *tok_out = bi;
+    if (history) {
+      history[*hist_n] = bi;
+      *hist_n = *hist_n + 1;
+    }
+    if (pos) *pos = *pos + 1;
+  }
+}
+
+// RoPE on (B,S,H,Dh), one thread per (pair)
+__global__ __launch_bounds__(256) void k_rope(float *__restrict__ out, const float *__restrict__ x, int64_t npairs,
+                                              int S, int H, int Dh, float log2_base, int start_pos,
+                                              const int *__restrict__ pos) {
+  int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= npairs) return;
+  const int half = Dh >> 1;
+  const int i = (int)(p % half);
+  const int64_t r = p / half;  // (b*S + s)*H + h
+  const int s = (int)((r / H) % S);
+  const int at = s + start_pos + (pos ? pos[0] : 0);
+  // theta_i = exp(-(2i/Dh) * ln base), spelled through exp2/log2 with a float rounding at each
+  // tensor the reference materialises (positional-encoding.lisp:26-35)
+  const float expo = (float)(2 * i) / (float)Dh;
+  const float logb = log2_base * 0.6931472f;
+  const float theta = exp2f(-(expo * logb) * 1.442695f);
+  const float ang = (float)at * theta;
+  float sn, cs;
+  sincosf(ang, &sn, &cs);
+  const float x0 = x[2 * p], x1 = x[2 * p + 1];
+  out[2 * p] = x0 * cs - x1 * sn;
+  out[2 * p + 1] = x0 * sn + x1 * cs;
+}
+
+// Llama-shaped decode: rotate the new key row (Hkv,Dh) at position pos[0] into the K cache and
+// copy the new value row beside it.  kv holds k then v, KD floats each.
+__global__ __launch_bounds__(256) void k_rope_append(float *__restrict__ kc, float *__restrict__ vc,
+                                                     const float *__restrict__ kv, int Hkv, int Dh, float log2_base,
+                                                     const int *__restrict__ pos) {
+  const int KD = Hkv * Dh;
+  const int p = blockIdx.x * blockDim.x + threadIdx.x;  // pair index
+  if (p >= KD / 2) return;
+  const int at = pos[0];
+  const int i = p % (Dh / 2);
+  const float expo = (float)(2 * i) / (float)Dh;
+  const float logb = log2_base * 0.6931472f;
+  const float theta = exp2f(-(expo * logb) * 1.442695f);
+  const float ang = (float)at * theta;
+  float sn, cs;
+  sincosf(ang, &sn, &cs);
+  const float x0 = kv[2 * p], x1 = kv[2 * p + 1];
+  float *ko = kc + (int64_t)at * KD;
+  float *vo = vc + (int64_t)at * KD;
+  ko[2 * p] = x0 * cs - x1 * sn;
+  ko[2 * p + 1] = x0 * sn + x1 * cs;
+  vo[2 * p] = kv[KD + 2 * p];
+  vo[2 * p + 1] = kv[KD + 2 * p + 1];
+}
+
+// ------------------------------------------------------------------ attention over the KV cache
+// One 256-thread block per (query head h, query row i).  Keys 0..T-1 with T = pos+i+1 (causal mask of
+// layers.lisp:83).  Scores live in LDS (max_seq floats).  K/V cache layout (max_len, Hkv, Dh).
+template <int DH>
+__global__ __launch_bounds__(256) void k_attn_cached(float *__restrict__ out, const float *__restrict__ q,
+                                                     const float *__restrict__ kc, const float *__restrict__ vc,
+                                                     int start_pos, const int *__restrict__ pos, int H, int Hkv) {
+  extern __shared__ float sc[];  // T scores, then 4 + (256/DH)*DH floats of scratch
+  __shared__ float red[4];
+  __shared__ float qs[DH];
+  const int h = blockIdx.x, i = blockIdx.y;
+  const int T = start_pos + (pos ? pos[0] : 0) + i + 1;
+  const int hk = h / (H / Hkv);
+  const int tid = threadIdx.x;
+  const int64_t kv_stride = (int64_t)Hkv * DH;
+  if (tid < DH) qs[tid] = q[((int64_t)i * H + h) * DH + tid];
+  __syncthreads();
+  // scores: one key per thread
+  float lmax = -INFINITY;
+  for (int j = tid; j < T; j += 256) {
+    const float4 *kp = (const float4 *)(kc + j * kv_stride + (int64_t)hk * DH);
+    float acc = 0.0f;
+#pragma unroll
+    for (int d = 0; d < DH / 4; d++) {
+      float4 kk = kp[d];
+      acc = fmaf(qs[4 * d + 0], kk.x, acc);
+      acc = fmaf(qs[4 * d + 1], kk.y, acc);
+      acc = fmaf(qs[4 * d + 2], kk.z, acc);
+      acc = fmaf(qs[4 * d + 3], kk.w, acc);
+    }
+    acc = acc / sqrtf((float)DH);
+    sc[j] = acc;
+    lmax = fmaxf(lmax, acc);
+  }
+  lmax = wave_max(lmax);
+  if ((tid & 63) == 0) red[tid >> 6] = lmax;
+  __syncthreads();
+  const float m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  __syncthreads();
+  float lsum = 0.0f;
+  for (int j = tid; j < T; j += 256) {
+    float e = ct_exp(sc[j] - m);
+    sc[j] = e;
+    lsum += e;
+  }
+  lsum = wave_sum(lsum);
+  if ((tid & 63) == 0) red[tid >> 6] = lsum;
+  __syncthreads();
+  const float inv = 1.0f / (red[0] + red[1] + red[2] + red[3]);
+  // out[d] = sum_j p_j V[j,d]: thread (grp, d) walks keys grp, grp+NG, ...
+  constexpr int NG = 256 / DH;
+  float *part = sc + T;
+  const int d = tid % DH, grp = tid / DH;
+  float acc = 0.0f;
+  for (int j = grp; j < T; j += NG) acc = fmaf(sc[j] * inv, vc[j * kv_stride + (int64_t)hk * DH + d], acc);
+  part[grp * DH + d] = acc;
+  __syncthreads();
+  if (tid < DH) {
+    float s = 0.0f;
+#pragma unroll
+    for (int g2 = 0; g2 < NG; g2++) s += part[g2 * DH + tid];
+    out[((int64_t)i * H + h) * DH + tid] = s;
+  }
+}
+
+int launch_attn(float *out, const float *q, const float *kc, const float *vc, int S, int start_pos, const int *pos,
+                int max_T, int H, int Hkv, int Dh) {
+  if (S == 0) return 0;
+  hipStream_t st = state().stream;
+  const size_t lds = sizeof(float) * ((size_t)max_T + 256);
+  if (lds > 60 * 1024) return fail(CTHIP_E_UNSUPPORTED, "attention: %d cached positions exceed the LDS score buffer", max_T);
+  dim3 grid(H, S), block(256);
+  switch (Dh) {
+    case 32: hipLaunchKernelGGL(k_attn_cached<32>, grid, block, lds, st, out, q, kc, vc, start_pos, pos, H, Hkv); break;
+    case 64: hipLaunchKernelGGL(k_attn_cached<64>, grid, block, lds, st, out, q, kc, vc, start_pos, pos, H, Hkv); break;
+    case 128: hipLaunchKernelGGL(k_attn_cached<128>, grid, block, lds, st, out, q, kc, vc, start_pos, pos, H, Hkv); break;
+    default: return fail(CTHIP_E_UNSUPPORTED, "attention: head_dim %d (supported: 32, 64, 128)", Dh);
+  }
+  CTHIP_LAUNCH_CHECK();
+  return 0;
+}
+
+int launch_embedding(float *out, const float *W, const float *idx_f, const int *idx_i, int ntok, int vocab, int dim,
+                     const float *W2, const int *pos, int max_pos) {
+  if (ntok == 0) return 0;
+  hipLaunchKernelGGL(k_embedding, dim3(ntok), dim3(256), 0, state().stream, out, W, idx_f, idx_i, vocab, dim, W2, pos,
+                     max_pos);
+  CTHIP_LAUNCH_CHECK();
+  return 0;
+}
+
+int launch_argmax(int64_t *out, const float *x, int64_t rows, int n, int *tok_out, int *pos, int64_t *history,
+                  int *hist_n) {
+  if (rows == 0) return 0;
+  hipLaunchKernelGGL(k_argmax, dim3((unsigned)rows), dim3(1024), 0, state().stream, out, x, n, tok_out, pos, history,
+                     hist_n);
+  CTHIP_LAUNCH_CHECK();
+  return 0;
+}
+
+int launch_rope(float *out, const float *x, int B, int S, int H, int Dh, float base, int start_pos, const int *pos) {
+  const int64_t npairs = (int64_t)B * S * H * (Dh / 2);
+  if (npairs == 0) return 0;
+  hipLaunchKernelGGL(k_rope, dim3((unsigned)((npairs + 255) / 256)), dim3(256), 0, state().stream, out, x, npairs, S, H,
+                     Dh, log2f(base), start_pos, pos);
+  CTHIP_LAUNCH_CHECK();
+  return 0;
+}
+
+int launch_rope_append(float *kc, float *vc, const float *kv, int Hkv, int Dh, float base, const int *pos) {
+  const int pairs = Hkv * Dh / 2;
+  hipLaunchKernelGGL(k_rope_append, dim3((pairs + 255) / 256), dim3(256), 0, state().stream, kc, vc, kv, Hkv, Dh,
+                     log2f(base), pos);
+  CTHIP_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // namespace cthip
+
+using namespace cthip;
+
+extern "C" {
+
+int cthip_softmax(float *y, const float *x, int64_t rows, int n) {
+  CTHIP_REQUIRE_INIT();
+  CTHIP_ARG(rows >= 0 && n >= 0 && (rows * n == 0 || (y && x)));
+  RowArgs a = {y, x, nullptr, nullptr, 0.0f, rows, n};
+  return launch_rowop<ROW_SOFTMAX>(a);
+}
+
+int cthip_layernorm(float *y, const float *x, const float *gamma, const float *beta, float eps, int64_t rows, int n) {
+  CTHIP_REQUIRE_INIT();
+  CTHIP_ARG(rows >= 0 && n >= 0 && (rows * n == 0 || (y && x)));
+  RowArgs a = {y, x, gamma, beta, eps, rows, n};
+  return launch_rowop<ROW_LAYERNORM>(a);
+}
+
+int cthip_rmsnorm(float *y, const float *x, const float *w, float eps, int64_t rows, int n) {
+  CTHIP_REQUIRE_INIT();
+  CTHIP_ARG(rows >= 0 && n >= 0 && (rows * n == 0 || (y && x)));
+  RowArgs a = {y, x, w, nullptr, eps, rows, n};
+  return launch_rowop<ROW_RMSNORM>(a);
+}
+
+int cthip_layernorm_softmax(float *y, const float *x, const float *gamma, const float *beta, float eps, int64_t rows,
+                            int n) {
+  CTHIP_REQUIRE_INIT();
+  CTHIP_ARG(rows >= 0 && n >= 0 && (rows * n == 0 || (y && x)));
+  RowArgs a = {y, x, gamma, beta, eps, rows, n};
+  return launch_rowop<ROW_LN_SOFTMAX>(a);
+}
+
+int cthip_unary(int kind, float *y, const float *x, int64_t n) {
+  CTHIP_REQUIRE_INIT();
+  CTHIP_ARG(n >= 0 && (n == 0 || (y && x)));
+  CTHIP_ARG(kind >= CTHIP_ACT_NONE && kind <= CTHIP_ACT_TANH);
+  if (n == 0) return 0;
+  int64_t blocks = (n / 4 + 255) / 256;
+  const int64_t cap = (int64_t)state().compute_units * 16;
+  if (blocks > cap) blocks = cap;
+  if (blocks < 1) blocks = 1;
+  hipLaunchKernelGGL(k_unary, dim3((unsigned)blocks), dim3(256), 0, state().stream, kind, y, x, n);
+  CTHIP_LAUNCH_CHECK();
+  return 0;
+}
+
+int cthip_embedding(float *out, const float *W, const float *idx, int ntok, int vocab, int dim) {
+  CTHIP_REQUIRE_INIT();
+  CTHIP_ARG(ntok >= 0 && vocab > 0 && dim > 0 && (ntok == 0 || (out && W && idx)));
+  return launch_embedding(out, W, idx, nullptr, ntok, vocab, dim, nullptr, nullptr, 0);
+}
+
+int cthip_argmax(int64_t *out, const float *x, int64_t rows, int n) {
+  CTHIP_REQUIRE_INIT();
+  CTHIP_ARG(rows >= 0 && n > 0 && (rows == 0 || (out && x)));
+  if (rows > 0x7fffffff) return fail(CTHIP_E_BAD_ARG, "cthip_argmax: too many rows");
+  return launch_argmax(out, x, rows, n, nullptr, nullptr, nullptr, nullptr);
+}
+
+int cthip_rope(float *out, const float *x, int B, int S, int H, int Dh, float base, int start_pos) {
+  CTHIP_REQUIRE_INIT();
+  CTHIP_ARG(B >= 0 && S >= 0 && H >= 0 && Dh >= 0 && Dh % 2 == 0 && base > 0.0f);
+  CTHIP_ARG((int64_t)B * S * H * Dh == 0 || (out && x));
+  return launch_rope(out, x, B, S, H, Dh, base, start_pos, nullptr);
+}
+
+int cthip_sdpa_cached(float *out, const float *q, const float *k_cache, const float *v_cache, int S, int start_pos,
+                      int H, int Hkv, int Dh) {
+  CTHIP_REQUIRE_INIT();
+  CTHIP_ARG(S >= 0 && start_pos >= 0 && H > 0 && Hkv > 0 && H % Hkv == 0);
+  CTHIP_ARG(S == 0 || (out && q && k_cache && v_cache));
+  return launch_attn(out, q, k_cache, v_cache, S, start_pos, nullptr, start_pos + S, H, Hkv, Dh);
+}
+
+}  // extern "C"

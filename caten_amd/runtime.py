@@ -1,0 +1,255 @@
+"""HipRuntime: the VM half of the `:HIP` backend.
+
+Mirrors Caten's GraphRuntime (source/runtime/runtime.lisp:39-145,228-284) and the
+JIT_KERNEL node (source/codegen/jit.lisp:92-143, source/codegen/runner.lisp:20-32):
+a program counter walks a flat node list; `:Allocate` opens (or reuses) buffers,
+`:View` re-describes storage without moving data, `:JIT_KERNEL` launches one
+compiled kernel and returns the arguments at its out-positions.  Custom,
+non-rendered ops (the hand-written fused kernels) are ordinary node types with a
+`realize_node` method, the extension mechanism of source/runtime/runtime.lisp:118.
+
+The graph is handed over as plain data (see `Node`): in a Lisp process the same
+walk is driven by Caten itself and only the C ABI below it is shared.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import time
+from dataclasses import dataclass, field
+from typing import Any, Callable, Dict, List, Optional, Sequence
+
+import numpy as np
+
+from . import _lib
+from .backend import define_backend
+from .buffer import (AbstractBuffer, DTYPES, HipBuffer, close_buffer, make_buffer, open_buffer,
+                     transfer_from_array, transfer_into_array)
+
+
+@dataclass
+class Node:
+    """caten/air Node: type, writes, reads and an attribute plist."""
+    type: str
+    writes: List[str]
+    reads: List[Any]
+    attrs: Dict[str, Any] = field(default_factory=dict)
+
+
+class RuntimeError_(RuntimeError):
+    """runtime-error (runtime.lisp:84-104): carries the pc and a disassembly."""
+
+    def __init__(self, runtime: "GraphRuntime", cond: BaseException):
+        lines = []
+        for i, n in enumerate(runtime.graph):
+            lines.append(f"{'*' if i == runtime.pc else ' '}{i} | {n.type} {n.writes} <- {n.reads}")
+        super().__init__(f"Runtime-Error: Encountered the runtime error at instruction {runtime.pc}.\n"
+                         f"condition:\n  {cond}\ndisassemble:\n" + "\n".join(lines))
+        self.cond = cond
+
+
+@dataclass
+class CompiledKernel:
+    """Compiled-Kernel (jit.lisp:92-103)."""
+    name: str
+    caller: Callable
+    device: str = "HIP"
+    code: str = ""
+    out_positions: Sequence[int] = (0,)
+    flops: Optional[int] = None
+
+
+def coerce_dtyped_buffer(arg, dtype: str):
+    """coerce-dtyped-buffer (source/codegen/helpers.lisp:118-125): rank-0 buffers are
+    passed by value, cast to the declared dtype."""
+    if isinstance(arg, AbstractBuffer):
+        if arg.nrank == 0:
+            return DTYPES[dtype](arg.value).item()
+        return arg
+    return DTYPES[dtype](arg).item()
+
+
+class GraphRuntime:
+    buffer_type = AbstractBuffer
+
+    def __init__(self, graph: List[Node], fw_outputs: Sequence[str] = (), variables: Optional[dict] = None,
+                 renderer=None):
+        self.graph = list(graph)
+        self.fw_outputs = list(fw_outputs)
+        self.variables: Dict[Any, Any] = dict(variables or {})
+        self.renderer = renderer
+        self.pc = 0
+        self.profile = os.environ.get("PROFILE", "0") == "1"
+        self.times = {"kernel": 0.0, "vm": 0.0, "allocate": 0.0}
+
+    # runtime-setvar / runtime-getvar (runtime.lisp:66-74)
+    def setvar(self, var, value):
+        if not (isinstance(value, (int, float, bool, np.number, AbstractBuffer))):
+            raise TypeError(f"Runtime: the value {value!r} is not one of AbstractBuffer, number, boolean")
+        self.variables[var] = value
+
+    def getvar(self, var):
+        if var not in self.variables:
+            raise KeyError(f"Runtime: the variable {var} is not defined in the graph.")
+        return self.variables[var]
+
+    def step(self) -> bool:
+        """runtime-step (runtime.lisp:106-132)"""
+        node = self.graph[self.pc]
+        t1 = time.perf_counter()
+        try:
+            args = [a if isinstance(a, (int, float)) and not isinstance(a, bool) else self.getvar(a)
+                    for a in node.reads]
+            out = self.realize_node(node, args)
+        except Exception as e:  # wrapped like handler-bind ... runtime-error
+            raise RuntimeError_(self, e) from e
+        if self.profile and node.type != "JIT_KERNEL":
+            self.times["allocate" if node.type == "Allocate" else "vm"] += time.perf_counter() - t1
+        if not isinstance(out, tuple):
+            out = (out,)
+        if node.writes and len(out) != len(node.writes):
+            raise RuntimeError_(self, AssertionError("Runtime: the number of outputs does not match the number of writes."))
+        for place, value in zip(node.writes, out):
+            self.setvar(place, value)
+        self.pc += 1
+        return True
+
+    def forward(self, *params):
+        """runtime-forward after runtime-set-params (api/iseq.lisp:481-529): params are
+        (symbol, buffer-or-number) pairs; returns the fw-outputs."""
+        for k, v in params:
+            self.setvar(k, v)
+        self.pc = 0
+        while self.pc < len(self.graph):
+            self.step()
+        outs = tuple(self.getvar(o) for o in self.fw_outputs)
+        return outs[0] if len(outs) == 1 else outs
+
+    def free(self):
+        """free-runtime (runtime.lisp:76-81)"""
+        for v in self.variables.values():
+            if isinstance(v, AbstractBuffer):
+                close_buffer(self, v)
+        for n in self.graph:
+            pool = n.attrs.get("pool")
+            if isinstance(pool, AbstractBuffer):
+                close_buffer(self, pool)
+                n.attrs["pool"] = None
+
+    # ---- realize-node ----
+    def realize_node(self, node: Node, args):
+        fn = getattr(self, "realize_" + node.type.lower().replace("/", "_").replace("-", "_"), None)
+        if fn is None:
+            raise NotImplementedError(f"realize-node: no method for node type :{node.type} on {type(self).__name__}")
+        return fn(node, args)
+
+    def _num(self, x):
+        return x.value if isinstance(x, AbstractBuffer) else x
+
+    def realize_allocate(self, node: Node, args):
+        """realize-node :Allocate incl. the :from case and pool reuse (runtime.lisp:228-259).
+        args = shape numbers then stride numbers (nrank each)."""
+        frm = node.attrs.get("from")
+        if frm is not None:
+            val = self.getvar(frm) if not isinstance(frm, AbstractBuffer) else frm
+            if not isinstance(val, AbstractBuffer):
+                raise TypeError(f"The :from attribute in the {node.type} node should be a buffer or a symbol.")
+            return self.adopt(val)
+        nrank = node.attrs["nrank"]
+        shape = [int(self._num(a)) for a in args[:nrank]]
+        stride = [int(self._num(a)) for a in args[nrank:2 * nrank]]
+        pool = node.attrs.get("pool")
+        if isinstance(pool, AbstractBuffer) and shape:
+            if shape == list(pool.shape):
+                return pool
+            close_buffer(self, pool)
+        buf = make_buffer(shape, stride, node.attrs["dtype"], None, device=self.buffer_type)
+        open_buffer(self, buf)
+        node.attrs["pool"] = buf
+        return buf
+
+    def adopt(self, buf: AbstractBuffer) -> AbstractBuffer:
+        return buf
+
+    def realize_view(self, node: Node, args):
+        """realize-node :View (runtime.lisp:261-284): args = buffer, shape, from, to, by, stride (nrank each)."""
+        nrank = node.attrs["nrank"]
+        base = args[0]
+        rest = [self._num(a) for a in args[1:]]
+        shape, v1, v2, v3, stride = (rest[i * nrank:(i + 1) * nrank] for i in range(5))
+        bc = node.attrs.get("broadcast", [False] * nrank)
+        buf = base.copy()
+        buf.shape, buf.stride = [int(s) for s in shape], [int(s) for s in stride]
+        buf.views = [(int(a), int(b), int(c), bool(d)) for a, b, c, d in zip(v1, v2, v3, bc)]
+        buf.nrank = nrank
+        return buf
+
+    def realize_jit_kernel(self, node: Node, args):
+        """realize-node :JIT_KERNEL (runner.lisp:23-32)"""
+        info: CompiledKernel = node.attrs["kernel_info"]
+        args = [coerce_dtyped_buffer(a, dt) for a, dt in zip(args, node.attrs["dtypes"])]
+        t1 = time.perf_counter()
+        self.invoke_jit_kernel(info, node, args)
+        if self.profile:
+            _lib.check(_lib.load().cthip_sync())  # PROFILE assumes synchronous kernels (runner.lisp:27)
+            dt = time.perf_counter() - t1
+            self.times["kernel"] += dt
+            print(f"{self.pc} |  KERNEL  | {dt:.6f}s | {info.device}[{info.name}]")
+        outs = tuple(args[i] for i in info.out_positions)
+        return outs if len(outs) != 1 else outs[0]
+
+    def invoke_jit_kernel(self, info: CompiledKernel, node: Node, args):
+        """runtime-invoke-jit-kernel (runner.lisp:20-21; Metal passes the node too, metal.lisp:285-286)"""
+        info.caller(node, *args)
+
+    def realize_pause_backward(self, node: Node, args):
+        return tuple(args) if len(args) != 1 else args[0]
+
+
+class HipRuntime(GraphRuntime):
+    """GraphRuntime whose buffers live in HBM; opens the device on creation
+    (cf. MetalRuntime's initialize-instance :after, source/byoc/metal.lisp:106-112)."""
+    buffer_type = HipBuffer
+
+    def __init__(self, graph=(), fw_outputs=(), variables=None, renderer=None, device: int = 0):
+        super().__init__(list(graph), fw_outputs, variables, renderer)
+        self.lib = _lib.init(device)
+        self._uploaded: Dict[int, HipBuffer] = {}
+
+    def adopt(self, buf: AbstractBuffer) -> AbstractBuffer:
+        """Weights loaded from GGUF are host buffers whatever the backend
+        (external/gguf/tensor-info.lisp:104-120) and enter through `:Allocate :from`
+        untouched (runtime.lisp:228-243): upload once and cache the device copy."""
+        if isinstance(buf, HipBuffer) or buf.nrank == 0:
+            return buf
+        key = id(buf)
+        if key not in self._uploaded:
+            dev = make_buffer(buf.shape, buf.stride, buf.dtype, buf.views, device=HipBuffer)
+            open_buffer(self, dev)
+            transfer_from_array(self, dev, np.asarray(buf.value))
+            self._uploaded[key] = dev
+        return self._uploaded[key]
+
+    def sync(self):
+        _lib.check(self.lib.cthip_sync())
+
+    def free(self):
+        super().free()
+        for b in self._uploaded.values():
+            close_buffer(self, b)
+        self._uploaded.clear()
+
+
+class HipAutoScheduler:
+    """define-auto-scheduler (Hip-Auto-Scheduler ()) :n-global-loop 3 (cf. metal.lisp:153).
+    Work distribution is chosen by the renderer per kernel pattern, not by ISL marks."""
+    n_global_loop = 3
+    tile_sizes = (2, 4, 8, 16, 32)
+
+
+def _register():
+    from .renderer import HipRenderer
+    define_backend("HIP", HipBuffer, HipRuntime, HipRenderer, HipAutoScheduler, True)
+
+
+_register()

@@ -1,0 +1,237 @@
+/*
+ * caten_hip.h -- C ABI of libcaten_hip.so, the MI355X (gfx950) execution
+ * backend that plugs into Caten's BYOC backend interface as `:HIP`.
+ *
+ * Everything here is plain C: opaque pointers, sizes, integer status returns.
+ * A host in any language binds it the way Caten's CLANG backend binds the
+ * shared library gcc produces (source/byoc/clang.lisp:127-157,163-205): one
+ * foreign-funcall per entry point, no callbacks into the host.
+ *
+ * Status: 0 = ok; >0 = a hipError_t / hiprtcResult from the runtime;
+ * <0 = an argument or state error detected by this library.  After any
+ * non-zero return cthip_last_error() describes the failure (the Lisp side
+ * signals `error` with that text so it surfaces as a runtime-error,
+ * source/runtime/runtime.lisp:84-104).
+ *
+ * Threading: one in-order HIP stream per process, as Caten's VM is single
+ * threaded (source/runtime/runtime.lisp:134-145).  Every launch and copy below
+ * is asynchronous on that stream except cthip_d2h, cthip_sync and the entry
+ * points documented as synchronous.
+ */
+#ifndef CATEN_HIP_H
+#define CATEN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- error codes detected here ---- */
+#define CTHIP_OK 0
+#define CTHIP_E_NOT_INIT (-1)
+#define CTHIP_E_BAD_ARG (-2)
+#define CTHIP_E_UNSUPPORTED (-3)
+#define CTHIP_E_COMPILE (-4)
+#define CTHIP_E_STATE (-5)
+
+/* ggml tensor type ids (external/gguf/tensor-info.lisp:3-31) */
+#define CTHIP_F32 0
+#define CTHIP_F16 1
+#define CTHIP_Q4_0 2
+#define CTHIP_Q8_0 8
+
+/* ================================================================== */
+/* Runtime: device, buffers, modules, launches                         */
+/* ================================================================== */
+
+/* HipRuntime's initialize-instance :after (cf. MetalRuntime,
+ * source/byoc/metal.lisp:106-112): selects the device, creates the stream.
+ * Idempotent for the same device. */
+int cthip_init(int device);
+/* Frees every cached block and destroys the stream (free-runtime,
+ * source/runtime/runtime.lisp:76-81). */
+int cthip_shutdown(void);
+const char *cthip_last_error(void);
+/* name_cap bytes of device name, compute units, wavefront size, LDS bytes per
+ * workgroup, total device memory.  Any out pointer may be NULL. */
+int cthip_device_info(char *name, int name_cap, int *compute_units, int *wave_size,
+                      size_t *lds_bytes, size_t *mem_bytes);
+
+/* open-buffer (source/runtime/buffer.lisp:78-79): device storage of `bytes`
+ * bytes, contents zeroed.  Backed by a caching allocator because every buffer
+ * whose shape mentions the symbolic `s`/`n` is re-opened on each decode step
+ * (source/runtime/runtime.lisp:248-259). bytes == 0 yields a valid 256-byte block. */
+int cthip_alloc(void **out, size_t bytes);
+/* close-buffer (buffer.lisp:81): returns the block to the cache. NULL is a no-op. */
+int cthip_free(void *p);
+/* Releases all cached (unused) blocks back to the driver. */
+int cthip_cache_trim(void);
+int cthip_cache_stats(size_t *live_bytes, size_t *cached_bytes, size_t *driver_allocs);
+
+/* transfer-from-array (buffer.lisp:83): host -> device.  The source is staged
+ * so the caller's array may be unpinned as soon as the call returns
+ * (cffi:with-pointer-to-vector-data only pins for the call, clang.lisp:177-178). */
+int cthip_h2d(void *dst, const void *src, size_t bytes);
+/* transfer-into-array (buffer.lisp:85): device -> host; synchronises the stream. */
+int cthip_d2h(void *dst, const void *src, size_t bytes);
+/* copy-buffer-value (buffer.lisp:87) */
+int cthip_d2d(void *dst, const void *src, size_t bytes);
+int cthip_memset(void *dst, int byte, size_t bytes);
+int cthip_sync(void);
+/* The hipStream_t all work is queued on (for event timing by a harness). */
+void *cthip_stream(void);
+
+/* %compile-kernel (source/codegen/renderer.lisp:30-34; CLANG: clang.lisp:207-226;
+ * METAL: metal.lisp:326-345): compile one HIP source holding every rendered
+ * kernel of a graph with hipRTC for `arch` (NULL = "gfx950").  On success
+ * `*code` / `*code_size` hold the code object; on failure returns CTHIP_E_COMPILE
+ * and *log (if non-NULL) holds the compiler output.  Release both with
+ * cthip_release(). Needs no GPU. */
+int cthip_compile(const char *hip_source, const char *arch, void **code, size_t *code_size, char **log);
+void cthip_release(void *p);
+/* Metal-Program's newLibraryWithData / newFunctionWithName (metal.lisp:263-277) */
+int cthip_module_load(void **module, const void *code);
+int cthip_module_unload(void *module);
+int cthip_get_function(void **fn, void *module, const char *name);
+/* Metal-Program invoke (metal.lisp:288-322): args[i] points at the i-th kernel
+ * argument value (a device pointer or a by-value scalar), in Caten's order
+ * outputs -> dynamic shapes -> inputs (source/codegen/rewriting-rules.lisp:207-231). */
+int cthip_launch(void *fn, const unsigned grid[3], const unsigned block[3], unsigned lds_bytes,
+                 void **args, int nargs);
+
+/* Event timing on the library's stream (PROFILE=1 in the reference times each
+ * JIT kernel on the host clock, source/codegen/runner.lisp:7-31). */
+int cthip_timer_start(void);
+int cthip_timer_stop(float *milliseconds); /* synchronous */
+
+/* ================================================================== */
+/* GGUF block codecs                                                   */
+/* ================================================================== */
+
+/* dequantize (external/gguf/dequantize.lisp:14-53) on the device: `raw` is the
+ * tensor's bytes exactly as they sit in a GGUF file (device pointer), `n` the
+ * element count (Q8_0: the last block may be short; Q4_0, which the reference
+ * lacks, needs n % 32 == 0).  out[i] is bit-exact single float. */
+int cthip_dequant(int ggml_type, const void *raw, int64_t n, float *out);
+
+/* A weight matrix (rows x cols, Linear's (out,in) layout, source/nn/linear.lisp:9)
+ * kept PACKED in HBM for dequant-in-register products.  `raw` = GGUF bytes on
+ * the device, row-major, cols % 32 == 0 for quantised types.  The bytes are
+ * re-laid into a quant plane and a scale plane (same total size) so that every
+ * lane issues aligned 128-bit loads.  The raw buffer may be freed afterwards. */
+int cthip_wmat_create(void **wmat, int ggml_type, const void *raw, int64_t rows, int64_t cols);
+int cthip_wmat_destroy(void *wmat);
+/* Bytes the matrix occupies in HBM (the algorithmic bytes of one GEMV over it). */
+int64_t cthip_wmat_nbytes(const void *wmat);
+/* Expands the packed planes to fp32 (rows*cols); bit-exact with cthip_dequant of the raw bytes. */
+int cthip_wmat_dequant(const void *wmat, float *out);
+
+/* ================================================================== */
+/* Hand-written fused items (what Caten's Schedule-Items compute)      */
+/* ================================================================== */
+
+/* prologue applied to the input vector(s) of cthip_linear */
+#define CTHIP_PRO_NONE 0
+#define CTHIP_PRO_LAYERNORM 1 /* LayerNorm, nn/normalization.lisp:39-58 */
+#define CTHIP_PRO_RMSNORM 2   /* RMSNorm,   nn/normalization.lisp:70-85 */
+#define CTHIP_PRO_SWIGLU 3    /* x is (m, 2*cols): silu(x[:cols]) * x[cols:], nn/activations.lisp:180-189 */
+/* epilogue activation */
+#define CTHIP_ACT_NONE 0
+#define CTHIP_ACT_RELU 1 /* nn/activations.lisp:34-44 */
+#define CTHIP_ACT_GELU 2 /* GeLU :tanh, nn/activations.lisp:202-215 */
+#define CTHIP_ACT_SILU 3
+
+/* Linear (source/nn/linear.lisp:3-17) with the elementwise neighbours Caten's
+ * scheduler fuses around it (test-scheduler.lisp:140-163):
+ *   y[m,:] = act( prologue(x[m,:]) @ W^T + bias ) + residual[m,:]
+ * x (m, cols) [(m, 2*cols) for SWIGLU], y/residual (m, rows), fp32, contiguous.
+ * norm_g/norm_b/bias/residual may be NULL.  m == 1 is the dequant-in-register
+ * GEMV of batch-1 decode; m > 1 uses the tiled path. */
+int cthip_linear(float *y, const void *wmat, const float *x, int m, const float *bias,
+                 const float *residual, int act, int prologue, const float *norm_g,
+                 const float *norm_b, float eps);
+
+/* !relu(!matmul A B) (api/high-level-ops.lisp:76-99; fused per test-scheduler.lisp:140-163):
+ * C (M,N) = act(A (M,K) @ B (K,N)), row-major fp32.  precision 0 = fp32 MFMA
+ * accumulate-in-order-free fp32 (rtol 1e-3/atol 1e-4), 1 = bf16 MFMA inputs with
+ * fp32 accumulation (rtol/atol 1e-2). */
+int cthip_matmul(float *C, const float *A, const float *B, int M, int N, int K, int act, int precision);
+
+/* Row ops over the last axis, fp32, rows x n contiguous. */
+int cthip_softmax(float *y, const float *x, int64_t rows, int n);   /* nn/activations.lisp:59-62,107-119 */
+int cthip_layernorm(float *y, const float *x, const float *gamma, const float *beta, float eps,
+                    int64_t rows, int n);                            /* nn/normalization.lisp:39-58 */
+int cthip_rmsnorm(float *y, const float *x, const float *w, float eps, int64_t rows, int n); /* :70-85 */
+/* LayerNorm immediately followed by softmax over the same axis, one pass over HBM. */
+int cthip_layernorm_softmax(float *y, const float *x, const float *gamma, const float *beta, float eps,
+                            int64_t rows, int n);
+/* Elementwise: kind is a CTHIP_ACT_* (plus 4 = sigmoid, 5 = tanh). */
+#define CTHIP_ACT_SIGMOID 4
+#define CTHIP_ACT_TANH 5
+int cthip_unary(int kind, float *y, const float *x, int64_t n);
+/* Embedding (nn/embedding.lisp:3-25): out[t,:] = W[idx[t],:], idx given as
+ * floats as the reference feeds them (apps/gpt2/gpt2.lisp:95).  The reference
+ * sums a one-hot mask over the vocabulary; the result is the same row. */
+int cthip_embedding(float *out, const float *W, const float *idx, int ntok, int vocab, int dim);
+/* ArgMaxNode over the last axis (api/high-level-ops.lisp:314-343): lowest index among ties. */
+int cthip_argmax(int64_t *out, const float *x, int64_t rows, int n);
+/* RoPE (nn/positional-encoding.lisp:3-64) on (B,S,H,Dh), interleaved pairs;
+ * start_pos shifts the positions (0 reproduces the reference). */
+int cthip_rope(float *out, const float *x, int B, int S, int H, int Dh, float base, int start_pos);
+/* scaled-dot-product-attention (external/llm/layers.lisp:3-5) of S query rows
+ * (S,H,Dh) at positions start_pos..start_pos+S-1 against a KV cache laid out
+ * (max_len, Hkv, Dh) (layers.lisp:19-33) holding T = start_pos+S rows, with the
+ * causal mask of layers.lisp:83 applied.  out (S,H,Dh). */
+int cthip_sdpa_cached(float *out, const float *q, const float *k_cache, const float *v_cache,
+                      int S, int start_pos, int H, int Hkv, int Dh);
+
+/* ================================================================== */
+/* Decoder session: Transformer (external/llm/layers.lisp:73-90) and   */
+/* the gpt2-generate loop (apps/gpt2/gpt2.lisp:97-113)                 */
+/* ================================================================== */
+
+#define CTHIP_ARCH_GPT2 0  /* LayerNorm, learned positions, fused qkv + biases, GELU MLP */
+#define CTHIP_ARCH_LLAMA 1 /* RMSNorm, RoPE, GQA, SwiGLU, no biases (not in the reference) */
+
+typedef struct {
+  int arch;
+  int n_layers, dim, n_heads, n_kv_heads, ffn, vocab, max_seq;
+  float eps;
+  float rope_base;
+} cthip_decoder_config;
+
+int cthip_decoder_create(void **dec, const cthip_decoder_config *cfg);
+int cthip_decoder_destroy(void *dec);
+/* load-state-dict (source/api/module.lisp:290-320): hands one tensor to the
+ * session under its reference state-dict key ("wte.weight", "h.3.attn.c_attn.weight",
+ * "h.3.ln_1.affine", "ln_f.bias", "lm_head.weight", ... apps/gpt2/gpt2.lisp:52-70).
+ * `host_raw` are the tensor's GGUF bytes in HOST memory (weights arrive as host
+ * buffers whatever the backend, external/gguf/tensor-info.lisp:104-120); they
+ * are uploaded once and, for 2-D Linear weights, kept packed. */
+int cthip_decoder_load(void *dec, const char *key, int ggml_type, const void *host_raw,
+                       int64_t rows, int64_t cols);
+/* Number of tensors still missing before the session can run. */
+int cthip_decoder_missing(const void *dec);
+/* One `forward` of the compiled graph (apps/gpt2/gpt2.lisp:104): s token ids AS
+ * FLOATS starting at position n.  Writes the greedy token of the last position
+ * to *token; logits_out (host, vocab floats) may be NULL.  Synchronous. */
+int cthip_decoder_forward(void *dec, const float *tokens, int s, int n, int64_t *token,
+                          float *logits_out);
+/* gpt2-generate's loop kept on the device: after a forward has left position
+ * and last token on the device, runs `steps` further single-token forwards
+ * without host round trips and writes their greedy tokens to tokens_out (host).
+ * Synchronous at the end only. */
+int cthip_decoder_generate(void *dec, int steps, int64_t *tokens_out);
+/* Current position (tokens in the KV cache). */
+int cthip_decoder_position(const void *dec);
+/* Bytes of HBM one decode step must read at position t (weights + norms/biases + KV rows). */
+int64_t cthip_decoder_step_bytes(const void *dec, int t);
+/* Device pointers into the session, for parity tests: "k_cache.<l>", "v_cache.<l>", "logits", "x". */
+int cthip_decoder_peek(void *dec, const char *what, void **ptr, int64_t *n_floats);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CATEN_HIP_H */

@@ -1,0 +1,267 @@
+"""GPU parity: every hand-written fused item, called through the C ABI, against the CPU oracle.
+
+Bars (BASELINE north star): bit-exact for dequantised weight values and indices/argmax;
+rtol 1e-3 / atol 1e-4 for fp32 arithmetic.
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-3, 1e-4
+
+
+def close(a, b, rtol=RTOL, atol=ATOL):
+    a = np.asarray(a, np.float64)
+    b = np.asarray(b, np.float64)
+    bad = np.abs(a - b) > atol + rtol * np.abs(b)
+    assert not bad.any(), f"{bad.sum()} of {bad.size} differ; max abs err {np.abs(a - b).max():.3e}"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from caten_amd import _lib, ops as o
+    _lib.init(0)
+    return o
+
+
+def _bits(a):
+    return np.ascontiguousarray(a, np.float32).view(np.uint32)
+
+
+# ------------------------------------------------------------------ codecs
+@pytest.mark.parametrize("n", [32, 64, 40, 1, 31, 33, 32 * 1000 + 7, 768 * 2304])
+def test_dequant_q8_0_bit_exact(ops, oracle, n):
+    print(f"case: q8_0 dequant n={n}", flush=True)
+    rng = np.random.default_rng(n)
+    nb = (n + 31) // 32
+    raw = rng.integers(0, 256, size=nb * 34, dtype=np.uint8)
+    sc = rng.normal(0, 0.01, nb).astype(np.float16)
+    raw.reshape(nb, 34)[:, :2] = sc.view(np.uint8).reshape(nb, 2)
+    got = ops.dequantize("q8_0", raw, n)
+    want = oracle.dequant("q8_0", raw, n)
+    assert np.array_equal(_bits(got), _bits(want))
+
+
+def test_dequant_q8_0_all_scales(ops, oracle):
+    # every finite fp16 scale (incl. denormals) x int8 values
+    scales = np.arange(65536, dtype=np.uint16)
+    scales = scales[np.isfinite(scales.view(np.float16))]
+    nb = scales.size
+    raw = np.empty((nb, 34), np.uint8)
+    raw[:, :2] = scales.view(np.uint8).reshape(nb, 2)
+    q = (np.arange(nb * 32) * 7 % 256).astype(np.uint8)
+    raw[:, 2:] = q.reshape(nb, 32)
+    got = ops.dequantize("q8_0", raw, nb * 32)
+    want = oracle.dequant("q8_0", raw, nb * 32)
+    assert np.array_equal(_bits(got), _bits(want))
+
+
+@pytest.mark.parametrize("n", [32, 64, 32 * 999])
+def test_dequant_q4_0_bit_exact(ops, oracle, n):
+    rng = np.random.default_rng(n)
+    nb = n // 32
+    raw = rng.integers(0, 256, size=nb * 18, dtype=np.uint8)
+    raw.reshape(nb, 18)[:, :2] = rng.normal(0, 0.01, nb).astype(np.float16).view(np.uint8).reshape(nb, 2)
+    assert np.array_equal(_bits(ops.dequantize("q4_0", raw, n)), _bits(oracle.dequant("q4_0", raw, n)))
+
+
+def test_dequant_q4_0_rejects_ragged(ops):
+    from caten_amd import HipError
+    with pytest.raises(HipError):
+        ops.dequantize("q4_0", np.zeros(36, np.uint8), 40)
+
+
+def test_dequant_f16_f32(ops, oracle):
+    bits = np.arange(65536, dtype=np.uint16)
+    got = ops.dequantize("f16", bits.view(np.uint8), 65536)
+    want = oracle.dequant("f16", bits.view(np.uint8), 65536)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan) and np.array_equal(_bits(got[~nan]), _bits(want[~nan]))
+    x = np.random.default_rng(0).normal(size=1001).astype(np.float32)
+    assert np.array_equal(_bits(ops.dequantize("f32", x.view(np.uint8), 1001)), _bits(x))
+
+
+@pytest.mark.parametrize("kind", ["q8_0", "q4_0", "f16", "f32"])
+def test_weight_matrix_planes_keep_values(ops, oracle, kind):
+    from caten_amd.llm import Tensor
+    rng = np.random.default_rng(11)
+    w = rng.normal(0, 0.02, (37, 256)).astype(np.float32)
+    t = Tensor.from_f32(w, kind)
+    wm = ops.WeightMatrix(kind, t.raw, 37, 256)
+    assert wm.nbytes == t.raw.size
+    got = wm.dequantize()
+    want = oracle.dequant(kind, t.raw, w.size).reshape(37, 256)
+    assert np.array_equal(_bits(got), _bits(want))
+
+
+def test_quantisers_match_oracle(oracle):
+    from caten_amd import quant
+    rng = np.random.default_rng(12)
+    w = rng.normal(0, 0.02, 32 * 500).astype(np.float32)
+    w[:32] = 0.0  # an all-zero block
+    for kind in ("q8_0", "q4_0"):
+        assert np.array_equal(quant.quantize(kind, w), oracle.quantize(kind, w))
+
+
+# ------------------------------------------------------------------ Linear / GEMV
+SHAPES = [(768, 768), (2304, 768), (3072, 768), (768, 3072), (5003, 768), (1000, 256), (64, 2048), (96, 5632),
+          (33, 96), (17, 1024), (50257, 768)]
+
+
+@pytest.mark.parametrize("kind", ["q8_0", "q4_0", "f32", "f16"])
+@pytest.mark.parametrize("rows,cols", SHAPES)
+def test_gemv_plain(ops, oracle, kind, rows, cols):
+    if kind in ("f32", "f16") and rows > 6000:
+        pytest.skip("large fp32 case covered by the decoder test")
+    print(f"case: gemv {kind} ({rows},{cols})", flush=True)
+    from caten_amd.llm import Tensor
+    rng = np.random.default_rng(rows * 7 + cols)
+    w = rng.normal(0, 0.02, (rows, cols)).astype(np.float32)
+    x = rng.normal(0, 1, cols).astype(np.float32)
+    t = Tensor.from_f32(w, kind)
+    wd = oracle.dequant(kind, t.raw, w.size).reshape(rows, cols)
+    wm = ops.WeightMatrix(kind, t.raw, rows, cols)
+    close(ops.linear(x, wm), oracle.linear(x, wd))
+
+
+@pytest.mark.parametrize("kind", ["q8_0", "q4_0", "f32"])
+def test_gemv_fused_neighbours(ops, oracle, kind):
+    from caten_amd.llm import Tensor
+    rng = np.random.default_rng(21)
+    rows, cols = 3072, 768
+    w = rng.normal(0, 0.02, (rows, cols)).astype(np.float32)
+    x = rng.normal(0.3, 2, cols).astype(np.float32)
+    b = rng.normal(0, 0.02, rows).astype(np.float32)
+    r = rng.normal(0, 1, rows).astype(np.float32)
+    g = rng.normal(1, 0.02, cols).astype(np.float32)
+    be = rng.normal(0, 0.02, cols).astype(np.float32)
+    t = Tensor.from_f32(w, kind)
+    wd = oracle.dequant(kind, t.raw, w.size).reshape(rows, cols)
+    wm = ops.WeightMatrix(kind, t.raw, rows, cols)
+    # LayerNorm -> Linear + bias -> GELU (items 9+10 of a decode step)
+    want = oracle.gelu_tanh(oracle.linear(oracle.layernorm(x, g, be), wd, b))
+    close(ops.linear(x, wm, bias=b, act="gelu", prologue="layernorm", norm_g=g, norm_b=be), want)
+    # Linear + bias + residual
+    close(ops.linear(x, wm, bias=b, residual=r), oracle.linear(x, wd, b) + r)
+    # RMSNorm -> Linear, ReLU
+    close(ops.linear(x, wm, act="relu", prologue="rmsnorm", norm_g=g), oracle.relu(oracle.linear(oracle.rmsnorm(x, g), wd)))
+    # SwiGLU prologue: silu(gate) * up
+    xx = rng.normal(0, 1, 2 * cols).astype(np.float32)
+    want = oracle.linear(oracle.silu(xx[:cols]) * xx[cols:], wd)
+    close(ops.linear(xx, wm, prologue="swiglu"), want)
+
+
+def test_gemv_fallback_shapes_with_prologue(ops, oracle):
+    from caten_amd.llm import Tensor
+    rng = np.random.default_rng(22)
+    rows, cols = 45, 9984  # no register-resident variant covers 9984 columns of q8_0
+    w = rng.normal(0, 0.02, (rows, cols)).astype(np.float32)
+    x = rng.normal(0, 1, cols).astype(np.float32)
+    g = rng.normal(1, 0.02, cols).astype(np.float32)
+    t = Tensor.from_f32(w, "q8_0")
+    wd = oracle.dequant("q8_0", t.raw, w.size).reshape(rows, cols)
+    wm = ops.WeightMatrix("q8_0", t.raw, rows, cols)
+    close(ops.linear(x, wm, prologue="layernorm", norm_g=g), oracle.linear(oracle.layernorm(x, g), wd))
+
+
+def test_linear_batched_rows(ops, oracle):
+    from caten_amd.llm import Tensor
+    rng = np.random.default_rng(23)
+    rows, cols, m = 300, 768, 5
+    w = rng.normal(0, 0.02, (rows, cols)).astype(np.float32)
+    x = rng.normal(0, 1, (m, cols)).astype(np.float32)
+    b = rng.normal(0, 0.02, rows).astype(np.float32)
+    t = Tensor.from_f32(w, "q8_0")
+    wd = oracle.dequant("q8_0", t.raw, w.size).reshape(rows, cols)
+    wm = ops.WeightMatrix("q8_0", t.raw, rows, cols)
+    close(ops.linear(x, wm, bias=b), oracle.linear(x, wd, b))
+    assert ops.linear(np.zeros((0, cols), np.float32), wm).shape == (0, rows)
+
+
+def test_linear_argument_errors(ops):
+    from caten_amd import HipError
+    with pytest.raises(ValueError):
+        ops.WeightMatrix("q8_0", np.zeros(10, np.uint8), 4, 32)  # wrong byte count
+    with pytest.raises(HipError):
+        ops.WeightMatrix("q8_0", np.zeros(68, np.uint8), 3, 16)  # quantised rows need cols % 32 == 0
+    wm = ops.WeightMatrix("f32", np.zeros(4 * 64, np.uint8), 2, 32)
+    with pytest.raises(ValueError):
+        ops.linear(np.zeros(31, np.float32), wm)
+
+
+# ------------------------------------------------------------------ row ops
+@pytest.mark.parametrize("shape", [(128, 128), (64, 768), (7, 40), (3, 2048), (2, 5000), (5, 1), (300, 36)])
+def test_rowops(ops, oracle, shape):
+    print(f"case: rowops {shape}", flush=True)
+    rng = np.random.default_rng(shape[0] + shape[1])
+    x = rng.normal(0, 1, shape).astype(np.float32)
+    g = rng.normal(1, 0.02, shape[-1]).astype(np.float32)
+    b = rng.normal(0, 0.02, shape[-1]).astype(np.float32)
+    close(ops.softmax(x), oracle.softmax(x), 1e-5, 1e-6)
+    if shape[-1] > 1:
+        close(ops.layernorm(x, g, b), oracle.layernorm(x, g, b), 1e-4, 1e-5)
+        close(ops.layernorm(x), oracle.layernorm(x), 1e-4, 1e-5)
+        close(ops.layernorm_softmax(x, g, b), oracle.softmax(oracle.layernorm(x, g, b)), 1e-4, 1e-6)
+    close(ops.rmsnorm(x, g), oracle.rmsnorm(x, g), 1e-4, 1e-5)
+
+
+def test_softmax_fuzz_large_values(ops, oracle):
+    rng = np.random.default_rng(31)
+    x = rng.normal(10, 100, (512, 512)).astype(np.float32)  # test-activations.lisp:60-73
+    y = ops.softmax(x)
+    close(y, oracle.softmax(x), 1e-5, 1e-5)
+    assert np.allclose(y.sum(-1), 1.0, atol=1e-5)
+
+
+def test_rowops_empty(ops):
+    assert ops.softmax(np.zeros((0, 8), np.float32)).shape == (0, 8)
+    assert ops.layernorm(np.zeros((0, 8), np.float32)).shape == (0, 8)
+
+
+def test_unary(ops, oracle):
+    x = np.linspace(-9, 9, 100003).astype(np.float32)
+    assert np.array_equal(ops.relu(x), oracle.relu(x))
+    close(ops.gelu(x), oracle.gelu_tanh(x), 1e-5, 1e-6)
+    close(ops.silu(x), oracle.silu(x), 1e-5, 1e-6)
+    close(ops.sigmoid(x), oracle.sigmoid(x), 1e-5, 1e-6)
+    close(ops.tanh(x), oracle.tanh(x), 1e-5, 1e-6)
+    assert ops.gelu(np.zeros(0, np.float32)).shape == (0,)
+
+
+def test_embedding_and_argmax(ops, oracle):
+    rng = np.random.default_rng(41)
+    W = rng.normal(size=(523, 48)).astype(np.float32)
+    idx = rng.integers(0, 523, (3, 7)).astype(np.float32)
+    assert np.array_equal(ops.embedding(W, idx), oracle.embedding_onehot(W, idx))
+    # an index that equals no vocabulary row selects nothing in the one-hot sum
+    odd = np.array([1.0, 522.0, 523.0, -1.0, 2.5], np.float32)
+    assert np.array_equal(ops.embedding(W, odd), oracle.embedding_onehot(W, odd))
+    for n in (1, 10, 63, 64, 65, 1024, 50257):
+        x = rng.integers(0, 5, n).astype(np.float32)  # many ties -> lowest index
+        assert ops.argmax(x) == oracle.argmax(x)
+    x = rng.normal(size=(9, 50257)).astype(np.float32)
+    assert np.array_equal(ops.argmax(x), np.array([oracle.argmax(r) for r in x]))
+    assert ops.argmax(np.arange(10, dtype=np.float32)) == 9  # test-ops.lisp:107-114
+
+
+def test_rope(ops, oracle):
+    rng = np.random.default_rng(51)
+    x = rng.uniform(0, 1, (1, 10, 10, 10)).astype(np.float32)
+    close(ops.rope(x), oracle.rope(x), 5e-4, 1e-5)  # test-rope.lisp:58-66
+    x = rng.normal(size=(2, 6, 4, 64)).astype(np.float32)
+    close(ops.rope(x, start_pos=900), oracle.rope(x, start_pos=900), 1e-3, 1e-4)
+
+
+@pytest.mark.parametrize("S,start,H,Hkv,Dh", [(1, 0, 4, 4, 64), (1, 37, 12, 12, 64), (5, 3, 8, 2, 64),
+                                             (1, 700, 4, 1, 128), (3, 0, 2, 2, 32)])
+def test_sdpa_cached(ops, oracle, S, start, H, Hkv, Dh):
+    rng = np.random.default_rng(S + start)
+    T = start + S
+    maxlen = T + 5
+    q = rng.normal(size=(S, H, Dh)).astype(np.float32)
+    k = rng.normal(size=(maxlen, Hkv, Dh)).astype(np.float32)
+    v = rng.normal(size=(maxlen, Hkv, Dh)).astype(np.float32)
+    mask = oracle.triu_neginf(S, T, 1 + start)
+    want = oracle.sdpa(q, np.ascontiguousarray(k[:T]), np.ascontiguousarray(v[:T]), mask)
+    close(ops.sdpa_cached(q, k, v, start), want, 1e-4, 1e-5)

@@ -73,7 +73,18 @@ struct GemvArgs {
   int rows, cols;
   int act, pro;
   int64_t x_stride, y_stride;  // between the m input / output vectors (blockIdx.y)
+  // fused greedy argmax over the output rows (m == 1 only); all null when unused.
+  // am_val/am_idx hold one partial (best value, lowest row) per wavefront of the launch.
+  float *am_val;
+  int *am_idx;
+  long long *am_token64;
+  int *am_tok;
+  int *am_pos;
+  long long *am_hist;
+  int *am_hist_n;
 };
+// most wavefronts any GEMV launch uses (sizes the am_val / am_idx scratch)
+constexpr int kGemvMaxWaves = 16384;
 int launch_gemv(const WMat *w, GemvArgs a, int m);
 int wmat_create_impl(WMat **out, int type, const void *raw, int64_t rows, int64_t cols);
 // true when a register-resident GEMV variant covers the matrix (no temporary is allocated at launch)

@@ -72,6 +72,9 @@ struct Decoder {
   int64_t *token64 = nullptr;
   int64_t *history = nullptr;
   int *hist_n = nullptr;
+  // scratch of the argmax fused behind lm_head: one partial per wavefront
+  float *am_val = nullptr;
+  int *am_idx = nullptr;
   int position = 0;
   bool primed = false;  // a forward has left token/position on the device
   bool use_graph = true;
@@ -247,6 +250,8 @@ static int finalize(Decoder *d) {
   TRY(dev_alloc(d, (void **)&d->token64, 256));
   TRY(dev_alloc(d, (void **)&d->history, sizeof(int64_t) * (size_t)(c.max_seq + 1)));
   TRY(dev_alloc(d, (void **)&d->hist_n, 256));
+  TRY(dev_alloc(d, (void **)&d->am_val, sizeof(float) * kGemvMaxWaves));
+  TRY(dev_alloc(d, (void **)&d->am_idx, sizeof(int) * kGemvMaxWaves));
 
   const char *ng = getenv("CTHIP_NO_GRAPH");
   if (ng && *ng && *ng != '0') d->use_graph = false;
@@ -356,9 +361,15 @@ static int queue_step(Decoder *d, bool with_head) {
     o.y = d->logits;
     o.x_stride = D;
     o.y_stride = V;
-    TRY(launch_gemv(d->lm_head, o, 1));
     // greedy token -> next step's input; position advances (apps/gpt2/gpt2.lisp:105-107)
-    TRY(launch_argmax(d->token64, d->logits, 1, V, d->tokpos, d->tokpos + 1, d->history, d->hist_n));
+    o.am_val = d->am_val;
+    o.am_idx = d->am_idx;
+    o.am_token64 = (long long *)d->token64;
+    o.am_tok = d->tokpos;
+    o.am_pos = d->tokpos + 1;
+    o.am_hist = (long long *)d->history;
+    o.am_hist_n = d->hist_n;
+    TRY(launch_gemv(d->lm_head, o, 1));
   }
 #undef TRY
   return 0;

@@ -188,11 +188,163 @@ __device__ __forceinline__ float chunk_dot<CTHIP_F16>(const uint4 w, float, cons
   return s;
 }
 
-template <int TYPE, int G, int KC>
+// lowest-index argmax merge: (v, i) <- better of (v, i) and (ov, oi)
+__device__ __forceinline__ void argmax_merge(float &v, int &i, float ov, int oi) {
+  if (ov > v || (ov == v && oi < i)) {
+    v = ov;
+    i = oi;
+  }
+}
+
+// Epilogue shared by the GEMV kernels: bias, activation, residual, routing of fused-qkv rows.
+__device__ __forceinline__ float gemv_store(const GemvArgs &a, int m, int row, float acc, int posv, float bias,
+                                            float resid) {
+  float v = acc + bias;
+  v = apply_act(a.act, v);
+  v += resid;
+  float *dst;
+  if (row < a.split1) {
+    dst = a.y + (int64_t)m * a.y_stride + row;
+  } else {
+    const int64_t off = (int64_t)(posv + m) * a.pos_stride;
+    dst = (row < a.split2) ? a.y1 + off + (row - a.split1) : a.y2 + off + (row - a.split2);
+  }
+  *dst = v;
+  return v;
+}
+
+// ArgMaxNode fused behind the last Linear (lm_head): every wavefront publishes the best
+// (value, lowest row) of the rows it produced; k_argmax_finish combines them.  (A single ticket
+// counter instead of a second launch would serialise thousands of same-address atomics.)
+__device__ __forceinline__ void gemv_argmax_tail(const GemvArgs &a, int wave, int lane, float bv, int bi) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) argmax_merge(bv, bi, __shfl_xor(bv, o, 64), __shfl_xor(bi, o, 64));
+  if (lane == 0) {
+    a.am_val[wave] = bv;
+    a.am_idx[wave] = bi;
+  }
+}
+
+// one block: the greedy token goes where the next step's embedding reads it, is appended to the
+// history, and the position advances
+__global__ __launch_bounds__(1024) void k_argmax_finish(GemvArgs a, int nparts) {
+  __shared__ float sv[16];
+  __shared__ int si[16];
+  float bv = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int i = threadIdx.x; i < nparts; i += 1024) argmax_merge(bv, bi, a.am_val[i], a.am_idx[i]);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) argmax_merge(bv, bi, __shfl_xor(bv, o, 64), __shfl_xor(bi, o, 64));
+  if ((threadIdx.x & 63) == 0) {
+    sv[threadIdx.x >> 6] = bv;
+    si[threadIdx.x >> 6] = bi;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int k = 1; k < 16; k++) argmax_merge(bv, bi, sv[k], si[k]);
+    if (bi == 0x7fffffff) bi = 0;  // no comparable value (all NaN)
+    *a.am_token64 = bi;
+    if (a.am_tok) *a.am_tok = bi;
+    if (a.am_hist) {
+      a.am_hist[*a.am_hist_n] = bi;
+      *a.am_hist_n = *a.am_hist_n + 1;
+    }
+    if (a.am_pos) *a.am_pos = *a.am_pos + 1;
+  }
+}
+
+// Block-cooperative prologue: the workgroup normalises (or gates) the input vector ONCE into LDS --
+// every thread owns cols/blockDim elements, the two reductions go wavefront-shuffle then LDS --
+// instead of every wavefront redoing it in registers.  xs must hold a.cols floats.
+__device__ __forceinline__ void coop_prologue(const GemvArgs &a, const float *__restrict__ x, float *xs, float *red) {
+  const int tid = threadIdx.x, nthr = blockDim.x, nw = nthr >> 6;
+  const int n4 = a.cols >> 2;
+  if (a.pro == CTHIP_PRO_SWIGLU) {
+    for (int i = tid; i < n4; i += nthr) {
+      float4 v = ((const float4 *)x)[i];
+      float4 u = ((const float4 *)(x + a.cols))[i];
+      ((float4 *)xs)[i] = make_float4(ct_silu(v.x) * u.x, ct_silu(v.y) * u.y, ct_silu(v.z) * u.z, ct_silu(v.w) * u.w);
+    }
+    __syncthreads();
+    return;
+  }
+  // LayerNorm / RMSNorm; a thread keeps up to 4 float4 in registers, longer vectors re-read x
+  constexpr int KEEP = 4;
+  float4 xv[KEEP], gv[KEEP], bv[KEEP];
+#pragma unroll
+  for (int k = 0; k < KEEP; k++) {
+    const int i = tid + k * nthr;
+    const bool ok = i < n4;
+    xv[k] = ok ? ((const float4 *)x)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+    gv[k] = (ok && a.norm_g) ? ((const float4 *)a.norm_g)[i] : make_float4(1.f, 1.f, 1.f, 1.f);
+    bv[k] = (ok && a.norm_b) ? ((const float4 *)a.norm_b)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+  const bool fits = n4 <= KEEP * nthr;
+  const float inv_n = 1.0f / (float)a.cols;
+  auto block_sum = [&](float v) {
+    v = wave_sum(v);
+    __syncthreads();
+    if ((tid & 63) == 0) red[tid >> 6] = v;
+    __syncthreads();
+    float t = 0.0f;
+    for (int w = 0; w < nw; w++) t += red[w];
+    return t;
+  };
+  float mean = 0.0f;
+  if (a.pro == CTHIP_PRO_LAYERNORM) {
+    float s = 0.0f;
+#pragma unroll
+    for (int k = 0; k < KEEP; k++) s += (xv[k].x + xv[k].y) + (xv[k].z + xv[k].w);
+    if (!fits)
+      for (int i = tid + KEEP * nthr; i < n4; i += nthr) {
+        float4 v = ((const float4 *)x)[i];
+        s += (v.x + v.y) + (v.z + v.w);
+      }
+    mean = block_sum(s) * inv_n;
+  }
+  float q = 0.0f;
+#pragma unroll
+  for (int k = 0; k < KEEP; k++) {
+    if (tid + k * nthr < n4) {
+      xv[k].x -= mean; xv[k].y -= mean; xv[k].z -= mean; xv[k].w -= mean;
+      q = fmaf(xv[k].x, xv[k].x, q); q = fmaf(xv[k].y, xv[k].y, q);
+      q = fmaf(xv[k].z, xv[k].z, q); q = fmaf(xv[k].w, xv[k].w, q);
+    }
+  }
+  if (!fits)
+    for (int i = tid + KEEP * nthr; i < n4; i += nthr) {
+      float4 v = ((const float4 *)x)[i];
+      v.x -= mean; v.y -= mean; v.z -= mean; v.w -= mean;
+      q = fmaf(v.x, v.x, q); q = fmaf(v.y, v.y, q); q = fmaf(v.z, v.z, q); q = fmaf(v.w, v.w, q);
+    }
+  const float rstd = 1.0f / sqrtf(block_sum(q) * inv_n + a.eps);
+#pragma unroll
+  for (int k = 0; k < KEEP; k++) {
+    const int i = tid + k * nthr;
+    if (i < n4)
+      ((float4 *)xs)[i] = make_float4(xv[k].x * rstd * gv[k].x + bv[k].x, xv[k].y * rstd * gv[k].y + bv[k].y,
+                                      xv[k].z * rstd * gv[k].z + bv[k].z, xv[k].w * rstd * gv[k].w + bv[k].w);
+  }
+  if (!fits)
+    for (int i = tid + KEEP * nthr; i < n4; i += nthr) {
+      float4 v = ((const float4 *)x)[i];
+      float4 gg = a.norm_g ? ((const float4 *)a.norm_g)[i] : make_float4(1.f, 1.f, 1.f, 1.f);
+      float4 bb = a.norm_b ? ((const float4 *)a.norm_b)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+      ((float4 *)xs)[i] = make_float4((v.x - mean) * rstd * gg.x + bb.x, (v.y - mean) * rstd * gg.y + bb.y,
+                                      (v.z - mean) * rstd * gg.z + bb.z, (v.w - mean) * rstd * gg.w + bb.w);
+    }
+  __syncthreads();
+}
+
+// PD = weight tiles a wavefront keeps in flight: 1 for the small, latency-bound launches (one tile
+// per wavefront), 4 for the large ones, whose throughput is bytes-in-flight / memory latency.
+template <int TYPE, int G, int KC, int PD>
 __global__ __launch_bounds__(256) void k_gemv(GemvArgs a) {
   constexpr int XPC = Fmt<TYPE>::XPC;
   constexpr int RPW = 64 / G;  // rows per wavefront per iteration
   constexpr bool QUANT = (TYPE == CTHIP_Q8_0 || TYPE == CTHIP_Q4_0);
+  extern __shared__ float xs_lds[];  // a.cols floats when a prologue is fused
+  __shared__ float red[4];
   const int lane = threadIdx.x & 63;
   const int g = lane / G, l = lane % G;
   const int waves_per_block = blockDim.x >> 6;
@@ -201,90 +353,17 @@ __global__ __launch_bounds__(256) void k_gemv(GemvArgs a) {
   const int nchunks = a.cols / XPC;
   const int m = blockIdx.y;
   const float *__restrict__ x = a.x + (int64_t)m * a.x_stride;
-
-  // ---- input slice -> registers, with the fused prologue ----
-  float xr[KC][XPC];
-  float xs[KC];
-#pragma unroll
-  for (int j = 0; j < KC; j++) {
-    const int c = l + G * j;
-    const bool ok = c < nchunks;
-#pragma unroll
-    for (int t = 0; t < XPC / 4; t++) {
-      float4 v = ok ? *(const float4 *)(x + (int64_t)c * XPC + 4 * t) : make_float4(0.f, 0.f, 0.f, 0.f);
-      if (a.pro == CTHIP_PRO_SWIGLU && ok) {
-        float4 u = *(const float4 *)(x + a.cols + (int64_t)c * XPC + 4 * t);
-        v.x = ct_silu(v.x) * u.x;
-        v.y = ct_silu(v.y) * u.y;
-        v.z = ct_silu(v.z) * u.z;
-        v.w = ct_silu(v.w) * u.w;
-      }
-      xr[j][4 * t + 0] = v.x;
-      xr[j][4 * t + 1] = v.y;
-      xr[j][4 * t + 2] = v.z;
-      xr[j][4 * t + 3] = v.w;
-    }
-  }
-  if (a.pro == CTHIP_PRO_LAYERNORM || a.pro == CTHIP_PRO_RMSNORM) {
-    const float inv_n = 1.0f / (float)a.cols;
-    float mean = 0.0f;
-    if (a.pro == CTHIP_PRO_LAYERNORM) {
-      float s = 0.0f;
-#pragma unroll
-      for (int j = 0; j < KC; j++)
-#pragma unroll
-        for (int e = 0; e < XPC; e++) s += xr[j][e];
-      mean = group_sum<G>(s) * inv_n;
-    }
-    float v = 0.0f;
-#pragma unroll
-    for (int j = 0; j < KC; j++) {
-      const bool ok = (l + G * j) < nchunks;
-#pragma unroll
-      for (int e = 0; e < XPC; e++) {
-        float dlt = ok ? xr[j][e] - mean : 0.0f;
-        xr[j][e] = dlt;
-        v = fmaf(dlt, dlt, v);
-      }
-    }
-    const float rstd = 1.0f / sqrtf(group_sum<G>(v) * inv_n + a.eps);
-#pragma unroll
-    for (int j = 0; j < KC; j++) {
-      const int c = l + G * j;
-      if (c < nchunks) {
-#pragma unroll
-        for (int t = 0; t < XPC / 4; t++) {
-          float4 gm = a.norm_g ? *(const float4 *)(a.norm_g + (int64_t)c * XPC + 4 * t) : make_float4(1.f, 1.f, 1.f, 1.f);
-          float4 bt = a.norm_b ? *(const float4 *)(a.norm_b + (int64_t)c * XPC + 4 * t) : make_float4(0.f, 0.f, 0.f, 0.f);
-          xr[j][4 * t + 0] = xr[j][4 * t + 0] * rstd * gm.x + bt.x;
-          xr[j][4 * t + 1] = xr[j][4 * t + 1] * rstd * gm.y + bt.y;
-          xr[j][4 * t + 2] = xr[j][4 * t + 2] * rstd * gm.z + bt.z;
-          xr[j][4 * t + 3] = xr[j][4 * t + 3] * rstd * gm.w + bt.w;
-        }
-      }
-    }
-  }
-#pragma unroll
-  for (int j = 0; j < KC; j++) {
-    float s = 0.0f;
-    if (TYPE == CTHIP_Q4_0) {
-#pragma unroll
-      for (int e = 0; e < XPC; e++) s += xr[j][e];
-    }
-    xs[j] = s;
-  }
-
-  // ---- stream the rows ----
   const uint4 *__restrict__ qp = (const uint4 *)a.q;
-  const int64_t row_chunks = nchunks;            // 16-byte chunks per row in the quant plane
+  const int64_t row_chunks = nchunks;  // 16-byte chunks per row in the quant plane
   const int scales_per_row = a.cols >> 5;
   const int nrq = (a.rows + RPW - 1) / RPW;
 
-  uint4 wc[KC];
-  unsigned short sc[KC];
-  auto load = [&](int rq, uint4 *w, unsigned short *s) {
+  auto load = [&](int rq, uint4 *w, unsigned short *s, float &bias, float &resid) {
     const int row = rq * RPW + g;
     const bool rok = row < a.rows;
+    // the epilogue operands of the row travel with its weights
+    bias = (rok && a.bias) ? a.bias[row] : 0.0f;
+    resid = (rok && a.residual) ? a.residual[(int64_t)m * a.y_stride + row] : 0.0f;
 #pragma unroll
     for (int j = 0; j < KC; j++) {
       const int c = l + G * j;
@@ -297,44 +376,72 @@ __global__ __launch_bounds__(256) void k_gemv(GemvArgs a) {
     }
   };
 
-  int rq = wave;
-  if (rq < nrq) load(rq, wc, sc);
-  while (rq < nrq) {
-    const int rqn = rq + total_waves;
-    uint4 wn[KC];
-    unsigned short sn[KC];
-    if (rqn < nrq) load(rqn, wn, sn);
-    float acc = 0.0f;
+  // Everything this wavefront needs from memory is requested before any arithmetic so the
+  // latencies overlap: position, the first weight tiles, then the input vector.
+  const int posv = a.pos ? a.pos[0] : 0;
+  uint4 wt[PD][KC];
+  unsigned short st[PD][KC];
+  float bias_t[PD], resid_t[PD];
 #pragma unroll
-    for (int j = 0; j < KC; j++) {
-      const float scale = QUANT ? half_bits_to_float(sc[j]) : 1.0f;
-      acc += chunk_dot<TYPE>(wc[j], scale, xr[j], xs[j]);
-    }
-    acc = group_sum<G>(acc);
-    const int row = rq * RPW + g;
-    if (l == 0 && row < a.rows) {
-      float v = acc;
-      if (a.bias) v += a.bias[row];
-      v = apply_act(a.act, v);
-      if (a.residual) v += a.residual[(int64_t)m * a.y_stride + row];
-      float *dst;
-      if (row < a.split1) {
-        dst = a.y + (int64_t)m * a.y_stride + row;
-      } else {
-        const int64_t off = (int64_t)(a.pos ? a.pos[0] + m : m) * a.pos_stride;
-        dst = (row < a.split2) ? a.y1 + off + (row - a.split1) : a.y2 + off + (row - a.split2);
-      }
-      *dst = v;
-    }
-    if (rqn < nrq) {
-#pragma unroll
-      for (int j = 0; j < KC; j++) {
-        wc[j] = wn[j];
-        sc[j] = sn[j];
-      }
-    }
-    rq = rqn;
+  for (int p = 0; p < PD; p++) {
+    bias_t[p] = resid_t[p] = 0.0f;
+    const int rq = wave + p * total_waves;
+    if (rq < nrq) load(rq, wt[p], st[p], bias_t[p], resid_t[p]);
   }
+
+  float xr[KC][XPC];
+  float xs[KC];
+  if (a.pro != CTHIP_PRO_NONE) coop_prologue(a, x, xs_lds, red);
+  const float *__restrict__ xsrc = (a.pro != CTHIP_PRO_NONE) ? xs_lds : x;
+#pragma unroll
+  for (int j = 0; j < KC; j++) {
+    const int c = l + G * j;
+    const bool ok = c < nchunks;
+#pragma unroll
+    for (int t = 0; t < XPC / 4; t++) {
+      float4 v = ok ? *(const float4 *)(xsrc + (int64_t)c * XPC + 4 * t) : make_float4(0.f, 0.f, 0.f, 0.f);
+      xr[j][4 * t + 0] = v.x;
+      xr[j][4 * t + 1] = v.y;
+      xr[j][4 * t + 2] = v.z;
+      xr[j][4 * t + 3] = v.w;
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < KC; j++) {
+    float s = 0.0f;
+    if (TYPE == CTHIP_Q4_0) {
+#pragma unroll
+      for (int e = 0; e < XPC; e++) s += xr[j][e];
+    }
+    xs[j] = s;
+  }
+
+  // ---- stream the rows: slot p of the ring holds tile base + p*total_waves ----
+  float best_v = -INFINITY;
+  int best_i = 0x7fffffff;
+  for (int base = wave; base < nrq; base += PD * total_waves) {
+#pragma unroll
+    for (int p = 0; p < PD; p++) {
+      const int rq = base + p * total_waves;
+      if (rq < nrq) {  // wavefront-uniform
+        float acc = 0.0f;
+#pragma unroll
+        for (int j = 0; j < KC; j++) {
+          const float scale = QUANT ? half_bits_to_float(st[p][j]) : 1.0f;
+          acc += chunk_dot<TYPE>(wt[p][j], scale, xr[j], xs[j]);
+        }
+        acc = group_sum<G>(acc);
+        const int row = rq * RPW + g;
+        if (l == 0 && row < a.rows) {
+          const float v = gemv_store(a, m, row, acc, posv, bias_t[p], resid_t[p]);
+          argmax_merge(best_v, best_i, v, row);
+        }
+        const int nxt = rq + PD * total_waves;
+        if (nxt < nrq) load(nxt, wt[p], st[p], bias_t[p], resid_t[p]);
+      }
+    }
+  }
+  if (a.am_val) gemv_argmax_tail(a, wave, lane, best_v, best_i);
 }
 
 // Fallback for shapes no (G,KC) instantiation covers: one wavefront per row, the
@@ -350,6 +457,9 @@ __global__ __launch_bounds__(256) void k_gemv_generic(GemvArgs a) {
   const int m = blockIdx.y;
   const float *__restrict__ x = a.x + (int64_t)m * a.x_stride;
   const uint4 *__restrict__ qp = (const uint4 *)a.q;
+  const int posv = a.pos ? a.pos[0] : 0;
+  float best_v = -INFINITY;
+  int best_i = 0x7fffffff;
   for (int row = wave; row < a.rows; row += total_waves) {
     float acc = 0.0f;
     for (int c = lane; c < nchunks; c += 64) {
@@ -370,20 +480,12 @@ __global__ __launch_bounds__(256) void k_gemv_generic(GemvArgs a) {
     }
     acc = wave_sum(acc);
     if (lane == 0) {
-      float v = acc;
-      if (a.bias) v += a.bias[row];
-      v = apply_act(a.act, v);
-      if (a.residual) v += a.residual[(int64_t)m * a.y_stride + row];
-      float *dst;
-      if (row < a.split1) {
-        dst = a.y + (int64_t)m * a.y_stride + row;
-      } else {
-        const int64_t off = (int64_t)(a.pos ? a.pos[0] + m : m) * a.pos_stride;
-        dst = (row < a.split2) ? a.y1 + off + (row - a.split1) : a.y2 + off + (row - a.split2);
-      }
-      *dst = v;
+      const float v = gemv_store(a, m, row, acc, posv, a.bias ? a.bias[row] : 0.0f,
+                                 a.residual ? a.residual[(int64_t)m * a.y_stride + row] : 0.0f);
+      argmax_merge(best_v, best_i, v, row);
     }
   }
+  if (a.am_val) gemv_argmax_tail(a, wave, lane, best_v, best_i);
 }
 
 // prologue as a kernel of its own, for the generic fallback: one block per input vector
@@ -429,9 +531,11 @@ __global__ __launch_bounds__(256) void k_prologue(float *__restrict__ out, const
 typedef void (*gemv_fn)(GemvArgs);
 struct GemvVariant {
   int type, G, KC;
-  gemv_fn fn;
+  gemv_fn fn;       // large launches
+  gemv_fn fn_small; // small, latency-bound launches
 };
-#define V(T, G, KC) {T, G, KC, k_gemv<T, G, KC>}
+// large launches keep about 12 sixteen-byte loads per lane in flight
+#define V(T, G, KC) {T, G, KC, k_gemv<T, G, KC, (KC >= 12 ? 1 : KC >= 6 ? 2 : 4)>, k_gemv<T, G, KC, 1>}
 static const GemvVariant kVariants[] = {
     V(CTHIP_Q8_0, 16, 1), V(CTHIP_Q8_0, 16, 2), V(CTHIP_Q8_0, 16, 3), V(CTHIP_Q8_0, 16, 4),
     V(CTHIP_Q8_0, 32, 3), V(CTHIP_Q8_0, 32, 4), V(CTHIP_Q8_0, 64, 3), V(CTHIP_Q8_0, 64, 4),
@@ -481,22 +585,51 @@ int launch_gemv(const WMat *w, GemvArgs a, int m) {
   a.rows = (int)w->rows;
   a.cols = (int)w->cols;
   if (a.split1 <= 0) a.split1 = a.split2 = a.rows;
+  if (a.am_val && m != 1) return fail(CTHIP_E_BAD_ARG, "gemv: the fused argmax needs m == 1");
   const GemvVariant *v = pick_variant(w->type, a.cols);
   if (v) {
     const int rpw = 64 / v->G;
     const int nrq = (a.rows + rpw - 1) / rpw;
     dim3 grid, block;
-    if (nrq <= 2048) {
-      block = dim3(64);
-      grid = dim3(nrq, m);
+    const bool small = nrq <= 2048;
+    const size_t lds = a.pro != CTHIP_PRO_NONE ? sizeof(float) * (size_t)a.cols : 0;
+    if (lds > 64 * 1024) return fail(CTHIP_E_UNSUPPORTED, "gemv: %d input features exceed the LDS prologue buffer", a.cols);
+    if (small) {
+      // small matrices are pure latency: one tile per wavefront.  Without a prologue, one wavefront
+      // per workgroup spreads the tiles over as many compute units as possible; with one, four
+      // wavefronts share the normalised input through LDS.
+      if (a.pro == CTHIP_PRO_NONE) {
+        block = dim3(64);
+        grid = dim3(nrq, m);
+      } else {
+        block = dim3(256);
+        grid = dim3((nrq + 3) / 4, m);
+      }
     } else {
+      // large matrices: as many resident wavefronts as the register budget allows, every one
+      // looping over the same number of tiles (an uneven last pass would idle most of the chip)
+      static int occ_cache[sizeof(kVariants) / sizeof(kVariants[0])];
+      const int vi = (int)(v - kVariants);
+      if (occ_cache[vi] == 0) {
+        int nb = 0;
+        CTHIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, v->fn, 256, 16 * 1024));
+        occ_cache[vi] = nb > 0 ? nb : 1;
+      }
       block = dim3(256);
-      int blocks = (nrq + 3) / 4;
-      int cap = s.compute_units * 4;
-      grid = dim3(blocks < cap ? blocks : cap, m);
+      const int capacity = s.compute_units * occ_cache[vi] * 4;
+      const int iters = (nrq + capacity - 1) / capacity;
+      const int waves = (nrq + iters - 1) / iters;
+      grid = dim3((waves + 3) / 4, m);
     }
-    hipLaunchKernelGGL(v->fn, grid, block, 0, s.stream, a);
+    const int nwaves = (int)(grid.x * (block.x / 64));
+    if (a.am_val && nwaves > kGemvMaxWaves)
+      return fail(CTHIP_E_UNSUPPORTED, "gemv: %d wavefronts exceed the argmax scratch", nwaves);
+    hipLaunchKernelGGL(small ? v->fn_small : v->fn, grid, block, lds, s.stream, a);
     CTHIP_LAUNCH_CHECK();
+    if (a.am_val) {
+      hipLaunchKernelGGL(k_argmax_finish, dim3(1), dim3(1024), 0, s.stream, a, nwaves);
+      CTHIP_LAUNCH_CHECK();
+    }
     return 0;
   }
   // generic path: prologue into a temporary, then wave-per-row
@@ -513,6 +646,7 @@ int launch_gemv(const WMat *w, GemvArgs a, int m) {
   }
   int blocks = (a.rows + 3) / 4;
   int cap = s.compute_units * 8;
+  if (cap * 4 > kGemvMaxWaves) cap = kGemvMaxWaves / 4;
   dim3 grid(blocks < cap ? blocks : cap, m), block(256);
   switch (w->type) {
     case CTHIP_Q8_0: hipLaunchKernelGGL(k_gemv_generic<CTHIP_Q8_0>, grid, block, 0, s.stream, a); break;
@@ -521,6 +655,10 @@ int launch_gemv(const WMat *w, GemvArgs a, int m) {
     default: hipLaunchKernelGGL(k_gemv_generic<CTHIP_F32>, grid, block, 0, s.stream, a); break;
   }
   CTHIP_LAUNCH_CHECK();
+  if (a.am_val) {
+    hipLaunchKernelGGL(k_argmax_finish, dim3(1), dim3(1024), 0, s.stream, a, (int)(grid.x * 4));
+    CTHIP_LAUNCH_CHECK();
+  }
   if (tmp) return cthip_free(tmp);
   return 0;
 }

@@ -331,81 +331,119 @@ __global__ __launch_bounds__(256) void k_rope_append(float *__restrict__ kc, flo
 }
 
 // ------------------------------------------------------------------ attention over the KV cache
-// One 256-thread block per (query head h, query row i).  Keys 0..T-1 with T = pos+i+1 (causal mask of
-// layers.lisp:83).  Scores live in LDS (max_seq floats).  K/V cache layout (max_len, Hkv, Dh).
+// One 1024-thread block per (query head h, query row i); keys 0..T-1 with T = pos+i+1 (the causal
+// mask of layers.lisp:83 is implicit).  K/V cache layout (max_len, Hkv, Dh).
+//
+// A key row is read by DH/4 adjacent lanes as one float4 each (coalesced 16*DH/4 bytes), so the block
+// covers 1024/(DH/4) keys per pass and every thread holds KPT keys of a tile in registers.  K and V of a
+// tile are requested together, before any arithmetic, so a tile costs one memory latency; tiles are
+// combined with the running-max rescaling of an online softmax.  Partial outputs are reduced with
+// shuffles inside a wavefront and through LDS across the 16 wavefronts.
 template <int DH>
-__global__ __launch_bounds__(256) void k_attn_cached(float *__restrict__ out, const float *__restrict__ q,
-                                                     const float *__restrict__ kc, const float *__restrict__ vc,
-                                                     int start_pos, const int *__restrict__ pos, int H, int Hkv) {
-  extern __shared__ float sc[];  // T scores, then 4 + (256/DH)*DH floats of scratch
-  __shared__ float red[4];
-  __shared__ float qs[DH];
+__global__ __launch_bounds__(1024) void k_attn_cached(float *__restrict__ out, const float *__restrict__ q,
+                                                      const float *__restrict__ kc, const float *__restrict__ vc,
+                                                      int start_pos, const int *__restrict__ pos, int H, int Hkv) {
+  constexpr int LPK = DH / 4;      // lanes per key
+  constexpr int NG = 1024 / LPK;   // keys per pass
+  constexpr int KPT = 8;           // keys per thread per tile
+  constexpr int TILE = NG * KPT;
+  __shared__ float red[16];
+  __shared__ float part[16][DH];
   const int h = blockIdx.x, i = blockIdx.y;
   const int T = start_pos + (pos ? pos[0] : 0) + i + 1;
   const int hk = h / (H / Hkv);
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int g = tid / LPK, c = tid % LPK;
   const int64_t kv_stride = (int64_t)Hkv * DH;
-  if (tid < DH) qs[tid] = q[((int64_t)i * H + h) * DH + tid];
-  __syncthreads();
-  // scores: one key per thread
-  float lmax = -INFINITY;
-  for (int j = tid; j < T; j += 256) {
-    const float4 *kp = (const float4 *)(kc + j * kv_stride + (int64_t)hk * DH);
-    float acc = 0.0f;
+  const float4 q4 = *(const float4 *)(q + ((int64_t)i * H + h) * DH + 4 * c);
+  const float4 *__restrict__ kp = (const float4 *)(kc + (int64_t)hk * DH) + c;
+  const float4 *__restrict__ vp = (const float4 *)(vc + (int64_t)hk * DH) + c;
+  const float scale = 1.0f / sqrtf((float)DH);
+  float m = -INFINITY, l = 0.0f;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int t0 = 0; t0 < T; t0 += TILE) {
+    float4 kr[KPT], vr[KPT];
 #pragma unroll
-    for (int d = 0; d < DH / 4; d++) {
-      float4 kk = kp[d];
-      acc = fmaf(qs[4 * d + 0], kk.x, acc);
-      acc = fmaf(qs[4 * d + 1], kk.y, acc);
-      acc = fmaf(qs[4 * d + 2], kk.z, acc);
-      acc = fmaf(qs[4 * d + 3], kk.w, acc);
+    for (int u = 0; u < KPT; u++) {
+      const int j = t0 + g + NG * u;
+      const bool ok = j < T;
+      kr[u] = ok ? kp[j * (kv_stride / 4)] : make_float4(0.f, 0.f, 0.f, 0.f);
+      vr[u] = ok ? vp[j * (kv_stride / 4)] : make_float4(0.f, 0.f, 0.f, 0.f);
     }
-    acc = acc / sqrtf((float)DH);
-    sc[j] = acc;
-    lmax = fmaxf(lmax, acc);
+    float sc[KPT];
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < KPT; u++) {
+      float d = q4.x * kr[u].x;
+      d = fmaf(q4.y, kr[u].y, d);
+      d = fmaf(q4.z, kr[u].z, d);
+      d = fmaf(q4.w, kr[u].w, d);
+#pragma unroll
+      for (int o = LPK / 2; o > 0; o >>= 1) d += __shfl_xor(d, o, 64);
+      const bool ok = (t0 + g + NG * u) < T;
+      sc[u] = ok ? d * scale : -INFINITY;
+      tmax = fmaxf(tmax, sc[u]);
+    }
+    tmax = wave_max(tmax);
+    __syncthreads();  // previous users of red[] are done
+    if (lane == 0) red[wv] = tmax;
+    __syncthreads();
+    float mt = red[0];
+#pragma unroll
+    for (int w = 1; w < 16; w++) mt = fmaxf(mt, red[w]);
+    const float m_new = fmaxf(m, mt);
+    const float corr = ct_exp(m - m_new);  // 0 on the first tile (m = -inf)
+    float ps = 0.0f;
+#pragma unroll
+    for (int k2 = 0; k2 < 4; k2++) acc[k2] *= corr;
+#pragma unroll
+    for (int u = 0; u < KPT; u++) {
+      const float p = ct_exp(sc[u] - m_new);  // exp2(-inf) = 0 for masked keys
+      if (c == 0) ps += p;
+      acc[0] = fmaf(p, vr[u].x, acc[0]);
+      acc[1] = fmaf(p, vr[u].y, acc[1]);
+      acc[2] = fmaf(p, vr[u].z, acc[2]);
+      acc[3] = fmaf(p, vr[u].w, acc[3]);
+    }
+    ps = wave_sum(ps);
+    __syncthreads();
+    if (lane == 0) red[wv] = ps;
+    __syncthreads();
+    float st = 0.0f;
+#pragma unroll
+    for (int w = 0; w < 16; w++) st += red[w];
+    l = l * corr + st;
+    m = m_new;
   }
-  lmax = wave_max(lmax);
-  if ((tid & 63) == 0) red[tid >> 6] = lmax;
-  __syncthreads();
-  const float m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-  __syncthreads();
-  float lsum = 0.0f;
-  for (int j = tid; j < T; j += 256) {
-    float e = ct_exp(sc[j] - m);
-    sc[j] = e;
-    lsum += e;
+  // combine the key groups: inside the wavefront by shuffles, across wavefronts through LDS
+#pragma unroll
+  for (int o = LPK; o < 64; o <<= 1) {
+#pragma unroll
+    for (int k2 = 0; k2 < 4; k2++) acc[k2] += __shfl_xor(acc[k2], o, 64);
   }
-  lsum = wave_sum(lsum);
-  if ((tid & 63) == 0) red[tid >> 6] = lsum;
-  __syncthreads();
-  const float inv = 1.0f / (red[0] + red[1] + red[2] + red[3]);
-  // out[d] = sum_j p_j V[j,d]: thread (grp, d) walks keys grp, grp+NG, ...
-  constexpr int NG = 256 / DH;
-  float *part = sc + T;
-  const int d = tid % DH, grp = tid / DH;
-  float acc = 0.0f;
-  for (int j = grp; j < T; j += NG) acc = fmaf(sc[j] * inv, vc[j * kv_stride + (int64_t)hk * DH + d], acc);
-  part[grp * DH + d] = acc;
+  if (lane < LPK) {
+#pragma unroll
+    for (int k2 = 0; k2 < 4; k2++) part[wv][4 * lane + k2] = acc[k2];
+  }
   __syncthreads();
   if (tid < DH) {
     float s = 0.0f;
 #pragma unroll
-    for (int g2 = 0; g2 < NG; g2++) s += part[g2 * DH + tid];
-    out[((int64_t)i * H + h) * DH + tid] = s;
+    for (int w = 0; w < 16; w++) s += part[w][tid];
+    out[((int64_t)i * H + h) * DH + tid] = s / l;
   }
 }
 
 int launch_attn(float *out, const float *q, const float *kc, const float *vc, int S, int start_pos, const int *pos,
                 int max_T, int H, int Hkv, int Dh) {
   if (S == 0) return 0;
+  (void)max_T;
   hipStream_t st = state().stream;
-  const size_t lds = sizeof(float) * ((size_t)max_T + 256);
-  if (lds > 60 * 1024) return fail(CTHIP_E_UNSUPPORTED, "attention: %d cached positions exceed the LDS score buffer", max_T);
-  dim3 grid(H, S), block(256);
+  dim3 grid(H, S), block(1024);
   switch (Dh) {
-    case 32: hipLaunchKernelGGL(k_attn_cached<32>, grid, block, lds, st, out, q, kc, vc, start_pos, pos, H, Hkv); break;
-    case 64: hipLaunchKernelGGL(k_attn_cached<64>, grid, block, lds, st, out, q, kc, vc, start_pos, pos, H, Hkv); break;
-    case 128: hipLaunchKernelGGL(k_attn_cached<128>, grid, block, lds, st, out, q, kc, vc, start_pos, pos, H, Hkv); break;
+    case 32: hipLaunchKernelGGL(k_attn_cached<32>, grid, block, 0, st, out, q, kc, vc, start_pos, pos, H, Hkv); break;
+    case 64: hipLaunchKernelGGL(k_attn_cached<64>, grid, block, 0, st, out, q, kc, vc, start_pos, pos, H, Hkv); break;
+    case 128: hipLaunchKernelGGL(k_attn_cached<128>, grid, block, 0, st, out, q, kc, vc, start_pos, pos, H, Hkv); break;
     default: return fail(CTHIP_E_UNSUPPORTED, "attention: head_dim %d (supported: 32, 64, 128)", Dh);
   }
   CTHIP_LAUNCH_CHECK();

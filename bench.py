@@ -4,9 +4,11 @@
 A "step" is one decode step (one token).  Weights, KV cache, token and position are resident in
 HBM before the timed region; the timed region is K back-to-back steps of the device-resident loop
 (cthip_decoder_generate), bracketed by stream synchronisation, host wall clock.  `roofline` is
-the whole decode step (one hipGraph replay) measured with HIP events on the library's stream:
-algorithmic bytes of a step (packed weights + norms/biases + embedding rows + KV rows) over its
-average duration, against 8 TB/s.  `cpu_baseline` times the CPU oracle (a single-thread C
+the dominant kernel of a step -- the dequant-in-register GEMV, on its largest launch (lm_head,
+50257x768, 31 % of a step's bytes) -- measured with HIP events on the library's stream:
+algorithmic bytes (packed weights + input + output) over the average launch duration, against
+8 TB/s; `roofline.step` gives the same ratio for the whole step (one hipGraph replay: packed
+weights + norms/biases + embedding rows + KV rows).  `cpu_baseline` times the CPU oracle (a single-thread C
 restatement of Caten's BACKEND=CLANG kernels, incl. its one-hot embedding and 3-reduction argmax)
 on the host cores, on a bounded sample of the same workload.
 """
@@ -22,6 +24,9 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+# (profiles/), scaled by a copy kernel of known size; None where it has not been measured.
+TRAFFIC_BYTES = {("gpt2", "q8_0"): 41540414}  # profiles/gemv_q8_0_lm_head_pmc.txt
 
 
 def cpu_baseline(cfg, weights, prompt, budget_s):
@@ -60,7 +65,14 @@ def main():
     ap.add_argument("--kind", default="q8_0")
     ap.add_argument("--prompt", type=int, default=16)
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU baseline budget (0 disables)")
+    ap.add_argument("--no-graph", action="store_true",
+                    help="launch the step's kernels one by one instead of replaying the hipGraph (for kernel tracing)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one 256 MiB device-to-device copy (a kernel of known traffic to scale "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings by)")
     args = ap.parse_args()
+    if args.no_graph:
+        os.environ["CTHIP_NO_GRAPH"] = "1"
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (batch-1 decode does not use a second); run with --gpus 1",
               file=sys.stderr)
@@ -120,7 +132,29 @@ def main():
     _lib.check(lib.cthip_timer_stop(C.byref(ms)))
     step_us = ms.value * 1e3 / k
     step_bytes = float(np.mean([model.step_bytes(t + 1) for t in range(pos0, pos0 + k)]))
-    achieved = step_bytes / (step_us * 1e-6) / 1e9
+    step_gbs = step_bytes / (step_us * 1e-6) / 1e9
+
+    # ---- the dominant kernel on its largest launch: ln_f -> lm_head GEMV (+ per-wavefront argmax partials) ----
+    from caten_amd import ops
+    from caten_amd.llm import Tensor
+    V, D = cfg["vocab"], cfg["dim"]
+    t = Tensor.from_f32(weights["lm_head"], args.kind)
+    wm = ops.WeightMatrix(args.kind, t.raw, V, D)
+    dx = ops.DeviceArray.from_numpy(np.random.default_rng(1).normal(size=D).astype(np.float32))
+    dg = ops.DeviceArray.from_numpy(weights["lnf_g"])
+    db = ops.DeviceArray.from_numpy(weights["lnf_b"])
+    dy = ops.DeviceArray((V,), np.float32)
+    reps = 200
+    for _ in range(20):
+        _lib.check(lib.cthip_linear(dy.ptr, wm.handle, dx.ptr, 1, None, None, 0, _lib.PRO_LAYERNORM, dg.ptr, db.ptr, 1e-5))
+    _lib.check(lib.cthip_sync())
+    _lib.check(lib.cthip_timer_start())
+    for _ in range(reps):
+        _lib.check(lib.cthip_linear(dy.ptr, wm.handle, dx.ptr, 1, None, None, 0, _lib.PRO_LAYERNORM, dg.ptr, db.ptr, 1e-5))
+    _lib.check(lib.cthip_timer_stop(C.byref(ms)))
+    gemv_us = ms.value * 1e3 / reps
+    gemv_bytes = wm.nbytes + 4 * (3 * D + V)  # packed weights + x, gamma, beta + logits
+    achieved = gemv_bytes / (gemv_us * 1e-6) / 1e9
 
     res = {
         "metric": "decode tokens/sec at batch 1 on 1 MI355X; fused-kernel HBM GB/s vs peak",
@@ -132,10 +166,18 @@ def main():
                                f"{args.prompt}-token prompt, batch-1 greedy decode, positions {min(positions)}..{max(positions)}",
                    "model": args.model, "weights": args.kind, "batch": 1},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
-                     "kernel": "one decode step (hipGraph of the fused GEMV/attention/argmax launches)",
-                     "bytes_per_step": step_bytes, "us_per_step": step_us},
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": TRAFFIC_BYTES.get((args.model, args.kind)),
+                     "kernel": f"cthip::k_gemv<{args.kind}> on lm_head ({V}x{D}) with the ln_f prologue",
+                     "bytes_per_launch": gemv_bytes, "us_per_launch": gemv_us,
+                     "step": {"bytes": step_bytes, "us": step_us, "achieved": step_gbs,
+                              "frac": step_gbs / HBM_PEAK_GBS,
+                              "what": "one decode step = one hipGraph replay of every fused launch"}},
     }
+    if args.calibrate_copy:
+        n = 256 << 20
+        a, b = ops.DeviceArray((n,), np.uint8), ops.DeviceArray((n,), np.uint8)
+        _lib.check(lib.cthip_d2d(b.ptr, a.ptr, n))
+        _lib.check(lib.cthip_sync())
     if args.cpu_seconds > 0:
         res["cpu_baseline"] = cpu_baseline(cfg, weights, prompt, args.cpu_seconds)
     model.close()

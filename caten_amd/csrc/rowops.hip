@@ -334,41 +334,43 @@ __global__ __launch_bounds__(256) void k_rope_append(float *__restrict__ kc, flo
 // One 1024-thread block per (query head h, query row i); keys 0..T-1 with T = pos+i+1 (the causal
 // mask of layers.lisp:83 is implicit).  K/V cache layout (max_len, Hkv, Dh).
 //
-// A key row is read by DH/4 adjacent lanes as one float4 each (coalesced 16*DH/4 bytes), so the block
-// covers 1024/(DH/4) keys per pass and every thread holds KPT keys of a tile in registers.  K and V of a
-// tile are requested together, before any arithmetic, so a tile costs one memory latency; tiles are
-// combined with the running-max rescaling of an online softmax.  Partial outputs are reduced with
-// shuffles inside a wavefront and through LDS across the 16 wavefronts.
+// A key row is read by DH/4 adjacent lanes as one float4 each (coalesced 4*DH bytes), so a wavefront
+// covers 64/(DH/4) keys per pass and holds KPT passes of K and V in registers, all requested before
+// any arithmetic.  Every wavefront runs its own online softmax over its keys (shuffles only); the 16
+// per-wavefront partials (max, sum, DH outputs) meet once in LDS, so a block needs one barrier.
 template <int DH>
 __global__ __launch_bounds__(1024) void k_attn_cached(float *__restrict__ out, const float *__restrict__ q,
                                                       const float *__restrict__ kc, const float *__restrict__ vc,
                                                       int start_pos, const int *__restrict__ pos, int H, int Hkv) {
   constexpr int LPK = DH / 4;      // lanes per key
-  constexpr int NG = 1024 / LPK;   // keys per pass
-  constexpr int KPT = 8;           // keys per thread per tile
-  constexpr int TILE = NG * KPT;
-  __shared__ float red[16];
-  __shared__ float part[16][DH];
+  constexpr int KPW = 64 / LPK;    // keys per wavefront per pass
+  constexpr int KPT = 8;           // passes held in registers
+  constexpr int NW = 16;
+  constexpr int TILE = NW * KPW * KPT;
+  __shared__ float part[NW][DH];
+  __shared__ float pm[NW], pl[NW];
   const int h = blockIdx.x, i = blockIdx.y;
   const int T = start_pos + (pos ? pos[0] : 0) + i + 1;
   const int hk = h / (H / Hkv);
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
-  const int g = tid / LPK, c = tid % LPK;
-  const int64_t kv_stride = (int64_t)Hkv * DH;
+  const int g = lane / LPK, c = lane % LPK;
+  const unsigned kvs4 = (unsigned)(Hkv * DH / 4);
   const float4 q4 = *(const float4 *)(q + ((int64_t)i * H + h) * DH + 4 * c);
   const float4 *__restrict__ kp = (const float4 *)(kc + (int64_t)hk * DH) + c;
   const float4 *__restrict__ vp = (const float4 *)(vc + (int64_t)hk * DH) + c;
   const float scale = 1.0f / sqrtf((float)DH);
   float m = -INFINITY, l = 0.0f;
   float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  // wavefront wv owns keys t0 + (wv*KPT + u)*KPW + g
   for (int t0 = 0; t0 < T; t0 += TILE) {
+    if (t0 + wv * KPT * KPW >= T) break;  // nothing left for this wavefront (uniform)
     float4 kr[KPT], vr[KPT];
 #pragma unroll
     for (int u = 0; u < KPT; u++) {
-      const int j = t0 + g + NG * u;
-      const bool ok = j < T;
-      kr[u] = ok ? kp[j * (kv_stride / 4)] : make_float4(0.f, 0.f, 0.f, 0.f);
-      vr[u] = ok ? vp[j * (kv_stride / 4)] : make_float4(0.f, 0.f, 0.f, 0.f);
+      const int j = t0 + (wv * KPT + u) * KPW + g;
+      const unsigned jj = (unsigned)min(j, T - 1);  // clamp: masked below, never out of the cache
+      kr[u] = kp[jj * kvs4];
+      vr[u] = vp[jj * kvs4];
     }
     float sc[KPT];
     float tmax = -INFINITY;
@@ -380,42 +382,32 @@ __global__ __launch_bounds__(1024) void k_attn_cached(float *__restrict__ out, c
       d = fmaf(q4.w, kr[u].w, d);
 #pragma unroll
       for (int o = LPK / 2; o > 0; o >>= 1) d += __shfl_xor(d, o, 64);
-      const bool ok = (t0 + g + NG * u) < T;
+      const bool ok = (t0 + (wv * KPT + u) * KPW + g) < T;
       sc[u] = ok ? d * scale : -INFINITY;
       tmax = fmaxf(tmax, sc[u]);
     }
-    tmax = wave_max(tmax);
-    __syncthreads();  // previous users of red[] are done
-    if (lane == 0) red[wv] = tmax;
-    __syncthreads();
-    float mt = red[0];
 #pragma unroll
-    for (int w = 1; w < 16; w++) mt = fmaxf(mt, red[w]);
-    const float m_new = fmaxf(m, mt);
-    const float corr = ct_exp(m - m_new);  // 0 on the first tile (m = -inf)
+    for (int o = LPK; o < 64; o <<= 1) tmax = fmaxf(tmax, __shfl_xor(tmax, o, 64));
+    const float m_new = fmaxf(m, tmax);   // finite: this wavefront has at least one key here
+    const float corr = ct_exp(m - m_new);  // 0 on its first tile (m = -inf)
     float ps = 0.0f;
 #pragma unroll
     for (int k2 = 0; k2 < 4; k2++) acc[k2] *= corr;
 #pragma unroll
     for (int u = 0; u < KPT; u++) {
       const float p = ct_exp(sc[u] - m_new);  // exp2(-inf) = 0 for masked keys
-      if (c == 0) ps += p;
+      ps += p;
       acc[0] = fmaf(p, vr[u].x, acc[0]);
       acc[1] = fmaf(p, vr[u].y, acc[1]);
       acc[2] = fmaf(p, vr[u].z, acc[2]);
       acc[3] = fmaf(p, vr[u].w, acc[3]);
     }
-    ps = wave_sum(ps);
-    __syncthreads();
-    if (lane == 0) red[wv] = ps;
-    __syncthreads();
-    float st = 0.0f;
 #pragma unroll
-    for (int w = 0; w < 16; w++) st += red[w];
-    l = l * corr + st;
+    for (int o = LPK; o < 64; o <<= 1) ps += __shfl_xor(ps, o, 64);  // every lane of a key holds the same p
+    l = l * corr + ps;
     m = m_new;
   }
-  // combine the key groups: inside the wavefront by shuffles, across wavefronts through LDS
+  // combine the key groups inside the wavefront, then the wavefronts through LDS
 #pragma unroll
   for (int o = LPK; o < 64; o <<= 1) {
 #pragma unroll
@@ -425,12 +417,23 @@ __global__ __launch_bounds__(1024) void k_attn_cached(float *__restrict__ out, c
 #pragma unroll
     for (int k2 = 0; k2 < 4; k2++) part[wv][4 * lane + k2] = acc[k2];
   }
+  if (lane == 0) {
+    pm[wv] = m;
+    pl[wv] = l;
+  }
   __syncthreads();
   if (tid < DH) {
-    float s = 0.0f;
+    float M = pm[0];
 #pragma unroll
-    for (int w = 0; w < 16; w++) s += part[w][tid];
-    out[((int64_t)i * H + h) * DH + tid] = s / l;
+    for (int w = 1; w < NW; w++) M = fmaxf(M, pm[w]);
+    float o = 0.0f, L = 0.0f;
+#pragma unroll
+    for (int w = 0; w < NW; w++) {
+      const float e = ct_exp(pm[w] - M);  // wavefronts without keys hold m = -inf: weight 0
+      o = fmaf(e, part[w][tid], o);
+      L = fmaf(e, pl[w], L);
+    }
+    out[((int64_t)i * H + h) * DH + tid] = o / L;
   }
 }
 

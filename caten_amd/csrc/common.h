@@ -17,6 +17,7 @@ struct State {
   hipStream_t stream = nullptr;
   int compute_units = 0;
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  int gemm_bf16 = 0;  // option "gemm_bf16": round MFMA operands of m > 1 Linear launches to bf16
 };
 State &state();
 void set_error(const char *fmt, ...);
@@ -95,6 +96,9 @@ int launch_embedding(float *out, const float *W, const float *idx_f, const int *
                      const float *W2, const int *pos, int max_pos);
 int launch_argmax(int64_t *out, const float *x, int64_t rows, int n, int *tok_out, int *pos, int64_t *history,
                   int *hist_n);
+// Linear over m rows on the MFMA path (weights dequantised while staged); bf16 rounds the operands.
+int launch_linear_gemm(float *y, const WMat *w, const float *x, int m, const float *bias, const float *residual,
+                       int act, bool bf16);
 int launch_rope_append(float *kc, float *vc, const float *kv, int Hkv, int Dh, float base, const int *pos);
 int launch_rope(float *out, const float *x, int B, int S, int H, int Dh, float base, int start_pos, const int *pos);
 

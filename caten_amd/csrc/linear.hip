@@ -20,6 +20,8 @@
 // wavefront visits, so the steady state touches nothing but weights.  Partial
 // sums are combined with DPP/shuffle steps inside the group and the group's
 // first lane applies the epilogue.
+#include <string.h>
+
 #include "common.h"
 
 namespace cthip {
@@ -779,6 +781,22 @@ int cthip_linear(float *y, const void *wmat, const float *x, int m, const float 
   if (m == 0) return 0;
   if (m > 65535) return fail(CTHIP_E_BAD_ARG, "cthip_linear: m = %d exceeds 65535", m);
   const WMat *w = (const WMat *)wmat;
+  if (m >= 8) {
+    // several input rows: the MFMA tile path reads the weights once instead of once per row
+    const float *xin = x;
+    float *tmp = nullptr;
+    int rc;
+    if (prologue != CTHIP_PRO_NONE) {
+      if ((rc = cthip_alloc((void **)&tmp, sizeof(float) * (size_t)w->cols * m))) return rc;
+      hipLaunchKernelGGL(k_prologue, dim3(m), dim3(256), 0, state().stream, tmp, x, (int)w->cols, prologue, norm_g, norm_b,
+                         eps, (int64_t)(prologue == CTHIP_PRO_SWIGLU ? 2 * w->cols : w->cols));
+      CTHIP_LAUNCH_CHECK();
+      xin = tmp;
+    }
+    rc = launch_linear_gemm(y, w, xin, m, bias, residual, act, state().gemm_bf16 != 0);
+    if (tmp) cthip_free(tmp);
+    return rc;
+  }
   GemvArgs a = {};
   a.y = y;
   a.x = x;
@@ -792,6 +810,15 @@ int cthip_linear(float *y, const void *wmat, const float *x, int m, const float 
   a.x_stride = (prologue == CTHIP_PRO_SWIGLU) ? 2 * w->cols : w->cols;
   a.y_stride = w->rows;
   return launch_gemv(w, a, m);
+}
+
+int cthip_set_option(const char *name, int value) {
+  if (!name) return fail(CTHIP_E_BAD_ARG, "cthip_set_option: null name");
+  if (!strcmp(name, "gemm_bf16")) {
+    state().gemm_bf16 = value != 0;
+    return 0;
+  }
+  return fail(CTHIP_E_BAD_ARG, "cthip_set_option: unknown option '%s'", name);
 }
 
 }  // extern "C"

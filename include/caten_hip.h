@@ -148,10 +148,14 @@ int cthip_wmat_dequant(const void *wmat, float *out);
  *   y[m,:] = act( prologue(x[m,:]) @ W^T + bias ) + residual[m,:]
  * x (m, cols) [(m, 2*cols) for SWIGLU], y/residual (m, rows), fp32, contiguous.
  * norm_g/norm_b/bias/residual may be NULL.  m == 1 is the dequant-in-register
- * GEMV of batch-1 decode; m > 1 uses the tiled path. */
+ * GEMV of batch-1 decode; m >= 8 uses the MFMA tile path (weights dequantised while staged). */
 int cthip_linear(float *y, const void *wmat, const float *x, int m, const float *bias,
                  const float *residual, int act, int prologue, const float *norm_g,
                  const float *norm_b, float eps);
+
+/* Library options.  "gemm_bf16" = 1: Linear launches with m >= 8 input rows (prefill) round their MFMA
+ * operands to bf16 (fp32 accumulation; rtol/atol 1e-2 instead of 1e-3/1e-4).  Default 0. */
+int cthip_set_option(const char *name, int value);
 
 /* !relu(!matmul A B) (api/high-level-ops.lisp:76-99; fused per test-scheduler.lisp:140-163):
  * C (M,N) = act(A (M,K) @ B (K,N)), row-major fp32.  precision 0 = fp32 MFMA

@@ -265,3 +265,61 @@ def test_sdpa_cached(ops, oracle, S, start, H, Hkv, Dh):
     mask = oracle.triu_neginf(S, T, 1 + start)
     want = oracle.sdpa(q, np.ascontiguousarray(k[:T]), np.ascontiguousarray(v[:T]), mask)
     close(ops.sdpa_cached(q, k, v, start), want, 1e-4, 1e-5)
+
+
+# ------------------------------------------------------------------ matmul (MFMA)
+@pytest.mark.parametrize("M,N,K", [(256, 256, 256), (64, 64, 32), (3, 5, 7), (65, 33, 17), (100, 768, 1024), (1, 64, 64)])
+def test_matmul_relu_vs_oracle(ops, oracle, M, N, K):
+    print(f"case: matmul {M}x{N}x{K}", flush=True)
+    rng = np.random.default_rng(M * 31 + N * 7 + K)
+    A = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+    B = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    close(ops.matmul(A, B, relu=True), oracle.matmul(A, B, relu=True))
+    close(ops.matmul(A, B), oracle.matmul(A, B))
+    close(ops.matmul(A, B, relu=True, precision="bf16"), oracle.matmul(A, B, relu=True), 1e-2, 1e-2 * np.sqrt(K))
+
+
+def test_matmul_1024_cubed(ops):
+    # BASELINE config 1: A, B ~ U(-1,1) fp32 (1024,1024); fp64 NumPy is the tie-breaker at this size
+    rng = np.random.default_rng(0)
+    A = rng.uniform(-1, 1, (1024, 1024)).astype(np.float32)
+    B = rng.uniform(-1, 1, (1024, 1024)).astype(np.float32)
+    want = np.maximum(A.astype(np.float64) @ B.astype(np.float64), 0)
+    close(ops.matmul(A, B, relu=True), want)
+    got = ops.matmul(A, B, relu=True, precision="bf16")
+    assert np.max(np.abs(got - want)) < 1e-2 * np.sqrt(1024) and np.all(got >= 0)
+    # all-ones closed form (test-runtime.lisp:241-252): every entry is K
+    assert np.all(ops.matmul(np.ones((64, 96), np.float32), np.ones((96, 32), np.float32)) == 96)
+
+
+def test_matmul_degenerate(ops):
+    assert ops.matmul(np.zeros((0, 8), np.float32), np.zeros((8, 4), np.float32)).shape == (0, 4)
+    assert np.all(ops.matmul(np.zeros((3, 0), np.float32), np.zeros((0, 4), np.float32)) == 0)
+
+
+@pytest.mark.parametrize("kind", ["q8_0", "q4_0", "f16", "f32"])
+def test_linear_prefill_rows_mfma(ops, oracle, kind):
+    # m >= 8 input rows take the MFMA tile path with the weights dequantised while staged
+    from caten_amd import _lib
+    from caten_amd.llm import Tensor
+    rng = np.random.default_rng(61)
+    rows, cols, m = 300, 768, 37
+    w = rng.normal(0, 0.02, (rows, cols)).astype(np.float32)
+    x = rng.normal(0, 1, (m, cols)).astype(np.float32)
+    b = rng.normal(0, 0.02, rows).astype(np.float32)
+    r = rng.normal(0, 1, (m, rows)).astype(np.float32)
+    g = rng.normal(1, 0.02, cols).astype(np.float32)
+    be = rng.normal(0, 0.02, cols).astype(np.float32)
+    t = Tensor.from_f32(w, kind)
+    wd = oracle.dequant(kind, t.raw, w.size).reshape(rows, cols)
+    wm = ops.WeightMatrix(kind, t.raw, rows, cols)
+    close(ops.linear(x, wm, bias=b, residual=r), oracle.linear(x, wd, b) + r)
+    want = oracle.gelu_tanh(oracle.linear(oracle.layernorm(x, g, be), wd, b))
+    close(ops.linear(x, wm, bias=b, act="gelu", prologue="layernorm", norm_g=g, norm_b=be), want)
+    _lib.check(_lib.load().cthip_set_option(b"gemm_bf16", 1))
+    try:
+        close(ops.linear(x, wm, bias=b, residual=r), oracle.linear(x, wd, b) + r, 1e-2, 1e-2)
+    finally:
+        _lib.check(_lib.load().cthip_set_option(b"gemm_bf16", 0))
+    with pytest.raises(_lib.HipError):
+        _lib.check(_lib.load().cthip_set_option(b"no_such_option", 1))

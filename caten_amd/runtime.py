@@ -16,6 +16,7 @@ from __future__ import annotations
 import ctypes as C
 import os
 import time
+import weakref
 from dataclasses import dataclass, field
 from typing import Any, Callable, Dict, List, Optional, Sequence
 
@@ -228,7 +229,15 @@ class HipRuntime(GraphRuntime):
             open_buffer(self, dev)
             transfer_from_array(self, dev, np.asarray(buf.value))
             self._uploaded[key] = dev
+            # the device copy lives exactly as long as the host buffer it mirrors (an id may be
+            # reused once that object is collected)
+            weakref.finalize(buf, self._drop_upload, key)
         return self._uploaded[key]
+
+    def _drop_upload(self, key):
+        dev = self._uploaded.pop(key, None)
+        if dev is not None:
+            close_buffer(self, dev)
 
     def sync(self):
         _lib.check(self.lib.cthip_sync())

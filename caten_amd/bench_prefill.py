@@ -1,0 +1,42 @@
+"""Prefill timing on one MI355X (`python -m caten_amd.bench_prefill`): a 512-token prompt through the
+GPT-2-small shaped Q8_0 model as one batch (BASELINE config 4's prefill leg): MFMA GEMMs over the
+rows with the weights dequantised while staged.  Reports the wall time of `forward` (synchronous) and
+the linear-layer FLOP rate against the MFMA peak of the operand type."""
+from __future__ import annotations
+
+import json
+import time
+
+import numpy as np
+
+from . import _lib, llm, synth
+
+
+def main(model="gpt2", kind="q8_0", s=512):
+    cfg = synth.GPT2_CONFIGS[model]
+    w = synth.gpt2_weights(cfg, seed=0)
+    prompt = [float(t) for t in synth.prompt(cfg["vocab"], s, seed=0)]
+    lib = _lib.init(0)
+    m = llm.make_gpt2(cfg, llm.gpt2_state_dict(w, kind))
+    D, F, L, V = cfg["dim"], cfg["ffn"], cfg["n_layers"], cfg["vocab"]
+    lin_flop = 2.0 * s * L * (3 * D * D + D * D + 2 * D * F) + 2.0 * V * D  # lm_head on the last row only
+    att_flop = 2.0 * 2.0 * L * cfg["n_heads"] * (D // cfg["n_heads"]) * s * (s + 1) / 2
+    for bf16, peak in ((0, 157.3), (1, 2500.0)):
+        _lib.check(lib.cthip_set_option(b"gemm_bf16", bf16))
+        m.forward(prompt, s, 0)
+        ts = []
+        for _ in range(5):
+            t0 = time.perf_counter()
+            m.forward(prompt, s, 0)
+            ts.append(time.perf_counter() - t0)
+        t = min(ts)
+        print(json.dumps({"item": f"prefill {s} tokens {model} {kind} ({'bf16' if bf16 else 'fp32'} MFMA operands)",
+                          "ms": t * 1e3, "tokens_per_s": s / t, "linear_TFLOPs": lin_flop / t / 1e12,
+                          "peak_TFLOPs": peak, "frac": lin_flop / t / 1e12 / peak,
+                          "linear_GFLOP": lin_flop / 1e9, "attention_GFLOP": att_flop / 1e9}))
+    _lib.check(lib.cthip_set_option(b"gemm_bf16", 0))
+    m.close()
+
+
+if __name__ == "__main__":
+    main()

@@ -70,6 +70,9 @@ struct GemvArgs {
   const float *residual;
   const float *norm_g;
   const float *norm_b;
+  // LayerNorm folded through the product (see k_gemv): fold_s[r] = sum_k W[r,k]*gamma[k]; the caller
+  // passes sum_k W[r,k]*beta[k] + b[r] as `bias`.  Null = normalise the input first.
+  const float *fold_s;
   float eps;
   int rows, cols;
   int act, pro;
@@ -99,6 +102,12 @@ int launch_argmax(int64_t *out, const float *x, int64_t rows, int n, int *tok_ou
 // Linear over m rows on the MFMA path (weights dequantised while staged); bf16 rounds the operands.
 int launch_linear_gemm(float *y, const WMat *w, const float *x, int m, const float *bias, const float *residual,
                        int act, bool bf16);
+// gate|up rows (m, 2*cols) -> silu(gate)*up (m, cols), or a norm, as a launch of its own
+int launch_prologue(float *out, const float *x, int cols, int pro, const float *g, const float *b, float eps,
+                    int64_t x_stride, int m);
+// prefill: split fused qkv rows (S, D+2KD) into q (S,D) and cache rows start_pos.., rotating q and k when rope_base > 0
+int launch_qkv_split(float *q, float *kc, float *vc, const float *qkv, int S, int start_pos, int H, int Hkv, int Dh,
+                     float rope_base);
 int launch_rope_append(float *kc, float *vc, const float *kv, int Hkv, int Dh, float base, const int *pos);
 int launch_rope(float *out, const float *x, int B, int S, int H, int Dh, float base, int start_pos, const int *pos);
 

@@ -17,9 +17,10 @@
 // kernel, GQA attention and a fused gate|up matrix whose SwiGLU is the prologue of
 // the down projection.
 //
-// The reference pushes a whole prompt through one forward (s > 1).  Here a prompt is
-// fed row by row through the same step (causal attention makes that the same
-// function); only the last row runs lm_head and argmax.
+// The reference pushes a whole prompt through one forward (s > 1).  Prompts of 8 or more rows
+// run as one batch (MFMA GEMMs over the rows, see prefill()); shorter ones are fed row by row
+// through the decode step (causal attention makes that the same function).  Either way only the
+// last row runs lm_head and argmax.
 #include <stdlib.h>
 #include <string.h>
 
@@ -53,6 +54,8 @@ struct Layer {
   float *ln1_g = nullptr, *ln1_b = nullptr, *ln2_g = nullptr, *ln2_b = nullptr;
   WMat *attn = nullptr, *proj = nullptr, *fc = nullptr, *fc2 = nullptr;
   float *attn_b = nullptr, *proj_b = nullptr, *fc_b = nullptr, *fc2_b = nullptr;
+  // LayerNorm folded through c_attn / c_fc: S = W.gamma, C = W.beta + bias
+  float *attn_s = nullptr, *attn_c = nullptr, *fc_s = nullptr, *fc_c = nullptr;
   // Llama: attn = wq|wk|wv, proj = wo, fc = gate|up, fc2 = down, ln1_g/ln2_g = rms weights
   float *k_cache = nullptr, *v_cache = nullptr;
 };
@@ -65,6 +68,7 @@ struct Decoder {
   std::vector<Layer> layers;
   float *wte = nullptr, *wpe = nullptr, *lnf_g = nullptr, *lnf_b = nullptr;
   WMat *lm_head = nullptr;
+  float *lm_s = nullptr, *lm_c = nullptr;  // ln_f folded through lm_head
   // activations
   float *x = nullptr, *q = nullptr, *kv_tmp = nullptr, *att = nullptr, *h = nullptr, *logits = nullptr;
   // device-resident loop state: [0] = current token, [1] = position
@@ -175,6 +179,28 @@ static int to_wmat(Decoder *d, const std::vector<std::string> &keys, int64_t wan
 }
 
 static int queue_step(Decoder *d, bool with_head);
+static int queue_head(Decoder *d);
+
+// S = W.gamma and C = W.beta + bias for a LayerNorm that precedes the Linear W
+static int make_fold(Decoder *d, const WMat *w, const float *gamma, const float *beta, const float *bias, float **S,
+                     float **C) {
+  int rc;
+  if ((rc = dev_alloc(d, (void **)S, sizeof(float) * (size_t)w->rows))) return rc;
+  if ((rc = dev_alloc(d, (void **)C, sizeof(float) * (size_t)w->rows))) return rc;
+  GemvArgs a = {};
+  a.x = gamma;
+  a.y = *S;
+  a.x_stride = w->cols;
+  a.y_stride = w->rows;
+  if ((rc = launch_gemv(w, a, 1))) return rc;
+  GemvArgs b = {};
+  b.x = beta;
+  b.bias = bias;
+  b.y = *C;
+  b.x_stride = w->cols;
+  b.y_stride = w->rows;
+  return launch_gemv(w, b, 1);
+}
 
 static int finalize(Decoder *d) {
   if (d->finalized) return 0;
@@ -211,7 +237,10 @@ static int finalize(Decoder *d) {
       TRY(to_f32(d, key(l, "mlp.c_fc.bias"), F, &L.fc_b));
       TRY(to_wmat(d, {key(l, "mlp.c_proj.weight")}, D, F, &L.fc2));
       TRY(to_f32(d, key(l, "mlp.c_proj.bias"), D, &L.fc2_b));
+      TRY(make_fold(d, L.attn, L.ln1_g, L.ln1_b, L.attn_b, &L.attn_s, &L.attn_c));
+      TRY(make_fold(d, L.fc, L.ln2_g, L.ln2_b, L.fc_b, &L.fc_s, &L.fc_c));
     }
+    TRY(make_fold(d, d->lm_head, d->lnf_g, d->lnf_b, nullptr, &d->lm_s, &d->lm_c));
   } else {
     TRY(to_f32(d, "tok_embeddings.weight", (int64_t)V * D, &d->wte));
     TRY(to_f32(d, "norm.weight", D, &d->lnf_g));
@@ -297,7 +326,8 @@ static int queue_step(Decoder *d, bool with_head) {
     a.norm_g = L.ln1_g;
     a.norm_b = L.ln1_b;
     a.eps = c.eps;
-    a.bias = L.attn_b;
+    a.bias = gpt2 ? L.attn_c : L.attn_b;
+    a.fold_s = L.attn_s;
     a.y = d->q;
     a.split1 = D;
     a.split2 = D + KD;
@@ -335,7 +365,8 @@ static int queue_step(Decoder *d, bool with_head) {
     f.norm_g = L.ln2_g;
     f.norm_b = L.ln2_b;
     f.eps = c.eps;
-    f.bias = L.fc_b;
+    f.bias = gpt2 ? L.fc_c : L.fc_b;
+    f.fold_s = L.fc_s;
     f.act = gpt2 ? CTHIP_ACT_GELU : CTHIP_ACT_NONE;
     f.y = d->h;
     f.x_stride = D;
@@ -351,28 +382,103 @@ static int queue_step(Decoder *d, bool with_head) {
     g.y_stride = D;
     TRY(launch_gemv(L.fc2, g, 1));
   }
-  if (with_head) {
-    GemvArgs o = {};
-    o.x = d->x;
-    o.pro = gpt2 ? CTHIP_PRO_LAYERNORM : CTHIP_PRO_RMSNORM;
-    o.norm_g = d->lnf_g;
-    o.norm_b = d->lnf_b;
-    o.eps = c.eps;
-    o.y = d->logits;
-    o.x_stride = D;
-    o.y_stride = V;
-    // greedy token -> next step's input; position advances (apps/gpt2/gpt2.lisp:105-107)
-    o.am_val = d->am_val;
-    o.am_idx = d->am_idx;
-    o.am_token64 = (long long *)d->token64;
-    o.am_tok = d->tokpos;
-    o.am_pos = d->tokpos + 1;
-    o.am_hist = (long long *)d->history;
-    o.am_hist_n = d->hist_n;
-    TRY(launch_gemv(d->lm_head, o, 1));
-  }
+  if (with_head) TRY(queue_head(d));
 #undef TRY
   return 0;
+}
+
+// ln_f -> lm_head GEMV on d->x, greedy token -> tokpos[0] and the history, position + 1
+static int queue_head(Decoder *d) {
+  const cthip_decoder_config &c = d->cfg;
+  const bool gpt2 = c.arch == CTHIP_ARCH_GPT2;
+  GemvArgs o = {};
+  o.x = d->x;
+  o.pro = gpt2 ? CTHIP_PRO_LAYERNORM : CTHIP_PRO_RMSNORM;
+  o.norm_g = d->lnf_g;
+  o.norm_b = d->lnf_b;
+  o.eps = c.eps;
+  o.bias = d->lm_c;
+  o.fold_s = d->lm_s;
+  o.y = d->logits;
+  o.x_stride = c.dim;
+  o.y_stride = c.vocab;
+  // greedy token -> next step's input; position advances (apps/gpt2/gpt2.lisp:105-107)
+  o.am_val = d->am_val;
+  o.am_idx = d->am_idx;
+  o.am_token64 = (long long *)d->token64;
+  o.am_tok = d->tokpos;
+  o.am_pos = d->tokpos + 1;
+  o.am_hist = (long long *)d->history;
+  o.am_hist_n = d->hist_n;
+  return launch_gemv(d->lm_head, o, 1);
+}
+
+// A prompt of s >= kPrefillMin rows as one batch (the reference's forward with s > 1): every Linear is
+// an MFMA GEMM over the s rows (weights dequantised while staged), attention runs all s query rows
+// against the cache under the causal mask; only the last row goes through lm_head.
+static const int kPrefillMin = 8;
+static int prefill(Decoder *d, const int *ids, int s, int n) {
+  const cthip_decoder_config &c = d->cfg;
+  const bool gpt2 = c.arch == CTHIP_ARCH_GPT2;
+  const int D = c.dim, F = c.ffn, V = c.vocab, KD = kv_dim(c), Dh = c.dim / c.n_heads;
+  const int QW = D + 2 * KD, HW = gpt2 ? F : 2 * F;
+  const bool bf16 = state().gemm_bf16 != 0;
+  int rc = 0;
+  float *X = nullptr, *XN = nullptr, *QKV = nullptr, *Q = nullptr, *ATT = nullptr, *Hb = nullptr, *G = nullptr;
+  int *ids_dev = nullptr;
+  std::vector<void *> tmp;
+  auto alloc = [&](void **p, size_t bytes) {
+    int r = cthip_alloc(p, bytes);
+    if (r == 0) tmp.push_back(*p);
+    return r;
+  };
+#define TRY(e)                \
+  do {                        \
+    if ((rc = (e))) goto done; \
+  } while (0)
+  TRY(alloc((void **)&X, sizeof(float) * (size_t)s * D));
+  TRY(alloc((void **)&XN, sizeof(float) * (size_t)s * D));
+  TRY(alloc((void **)&QKV, sizeof(float) * (size_t)s * QW));
+  TRY(alloc((void **)&Q, sizeof(float) * (size_t)s * D));
+  TRY(alloc((void **)&ATT, sizeof(float) * (size_t)s * D));
+  TRY(alloc((void **)&Hb, sizeof(float) * (size_t)s * HW));
+  if (!gpt2) TRY(alloc((void **)&G, sizeof(float) * (size_t)s * F));
+  TRY(alloc((void **)&ids_dev, sizeof(int) * (size_t)s));
+  TRY(cthip_h2d(ids_dev, ids, sizeof(int) * (size_t)s));
+  {
+    int tp[2] = {ids[s - 1], n};  // position base for the learned position rows
+    TRY(cthip_h2d(d->tokpos, tp, sizeof(tp)));
+  }
+  TRY(launch_embedding(X, d->wte, nullptr, ids_dev, s, V, D, gpt2 ? d->wpe : nullptr, d->tokpos + 1, c.max_seq));
+  for (int l = 0; l < c.n_layers; l++) {
+    Layer &L = d->layers[l];
+    if (gpt2) TRY(cthip_layernorm(XN, X, L.ln1_g, L.ln1_b, c.eps, s, D));
+    else TRY(cthip_rmsnorm(XN, X, L.ln1_g, c.eps, s, D));
+    TRY(launch_linear_gemm(QKV, L.attn, XN, s, L.attn_b, nullptr, CTHIP_ACT_NONE, bf16));
+    TRY(launch_qkv_split(Q, L.k_cache, L.v_cache, QKV, s, n, c.n_heads, c.n_kv_heads, Dh, gpt2 ? 0.0f : c.rope_base));
+    TRY(launch_attn(ATT, Q, L.k_cache, L.v_cache, s, n, nullptr, n + s, c.n_heads, c.n_kv_heads, Dh));
+    TRY(launch_linear_gemm(X, L.proj, ATT, s, L.proj_b, X, CTHIP_ACT_NONE, bf16));
+    if (gpt2) TRY(cthip_layernorm(XN, X, L.ln2_g, L.ln2_b, c.eps, s, D));
+    else TRY(cthip_rmsnorm(XN, X, L.ln2_g, c.eps, s, D));
+    TRY(launch_linear_gemm(Hb, L.fc, XN, s, L.fc_b, nullptr, gpt2 ? CTHIP_ACT_GELU : CTHIP_ACT_NONE, bf16));
+    const float *hin = Hb;
+    if (!gpt2) {
+      TRY(launch_prologue(G, Hb, F, CTHIP_PRO_SWIGLU, nullptr, nullptr, 0.0f, 2 * (int64_t)F, s));
+      hin = G;
+    }
+    TRY(launch_linear_gemm(X, L.fc2, hin, s, L.fc2_b, X, CTHIP_ACT_NONE, bf16));
+  }
+  // the last row continues through the decode-step head
+  TRY(cthip_d2d(d->x, X + (size_t)(s - 1) * D, sizeof(float) * D));
+  {
+    int tp[2] = {ids[s - 1], n + s - 1};
+    TRY(cthip_h2d(d->tokpos, tp, sizeof(tp)));
+  }
+  TRY(queue_head(d));
+#undef TRY
+done:
+  for (void *p : tmp) cthip_free(p);
+  return rc;
 }
 
 static int run_step(Decoder *d, bool with_head) {
@@ -483,13 +589,21 @@ int cthip_decoder_forward(void *dec, const float *tokens, int s, int n, int64_t 
   if (rc) return rc;
   int zero = 0;
   if ((rc = cthip_h2d(d->hist_n, &zero, sizeof(int)))) return rc;
+  // ids arrive as floats (gpt2.lisp:95); one that equals no vocabulary index selects no row
+  std::vector<int> ids(s);
   for (int i = 0; i < s; i++) {
-    // ids arrive as floats (gpt2.lisp:95); one that equals no vocabulary index selects no row
     const float tf = tokens[i];
-    int id = (tf >= 0.0f && tf < (float)c.vocab && (float)(int)tf == tf) ? (int)tf : -1;
-    int tp[2] = {id, n + i};
-    if ((rc = cthip_h2d(d->tokpos, tp, sizeof(tp)))) return rc;
-    if ((rc = run_step(d, i == s - 1))) return rc;
+    ids[i] = (tf >= 0.0f && tf < (float)c.vocab && (float)(int)tf == tf) ? (int)tf : -1;
+  }
+  const char *np = getenv("CTHIP_NO_PREFILL_GEMM");
+  if (s >= kPrefillMin && !(np && *np && *np != '0')) {
+    if ((rc = prefill(d, ids.data(), s, n))) return rc;
+  } else {
+    for (int i = 0; i < s; i++) {
+      int tp[2] = {ids[i], n + i};
+      if ((rc = cthip_h2d(d->tokpos, tp, sizeof(tp)))) return rc;
+      if ((rc = run_step(d, i == s - 1))) return rc;
+    }
   }
   if (logits_out && (rc = cthip_d2h(logits_out, d->logits, sizeof(float) * (size_t)c.vocab))) return rc;
   if ((rc = cthip_d2h(token, d->token64, sizeof(int64_t)))) return rc;

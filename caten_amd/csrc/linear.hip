@@ -360,12 +360,20 @@ __global__ __launch_bounds__(256) void k_gemv(GemvArgs a) {
   const int scales_per_row = a.cols >> 5;
   const int nrq = (a.rows + RPW - 1) / RPW;
 
-  auto load = [&](int rq, uint4 *w, unsigned short *s, float &bias, float &resid) {
+  // LayerNorm / RMSNorm folded through the product instead of applied to the input first:
+  //   sum_k W[r,k] * (((x_k - mu) * rstd) * g_k + b_k) = rstd * (sum_k W[r,k] (g_k x_k) - mu * S_r) + C_r
+  // with S_r = sum_k W[r,k] g_k and C_r = sum_k W[r,k] b_k (+ bias) precomputed per matrix.  The
+  // statistics mu, rstd are then needed only by the epilogue, so their reductions overlap the weight
+  // stream instead of preceding it.  RMSNorm has no mu / beta term and needs no precomputation.
+  const bool folded = (a.pro == CTHIP_PRO_RMSNORM) || (a.pro == CTHIP_PRO_LAYERNORM && a.fold_s != nullptr);
+  const bool coop = (a.pro != CTHIP_PRO_NONE) && !folded;
+  auto load = [&](int rq, uint4 *w, unsigned short *s, float &bias, float &resid, float &fs) {
     const int row = rq * RPW + g;
     const bool rok = row < a.rows;
     // the epilogue operands of the row travel with its weights
     bias = (rok && a.bias) ? a.bias[row] : 0.0f;
     resid = (rok && a.residual) ? a.residual[(int64_t)m * a.y_stride + row] : 0.0f;
+    fs = (rok && a.fold_s) ? a.fold_s[row] : 0.0f;
 #pragma unroll
     for (int j = 0; j < KC; j++) {
       const int c = l + G * j;
@@ -383,18 +391,18 @@ __global__ __launch_bounds__(256) void k_gemv(GemvArgs a) {
   const int posv = a.pos ? a.pos[0] : 0;
   uint4 wt[PD][KC];
   unsigned short st[PD][KC];
-  float bias_t[PD], resid_t[PD];
+  float bias_t[PD], resid_t[PD], fs_t[PD];
 #pragma unroll
   for (int p = 0; p < PD; p++) {
-    bias_t[p] = resid_t[p] = 0.0f;
+    bias_t[p] = resid_t[p] = fs_t[p] = 0.0f;
     const int rq = wave + p * total_waves;
-    if (rq < nrq) load(rq, wt[p], st[p], bias_t[p], resid_t[p]);
+    if (rq < nrq) load(rq, wt[p], st[p], bias_t[p], resid_t[p], fs_t[p]);
   }
 
   float xr[KC][XPC];
   float xs[KC];
-  if (a.pro != CTHIP_PRO_NONE) coop_prologue(a, x, xs_lds, red);
-  const float *__restrict__ xsrc = (a.pro != CTHIP_PRO_NONE) ? xs_lds : x;
+  if (coop) coop_prologue(a, x, xs_lds, red);
+  const float *__restrict__ xsrc = coop ? xs_lds : x;
 #pragma unroll
   for (int j = 0; j < KC; j++) {
     const int c = l + G * j;
@@ -406,6 +414,40 @@ __global__ __launch_bounds__(256) void k_gemv(GemvArgs a) {
       xr[j][4 * t + 1] = v.y;
       xr[j][4 * t + 2] = v.z;
       xr[j][4 * t + 3] = v.w;
+    }
+  }
+  float mu = 0.0f, rstd = 1.0f;
+  if (folded) {
+    // every group of G lanes holds the whole vector: shifted one-pass mean / variance (the shift by
+    // x[0] keeps E[d^2] - E[d]^2 well conditioned), then scale the slice by gamma
+    const float pivot = (a.pro == CTHIP_PRO_LAYERNORM) ? x[0] : 0.0f;
+    float s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+    for (int j = 0; j < KC; j++) {
+      const int c = l + G * j;
+      const bool ok = c < nchunks;
+#pragma unroll
+      for (int t = 0; t < XPC / 4; t++) {
+        const float4 gv = (ok && a.norm_g) ? *(const float4 *)(a.norm_g + (int64_t)c * XPC + 4 * t)
+                                           : make_float4(1.f, 1.f, 1.f, 1.f);
+        const float gg[4] = {gv.x, gv.y, gv.z, gv.w};
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const float d = ok ? xr[j][4 * t + e] - pivot : 0.0f;
+          s1 += d;
+          s2 = fmaf(d, d, s2);
+          xr[j][4 * t + e] *= gg[e];
+        }
+      }
+    }
+    const float inv_n = 1.0f / (float)a.cols;
+    const float m1 = group_sum<G>(s1) * inv_n;
+    const float m2 = group_sum<G>(s2) * inv_n;
+    if (a.pro == CTHIP_PRO_LAYERNORM) {
+      mu = pivot + m1;
+      rstd = 1.0f / sqrtf(fmaxf(m2 - m1 * m1, 0.0f) + a.eps);
+    } else {
+      rstd = 1.0f / sqrtf(m2 + a.eps);
     }
   }
 #pragma unroll
@@ -433,13 +475,14 @@ __global__ __launch_bounds__(256) void k_gemv(GemvArgs a) {
           acc += chunk_dot<TYPE>(wt[p][j], scale, xr[j], xs[j]);
         }
         acc = group_sum<G>(acc);
+        if (folded) acc = rstd * (acc - mu * fs_t[p]);
         const int row = rq * RPW + g;
         if (l == 0 && row < a.rows) {
           const float v = gemv_store(a, m, row, acc, posv, bias_t[p], resid_t[p]);
           argmax_merge(best_v, best_i, v, row);
         }
         const int nxt = rq + PD * total_waves;
-        if (nxt < nrq) load(nxt, wt[p], st[p], bias_t[p], resid_t[p]);
+        if (nxt < nrq) load(nxt, wt[p], st[p], bias_t[p], resid_t[p], fs_t[p]);
       }
     }
   }
@@ -577,6 +620,14 @@ static const GemvVariant *pick_variant(int type, int cols) {
   return best;
 }
 
+int launch_prologue(float *out, const float *x, int cols, int pro, const float *g, const float *b, float eps,
+                    int64_t x_stride, int m) {
+  if (m == 0) return 0;
+  hipLaunchKernelGGL(k_prologue, dim3(m), dim3(256), 0, state().stream, out, x, cols, pro, g, b, eps, x_stride);
+  CTHIP_LAUNCH_CHECK();
+  return 0;
+}
+
 bool gemv_is_direct(const WMat *w) { return pick_variant(w->type, (int)w->cols) != nullptr; }
 
 // Queues one fused Linear on the stream. Used by cthip_linear and by the decoder.
@@ -594,13 +645,15 @@ int launch_gemv(const WMat *w, GemvArgs a, int m) {
     const int nrq = (a.rows + rpw - 1) / rpw;
     dim3 grid, block;
     const bool small = nrq <= 2048;
-    const size_t lds = a.pro != CTHIP_PRO_NONE ? sizeof(float) * (size_t)a.cols : 0;
+    const bool folded = (a.pro == CTHIP_PRO_RMSNORM) || (a.pro == CTHIP_PRO_LAYERNORM && a.fold_s != nullptr);
+    const bool coop = a.pro != CTHIP_PRO_NONE && !folded;
+    const size_t lds = coop ? sizeof(float) * (size_t)a.cols : 0;
     if (lds > 64 * 1024) return fail(CTHIP_E_UNSUPPORTED, "gemv: %d input features exceed the LDS prologue buffer", a.cols);
     if (small) {
       // small matrices are pure latency: one tile per wavefront.  Without a prologue, one wavefront
       // per workgroup spreads the tiles over as many compute units as possible; with one, four
       // wavefronts share the normalised input through LDS.
-      if (a.pro == CTHIP_PRO_NONE) {
+      if (!coop) {
         block = dim3(64);
         grid = dim3(nrq, m);
       } else {

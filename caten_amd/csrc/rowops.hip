@@ -330,6 +330,37 @@ __global__ __launch_bounds__(256) void k_rope_append(float *__restrict__ kc, flo
   vo[2 * p + 1] = kv[KD + 2 * p + 1];
 }
 
+// Prefill: one fused-qkv row per block -> q (contiguous, rotated for RoPE models), k (rotated) and v
+// into the cache rows start_pos + i.
+__global__ __launch_bounds__(256) void k_qkv_split(float *__restrict__ q, float *__restrict__ kc,
+                                                   float *__restrict__ vc, const float *__restrict__ qkv, int start_pos,
+                                                   int H, int Hkv, int Dh, float log2_base, int rope) {
+  const int i = blockIdx.x;
+  const int D = H * Dh, KD = Hkv * Dh;
+  const float *row = qkv + (int64_t)i * (D + 2 * KD);
+  const int at = start_pos + i;
+  float *ko = kc + (int64_t)at * KD, *vo = vc + (int64_t)at * KD, *qo = q + (int64_t)i * D;
+  for (int p = threadIdx.x; p < (D + KD) / 2; p += blockDim.x) {  // pairs of q then k
+    const bool isq = p < D / 2;
+    const int pp = isq ? p : p - D / 2;
+    const float x0 = isq ? row[2 * pp] : row[D + 2 * pp], x1 = isq ? row[2 * pp + 1] : row[D + 2 * pp + 1];
+    float o0 = x0, o1 = x1;
+    if (rope) {
+      const int ii = pp % (Dh / 2);
+      const float expo = (float)(2 * ii) / (float)Dh;
+      const float theta = exp2f(-(expo * (log2_base * 0.6931472f)) * 1.442695f);
+      float sn, cs;
+      sincosf((float)at * theta, &sn, &cs);
+      o0 = x0 * cs - x1 * sn;
+      o1 = x0 * sn + x1 * cs;
+    }
+    float *dst = isq ? qo : ko;
+    dst[2 * pp] = o0;
+    dst[2 * pp + 1] = o1;
+  }
+  for (int j = threadIdx.x; j < KD; j += blockDim.x) vo[j] = row[D + KD + j];
+}
+
 // ------------------------------------------------------------------ attention over the KV cache
 // One 1024-thread block per (query head h, query row i); keys 0..T-1 with T = pos+i+1 (the causal
 // mask of layers.lisp:83 is implicit).  K/V cache layout (max_len, Hkv, Dh).
@@ -476,6 +507,15 @@ int launch_rope(float *out, const float *x, int B, int S, int H, int Dh, float b
   if (npairs == 0) return 0;
   hipLaunchKernelGGL(k_rope, dim3((unsigned)((npairs + 255) / 256)), dim3(256), 0, state().stream, out, x, npairs, S, H,
                      Dh, log2f(base), start_pos, pos);
+  CTHIP_LAUNCH_CHECK();
+  return 0;
+}
+
+int launch_qkv_split(float *q, float *kc, float *vc, const float *qkv, int S, int start_pos, int H, int Hkv, int Dh,
+                     float rope_base) {
+  if (S == 0) return 0;
+  hipLaunchKernelGGL(k_qkv_split, dim3(S), dim3(256), 0, state().stream, q, kc, vc, qkv, start_pos, H, Hkv, Dh,
+                     rope_base > 0.0f ? log2f(rope_base) : 0.0f, rope_base > 0.0f ? 1 : 0);
   CTHIP_LAUNCH_CHECK();
   return 0;
 }

@@ -124,3 +124,51 @@ def test_llama_generate_matches_oracle(oracle, kind):
     model = llm.make_llama(cfg, llm.llama_state_dict(w, kind))
     assert llm.gpt2_generate(model, prompt, steps, on_device=True) == want_tokens
     model.close()
+
+
+def test_prefill_batch_equals_token_by_token(oracle):
+    """A prompt pushed through one forward as a batch (MFMA GEMMs) and the same prompt fed row by row
+    through the decode step are the same function: identical greedy tokens, logits and cache rows
+    within the fp32 band; with bf16 MFMA operands within the 1e-2 band the north star allows."""
+    import os
+    from caten_amd import synth, llm, _lib
+    cfg = synth.GPT2_CONFIGS["gpt2-mini"]
+    w = synth.gpt2_weights(cfg, seed=2)
+    prompt = synth.prompt(cfg["vocab"], 100, seed=2)
+    sd = llm.gpt2_state_dict(w, "q8_0")
+    x = [float(t) for t in prompt]
+    m1 = llm.make_gpt2(cfg, sd)
+    tok1, lg1 = m1.forward(x, len(x), 0, return_logits=True)
+    os.environ["CTHIP_NO_PREFILL_GEMM"] = "1"
+    try:
+        m2 = llm.make_gpt2(cfg, sd)
+        tok2, lg2 = m2.forward(x, len(x), 0, return_logits=True)
+    finally:
+        del os.environ["CTHIP_NO_PREFILL_GEMM"]
+    assert tok1 == tok2
+    close(lg1, lg2)
+    close(m1.peek("k_cache.2")[:100 * cfg["dim"]], m2.peek("k_cache.2")[:100 * cfg["dim"]])
+    close(m1.peek("v_cache.2")[:100 * cfg["dim"]], m2.peek("v_cache.2")[:100 * cfg["dim"]])
+    # continuing from either cache gives the same tokens
+    assert m1.generate_on_device(6) == m2.generate_on_device(6)
+    # prefill appended to an existing sequence (n > 0)
+    more = [float(t) for t in synth.prompt(cfg["vocab"], 9, seed=4)]
+    ta, la = m1.forward(more, 9, m1.position, return_logits=True)
+    os.environ["CTHIP_NO_PREFILL_GEMM"] = "1"
+    try:
+        tb, lb = m2.forward(more, 9, m2.position, return_logits=True)
+    finally:
+        del os.environ["CTHIP_NO_PREFILL_GEMM"]
+    assert ta == tb
+    close(la, lb)
+    m1.close()
+    # bf16 MFMA operands
+    _lib.check(_lib.load().cthip_set_option(b"gemm_bf16", 1))
+    try:
+        m3 = llm.make_gpt2(cfg, sd)
+        tok3, lg3 = m3.forward(x, len(x), 0, return_logits=True)
+    finally:
+        _lib.check(_lib.load().cthip_set_option(b"gemm_bf16", 0))
+    close(lg3, lg2, 1e-2, 1e-2)
+    m2.close()
+    m3.close()

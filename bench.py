@@ -29,23 +29,26 @@ HBM_PEAK_GBS = 8000.0
 TRAFFIC_BYTES = {("gpt2", "q8_0"): 41540414}  # profiles/gemv_q8_0_lm_head_pmc.txt
 
 
-def cpu_baseline(cfg, weights, prompt, budget_s):
-    """Oracle ("port" of the CLANG path), one thread: decode steps at the same positions."""
+def cpu_baseline(cfg, weights, prompt, budget_s, kind, llama):
+    """Oracle ("port" of the CLANG path), one thread: decode steps at the same positions, on the
+    dequantised fp32 weights (the reference has no quantised compute, dequantize.lisp:3-5)."""
     import oracle
     from caten_amd import synth
     from caten_amd.llm import Tensor
     wd = dict(weights)
-    for k in synth.GPT2_LINEAR_KEYS:
-        wd[k] = [oracle.dequant("q8_0", Tensor.from_f32(a, "q8_0").raw, a.size).reshape(a.shape) for a in weights[k]]
-    wd["lm_head"] = oracle.dequant("q8_0", Tensor.from_f32(weights["lm_head"], "q8_0").raw,
-                                   weights["lm_head"].size).reshape(weights["lm_head"].shape)
-    m = oracle.GPT2(cfg, wd)
-    # prefill untimed and with the row-copy embedding so the sample is decode steps only
-    tok, _ = m.forward([float(t) for t in prompt], 0, onehot=False, all_logits=False)
+    if kind != "f32":
+        for k in (synth.LLAMA_LINEAR_KEYS if llama else synth.GPT2_LINEAR_KEYS):
+            wd[k] = [oracle.dequant(kind, Tensor.from_f32(a, kind).raw, a.size).reshape(a.shape) for a in weights[k]]
+        wd["lm_head"] = oracle.dequant(kind, Tensor.from_f32(weights["lm_head"], kind).raw,
+                                       weights["lm_head"].size).reshape(weights["lm_head"].shape)
+    m = oracle.Llama(cfg, wd) if llama else oracle.GPT2(cfg, wd)
+    # prefill untimed (and with the row-copy embedding) so the sample is decode steps only
+    tok, _ = m.forward([float(t) for t in prompt], 0) if llama else \
+        m.forward([float(t) for t in prompt], 0, onehot=False, all_logits=False)
     n = len(prompt)
     steps, t0 = 0, time.perf_counter()
     while True:
-        tok, _ = m.forward([float(tok)], n, onehot=True, all_logits=True)
+        tok, _ = m.forward([float(tok)], n) if llama else m.forward([float(tok)], n, onehot=True, all_logits=True)
         n += 1
         steps += 1
         el = time.perf_counter() - t0
@@ -80,15 +83,17 @@ def main():
 
     import ctypes as C
     from caten_amd import _lib, synth, llm
-    cfg = dict(synth.GPT2_CONFIGS[args.model])
-    weights = synth.gpt2_weights(cfg, seed=0)
+    llama = args.model in synth.LLAMA_CONFIGS
+    cfg = dict(synth.LLAMA_CONFIGS[args.model] if llama else synth.GPT2_CONFIGS[args.model])
+    weights = synth.llama_weights(cfg, seed=0) if llama else synth.gpt2_weights(cfg, seed=0)
     prompt = synth.prompt(cfg["vocab"], args.prompt, seed=0)
     total = args.warmup + args.steps
     if args.prompt + total + 1 > cfg["max_seq"]:
         # the KV cache bounds how many tokens one sequence can hold: restart sequences as needed
         pass
     lib = _lib.init(0)
-    model = llm.make_gpt2(cfg, llm.gpt2_state_dict(weights, args.kind))
+    model = (llm.make_llama(cfg, llm.llama_state_dict(weights, args.kind)) if llama
+             else llm.make_gpt2(cfg, llm.gpt2_state_dict(weights, args.kind)))
 
     def run(n_steps):
         """n_steps decode steps, restarting from the prompt whenever the KV cache is full."""
@@ -141,8 +146,8 @@ def main():
     t = Tensor.from_f32(weights["lm_head"], args.kind)
     wm = ops.WeightMatrix(args.kind, t.raw, V, D)
     dx = ops.DeviceArray.from_numpy(np.random.default_rng(1).normal(size=D).astype(np.float32))
-    dg = ops.DeviceArray.from_numpy(weights["lnf_g"])
-    db = ops.DeviceArray.from_numpy(weights["lnf_b"])
+    dg = ops.DeviceArray.from_numpy(weights["norm_w" if llama else "lnf_g"])
+    db = ops.DeviceArray.from_numpy(np.zeros(D, np.float32) if llama else weights["lnf_b"])
     dy = ops.DeviceArray((V,), np.float32)
     reps = 200
     for _ in range(20):
@@ -161,8 +166,9 @@ def main():
         "value": tok_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": f"GPT-2-small shape ({cfg['n_layers']}L d{cfg['dim']} h{cfg['n_heads']} ffn{cfg['ffn']} "
-                               f"vocab{cfg['vocab']}), GGUF-{args.kind.upper()} linear weights, fp32 embeddings/LayerNorm/KV, "
+        "config": {"workload": f"{'Llama' if llama else 'GPT-2'} shape {args.model} ({cfg['n_layers']}L d{cfg['dim']} "
+                               f"h{cfg['n_heads']} ffn{cfg['ffn']} "
+                               f"vocab{cfg['vocab']}), GGUF-{args.kind.upper()} linear weights, fp32 embeddings/norms/KV, "
                                f"{args.prompt}-token prompt, batch-1 greedy decode, positions {min(positions)}..{max(positions)}",
                    "model": args.model, "weights": args.kind, "batch": 1},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -179,7 +185,7 @@ def main():
         _lib.check(lib.cthip_d2d(b.ptr, a.ptr, n))
         _lib.check(lib.cthip_sync())
     if args.cpu_seconds > 0:
-        res["cpu_baseline"] = cpu_baseline(cfg, weights, prompt, args.cpu_seconds)
+        res["cpu_baseline"] = cpu_baseline(cfg, weights, prompt, args.cpu_seconds, args.kind, llama)
     model.close()
     print(json.dumps(res))
 

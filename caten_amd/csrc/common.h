@@ -73,6 +73,7 @@ struct GemvArgs {
   // LayerNorm folded through the product (see k_gemv): fold_s[r] = sum_k W[r,k]*gamma[k]; the caller
   // passes sum_k W[r,k]*beta[k] + b[r] as `bias`.  Null = normalise the input first.
   const float *fold_s;
+  int stage_x;  // set by the launcher: the workgroup stages the input vector in LDS once
   float eps;
   int rows, cols;
   int act, pro;
@@ -117,21 +118,46 @@ int launch_rope(float *out, const float *x, int B, int S, int H, int Dh, float b
 #if defined(__HIPCC__)
 namespace cthip {
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+// Cross-lane reductions.  Steps inside a row of 16 lanes are DPP modifiers on the add itself
+// (quad_perm xor 1, xor 2, row_half_mirror, row_mirror: a few cycles each, no LDS traffic); the four
+// row totals of a wavefront are then combined through readlane.  A chain of ds_bpermute shuffles
+// costs an LDS round trip per step, which dominates a short kernel's critical path.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+// every lane gets the sum over its row of 16 lanes
+__device__ __forceinline__ float row16_sum(float v) {
+  v += dpp_f<0xB1>(v);   // quad_perm [1,0,3,2]
+  v += dpp_f<0x4E>(v);   // quad_perm [2,3,0,1]
+  v += dpp_f<0x141>(v);  // row_half_mirror
+  v += dpp_f<0x140>(v);  // row_mirror
   return v;
 }
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+__device__ __forceinline__ float row16_max(float v) {
+  v = fmaxf(v, dpp_f<0xB1>(v));
+  v = fmaxf(v, dpp_f<0x4E>(v));
+  v = fmaxf(v, dpp_f<0x141>(v));
+  v = fmaxf(v, dpp_f<0x140>(v));
   return v;
+}
+__device__ __forceinline__ float lane_bcast(float v, int lane) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+__device__ __forceinline__ float wave_sum(float v) {
+  v = row16_sum(v);
+  return (lane_bcast(v, 0) + lane_bcast(v, 16)) + (lane_bcast(v, 32) + lane_bcast(v, 48));
+}
+__device__ __forceinline__ float wave_max(float v) {
+  v = row16_max(v);
+  return fmaxf(fmaxf(lane_bcast(v, 0), lane_bcast(v, 16)), fmaxf(lane_bcast(v, 32), lane_bcast(v, 48)));
 }
 // sum over aligned groups of G lanes (G = 16, 32, 64); every lane gets the group's sum
 template <int G>
 __device__ __forceinline__ float group_sum(float v) {
-#pragma unroll
-  for (int o = G / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  if (G == 64) return wave_sum(v);
+  v = row16_sum(v);
+  if (G == 32) v += __shfl_xor(v, 16, 64);
   return v;
 }
 

@@ -20,6 +20,7 @@
 // wavefront visits, so the steady state touches nothing but weights.  Partial
 // sums are combined with DPP/shuffle steps inside the group and the group's
 // first lane applies the epilogue.
+#include <stdlib.h>
 #include <string.h>
 
 #include "common.h"
@@ -258,9 +259,15 @@ __global__ __launch_bounds__(1024) void k_argmax_finish(GemvArgs a, int nparts) 
 // Block-cooperative prologue: the workgroup normalises (or gates) the input vector ONCE into LDS --
 // every thread owns cols/blockDim elements, the two reductions go wavefront-shuffle then LDS --
 // instead of every wavefront redoing it in registers.  xs must hold a.cols floats.
-__device__ __forceinline__ void coop_prologue(const GemvArgs &a, const float *__restrict__ x, float *xs, float *red) {
+__device__ __forceinline__ void coop_prologue(const GemvArgs &a, const float *__restrict__ x, float *xs, float *red,
+                                              bool normalise) {
   const int tid = threadIdx.x, nthr = blockDim.x, nw = nthr >> 6;
   const int n4 = a.cols >> 2;
+  if (a.pro != CTHIP_PRO_SWIGLU && !normalise) {  // plain copy: the norm (if any) is folded through the product
+    for (int i = tid; i < n4; i += nthr) ((float4 *)xs)[i] = ((const float4 *)x)[i];
+    __syncthreads();
+    return;
+  }
   if (a.pro == CTHIP_PRO_SWIGLU) {
     for (int i = tid; i < n4; i += nthr) {
       float4 v = ((const float4 *)x)[i];
@@ -366,7 +373,7 @@ __global__ __launch_bounds__(256) void k_gemv(GemvArgs a) {
   // statistics mu, rstd are then needed only by the epilogue, so their reductions overlap the weight
   // stream instead of preceding it.  RMSNorm has no mu / beta term and needs no precomputation.
   const bool folded = (a.pro == CTHIP_PRO_RMSNORM) || (a.pro == CTHIP_PRO_LAYERNORM && a.fold_s != nullptr);
-  const bool coop = (a.pro != CTHIP_PRO_NONE) && !folded;
+  const bool coop = a.stage_x != 0;  // input staged (and normalised, unless folded) once per workgroup
   auto load = [&](int rq, uint4 *w, unsigned short *s, float &bias, float &resid, float &fs) {
     const int row = rq * RPW + g;
     const bool rok = row < a.rows;
@@ -401,7 +408,7 @@ __global__ __launch_bounds__(256) void k_gemv(GemvArgs a) {
 
   float xr[KC][XPC];
   float xs[KC];
-  if (coop) coop_prologue(a, x, xs_lds, red);
+  if (coop) coop_prologue(a, x, xs_lds, red, a.pro != CTHIP_PRO_NONE && !folded);
   const float *__restrict__ xsrc = coop ? xs_lds : x;
 #pragma unroll
   for (int j = 0; j < KC; j++) {
@@ -644,25 +651,30 @@ int launch_gemv(const WMat *w, GemvArgs a, int m) {
     const int rpw = 64 / v->G;
     const int nrq = (a.rows + rpw - 1) / rpw;
     dim3 grid, block;
-    const bool small = nrq <= 2048;
     const bool folded = (a.pro == CTHIP_PRO_RMSNORM) || (a.pro == CTHIP_PRO_LAYERNORM && a.fold_s != nullptr);
-    const bool coop = a.pro != CTHIP_PRO_NONE && !folded;
-    const size_t lds = coop ? sizeof(float) * (size_t)a.cols : 0;
-    if (lds > 64 * 1024) return fail(CTHIP_E_UNSUPPORTED, "gemv: %d input features exceed the LDS prologue buffer", a.cols);
-    if (small) {
-      // small matrices are pure latency: one tile per wavefront.  Without a prologue, one wavefront
-      // per workgroup spreads the tiles over as many compute units as possible; with one, four
-      // wavefronts share the normalised input through LDS.
-      if (!coop) {
-        block = dim3(64);
-        grid = dim3(nrq, m);
-      } else {
-        block = dim3(256);
-        grid = dim3((nrq + 3) / 4, m);
-      }
+    // The input vector goes through LDS once per workgroup when it must be normalised or gated first,
+    // or when it is large next to a weight tile (a 4-bit tile multiplies 8 input bytes per weight byte):
+    // then four wavefronts share one copy and every wavefront takes several tiles.
+    const bool stage = (a.pro != CTHIP_PRO_NONE && !folded) || (w->type == CTHIP_Q4_0 && a.cols >= 1024);
+    const size_t lds = stage ? sizeof(float) * (size_t)a.cols : 0;
+    if (lds > 64 * 1024) return fail(CTHIP_E_UNSUPPORTED, "gemv: %d input features exceed the LDS staging buffer", a.cols);
+    a.stage_x = stage ? 1 : 0;
+    bool small;
+    if (!stage && nrq <= 2048) {
+      // small matrices are pure latency: one tile per wavefront, one wavefront per workgroup, spread
+      // over as many compute units as there are tiles
+      small = true;
+      block = dim3(64);
+      grid = dim3(nrq, m);
+    } else if (stage && nrq <= s.compute_units * 4) {
+      small = true;
+      block = dim3(256);
+      grid = dim3((nrq + 3) / 4, m);
     } else {
-      // large matrices: as many resident wavefronts as the register budget allows, every one
-      // looping over the same number of tiles (an uneven last pass would idle most of the chip)
+      // larger matrices: at least one wavefront per SIMD, more (up to what the register budget keeps
+      // resident) once every wavefront has four tiles; all loop over the same number of tiles (an
+      // uneven last pass would idle most of the chip)
+      small = false;
       static int occ_cache[sizeof(kVariants) / sizeof(kVariants[0])];
       const int vi = (int)(v - kVariants);
       if (occ_cache[vi] == 0) {
@@ -671,8 +683,13 @@ int launch_gemv(const WMat *w, GemvArgs a, int m) {
         occ_cache[vi] = nb > 0 ? nb : 1;
       }
       block = dim3(256);
-      const int capacity = s.compute_units * occ_cache[vi] * 4;
-      const int iters = (nrq + capacity - 1) / capacity;
+      const int base = s.compute_units * 4;
+      int wanted = (nrq + 3) / 4;
+      if (wanted < base) wanted = base;
+      if (wanted > base * occ_cache[vi]) wanted = base * occ_cache[vi];
+      static const char *ovr = getenv("CTHIP_GEMV_WAVES");  // tuning aid: overrides the wavefront count
+      if (ovr && atoi(ovr) > 0) wanted = atoi(ovr);
+      const int iters = (nrq + wanted - 1) / wanted;
       const int waves = (nrq + iters - 1) / iters;
       grid = dim3((waves + 3) / 4, m);
     }

@@ -99,74 +99,85 @@ __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
 #pragma unroll
   for (int r = 0; r < 16; r++) acc[r] = 0.0f;
 
-  for (int k0 = 0; k0 < a.K; k0 += BK) {
-    // ---- stage A: thread -> (row r = tid/4, 8 consecutive k) ----
-    {
-      const int r = tid >> 2, kc = (tid & 3) * 8;
-      const int gm = m0 + r;
-      float v[8];
+  // thread -> staging coordinates
+  const int ar = tid >> 2, akc = (tid & 3) * 8;            // A: row ar, 8 consecutive k
+  const int bk = tid >> 3, bnc = (tid & 7) * 8;            // B row-major: row k = bk, 8 consecutive n
+  const int wr = tid >> 2, wkc = (tid & 3) * 8;            // B packed: weight row wr, 8 consecutive k
+
+  auto fetch_a = [&](int k0, float *v) {
 #pragma unroll
-      for (int j = 0; j < 8; j++) v[j] = 0.0f;
-      if (gm < a.M) {
-        const float *src = a.A + (int64_t)gm * a.K + k0 + kc;
-        if (vecA && k0 + kc + 8 <= a.K) {
-          const float4 f0 = *(const float4 *)src, f1 = *(const float4 *)(src + 4);
-          v[0] = f0.x; v[1] = f0.y; v[2] = f0.z; v[3] = f0.w; v[4] = f1.x; v[5] = f1.y; v[6] = f1.z; v[7] = f1.w;
-        } else {
-#pragma unroll
-          for (int j = 0; j < 8; j++)
-            if (k0 + kc + j < a.K) v[j] = src[j];
-        }
-      }
-      if (BF16) {
-#pragma unroll
-        for (int j = 0; j < 8; j++) As_h[BF16 ? r : 0][BF16 ? kc + j : 0] = f32_to_bf16_bits(v[j]);
+    for (int j = 0; j < 8; j++) v[j] = 0.0f;
+    const int gm = m0 + ar;
+    if (gm < a.M) {
+      const float *src = a.A + (int64_t)gm * a.K + k0 + akc;
+      if (vecA && k0 + akc + 8 <= a.K) {
+        const float4 f0 = *(const float4 *)src, f1 = *(const float4 *)(src + 4);
+        v[0] = f0.x; v[1] = f0.y; v[2] = f0.z; v[3] = f0.w; v[4] = f1.x; v[5] = f1.y; v[6] = f1.z; v[7] = f1.w;
       } else {
 #pragma unroll
-        for (int j = 0; j < 8; j++) As_f[BF16 ? 0 : kc + j][BF16 ? 0 : r] = v[j];
+        for (int j = 0; j < 8; j++)
+          if (k0 + akc + j < a.K) v[j] = src[j];
       }
     }
-    // ---- stage B ----
-    if (BMODE == B_ROWMAJOR) {
-      // thread -> (k = tid/8, 8 consecutive n)
-      const int k = tid >> 3, nc = (tid & 7) * 8;
-      float v[8];
+  };
+  auto fetch_b = [&](int k0, float *v) {
 #pragma unroll
-      for (int j = 0; j < 8; j++) v[j] = 0.0f;
-      if (k0 + k < a.K) {
-        const float *src = a.B + (int64_t)(k0 + k) * a.N + n0 + nc;
-        if (vecB && n0 + nc + 8 <= a.N) {
+    for (int j = 0; j < 8; j++) v[j] = 0.0f;
+    if (BMODE == B_ROWMAJOR) {
+      if (k0 + bk < a.K) {
+        const float *src = a.B + (int64_t)(k0 + bk) * a.N + n0 + bnc;
+        if (vecB && n0 + bnc + 8 <= a.N) {
           const float4 f0 = *(const float4 *)src, f1 = *(const float4 *)(src + 4);
           v[0] = f0.x; v[1] = f0.y; v[2] = f0.z; v[3] = f0.w; v[4] = f1.x; v[5] = f1.y; v[6] = f1.z; v[7] = f1.w;
         } else {
 #pragma unroll
           for (int j = 0; j < 8; j++)
-            if (n0 + nc + j < a.N) v[j] = src[j];
+            if (n0 + bnc + j < a.N) v[j] = src[j];
         }
-      }
-      if (BF16) {
-#pragma unroll
-        for (int j = 0; j < 8; j++) Bs_h[BF16 ? nc + j : 0][BF16 ? k : 0] = f32_to_bf16_bits(v[j]);
-      } else {
-#pragma unroll
-        for (int j = 0; j < 8; j++) Bs_f[BF16 ? 0 : k][BF16 ? 0 : nc + j] = v[j];
       }
     } else {
-      // packed weights: thread -> (row n = tid/4, 8 consecutive k); K % 32 == 0 for every packed type here
-      const int n = tid >> 2, kc = (tid & 3) * 8;
-      float v[8];
+      // packed weights (K % 32 == 0 for every packed type here): dequantised on the way in
+      if (n0 + wr < a.N && k0 + wkc < a.K) wmat_load8(a, n0 + wr, k0 + wkc, v);
+    }
+  };
+  auto stage = [&](const float *va, const float *vb) {
+    if (BF16) {
 #pragma unroll
-      for (int j = 0; j < 8; j++) v[j] = 0.0f;
-      if (n0 + n < a.N && k0 + kc < a.K) wmat_load8(a, n0 + n, k0 + kc, v);
+      for (int j = 0; j < 8; j++) As_h[BF16 ? ar : 0][BF16 ? akc + j : 0] = f32_to_bf16_bits(va[j]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; j++) As_f[BF16 ? 0 : akc + j][BF16 ? 0 : ar] = va[j];
+    }
+    if (BMODE == B_ROWMAJOR) {
       if (BF16) {
 #pragma unroll
-        for (int j = 0; j < 8; j++) Bs_h[BF16 ? n : 0][BF16 ? kc + j : 0] = f32_to_bf16_bits(v[j]);
+        for (int j = 0; j < 8; j++) Bs_h[BF16 ? bnc + j : 0][BF16 ? bk : 0] = f32_to_bf16_bits(vb[j]);
       } else {
 #pragma unroll
-        for (int j = 0; j < 8; j++) Bs_f[BF16 ? 0 : kc + j][BF16 ? 0 : n] = v[j];
+        for (int j = 0; j < 8; j++) Bs_f[BF16 ? 0 : bk][BF16 ? 0 : bnc + j] = vb[j];
+      }
+    } else {
+      if (BF16) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) Bs_h[BF16 ? wr : 0][BF16 ? wkc + j : 0] = f32_to_bf16_bits(vb[j]);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; j++) Bs_f[BF16 ? 0 : wkc + j][BF16 ? 0 : wr] = vb[j];
       }
     }
+  };
+
+  // software pipeline: the next K-step's global loads are in flight while the MFMAs of this one run
+  float va[8], vb[8];
+  fetch_a(0, va);
+  fetch_b(0, vb);
+  for (int k0 = 0; k0 < a.K; k0 += BK) {
+    stage(va, vb);
     __syncthreads();
+    if (k0 + BK < a.K) {
+      fetch_a(k0 + BK, va);
+      fetch_b(k0 + BK, vb);
+    }
     if (BF16) {
       // 32x32x8: lane l holds A[i = l%32][k = 4*(l/32) .. +3] and B[k = 4*(l/32) .. +3][j = l%32]
 #pragma unroll

@@ -172,3 +172,33 @@ def test_prefill_batch_equals_token_by_token(oracle):
     close(lg3, lg2, 1e-2, 1e-2)
     m2.close()
     m3.close()
+
+
+def test_gpt2_small_q8_0_full_size_matches_oracle(oracle):
+    """BASELINE config 4 at its real size (12 layers, d 768, vocab 50257, Q8_0): a 16-token prompt and
+    greedy decode against the CPU oracle on the dequantised weights -- identical tokens, logits inside
+    rtol 1e-3 / atol 1e-4.  (The oracle needs ~0.1 s per token, so a handful of steps.)"""
+    print("case: gpt2 small q8_0 full size", flush=True)
+    from caten_amd import synth, llm
+    cfg = synth.GPT2_CONFIGS["gpt2"]
+    w = synth.gpt2_weights(cfg, seed=0)
+    prompt = synth.prompt(cfg["vocab"], 16, seed=0)
+    steps = 6
+    ref = oracle.GPT2(cfg, _dequantised(oracle, w, synth.GPT2_LINEAR_KEYS + ("lm_head",), "q8_0"))
+    want_tokens, want_logits = ref.generate(prompt, steps, onehot=False, keep_logits=True)
+    model = llm.make_gpt2(cfg, llm.gpt2_state_dict(w, "q8_0"))
+    got_tokens, got_logits = llm.gpt2_generate(model, prompt, steps, on_device=False, keep_logits=True)
+    assert got_tokens == want_tokens
+    for g, r in zip(got_logits, want_logits):
+        close(g, r)
+    assert model.step_bytes(17) == 131252784 + 4 * (12 * (2 * 768 * 2 + 2304 + 768 + 3072 + 768) + 2 * 768) \
+        + 2 * 768 * 4 + 2 * 12 * 17 * 768 * 4 + 2 * 12 * 768 * 4
+    model.close()
+    # size-independent property at the full size: the device-resident loop reproduces the host-driven one
+    model = llm.make_gpt2(cfg, llm.gpt2_state_dict(w, "q8_0"))
+    long_run = llm.gpt2_generate(model, prompt, 40, on_device=True)
+    assert long_run[:steps] == want_tokens
+    model2 = llm.make_gpt2(cfg, llm.gpt2_state_dict(w, "q8_0"))
+    assert llm.gpt2_generate(model2, prompt, 40, on_device=False) == long_run
+    model.close()
+    model2.close()

@@ -87,6 +87,21 @@ PROTOTYPES = {
     "cthip_decoder_position": (_i, [_vp]),
     "cthip_decoder_step_bytes": (_i64, [_vp, _i]),
     "cthip_decoder_peek": (_i, [_vp, C.c_char_p, _vpp, C.POINTER(_i64)]),
+    "cthip_gguf_open": (_i, [_vpp, C.c_char_p]),
+    "cthip_gguf_close": (_i, [_vp]),
+    "cthip_gguf_version": (_i, [_vp]),
+    "cthip_gguf_tensor_count": (_i64, [_vp]),
+    "cthip_gguf_metadata_count": (_i64, [_vp]),
+    "cthip_gguf_alignment": (_i64, [_vp]),
+    "cthip_gguf_tensor_info": (_i, [_vp, _i64, C.POINTER(C.c_char_p), C.POINTER(_i), C.POINTER(_i), C.POINTER(_i64),
+                                    C.POINTER(_i64), C.POINTER(_i64)]),
+    "cthip_gguf_find_tensor": (_i64, [_vp, C.c_char_p]),
+    "cthip_gguf_tensor_data": (_vp, [_vp, _i64]),
+    "cthip_gguf_find_metadata": (_i64, [_vp, C.c_char_p]),
+    "cthip_gguf_metadata_info": (_i, [_vp, _i64, C.POINTER(C.c_char_p), C.POINTER(_i), C.POINTER(_i), C.POINTER(_i64)]),
+    "cthip_gguf_metadata_number": (_i, [_vp, _i64, C.POINTER(C.c_double)]),
+    "cthip_gguf_metadata_string": (_i, [_vp, _i64, _i64, C.POINTER(C.c_void_p), C.POINTER(_i64)]),
+    "cthip_decoder_load_gguf": (_i, [_vp, _vp, _i, C.POINTER(_i)]),
 }
 
 _lib = None

@@ -235,6 +235,36 @@ int64_t cthip_decoder_step_bytes(const void *dec, int t);
 /* Device pointers into the session, for parity tests: "k_cache.<l>", "v_cache.<l>", "logits", "x". */
 int cthip_decoder_peek(void *dec, const char *what, void **ptr, int64_t *n_floats);
 
+/* ================================================================== */
+/* GGUF files (external/gguf/gguf-file.lisp, metadata.lisp,            */
+/* tensor-info.lisp).  Host side only: needs no device.                */
+/* ================================================================== */
+
+/* load-gguf (gguf-file.lisp:93-104): maps the file, parses header (magic "GGUF", version 2 or 3),
+ * metadata key/values and tensor infos; absolute tensor offsets follow general.alignment
+ * (default 32; tensor-info.lisp:88-98). */
+int cthip_gguf_open(void **gguf, const char *path);
+int cthip_gguf_close(void *gguf);
+int cthip_gguf_version(const void *gguf);
+int64_t cthip_gguf_tensor_count(const void *gguf);
+int64_t cthip_gguf_metadata_count(const void *gguf);
+int64_t cthip_gguf_alignment(const void *gguf);
+/* Tensor-Info (tensor-info.lisp:43-60).  dims are as stored, innermost first: the row-major shape is
+ * their reverse (tensor-info.lisp:104-120).  nbytes is 0 for ggml types without a decoder here. */
+int cthip_gguf_tensor_info(const void *gguf, int64_t i, const char **name, int *ggml_type, int *n_dims,
+                           int64_t dims[4], int64_t *abs_offset, int64_t *nbytes);
+int64_t cthip_gguf_find_tensor(const void *gguf, const char *name); /* -1 if absent */
+const void *cthip_gguf_tensor_data(const void *gguf, int64_t i);    /* host pointer into the mapping */
+/* gguf-metadata-get (gguf-file.lisp:26-27) */
+int64_t cthip_gguf_find_metadata(const void *gguf, const char *key); /* -1 if absent */
+int cthip_gguf_metadata_info(const void *gguf, int64_t i, const char **key, int *type, int *elem_type, int64_t *count);
+int cthip_gguf_metadata_number(const void *gguf, int64_t i, double *out);
+/* a string value, or element j of an array of strings; not NUL-terminated */
+int cthip_gguf_metadata_string(const void *gguf, int64_t i, int64_t j, const char **data, int64_t *len);
+/* make-gpt2's load path (apps/gpt2/gpt2.lisp:82-93): gguf->state-dict + remap-key + load-state-dict
+ * for a decoder session; tensors go from the mapping to the device still packed. */
+int cthip_decoder_load_gguf(void *dec, const void *gguf, int arch, int *n_loaded);
+
 #ifdef __cplusplus
 }
 #endif

@@ -230,12 +230,18 @@ __device__ __forceinline__ void gemv_argmax_tail(const GemvArgs &a, int wave, in
 
 // one block: the greedy token goes where the next step's embedding reads it, is appended to the
 // history, and the position advances
-__global__ __launch_bounds__(1024) void k_argmax_finish(GemvArgs a, int nparts) {
-  __shared__ float sv[16];
-  __shared__ int si[16];
+__global__ __launch_bounds__(256) void k_argmax_finish(GemvArgs a, int nparts) {
+  __shared__ float sv[4];
+  __shared__ int si[4];
+  // the loop state is requested up front so its latency overlaps the reduction
+  int hist_n = 0, pos = 0;
+  if (threadIdx.x == 0) {
+    if (a.am_hist) hist_n = *a.am_hist_n;
+    if (a.am_pos) pos = *a.am_pos;
+  }
   float bv = -INFINITY;
   int bi = 0x7fffffff;
-  for (int i = threadIdx.x; i < nparts; i += 1024) argmax_merge(bv, bi, a.am_val[i], a.am_idx[i]);
+  for (int i = threadIdx.x; i < nparts; i += 256) argmax_merge(bv, bi, a.am_val[i], a.am_idx[i]);
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) argmax_merge(bv, bi, __shfl_xor(bv, o, 64), __shfl_xor(bi, o, 64));
   if ((threadIdx.x & 63) == 0) {
@@ -244,15 +250,15 @@ __global__ __launch_bounds__(1024) void k_argmax_finish(GemvArgs a, int nparts) 
   }
   __syncthreads();
   if (threadIdx.x == 0) {
-    for (int k = 1; k < 16; k++) argmax_merge(bv, bi, sv[k], si[k]);
+    for (int k = 1; k < 4; k++) argmax_merge(bv, bi, sv[k], si[k]);
     if (bi == 0x7fffffff) bi = 0;  // no comparable value (all NaN)
     *a.am_token64 = bi;
     if (a.am_tok) *a.am_tok = bi;
     if (a.am_hist) {
-      a.am_hist[*a.am_hist_n] = bi;
-      *a.am_hist_n = *a.am_hist_n + 1;
+      a.am_hist[hist_n] = bi;
+      *a.am_hist_n = hist_n + 1;
     }
-    if (a.am_pos) *a.am_pos = *a.am_pos + 1;
+    if (a.am_pos) *a.am_pos = pos + 1;
   }
 }
 
@@ -699,7 +705,7 @@ int launch_gemv(const WMat *w, GemvArgs a, int m) {
     hipLaunchKernelGGL(small ? v->fn_small : v->fn, grid, block, lds, s.stream, a);
     CTHIP_LAUNCH_CHECK();
     if (a.am_val) {
-      hipLaunchKernelGGL(k_argmax_finish, dim3(1), dim3(1024), 0, s.stream, a, nwaves);
+      hipLaunchKernelGGL(k_argmax_finish, dim3(1), dim3(256), 0, s.stream, a, nwaves);
       CTHIP_LAUNCH_CHECK();
     }
     return 0;
@@ -728,7 +734,7 @@ int launch_gemv(const WMat *w, GemvArgs a, int m) {
   }
   CTHIP_LAUNCH_CHECK();
   if (a.am_val) {
-    hipLaunchKernelGGL(k_argmax_finish, dim3(1), dim3(1024), 0, s.stream, a, (int)(grid.x * 4));
+    hipLaunchKernelGGL(k_argmax_finish, dim3(1), dim3(256), 0, s.stream, a, (int)(grid.x * 4));
     CTHIP_LAUNCH_CHECK();
   }
   if (tmp) return cthip_free(tmp);

@@ -34,7 +34,9 @@ def main():
     A = DeviceArray.from_numpy(rng.uniform(-1, 1, (n, n)).astype(np.float32))
     B = DeviceArray.from_numpy(rng.uniform(-1, 1, (n, n)).astype(np.float32))
     Cm = DeviceArray((n, n), np.float32)
-    for prec, name, peak in ((0, "fp32 MFMA", 157.3), (1, "bf16 MFMA / fp32 acc", 2500.0)):
+    for prec, name, peak in ((0, "fp32 MFMA", 157.3), (3, "bf16 MFMA, operands split in 3 terms (6 MFMAs per product), fp32 acc", 2500.0),
+                             (2, "bf16 MFMA, operands split in 2 terms (3 MFMAs per product), fp32 acc", 2500.0),
+                             (1, "bf16 MFMA / fp32 acc", 2500.0)):
         us = _time(lib, lambda: _lib.check(lib.cthip_matmul(Cm.ptr, A.ptr, B.ptr, n, n, n, _lib.ACT_RELU, prec)))
         tf = 2.0 * n ** 3 / (us * 1e-6) / 1e12
         out.append({"item": f"relu(matmul) 1024^3 {name}", "us": us, "achieved": tf, "unit": "TFLOP/s", "peak": peak,

@@ -10,6 +10,8 @@
 
 namespace cthip {
 
+constexpr int GEMM_BF16X3_DEFAULT = 2;
+
 // ---- process-wide state (one device, one in-order stream) ----
 struct State {
   bool inited = false;
@@ -17,7 +19,7 @@ struct State {
   hipStream_t stream = nullptr;
   int compute_units = 0;
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
-  int gemm_bf16 = 0;  // option "gemm_bf16": round MFMA operands of m > 1 Linear launches to bf16
+  int gemm_precision = GEMM_BF16X3_DEFAULT;  // option "gemm_precision" (GEMM_*) of m > 1 Linear launches
 };
 State &state();
 void set_error(const char *fmt, ...);
@@ -100,9 +102,11 @@ int launch_embedding(float *out, const float *W, const float *idx_f, const int *
                      const float *W2, const int *pos, int max_pos);
 int launch_argmax(int64_t *out, const float *x, int64_t rows, int n, int *tok_out, int *pos, int64_t *history,
                   int *hist_n);
-// Linear over m rows on the MFMA path (weights dequantised while staged); bf16 rounds the operands.
+// Linear over m rows on the MFMA path (weights dequantised while staged).  precision: fp32 MFMA operands,
+// operands rounded to bf16, or operands split in two / three bf16 terms (2^-16 / fp32-grade).
+enum { GEMM_FP32 = 0, GEMM_BF16 = 1, GEMM_BF16X3 = 2, GEMM_BF16X6 = 3 };
 int launch_linear_gemm(float *y, const WMat *w, const float *x, int m, const float *bias, const float *residual,
-                       int act, bool bf16);
+                       int act, int precision);
 // gate|up rows (m, 2*cols) -> silu(gate)*up (m, cols), or a norm, as a launch of its own
 int launch_prologue(float *out, const float *x, int cols, int pro, const float *g, const float *b, float eps,
                     int64_t x_stride, int m);

@@ -422,7 +422,7 @@ static int prefill(Decoder *d, const int *ids, int s, int n) {
   const bool gpt2 = c.arch == CTHIP_ARCH_GPT2;
   const int D = c.dim, F = c.ffn, V = c.vocab, KD = kv_dim(c), Dh = c.dim / c.n_heads;
   const int QW = D + 2 * KD, HW = gpt2 ? F : 2 * F;
-  const bool bf16 = state().gemm_bf16 != 0;
+  const int prec = state().gemm_precision;
   int rc = 0;
   float *X = nullptr, *XN = nullptr, *QKV = nullptr, *Q = nullptr, *ATT = nullptr, *Hb = nullptr, *G = nullptr;
   int *ids_dev = nullptr;
@@ -454,19 +454,19 @@ static int prefill(Decoder *d, const int *ids, int s, int n) {
     Layer &L = d->layers[l];
     if (gpt2) TRY(cthip_layernorm(XN, X, L.ln1_g, L.ln1_b, c.eps, s, D));
     else TRY(cthip_rmsnorm(XN, X, L.ln1_g, c.eps, s, D));
-    TRY(launch_linear_gemm(QKV, L.attn, XN, s, L.attn_b, nullptr, CTHIP_ACT_NONE, bf16));
+    TRY(launch_linear_gemm(QKV, L.attn, XN, s, L.attn_b, nullptr, CTHIP_ACT_NONE, prec));
     TRY(launch_qkv_split(Q, L.k_cache, L.v_cache, QKV, s, n, c.n_heads, c.n_kv_heads, Dh, gpt2 ? 0.0f : c.rope_base));
     TRY(launch_attn(ATT, Q, L.k_cache, L.v_cache, s, n, nullptr, n + s, c.n_heads, c.n_kv_heads, Dh));
-    TRY(launch_linear_gemm(X, L.proj, ATT, s, L.proj_b, X, CTHIP_ACT_NONE, bf16));
+    TRY(launch_linear_gemm(X, L.proj, ATT, s, L.proj_b, X, CTHIP_ACT_NONE, prec));
     if (gpt2) TRY(cthip_layernorm(XN, X, L.ln2_g, L.ln2_b, c.eps, s, D));
     else TRY(cthip_rmsnorm(XN, X, L.ln2_g, c.eps, s, D));
-    TRY(launch_linear_gemm(Hb, L.fc, XN, s, L.fc_b, nullptr, gpt2 ? CTHIP_ACT_GELU : CTHIP_ACT_NONE, bf16));
+    TRY(launch_linear_gemm(Hb, L.fc, XN, s, L.fc_b, nullptr, gpt2 ? CTHIP_ACT_GELU : CTHIP_ACT_NONE, prec));
     const float *hin = Hb;
     if (!gpt2) {
       TRY(launch_prologue(G, Hb, F, CTHIP_PRO_SWIGLU, nullptr, nullptr, 0.0f, 2 * (int64_t)F, s));
       hin = G;
     }
-    TRY(launch_linear_gemm(X, L.fc2, hin, s, L.fc2_b, X, CTHIP_ACT_NONE, bf16));
+    TRY(launch_linear_gemm(X, L.fc2, hin, s, L.fc2_b, X, CTHIP_ACT_NONE, prec));
   }
   // the last row continues through the decode-step head
   TRY(cthip_d2d(d->x, X + (size_t)(s - 1) * D, sizeof(float) * D));

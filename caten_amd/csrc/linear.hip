@@ -869,7 +869,7 @@ int cthip_linear(float *y, const void *wmat, const float *x, int m, const float 
       CTHIP_LAUNCH_CHECK();
       xin = tmp;
     }
-    rc = launch_linear_gemm(y, w, xin, m, bias, residual, act, state().gemm_bf16 != 0);
+    rc = launch_linear_gemm(y, w, xin, m, bias, residual, act, state().gemm_precision);
     if (tmp) cthip_free(tmp);
     return rc;
   }
@@ -890,8 +890,13 @@ int cthip_linear(float *y, const void *wmat, const float *x, int m, const float 
 
 int cthip_set_option(const char *name, int value) {
   if (!name) return fail(CTHIP_E_BAD_ARG, "cthip_set_option: null name");
-  if (!strcmp(name, "gemm_bf16")) {
-    state().gemm_bf16 = value != 0;
+  if (!strcmp(name, "gemm_precision")) {
+    if (value < GEMM_FP32 || value > GEMM_BF16X6) return fail(CTHIP_E_BAD_ARG, "cthip_set_option: gemm_precision is 0..3");
+    state().gemm_precision = value;
+    return 0;
+  }
+  if (!strcmp(name, "gemm_bf16")) {  // 1 = operands rounded to bf16, 0 = back to the default
+    state().gemm_precision = value ? GEMM_BF16 : GEMM_BF16X3;
     return 0;
   }
   return fail(CTHIP_E_BAD_ARG, "cthip_set_option: unknown option '%s'", name);

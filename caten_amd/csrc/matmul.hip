@@ -215,18 +215,349 @@ __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
   }
 }
 
-int launch_gemm(GemmArgs a, int bmode, bool bf16) {
+// ---------------------------------------------------------------------------------------------
+// bf16 MFMA GEMM with fp32 accumulation, operands optionally split in two bf16 terms.
+//
+// v_mfma_f32_32x32x16_bf16 runs at 16x the rate of the fp32-operand MFMA.  NS = 1 rounds both operands
+// to bf16 (rtol/atol 1e-2 class).  NS = 3 writes every operand as hi + lo with hi = bf16(x) and
+// lo = bf16(x - hi) and accumulates hi*hi + lo*hi + hi*lo: what is dropped is below 2^-16 of a product.
+// NS = 6 uses three terms per operand (24 significant bits: the fp32 value itself) and the six
+// products above 2^-24: fp32-grade results at a sixth of the bf16 rate, which is still 2.6 times the
+// fp32-operand MFMA peak.
+//
+// One 256-thread workgroup (2x2 wavefronts) owns a 64x64 tile of C and walks K in steps of 64.  The
+// fp32 (or packed) operands of a step are converted ONCE per workgroup on their way into LDS, which
+// holds them k-contiguous per row in bf16, 16-byte chunks swizzled by row so that neither the operand
+// reads nor the staging writes collide on banks.  Two LDS buffers and three register sets keep the
+// global loads three K-steps ahead of the MFMAs with one barrier per step.
+enum { W_ROWMAJOR = 0, W_F32 = 1, W_F16 = 2, W_Q4 = 3, W_Q8 = 4 };
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+typedef float v2f __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ unsigned pack_bf16(float x0, float x1) {  // round to nearest even, x0 in the low half
+  const unsigned lo = __builtin_bit_cast(unsigned short, (__bf16)x0), hi = __builtin_bit_cast(unsigned short, (__bf16)x1);
+  return lo | (hi << 16);
+}
+// 4 consecutive k -> NP planes of 4 bf16: plane 0 = bf16(x), plane p = bf16(what planes 0..p-1 miss)
+template <int NP>
+__device__ __forceinline__ void split4(const float x[4], uint2 *pl) {
+  float r[4] = {x[0], x[1], x[2], x[3]};
+#pragma unroll
+  for (int p = 0; p < NP; p++) {
+    pl[p].x = pack_bf16(r[0], r[1]);
+    pl[p].y = pack_bf16(r[2], r[3]);
+    if (p + 1 < NP) {  // exact: the difference of a float and its own leading bits
+      r[0] -= __uint_as_float(pl[p].x << 16);
+      r[1] -= __uint_as_float(pl[p].x & 0xffff0000u);
+      r[2] -= __uint_as_float(pl[p].y << 16);
+      r[3] -= __uint_as_float(pl[p].y & 0xffff0000u);
+    }
+  }
+}
+
+struct ARegs {  // one K-step of A held by a thread: rows ar + 16 i
+  float4 v0, v1, v2, v3;
+};
+
+template <int BMODE>
+struct BRegs {  // one K-step of B held by a thread between its request and its conversion
+  static constexpr int NV = (BMODE == W_ROWMAJOR || BMODE == W_F32) ? 4 : (BMODE == W_F16 ? 2 : 1);
+  uint4 v[NV];
+  unsigned short s;
+};
+
+// LDS rows are 64 bf16 = eight 16-byte chunks; chunk c of row r is stored at position c ^ swz(r), which
+// spreads the 128-bit operand reads of 8 consecutive rows, the 64-bit writes of the transposing B
+// staging and the row-wise A writes over all banks.
+__device__ __forceinline__ int swz(int row) { return (row ^ (row >> 3)) & 7; }
+
+template <int BMODE, int NS>
+__global__ __launch_bounds__(256) void k_gemm_split(GemmArgs a) {
+  constexpr int BM = 64, BN = 64, BK = 64, LDK = BK, NP = (NS == 1) ? 1 : (NS == 3) ? 2 : 3;
+  constexpr int NSET = 3;  // register sets = K-steps of global loads in flight
+  __shared__ __align__(16) unsigned short As[2][NP][BM][LDK];
+  __shared__ __align__(16) unsigned short Bs[2][NP][BN][LDK];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int tiles_m = (a.M + BM - 1) / BM;
+  const int m0 = (blockIdx.x % tiles_m) * BM, n0 = (blockIdx.x / tiles_m) * BN;
+  const int M = a.M, N = a.N, K = a.K;
+  const bool vecA = (K % 4 == 0), vecB = (N % 4 == 0);
+  v16f acc;
+#pragma unroll
+  for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+
+  // A: thread -> rows ar + 16 i (i < 4), k = 4 akq .. +3
+  const int ar = tid >> 4, akq = tid & 15;
+  // B row-major (K,N): thread -> the 4x4 block k = 4 bkq + j, n = 4 bnq .. +3
+  const int bkq = tid >> 4, bnq = tid & 15;
+  // B packed (N rows of K): thread -> weight row wr, k = 16 wkc .. +15
+  const int wr = tid >> 2, wkc = tid & 3;
+
+  auto fetch_a = [&](int k0, ARegs &ra) {
+    auto ld = [&](int i) {
+      const int row = m0 + ar + 16 * i, k = k0 + 4 * akq;
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (row < M) {
+        const float *src = a.A + (int64_t)row * K + k;
+        if (vecA && k + 4 <= K) {
+          v = *(const float4 *)src;
+        } else {
+          if (k + 0 < K) v.x = src[0];
+          if (k + 1 < K) v.y = src[1];
+          if (k + 2 < K) v.z = src[2];
+          if (k + 3 < K) v.w = src[3];
+        }
+      }
+      return v;
+    };
+    ra.v0 = ld(0);
+    ra.v1 = ld(1);
+    ra.v2 = ld(2);
+    ra.v3 = ld(3);
+  };
+  auto fetch_b = [&](int k0, BRegs<BMODE> &rb) {
+    if (BMODE == W_ROWMAJOR) {
+      auto ld = [&](int j) {
+        const int k = k0 + 4 * bkq + j, n = n0 + 4 * bnq;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (k < K) {
+          const float *src = a.B + (int64_t)k * N + n;
+          if (vecB && n + 4 <= N) {
+            v = *(const float4 *)src;
+          } else {
+            if (n + 0 < N) v.x = src[0];
+            if (n + 1 < N) v.y = src[1];
+            if (n + 2 < N) v.z = src[2];
+            if (n + 3 < N) v.w = src[3];
+          }
+        }
+        return make_uint4(__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z), __float_as_uint(v.w));
+      };
+      // constant indices only: the sets must stay in registers
+      rb.v[0] = ld(0);
+      rb.v[BRegs<BMODE>::NV > 1 ? 1 : 0] = ld(1);
+      rb.v[BRegs<BMODE>::NV > 2 ? 2 : 0] = ld(2);
+      rb.v[BRegs<BMODE>::NV > 3 ? 3 : 0] = ld(3);
+    } else {
+      // packed rows: K is a multiple of 32, so a 16-wide k chunk is inside the row or past its end
+      const int n = n0 + wr, k = k0 + 16 * wkc;
+      const bool ok = n < N && k < K;
+      rb.v[0] = make_uint4(0u, 0u, 0u, 0u);
+      if (BRegs<BMODE>::NV > 1) rb.v[BRegs<BMODE>::NV > 1 ? 1 : 0] = make_uint4(0u, 0u, 0u, 0u);
+      if (BRegs<BMODE>::NV > 2) {
+        rb.v[BRegs<BMODE>::NV > 2 ? 2 : 0] = make_uint4(0u, 0u, 0u, 0u);
+        rb.v[BRegs<BMODE>::NV > 3 ? 3 : 0] = make_uint4(0u, 0u, 0u, 0u);
+      }
+      rb.s = 0;
+      if (ok) {
+        const int64_t e = (int64_t)n * K + k;  // element index of the chunk
+        if (BMODE == W_F32) {
+          rb.v[0] = *(const uint4 *)((const float *)a.wq + e);
+          rb.v[BRegs<BMODE>::NV > 1 ? 1 : 0] = *(const uint4 *)((const float *)a.wq + e + 4);
+          rb.v[BRegs<BMODE>::NV > 2 ? 2 : 0] = *(const uint4 *)((const float *)a.wq + e + 8);
+          rb.v[BRegs<BMODE>::NV > 3 ? 3 : 0] = *(const uint4 *)((const float *)a.wq + e + 12);
+        } else if (BMODE == W_F16) {
+          rb.v[0] = *(const uint4 *)((const unsigned short *)a.wq + e);
+          rb.v[BRegs<BMODE>::NV > 1 ? 1 : 0] = *(const uint4 *)((const unsigned short *)a.wq + e + 8);
+        } else if (BMODE == W_Q8) {
+          rb.v[0] = *(const uint4 *)((const int8_t *)a.wq + e);
+          rb.s = a.wd[e >> 5];
+        } else {  // W_Q4: the 32-weight block's 16 bytes; this chunk is its low (k % 32 == 0) or high nibbles
+          rb.v[0] = *(const uint4 *)((const uint8_t *)a.wq + ((e >> 5) << 4));
+          rb.s = a.wd[e >> 5];
+        }
+      }
+    }
+  };
+  auto stage_a = [&](const ARegs &ra, int buf) {
+    auto put = [&](int i, const float4 v) {
+      const float x[4] = {v.x, v.y, v.z, v.w};
+      uint2 pl[NP];
+      split4<NP>(x, pl);
+#pragma unroll
+      for (int p = 0; p < NP; p++)
+        *(uint2 *)&As[buf][p][ar + 16 * i][8 * ((akq >> 1) ^ swz(ar + 16 * i)) + 4 * (akq & 1)] = pl[p];
+    };
+    put(0, ra.v0);
+    put(1, ra.v1);
+    put(2, ra.v2);
+    put(3, ra.v3);
+  };
+  auto stage_b = [&](const BRegs<BMODE> &rb, int buf) {
+    if (BMODE == W_ROWMAJOR) {
+      // column 4 bnq + i gets its 4 consecutive k: a 4x4 transpose in registers
+      auto put = [&](int i, unsigned x0, unsigned x1, unsigned x2, unsigned x3) {
+        const float x[4] = {__uint_as_float(x0), __uint_as_float(x1), __uint_as_float(x2), __uint_as_float(x3)};
+        uint2 pl[NP];
+        split4<NP>(x, pl);
+#pragma unroll
+        for (int p = 0; p < NP; p++)
+          *(uint2 *)&Bs[buf][p][4 * bnq + i][8 * ((bkq >> 1) ^ swz(4 * bnq + i)) + 4 * (bkq & 1)] = pl[p];
+      };
+      put(0, rb.v[0].x, rb.v[1].x, rb.v[2].x, rb.v[3].x);
+      put(1, rb.v[0].y, rb.v[1].y, rb.v[2].y, rb.v[3].y);
+      put(2, rb.v[0].z, rb.v[1].z, rb.v[2].z, rb.v[3].z);
+      put(3, rb.v[0].w, rb.v[1].w, rb.v[2].w, rb.v[3].w);
+    } else {
+      float x[16];
+      if (BMODE == W_F32) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          const uint4 q = rb.v[j];
+          x[4 * j + 0] = __uint_as_float(q.x);
+          x[4 * j + 1] = __uint_as_float(q.y);
+          x[4 * j + 2] = __uint_as_float(q.z);
+          x[4 * j + 3] = __uint_as_float(q.w);
+        }
+      } else if (BMODE == W_F16) {
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+          const uint4 q = rb.v[BRegs<BMODE>::NV > 1 ? j : 0];
+          const unsigned dw[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+          for (int t = 0; t < 4; t++) {
+            x[8 * j + 2 * t] = half_bits_to_float((unsigned short)(dw[t] & 0xffff));
+            x[8 * j + 2 * t + 1] = half_bits_to_float((unsigned short)(dw[t] >> 16));
+          }
+        }
+      } else if (BMODE == W_Q8) {
+        const float d = half_bits_to_float(rb.s);
+        const unsigned dw[4] = {rb.v[0].x, rb.v[0].y, rb.v[0].z, rb.v[0].w};
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+          const int v = (int)dw[t];
+          x[4 * t + 0] = (float)(int)(int8_t)(v)*d;
+          x[4 * t + 1] = (float)(int)(int8_t)(v >> 8) * d;
+          x[4 * t + 2] = (float)(int)(int8_t)(v >> 16) * d;
+          x[4 * t + 3] = (float)(v >> 24) * d;
+        }
+      } else {
+        const float d = half_bits_to_float(rb.s);
+        const unsigned dw[4] = {rb.v[0].x, rb.v[0].y, rb.v[0].z, rb.v[0].w};
+        const int sh = (wkc & 1) ? 4 : 0;  // BK = 64 = two blocks: chunks 0, 2 are low nibbles, 1, 3 high
+#pragma unroll
+        for (int t = 0; t < 16; t++) x[t] = (float)((int)((dw[t >> 2] >> (8 * (t & 3) + sh)) & 0xf) - 8) * d;
+      }
+#pragma unroll
+      for (int j = 0; j < 2; j++) {
+        uint2 p0[NP], p1[NP];
+        split4<NP>(x + 8 * j, p0);
+        split4<NP>(x + 8 * j + 4, p1);
+#pragma unroll
+        for (int p = 0; p < NP; p++)
+          *(uint4 *)&Bs[buf][p][wr][8 * ((2 * wkc + j) ^ swz(wr))] = make_uint4(p0[p].x, p0[p].y, p1[p].x, p1[p].y);
+      }
+    }
+  };
+  auto mma = [&](int buf) {
+    // 32x32x16: lane l holds A[i = l%32][k = 8*(l/32) .. +7] and B[k = 8*(l/32) .. +7][j = l%32]
+#pragma unroll
+    for (int s = 0; s < BK / 16; s++) {
+      const int ch = 2 * s + (lane >> 5), rowa = 32 * wm + (lane & 31), rowb = 32 * wn + (lane & 31);
+      v8bf av[NP], bv[NP];
+#pragma unroll
+      for (int p = 0; p < NP; p++) {
+        av[p] = __builtin_bit_cast(v8bf, *(const uint4 *)&As[buf][p][rowa][8 * (ch ^ swz(rowa))]);
+        bv[p] = __builtin_bit_cast(v8bf, *(const uint4 *)&Bs[buf][p][rowb][8 * (ch ^ swz(rowb))]);
+      }
+      // every pair of planes whose product is above 2^-8(NP) of the leading one, smallest first
+#pragma unroll
+      for (int t = NP - 1; t >= 0; t--) {
+#pragma unroll
+        for (int p = 0; p <= t; p++) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[p], bv[t - p], acc, 0, 0, 0);
+      }
+    }
+  };
+
+  ARegs ra0, ra1, ra2;  // separate objects with named members: every set stays in registers
+  BRegs<BMODE> rb0, rb1, rb2;
+  const int nsteps = (K + BK - 1) / BK;
+  if (nsteps > 0) {
+    fetch_a(0, ra0);
+    fetch_b(0, rb0);
+  }
+  if (nsteps > 1) {
+    fetch_a(BK, ra1);
+    fetch_b(BK, rb1);
+  }
+  if (nsteps > 2) {
+    fetch_a(2 * BK, ra2);
+    fetch_b(2 * BK, rb2);
+  }
+  if (nsteps > 0) {
+    stage_a(ra0, 0);
+    stage_b(rb0, 0);
+  }
+  if (nsteps > 3) {
+    fetch_a(3 * BK, ra0);
+    fetch_b(3 * BK, rb0);
+  }
+  __syncthreads();
+  // step i: LDS buffer i%2 holds it; register set (i+1) % NSET holds step i+1, requested NSET steps ago
+  auto step = [&](int i, ARegs &ran, BRegs<BMODE> &rbn) {
+    if (i + 1 < nsteps) {
+      stage_a(ran, (i + 1) & 1);
+      stage_b(rbn, (i + 1) & 1);
+    }
+    if (i + 1 + NSET < nsteps) {
+      fetch_a((i + 1 + NSET) * BK, ran);
+      fetch_b((i + 1 + NSET) * BK, rbn);
+    }
+    mma(i & 1);
+    __syncthreads();
+  };
+  static_assert(NSET == 3, "the loop below is unrolled by hand over the register sets");
+  for (int i = 0; i < nsteps; i += NSET) {
+    step(i, ra1, rb1);
+    if (i + 1 < nsteps) step(i + 1, ra2, rb2);
+    if (i + 2 < nsteps) step(i + 2, ra0, rb0);
+  }
+  // ---- epilogue: acc[r] is C[row = 8*(r/4) + 4*(l/32) + r%4][col = l%32] of the 32x32 sub-tile ----
+  const int col = n0 + 32 * wn + (lane & 31);
+  if (col < N) {
+    const float bias = a.bias ? a.bias[col] : 0.0f;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int row = m0 + 32 * wm + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+      if (row < M) {
+        float v = apply_act(a.act, acc[r] + bias);
+        if (a.residual) v += a.residual[(int64_t)row * N + col];
+        a.C[(int64_t)row * N + col] = v;
+      }
+    }
+  }
+}
+
+// precision: GEMM_FP32 = fp32 MFMA operands (k_gemm), GEMM_BF16 = operands rounded to bf16,
+// GEMM_BF16X3 / GEMM_BF16X6 = operands split in two / three bf16 terms
+int launch_gemm(GemmArgs a, int bmode, int precision) {
   if (a.M == 0 || a.N == 0) return 0;
   const int64_t tiles = (int64_t)((a.M + 63) / 64) * ((a.N + 63) / 64);
   if (tiles > 0x7fffffff) return fail(CTHIP_E_BAD_ARG, "gemm: too many tiles");
   dim3 grid((unsigned)tiles), block(256);
   hipStream_t st = state().stream;
-  if (bmode == B_ROWMAJOR) {
-    if (bf16) hipLaunchKernelGGL((k_gemm<B_ROWMAJOR, true>), grid, block, 0, st, a);
-    else hipLaunchKernelGGL((k_gemm<B_ROWMAJOR, false>), grid, block, 0, st, a);
-  } else {
-    if (bf16) hipLaunchKernelGGL((k_gemm<B_WMAT, true>), grid, block, 0, st, a);
+  if (precision == GEMM_FP32) {
+    if (bmode == B_ROWMAJOR) hipLaunchKernelGGL((k_gemm<B_ROWMAJOR, false>), grid, block, 0, st, a);
     else hipLaunchKernelGGL((k_gemm<B_WMAT, false>), grid, block, 0, st, a);
+  } else {
+    int wm = W_ROWMAJOR;
+    if (bmode == B_WMAT) wm = a.wtype == CTHIP_Q8_0 ? W_Q8 : a.wtype == CTHIP_Q4_0 ? W_Q4 : a.wtype == CTHIP_F16 ? W_F16 : W_F32;
+#define SPLIT(MODE)                                                                                          \
+  case MODE:                                                                                                 \
+    if (precision == GEMM_BF16X6) hipLaunchKernelGGL((k_gemm_split<MODE, 6>), grid, block, 0, st, a);        \
+    else if (precision == GEMM_BF16X3) hipLaunchKernelGGL((k_gemm_split<MODE, 3>), grid, block, 0, st, a);   \
+    else hipLaunchKernelGGL((k_gemm_split<MODE, 1>), grid, block, 0, st, a);                                 \
+    break
+    switch (wm) {
+      SPLIT(W_ROWMAJOR);
+      SPLIT(W_F32);
+      SPLIT(W_F16);
+      SPLIT(W_Q4);
+      SPLIT(W_Q8);
+    }
+#undef SPLIT
   }
   CTHIP_LAUNCH_CHECK();
   return 0;
@@ -234,7 +565,7 @@ int launch_gemm(GemmArgs a, int bmode, bool bf16) {
 
 // Linear over m rows with packed weights: y (m, rows) = act(x (m, cols) @ W^T + bias) + residual
 int launch_linear_gemm(float *y, const WMat *w, const float *x, int m, const float *bias, const float *residual,
-                       int act, bool bf16) {
+                       int act, int precision) {
   GemmArgs a = {};
   a.C = y;
   a.A = x;
@@ -247,7 +578,7 @@ int launch_linear_gemm(float *y, const WMat *w, const float *x, int m, const flo
   a.N = (int)w->rows;
   a.K = (int)w->cols;
   a.act = act;
-  return launch_gemm(a, B_WMAT, bf16);
+  return launch_gemm(a, B_WMAT, precision);
 }
 
 }  // namespace cthip
@@ -259,7 +590,7 @@ extern "C" int cthip_matmul(float *C, const float *A, const float *B, int M, int
   CTHIP_ARG(M >= 0 && N >= 0 && K >= 0);
   CTHIP_ARG((int64_t)M * N == 0 || (C != nullptr && (K == 0 || (A != nullptr && B != nullptr))));
   CTHIP_ARG(act >= CTHIP_ACT_NONE && act <= CTHIP_ACT_TANH);
-  CTHIP_ARG(precision == 0 || precision == 1);
+  CTHIP_ARG(precision >= GEMM_FP32 && precision <= GEMM_BF16X6);
   GemmArgs a = {};
   a.C = C;
   a.A = A;
@@ -268,5 +599,5 @@ extern "C" int cthip_matmul(float *C, const float *A, const float *B, int M, int
   a.N = N;
   a.K = K;
   a.act = act;
-  return launch_gemm(a, B_ROWMAJOR, precision == 1);
+  return launch_gemm(a, B_ROWMAJOR, precision);
 }

@@ -126,8 +126,11 @@ def linear(x, w: WeightMatrix, bias=None, residual=None, act=None, prologue=None
     return y.numpy()
 
 
-def matmul(A, B, relu: bool = False, precision: str = "fp32") -> np.ndarray:
-    """!matmul (+ fused !relu) (api/high-level-ops.lisp:76-99)."""
+def matmul(A, B, relu: bool = False, precision: str = "bf16x6") -> np.ndarray:
+    """!matmul (+ fused !relu) (api/high-level-ops.lisp:76-99).
+
+    precision: "fp32" = fp32 MFMA operands; "bf16x6" (default) = operands split in three bf16 terms,
+    fp32-grade; "bf16x3" = two terms (2^-16 per product); "bf16" = operands rounded to bf16."""
     A, B = np.ascontiguousarray(A, np.float32), np.ascontiguousarray(B, np.float32)
     M, K = A.shape
     K2, N = B.shape
@@ -135,7 +138,7 @@ def matmul(A, B, relu: bool = False, precision: str = "fp32") -> np.ndarray:
         raise ValueError("matmul: inner dimensions differ")
     dA, dB, dC = _dev(A), _dev(B), DeviceArray((M, N), np.float32)
     _lib.check(_lib.load().cthip_matmul(dC.ptr, dA.ptr, dB.ptr, M, N, K, _lib.ACT_RELU if relu else _lib.ACT_NONE,
-                                        {"fp32": 0, "bf16": 1}[precision]))
+                                        {"fp32": 0, "bf16": 1, "bf16x3": 2, "bf16x6": 3}[precision]))
     return dC.numpy()
 
 

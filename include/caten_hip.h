@@ -153,14 +153,20 @@ int cthip_linear(float *y, const void *wmat, const float *x, int m, const float 
                  const float *residual, int act, int prologue, const float *norm_g,
                  const float *norm_b, float eps);
 
-/* Library options.  "gemm_bf16" = 1: Linear launches with m >= 8 input rows (prefill) round their MFMA
- * operands to bf16 (fp32 accumulation; rtol/atol 1e-2 instead of 1e-3/1e-4).  Default 0. */
+/* Library options.
+ * "gemm_precision": operand format of the MFMA launches behind cthip_linear with m >= 8 input rows and
+ *   the decoder's prefill: 2 (default) = every operand split into two bf16 terms, three bf16 MFMAs
+ *   per product, fp32 accumulation (2^-16 of a product is lost); 3 = three terms, six MFMAs per
+ *   product: all 24 bits of an fp32 operand; 0 = fp32 MFMA operands; 1 = operands rounded to bf16
+ *   (rtol/atol 1e-2).
+ * "gemm_bf16": 1 = shorthand for gemm_precision 1, 0 = back to the default. */
 int cthip_set_option(const char *name, int value);
 
 /* !relu(!matmul A B) (api/high-level-ops.lisp:76-99; fused per test-scheduler.lisp:140-163):
- * C (M,N) = act(A (M,K) @ B (K,N)), row-major fp32.  precision 0 = fp32 MFMA
- * accumulate-in-order-free fp32 (rtol 1e-3/atol 1e-4), 1 = bf16 MFMA inputs with
- * fp32 accumulation (rtol/atol 1e-2). */
+ * C (M,N) = act(A (M,K) @ B (K,N)), row-major fp32.  precision 0 = fp32 MFMA operands,
+ * 3 = operands split into three bf16 terms (both rtol 1e-3/atol 1e-4), 2 = two bf16 terms
+ * (2^-16 of a product is lost), 1 = bf16 MFMA operands (rtol/atol 1e-2); fp32 accumulation
+ * in every mode. */
 int cthip_matmul(float *C, const float *A, const float *B, int M, int N, int K, int act, int precision);
 
 /* Row ops over the last axis, fp32, rows x n contiguous. */

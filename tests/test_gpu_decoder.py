@@ -65,6 +65,23 @@ def test_gpt2_generate_matches_oracle(oracle, name, kind):
     model.close()
 
 
+def test_gpt2_long_context_attention(oracle):
+    """Positions past 512: the attention kernel walks the cache in several passes."""
+    print("case: gpt2 decode to position 600", flush=True)
+    from caten_amd import synth, llm
+    cfg = dict(synth.GPT2_CONFIGS["gpt2-tiny"], max_seq=640)
+    w = synth.gpt2_weights(cfg, seed=6)
+    prompt = synth.prompt(cfg["vocab"], 250, seed=6)
+    steps = 350
+    ref = oracle.GPT2(cfg, _dequantised(oracle, w, synth.GPT2_LINEAR_KEYS + ("lm_head",), "q8_0"))
+    want = ref.generate(prompt, steps)
+    model = llm.make_gpt2(cfg, llm.gpt2_state_dict(w, "q8_0"))
+    assert llm.gpt2_generate(model, prompt, steps, on_device=True) == want
+    T = len(prompt) + steps - 1
+    close(model.peek("k_cache.1")[:T * cfg["dim"]], ref.k_cache[1].ravel()[:T * cfg["dim"]])
+    model.close()
+
+
 def test_gpt2_prompt_lengths_and_restart(oracle):
     from caten_amd import synth, llm
     cfg = synth.GPT2_CONFIGS["gpt2-tiny"]

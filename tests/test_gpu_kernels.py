@@ -274,8 +274,11 @@ def test_matmul_relu_vs_oracle(ops, oracle, M, N, K):
     rng = np.random.default_rng(M * 31 + N * 7 + K)
     A = rng.uniform(-1, 1, (M, K)).astype(np.float32)
     B = rng.uniform(-1, 1, (K, N)).astype(np.float32)
-    close(ops.matmul(A, B, relu=True), oracle.matmul(A, B, relu=True))
-    close(ops.matmul(A, B), oracle.matmul(A, B))
+    for precision in ("fp32", "bf16x6"):  # both hold the fp32 bar
+        close(ops.matmul(A, B, relu=True, precision=precision), oracle.matmul(A, B, relu=True))
+        close(ops.matmul(A, B, precision=precision), oracle.matmul(A, B))
+    # two bf16 terms per operand: 2^-16 of a product is lost, sqrt(K) of them add up
+    close(ops.matmul(A, B, relu=True, precision="bf16x3"), oracle.matmul(A, B, relu=True), 1e-3, 2e-5 * np.sqrt(K))
     close(ops.matmul(A, B, relu=True, precision="bf16"), oracle.matmul(A, B, relu=True), 1e-2, 1e-2 * np.sqrt(K))
 
 
@@ -285,11 +288,16 @@ def test_matmul_1024_cubed(ops):
     A = rng.uniform(-1, 1, (1024, 1024)).astype(np.float32)
     B = rng.uniform(-1, 1, (1024, 1024)).astype(np.float32)
     want = np.maximum(A.astype(np.float64) @ B.astype(np.float64), 0)
-    close(ops.matmul(A, B, relu=True), want)
+    close(ops.matmul(A, B, relu=True, precision="fp32"), want)
+    got = ops.matmul(A, B, relu=True, precision="bf16x6")
+    close(got, want)
+    assert np.max(np.abs(got - want)) < 1e-4  # three bf16 terms carry all 24 bits; what is left is fp32 accumulation
+    assert np.max(np.abs(ops.matmul(A, B, relu=True, precision="bf16x3") - want)) < 6e-4
     got = ops.matmul(A, B, relu=True, precision="bf16")
     assert np.max(np.abs(got - want)) < 1e-2 * np.sqrt(1024) and np.all(got >= 0)
     # all-ones closed form (test-runtime.lisp:241-252): every entry is K
-    assert np.all(ops.matmul(np.ones((64, 96), np.float32), np.ones((96, 32), np.float32)) == 96)
+    for precision in ("fp32", "bf16x6", "bf16x3", "bf16"):
+        assert np.all(ops.matmul(np.ones((64, 96), np.float32), np.ones((96, 32), np.float32), precision=precision) == 96)
 
 
 def test_matmul_degenerate(ops):
@@ -313,13 +321,18 @@ def test_linear_prefill_rows_mfma(ops, oracle, kind):
     t = Tensor.from_f32(w, kind)
     wd = oracle.dequant(kind, t.raw, w.size).reshape(rows, cols)
     wm = ops.WeightMatrix(kind, t.raw, rows, cols)
-    close(ops.linear(x, wm, bias=b, residual=r), oracle.linear(x, wd, b) + r)
     want = oracle.gelu_tanh(oracle.linear(oracle.layernorm(x, g, be), wd, b))
-    close(ops.linear(x, wm, bias=b, act="gelu", prologue="layernorm", norm_g=g, norm_b=be), want)
-    _lib.check(_lib.load().cthip_set_option(b"gemm_bf16", 1))
+    lib = _lib.load()
     try:
+        for mode in (2, 3, 0):  # split bf16 operands (two terms = the default, three terms), fp32 operands
+            _lib.check(lib.cthip_set_option(b"gemm_precision", mode))
+            close(ops.linear(x, wm, bias=b, residual=r), oracle.linear(x, wd, b) + r)
+            close(ops.linear(x, wm, bias=b, act="gelu", prologue="layernorm", norm_g=g, norm_b=be), want)
+        _lib.check(lib.cthip_set_option(b"gemm_bf16", 1))
         close(ops.linear(x, wm, bias=b, residual=r), oracle.linear(x, wd, b) + r, 1e-2, 1e-2)
     finally:
-        _lib.check(_lib.load().cthip_set_option(b"gemm_bf16", 0))
+        _lib.check(lib.cthip_set_option(b"gemm_bf16", 0))
+    with pytest.raises(_lib.HipError):
+        _lib.check(lib.cthip_set_option(b"gemm_precision", 4))
     with pytest.raises(_lib.HipError):
         _lib.check(_lib.load().cthip_set_option(b"no_such_option", 1))

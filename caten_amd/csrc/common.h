@@ -22,6 +22,8 @@ struct State {
   int gemm_precision = GEMM_BF16X3_DEFAULT;  // option "gemm_precision" (GEMM_*) of m > 1 Linear launches
 };
 State &state();
+// cthip_alloc without the zero fill, for temporaries that are fully written before they are read
+int alloc_scratch(void **out, size_t bytes);
 void set_error(const char *fmt, ...);
 int fail(int code, const char *fmt, ...);
 

@@ -428,7 +428,7 @@ static int prefill(Decoder *d, const int *ids, int s, int n) {
   int *ids_dev = nullptr;
   std::vector<void *> tmp;
   auto alloc = [&](void **p, size_t bytes) {
-    int r = cthip_alloc(p, bytes);
+    int r = alloc_scratch(p, bytes);  // every temporary below is fully written before it is read
     if (r == 0) tmp.push_back(*p);
     return r;
   };

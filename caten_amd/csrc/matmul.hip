@@ -29,6 +29,10 @@ struct GemmArgs {
   const float *residual; // (M,N), may be null
   int M, N, K;
   int act;
+  // split-K (k_gemm_split only): workgroup (tile, z) covers k in [z * kper, (z + 1) * kper) and writes
+  // its raw partial tile to ws[z][M][N]; k_splitk_reduce adds the partials in z order and applies the epilogue
+  int ksplit, kper;
+  float *ws;
 };
 
 __device__ __forceinline__ unsigned short f32_to_bf16_bits(float f) {
@@ -282,8 +286,10 @@ __global__ __launch_bounds__(256) void k_gemm_split(GemmArgs a) {
   const int wm = wave >> 1, wn = wave & 1;
   const int tiles_m = (a.M + BM - 1) / BM;
   const int m0 = (blockIdx.x % tiles_m) * BM, n0 = (blockIdx.x / tiles_m) * BN;
-  const int M = a.M, N = a.N, K = a.K;
-  const bool vecA = (K % 4 == 0), vecB = (N % 4 == 0);
+  const int M = a.M, N = a.N, ldk = a.K;
+  const int kbeg = blockIdx.y * a.kper;      // this workgroup's share of the reduction axis
+  const int K = min(a.K, kbeg + a.kper);
+  const bool vecA = (ldk % 4 == 0), vecB = (N % 4 == 0);
   v16f acc;
 #pragma unroll
   for (int r = 0; r < 16; r++) acc[r] = 0.0f;
@@ -295,12 +301,12 @@ __global__ __launch_bounds__(256) void k_gemm_split(GemmArgs a) {
   // B packed (N rows of K): thread -> weight row wr, k = 16 wkc .. +15
   const int wr = tid >> 2, wkc = tid & 3;
 
-  auto fetch_a = [&](int k0, ARegs &ra) {
+  auto fetch_a = [&](int k0, ARegs &ra) {  // k0 counts from kbeg
     auto ld = [&](int i) {
-      const int row = m0 + ar + 16 * i, k = k0 + 4 * akq;
+      const int row = m0 + ar + 16 * i, k = kbeg + k0 + 4 * akq;
       float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
       if (row < M) {
-        const float *src = a.A + (int64_t)row * K + k;
+        const float *src = a.A + (int64_t)row * ldk + k;
         if (vecA && k + 4 <= K) {
           v = *(const float4 *)src;
         } else {
@@ -320,7 +326,7 @@ __global__ __launch_bounds__(256) void k_gemm_split(GemmArgs a) {
   auto fetch_b = [&](int k0, BRegs<BMODE> &rb) {
     if (BMODE == W_ROWMAJOR) {
       auto ld = [&](int j) {
-        const int k = k0 + 4 * bkq + j, n = n0 + 4 * bnq;
+        const int k = kbeg + k0 + 4 * bkq + j, n = n0 + 4 * bnq;
         float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
         if (k < K) {
           const float *src = a.B + (int64_t)k * N + n;
@@ -342,7 +348,7 @@ __global__ __launch_bounds__(256) void k_gemm_split(GemmArgs a) {
       rb.v[BRegs<BMODE>::NV > 3 ? 3 : 0] = ld(3);
     } else {
       // packed rows: K is a multiple of 32, so a 16-wide k chunk is inside the row or past its end
-      const int n = n0 + wr, k = k0 + 16 * wkc;
+      const int n = n0 + wr, k = kbeg + k0 + 16 * wkc;
       const bool ok = n < N && k < K;
       rb.v[0] = make_uint4(0u, 0u, 0u, 0u);
       if (BRegs<BMODE>::NV > 1) rb.v[BRegs<BMODE>::NV > 1 ? 1 : 0] = make_uint4(0u, 0u, 0u, 0u);
@@ -352,7 +358,7 @@ __global__ __launch_bounds__(256) void k_gemm_split(GemmArgs a) {
       }
       rb.s = 0;
       if (ok) {
-        const int64_t e = (int64_t)n * K + k;  // element index of the chunk
+        const int64_t e = (int64_t)n * ldk + k;  // element index of the chunk
         if (BMODE == W_F32) {
           rb.v[0] = *(const uint4 *)((const float *)a.wq + e);
           rb.v[BRegs<BMODE>::NV > 1 ? 1 : 0] = *(const uint4 *)((const float *)a.wq + e + 4);
@@ -473,7 +479,7 @@ __global__ __launch_bounds__(256) void k_gemm_split(GemmArgs a) {
 
   ARegs ra0, ra1, ra2;  // separate objects with named members: every set stays in registers
   BRegs<BMODE> rb0, rb1, rb2;
-  const int nsteps = (K + BK - 1) / BK;
+  const int nsteps = K > kbeg ? (K - kbeg + BK - 1) / BK : 0;
   if (nsteps > 0) {
     fetch_a(0, ra0);
     fetch_b(0, rb0);
@@ -517,6 +523,15 @@ __global__ __launch_bounds__(256) void k_gemm_split(GemmArgs a) {
   // ---- epilogue: acc[r] is C[row = 8*(r/4) + 4*(l/32) + r%4][col = l%32] of the 32x32 sub-tile ----
   const int col = n0 + 32 * wn + (lane & 31);
   if (col < N) {
+    if (a.ksplit > 1) {
+      float *ws = a.ws + (int64_t)blockIdx.y * M * N;
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int row = m0 + 32 * wm + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        if (row < M) ws[(int64_t)row * N + col] = acc[r];
+      }
+      return;
+    }
     const float bias = a.bias ? a.bias[col] : 0.0f;
 #pragma unroll
     for (int r = 0; r < 16; r++) {
@@ -530,6 +545,19 @@ __global__ __launch_bounds__(256) void k_gemm_split(GemmArgs a) {
   }
 }
 
+// C = act(sum_z ws[z] + bias) + residual, z in ascending order (the result does not depend on timing)
+__global__ __launch_bounds__(256) void k_splitk_reduce(GemmArgs a) {
+  const int64_t n = (int64_t)a.M * a.N;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+    float v = a.ws[i];
+    for (int z = 1; z < a.ksplit; z++) v += a.ws[(int64_t)z * n + i];
+    if (a.bias) v += a.bias[i % a.N];
+    v = apply_act(a.act, v);
+    if (a.residual) v += a.residual[i];
+    a.C[i] = v;
+  }
+}
+
 // precision: GEMM_FP32 = fp32 MFMA operands (k_gemm), GEMM_BF16 = operands rounded to bf16,
 // GEMM_BF16X3 / GEMM_BF16X6 = operands split in two / three bf16 terms
 int launch_gemm(GemmArgs a, int bmode, int precision) {
@@ -538,6 +566,28 @@ int launch_gemm(GemmArgs a, int bmode, int precision) {
   if (tiles > 0x7fffffff) return fail(CTHIP_E_BAD_ARG, "gemm: too many tiles");
   dim3 grid((unsigned)tiles), block(256);
   hipStream_t st = state().stream;
+  a.ksplit = 1;
+  a.kper = a.K > 0 ? a.K : 1;
+  a.ws = nullptr;
+  if (precision != GEMM_FP32) {
+    // too few tiles to occupy the chip and a long reduction axis: split K over several workgroups per tile
+    const int cus = state().compute_units, nsteps = (a.K + 63) / 64;
+    int ks = (int)((cus * 3 / 2) / tiles);
+    if (ks > nsteps / 6) ks = nsteps / 6;
+    if (ks > 16) ks = 16;
+    if (ks > 1) {
+      const int steps_per = (nsteps + ks - 1) / ks;
+      a.kper = steps_per * 64;
+      a.ksplit = (nsteps + steps_per - 1) / steps_per;
+      if (a.ksplit > 1) {
+        int rc = alloc_scratch((void **)&a.ws, sizeof(float) * (size_t)a.ksplit * a.M * a.N);
+        if (rc) return rc;
+        grid.y = a.ksplit;
+      } else {
+        a.kper = a.K;
+      }
+    }
+  }
   if (precision == GEMM_FP32) {
     if (bmode == B_ROWMAJOR) hipLaunchKernelGGL((k_gemm<B_ROWMAJOR, false>), grid, block, 0, st, a);
     else hipLaunchKernelGGL((k_gemm<B_WMAT, false>), grid, block, 0, st, a);
@@ -560,6 +610,13 @@ int launch_gemm(GemmArgs a, int bmode, int precision) {
 #undef SPLIT
   }
   CTHIP_LAUNCH_CHECK();
+  if (a.ksplit > 1) {
+    int64_t blocks = ((int64_t)a.M * a.N + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(k_splitk_reduce, dim3((unsigned)blocks), dim3(256), 0, st, a);
+    CTHIP_LAUNCH_CHECK();
+    return cthip_free(a.ws);  // stream-ordered: the block is reused only by later work on the same stream
+  }
   return 0;
 }
 

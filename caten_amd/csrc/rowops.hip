@@ -468,11 +468,148 @@ __global__ __launch_bounds__(1024) void k_attn_cached(float *__restrict__ out, c
   }
 }
 
+// sum over aligned groups of LPK lanes (8, 16 or 32), every lane gets the sum
+template <int LPK>
+__device__ __forceinline__ float lpk_sum(float v) {
+  v += dpp_f<0xB1>(v);   // quad_perm [1,0,3,2]
+  v += dpp_f<0x4E>(v);   // quad_perm [2,3,0,1]
+  v += dpp_f<0x141>(v);  // row_half_mirror: 8 lanes
+  if (LPK >= 16) v += dpp_f<0x140>(v);  // row_mirror: 16 lanes
+  if (LPK >= 32) v += __shfl_xor(v, 16, 64);
+  return v;
+}
+
+// Prompt rows (s > 1): one 256-thread block per (head, group of R consecutive query rows).  The group
+// shares every K / V tile it loads, so the cache is read once per R rows instead of once per row; the
+// causal mask (layers.lisp:83) is applied per row.  Same lane layout and per-wavefront online softmax
+// as k_attn_cached, with R running (max, sum, output) triples.
+template <int DH, int R>
+__global__ __launch_bounds__(256) void k_attn_rows(float *__restrict__ out, const float *__restrict__ q,
+                                                   const float *__restrict__ kc, const float *__restrict__ vc, int S,
+                                                   int start_pos, const int *__restrict__ pos, int H, int Hkv) {
+  constexpr int LPK = DH / 4, KPW = 64 / LPK, KPT = 8, NW = 4, TILE = NW * KPW * KPT;
+  __shared__ float part[NW][R][DH];
+  __shared__ float pm[NW][R], pl[NW][R];
+  const int h = blockIdx.x, i0 = blockIdx.y * R;
+  const int base = start_pos + (pos ? pos[0] : 0);
+  const int nrows = min(R, S - i0);
+  const int Tmax = base + i0 + nrows;  // keys the last row of the group sees
+  const int hk = h / (H / Hkv);
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int g = lane / LPK, c = lane % LPK;
+  const unsigned kvs4 = (unsigned)(Hkv * DH / 4);
+  const float4 *__restrict__ kp = (const float4 *)(kc + (int64_t)hk * DH) + c;
+  const float4 *__restrict__ vp = (const float4 *)(vc + (int64_t)hk * DH) + c;
+  const float scale = 1.0f / sqrtf((float)DH);
+  float4 q4[R];
+  float m[R], l[R], acc[R][4];
+#pragma unroll
+  for (int r = 0; r < R; r++) {
+    const int row = min(i0 + r, S - 1);  // rows past the end repeat the last one and are not stored
+    q4[r] = *(const float4 *)(q + ((int64_t)row * H + h) * DH + 4 * c);
+    m[r] = -INFINITY;
+    l[r] = 0.0f;
+    acc[r][0] = acc[r][1] = acc[r][2] = acc[r][3] = 0.0f;
+  }
+  for (int t0 = 0; t0 < Tmax; t0 += TILE) {
+    if (t0 + wv * KPT * KPW >= Tmax) break;  // nothing left for this wavefront (uniform)
+    float4 kr[KPT], vr[KPT];
+#pragma unroll
+    for (int u = 0; u < KPT; u++) {
+      const int j = t0 + (wv * KPT + u) * KPW + g;
+      const unsigned jj = (unsigned)min(j, Tmax - 1);
+      kr[u] = kp[jj * kvs4];
+      vr[u] = vp[jj * kvs4];
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+      const int Tr = base + min(i0 + r, S - 1) + 1;  // keys row r sees
+      float sc[KPT];
+      float tmax = -INFINITY;
+#pragma unroll
+      for (int u = 0; u < KPT; u++) {
+        float d = q4[r].x * kr[u].x;
+        d = fmaf(q4[r].y, kr[u].y, d);
+        d = fmaf(q4[r].z, kr[u].z, d);
+        d = fmaf(q4[r].w, kr[u].w, d);
+        d = lpk_sum<LPK>(d);
+        const bool ok = (t0 + (wv * KPT + u) * KPW + g) < Tr;
+        sc[u] = ok ? d * scale : -INFINITY;
+        tmax = fmaxf(tmax, sc[u]);
+      }
+#pragma unroll
+      for (int o = LPK; o < 64; o <<= 1) tmax = fmaxf(tmax, __shfl_xor(tmax, o, 64));
+      const float m_new = fmaxf(m[r], tmax);
+      const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;  // every key of this tile masked for row r so far
+      const float corr = ct_exp(m[r] - m_use);
+      float ps = 0.0f;
+#pragma unroll
+      for (int k2 = 0; k2 < 4; k2++) acc[r][k2] *= corr;
+#pragma unroll
+      for (int u = 0; u < KPT; u++) {
+        const float p = ct_exp(sc[u] - m_use);
+        ps += p;
+        acc[r][0] = fmaf(p, vr[u].x, acc[r][0]);
+        acc[r][1] = fmaf(p, vr[u].y, acc[r][1]);
+        acc[r][2] = fmaf(p, vr[u].z, acc[r][2]);
+        acc[r][3] = fmaf(p, vr[u].w, acc[r][3]);
+      }
+#pragma unroll
+      for (int o = LPK; o < 64; o <<= 1) ps += __shfl_xor(ps, o, 64);
+      l[r] = l[r] * corr + ps;
+      m[r] = m_new;
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < R; r++) {
+#pragma unroll
+    for (int o = LPK; o < 64; o <<= 1) {
+#pragma unroll
+      for (int k2 = 0; k2 < 4; k2++) acc[r][k2] += __shfl_xor(acc[r][k2], o, 64);
+    }
+    if (lane < LPK) {
+#pragma unroll
+      for (int k2 = 0; k2 < 4; k2++) part[wv][r][4 * lane + k2] = acc[r][k2];
+    }
+    if (lane == 0) {
+      pm[wv][r] = m[r];
+      pl[wv][r] = l[r];
+    }
+  }
+  __syncthreads();
+  for (int e = tid; e < nrows * DH; e += 256) {
+    const int r = e / DH, d = e % DH;
+    float M = pm[0][r];
+#pragma unroll
+    for (int w = 1; w < NW; w++) M = fmaxf(M, pm[w][r]);  // finite: key 0 is visible to every row
+    float o = 0.0f, L = 0.0f;
+#pragma unroll
+    for (int w = 0; w < NW; w++) {
+      const float wgt = ct_exp(pm[w][r] - M);
+      o = fmaf(wgt, part[w][r][d], o);
+      L = fmaf(wgt, pl[w][r], L);
+    }
+    out[((int64_t)(i0 + r) * H + h) * DH + d] = o / L;
+  }
+}
+
 int launch_attn(float *out, const float *q, const float *kc, const float *vc, int S, int start_pos, const int *pos,
                 int max_T, int H, int Hkv, int Dh) {
   if (S == 0) return 0;
   (void)max_T;
   hipStream_t st = state().stream;
+  constexpr int R = 8;
+  if (S >= 2 * R) {  // prompt rows: groups of R rows share their K / V loads
+    dim3 grid(H, (S + R - 1) / R), block(256);
+    switch (Dh) {
+      case 32: hipLaunchKernelGGL((k_attn_rows<32, R>), grid, block, 0, st, out, q, kc, vc, S, start_pos, pos, H, Hkv); break;
+      case 64: hipLaunchKernelGGL((k_attn_rows<64, R>), grid, block, 0, st, out, q, kc, vc, S, start_pos, pos, H, Hkv); break;
+      case 128: hipLaunchKernelGGL((k_attn_rows<128, R>), grid, block, 0, st, out, q, kc, vc, S, start_pos, pos, H, Hkv); break;
+      default: return fail(CTHIP_E_UNSUPPORTED, "attention: head_dim %d (supported: 32, 64, 128)", Dh);
+    }
+    CTHIP_LAUNCH_CHECK();
+    return 0;
+  }
   dim3 grid(H, S), block(1024);
   switch (Dh) {
     case 32: hipLaunchKernelGGL(k_attn_cached<32>, grid, block, 0, st, out, q, kc, vc, start_pos, pos, H, Hkv); break;

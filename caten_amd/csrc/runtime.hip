@@ -171,7 +171,11 @@ int cthip_device_info(char *name, int name_cap, int *compute_units, int *wave_si
   return 0;
 }
 
-int cthip_alloc(void **out, size_t bytes) {
+}  // extern "C"
+
+// a block of the caching allocator with whatever its last owner left in it (temporaries that are
+// fully written before they are read); released with cthip_free like any other block
+int cthip::alloc_scratch(void **out, size_t bytes) {
   CTHIP_REQUIRE_INIT();
   CTHIP_ARG(out != nullptr);
   size_t cls = size_class(bytes);
@@ -202,10 +206,16 @@ int cthip_alloc(void **out, size_t bytes) {
     a.live[p] = cls;
     a.live_bytes += cls;
   }
-  int rc = zero_fill(p, cls);
-  if (rc) return rc;
   *out = p;
   return 0;
+}
+
+extern "C" {
+
+int cthip_alloc(void **out, size_t bytes) {
+  int rc = cthip::alloc_scratch(out, bytes);
+  if (rc) return rc;
+  return zero_fill(*out, size_class(bytes));
 }
 
 int cthip_free(void *p) {

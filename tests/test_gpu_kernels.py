@@ -254,7 +254,10 @@ def test_rope(ops, oracle):
 
 
 @pytest.mark.parametrize("S,start,H,Hkv,Dh", [(1, 0, 4, 4, 64), (1, 37, 12, 12, 64), (5, 3, 8, 2, 64),
-                                             (1, 700, 4, 1, 128), (3, 0, 2, 2, 32)])
+                                             (1, 700, 4, 1, 128), (3, 0, 2, 2, 32),
+                                             # prompt-sized row counts: groups of rows share their K / V tiles
+                                             (16, 0, 4, 4, 64), (37, 5, 8, 2, 64), (130, 0, 2, 2, 64), (21, 200, 2, 1, 128),
+                                             (19, 3, 2, 2, 32), (512, 0, 2, 2, 64)])
 def test_sdpa_cached(ops, oracle, S, start, H, Hkv, Dh):
     rng = np.random.default_rng(S + start)
     T = start + S
@@ -268,7 +271,8 @@ def test_sdpa_cached(ops, oracle, S, start, H, Hkv, Dh):
 
 
 # ------------------------------------------------------------------ matmul (MFMA)
-@pytest.mark.parametrize("M,N,K", [(256, 256, 256), (64, 64, 32), (3, 5, 7), (65, 33, 17), (100, 768, 1024), (1, 64, 64)])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 256), (64, 64, 32), (3, 5, 7), (65, 33, 17), (100, 768, 1024), (1, 64, 64),
+                                   (100, 70, 2000), (33, 65, 1030), (64, 64, 4096)])  # the last three split K
 def test_matmul_relu_vs_oracle(ops, oracle, M, N, K):
     print(f"case: matmul {M}x{N}x{K}", flush=True)
     rng = np.random.default_rng(M * 31 + N * 7 + K)

@@ -490,7 +490,8 @@ __global__ __launch_bounds__(256) void k_attn_rows(float *__restrict__ out, cons
   constexpr int LPK = DH / 4, KPW = 64 / LPK, KPT = 8, NW = 4, TILE = NW * KPW * KPT;
   __shared__ float part[NW][R][DH];
   __shared__ float pm[NW][R], pl[NW][R];
-  const int h = blockIdx.x, i0 = blockIdx.y * R;
+  // the last groups see the most keys: they are dispatched first so the short ones fill the tail
+  const int h = blockIdx.x, i0 = (gridDim.y - 1 - blockIdx.y) * R;
   const int base = start_pos + (pos ? pos[0] : 0);
   const int nrows = min(R, S - i0);
   const int Tmax = base + i0 + nrows;  // keys the last row of the group sees

@@ -33,6 +33,10 @@ struct GemmArgs {
   // its raw partial tile to ws[z][M][N]; k_splitk_reduce adds the partials in z order and applies the epilogue
   int ksplit, kper;
   float *ws;
+  // tile -> workgroup mapping of k_gemm_split: the tm x tn tile grid is cut into rx x ry = 8 regions of
+  // rm x rn tiles, one per XCD (workgroup i is dispatched to XCD i % 8), so that every L2 holds only
+  // its region's rows of A and columns of B
+  int tm, tn, rx, rm, rn;
 };
 
 __device__ __forceinline__ unsigned short f32_to_bf16_bits(float f) {
@@ -284,8 +288,11 @@ __global__ __launch_bounds__(256) void k_gemm_split(GemmArgs a) {
   __shared__ __align__(16) unsigned short Bs[2][NP][BN][LDK];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
-  const int tiles_m = (a.M + BM - 1) / BM;
-  const int m0 = (blockIdx.x % tiles_m) * BM, n0 = (blockIdx.x / tiles_m) * BN;
+  const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+  if (local >= a.rm * a.rn) return;
+  const int mi = (xcd % a.rx) * a.rm + local % a.rm, ni = (xcd / a.rx) * a.rn + local / a.rm;
+  if (mi >= a.tm || ni >= a.tn) return;  // the regions overhang a grid they do not divide
+  const int m0 = mi * BM, n0 = ni * BN;
   const int M = a.M, N = a.N, ldk = a.K;
   const int kbeg = blockIdx.y * a.kper;      // this workgroup's share of the reduction axis
   const int K = min(a.K, kbeg + a.kper);
@@ -570,6 +577,22 @@ int launch_gemm(GemmArgs a, int bmode, int precision) {
   a.kper = a.K > 0 ? a.K : 1;
   a.ws = nullptr;
   if (precision != GEMM_FP32) {
+    // one region of tiles per XCD: the split with the fewest tiles per XCD, then the least operand bytes per L2
+    a.tm = (a.M + 63) / 64;
+    a.tn = (a.N + 63) / 64;
+    const double sza = 4.0, szb = bmode == B_ROWMAJOR ? 4.0 : a.wtype == CTHIP_Q8_0 ? 1.0625 : a.wtype == CTHIP_Q4_0 ? 0.5625 : a.wtype == CTHIP_F16 ? 2.0 : 4.0;
+    double best = -1.0;
+    for (int rx = 1; rx <= 8; rx *= 2) {
+      const int ry = 8 / rx, rm = (a.tm + rx - 1) / rx, rn = (a.tn + ry - 1) / ry;
+      const double score = (double)rm * rn * 1e6 + rm * sza + rn * szb;
+      if (best < 0 || score < best) {
+        best = score;
+        a.rx = rx;
+        a.rm = rm;
+        a.rn = rn;
+      }
+    }
+    grid.x = 8u * (unsigned)a.rm * (unsigned)a.rn;
     // too few tiles to occupy the chip and a long reduction axis: split K over several workgroups per tile
     const int cus = state().compute_units, nsteps = (a.K + 63) / 64;
     int ks = (int)((cus * 3 / 2) / tiles);

@@ -115,6 +115,8 @@ int launch_prologue(float *out, const float *x, int cols, int pro, const float *
 // prefill: split fused qkv rows (S, D+2KD) into q (S,D) and cache rows start_pos.., rotating q and k when rope_base > 0
 int launch_qkv_split(float *q, float *kc, float *vc, const float *qkv, int S, int start_pos, int H, int Hkv, int Dh,
                      float rope_base);
+int launch_attn_rope_append(float *out, const float *q, float *kc, float *vc, const float *newkv, const int *pos, int H,
+                            int Hkv, int Dh, float base);
 int launch_rope_append(float *kc, float *vc, const float *kv, int Hkv, int Dh, float base, const int *pos);
 int launch_rope(float *out, const float *x, int B, int S, int H, int Dh, float base, int start_pos, const int *pos);
 

@@ -346,11 +346,12 @@ static int queue_step(Decoder *d, bool with_head) {
     }
     TRY(launch_gemv(L.attn, a, 1));
     if (!gpt2) {
-      // rotate q in place and k into the cache at `pos`; v is copied beside it
-      TRY(launch_rope(d->q, d->q, 1, 1, c.n_heads, Dh, c.rope_base, 0, pos));
-      TRY(launch_rope_append(L.k_cache, L.v_cache, d->kv_tmp, c.n_kv_heads, Dh, c.rope_base, pos));
+      // q and the new key are rotated inside the attention launch, which also appends k / v at `pos`
+      TRY(launch_attn_rope_append(d->att, d->q, L.k_cache, L.v_cache, d->kv_tmp, pos, c.n_heads, c.n_kv_heads, Dh,
+                                  c.rope_base));
+    } else {
+      TRY(launch_attn(d->att, d->q, L.k_cache, L.v_cache, 1, 0, pos, c.max_seq, c.n_heads, c.n_kv_heads, Dh));
     }
-    TRY(launch_attn(d->att, d->q, L.k_cache, L.v_cache, 1, 0, pos, c.max_seq, c.n_heads, c.n_kv_heads, Dh));
     GemvArgs p = {};
     p.x = d->att;
     p.bias = L.proj_b;

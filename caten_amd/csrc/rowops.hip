@@ -369,10 +369,36 @@ __global__ __launch_bounds__(256) void k_qkv_split(float *__restrict__ q, float 
 // covers 64/(DH/4) keys per pass and holds KPT passes of K and V in registers, all requested before
 // any arithmetic.  Every wavefront runs its own online softmax over its keys (shuffles only); the 16
 // per-wavefront partials (max, sum, DH outputs) meet once in LDS, so a block needs one barrier.
-template <int DH>
+//
+// APPEND (decode of RoPE models, one row): the step's new key / value row is still in `newkv` (k then v,
+// Hkv*DH floats each, unrotated).  Every block rotates its query and its kv head's new key in registers
+// (positional-encoding.lisp:3-64 at position pos), uses them for key T-1, and the first query head of each
+// kv group stores the rotated key and the value into cache row T-1 -- the rotation and the `!assign` into
+// the cache (layers.lisp:13-33) need no launches of their own.
+__device__ __forceinline__ float4 rope4(float4 x, int c, int DH, float log2_base, int at) {
+  // lane c holds elements 4c..4c+3 = pairs 2c and 2c+1 of the head; same arithmetic as k_rope
+  float o[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+  for (int t = 0; t < 2; t++) {
+    const int i = 2 * c + t;
+    const float expo = (float)(2 * i) / (float)DH;
+    const float logb = log2_base * 0.6931472f;
+    const float theta = exp2f(-(expo * logb) * 1.442695f);
+    const float ang = (float)at * theta;
+    float sn, cs;
+    sincosf(ang, &sn, &cs);
+    const float x0 = o[2 * t], x1 = o[2 * t + 1];
+    o[2 * t] = x0 * cs - x1 * sn;
+    o[2 * t + 1] = x0 * sn + x1 * cs;
+  }
+  return make_float4(o[0], o[1], o[2], o[3]);
+}
+
+template <int DH, bool APPEND>
 __global__ __launch_bounds__(1024) void k_attn_cached(float *__restrict__ out, const float *__restrict__ q,
-                                                      const float *__restrict__ kc, const float *__restrict__ vc,
-                                                      int start_pos, const int *__restrict__ pos, int H, int Hkv) {
+                                                      float *__restrict__ kc, float *__restrict__ vc,
+                                                      int start_pos, const int *__restrict__ pos, int H, int Hkv,
+                                                      const float *__restrict__ newkv, float log2_base) {
   constexpr int LPK = DH / 4;      // lanes per key
   constexpr int KPW = 64 / LPK;    // keys per wavefront per pass
   constexpr int KPT = 8;           // passes held in registers
@@ -386,10 +412,21 @@ __global__ __launch_bounds__(1024) void k_attn_cached(float *__restrict__ out, c
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int g = lane / LPK, c = lane % LPK;
   const unsigned kvs4 = (unsigned)(Hkv * DH / 4);
-  const float4 q4 = *(const float4 *)(q + ((int64_t)i * H + h) * DH + 4 * c);
+  float4 q4 = *(const float4 *)(q + ((int64_t)i * H + h) * DH + 4 * c);
   const float4 *__restrict__ kp = (const float4 *)(kc + (int64_t)hk * DH) + c;
   const float4 *__restrict__ vp = (const float4 *)(vc + (int64_t)hk * DH) + c;
   const float scale = 1.0f / sqrtf((float)DH);
+  float4 kn = make_float4(0.f, 0.f, 0.f, 0.f), vn = kn;
+  if (APPEND) {
+    const int KD = Hkv * DH;
+    q4 = rope4(q4, c, DH, log2_base, T - 1);
+    kn = rope4(*(const float4 *)(newkv + hk * DH + 4 * c), c, DH, log2_base, T - 1);
+    vn = *(const float4 *)(newkv + KD + hk * DH + 4 * c);
+    if (h % (H / Hkv) == 0 && tid < LPK) {
+      ((float4 *)(kc + (int64_t)(T - 1) * KD + hk * DH))[c] = kn;
+      ((float4 *)(vc + (int64_t)(T - 1) * KD + hk * DH))[c] = vn;
+    }
+  }
   float m = -INFINITY, l = 0.0f;
   float acc[4] = {0.f, 0.f, 0.f, 0.f};
   // wavefront wv owns keys t0 + (wv*KPT + u)*KPW + g
@@ -399,9 +436,14 @@ __global__ __launch_bounds__(1024) void k_attn_cached(float *__restrict__ out, c
 #pragma unroll
     for (int u = 0; u < KPT; u++) {
       const int j = t0 + (wv * KPT + u) * KPW + g;
-      const unsigned jj = (unsigned)min(j, T - 1);  // clamp: masked below, never out of the cache
+      // clamp: masked below, never out of the cache; APPEND: row T-1 comes from the registers
+      const unsigned jj = (unsigned)min(j, APPEND ? max(T - 2, 0) : T - 1);
       kr[u] = kp[jj * kvs4];
       vr[u] = vp[jj * kvs4];
+      if (APPEND && j >= T - 1) {
+        kr[u] = kn;
+        vr[u] = vn;
+      }
     }
     float sc[KPT];
     float tmax = -INFINITY;
@@ -612,10 +654,28 @@ int launch_attn(float *out, const float *q, const float *kc, const float *vc, in
     return 0;
   }
   dim3 grid(H, S), block(1024);
+  float *kcw = const_cast<float *>(kc), *vcw = const_cast<float *>(vc);
+  const float *nokv = nullptr;
   switch (Dh) {
-    case 32: hipLaunchKernelGGL(k_attn_cached<32>, grid, block, 0, st, out, q, kc, vc, start_pos, pos, H, Hkv); break;
-    case 64: hipLaunchKernelGGL(k_attn_cached<64>, grid, block, 0, st, out, q, kc, vc, start_pos, pos, H, Hkv); break;
-    case 128: hipLaunchKernelGGL(k_attn_cached<128>, grid, block, 0, st, out, q, kc, vc, start_pos, pos, H, Hkv); break;
+    case 32: hipLaunchKernelGGL((k_attn_cached<32, false>), grid, block, 0, st, out, q, kcw, vcw, start_pos, pos, H, Hkv, nokv, 0.0f); break;
+    case 64: hipLaunchKernelGGL((k_attn_cached<64, false>), grid, block, 0, st, out, q, kcw, vcw, start_pos, pos, H, Hkv, nokv, 0.0f); break;
+    case 128: hipLaunchKernelGGL((k_attn_cached<128, false>), grid, block, 0, st, out, q, kcw, vcw, start_pos, pos, H, Hkv, nokv, 0.0f); break;
+    default: return fail(CTHIP_E_UNSUPPORTED, "attention: head_dim %d (supported: 32, 64, 128)", Dh);
+  }
+  CTHIP_LAUNCH_CHECK();
+  return 0;
+}
+
+// one decode row of a RoPE model: rotates q and the new key, appends k / v at `pos`, attends (see k_attn_cached)
+int launch_attn_rope_append(float *out, const float *q, float *kc, float *vc, const float *newkv, const int *pos, int H,
+                            int Hkv, int Dh, float base) {
+  hipStream_t st = state().stream;
+  dim3 grid(H, 1), block(1024);
+  const float lb = log2f(base);
+  switch (Dh) {
+    case 32: hipLaunchKernelGGL((k_attn_cached<32, true>), grid, block, 0, st, out, q, kc, vc, 0, pos, H, Hkv, newkv, lb); break;
+    case 64: hipLaunchKernelGGL((k_attn_cached<64, true>), grid, block, 0, st, out, q, kc, vc, 0, pos, H, Hkv, newkv, lb); break;
+    case 128: hipLaunchKernelGGL((k_attn_cached<128, true>), grid, block, 0, st, out, q, kc, vc, 0, pos, H, Hkv, newkv, lb); break;
     default: return fail(CTHIP_E_UNSUPPORTED, "attention: head_dim %d (supported: 32, 64, 128)", Dh);
   }
   CTHIP_LAUNCH_CHECK();

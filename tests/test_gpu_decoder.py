@@ -137,9 +137,19 @@ def test_llama_generate_matches_oracle(oracle, kind):
     assert got_tokens == want_tokens
     for g, r in zip(got_logits, want_logits):
         close(g, r)
+    # rotated keys and values appended by the decode step's attention launch equal the oracle's cache rows
+    kd = cfg["dim"] // cfg["n_heads"] * cfg["n_kv_heads"]
+    T = len(prompt) + steps - 1
+    for l in (0, cfg["n_layers"] - 1):
+        close(model.peek(f"k_cache.{l}")[:T * kd], ref.k_cache[l].ravel()[:T * kd])
+        close(model.peek(f"v_cache.{l}")[:T * kd], ref.v_cache[l].ravel()[:T * kd])
     model.close()
     model = llm.make_llama(cfg, llm.llama_state_dict(w, kind))
     assert llm.gpt2_generate(model, prompt, steps, on_device=True) == want_tokens
+    # a prompt shorter than the batch threshold goes row by row through the decode step, from position 0
+    short = synth.prompt(cfg["vocab"], 3, seed=2)
+    ref2 = oracle.Llama(cfg, _dequantised(oracle, w, synth.LLAMA_LINEAR_KEYS + ("lm_head",), kind))
+    assert llm.gpt2_generate(model, short, 6, on_device=True) == ref2.generate(short, 6)
     model.close()
 
 

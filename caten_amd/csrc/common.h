@@ -24,6 +24,7 @@ struct State {
 State &state();
 // cthip_alloc without the zero fill, for temporaries that are fully written before they are read
 int alloc_scratch(void **out, size_t bytes);
+bool device_readable(const void *p);
 void set_error(const char *fmt, ...);
 int fail(int code, const char *fmt, ...);
 

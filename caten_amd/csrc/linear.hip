@@ -790,6 +790,8 @@ int cthip_dequant(int ggml_type, const void *raw, int64_t n, float *out) {
   CTHIP_REQUIRE_INIT();
   if (n == 0) return 0;
   CTHIP_ARG(raw != nullptr && out != nullptr && n > 0);
+  if (!device_readable(raw) || !device_readable(out))
+    return fail(CTHIP_E_BAD_ARG, "cthip_dequant: raw and out must be device pointers (upload the bytes with cthip_h2d first)");
   dim3 grid((unsigned)((n + 255) / 256)), block(256);
   hipStream_t st = state().stream;
   switch (ggml_type) {
@@ -816,6 +818,8 @@ int cthip_wmat_create(void **wmat, int ggml_type, const void *raw, int64_t rows,
   if ((ggml_type == CTHIP_Q8_0 || ggml_type == CTHIP_Q4_0) && cols % 32)
     return fail(CTHIP_E_BAD_ARG, "cthip_wmat_create: quantised rows need cols %% 32 == 0, got %lld", (long long)cols);
   if (rows > 0x7fffffff || cols > 0x7fffffff) return fail(CTHIP_E_BAD_ARG, "cthip_wmat_create: dimension too large");
+  if (!device_readable(raw))
+    return fail(CTHIP_E_BAD_ARG, "cthip_wmat_create: raw must be a device pointer (upload the bytes with cthip_h2d first)");
   WMat *w = nullptr;
   int rc = wmat_create_impl(&w, ggml_type, raw, rows, cols);
   if (rc) return rc;

@@ -173,6 +173,17 @@ int cthip_device_info(char *name, int name_cap, int *compute_units, int *wave_si
 
 }  // extern "C"
 
+// true when a kernel may dereference p: device, managed or pinned host memory.  Pageable host memory handed
+// to a kernel would fault the GPU, so entry points that take device pointers from callers check first.
+bool cthip::device_readable(const void *p) {
+  hipPointerAttribute_t attr;
+  if (hipPointerGetAttributes(&attr, p) != hipSuccess) {
+    (void)hipGetLastError();  // the failed query must not be reported by the next launch check
+    return false;
+  }
+  return attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeManaged || attr.type == hipMemoryTypeHost;
+}
+
 // a block of the caching allocator with whatever its last owner left in it (temporaries that are
 // fully written before they are read); released with cthip_free like any other block
 int cthip::alloc_scratch(void **out, size_t bytes) {

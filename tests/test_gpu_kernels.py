@@ -72,6 +72,20 @@ def test_dequant_q4_0_rejects_ragged(ops):
         ops.dequantize("q4_0", np.zeros(36, np.uint8), 40)
 
 
+def test_host_pointers_are_refused_not_dereferenced(ops):
+    """The codecs take device pointers; pageable host memory is rejected on the host side, before any launch."""
+    import ctypes as C
+    from caten_amd import _lib, HipError
+    lib = _lib.load()
+    raw = np.zeros(34 * 8, np.uint8)
+    out = ops.DeviceArray((256,), np.float32)
+    with pytest.raises(HipError, match="device pointer"):
+        _lib.check(lib.cthip_dequant(_lib.Q8_0, raw.ctypes.data, 256, out.ptr))
+    h = C.c_void_p()
+    with pytest.raises(HipError, match="device pointer"):
+        _lib.check(lib.cthip_wmat_create(C.byref(h), _lib.Q8_0, raw.ctypes.data, 8, 32))
+
+
 def test_dequant_f16_f32(ops, oracle):
     bits = np.arange(65536, dtype=np.uint16)
     got = ops.dequantize("f16", bits.view(np.uint8), 65536)

@@ -351,6 +351,38 @@ __device__ __forceinline__ void coop_prologue(const GemvArgs &a, const float *__
   __syncthreads();
 }
 
+// Folded norm with a staged input: the workgroup writes gamma * x into LDS once and reduces the
+// shifted sums  s1 = sum(x - pivot), s2 = sum((x - pivot)^2)  over the whole vector, so no wavefront
+// loads gamma or repeats the statistics.  xs must hold a.cols floats; blockDim.x <= 256.
+__device__ __forceinline__ void coop_fold(const GemvArgs &a, const float *__restrict__ x, float *xs, float *red,
+                                          float pivot, float &s1_out, float &s2_out) {
+  const int tid = threadIdx.x, nthr = blockDim.x, nw = nthr >> 6;
+  const int n4 = a.cols >> 2;
+  float s1 = 0.0f, s2 = 0.0f;
+  for (int i = tid; i < n4; i += nthr) {
+    const float4 v = ((const float4 *)x)[i];
+    const float4 g = a.norm_g ? ((const float4 *)a.norm_g)[i] : make_float4(1.f, 1.f, 1.f, 1.f);
+    const float d0 = v.x - pivot, d1 = v.y - pivot, d2 = v.z - pivot, d3 = v.w - pivot;
+    s1 += (d0 + d1) + (d2 + d3);
+    s2 = fmaf(d0, d0, s2);
+    s2 = fmaf(d1, d1, s2);
+    s2 = fmaf(d2, d2, s2);
+    s2 = fmaf(d3, d3, s2);
+    ((float4 *)xs)[i] = make_float4(v.x * g.x, v.y * g.y, v.z * g.z, v.w * g.w);
+  }
+  auto block_sum = [&](float v) {
+    v = wave_sum(v);
+    __syncthreads();
+    if ((tid & 63) == 0) red[tid >> 6] = v;
+    __syncthreads();
+    float t = 0.0f;
+    for (int w = 0; w < nw; w++) t += red[w];
+    return t;
+  };
+  s1_out = block_sum(s1);
+  s2_out = block_sum(s2);  // its barriers also publish xs
+}
+
 // PD = weight tiles a wavefront keeps in flight: 1 for the small, latency-bound launches (one tile
 // per wavefront), 4 for the large ones, whose throughput is bytes-in-flight / memory latency.
 template <int TYPE, int G, int KC, int PD>
@@ -414,7 +446,12 @@ __global__ __launch_bounds__(256) void k_gemv(GemvArgs a) {
 
   float xr[KC][XPC];
   float xs[KC];
-  if (coop) coop_prologue(a, x, xs_lds, red, a.pro != CTHIP_PRO_NONE && !folded);
+  float bs1 = 0.0f, bs2 = 0.0f;  // block-wide statistics when the folded norm is staged
+  const float pivot = (folded && a.pro == CTHIP_PRO_LAYERNORM) ? x[0] : 0.0f;
+  if (coop) {
+    if (folded) coop_fold(a, x, xs_lds, red, pivot, bs1, bs2);
+    else coop_prologue(a, x, xs_lds, red, a.pro != CTHIP_PRO_NONE);
+  }
   const float *__restrict__ xsrc = coop ? xs_lds : x;
 #pragma unroll
   for (int j = 0; j < KC; j++) {
@@ -432,9 +469,10 @@ __global__ __launch_bounds__(256) void k_gemv(GemvArgs a) {
   float mu = 0.0f, rstd = 1.0f;
   if (folded) {
     // every group of G lanes holds the whole vector: shifted one-pass mean / variance (the shift by
-    // x[0] keeps E[d^2] - E[d]^2 well conditioned), then scale the slice by gamma
-    const float pivot = (a.pro == CTHIP_PRO_LAYERNORM) ? x[0] : 0.0f;
+    // x[0] keeps E[d^2] - E[d]^2 well conditioned), then scale the slice by gamma -- unless the
+    // workgroup has already done both while staging
     float s1 = 0.0f, s2 = 0.0f;
+    if (!coop) {
 #pragma unroll
     for (int j = 0; j < KC; j++) {
       const int c = l + G * j;
@@ -453,9 +491,10 @@ __global__ __launch_bounds__(256) void k_gemv(GemvArgs a) {
         }
       }
     }
+    }
     const float inv_n = 1.0f / (float)a.cols;
-    const float m1 = group_sum<G>(s1) * inv_n;
-    const float m2 = group_sum<G>(s2) * inv_n;
+    const float m1 = (coop ? bs1 : group_sum<G>(s1)) * inv_n;
+    const float m2 = (coop ? bs2 : group_sum<G>(s2)) * inv_n;
     if (a.pro == CTHIP_PRO_LAYERNORM) {
       mu = pivot + m1;
       rstd = 1.0f / sqrtf(fmaxf(m2 - m1 * m1, 0.0f) + a.eps);
@@ -661,7 +700,8 @@ int launch_gemv(const WMat *w, GemvArgs a, int m) {
     // The input vector goes through LDS once per workgroup when it must be normalised or gated first,
     // or when it is large next to a weight tile (a 4-bit tile multiplies 8 input bytes per weight byte):
     // then four wavefronts share one copy and every wavefront takes several tiles.
-    const bool stage = (a.pro != CTHIP_PRO_NONE && !folded) || (w->type == CTHIP_Q4_0 && a.cols >= 1024);
+    const bool stage = (a.pro != CTHIP_PRO_NONE && !folded) || (w->type == CTHIP_Q4_0 && a.cols >= 1024) ||
+                       (folded && a.cols >= 2048);
     const size_t lds = stage ? sizeof(float) * (size_t)a.cols : 0;
     if (lds > 64 * 1024) return fail(CTHIP_E_UNSUPPORTED, "gemv: %d input features exceed the LDS staging buffer", a.cols);
     a.stage_x = stage ? 1 : 0;
@@ -693,6 +733,9 @@ int launch_gemv(const WMat *w, GemvArgs a, int m) {
       int wanted = (nrq + 3) / 4;
       if (wanted < base) wanted = base;
       if (wanted > base * occ_cache[vi]) wanted = base * occ_cache[vi];
+      // staged launches pay the input staging once per workgroup: whole workgroups per compute unit, two
+      // when there is work for more than one (measured best; a third does not fit beside the first two)
+      if (stage && wanted > base && occ_cache[vi] >= 2) wanted = 2 * base;
       static const char *ovr = getenv("CTHIP_GEMV_WAVES");  // tuning aid: overrides the wavefront count
       if (ovr && atoi(ovr) > 0) wanted = atoi(ovr);
       const int iters = (nrq + wanted - 1) / wanted;

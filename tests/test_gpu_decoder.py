@@ -82,6 +82,25 @@ def test_gpt2_long_context_attention(oracle):
     model.close()
 
 
+@pytest.mark.parametrize("kind", ["q4_0", "q8_0"])
+def test_gpt2_wide_model_folded_layernorm(oracle, kind):
+    """d_model 1024 (GPT-2 medium's width): the 4-bit decode GEMVs stage the input per workgroup, with the
+    folded LayerNorm's statistics computed there."""
+    print(f"case: gpt2 d1024 {kind}", flush=True)
+    from caten_amd import synth, llm
+    cfg = dict(n_layers=2, n_heads=16, dim=1024, ffn=2048, vocab=700, max_seq=48, eps=1e-5)
+    w = synth.gpt2_weights(cfg, seed=8)
+    prompt = synth.prompt(cfg["vocab"], 5, seed=8)
+    ref = oracle.GPT2(cfg, _dequantised(oracle, w, synth.GPT2_LINEAR_KEYS + ("lm_head",), kind))
+    want_tokens, want_logits = ref.generate(prompt, 8, keep_logits=True)
+    model = llm.make_gpt2(cfg, llm.gpt2_state_dict(w, kind))
+    got_tokens, got_logits = llm.gpt2_generate(model, prompt, 8, on_device=False, keep_logits=True)
+    assert got_tokens == want_tokens
+    for g, r in zip(got_logits, want_logits):
+        close(g, r)
+    model.close()
+
+
 def test_gpt2_prompt_lengths_and_restart(oracle):
     from caten_amd import synth, llm
     cfg = synth.GPT2_CONFIGS["gpt2-tiny"]

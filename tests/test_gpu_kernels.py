@@ -166,6 +166,26 @@ def test_gemv_fused_neighbours(ops, oracle, kind):
     close(ops.linear(xx, wm, prologue="swiglu"), want)
 
 
+@pytest.mark.parametrize("kind", ["q4_0", "q8_0"])
+def test_gemv_wide_input_with_norms(ops, oracle, kind):
+    """2048 input features: 4-bit launches stage the input (and the folded RMSNorm's gamma * x and statistics)
+    in LDS once per workgroup."""
+    from caten_amd.llm import Tensor
+    rng = np.random.default_rng(24)
+    cols = 2048
+    for rows in (200, 2560):
+        w = rng.normal(0, 0.02, (rows, cols)).astype(np.float32)
+        x = rng.normal(0.2, 1.5, cols).astype(np.float32)
+        g = rng.normal(1, 0.05, cols).astype(np.float32)
+        be = rng.normal(0, 0.05, cols).astype(np.float32)
+        t = Tensor.from_f32(w, kind)
+        wd = oracle.dequant(kind, t.raw, w.size).reshape(rows, cols)
+        wm = ops.WeightMatrix(kind, t.raw, rows, cols)
+        close(ops.linear(x, wm, prologue="rmsnorm", norm_g=g), oracle.linear(oracle.rmsnorm(x, g), wd))
+        close(ops.linear(x, wm, prologue="layernorm", norm_g=g, norm_b=be), oracle.linear(oracle.layernorm(x, g, be), wd))
+        close(ops.linear(x, wm), oracle.linear(x, wd))
+
+
 def test_gemv_fallback_shapes_with_prologue(ops, oracle):
     from caten_amd.llm import Tensor
     rng = np.random.default_rng(22)

@@ -78,6 +78,9 @@ struct GemvArgs {
   // LayerNorm folded through the product (see k_gemv): fold_s[r] = sum_k W[r,k]*gamma[k]; the caller
   // passes sum_k W[r,k]*beta[k] + b[r] as `bias`.  Null = normalise the input first.
   const float *fold_s;
+  // rows 2r / 2r+1 are a (gate, up) pair: the launch writes silu(gate_r) * up_r to y[r] (rows/2 outputs)
+  // instead of the two products.  Needs a variant with at least two rows per wavefront.
+  int pair_swiglu;
   int stage_x;  // set by the launcher: the workgroup stages the input vector in LDS once
   float eps;
   int rows, cols;
@@ -99,6 +102,10 @@ int launch_gemv(const WMat *w, GemvArgs a, int m);
 int wmat_create_impl(WMat **out, int type, const void *raw, int64_t rows, int64_t cols);
 // true when a register-resident GEMV variant covers the matrix (no temporary is allocated at launch)
 bool gemv_is_direct(const WMat *w);
+// rows a wavefront of the register-resident variant for (type, cols) produces per pass; 0 = no such variant
+int gemv_rows_per_wave(int type, int64_t cols);
+// out[i] = silu(in[2i]) * in[2i+1], i < n (gate / up columns interleaved)
+int launch_swiglu_pairs(float *out, const float *in, int64_t n);
 int launch_attn(float *out, const float *q, const float *kc, const float *vc, int S, int start_pos, const int *pos,
                 int max_T, int H, int Hkv, int Dh);
 int launch_embedding(float *out, const float *W, const float *idx_f, const int *idx_i, int ntok, int vocab, int dim,

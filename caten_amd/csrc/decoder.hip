@@ -57,6 +57,7 @@ struct Layer {
   // LayerNorm folded through c_attn / c_fc: S = W.gamma, C = W.beta + bias
   float *attn_s = nullptr, *attn_c = nullptr, *fc_s = nullptr, *fc_c = nullptr;
   // Llama: attn = wq|wk|wv, proj = wo, fc = gate|up, fc2 = down, ln1_g/ln2_g = rms weights
+  bool fc_pairs = false;  // gate / up rows interleaved, SwiGLU in the gate|up launch
   float *k_cache = nullptr, *v_cache = nullptr;
 };
 
@@ -140,7 +141,9 @@ static int to_f32(Decoder *d, const std::string &key, int64_t want_n, float **ou
 }
 
 // pack one or more raw tensors (row-concatenated) into a weight matrix
-static int to_wmat(Decoder *d, const std::vector<std::string> &keys, int64_t want_rows, int64_t want_cols, WMat **out) {
+// interleave: two parts of equal height are merged row by row (a0, b0, a1, b1, ...) instead of stacked
+static int to_wmat(Decoder *d, const std::vector<std::string> &keys, int64_t want_rows, int64_t want_cols, WMat **out,
+                   bool interleave = false) {
   std::vector<RawTensor *> parts;
   int64_t rows = 0;
   for (const std::string &k : keys) {
@@ -164,10 +167,19 @@ static int to_wmat(Decoder *d, const std::vector<std::string> &keys, int64_t wan
     for (RawTensor *p : parts) total += p->nbytes;
     void *cat = nullptr;
     if ((rc = cthip_alloc(&cat, total))) return rc;
-    size_t off = 0;
-    for (RawTensor *p : parts) {
-      if ((rc = cthip_d2d((char *)cat + off, p->dev, p->nbytes))) return rc;
-      off += p->nbytes;
+    if (interleave) {
+      if (parts.size() != 2 || parts[0]->rows != parts[1]->rows || parts[0]->nbytes != parts[1]->nbytes)
+        return fail(CTHIP_E_BAD_ARG, "decoder: '%s' cannot be interleaved with its partner", keys[0].c_str());
+      const size_t rowbytes = parts[0]->nbytes / (size_t)parts[0]->rows;  // GGUF rows are contiguous runs of blocks
+      for (int k = 0; k < 2; k++)
+        CTHIP_CHECK(hipMemcpy2DAsync((char *)cat + k * rowbytes, 2 * rowbytes, parts[k]->dev, rowbytes, rowbytes,
+                                     (size_t)parts[k]->rows, hipMemcpyDeviceToDevice, state().stream));
+    } else {
+      size_t off = 0;
+      for (RawTensor *p : parts) {
+        if ((rc = cthip_d2d((char *)cat + off, p->dev, p->nbytes))) return rc;
+        off += p->nbytes;
+      }
     }
     rc = wmat_create_impl(out, parts[0]->type, cat, rows, want_cols);
     cthip_free(cat);
@@ -252,7 +264,10 @@ static int finalize(Decoder *d) {
                   D + 2 * KD, D, &L.attn));
       TRY(to_wmat(d, {key(l, "attention.wo.weight")}, D, D, &L.proj));
       TRY(to_f32(d, key(l, "ffn_norm.weight"), D, &L.ln2_g));
-      TRY(to_wmat(d, {key(l, "feed_forward.w1.weight"), key(l, "feed_forward.w3.weight")}, 2 * F, D, &L.fc));
+      // gate and up rows interleaved when the GEMV variant keeps a row pair in one wavefront: SwiGLU then
+      // happens in that launch's epilogue and the down projection reads ffn floats instead of 2 * ffn
+      L.fc_pairs = gemv_rows_per_wave(d->raw.at(key(l, "feed_forward.w1.weight")).type, D) >= 2;
+      TRY(to_wmat(d, {key(l, "feed_forward.w1.weight"), key(l, "feed_forward.w3.weight")}, 2 * F, D, &L.fc, L.fc_pairs));
       TRY(to_wmat(d, {key(l, "feed_forward.w2.weight")}, D, F, &L.fc2));
     }
   }
@@ -369,17 +384,18 @@ static int queue_step(Decoder *d, bool with_head) {
     f.bias = gpt2 ? L.fc_c : L.fc_b;
     f.fold_s = L.fc_s;
     f.act = gpt2 ? CTHIP_ACT_GELU : CTHIP_ACT_NONE;
+    f.pair_swiglu = L.fc_pairs ? 1 : 0;
     f.y = d->h;
     f.x_stride = D;
-    f.y_stride = gpt2 ? F : 2 * F;
+    f.y_stride = (gpt2 || L.fc_pairs) ? F : 2 * F;
     TRY(launch_gemv(L.fc, f, 1));
     GemvArgs g = {};
     g.x = d->h;
-    g.pro = gpt2 ? CTHIP_PRO_NONE : CTHIP_PRO_SWIGLU;
+    g.pro = (gpt2 || L.fc_pairs) ? CTHIP_PRO_NONE : CTHIP_PRO_SWIGLU;
     g.bias = L.fc2_b;
     g.residual = d->x;
     g.y = d->x;
-    g.x_stride = gpt2 ? F : 2 * F;
+    g.x_stride = (gpt2 || L.fc_pairs) ? F : 2 * F;
     g.y_stride = D;
     TRY(launch_gemv(L.fc2, g, 1));
   }
@@ -464,7 +480,8 @@ static int prefill(Decoder *d, const int *ids, int s, int n) {
     TRY(launch_linear_gemm(Hb, L.fc, XN, s, L.fc_b, nullptr, gpt2 ? CTHIP_ACT_GELU : CTHIP_ACT_NONE, prec));
     const float *hin = Hb;
     if (!gpt2) {
-      TRY(launch_prologue(G, Hb, F, CTHIP_PRO_SWIGLU, nullptr, nullptr, 0.0f, 2 * (int64_t)F, s));
+      if (L.fc_pairs) TRY(launch_swiglu_pairs(G, Hb, (int64_t)s * F));
+      else TRY(launch_prologue(G, Hb, F, CTHIP_PRO_SWIGLU, nullptr, nullptr, 0.0f, 2 * (int64_t)F, s));
       hin = G;
     }
     TRY(launch_linear_gemm(X, L.fc2, hin, s, L.fc2_b, X, CTHIP_ACT_NONE, prec));

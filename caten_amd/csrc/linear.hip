@@ -529,7 +529,12 @@ __global__ __launch_bounds__(256) void k_gemv(GemvArgs a) {
         acc = group_sum<G>(acc);
         if (folded) acc = rstd * (acc - mu * fs_t[p]);
         const int row = rq * RPW + g;
-        if (l == 0 && row < a.rows) {
+        if (RPW >= 2 && a.pair_swiglu) {
+          // SwiGLU across the (gate, up) row pair held by neighbouring lane groups
+          const float mine = acc + bias_t[p];
+          const float other = __shfl_xor(mine, G & 63, 64);
+          if (l == 0 && (g & 1) == 0 && row < a.rows) a.y[(int64_t)m * a.y_stride + (row >> 1)] = ct_silu(mine) * other;
+        } else if (l == 0 && row < a.rows) {
           const float v = gemv_store(a, m, row, acc, posv, bias_t[p], resid_t[p]);
           argmax_merge(best_v, best_i, v, row);
         }
@@ -681,6 +686,25 @@ int launch_prologue(float *out, const float *x, int cols, int pro, const float *
 }
 
 bool gemv_is_direct(const WMat *w) { return pick_variant(w->type, (int)w->cols) != nullptr; }
+int gemv_rows_per_wave(int type, int64_t cols) {
+  const GemvVariant *v = cols <= 0x7fffffff ? pick_variant(type, (int)cols) : nullptr;
+  return v ? 64 / v->G : 0;
+}
+
+__global__ __launch_bounds__(256) void k_swiglu_pairs(float *__restrict__ out, const float *__restrict__ in, int64_t n) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+    const float2 v = ((const float2 *)in)[i];
+    out[i] = ct_silu(v.x) * v.y;
+  }
+}
+int launch_swiglu_pairs(float *out, const float *in, int64_t n) {
+  if (n <= 0) return 0;
+  int64_t blocks = (n + 255) / 256;
+  if (blocks > 8192) blocks = 8192;
+  hipLaunchKernelGGL(k_swiglu_pairs, dim3((unsigned)blocks), dim3(256), 0, state().stream, out, in, n);
+  CTHIP_LAUNCH_CHECK();
+  return 0;
+}
 
 // Queues one fused Linear on the stream. Used by cthip_linear and by the decoder.
 int launch_gemv(const WMat *w, GemvArgs a, int m) {
@@ -692,6 +716,8 @@ int launch_gemv(const WMat *w, GemvArgs a, int m) {
   if (a.split1 <= 0) a.split1 = a.split2 = a.rows;
   if (a.am_val && m != 1) return fail(CTHIP_E_BAD_ARG, "gemv: the fused argmax needs m == 1");
   const GemvVariant *v = pick_variant(w->type, a.cols);
+  if (a.pair_swiglu && (!v || v->G > 32 || (a.rows & 1) || a.am_val || a.residual || a.split1 != a.rows))
+    return fail(CTHIP_E_UNSUPPORTED, "gemv: the paired SwiGLU epilogue needs two rows per wavefront and plain outputs");
   if (v) {
     const int rpw = 64 / v->G;
     const int nrq = (a.rows + rpw - 1) / rpw;

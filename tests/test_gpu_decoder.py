@@ -248,3 +248,26 @@ def test_gpt2_small_q8_0_full_size_matches_oracle(oracle):
     assert llm.gpt2_generate(model2, prompt, 40, on_device=False) == long_run
     model.close()
     model2.close()
+
+
+def test_llama_1b_width_q4_0_matches_oracle(oracle):
+    """BASELINE config 5's layer shape at its real width (d 2048, 32 query / 4 KV heads, SwiGLU 5632, vocab 32000,
+    Q4_0) with 2 of the 22 layers so the CPU oracle finishes in seconds: a 12-token prompt (batched prefill)
+    and greedy decode -- identical tokens, logits inside rtol 1e-3 / atol 1e-4, cache rows equal."""
+    print("case: llama 1.1b width q4_0, 2 layers", flush=True)
+    from caten_amd import synth, llm
+    cfg = dict(synth.LLAMA_CONFIGS["llama-1.1b"], n_layers=2, max_seq=64)
+    w = synth.llama_weights(cfg, seed=2)
+    prompt = synth.prompt(cfg["vocab"], 12, seed=2)
+    steps = 5
+    ref = oracle.Llama(cfg, _dequantised(oracle, w, synth.LLAMA_LINEAR_KEYS + ("lm_head",), "q4_0"))
+    want_tokens, want_logits = ref.generate(prompt, steps, keep_logits=True)
+    model = llm.make_llama(cfg, llm.llama_state_dict(w, "q4_0"))
+    got_tokens, got_logits = llm.gpt2_generate(model, prompt, steps, on_device=False, keep_logits=True)
+    assert got_tokens == want_tokens
+    for g, r in zip(got_logits, want_logits):
+        close(g, r)
+    kd = cfg["dim"] // cfg["n_heads"] * cfg["n_kv_heads"]
+    T = len(prompt) + steps - 1
+    close(model.peek("k_cache.1")[:T * kd], ref.k_cache[1].ravel()[:T * kd])
+    model.close()

@@ -49,6 +49,8 @@ static size_t raw_nbytes(int type, int64_t n) {
   }
 }
 
+static const int kStepsPerGraph = 8;
+
 struct Layer {
   // GPT-2
   float *ln1_g = nullptr, *ln1_b = nullptr, *ln2_g = nullptr, *ln2_b = nullptr;
@@ -83,7 +85,7 @@ struct Decoder {
   int position = 0;
   bool primed = false;  // a forward has left token/position on the device
   bool use_graph = true;
-  hipGraphExec_t g_step = nullptr, g_body = nullptr;
+  hipGraphExec_t g_step = nullptr, g_body = nullptr, g_multi = nullptr;
   int64_t weight_bytes = 0, vector_bytes = 0;
   std::vector<void *> owned;  // device blocks to free
 };
@@ -301,10 +303,13 @@ static int finalize(Decoder *d) {
   if (ng && *ng && *ng != '0') d->use_graph = false;
   if (d->use_graph) {
     hipStream_t st = state().stream;
-    for (int pass = 0; pass < 2; pass++) {
+    // 0: one step with the head; 1: one step without (prompt rows fed one by one); 2: kStepsPerGraph steps
+    // with their heads back to back (the device-resident loop: fewer graph launches per token)
+    for (int pass = 0; pass < 3; pass++) {
       hipGraph_t g = nullptr;
       CTHIP_CHECK(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
-      rc = queue_step(d, pass == 0);
+      rc = queue_step(d, pass != 1);
+      for (int k = 1; pass == 2 && k < kStepsPerGraph && !rc; k++) rc = queue_step(d, true);
       hipError_t e = hipStreamEndCapture(st, &g);
       if (rc) {
         if (g) (void)hipGraphDestroy(g);
@@ -315,7 +320,7 @@ static int finalize(Decoder *d) {
       e = hipGraphInstantiate(&ex, g, nullptr, nullptr, 0);
       (void)hipGraphDestroy(g);
       if (e != hipSuccess) return fail((int)e, "decoder: hipGraphInstantiate -> %s", hipGetErrorString(e));
-      (pass == 0 ? d->g_step : d->g_body) = ex;
+      (pass == 0 ? d->g_step : pass == 1 ? d->g_body : d->g_multi) = ex;
     }
   }
 #undef TRY
@@ -540,6 +545,7 @@ int cthip_decoder_destroy(void *dec) {
   if (state().inited) (void)hipStreamSynchronize(state().stream);
   if (d->g_step) (void)hipGraphExecDestroy(d->g_step);
   if (d->g_body) (void)hipGraphExecDestroy(d->g_body);
+  if (d->g_multi) (void)hipGraphExecDestroy(d->g_multi);
   for (auto &kv : d->raw) cthip_free(kv.second.dev);
   for (void *p : d->owned) cthip_free(p);
   for (Layer &L : d->layers) {
@@ -642,7 +648,10 @@ int cthip_decoder_generate(void *dec, int steps, int64_t *tokens_out) {
   if (steps == 0) return 0;
   int rc, zero = 0;
   if ((rc = cthip_h2d(d->hist_n, &zero, sizeof(int)))) return rc;
-  for (int i = 0; i < steps; i++)
+  int i = 0;
+  if (d->use_graph)
+    for (; i + kStepsPerGraph <= steps; i += kStepsPerGraph) CTHIP_CHECK(hipGraphLaunch(d->g_multi, state().stream));
+  for (; i < steps; i++)
     if ((rc = run_step(d, true))) return rc;
   if ((rc = cthip_d2h(tokens_out, d->history, sizeof(int64_t) * (size_t)steps))) return rc;
   d->position += steps;

@@ -1,5 +1,6 @@
 """Prefill timing on one MI355X (`python -m caten_amd.bench_prefill`): a 512-token prompt through the
-GPT-2-small shaped Q8_0 model as one batch (BASELINE config 4's prefill leg): MFMA GEMMs over the
+GPT-2-small shaped Q8_0 model as one batch (BASELINE config 4's prefill leg; `--model llama-1.1b --kind q4_0
+--tokens 128` is config 5's): MFMA GEMMs over the
 rows with the weights dequantised while staged.  Reports the wall time of `forward` (synchronous) and
 the linear-layer FLOP rate against the MFMA peak of the operand type."""
 from __future__ import annotations
@@ -13,13 +14,18 @@ from . import _lib, llm, synth
 
 
 def main(model="gpt2", kind="q8_0", s=512):
-    cfg = synth.GPT2_CONFIGS[model]
-    w = synth.gpt2_weights(cfg, seed=0)
+    llama = model in synth.LLAMA_CONFIGS
+    cfg = synth.LLAMA_CONFIGS[model] if llama else synth.GPT2_CONFIGS[model]
+    w = synth.llama_weights(cfg, seed=0) if llama else synth.gpt2_weights(cfg, seed=0)
     prompt = [float(t) for t in synth.prompt(cfg["vocab"], s, seed=0)]
     lib = _lib.init(0)
-    m = llm.make_gpt2(cfg, llm.gpt2_state_dict(w, kind))
+    m = llm.make_llama(cfg, llm.llama_state_dict(w, kind)) if llama else llm.make_gpt2(cfg, llm.gpt2_state_dict(w, kind))
     D, F, L, V = cfg["dim"], cfg["ffn"], cfg["n_layers"], cfg["vocab"]
-    lin_flop = 2.0 * s * L * (3 * D * D + D * D + 2 * D * F) + 2.0 * V * D  # lm_head on the last row only
+    if llama:
+        KD = D // cfg["n_heads"] * cfg["n_kv_heads"]
+        lin_flop = 2.0 * s * L * (D * (D + 2 * KD) + D * D + 3 * D * F) + 2.0 * V * D
+    else:
+        lin_flop = 2.0 * s * L * (3 * D * D + D * D + 2 * D * F) + 2.0 * V * D  # lm_head on the last row only
     att_flop = 2.0 * 2.0 * L * cfg["n_heads"] * (D // cfg["n_heads"]) * s * (s + 1) / 2
     names = {0: "fp32", 3: "3-term split bf16 (6 MFMAs per product)", 2: "2-term split bf16 (3 MFMAs per product)", 1: "bf16"}
     for mode, peak in ((0, 157.3), (3, 2500.0), (2, 2500.0), (1, 2500.0)):
@@ -40,4 +46,10 @@ def main(model="gpt2", kind="q8_0", s=512):
 
 
 if __name__ == "__main__":
-    main()
+    import argparse
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--model", default="gpt2")
+    ap.add_argument("--kind", default="q8_0")
+    ap.add_argument("--tokens", type=int, default=512)
+    a = ap.parse_args()
+    main(a.model, a.kind, a.tokens)

@@ -238,7 +238,7 @@ __global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
 // holds them k-contiguous per row in bf16, 16-byte chunks swizzled by row so that neither the operand
 // reads nor the staging writes collide on banks.  Two LDS buffers and three register sets keep the
 // global loads three K-steps ahead of the MFMAs with one barrier per step.
-enum { W_ROWMAJOR = 0, W_F32 = 1, W_F16 = 2, W_Q4 = 3, W_Q8 = 4 };
+enum { W_ROWMAJOR = 0, W_F32 = 1, W_F16 = 2, W_Q4 = 3, W_Q8 = 4 };  // W_Q4 / W_Q8: k_gemm_q only
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
 typedef float v2f __attribute__((ext_vector_type(2)));
@@ -272,7 +272,6 @@ template <int BMODE>
 struct BRegs {  // one K-step of B held by a thread between its request and its conversion
   static constexpr int NV = (BMODE == W_ROWMAJOR || BMODE == W_F32) ? 4 : (BMODE == W_F16 ? 2 : 1);
   uint4 v[NV];
-  unsigned short s;
 };
 
 // LDS rows are 64 bf16 = eight 16-byte chunks; chunk c of row r is stored at position c ^ swz(r), which
@@ -363,7 +362,6 @@ __global__ __launch_bounds__(256) void k_gemm_split(GemmArgs a) {
         rb.v[BRegs<BMODE>::NV > 2 ? 2 : 0] = make_uint4(0u, 0u, 0u, 0u);
         rb.v[BRegs<BMODE>::NV > 3 ? 3 : 0] = make_uint4(0u, 0u, 0u, 0u);
       }
-      rb.s = 0;
       if (ok) {
         const int64_t e = (int64_t)n * ldk + k;  // element index of the chunk
         if (BMODE == W_F32) {
@@ -374,12 +372,6 @@ __global__ __launch_bounds__(256) void k_gemm_split(GemmArgs a) {
         } else if (BMODE == W_F16) {
           rb.v[0] = *(const uint4 *)((const unsigned short *)a.wq + e);
           rb.v[BRegs<BMODE>::NV > 1 ? 1 : 0] = *(const uint4 *)((const unsigned short *)a.wq + e + 8);
-        } else if (BMODE == W_Q8) {
-          rb.v[0] = *(const uint4 *)((const int8_t *)a.wq + e);
-          rb.s = a.wd[e >> 5];
-        } else {  // W_Q4: the 32-weight block's 16 bytes; this chunk is its low (k % 32 == 0) or high nibbles
-          rb.v[0] = *(const uint4 *)((const uint8_t *)a.wq + ((e >> 5) << 4));
-          rb.s = a.wd[e >> 5];
         }
       }
     }
@@ -435,23 +427,6 @@ __global__ __launch_bounds__(256) void k_gemm_split(GemmArgs a) {
             x[8 * j + 2 * t + 1] = half_bits_to_float((unsigned short)(dw[t] >> 16));
           }
         }
-      } else if (BMODE == W_Q8) {
-        const float d = half_bits_to_float(rb.s);
-        const unsigned dw[4] = {rb.v[0].x, rb.v[0].y, rb.v[0].z, rb.v[0].w};
-#pragma unroll
-        for (int t = 0; t < 4; t++) {
-          const int v = (int)dw[t];
-          x[4 * t + 0] = (float)(int)(int8_t)(v)*d;
-          x[4 * t + 1] = (float)(int)(int8_t)(v >> 8) * d;
-          x[4 * t + 2] = (float)(int)(int8_t)(v >> 16) * d;
-          x[4 * t + 3] = (float)(v >> 24) * d;
-        }
-      } else {
-        const float d = half_bits_to_float(rb.s);
-        const unsigned dw[4] = {rb.v[0].x, rb.v[0].y, rb.v[0].z, rb.v[0].w};
-        const int sh = (wkc & 1) ? 4 : 0;  // BK = 64 = two blocks: chunks 0, 2 are low nibbles, 1, 3 high
-#pragma unroll
-        for (int t = 0; t < 16; t++) x[t] = (float)((int)((dw[t >> 2] >> (8 * (t & 3) + sh)) & 0xf) - 8) * d;
       }
 #pragma unroll
       for (int j = 0; j < 2; j++) {
@@ -552,6 +527,200 @@ __global__ __launch_bounds__(256) void k_gemm_split(GemmArgs a) {
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Linear over m rows with Q8_0 / Q4_0 weights: the dequantisation is fused into the accumulation.
+//
+// A quantised weight is q * d with q a small integer (int8, or nibble - 8) and d the fp16 scale of its
+// block of 32.  Every such q is exact in bf16, so the matrix cores multiply the activations (split in
+// NPA bf16 terms: 1 = rounded, 2 = 2^-17 per product, 3 = all 24 bits) by the INTEGER plane -- one
+// MFMA per activation term and k-slice, exact products, fp32 sums over the 32 weights of a block --
+// and the block's scale is applied once to that partial sum:  acc += d[n][block] * (sum_k a[m][k] q[n][k]).
+// Against dequantising to fp32 and splitting both operands this needs a third fewer MFMAs, an eighth
+// of the conversion work on the weight side, and is more accurate (no rounding of q * d).
+//
+// One 256-thread workgroup owns 64*MB x 64 of the output (a wavefront accumulates MB 32x32 blocks; MB = 1 is
+// what the launcher uses), walks K in steps of 64 = two quant blocks, same LDS layout / swizzle / prefetch
+// depth / XCD regions / split-K as k_gemm_split.
+template <int MB>
+struct ARegsQ {  // one K-step of A held by a thread: rows ar + 16 i, i < 4 * MB
+  float4 v[4 * MB];
+};
+struct BRegsQ {
+  uint4 v;           // Q8_0: 16 int8; Q4_0: the 16 bytes of a 32-weight block
+  unsigned short d;  // fp16 scale bits (threads tid < 128: row tid >> 1, block tid & 1 of the step)
+};
+
+// two small integers (as floats, exact) -> packed bf16 pair, x0 in the low half
+__device__ __forceinline__ unsigned pack_int_bf16(float x0, float x1) {
+  return (__float_as_uint(x1) & 0xffff0000u) | (__float_as_uint(x0) >> 16);
+}
+
+template <int WT, int NPA, int MB>
+__global__ __launch_bounds__(256) void k_gemm_q(GemmArgs a) {
+  constexpr int BM = 64 * MB, BN = 64, BK = 64, LDK = BK;
+  __shared__ __align__(16) unsigned short As[2][NPA][BM][LDK];
+  __shared__ __align__(16) unsigned short Bs[2][BN][LDK];
+  __shared__ float Ss[2][BN][2];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+  if (local >= a.rm * a.rn) return;
+  const int mi = (xcd % a.rx) * a.rm + local % a.rm, ni = (xcd / a.rx) * a.rn + local / a.rm;
+  if (mi >= a.tm || ni >= a.tn) return;
+  const int m0 = mi * BM, n0 = ni * BN;
+  const int M = a.M, N = a.N, ldk = a.K;
+  const int kbeg = blockIdx.y * a.kper;
+  const int K = min(a.K, kbeg + a.kper);
+  const bool vecA = (ldk % 4 == 0);
+  v16f acc[MB];
+#pragma unroll
+  for (int b = 0; b < MB; b++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[b][r] = 0.0f;
+
+  const int ar = tid >> 4, akq = tid & 15;  // A: rows ar + 16 i, k = 4 akq .. +3
+  const int wr = tid >> 2, wkc = tid & 3;   // B: weight row wr, k = 16 wkc .. +15
+  const int sr = tid >> 1, sb = tid & 1;    // scales (tid < 128): row sr, quant block sb of the step
+  const int blocks_per_row = ldk >> 5;
+
+  auto fetch = [&](int k0, ARegsQ<MB> &ra, BRegsQ &rb) {  // k0 counts from kbeg
+#pragma unroll
+    for (int i = 0; i < 4 * MB; i++) {
+      const int row = m0 + ar + 16 * i, k = kbeg + k0 + 4 * akq;
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (row < M) {
+        const float *src = a.A + (int64_t)row * ldk + k;
+        if (vecA && k + 4 <= K) {
+          v = *(const float4 *)src;
+        } else {
+          if (k + 0 < K) v.x = src[0];
+          if (k + 1 < K) v.y = src[1];
+          if (k + 2 < K) v.z = src[2];
+          if (k + 3 < K) v.w = src[3];
+        }
+      }
+      ra.v[i] = v;
+    }
+    // K is a multiple of 32: a 16-wide chunk / a quant block is inside the row or past this share's end
+    const int n = n0 + wr, k = kbeg + k0 + 16 * wkc;
+    rb.v = make_uint4(0u, 0u, 0u, 0u);
+    if (n < N && k < K) {
+      const int64_t e = (int64_t)n * ldk + k;
+      if (WT == W_Q8) rb.v = *(const uint4 *)((const int8_t *)a.wq + e);
+      else rb.v = *(const uint4 *)((const uint8_t *)a.wq + ((e >> 5) << 4));
+    }
+    rb.d = 0;
+    if (tid < 128) {
+      const int ns = n0 + sr, ks = kbeg + k0 + 32 * sb;
+      if (ns < N && ks < K) rb.d = a.wd[(int64_t)ns * blocks_per_row + (ks >> 5)];
+    }
+  };
+  auto stage = [&](const ARegsQ<MB> &ra, const BRegsQ &rb, int buf) {
+#pragma unroll
+    for (int i = 0; i < 4 * MB; i++) {
+      const float x[4] = {ra.v[i].x, ra.v[i].y, ra.v[i].z, ra.v[i].w};
+      uint2 pl[NPA];
+      split4<NPA>(x, pl);
+      const int row = ar + 16 * i;
+#pragma unroll
+      for (int p = 0; p < NPA; p++) *(uint2 *)&As[buf][p][row][8 * ((akq >> 1) ^ swz(row)) + 4 * (akq & 1)] = pl[p];
+    }
+    float q[16];
+    const unsigned dw[4] = {rb.v.x, rb.v.y, rb.v.z, rb.v.w};
+    if (WT == W_Q8) {
+#pragma unroll
+      for (int t = 0; t < 4; t++) {
+        const int v = (int)dw[t];
+        q[4 * t + 0] = (float)(int)(int8_t)(v);
+        q[4 * t + 1] = (float)(int)(int8_t)(v >> 8);
+        q[4 * t + 2] = (float)(int)(int8_t)(v >> 16);
+        q[4 * t + 3] = (float)(v >> 24);
+      }
+    } else {
+      const int sh = (wkc & 1) ? 4 : 0;  // chunks 0, 2 of the step are the low nibbles of their block, 1, 3 the high
+#pragma unroll
+      for (int t = 0; t < 16; t++) q[t] = (float)((int)((dw[t >> 2] >> (8 * (t & 3) + sh)) & 0xf) - 8);
+    }
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+      *(uint4 *)&Bs[buf][wr][8 * ((2 * wkc + j) ^ swz(wr))] =
+          make_uint4(pack_int_bf16(q[8 * j + 0], q[8 * j + 1]), pack_int_bf16(q[8 * j + 2], q[8 * j + 3]),
+                     pack_int_bf16(q[8 * j + 4], q[8 * j + 5]), pack_int_bf16(q[8 * j + 6], q[8 * j + 7]));
+    if (tid < 128) Ss[buf][sr][sb] = half_bits_to_float(rb.d);
+  };
+  auto mma = [&](int buf) {
+    const int rowb = 32 * wn + (lane & 31);
+#pragma unroll
+    for (int kb = 0; kb < 2; kb++) {  // the two quant blocks of the step
+      v16f tmp[MB];
+#pragma unroll
+      for (int b = 0; b < MB; b++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) tmp[b][r] = 0.0f;
+#pragma unroll
+      for (int s2 = 0; s2 < 2; s2++) {
+        const int ch = 4 * kb + 2 * s2 + (lane >> 5);
+        const v8bf bv = __builtin_bit_cast(v8bf, *(const uint4 *)&Bs[buf][rowb][8 * (ch ^ swz(rowb))]);
+#pragma unroll
+        for (int b = 0; b < MB; b++) {
+          const int rowa = 32 * MB * wm + 32 * b + (lane & 31);
+#pragma unroll
+          for (int p = NPA - 1; p >= 0; p--) {
+            const v8bf av = __builtin_bit_cast(v8bf, *(const uint4 *)&As[buf][p][rowa][8 * (ch ^ swz(rowa))]);
+            tmp[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv, tmp[b], 0, 0, 0);
+          }
+        }
+      }
+      const float d = Ss[buf][rowb][kb];  // scale of this lane's output column for this block
+#pragma unroll
+      for (int b = 0; b < MB; b++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[b][r] = fmaf(d, tmp[b][r], acc[b][r]);
+    }
+  };
+
+  ARegsQ<MB> ra0, ra1, ra2;
+  BRegsQ rb0, rb1, rb2;
+  const int nsteps = K > kbeg ? (K - kbeg + BK - 1) / BK : 0;
+  if (nsteps > 0) fetch(0, ra0, rb0);
+  if (nsteps > 1) fetch(BK, ra1, rb1);
+  if (nsteps > 2) fetch(2 * BK, ra2, rb2);
+  if (nsteps > 0) stage(ra0, rb0, 0);
+  if (nsteps > 3) fetch(3 * BK, ra0, rb0);
+  __syncthreads();
+  auto step = [&](int i, ARegsQ<MB> &ran, BRegsQ &rbn) {
+    if (i + 1 < nsteps) stage(ran, rbn, (i + 1) & 1);
+    if (i + 4 < nsteps) fetch((i + 4) * BK, ran, rbn);
+    mma(i & 1);
+    __syncthreads();
+  };
+  for (int i = 0; i < nsteps; i += 3) {
+    step(i, ra1, rb1);
+    if (i + 1 < nsteps) step(i + 1, ra2, rb2);
+    if (i + 2 < nsteps) step(i + 2, ra0, rb0);
+  }
+  // ---- epilogue: acc[b][r] is C[row = 8*(r/4) + 4*(l/32) + r%4][col = l%32] of the wavefront's block b ----
+  const int col = n0 + 32 * wn + (lane & 31);
+  if (col >= N) return;
+  const float bias = (a.ksplit > 1 || !a.bias) ? 0.0f : a.bias[col];
+  float *dst = a.ksplit > 1 ? a.ws + (int64_t)blockIdx.y * M * N : a.C;
+#pragma unroll
+  for (int b = 0; b < MB; b++) {
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int row = m0 + 32 * MB * wm + 32 * b + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+      if (row < M) {
+        float v = acc[b][r];
+        if (a.ksplit <= 1) {
+          v = apply_act(a.act, v + bias);
+          if (a.residual) v += a.residual[(int64_t)row * N + col];
+        }
+        dst[(int64_t)row * N + col] = v;
+      }
+    }
+  }
+}
+
 // C = act(sum_z ws[z] + bias) + residual, z in ascending order (the result does not depend on timing)
 __global__ __launch_bounds__(256) void k_splitk_reduce(GemmArgs a) {
   const int64_t n = (int64_t)a.M * a.N;
@@ -566,21 +735,27 @@ __global__ __launch_bounds__(256) void k_splitk_reduce(GemmArgs a) {
 }
 
 // precision: GEMM_FP32 = fp32 MFMA operands (k_gemm), GEMM_BF16 = operands rounded to bf16,
-// GEMM_BF16X3 / GEMM_BF16X6 = operands split in two / three bf16 terms
+// GEMM_BF16X3 / GEMM_BF16X6 = operands split in two / three bf16 terms.  Q8_0 / Q4_0 weights take k_gemm_q
+// (integer plane exact in bf16, block scales applied to the partial sums) with 1 / 2 / 3 activation terms.
 int launch_gemm(GemmArgs a, int bmode, int precision) {
   if (a.M == 0 || a.N == 0) return 0;
-  const int64_t tiles = (int64_t)((a.M + 63) / 64) * ((a.N + 63) / 64);
-  if (tiles > 0x7fffffff) return fail(CTHIP_E_BAD_ARG, "gemm: too many tiles");
-  dim3 grid((unsigned)tiles), block(256);
   hipStream_t st = state().stream;
+  const int cus = state().compute_units;
+  const bool quant = precision != GEMM_FP32 && bmode == B_WMAT && (a.wtype == CTHIP_Q8_0 || a.wtype == CTHIP_Q4_0);
+  // 64 output rows per workgroup.  (128-row tiles -- two accumulator blocks per wavefront, half the weight-side
+  // staging -- measured slower on every prefill shape: one workgroup per compute unit and 32 KB of A per step.)
+  const int bm = 64;
+  const int64_t tiles = (int64_t)((a.M + bm - 1) / bm) * ((a.N + 63) / 64);
+  if (tiles > 0x7fffffff / 16) return fail(CTHIP_E_BAD_ARG, "gemm: too many tiles");
+  dim3 grid((unsigned)tiles), block(256);
   a.ksplit = 1;
   a.kper = a.K > 0 ? a.K : 1;
   a.ws = nullptr;
   if (precision != GEMM_FP32) {
     // one region of tiles per XCD: the split with the fewest tiles per XCD, then the least operand bytes per L2
-    a.tm = (a.M + 63) / 64;
+    a.tm = (a.M + bm - 1) / bm;
     a.tn = (a.N + 63) / 64;
-    const double sza = 4.0, szb = bmode == B_ROWMAJOR ? 4.0 : a.wtype == CTHIP_Q8_0 ? 1.0625 : a.wtype == CTHIP_Q4_0 ? 0.5625 : a.wtype == CTHIP_F16 ? 2.0 : 4.0;
+    const double sza = 4.0 * bm / 64, szb = bmode == B_ROWMAJOR ? 4.0 : a.wtype == CTHIP_Q8_0 ? 1.0625 : a.wtype == CTHIP_Q4_0 ? 0.5625 : a.wtype == CTHIP_F16 ? 2.0 : 4.0;
     double best = -1.0;
     for (int rx = 1; rx <= 8; rx *= 2) {
       const int ry = 8 / rx, rm = (a.tm + rx - 1) / rx, rn = (a.tn + ry - 1) / ry;
@@ -594,7 +769,7 @@ int launch_gemm(GemmArgs a, int bmode, int precision) {
     }
     grid.x = 8u * (unsigned)a.rm * (unsigned)a.rn;
     // too few tiles to occupy the chip and a long reduction axis: split K over several workgroups per tile
-    const int cus = state().compute_units, nsteps = (a.K + 63) / 64;
+    const int nsteps = (a.K + 63) / 64;
     int ks = (int)((cus * 3 / 2) / tiles);
     if (ks > nsteps / 6) ks = nsteps / 6;
     if (ks > 16) ks = 16;
@@ -614,9 +789,23 @@ int launch_gemm(GemmArgs a, int bmode, int precision) {
   if (precision == GEMM_FP32) {
     if (bmode == B_ROWMAJOR) hipLaunchKernelGGL((k_gemm<B_ROWMAJOR, false>), grid, block, 0, st, a);
     else hipLaunchKernelGGL((k_gemm<B_WMAT, false>), grid, block, 0, st, a);
+  } else if (quant) {
+    const int npa = precision == GEMM_BF16X6 ? 3 : precision == GEMM_BF16X3 ? 2 : 1;
+#define QG(WT, NPA, MB) hipLaunchKernelGGL((k_gemm_q<WT, NPA, MB>), grid, block, 0, st, a)
+#define QSEL(WT)                  \
+  if (npa == 3) QG(WT, 3, 1);     \
+  else if (npa == 2) QG(WT, 2, 1); \
+  else QG(WT, 1, 1);
+    if (a.wtype == CTHIP_Q8_0) {
+      QSEL(W_Q8)
+    } else {
+      QSEL(W_Q4)
+    }
+#undef QSEL
+#undef QG
   } else {
     int wm = W_ROWMAJOR;
-    if (bmode == B_WMAT) wm = a.wtype == CTHIP_Q8_0 ? W_Q8 : a.wtype == CTHIP_Q4_0 ? W_Q4 : a.wtype == CTHIP_F16 ? W_F16 : W_F32;
+    if (bmode == B_WMAT) wm = a.wtype == CTHIP_F16 ? W_F16 : W_F32;
 #define SPLIT(MODE)                                                                                          \
   case MODE:                                                                                                 \
     if (precision == GEMM_BF16X6) hipLaunchKernelGGL((k_gemm_split<MODE, 6>), grid, block, 0, st, a);        \
@@ -627,18 +816,22 @@ int launch_gemm(GemmArgs a, int bmode, int precision) {
       SPLIT(W_ROWMAJOR);
       SPLIT(W_F32);
       SPLIT(W_F16);
-      SPLIT(W_Q4);
-      SPLIT(W_Q8);
     }
 #undef SPLIT
   }
-  CTHIP_LAUNCH_CHECK();
+  hipError_t le = hipGetLastError();
+  if (le != hipSuccess) {
+    if (a.ws) cthip_free(a.ws);
+    return fail((int)le, "gemm: launch -> %s", hipGetErrorString(le));
+  }
   if (a.ksplit > 1) {
     int64_t blocks = ((int64_t)a.M * a.N + 255) / 256;
     if (blocks > 4096) blocks = 4096;
     hipLaunchKernelGGL(k_splitk_reduce, dim3((unsigned)blocks), dim3(256), 0, st, a);
-    CTHIP_LAUNCH_CHECK();
-    return cthip_free(a.ws);  // stream-ordered: the block is reused only by later work on the same stream
+    le = hipGetLastError();
+    int rc = cthip_free(a.ws);  // stream-ordered: the block is reused only by later work on the same stream
+    if (le != hipSuccess) return fail((int)le, "gemm: launch -> %s", hipGetErrorString(le));
+    return rc;
   }
   return 0;
 }

@@ -343,6 +343,32 @@ def test_matmul_degenerate(ops):
     assert np.all(ops.matmul(np.zeros((3, 0), np.float32), np.zeros((0, 4), np.float32)) == 0)
 
 
+@pytest.mark.parametrize("kind", ["q8_0", "q4_0"])
+def test_linear_many_rows_quantised(ops, oracle, kind):
+    """130 input rows x 4100 weight rows, ragged tile edges in both directions: the integer plane times the block
+    scales (quantised MFMA path) must match the product with the dequantised weights."""
+    from caten_amd import _lib
+    from caten_amd.llm import Tensor
+    rng = np.random.default_rng(62)
+    rows, cols, m = 4100, 256, 130
+    w = rng.normal(0, 0.02, (rows, cols)).astype(np.float32)
+    x = rng.normal(0, 1, (m, cols)).astype(np.float32)
+    b = rng.normal(0, 0.02, rows).astype(np.float32)
+    t = Tensor.from_f32(w, kind)
+    wd = oracle.dequant(kind, t.raw, w.size).reshape(rows, cols)
+    wm = ops.WeightMatrix(kind, t.raw, rows, cols)
+    want = oracle.linear(x, wd, b)
+    lib = _lib.load()
+    try:
+        for mode in (2, 3):
+            _lib.check(lib.cthip_set_option(b"gemm_precision", mode))
+            close(ops.linear(x, wm, bias=b), want)
+        _lib.check(lib.cthip_set_option(b"gemm_precision", 1))
+        close(ops.linear(x, wm, bias=b), want, 1e-2, 1e-2)
+    finally:
+        _lib.check(lib.cthip_set_option(b"gemm_precision", 2))
+
+
 @pytest.mark.parametrize("kind", ["q8_0", "q4_0", "f16", "f32"])
 def test_linear_prefill_rows_mfma(ops, oracle, kind):
     # m >= 8 input rows take the MFMA tile path with the weights dequantised while staged

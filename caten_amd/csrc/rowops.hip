@@ -636,13 +636,151 @@ __global__ __launch_bounds__(256) void k_attn_rows(float *__restrict__ out, cons
   }
 }
 
+// Prompt rows on the matrix cores (s >= 32): one 256-thread block per (head, 32 consecutive query rows); its
+// four wavefronts take the 32-key tiles of the visible cache round-robin, each with its own online softmax
+// for all 32 rows, and meet once in LDS.  fp32 MFMA operands (v_mfma_f32_32x32x2_f32): the products are the
+// reference's fp32 products, only the summation order differs.
+//   S^T = K Q^T : lane l feeds K[key l%32][d = 2s + l/32] (from a d-major LDS copy of the key tile) and
+//                 Q[query l%32][d = 2s + l/32] (registers), so a lane ends up with 16 keys of ONE query;
+//   softmax     : per lane over its 16 registers + one exchange with lane l^32;
+//   O^T += V^T P^T : lane l feeds V[key of register s][d = l%32 (+32 per block)] straight from the cache
+//                 (128 contiguous bytes per half-wavefront) and P = its own register s: the output stays
+//                 one query per lane, so the running rescale is a per-lane scalar.
+typedef float v16f_t __attribute__((ext_vector_type(16)));
+
+template <int DH>
+__global__ __launch_bounds__(256) void k_attn_mfma(float *__restrict__ out, const float *__restrict__ q,
+                                                   const float *__restrict__ kc, const float *__restrict__ vc, int S,
+                                                   int start_pos, int H, int Hkv) {
+  constexpr int NS = DH / 2;   // k-steps of K Q^T
+  constexpr int DB = DH / 32;  // 32-wide blocks of the head dimension
+  __shared__ float Kt[4][DH][33];        // per wavefront: its key tile, d-major
+  __shared__ float Co[4][DB * 16][64];   // per wavefront: unnormalised outputs for the final combine
+  __shared__ float Cm[4][64], Cl[4][64];
+  const int h = blockIdx.x, i0 = (gridDim.y - 1 - blockIdx.y) * 32;  // the longest groups are dispatched first
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int half = lane >> 5, col = lane & 31;
+  const int hk = h / (H / Hkv), KD = Hkv * DH;
+  const int qrow = min(i0 + col, S - 1);  // rows past the end repeat the last one and are not stored
+  const int Tq = start_pos + qrow + 1;    // keys this lane's query sees
+  const int Tmax = start_pos + min(i0 + 32, S);
+  const int ntiles = (Tmax + 31) / 32;
+  const float scale = 1.0f / sqrtf((float)DH);
+  float qreg[NS];
+#pragma unroll
+  for (int s = 0; s < NS; s++) qreg[s] = q[((int64_t)qrow * H + h) * DH + 2 * s + half];
+  float m = -INFINITY, l = 0.0f;
+  v16f_t o[DB];
+#pragma unroll
+  for (int b = 0; b < DB; b++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) o[b][r] = 0.0f;
+
+  for (int t = wv; t < ntiles; t += 4) {
+    const int kb = t * 32;
+    // the key tile, transposed into LDS (rows clamped to the last visible one: masked below)
+#pragma unroll
+    for (int u = 0; u < DH / 8; u++) {
+      const int f = lane + 64 * u, key = f / (DH / 4), d4 = f % (DH / 4);
+      const int kr = min(kb + key, Tmax - 1);
+      const float4 v = *(const float4 *)(kc + (int64_t)kr * KD + hk * DH + 4 * d4);
+      Kt[wv][4 * d4 + 0][key] = v.x;
+      Kt[wv][4 * d4 + 1][key] = v.y;
+      Kt[wv][4 * d4 + 2][key] = v.z;
+      Kt[wv][4 * d4 + 3][key] = v.w;
+    }
+    __builtin_amdgcn_wave_barrier();
+    v16f_t sacc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) sacc[r] = 0.0f;
+#pragma unroll
+    for (int s = 0; s < NS; s++) sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(Kt[wv][2 * s + half][col], qreg[s], sacc, 0, 0, 0);
+    __builtin_amdgcn_wave_barrier();
+    // sacc[r] = score of key kb + 8*(r/4) + 4*half + r%4 against query `col`
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int key = kb + 8 * (r >> 2) + 4 * half + (r & 3);
+      const float sc = (key < Tq) ? sacc[r] * scale : -INFINITY;
+      sacc[r] = sc;
+      tmax = fmaxf(tmax, sc);
+    }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float m_new = fmaxf(m, tmax);
+    const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;  // no key of this tile visible to this query yet
+    const float corr = ct_exp(m - m_use);
+    float ps = 0.0f;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const float p = ct_exp(sacc[r] - m_use);
+      sacc[r] = p;
+      ps += p;
+    }
+    ps += __shfl_xor(ps, 32, 64);
+    l = l * corr + ps;
+    m = m_new;
+#pragma unroll
+    for (int b = 0; b < DB; b++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) o[b][r] *= corr;
+#pragma unroll
+    for (int s = 0; s < 16; s++) {
+      const int kr = min(kb + 8 * (s >> 2) + 4 * half + (s & 3), Tmax - 1);
+      const float *vrow = vc + (int64_t)kr * KD + hk * DH + col;
+#pragma unroll
+      for (int b = 0; b < DB; b++) o[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(vrow[32 * b], sacc[s], o[b], 0, 0, 0);
+    }
+  }
+  // o[b][r] = unnormalised output element d = 32b + 8*(r/4) + 4*half + r%4 of query `col`
+  Cm[wv][lane] = m;
+  Cl[wv][lane] = l;
+#pragma unroll
+  for (int b = 0; b < DB; b++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) Co[wv][b * 16 + r][lane] = o[b][r];
+  __syncthreads();
+  float M = Cm[0][lane];
+#pragma unroll
+  for (int w = 1; w < 4; w++) M = fmaxf(M, Cm[w][lane]);  // finite: the wavefront holding key 0 saw it
+  float e[4], L = 0.0f;
+#pragma unroll
+  for (int w = 0; w < 4; w++) {
+    e[w] = (Cm[w][lane] == -INFINITY) ? 0.0f : ct_exp(Cm[w][lane] - M);
+    L = fmaf(e[w], Cl[w][lane], L);
+  }
+  const float inv = 1.0f / L;
+  if (i0 + col < S) {
+    float *orow = out + ((int64_t)(i0 + col) * H + h) * DH;
+    // wavefront wv finishes registers wv * DB*4 .. of every lane
+#pragma unroll
+    for (int k = 0; k < DB * 4; k++) {
+      const int R = wv * DB * 4 + k, b = R >> 4, r = R & 15;
+      float v = 0.0f;
+#pragma unroll
+      for (int w = 0; w < 4; w++) v = fmaf(e[w], Co[w][R][lane], v);
+      orow[32 * b + 8 * (r >> 2) + 4 * half + (r & 3)] = v * inv;
+    }
+  }
+}
+
 int launch_attn(float *out, const float *q, const float *kc, const float *vc, int S, int start_pos, const int *pos,
                 int max_T, int H, int Hkv, int Dh) {
   if (S == 0) return 0;
   (void)max_T;
   hipStream_t st = state().stream;
+  if (S >= 32 && pos == nullptr) {  // prompt rows on the matrix cores
+    dim3 grid(H, (S + 31) / 32), block(256);
+    switch (Dh) {
+      case 32: hipLaunchKernelGGL(k_attn_mfma<32>, grid, block, 0, st, out, q, kc, vc, S, start_pos, H, Hkv); break;
+      case 64: hipLaunchKernelGGL(k_attn_mfma<64>, grid, block, 0, st, out, q, kc, vc, S, start_pos, H, Hkv); break;
+      case 128: hipLaunchKernelGGL(k_attn_mfma<128>, grid, block, 0, st, out, q, kc, vc, S, start_pos, H, Hkv); break;
+      default: return fail(CTHIP_E_UNSUPPORTED, "attention: head_dim %d (supported: 32, 64, 128)", Dh);
+    }
+    CTHIP_LAUNCH_CHECK();
+    return 0;
+  }
   constexpr int R = 8;
-  if (S >= 2 * R) {  // prompt rows: groups of R rows share their K / V loads
+  if (S >= 2 * R) {  // short prompts: groups of R rows share their K / V loads
     dim3 grid(H, (S + R - 1) / R), block(256);
     switch (Dh) {
       case 32: hipLaunchKernelGGL((k_attn_rows<32, R>), grid, block, 0, st, out, q, kc, vc, S, start_pos, pos, H, Hkv); break;

@@ -291,7 +291,9 @@ def test_rope(ops, oracle):
                                              (1, 700, 4, 1, 128), (3, 0, 2, 2, 32),
                                              # prompt-sized row counts: groups of rows share their K / V tiles
                                              (16, 0, 4, 4, 64), (37, 5, 8, 2, 64), (130, 0, 2, 2, 64), (21, 200, 2, 1, 128),
-                                             (19, 3, 2, 2, 32), (512, 0, 2, 2, 64)])
+                                             (19, 3, 2, 2, 32), (512, 0, 2, 2, 64),
+                                             # 32 rows and more: the matrix-core kernel (ragged last group, GQA, other head sizes)
+                                             (32, 0, 2, 2, 64), (33, 7, 4, 2, 64), (70, 100, 2, 1, 128), (45, 2, 2, 2, 32)])
 def test_sdpa_cached(ops, oracle, S, start, H, Hkv, Dh):
     rng = np.random.default_rng(S + start)
     T = start + S

@@ -125,8 +125,10 @@ def main():
     tok_s = args.steps / wall
 
     # ---- roofline of the step kernel sequence, HIP events on the launch stream ----
-    if model.position + args.steps > cfg["max_seq"]:
-        model.forward([float(t) for t in prompt], len(prompt), 0)
+    # the same positions as the timed region above: restart from the prompt and redo the warm-up steps
+    model.forward([float(t) for t in prompt], len(prompt), 0)
+    if args.warmup:
+        model.generate_on_device(min(args.warmup, cfg["max_seq"] - model.position - 1))
     k = min(args.steps, cfg["max_seq"] - model.position)
     pos0 = model.position
     out = np.empty(k, np.int64)

@@ -636,8 +636,8 @@ __global__ __launch_bounds__(256) void k_attn_rows(float *__restrict__ out, cons
   }
 }
 
-// Prompt rows on the matrix cores (s >= 32): one 256-thread block per (head, 32 consecutive query rows); its
-// four wavefronts take the 32-key tiles of the visible cache round-robin, each with its own online softmax
+// Prompt rows on the matrix cores (s >= 32): one block per (head, 32 consecutive query rows); its
+// NW wavefronts take the 32-key tiles of the visible cache round-robin, each with its own online softmax
 // for all 32 rows, and meet once in LDS.  fp32 MFMA operands (v_mfma_f32_32x32x2_f32): the products are the
 // reference's fp32 products, only the summation order differs.
 //   S^T = K Q^T : lane l feeds K[key l%32][d = 2s + l/32] (from a d-major LDS copy of the key tile) and
@@ -648,15 +648,15 @@ __global__ __launch_bounds__(256) void k_attn_rows(float *__restrict__ out, cons
 //                 one query per lane, so the running rescale is a per-lane scalar.
 typedef float v16f_t __attribute__((ext_vector_type(16)));
 
-template <int DH>
-__global__ __launch_bounds__(256) void k_attn_mfma(float *__restrict__ out, const float *__restrict__ q,
+template <int DH, int NW>
+__global__ __launch_bounds__(64 * NW) void k_attn_mfma(float *__restrict__ out, const float *__restrict__ q,
                                                    const float *__restrict__ kc, const float *__restrict__ vc, int S,
                                                    int start_pos, int H, int Hkv) {
   constexpr int NS = DH / 2;   // k-steps of K Q^T
   constexpr int DB = DH / 32;  // 32-wide blocks of the head dimension
-  __shared__ float Kt[4][DH][33];        // per wavefront: its key tile, d-major
-  __shared__ float Co[4][DB * 16][64];   // per wavefront: unnormalised outputs for the final combine
-  __shared__ float Cm[4][64], Cl[4][64];
+  __shared__ float Kt[NW][DH][33];        // per wavefront: its key tile, d-major
+  __shared__ float Co[NW][DB * 16][64];   // per wavefront: unnormalised outputs for the final combine
+  __shared__ float Cm[NW][64], Cl[NW][64];
   const int h = blockIdx.x, i0 = (gridDim.y - 1 - blockIdx.y) * 32;  // the longest groups are dispatched first
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int half = lane >> 5, col = lane & 31;
@@ -676,19 +676,38 @@ __global__ __launch_bounds__(256) void k_attn_mfma(float *__restrict__ out, cons
 #pragma unroll
     for (int r = 0; r < 16; r++) o[b][r] = 0.0f;
 
-  for (int t = wv; t < ntiles; t += 4) {
-    const int kb = t * 32;
-    // the key tile, transposed into LDS (rows clamped to the last visible one: masked below)
+  // the key tile of a pass is requested one pass ahead, its values at the start of the pass: both are in
+  // registers by the time the matrix cores need them
+  float4 kreg[DH / 8];
+  auto load_k = [&](int t) {
 #pragma unroll
     for (int u = 0; u < DH / 8; u++) {
       const int f = lane + 64 * u, key = f / (DH / 4), d4 = f % (DH / 4);
-      const int kr = min(kb + key, Tmax - 1);
-      const float4 v = *(const float4 *)(kc + (int64_t)kr * KD + hk * DH + 4 * d4);
-      Kt[wv][4 * d4 + 0][key] = v.x;
-      Kt[wv][4 * d4 + 1][key] = v.y;
-      Kt[wv][4 * d4 + 2][key] = v.z;
-      Kt[wv][4 * d4 + 3][key] = v.w;
+      const int kr = min(t * 32 + key, Tmax - 1);  // rows clamped to the last visible one: masked below
+      kreg[u] = *(const float4 *)(kc + (int64_t)kr * KD + hk * DH + 4 * d4);
     }
+  };
+  if (wv < ntiles) load_k(wv);
+  for (int t = wv; t < ntiles; t += NW) {
+    const int kb = t * 32;
+    // the key tile, transposed into LDS
+#pragma unroll
+    for (int u = 0; u < DH / 8; u++) {
+      const int f = lane + 64 * u, key = f / (DH / 4), d4 = f % (DH / 4);
+      Kt[wv][4 * d4 + 0][key] = kreg[u].x;
+      Kt[wv][4 * d4 + 1][key] = kreg[u].y;
+      Kt[wv][4 * d4 + 2][key] = kreg[u].z;
+      Kt[wv][4 * d4 + 3][key] = kreg[u].w;
+    }
+    float vreg[DB][16];
+#pragma unroll
+    for (int s = 0; s < 16; s++) {
+      const int kr = min(kb + 8 * (s >> 2) + 4 * half + (s & 3), Tmax - 1);
+      const float *vrow = vc + (int64_t)kr * KD + hk * DH + col;
+#pragma unroll
+      for (int b = 0; b < DB; b++) vreg[b][s] = vrow[32 * b];
+    }
+    if (t + NW < ntiles) load_k(t + NW);
     __builtin_amdgcn_wave_barrier();
     v16f_t sacc;
 #pragma unroll
@@ -724,12 +743,9 @@ __global__ __launch_bounds__(256) void k_attn_mfma(float *__restrict__ out, cons
 #pragma unroll
       for (int r = 0; r < 16; r++) o[b][r] *= corr;
 #pragma unroll
-    for (int s = 0; s < 16; s++) {
-      const int kr = min(kb + 8 * (s >> 2) + 4 * half + (s & 3), Tmax - 1);
-      const float *vrow = vc + (int64_t)kr * KD + hk * DH + col;
+    for (int s = 0; s < 16; s++)
 #pragma unroll
-      for (int b = 0; b < DB; b++) o[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(vrow[32 * b], sacc[s], o[b], 0, 0, 0);
-    }
+      for (int b = 0; b < DB; b++) o[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(vreg[b][s], sacc[s], o[b], 0, 0, 0);
   }
   // o[b][r] = unnormalised output element d = 32b + 8*(r/4) + 4*half + r%4 of query `col`
   Cm[wv][lane] = m;
@@ -741,23 +757,24 @@ __global__ __launch_bounds__(256) void k_attn_mfma(float *__restrict__ out, cons
   __syncthreads();
   float M = Cm[0][lane];
 #pragma unroll
-  for (int w = 1; w < 4; w++) M = fmaxf(M, Cm[w][lane]);  // finite: the wavefront holding key 0 saw it
-  float e[4], L = 0.0f;
+  for (int w = 1; w < NW; w++) M = fmaxf(M, Cm[w][lane]);  // finite: the wavefront holding key 0 saw it
+  float e[NW], L = 0.0f;
 #pragma unroll
-  for (int w = 0; w < 4; w++) {
+  for (int w = 0; w < NW; w++) {
     e[w] = (Cm[w][lane] == -INFINITY) ? 0.0f : ct_exp(Cm[w][lane] - M);
     L = fmaf(e[w], Cl[w][lane], L);
   }
   const float inv = 1.0f / L;
   if (i0 + col < S) {
     float *orow = out + ((int64_t)(i0 + col) * H + h) * DH;
-    // wavefront wv finishes registers wv * DB*4 .. of every lane
+    // wavefront wv finishes registers wv * RPW .. of every lane
+    constexpr int RPW = DB * 16 / NW;
 #pragma unroll
-    for (int k = 0; k < DB * 4; k++) {
-      const int R = wv * DB * 4 + k, b = R >> 4, r = R & 15;
+    for (int k = 0; k < RPW; k++) {
+      const int R = wv * RPW + k, b = R >> 4, r = R & 15;
       float v = 0.0f;
 #pragma unroll
-      for (int w = 0; w < 4; w++) v = fmaf(e[w], Co[w][R][lane], v);
+      for (int w = 0; w < NW; w++) v = fmaf(e[w], Co[w][R][lane], v);
       orow[32 * b + 8 * (r >> 2) + 4 * half + (r & 3)] = v * inv;
     }
   }
@@ -769,11 +786,12 @@ int launch_attn(float *out, const float *q, const float *kc, const float *vc, in
   (void)max_T;
   hipStream_t st = state().stream;
   if (S >= 32 && pos == nullptr) {  // prompt rows on the matrix cores
-    dim3 grid(H, (S + 31) / 32), block(256);
+    // eight wavefronts per block where their LDS tiles fit (head_dim <= 64), four otherwise
+    dim3 grid(H, (S + 31) / 32);
     switch (Dh) {
-      case 32: hipLaunchKernelGGL(k_attn_mfma<32>, grid, block, 0, st, out, q, kc, vc, S, start_pos, H, Hkv); break;
-      case 64: hipLaunchKernelGGL(k_attn_mfma<64>, grid, block, 0, st, out, q, kc, vc, S, start_pos, H, Hkv); break;
-      case 128: hipLaunchKernelGGL(k_attn_mfma<128>, grid, block, 0, st, out, q, kc, vc, S, start_pos, H, Hkv); break;
+      case 32: hipLaunchKernelGGL((k_attn_mfma<32, 8>), grid, dim3(512), 0, st, out, q, kc, vc, S, start_pos, H, Hkv); break;
+      case 64: hipLaunchKernelGGL((k_attn_mfma<64, 8>), grid, dim3(512), 0, st, out, q, kc, vc, S, start_pos, H, Hkv); break;
+      case 128: hipLaunchKernelGGL((k_attn_mfma<128, 4>), grid, dim3(256), 0, st, out, q, kc, vc, S, start_pos, H, Hkv); break;
       default: return fail(CTHIP_E_UNSUPPORTED, "attention: head_dim %d (supported: 32, 64, 128)", Dh);
     }
     CTHIP_LAUNCH_CHECK();

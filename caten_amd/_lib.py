@@ -102,6 +102,11 @@ PROTOTYPES = {
     "cthip_gguf_metadata_number": (_i, [_vp, _i64, C.POINTER(C.c_double)]),
     "cthip_gguf_metadata_string": (_i, [_vp, _i64, _i64, C.POINTER(C.c_void_p), C.POINTER(_i64)]),
     "cthip_decoder_load_gguf": (_i, [_vp, _vp, _i, C.POINTER(_i)]),
+    "cthip_bpe_create": (_i, [_vpp, C.c_char_p, _sz, C.c_char_p, _sz]),
+    "cthip_bpe_destroy": (_i, [_vp]),
+    "cthip_bpe_vocab_size": (_i, [_vp]),
+    "cthip_bpe_encode": (_i, [_vp, C.c_char_p, _sz, C.POINTER(_i), _sz, C.POINTER(_sz)]),
+    "cthip_bpe_decode": (_i, [_vp, C.POINTER(_i), _sz, C.c_char_p, _sz, C.POINTER(_sz)]),
 }
 
 _lib = None

@@ -190,3 +190,19 @@ def gpt2_generate(model: Transformer, prompt: Sequence[int], max_length: int = 1
         tokens.append(tok)
         out.append(tok)
     return (out, logs) if keep_logits else out
+
+
+def gpt2_generate_text(model: Transformer, tokenizer, text: str, max_length: int = 100, on_device: bool = True,
+                       expected: Optional[str] = None) -> str:
+    """gpt2-generate with its string interface (apps/gpt2/gpt2.lisp:97-113): encode the input, run `max_length`
+    greedy forwards, decode prompt + generated tokens; `expected` asserts the decoded text as the reference's
+    keyword does."""
+    if not isinstance(text, str):
+        raise TypeError("gpt2_generate_text: input must be a string")
+    prompt = tokenizer.encode(text)
+    if not prompt:
+        raise ValueError("gpt2_generate_text: the input encodes to no tokens")
+    decoded = tokenizer.decode(prompt + gpt2_generate(model, prompt, max_length, on_device=on_device))
+    if expected is not None and decoded != expected:
+        raise AssertionError(f"Expected output: {expected}, but got: {decoded}")
+    return decoded

@@ -271,6 +271,18 @@ int cthip_gguf_metadata_string(const void *gguf, int64_t i, int64_t j, const cha
  * for a decoder session; tensors go from the mapping to the device still packed. */
 int cthip_decoder_load_gguf(void *dec, const void *gguf, int arch, int *n_loaded);
 
+/* ---- BPE tokenizer (host code): caten/llm's BPETokenizer (external/llm/bpe.lisp) ----
+ * cthip_bpe_create mirrors make-bpe-tokenizer (bpe.lisp:14-38): `tokens` = the vocabulary, pieces separated by
+ * single spaces, the first piece dropped, the rest numbered from 0; `merges` = one "a b" pair per line, the first
+ * line dropped, ranked by line.  encode (bpe.lisp:85-100): GPT-2 pre-tokenisation, byte alphabet, merges by rank;
+ * a symbol the vocabulary lacks becomes id 0.  With ids == NULL it only counts.  decode (bpe.lisp:102-114): the
+ * inverse; with out == NULL it only measures.  Text is UTF-8 and is not NUL-terminated on output. */
+int cthip_bpe_create(void **bpe, const char *tokens, size_t tokens_len, const char *merges, size_t merges_len);
+int cthip_bpe_destroy(void *bpe);
+int cthip_bpe_vocab_size(const void *bpe);
+int cthip_bpe_encode(void *bpe, const char *text, size_t len, int *ids, size_t cap, size_t *n_ids);
+int cthip_bpe_decode(const void *bpe, const int *ids, size_t n, char *out, size_t cap, size_t *len);
+
 #ifdef __cplusplus
 }
 #endif

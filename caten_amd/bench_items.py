@@ -54,6 +54,19 @@ def main():
         ("LayerNorm (64,1024,768)", lambda: _lib.check(lib.cthip_layernorm(y.ptr, x.ptr, g.ptr, b.ptr, 1e-5, rows, d))),
         ("softmax (64,1024,768)", lambda: _lib.check(lib.cthip_softmax(y.ptr, x.ptr, rows, d))),
     ]
+    # the same softmax as a RENDERED kernel: blueprint -> HIP source (one wavefront per row) -> hipRTC
+    from . import blueprints
+    from .renderer import HipRenderer
+    from .buffer import HipBuffer
+
+    it = blueprints.softmax_rows()
+    rr = HipRenderer()
+    rr.render_kernel(it)
+    rr.compile_kernel([it])
+    # buffers over the same device arrays the hand-written items use
+    bx = HipBuffer(shape=[rows, d], stride=[d, 1], dtype="float32", nrank=2, value=x.ptr)
+    by = HipBuffer(shape=[rows, d], stride=[d, 1], dtype="float32", nrank=2, value=y.ptr)
+    items.append(("softmax (64,1024,768), RENDERED from its blueprint", lambda: it["compiled_object"](None, by, rows, d, bx)))
     for name, fn in items:
         us = _time(lib, fn)
         gbs = nbytes / (us * 1e-6) / 1e9

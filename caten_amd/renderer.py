@@ -32,6 +32,13 @@ fastest so that consecutive lanes touch consecutive addresses, and launched as
 256-thread workgroups with a bounds guard.  Reduction loops stay serial inside a
 thread.  Loops already marked ``scope: global`` are always mapped to threads.
 
+Row reductions (softmax, LayerNorm, RMSNorm, sums over the last axis: a parallel prefix whose body is a
+sequence of scalar statements and loops over one more axis, some of them reductions into scalars that start
+at their operation's identity) get one WAVEFRONT per row instead of one thread: the 64 lanes stride the inner
+axis together, so consecutive lanes read consecutive addresses, every lane keeps a partial, and the partials
+meet in a `__shfl_xor` butterfly after the loop; statements between the loops run redundantly in all lanes
+and only lane 0 performs their global writes.
+
 Spelling follows the CStyle renderer (renderer.lisp:314-411) with two deliberate
 differences for fp32 kernels: literals carry an `f` suffix and the libm calls are
 the float ones, so arithmetic stays in fp32 registers instead of promoting to
@@ -65,6 +72,16 @@ HEADER = """
 #define _nan __builtin_nanf("")
 #define ct_max(a, b) ((a) > (b) ? (a) : (b))
 #define ct_min(a, b) ((a) < (b) ? (a) : (b))
+// reductions over the 64 lanes of a wavefront (every lane gets the result)
+#define CT_WAVE_REDUCE(name, T, OP)                                        \\
+  static __device__ __forceinline__ T name(T v) {                          \\
+    for (int o = 32; o > 0; o >>= 1) { T w = __shfl_xor(v, o, 64); v = OP; } \\
+    return v;                                                              \\
+  }
+CT_WAVE_REDUCE(ct_wave_add_f, float, v + w)
+CT_WAVE_REDUCE(ct_wave_max_f, float, ct_max(v, w))
+CT_WAVE_REDUCE(ct_wave_min_f, float, ct_min(v, w))
+CT_WAVE_REDUCE(ct_wave_mul_f, float, v * w)
 """
 
 BLOCK = 256
@@ -185,6 +202,8 @@ class HipRenderer(Renderer):
         if isinstance(e, str):
             return e.lower() == sym.lower()
         if isinstance(e, dict):
+            if e.get("op") == "AREF" and e.get("index") is None and "space" not in e and e["id"].lower() == sym.lower():
+                return True  # a scalar named by an aref
             if any(HipRenderer._uses(x, sym) for x in e.get("args", [])):
                 return True
             if e.get("index") is not None and HipRenderer._uses(e["index"], sym):
@@ -233,6 +252,68 @@ class HipRenderer(Renderer):
             i += 1
         return depth
 
+    _IDENTITY = {"ADD": ("add", 0.0), "MAX": ("max", float("-inf")), "MIN": ("min", float("inf")), "MUL": ("mul", 1.0)}
+
+    @staticmethod
+    def _const_value(e):
+        if isinstance(e, (int, float, np.integer, np.floating)) and not isinstance(e, bool):
+            return float(e)
+        if isinstance(e, dict) and e.get("op") == "CONST" and isinstance(e.get("value"), (int, float)):
+            return float(e["value"])
+        if isinstance(e, dict) and e.get("op") == "NEG" and len(e.get("args", [])) == 1:
+            v = HipRenderer._const_value(e["args"][0])
+            return None if v is None else -v
+        return None
+
+    def _wave_reductions(self, body: List[dict]):
+        """If `body` (what is left inside the parallel prefix) is a row-reduction pattern, returns
+        {position of an ENDFOR: [(scalar, op)...]} = the scalars to combine across lanes after that loop;
+        otherwise None (the row then stays in one thread)."""
+        depth, init, found = 0, {}, {}
+        loop_red: List = []
+        for pos, n in enumerate(body):
+            t = n["type"]
+            if t == "FOR":
+                depth += 1
+                by = n.get("by", 1)
+                if depth > 1 or n.get("scope") == "global" or not (isinstance(by, (int, np.integer)) and int(by) == 1):
+                    return None
+                loop_red = []
+            elif t == "ENDFOR":
+                depth -= 1
+                if loop_red:
+                    found[pos] = loop_red
+                loop_red = []
+            elif t in ("IF", "ENDIF"):
+                return None
+            elif t == "EXPR":
+                if n.get("dtype", "float32") != "float32" or len(n["writes"]) != 1:
+                    return None
+                w = n["writes"][0]
+                scalar = w.get("index") is None and "space" not in w
+                name = w["id"].lower()
+                if depth == 0:
+                    if scalar:
+                        init[name] = self._const_value(n["expr"])  # None: not a constant
+                    continue
+                if not n.get("reduction"):
+                    if scalar:
+                        return None  # a loop-carried scalar that is not a reduction cannot be split over lanes
+                    continue
+                e = n["expr"]
+                if not (scalar and isinstance(e, dict) and e.get("op", "").upper() in self._IDENTITY and len(e.get("args", [])) == 2):
+                    return None
+                op, ident = self._IDENTITY[e["op"].upper()]
+                args = e["args"]
+                selfref = [isinstance(x, str) and x.lower() == name or isinstance(x, dict) and x.get("op") == "AREF"
+                           and x["id"].lower() == name and x.get("index") is None and "space" not in x for x in args]
+                if sum(selfref) != 1 or self._uses(args[1 - selfref.index(True)], name):
+                    return None
+                if init.get(name) != ident:  # lane partials only combine when each starts at the identity
+                    return None
+                loop_red.append((name, op))
+        return found or None
+
     @staticmethod
     def _is_zero(e) -> bool:
         return isinstance(e, (int, np.integer)) and int(e) == 0 or (isinstance(e, dict) and e.get("op") == "CONST" and e["value"] == 0)
@@ -271,27 +352,44 @@ class HipRenderer(Renderer):
         grid_bounds = []
         indent = 2
         pad = lambda: " " * indent  # noqa: E731
+        wave_red = self._wave_reductions(body[npar:len(body) - npar]) if npar else None
+        item["_rows_per_block"] = BLOCK
         if npar:
             loops = body[:npar]
             bounds = [self._upper_bound(f) for f in loops]
             grid_bounds = bounds
             total = "*".join(f"(long long)({self.render_expr(b, 'int64')})" for b in bounds)
             out.append(f"{pad()}const long long _total = {total};")
-            out.append(f"{pad()}long long _t = (long long)blockIdx.x * {BLOCK} + threadIdx.x;")
+            if wave_red is not None:
+                item["_rows_per_block"] = BLOCK // 64
+                out.append(f"{pad()}long long _t = ((long long)blockIdx.x * {BLOCK} + threadIdx.x) >> 6;  // one wavefront per row")
+                out.append(f"{pad()}const int _lane = threadIdx.x & 63;")
+            else:
+                out.append(f"{pad()}long long _t = (long long)blockIdx.x * {BLOCK} + threadIdx.x;")
             out.append(f"{pad()}if (_t >= _total) return;")
             for f, b in zip(reversed(loops), reversed(bounds)):  # innermost loop varies fastest
                 bs = self.render_expr(b, "int64")
                 out.append(f"{pad()}const int {f['idx'].lower()} = (int)(_t % (long long)({bs})); _t /= (long long)({bs});")
             body = body[npar:len(body) - npar]
-        for n in body:
+        depth = 0
+        for pos, n in enumerate(body):
             t = n["type"]
             if t == "FOR":
-                out.append(f"{pad()}for (int {n['idx'].lower()}={self.render_expr(n['upfrom'], 'int64')}; "
-                           f"{self.render_expr(n['below'], 'int64')}; {n['idx'].lower()}+={self.render_expr(n.get('by', 1), 'int64')}) {{")
+                if wave_red is not None:  # the lanes of the row's wavefront stride this axis together
+                    out.append(f"{pad()}for (int {n['idx'].lower()}=({self.render_expr(n['upfrom'], 'int64')})+_lane; "
+                               f"{self.render_expr(n['below'], 'int64')}; {n['idx'].lower()}+=64) {{")
+                else:
+                    out.append(f"{pad()}for (int {n['idx'].lower()}={self.render_expr(n['upfrom'], 'int64')}; "
+                               f"{self.render_expr(n['below'], 'int64')}; {n['idx'].lower()}+={self.render_expr(n.get('by', 1), 'int64')}) {{")
                 indent += 2
+                depth += 1
             elif t == "ENDFOR":
                 indent -= 2
+                depth -= 1
                 out.append(f"{pad()}}}")
+                if wave_red is not None:
+                    for var, op in wave_red.get(pos, []):
+                        out.append(f"{pad()}{var} = ct_wave_{op}_f({var});")
             elif t == "IF":
                 out.append(f"{pad()}if ({self.render_expr(n['condition'], 'int64')}) {{")
                 indent += 2
@@ -302,7 +400,11 @@ class HipRenderer(Renderer):
                 dt = n.get("dtype", "float32")
                 lhs = ", ".join(self.render_aref(w, dt) for w in n["writes"])
                 decl = f"{CDTYPE[dt]} " if n.get("declare_type") else ""
-                out.append(f"{pad()}{decl}{lhs} = {self.render_expr(n['expr'], dt)};")
+                stmt = f"{decl}{lhs} = {self.render_expr(n['expr'], dt)};"
+                if wave_red is not None and depth == 0 and not n.get("declare_type") and \
+                        any(w["id"].lower() not in self._locals for w in n["writes"]):
+                    stmt = f"if (_lane == 0) {{ {stmt} }}"  # every lane holds the value; one of them stores it
+                out.append(f"{pad()}{stmt}")
             else:
                 raise NotImplementedError(f"Hip-Renderer: unknown blueprint node :{t}")
         out.append("}")
@@ -340,15 +442,18 @@ class HipRenderer(Renderer):
                 continue
             fn = C.c_void_p()
             _lib.check(lib.cthip_get_function(C.byref(fn), mod, it["name"].lower().encode()))
-            it["compiled_object"] = HipProgram(it["name"].lower(), fn, self._args(it), it["_grid_bounds"], self)
+            it["compiled_object"] = HipProgram(it["name"].lower(), fn, self._args(it), it["_grid_bounds"], self,
+                                               it.get("_rows_per_block", BLOCK))
 
 
 class HipProgram:
     """Metal-Program's role (metal.lisp:252-322): holds the function handle, the argument
     dtypes and the grid expression; calling it marshals Caten's argument list and launches."""
 
-    def __init__(self, name: str, fn, defglobals: List[dict], grid_bounds: list, renderer: HipRenderer):
+    def __init__(self, name: str, fn, defglobals: List[dict], grid_bounds: list, renderer: HipRenderer,
+                 rows_per_block: int = BLOCK):
         self.name, self.fn, self.defglobals, self.grid_bounds, self.renderer = name, fn, defglobals, grid_bounds, renderer
+        self.rows_per_block = rows_per_block  # parallel iterations one 256-thread workgroup covers
 
     def _eval(self, e, env: Dict[str, Any]) -> int:
         if isinstance(e, (int, np.integer)):
@@ -392,7 +497,8 @@ class HipProgram:
         total = 1
         for b in self.grid_bounds:
             total *= max(self._eval(b, env), 0)
-        grid = (C.c_uint * 3)((total + BLOCK - 1) // BLOCK if self.grid_bounds else 1, 1, 1)
+        per = self.rows_per_block
+        grid = (C.c_uint * 3)((total + per - 1) // per if self.grid_bounds else 1, 1, 1)
         block = (C.c_uint * 3)(BLOCK if self.grid_bounds else 1, 1, 1)
         argv = (C.c_void_p * len(boxed))(*[C.cast(C.pointer(b), C.c_void_p) for b in boxed])
         _lib.check(_lib.load().cthip_launch(self.fn, grid, block, 0, argv, len(boxed)))

@@ -168,7 +168,9 @@ def test_rendered_rowwise_kernels_match_oracle(oracle):
     rt = ca.HipRuntime()
     r = ca.HipRenderer()
     src = r.render_kernel(item)
-    assert src.count("for (int") == 3 and "blockIdx.x" in src  # rows became threads, the row loops stayed
+    # rows became wavefronts: the three row loops are strided by the 64 lanes, the two reductions end in a butterfly
+    assert src.count("for (int") == 3 and src.count("+=64") == 3 and "blockIdx.x" in src
+    assert "m = ct_wave_max_f(m);" in src and "s = ct_wave_add_f(s);" in src
     r.compile_kernel([item])
     rows, n = 300, 77
     x = np.random.default_rng(1).normal(0, 3, (rows, n)).astype(np.float32)
@@ -181,3 +183,78 @@ def test_rendered_rowwise_kernels_match_oracle(oracle):
     got = transfer_into_array(by).reshape(rows, n)
     want = oracle.softmax(x)
     assert np.max(np.abs(got - want)) < 1e-6
+
+    # LayerNorm as Caten lowers it (one kernel; normalization.lisp:39-58, test-scheduler.lisp:37-45): mean, then
+    # biased variance of the centred row, then the affine output; scalar statements sit between the loops and
+    # a per-row result (the mean) is also stored, which only one lane of the row's wavefront may do
+    sub = lambda a, b: add(a, {"op": "NEG", "args": [b]})  # noqa: E731
+    xi = A("val_x", idx)
+    ln = {"name": "fused_layernorm", "blueprint": [
+        {"type": "DEFINE-GLOBAL", "id": "val_y", "dtype": "float32", "pointer_p": True, "arg_type": "output", "nrank": 2},
+        {"type": "DEFINE-GLOBAL", "id": "val_mean", "dtype": "float32", "pointer_p": True, "arg_type": "output", "nrank": 1},
+        {"type": "DEFINE-GLOBAL", "id": "rows", "dtype": "int64", "pointer_p": False, "arg_type": "shape", "nrank": 0},
+        {"type": "DEFINE-GLOBAL", "id": "n", "dtype": "int64", "pointer_p": False, "arg_type": "shape", "nrank": 0},
+        {"type": "DEFINE-GLOBAL", "id": "val_x", "dtype": "float32", "pointer_p": True, "arg_type": "input", "nrank": 2},
+        {"type": "DEFINE-GLOBAL", "id": "val_g", "dtype": "float32", "pointer_p": True, "arg_type": "input", "nrank": 1},
+        {"type": "DEFINE-GLOBAL", "id": "val_b", "dtype": "float32", "pointer_p": True, "arg_type": "input", "nrank": 1},
+        {"type": "FOR", "idx": "_gid0", "upfrom": 0, "below": lt("_gid0", "rows"), "by": 1},
+        {"type": "EXPR", "writes": [A("s", None)], "expr": 0.0, "declare_type": True, "dtype": "float32"},
+        {"type": "FOR", "idx": "_gid1", "upfrom": 0, "below": lt("_gid1", "n"), "by": 1},
+        {"type": "EXPR", "writes": [A("s", None)], "expr": add("s", xi), "dtype": "float32", "reduction": True},
+        {"type": "ENDFOR", "idx": "_gid1"},
+        {"type": "EXPR", "writes": [A("u", None)], "declare_type": True, "dtype": "float32",
+         "expr": mul("s", {"op": "RECIP", "args": [{"op": "CAST", "dtype": "float32", "args": ["n"]}]})},
+        {"type": "EXPR", "writes": [A("val_mean", "_gid0")], "expr": "u", "dtype": "float32"},
+        {"type": "EXPR", "writes": [A("q", None)], "expr": 0.0, "declare_type": True, "dtype": "float32"},
+        {"type": "FOR", "idx": "_gid1", "upfrom": 0, "below": lt("_gid1", "n"), "by": 1},
+        {"type": "EXPR", "writes": [A("q", None)], "expr": add("q", mul(sub(xi, "u"), sub(xi, "u"))), "dtype": "float32",
+         "reduction": True},
+        {"type": "ENDFOR", "idx": "_gid1"},
+        {"type": "EXPR", "writes": [A("r", None)], "declare_type": True, "dtype": "float32",
+         "expr": {"op": "RECIP", "args": [{"op": "SQRT", "args": [add(mul("q", {"op": "RECIP", "args": [
+             {"op": "CAST", "dtype": "float32", "args": ["n"]}]}), 1e-5)]}]}},
+        {"type": "FOR", "idx": "_gid1", "upfrom": 0, "below": lt("_gid1", "n"), "by": 1},
+        {"type": "EXPR", "writes": [A("val_y", idx)], "dtype": "float32",
+         "expr": add(mul(mul(sub(xi, "u"), "r"), A("val_g", "_gid1")), A("val_b", "_gid1"))},
+        {"type": "ENDFOR", "idx": "_gid1"},
+        {"type": "ENDFOR", "idx": "_gid0"},
+    ]}
+    # a row sum whose accumulator does NOT start at the operation's identity: lane partials would each carry the
+    # offset, so the row must stay in one thread
+    off = {"name": "offset_rowsum", "blueprint": [
+        {"type": "DEFINE-GLOBAL", "id": "val_o", "dtype": "float32", "pointer_p": True, "arg_type": "output", "nrank": 1},
+        {"type": "DEFINE-GLOBAL", "id": "rows", "dtype": "int64", "pointer_p": False, "arg_type": "shape", "nrank": 0},
+        {"type": "DEFINE-GLOBAL", "id": "n", "dtype": "int64", "pointer_p": False, "arg_type": "shape", "nrank": 0},
+        {"type": "DEFINE-GLOBAL", "id": "val_x", "dtype": "float32", "pointer_p": True, "arg_type": "input", "nrank": 2},
+        {"type": "FOR", "idx": "_gid0", "upfrom": 0, "below": lt("_gid0", "rows"), "by": 1},
+        {"type": "EXPR", "writes": [A("s", None)], "expr": 2.5, "declare_type": True, "dtype": "float32"},
+        {"type": "FOR", "idx": "_gid1", "upfrom": 0, "below": lt("_gid1", "n"), "by": 1},
+        {"type": "EXPR", "writes": [A("s", None)], "expr": add("s", xi), "dtype": "float32", "reduction": True},
+        {"type": "ENDFOR", "idx": "_gid1"},
+        {"type": "EXPR", "writes": [A("val_o", "_gid0")], "expr": "s", "dtype": "float32"},
+        {"type": "ENDFOR", "idx": "_gid0"},
+    ]}
+    r2 = ca.HipRenderer()
+    src_ln, src_off = r2.render_kernel(ln), r2.render_kernel(off)
+    assert src_ln.count("+=64") == 3 and "if (_lane == 0) { val_mean[_gid0] = u; }" in src_ln
+    assert "_lane" not in src_off and "+=64" not in src_off
+    r2.compile_kernel([ln, off])
+    for rows, n in ((300, 77), (5, 768), (64, 1)):
+        x = np.random.default_rng(rows).normal(0.5, 3, (rows, n)).astype(np.float32)
+        g = np.random.default_rng(2).normal(1, 0.1, n).astype(np.float32)
+        b = np.random.default_rng(3).normal(0, 0.1, n).astype(np.float32)
+        bufs = {}
+        for name, shape, arr in (("x", [rows, n], x), ("g", [n], g), ("b", [n], b), ("y", [rows, n], None),
+                                 ("mean", [rows], None), ("o", [rows], None)):
+            strides = [n, 1] if len(shape) == 2 else [1]
+            bufs[name] = make_buffer(shape, strides, "float32", device=HipBuffer)
+            open_buffer(rt, bufs[name])
+            if arr is not None:
+                transfer_from_array(rt, bufs[name], arr)
+        ln["compiled_object"](None, bufs["y"], bufs["mean"], rows, n, bufs["x"], bufs["g"], bufs["b"])
+        off["compiled_object"](None, bufs["o"], rows, n, bufs["x"])
+        got = transfer_into_array(bufs["y"]).reshape(rows, n)
+        want = oracle.layernorm(x, g, b)
+        assert np.max(np.abs(got - want)) < 2e-5
+        assert np.allclose(transfer_into_array(bufs["mean"]), x.mean(axis=1), rtol=1e-5, atol=1e-5)
+        assert np.allclose(transfer_into_array(bufs["o"]), 2.5 + x.sum(axis=1, dtype=np.float64), rtol=1e-5, atol=1e-4)

@@ -1,5 +1,5 @@
 """Timings of the single fused items on one MI355X (`python -m caten_amd.bench_items`):
-BASELINE config 1 (`!relu(!matmul A B)`, 1024^3 fp32) and config 2 (LayerNorm -> softmax and
+the benchmark configurations `!relu(!matmul A B)` at 1024^3 fp32 and the row ops (LayerNorm -> softmax and
 GELU(tanh) over fp32 (64,1024,768)), each against the roofline that bounds it.  HIP events on the
 library's stream; inputs resident on the device."""
 from __future__ import annotations

@@ -1,6 +1,6 @@
 """Prefill timing on one MI355X (`python -m caten_amd.bench_prefill`): a 512-token prompt through the
-GPT-2-small shaped Q8_0 model as one batch (BASELINE config 4's prefill leg; `--model llama-1.1b --kind q4_0
---tokens 128` is config 5's): MFMA GEMMs over the
+GPT-2-small shaped Q8_0 model as one batch (the prefill leg of the GPT-2 Q8_0 benchmark configuration; `--model llama-1.1b
+--kind q4_0 --tokens 128` is the Llama-1.1B Q4_0 configuration's): MFMA GEMMs over the
 rows with the weights dequantised while staged.  Reports the wall time of `forward` (synchronous) and
 the linear-layer FLOP rate against the MFMA peak of the operand type."""
 from __future__ import annotations

@@ -175,7 +175,7 @@ def test_llama_generate_matches_oracle(oracle, kind):
 def test_prefill_batch_equals_token_by_token(oracle):
     """A prompt pushed through one forward as a batch (MFMA GEMMs) and the same prompt fed row by row
     through the decode step are the same function: identical greedy tokens, logits and cache rows
-    within the fp32 band; with bf16 MFMA operands within the 1e-2 band the north star allows."""
+    within the fp32 band; with bf16 MFMA operands within the 1e-2 band."""
     import os
     from caten_amd import synth, llm, _lib
     cfg = synth.GPT2_CONFIGS["gpt2-mini"]
@@ -221,7 +221,7 @@ def test_prefill_batch_equals_token_by_token(oracle):
 
 
 def test_gpt2_small_q8_0_full_size_matches_oracle(oracle):
-    """BASELINE config 4 at its real size (12 layers, d 768, vocab 50257, Q8_0): a 16-token prompt and
+    """The GPT-2-small Q8_0 benchmark configuration at its real size (12 layers, d 768, vocab 50257, Q8_0): a 16-token prompt and
     greedy decode against the CPU oracle on the dequantised weights -- identical tokens, logits inside
     rtol 1e-3 / atol 1e-4.  (The oracle needs ~0.1 s per token, so a handful of steps.)"""
     print("case: gpt2 small q8_0 full size", flush=True)
@@ -251,7 +251,7 @@ def test_gpt2_small_q8_0_full_size_matches_oracle(oracle):
 
 
 def test_llama_1b_width_q4_0_matches_oracle(oracle):
-    """BASELINE config 5's layer shape at its real width (d 2048, 32 query / 4 KV heads, SwiGLU 5632, vocab 32000,
+    """The Llama-1.1B Q4_0 benchmark configuration's layer shape at its real width (d 2048, 32 query / 4 KV heads, SwiGLU 5632, vocab 32000,
     Q4_0) with 2 of the 22 layers so the CPU oracle finishes in seconds: a 12-token prompt (batched prefill)
     and greedy decode -- identical tokens, logits inside rtol 1e-3 / atol 1e-4, cache rows equal."""
     print("case: llama 1.1b width q4_0, 2 layers", flush=True)

@@ -1,6 +1,6 @@
 """GPU parity: every hand-written fused item, called through the C ABI, against the CPU oracle.
 
-Bars (BASELINE north star): bit-exact for dequantised weight values and indices/argmax;
+Bars: bit-exact for dequantised weight values and indices/argmax;
 rtol 1e-3 / atol 1e-4 for fp32 arithmetic.
 """
 import numpy as np
@@ -323,7 +323,7 @@ def test_matmul_relu_vs_oracle(ops, oracle, M, N, K):
 
 
 def test_matmul_1024_cubed(ops):
-    # BASELINE config 1: A, B ~ U(-1,1) fp32 (1024,1024); fp64 NumPy is the tie-breaker at this size
+    # the 1024^3 benchmark configuration: A, B ~ U(-1,1) fp32 (1024,1024); fp64 NumPy is the tie-breaker at this size
     rng = np.random.default_rng(0)
     A = rng.uniform(-1, 1, (1024, 1024)).astype(np.float32)
     B = rng.uniform(-1, 1, (1024, 1024)).astype(np.float32)

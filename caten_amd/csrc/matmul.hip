@@ -3,10 +3,10 @@
 // source/nn/linear.lisp:3-17) with the weights still packed (dequantised while they are staged).
 //
 // One 256-thread workgroup (4 wavefronts, 2x2) owns a 64x64 tile of C; each wavefront accumulates a
-// 32x32 sub-tile in 16 accumulator registers with v_mfma_f32_32x32x2_f32 (fp32 operands) or
-// v_mfma_f32_32x32x8_bf16 (operands rounded to bf16, fp32 accumulation).  A and B are staged through
-// LDS in K-steps of 32, k-major so that the MFMA operand reads are conflict-free (lane l reads row
-// k = l/32 + ..., column l%32).  1024x1024 outputs give 256 workgroups = one per compute unit.
+// 32x32 sub-tile in 16 accumulator registers, with v_mfma_f32_32x32x2_f32 (k_gemm_f32, fp32 operands)
+// or v_mfma_f32_32x32x16_bf16 (k_gemm_split / k_gemm_q, operands split into bf16 terms, fp32
+// accumulation).  Operands are staged through two LDS buffers with three K-steps of global loads in
+// flight; 1024x1024 outputs give 256 workgroups = one per compute unit.
 #include <hip/hip_bf16.h>
 
 #include "common.h"
@@ -29,199 +29,15 @@ struct GemmArgs {
   const float *residual; // (M,N), may be null
   int M, N, K;
   int act;
-  // split-K (k_gemm_split only): workgroup (tile, z) covers k in [z * kper, (z + 1) * kper) and writes
+  // split-K: workgroup (tile, z) covers k in [z * kper, (z + 1) * kper) and writes
   // its raw partial tile to ws[z][M][N]; k_splitk_reduce adds the partials in z order and applies the epilogue
   int ksplit, kper;
   float *ws;
-  // tile -> workgroup mapping of k_gemm_split: the tm x tn tile grid is cut into rx x ry = 8 regions of
+  // tile -> workgroup mapping: the tm x tn tile grid is cut into rx x ry = 8 regions of
   // rm x rn tiles, one per XCD (workgroup i is dispatched to XCD i % 8), so that every L2 holds only
   // its region's rows of A and columns of B
   int tm, tn, rx, rm, rn;
 };
-
-__device__ __forceinline__ unsigned short f32_to_bf16_bits(float f) {
-  // round to nearest even
-  unsigned u = __float_as_uint(f);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (unsigned short)(u >> 16);
-}
-
-// element (n, k) of a packed weight matrix as fp32
-__device__ __forceinline__ void wmat_load8(const GemmArgs &a, int n, int k, float *out) {
-  // 8 consecutive k (k % 8 == 0) of row n
-  const int64_t K = a.K;
-  if (a.wtype == CTHIP_Q8_0) {
-    const uint2 q = *(const uint2 *)((const int8_t *)a.wq + n * K + k);
-    const float d = half_bits_to_float(a.wd[n * (K >> 5) + (k >> 5)]);
-    const unsigned dw[2] = {q.x, q.y};
-#pragma unroll
-    for (int t = 0; t < 2; t++) {
-      const int v = (int)dw[t];
-      out[4 * t + 0] = (float)(int)(int8_t)(v)*d;
-      out[4 * t + 1] = (float)(int)(int8_t)(v >> 8) * d;
-      out[4 * t + 2] = (float)(int)(int8_t)(v >> 16) * d;
-      out[4 * t + 3] = (float)(v >> 24) * d;
-    }
-  } else if (a.wtype == CTHIP_Q4_0) {
-    // block b = k/32; elements j<16 are low nibbles of byte j, j>=16 high nibbles of byte j-16
-    const int64_t b = n * (K >> 5) + (k >> 5);
-    const int j0 = k & 31;
-    const uint2 q = *(const uint2 *)((const uint8_t *)a.wq + 16 * b + (j0 & 15));
-    const float d = half_bits_to_float(a.wd[b]);
-    const unsigned dw[2] = {q.x, q.y};
-    const int sh = (j0 < 16) ? 0 : 4;
-#pragma unroll
-    for (int t = 0; t < 8; t++) out[t] = (float)((int)((dw[t >> 2] >> (8 * (t & 3) + sh)) & 0xf) - 8) * d;
-  } else if (a.wtype == CTHIP_F16) {
-    const uint4 h = *(const uint4 *)((const unsigned short *)a.wq + n * K + k);
-    const unsigned dw[4] = {h.x, h.y, h.z, h.w};
-#pragma unroll
-    for (int t = 0; t < 4; t++) {
-      out[2 * t] = half_bits_to_float((unsigned short)(dw[t] & 0xffff));
-      out[2 * t + 1] = half_bits_to_float((unsigned short)(dw[t] >> 16));
-    }
-  } else {
-    const float4 f0 = *(const float4 *)((const float *)a.wq + n * K + k);
-    const float4 f1 = *(const float4 *)((const float *)a.wq + n * K + k + 4);
-    out[0] = f0.x; out[1] = f0.y; out[2] = f0.z; out[3] = f0.w;
-    out[4] = f1.x; out[5] = f1.y; out[6] = f1.z; out[7] = f1.w;
-  }
-}
-
-template <int BMODE, bool BF16>
-__global__ __launch_bounds__(256) void k_gemm(GemmArgs a) {
-  constexpr int BM = 64, BN = 64, BK = 32, PAD = 4;
-  // fp32: As[k][m], Bs[k][n] (k-major).  bf16: As[m][k], Bs[n][k] as 16-bit (k contiguous: a lane's
-  // MFMA operand is 4 consecutive k)
-  __shared__ float As_f[BF16 ? 1 : BK][BF16 ? 1 : BM + PAD];
-  __shared__ float Bs_f[BF16 ? 1 : BK][BF16 ? 1 : BN + PAD];
-  __shared__ unsigned short As_h[BF16 ? BM : 1][BF16 ? BK + PAD : 1];
-  __shared__ unsigned short Bs_h[BF16 ? BN : 1][BF16 ? BK + PAD : 1];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
-  // consecutive workgroups walk down a column of tiles: they share the B panel through L2
-  const int tiles_m = (a.M + BM - 1) / BM;
-  const int m0 = (blockIdx.x % tiles_m) * BM, n0 = (blockIdx.x / tiles_m) * BN;
-  const bool vecA = (a.K % 4 == 0), vecB = (a.N % 4 == 0);
-  v16f acc;
-#pragma unroll
-  for (int r = 0; r < 16; r++) acc[r] = 0.0f;
-
-  // thread -> staging coordinates
-  const int ar = tid >> 2, akc = (tid & 3) * 8;            // A: row ar, 8 consecutive k
-  const int bk = tid >> 3, bnc = (tid & 7) * 8;            // B row-major: row k = bk, 8 consecutive n
-  const int wr = tid >> 2, wkc = (tid & 3) * 8;            // B packed: weight row wr, 8 consecutive k
-
-  auto fetch_a = [&](int k0, float *v) {
-#pragma unroll
-    for (int j = 0; j < 8; j++) v[j] = 0.0f;
-    const int gm = m0 + ar;
-    if (gm < a.M) {
-      const float *src = a.A + (int64_t)gm * a.K + k0 + akc;
-      if (vecA && k0 + akc + 8 <= a.K) {
-        const float4 f0 = *(const float4 *)src, f1 = *(const float4 *)(src + 4);
-        v[0] = f0.x; v[1] = f0.y; v[2] = f0.z; v[3] = f0.w; v[4] = f1.x; v[5] = f1.y; v[6] = f1.z; v[7] = f1.w;
-      } else {
-#pragma unroll
-        for (int j = 0; j < 8; j++)
-          if (k0 + akc + j < a.K) v[j] = src[j];
-      }
-    }
-  };
-  auto fetch_b = [&](int k0, float *v) {
-#pragma unroll
-    for (int j = 0; j < 8; j++) v[j] = 0.0f;
-    if (BMODE == B_ROWMAJOR) {
-      if (k0 + bk < a.K) {
-        const float *src = a.B + (int64_t)(k0 + bk) * a.N + n0 + bnc;
-        if (vecB && n0 + bnc + 8 <= a.N) {
-          const float4 f0 = *(const float4 *)src, f1 = *(const float4 *)(src + 4);
-          v[0] = f0.x; v[1] = f0.y; v[2] = f0.z; v[3] = f0.w; v[4] = f1.x; v[5] = f1.y; v[6] = f1.z; v[7] = f1.w;
-        } else {
-#pragma unroll
-          for (int j = 0; j < 8; j++)
-            if (n0 + bnc + j < a.N) v[j] = src[j];
-        }
-      }
-    } else {
-      // packed weights (K % 32 == 0 for every packed type here): dequantised on the way in
-      if (n0 + wr < a.N && k0 + wkc < a.K) wmat_load8(a, n0 + wr, k0 + wkc, v);
-    }
-  };
-  auto stage = [&](const float *va, const float *vb) {
-    if (BF16) {
-#pragma unroll
-      for (int j = 0; j < 8; j++) As_h[BF16 ? ar : 0][BF16 ? akc + j : 0] = f32_to_bf16_bits(va[j]);
-    } else {
-#pragma unroll
-      for (int j = 0; j < 8; j++) As_f[BF16 ? 0 : akc + j][BF16 ? 0 : ar] = va[j];
-    }
-    if (BMODE == B_ROWMAJOR) {
-      if (BF16) {
-#pragma unroll
-        for (int j = 0; j < 8; j++) Bs_h[BF16 ? bnc + j : 0][BF16 ? bk : 0] = f32_to_bf16_bits(vb[j]);
-      } else {
-#pragma unroll
-        for (int j = 0; j < 8; j++) Bs_f[BF16 ? 0 : bk][BF16 ? 0 : bnc + j] = vb[j];
-      }
-    } else {
-      if (BF16) {
-#pragma unroll
-        for (int j = 0; j < 8; j++) Bs_h[BF16 ? wr : 0][BF16 ? wkc + j : 0] = f32_to_bf16_bits(vb[j]);
-      } else {
-#pragma unroll
-        for (int j = 0; j < 8; j++) Bs_f[BF16 ? 0 : wkc + j][BF16 ? 0 : wr] = vb[j];
-      }
-    }
-  };
-
-  // software pipeline: the next K-step's global loads are in flight while the MFMAs of this one run
-  float va[8], vb[8];
-  fetch_a(0, va);
-  fetch_b(0, vb);
-  for (int k0 = 0; k0 < a.K; k0 += BK) {
-    stage(va, vb);
-    __syncthreads();
-    if (k0 + BK < a.K) {
-      fetch_a(k0 + BK, va);
-      fetch_b(k0 + BK, vb);
-    }
-    if (BF16) {
-      // 32x32x8: lane l holds A[i = l%32][k = 4*(l/32) .. +3] and B[k = 4*(l/32) .. +3][j = l%32]
-#pragma unroll
-      for (int s = 0; s < BK / 8; s++) {
-        const int kk = 8 * s + 4 * (lane >> 5);
-        const v4s av = *(const v4s *)&As_h[BF16 ? 32 * wm + (lane & 31) : 0][BF16 ? kk : 0];
-        const v4s bv = *(const v4s *)&Bs_h[BF16 ? 32 * wn + (lane & 31) : 0][BF16 ? kk : 0];
-        acc = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(av, bv, acc, 0, 0, 0);
-      }
-    } else {
-      // 32x32x2: lane l holds A[i = l%32][k = l/32] and B[k = l/32][j = l%32]
-#pragma unroll
-      for (int s = 0; s < BK / 2; s++) {
-        const int kk = 2 * s + (lane >> 5);
-        const float av = As_f[BF16 ? 0 : kk][BF16 ? 0 : 32 * wm + (lane & 31)];
-        const float bv = Bs_f[BF16 ? 0 : kk][BF16 ? 0 : 32 * wn + (lane & 31)];
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc, 0, 0, 0);
-      }
-    }
-    __syncthreads();
-  }
-  // ---- epilogue: acc[r] is C[row = 8*(r/4) + 4*(l/32) + r%4][col = l%32] of the 32x32 sub-tile ----
-  const int col = n0 + 32 * wn + (lane & 31);
-  if (col < a.N) {
-    const float bias = a.bias ? a.bias[col] : 0.0f;
-#pragma unroll
-    for (int r = 0; r < 16; r++) {
-      const int row = m0 + 32 * wm + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-      if (row < a.M) {
-        float v = apply_act(a.act, acc[r] + bias);
-        if (a.residual) v += a.residual[(int64_t)row * a.N + col];
-        a.C[(int64_t)row * a.N + col] = v;
-      }
-    }
-  }
-}
 
 // ---------------------------------------------------------------------------------------------
 // bf16 MFMA GEMM with fp32 accumulation, operands optionally split in two bf16 terms.
@@ -264,6 +80,23 @@ __device__ __forceinline__ void split4(const float x[4], uint2 *pl) {
   }
 }
 
+// Zeros in device memory: what a request outside an operand reads.  (A load followed by a select would make
+// the request's own thread wait for it at once; a branch around it splits the run of requests.)
+__device__ __align__(16) unsigned g_zeros[8];  // zero-initialised, never written (not const: a load that may come from
+                                                // either here or an operand must stay a global-memory load)
+
+// Four consecutive floats at p without a branch or a dependent instruction: of the four, those past `nvalid`
+// (0..4) are read from g_zeros.  AL: the four are 16-byte aligned and all inside or all outside.  A K-step's
+// requests stay one straight run of loads, so that the waits before their use count the younger requests
+// instead of draining them.
+template <bool AL>
+__device__ __forceinline__ float4 load4(const float *p, int nvalid) {
+  const float *z = (const float *)g_zeros;
+  if (AL) return *(const float4 *)(nvalid > 0 ? p : z);
+  return make_float4(*(nvalid > 0 ? p : z), *(nvalid > 1 ? p + 1 : z), *(nvalid > 2 ? p + 2 : z), *(nvalid > 3 ? p + 3 : z));
+}
+__device__ __forceinline__ int clamp04(int v) { return v < 0 ? 0 : v > 4 ? 4 : v; }
+
 struct ARegs {  // one K-step of A held by a thread: rows ar + 16 i
   float4 v0, v1, v2, v3;
 };
@@ -279,7 +112,7 @@ struct BRegs {  // one K-step of B held by a thread between its request and its 
 // staging and the row-wise A writes over all banks.
 __device__ __forceinline__ int swz(int row) { return (row ^ (row >> 3)) & 7; }
 
-template <int BMODE, int NS>
+template <int BMODE, int NS, bool AL>
 __global__ __launch_bounds__(256) void k_gemm_split(GemmArgs a) {
   constexpr int BM = 64, BN = 64, BK = 64, LDK = BK, NP = (NS == 1) ? 1 : (NS == 3) ? 2 : 3;
   constexpr int NSET = 3;  // register sets = K-steps of global loads in flight
@@ -295,7 +128,6 @@ __global__ __launch_bounds__(256) void k_gemm_split(GemmArgs a) {
   const int M = a.M, N = a.N, ldk = a.K;
   const int kbeg = blockIdx.y * a.kper;      // this workgroup's share of the reduction axis
   const int K = min(a.K, kbeg + a.kper);
-  const bool vecA = (ldk % 4 == 0), vecB = (N % 4 == 0);
   v16f acc;
 #pragma unroll
   for (int r = 0; r < 16; r++) acc[r] = 0.0f;
@@ -307,22 +139,11 @@ __global__ __launch_bounds__(256) void k_gemm_split(GemmArgs a) {
   // B packed (N rows of K): thread -> weight row wr, k = 16 wkc .. +15
   const int wr = tid >> 2, wkc = tid & 3;
 
+  // requests without branches (see load4): outside the operands they read zeros
   auto fetch_a = [&](int k0, ARegs &ra) {  // k0 counts from kbeg
     auto ld = [&](int i) {
       const int row = m0 + ar + 16 * i, k = kbeg + k0 + 4 * akq;
-      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (row < M) {
-        const float *src = a.A + (int64_t)row * ldk + k;
-        if (vecA && k + 4 <= K) {
-          v = *(const float4 *)src;
-        } else {
-          if (k + 0 < K) v.x = src[0];
-          if (k + 1 < K) v.y = src[1];
-          if (k + 2 < K) v.z = src[2];
-          if (k + 3 < K) v.w = src[3];
-        }
-      }
-      return v;
+      return load4<AL>(a.A + (int64_t)row * ldk + k, row < M ? clamp04(K - k) : 0);
     };
     ra.v0 = ld(0);
     ra.v1 = ld(1);
@@ -333,18 +154,7 @@ __global__ __launch_bounds__(256) void k_gemm_split(GemmArgs a) {
     if (BMODE == W_ROWMAJOR) {
       auto ld = [&](int j) {
         const int k = kbeg + k0 + 4 * bkq + j, n = n0 + 4 * bnq;
-        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (k < K) {
-          const float *src = a.B + (int64_t)k * N + n;
-          if (vecB && n + 4 <= N) {
-            v = *(const float4 *)src;
-          } else {
-            if (n + 0 < N) v.x = src[0];
-            if (n + 1 < N) v.y = src[1];
-            if (n + 2 < N) v.z = src[2];
-            if (n + 3 < N) v.w = src[3];
-          }
-        }
+        const float4 v = load4<AL>(a.B + (int64_t)k * N + n, k < K ? clamp04(N - n) : 0);
         return make_uint4(__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z), __float_as_uint(v.w));
       };
       // constant indices only: the sets must stay in registers
@@ -353,26 +163,21 @@ __global__ __launch_bounds__(256) void k_gemm_split(GemmArgs a) {
       rb.v[BRegs<BMODE>::NV > 2 ? 2 : 0] = ld(2);
       rb.v[BRegs<BMODE>::NV > 3 ? 3 : 0] = ld(3);
     } else {
-      // packed rows: K is a multiple of 32, so a 16-wide k chunk is inside the row or past its end
+      // packed rows: K is a multiple of 16 here, so a 16-wide k chunk is inside the row or past its end
       const int n = n0 + wr, k = kbeg + k0 + 16 * wkc;
       const bool ok = n < N && k < K;
-      rb.v[0] = make_uint4(0u, 0u, 0u, 0u);
-      if (BRegs<BMODE>::NV > 1) rb.v[BRegs<BMODE>::NV > 1 ? 1 : 0] = make_uint4(0u, 0u, 0u, 0u);
-      if (BRegs<BMODE>::NV > 2) {
-        rb.v[BRegs<BMODE>::NV > 2 ? 2 : 0] = make_uint4(0u, 0u, 0u, 0u);
-        rb.v[BRegs<BMODE>::NV > 3 ? 3 : 0] = make_uint4(0u, 0u, 0u, 0u);
-      }
-      if (ok) {
-        const int64_t e = (int64_t)n * ldk + k;  // element index of the chunk
-        if (BMODE == W_F32) {
-          rb.v[0] = *(const uint4 *)((const float *)a.wq + e);
-          rb.v[BRegs<BMODE>::NV > 1 ? 1 : 0] = *(const uint4 *)((const float *)a.wq + e + 4);
-          rb.v[BRegs<BMODE>::NV > 2 ? 2 : 0] = *(const uint4 *)((const float *)a.wq + e + 8);
-          rb.v[BRegs<BMODE>::NV > 3 ? 3 : 0] = *(const uint4 *)((const float *)a.wq + e + 12);
-        } else if (BMODE == W_F16) {
-          rb.v[0] = *(const uint4 *)((const unsigned short *)a.wq + e);
-          rb.v[BRegs<BMODE>::NV > 1 ? 1 : 0] = *(const uint4 *)((const unsigned short *)a.wq + e + 8);
-        }
+      const int64_t e = (int64_t)n * ldk + k;  // element index of the chunk
+      if (BMODE == W_F32) {
+        const uint4 *src = ok ? (const uint4 *)((const float *)a.wq + e) : (const uint4 *)g_zeros;
+        const int st = ok ? 1 : 0;  // the zeros are 32 bytes long
+        rb.v[0] = src[0];
+        rb.v[BRegs<BMODE>::NV > 1 ? 1 : 0] = src[st];
+        rb.v[BRegs<BMODE>::NV > 2 ? 2 : 0] = src[2 * st];
+        rb.v[BRegs<BMODE>::NV > 3 ? 3 : 0] = src[3 * st];
+      } else if (BMODE == W_F16) {
+        const uint4 *src = ok ? (const uint4 *)((const unsigned short *)a.wq + e) : (const uint4 *)g_zeros;
+        rb.v[0] = src[0];
+        rb.v[BRegs<BMODE>::NV > 1 ? 1 : 0] = src[1];
       }
     }
   };
@@ -462,45 +267,38 @@ __global__ __launch_bounds__(256) void k_gemm_split(GemmArgs a) {
   ARegs ra0, ra1, ra2;  // separate objects with named members: every set stays in registers
   BRegs<BMODE> rb0, rb1, rb2;
   const int nsteps = K > kbeg ? (K - kbeg + BK - 1) / BK : 0;
-  if (nsteps > 0) {
-    fetch_a(0, ra0);
-    fetch_b(0, rb0);
-  }
-  if (nsteps > 1) {
-    fetch_a(BK, ra1);
-    fetch_b(BK, rb1);
-  }
-  if (nsteps > 2) {
-    fetch_a(2 * BK, ra2);
-    fetch_b(2 * BK, rb2);
-  }
-  if (nsteps > 0) {
-    stage_a(ra0, 0);
-    stage_b(rb0, 0);
-  }
-  if (nsteps > 3) {
-    fetch_a(3 * BK, ra0);
-    fetch_b(3 * BK, rb0);
-  }
-  __syncthreads();
-  // step i: LDS buffer i%2 holds it; register set (i+1) % NSET holds step i+1, requested NSET steps ago
+  // step i: LDS buffer i%2 holds it; register set (i+1) % NSET holds step i+1, requested NSET steps ago.
+  // No conditions inside a step (past the last one the requests read zeros and stage them) and no exit
+  // inside the loop: the waits before a set is staged then count on a known number of younger requests.
   auto step = [&](int i, ARegs &ran, BRegs<BMODE> &rbn) {
-    if (i + 1 < nsteps) {
-      stage_a(ran, (i + 1) & 1);
-      stage_b(rbn, (i + 1) & 1);
-    }
-    if (i + 1 + NSET < nsteps) {
-      fetch_a((i + 1 + NSET) * BK, ran);
-      fetch_b((i + 1 + NSET) * BK, rbn);
-    }
+    stage_a(ran, (i + 1) & 1);
+    stage_b(rbn, (i + 1) & 1);
+    fetch_a((i + 1 + NSET) * BK, ran);
+    fetch_b((i + 1 + NSET) * BK, rbn);
     mma(i & 1);
     __syncthreads();
   };
   static_assert(NSET == 3, "the loop below is unrolled by hand over the register sets");
-  for (int i = 0; i < nsteps; i += NSET) {
-    step(i, ra1, rb1);
+  if (nsteps > 0) {  // K = 0 comes without operands
+    fetch_a(0, ra0);
+    fetch_b(0, rb0);
+    fetch_a(BK, ra1);
+    fetch_b(BK, rb1);
+    fetch_a(2 * BK, ra2);
+    fetch_b(2 * BK, rb2);
+    stage_a(ra0, 0);
+    stage_b(rb0, 0);
+    fetch_a(3 * BK, ra0);
+    fetch_b(3 * BK, rb0);
+    __syncthreads();
+    int i = 0;
+    for (; i + NSET <= nsteps; i += NSET) {
+      step(i, ra1, rb1);
+      step(i + 1, ra2, rb2);
+      step(i + 2, ra0, rb0);
+    }
+    if (i < nsteps) step(i, ra1, rb1);
     if (i + 1 < nsteps) step(i + 1, ra2, rb2);
-    if (i + 2 < nsteps) step(i + 2, ra0, rb0);
   }
   // ---- epilogue: acc[r] is C[row = 8*(r/4) + 4*(l/32) + r%4][col = l%32] of the 32x32 sub-tile ----
   const int col = n0 + 32 * wn + (lane & 31);
@@ -571,7 +369,6 @@ __global__ __launch_bounds__(256) void k_gemm_q(GemmArgs a) {
   const int M = a.M, N = a.N, ldk = a.K;
   const int kbeg = blockIdx.y * a.kper;
   const int K = min(a.K, kbeg + a.kper);
-  const bool vecA = (ldk % 4 == 0);
   v16f acc[MB];
 #pragma unroll
   for (int b = 0; b < MB; b++)
@@ -580,40 +377,23 @@ __global__ __launch_bounds__(256) void k_gemm_q(GemmArgs a) {
 
   const int ar = tid >> 4, akq = tid & 15;  // A: rows ar + 16 i, k = 4 akq .. +3
   const int wr = tid >> 2, wkc = tid & 3;   // B: weight row wr, k = 16 wkc .. +15
-  const int sr = tid >> 1, sb = tid & 1;    // scales (tid < 128): row sr, quant block sb of the step
+  const int sr = (tid & 127) >> 1, sb = tid & 1;  // scales: row sr, quant block sb of the step (threads < 128 stage them)
   const int blocks_per_row = ldk >> 5;
 
+  // requests without branches (see load4; quantised rows are a multiple of 32 wide, so always aligned)
   auto fetch = [&](int k0, ARegsQ<MB> &ra, BRegsQ &rb) {  // k0 counts from kbeg
 #pragma unroll
     for (int i = 0; i < 4 * MB; i++) {
       const int row = m0 + ar + 16 * i, k = kbeg + k0 + 4 * akq;
-      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (row < M) {
-        const float *src = a.A + (int64_t)row * ldk + k;
-        if (vecA && k + 4 <= K) {
-          v = *(const float4 *)src;
-        } else {
-          if (k + 0 < K) v.x = src[0];
-          if (k + 1 < K) v.y = src[1];
-          if (k + 2 < K) v.z = src[2];
-          if (k + 3 < K) v.w = src[3];
-        }
-      }
-      ra.v[i] = v;
+      ra.v[i] = load4<true>(a.A + (int64_t)row * ldk + k, row < M ? clamp04(K - k) : 0);
     }
-    // K is a multiple of 32: a 16-wide chunk / a quant block is inside the row or past this share's end
+    // a 16-wide chunk / a quant block is inside the row or past this share's end
     const int n = n0 + wr, k = kbeg + k0 + 16 * wkc;
-    rb.v = make_uint4(0u, 0u, 0u, 0u);
-    if (n < N && k < K) {
-      const int64_t e = (int64_t)n * ldk + k;
-      if (WT == W_Q8) rb.v = *(const uint4 *)((const int8_t *)a.wq + e);
-      else rb.v = *(const uint4 *)((const uint8_t *)a.wq + ((e >> 5) << 4));
-    }
-    rb.d = 0;
-    if (tid < 128) {
-      const int ns = n0 + sr, ks = kbeg + k0 + 32 * sb;
-      if (ns < N && ks < K) rb.d = a.wd[(int64_t)ns * blocks_per_row + (ks >> 5)];
-    }
+    const int64_t e = (int64_t)n * ldk + k;
+    const uint8_t *q = (const uint8_t *)a.wq + (WT == W_Q8 ? e : ((e >> 5) << 4));
+    rb.v = *((n < N && k < K) ? (const uint4 *)q : (const uint4 *)g_zeros);
+    const int ns = n0 + sr, ks = kbeg + k0 + 32 * sb;  // threads 128.. ask for the same scales again: same cache lines
+    rb.d = *((ns < N && ks < K) ? a.wd + (int64_t)ns * blocks_per_row + (ks >> 5) : (const unsigned short *)g_zeros);
   };
   auto stage = [&](const ARegsQ<MB> &ra, const BRegsQ &rb, int buf) {
 #pragma unroll
@@ -682,22 +462,28 @@ __global__ __launch_bounds__(256) void k_gemm_q(GemmArgs a) {
   ARegsQ<MB> ra0, ra1, ra2;
   BRegsQ rb0, rb1, rb2;
   const int nsteps = K > kbeg ? (K - kbeg + BK - 1) / BK : 0;
-  if (nsteps > 0) fetch(0, ra0, rb0);
-  if (nsteps > 1) fetch(BK, ra1, rb1);
-  if (nsteps > 2) fetch(2 * BK, ra2, rb2);
-  if (nsteps > 0) stage(ra0, rb0, 0);
-  if (nsteps > 3) fetch(3 * BK, ra0, rb0);
-  __syncthreads();
+  // no conditions inside a step and no exit inside the loop, as in k_gemm_split
   auto step = [&](int i, ARegsQ<MB> &ran, BRegsQ &rbn) {
-    if (i + 1 < nsteps) stage(ran, rbn, (i + 1) & 1);
-    if (i + 4 < nsteps) fetch((i + 4) * BK, ran, rbn);
+    stage(ran, rbn, (i + 1) & 1);
+    fetch((i + 4) * BK, ran, rbn);
     mma(i & 1);
     __syncthreads();
   };
-  for (int i = 0; i < nsteps; i += 3) {
-    step(i, ra1, rb1);
+  if (nsteps > 0) {
+    fetch(0, ra0, rb0);
+    fetch(BK, ra1, rb1);
+    fetch(2 * BK, ra2, rb2);
+    stage(ra0, rb0, 0);
+    fetch(3 * BK, ra0, rb0);
+    __syncthreads();
+    int i = 0;
+    for (; i + 3 <= nsteps; i += 3) {
+      step(i, ra1, rb1);
+      step(i + 1, ra2, rb2);
+      step(i + 2, ra0, rb0);
+    }
+    if (i < nsteps) step(i, ra1, rb1);
     if (i + 1 < nsteps) step(i + 1, ra2, rb2);
-    if (i + 2 < nsteps) step(i + 2, ra0, rb0);
   }
   // ---- epilogue: acc[b][r] is C[row = 8*(r/4) + 4*(l/32) + r%4][col = l%32] of the wavefront's block b ----
   const int col = n0 + 32 * wn + (lane & 31);
@@ -717,6 +503,212 @@ __global__ __launch_bounds__(256) void k_gemm_q(GemmArgs a) {
         }
         dst[(int64_t)row * N + col] = v;
       }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// fp32-operand MFMA GEMM (v_mfma_f32_32x32x2_f32): the products are fp32 products, only the summation
+// order differs from a scalar loop.  Same skeleton as k_gemm_split -- 64x64 tile per 256-thread workgroup,
+// 2x2 wavefronts, two LDS buffers, three register sets of global loads in flight, one barrier per step,
+// XCD regions, split-K -- with K-steps of 32 and the operands kept as fp32 in LDS, k-major ([k][m], [k][n]):
+// lane l of a wavefront reads A[row l%32][k = 2s + l/32] and B[k = 2s + l/32][col l%32], i.e. 32
+// consecutive floats per half-wavefront.  A (and packed weights) arrive k-contiguous and are transposed by
+// the staging writes; a (K,N) row-major B is copied as it is.
+struct FRegsA {
+  float4 v0, v1;  // units tid and tid + 256 of the 64 x 8 float4 of a K-step
+};
+struct FRegsB {
+  uint4 r0, r1;      // row-major B: two float4; packed weights: the raw bytes of 8 consecutive k of one row
+  unsigned short d;  // block scale (quantised weights)
+};
+
+template <int BMODE, bool AL>
+__global__ __launch_bounds__(256) void k_gemm_f32(GemmArgs a) {
+  // row pitches: odd where the staging writes are transposing scalar writes (k varies fastest over the lanes,
+  // so k * pitch has to spread over the banks), a multiple of 4 where they are float4 rows
+  constexpr int BM = 64, BN = 64, BK = 32, LDA = BM + 1, LDB = BMODE == B_ROWMAJOR ? BN + 4 : BN + 1;
+  __shared__ __align__(16) float As[2][BK][LDA];
+  __shared__ __align__(16) float Bs[2][BK][LDB];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+  if (local >= a.rm * a.rn) return;
+  const int mi = (xcd % a.rx) * a.rm + local % a.rm, ni = (xcd / a.rx) * a.rn + local / a.rm;
+  if (mi >= a.tm || ni >= a.tn) return;
+  const int m0 = mi * BM, n0 = ni * BN;
+  const int M = a.M, N = a.N, ldk = a.K;
+  const int kbeg = blockIdx.y * a.kper;
+  const int K = min(a.K, kbeg + a.kper);
+  v16f acc;
+#pragma unroll
+  for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+
+  auto load_a = [&](int u, int k0) {  // unit u: row u / 8, k = 4 (u % 8) .. +3
+    const int row = m0 + (u >> 3), k = kbeg + k0 + 4 * (u & 7);
+    return load4<AL>(a.A + (int64_t)row * ldk + k, row < M ? clamp04(K - k) : 0);
+  };
+  auto load_b_rows = [&](int u, int k0) {  // row-major B, unit u: k = u / 16, n = 4 (u % 16) .. +3
+    const int k = kbeg + k0 + (u >> 4), n = n0 + 4 * (u & 15);
+    const float4 v = load4<AL>(a.B + (int64_t)k * N + n, k < K ? clamp04(N - n) : 0);
+    return make_uint4(__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z), __float_as_uint(v.w));
+  };
+  auto fetch = [&](int k0, FRegsA &ra, FRegsB &rb) {
+    ra.v0 = load_a(tid, k0);
+    ra.v1 = load_a(tid + 256, k0);
+    rb.r0 = rb.r1 = make_uint4(0u, 0u, 0u, 0u);
+    rb.d = 0;
+    if (BMODE == B_ROWMAJOR) {
+      rb.r0 = load_b_rows(tid, k0);
+      rb.r1 = load_b_rows(tid + 256, k0);
+    } else {
+      // packed weights: weight row tid / 4, k = 8 (tid % 4) .. +7 of the step.  AL: rows are a multiple of 8
+      // wide (quantised rows always are), so the 8 are inside the row or past its end
+      const int n = n0 + (tid >> 2), k = kbeg + k0 + 8 * (tid & 3);
+      const bool in = n < N && k < K;
+      const int64_t e = (int64_t)n * ldk + k;
+      const void *z = g_zeros;
+      if (!AL) {
+        // fp32 / fp16 rows of any width: element loads, zeros past the end of the row
+        unsigned x[8];
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+          const bool ok = in && k + t < K;
+          x[t] = a.wtype == CTHIP_F32 ? *(ok ? (const unsigned *)a.wq + e + t : (const unsigned *)z)
+                                      : *(ok ? (const unsigned short *)a.wq + e + t : (const unsigned short *)z);
+        }
+        if (a.wtype == CTHIP_F32) {
+          rb.r0 = make_uint4(x[0], x[1], x[2], x[3]);
+          rb.r1 = make_uint4(x[4], x[5], x[6], x[7]);
+        } else {
+          rb.r0 = make_uint4(x[0] | (x[1] << 16), x[2] | (x[3] << 16), x[4] | (x[5] << 16), x[6] | (x[7] << 16));
+        }
+      } else if (a.wtype == CTHIP_F32) {
+        const uint4 *src = in ? (const uint4 *)((const float *)a.wq + e) : (const uint4 *)z;
+        rb.r0 = src[0];
+        rb.r1 = src[1];
+      } else if (a.wtype == CTHIP_F16) {
+        rb.r0 = *(in ? (const uint4 *)((const unsigned short *)a.wq + e) : (const uint4 *)z);
+      } else {
+        // Q8_0: 8 int8.  Q4_0: elements j < 16 of a block are the low nibbles of its bytes j, j >= 16 the high
+        // nibbles of bytes j - 16 -- 8 bytes from (k % 16) on either way
+        const uint8_t *q = (const uint8_t *)a.wq + (a.wtype == CTHIP_Q8_0 ? e : ((e >> 5) << 4) + (k & 15));
+        const uint2 v = *(in ? (const uint2 *)q : (const uint2 *)z);
+        rb.r0.x = v.x;
+        rb.r0.y = v.y;
+        rb.d = *(in ? a.wd + (e >> 5) : (const unsigned short *)z);
+      }
+    }
+  };
+  auto put_a = [&](int u, const float4 v, int buf) {
+    const int row = u >> 3, k = 4 * (u & 7);
+    As[buf][k + 0][row] = v.x;
+    As[buf][k + 1][row] = v.y;
+    As[buf][k + 2][row] = v.z;
+    As[buf][k + 3][row] = v.w;
+  };
+  auto stage = [&](const FRegsA &ra, const FRegsB &rb, int buf) {
+    put_a(tid, ra.v0, buf);
+    put_a(tid + 256, ra.v1, buf);
+    if (BMODE == B_ROWMAJOR) {
+      *(uint4 *)&Bs[buf][tid >> 4][4 * (tid & 15)] = rb.r0;
+      *(uint4 *)&Bs[buf][(tid + 256) >> 4][4 * (tid & 15)] = rb.r1;
+    } else {
+      float w0, w1, w2, w3, w4, w5, w6, w7;
+      if (a.wtype == CTHIP_F32) {
+        w0 = __uint_as_float(rb.r0.x), w1 = __uint_as_float(rb.r0.y), w2 = __uint_as_float(rb.r0.z), w3 = __uint_as_float(rb.r0.w);
+        w4 = __uint_as_float(rb.r1.x), w5 = __uint_as_float(rb.r1.y), w6 = __uint_as_float(rb.r1.z), w7 = __uint_as_float(rb.r1.w);
+      } else if (a.wtype == CTHIP_F16) {
+        w0 = half_bits_to_float((unsigned short)(rb.r0.x & 0xffff)), w1 = half_bits_to_float((unsigned short)(rb.r0.x >> 16));
+        w2 = half_bits_to_float((unsigned short)(rb.r0.y & 0xffff)), w3 = half_bits_to_float((unsigned short)(rb.r0.y >> 16));
+        w4 = half_bits_to_float((unsigned short)(rb.r0.z & 0xffff)), w5 = half_bits_to_float((unsigned short)(rb.r0.z >> 16));
+        w6 = half_bits_to_float((unsigned short)(rb.r0.w & 0xffff)), w7 = half_bits_to_float((unsigned short)(rb.r0.w >> 16));
+      } else if (a.wtype == CTHIP_Q8_0) {
+        const float d = half_bits_to_float(rb.d);
+        const int v0 = (int)rb.r0.x, v1 = (int)rb.r0.y;
+        w0 = (float)(int)(int8_t)(v0)*d, w1 = (float)(int)(int8_t)(v0 >> 8) * d;
+        w2 = (float)(int)(int8_t)(v0 >> 16) * d, w3 = (float)(v0 >> 24) * d;
+        w4 = (float)(int)(int8_t)(v1)*d, w5 = (float)(int)(int8_t)(v1 >> 8) * d;
+        w6 = (float)(int)(int8_t)(v1 >> 16) * d, w7 = (float)(v1 >> 24) * d;
+      } else {
+        const float d = half_bits_to_float(rb.d);
+        // k = 8 (tid % 4) within the block: from 16 on the elements are the high nibbles
+        const unsigned sh = ((tid & 3) >= 2) ? 4u : 0u;
+        const unsigned v0 = rb.r0.x >> sh, v1 = rb.r0.y >> sh;
+        w0 = (float)((int)(v0 & 0xf) - 8) * d, w1 = (float)((int)((v0 >> 8) & 0xf) - 8) * d;
+        w2 = (float)((int)((v0 >> 16) & 0xf) - 8) * d, w3 = (float)((int)((v0 >> 24) & 0xf) - 8) * d;
+        w4 = (float)((int)(v1 & 0xf) - 8) * d, w5 = (float)((int)((v1 >> 8) & 0xf) - 8) * d;
+        w6 = (float)((int)((v1 >> 16) & 0xf) - 8) * d, w7 = (float)((int)((v1 >> 24) & 0xf) - 8) * d;
+      }
+      const int n = tid >> 2, k = 8 * (tid & 3);
+      Bs[buf][k + 0][n] = w0, Bs[buf][k + 1][n] = w1, Bs[buf][k + 2][n] = w2, Bs[buf][k + 3][n] = w3;
+      Bs[buf][k + 4][n] = w4, Bs[buf][k + 5][n] = w5, Bs[buf][k + 6][n] = w6, Bs[buf][k + 7][n] = w7;
+    }
+  };
+  // operands of matrix instructions 2j, 2j + 1 of a step (lane l: k = 4j + l/32 and 4j + 2 + l/32)
+  auto rd = [&](int buf, int j, float (&av)[2], float (&bv)[2]) {
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+      const int kk = 4 * j + 2 * t + (lane >> 5);
+      av[t] = As[buf][kk][32 * wm + (lane & 31)];
+      bv[t] = Bs[buf][kk][32 * wn + (lane & 31)];
+    }
+  };
+
+  FRegsA ra0, ra1, ra2;
+  FRegsB rb0, rb1, rb2;
+  const int nsteps = K > kbeg ? (K - kbeg + BK - 1) / BK : 0;
+  // no conditions inside a step: past the last step the requests read zeros and stage them
+  // A wavefront issues in order and a matrix instruction holds the pipe for 64 cycles.  The step is laid out by
+  // hand between scheduling fences: the operand reads run one pair of matrix instructions ahead of their use,
+  // the next step's staging and the requests four steps ahead sit between pairs.
+  auto step = [&](int i, FRegsA &ran, FRegsB &rbn) {
+    const int buf = i & 1;
+    float av[2][2], bv[2][2];
+    rd(buf, 0, av[0], bv[0]);
+#pragma unroll
+    for (int j = 0; j < BK / 4; j++) {
+      if (j + 1 < BK / 4) rd(buf, j + 1, av[(j + 1) & 1], bv[(j + 1) & 1]);
+      if (j == 1) stage(ran, rbn, buf ^ 1);
+      if (j == 4) fetch((i + 4) * BK, ran, rbn);
+      __builtin_amdgcn_sched_barrier(0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[j & 1][0], bv[j & 1][0], acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[j & 1][1], bv[j & 1][1], acc, 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    __syncthreads();
+  };
+  if (nsteps > 0) {  // K = 0 comes without operands
+    fetch(0, ra0, rb0);
+    fetch(BK, ra1, rb1);
+    fetch(2 * BK, ra2, rb2);
+    stage(ra0, rb0, 0);
+    fetch(3 * BK, ra0, rb0);
+    __syncthreads();
+    int i = 0;
+    for (; i + 3 <= nsteps; i += 3) {  // no exit inside: the waits at the top count on a known number of requests
+      step(i, ra1, rb1);
+      step(i + 1, ra2, rb2);
+      step(i + 2, ra0, rb0);
+    }
+    if (i < nsteps) step(i, ra1, rb1);
+    if (i + 1 < nsteps) step(i + 1, ra2, rb2);
+  }
+  // ---- epilogue: acc[r] is C[row = 8*(r/4) + 4*(l/32) + r%4][col = l%32] of the 32x32 sub-tile ----
+  const int col = n0 + 32 * wn + (lane & 31);
+  if (col >= N) return;
+  const float bias = (a.ksplit > 1 || !a.bias) ? 0.0f : a.bias[col];
+  float *dst = a.ksplit > 1 ? a.ws + (int64_t)blockIdx.y * M * N : a.C;
+#pragma unroll
+  for (int r = 0; r < 16; r++) {
+    const int row = m0 + 32 * wm + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+    if (row < M) {
+      float v = acc[r];
+      if (a.ksplit <= 1) {
+        v = apply_act(a.act, v + bias);
+        if (a.residual) v += a.residual[(int64_t)row * N + col];
+      }
+      dst[(int64_t)row * N + col] = v;
     }
   }
 }
@@ -741,6 +733,9 @@ int launch_gemm(GemmArgs a, int bmode, int precision) {
   if (a.M == 0 || a.N == 0) return 0;
   hipStream_t st = state().stream;
   const int cus = state().compute_units;
+  // the bf16 kernels read packed rows in 16-element chunks: fp32 / fp16 weight rows of another width go to
+  // the fp32 kernel, which is at least as accurate as any of the modes
+  if (bmode == B_WMAT && (a.K & 15)) precision = GEMM_FP32;
   const bool quant = precision != GEMM_FP32 && bmode == B_WMAT && (a.wtype == CTHIP_Q8_0 || a.wtype == CTHIP_Q4_0);
   // 64 output rows per workgroup.  (128-row tiles -- two accumulator blocks per wavefront, half the weight-side
   // staging -- measured slower on every prefill shape: one workgroup per compute unit and 32 KB of A per step.)
@@ -751,7 +746,7 @@ int launch_gemm(GemmArgs a, int bmode, int precision) {
   a.ksplit = 1;
   a.kper = a.K > 0 ? a.K : 1;
   a.ws = nullptr;
-  if (precision != GEMM_FP32) {
+  {
     // one region of tiles per XCD: the split with the fewest tiles per XCD, then the least operand bytes per L2
     a.tm = (a.M + bm - 1) / bm;
     a.tn = (a.N + 63) / 64;
@@ -769,9 +764,10 @@ int launch_gemm(GemmArgs a, int bmode, int precision) {
     }
     grid.x = 8u * (unsigned)a.rm * (unsigned)a.rn;
     // too few tiles to occupy the chip and a long reduction axis: split K over several workgroups per tile
-    const int nsteps = (a.K + 63) / 64;
+    const int nsteps = (a.K + 63) / 64;  // K-steps of 64 (two of the fp32 kernel's)
     int ks = (int)((cus * 3 / 2) / tiles);
     if (ks > nsteps / 6) ks = nsteps / 6;
+    if (const char *e = getenv("CTHIP_KS")) ks = atoi(e);  // TEMP
     if (ks > 16) ks = 16;
     if (ks > 1) {
       const int steps_per = (nsteps + ks - 1) / ks;
@@ -787,8 +783,15 @@ int launch_gemm(GemmArgs a, int bmode, int precision) {
     }
   }
   if (precision == GEMM_FP32) {
-    if (bmode == B_ROWMAJOR) hipLaunchKernelGGL((k_gemm<B_ROWMAJOR, false>), grid, block, 0, st, a);
-    else hipLaunchKernelGGL((k_gemm<B_WMAT, false>), grid, block, 0, st, a);
+    // aligned: every 4 (8 for packed weights) consecutive operand elements a thread asks for are one aligned vector
+    const bool al = bmode == B_ROWMAJOR ? (a.K % 4 == 0 && a.N % 4 == 0) : (a.K % 8 == 0);
+    if (bmode == B_ROWMAJOR) {
+      if (al) hipLaunchKernelGGL((k_gemm_f32<B_ROWMAJOR, true>), grid, block, 0, st, a);
+      else hipLaunchKernelGGL((k_gemm_f32<B_ROWMAJOR, false>), grid, block, 0, st, a);
+    } else {
+      if (al) hipLaunchKernelGGL((k_gemm_f32<B_WMAT, true>), grid, block, 0, st, a);
+      else hipLaunchKernelGGL((k_gemm_f32<B_WMAT, false>), grid, block, 0, st, a);
+    }
   } else if (quant) {
     const int npa = precision == GEMM_BF16X6 ? 3 : precision == GEMM_BF16X3 ? 2 : 1;
 #define QG(WT, NPA, MB) hipLaunchKernelGGL((k_gemm_q<WT, NPA, MB>), grid, block, 0, st, a)
@@ -806,17 +809,26 @@ int launch_gemm(GemmArgs a, int bmode, int precision) {
   } else {
     int wm = W_ROWMAJOR;
     if (bmode == B_WMAT) wm = a.wtype == CTHIP_F16 ? W_F16 : W_F32;
-#define SPLIT(MODE)                                                                                          \
-  case MODE:                                                                                                 \
-    if (precision == GEMM_BF16X6) hipLaunchKernelGGL((k_gemm_split<MODE, 6>), grid, block, 0, st, a);        \
-    else if (precision == GEMM_BF16X3) hipLaunchKernelGGL((k_gemm_split<MODE, 3>), grid, block, 0, st, a);   \
-    else hipLaunchKernelGGL((k_gemm_split<MODE, 1>), grid, block, 0, st, a);                                 \
+#define SPLIT3(MODE, AL)                                                                                      \
+  if (precision == GEMM_BF16X6) hipLaunchKernelGGL((k_gemm_split<MODE, 6, AL>), grid, block, 0, st, a);      \
+  else if (precision == GEMM_BF16X3) hipLaunchKernelGGL((k_gemm_split<MODE, 3, AL>), grid, block, 0, st, a); \
+  else hipLaunchKernelGGL((k_gemm_split<MODE, 1, AL>), grid, block, 0, st, a)
+#define SPLIT(MODE)      \
+  case MODE:             \
+    if (al) {            \
+      SPLIT3(MODE, true); \
+    } else {             \
+      SPLIT3(MODE, false); \
+    }                    \
     break
+    // aligned: every 4 consecutive floats a thread asks for are one 16-byte vector, inside or outside as a whole
+    const bool al = a.K % 4 == 0 && (bmode != B_ROWMAJOR || a.N % 4 == 0);
     switch (wm) {
       SPLIT(W_ROWMAJOR);
       SPLIT(W_F32);
       SPLIT(W_F16);
     }
+#undef SPLIT3
 #undef SPLIT
   }
   hipError_t le = hipGetLastError();

@@ -362,11 +362,38 @@ def test_linear_many_rows_quantised(ops, oracle, kind):
     want = oracle.linear(x, wd, b)
     lib = _lib.load()
     try:
-        for mode in (2, 3):
+        for mode in (2, 3, 0):
             _lib.check(lib.cthip_set_option(b"gemm_precision", mode))
             close(ops.linear(x, wm, bias=b), want)
         _lib.check(lib.cthip_set_option(b"gemm_precision", 1))
         close(ops.linear(x, wm, bias=b), want, 1e-2, 1e-2)
+    finally:
+        _lib.check(lib.cthip_set_option(b"gemm_precision", 2))
+
+
+@pytest.mark.parametrize("kind", ["f16", "f32"])
+@pytest.mark.parametrize("cols", [100, 203, 1000])
+def test_linear_many_rows_odd_width(ops, oracle, kind, cols):
+    """Unquantised weight rows whose width is no multiple of 16 (4, 8): several input rows must not read across
+    the end of a weight row, in any precision mode."""
+    from caten_amd import _lib
+    from caten_amd.llm import Tensor
+    rng = np.random.default_rng(63)
+    rows, m = 77, 70
+    w = rng.normal(0, 0.05, (rows, cols)).astype(np.float32)
+    x = rng.normal(0, 1, (m, cols)).astype(np.float32)
+    t = Tensor.from_f32(w, kind)
+    wd = oracle.dequant(kind, t.raw, w.size).reshape(rows, cols)
+    wm = ops.WeightMatrix(kind, t.raw, rows, cols)
+    want = oracle.linear(x, wd, None)
+    lib = _lib.load()
+    try:
+        for mode in (0, 1, 2, 3):
+            _lib.check(lib.cthip_set_option(b"gemm_precision", mode))
+            if mode == 1 and cols % 16 == 0:
+                close(ops.linear(x, wm), want, 1e-2, 1e-2)
+            else:
+                close(ops.linear(x, wm), want)
     finally:
         _lib.check(lib.cthip_set_option(b"gemm_precision", 2))
 

@@ -767,7 +767,6 @@ int launch_gemm(GemmArgs a, int bmode, int precision) {
     const int nsteps = (a.K + 63) / 64;  // K-steps of 64 (two of the fp32 kernel's)
     int ks = (int)((cus * 3 / 2) / tiles);
     if (ks > nsteps / 6) ks = nsteps / 6;
-    if (const char *e = getenv("CTHIP_KS")) ks = atoi(e);  // TEMP
     if (ks > 16) ks = 16;
     if (ks > 1) {
       const int steps_per = (nsteps + ks - 1) / ks;

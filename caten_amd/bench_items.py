@@ -59,14 +59,17 @@ def main():
     from .renderer import HipRenderer
     from .buffer import HipBuffer
 
-    it = blueprints.softmax_rows()
+    it = blueprints.softmax_rows()  # dynamic shape: rows and n are arguments
+    its = blueprints.softmax_rows("fused_softmax_static", rows, d)  # static shape: the bounds are literals
     rr = HipRenderer()
     rr.render_kernel(it)
-    rr.compile_kernel([it])
+    rr.render_kernel(its)
+    rr.compile_kernel([it, its])
     # buffers over the same device arrays the hand-written items use
     bx = HipBuffer(shape=[rows, d], stride=[d, 1], dtype="float32", nrank=2, value=x.ptr)
     by = HipBuffer(shape=[rows, d], stride=[d, 1], dtype="float32", nrank=2, value=y.ptr)
-    items.append(("softmax (64,1024,768), RENDERED from its blueprint", lambda: it["compiled_object"](None, by, rows, d, bx)))
+    items.append(("softmax (64,1024,768), RENDERED from its blueprint, dynamic shape", lambda: it["compiled_object"](None, by, rows, d, bx)))
+    items.append(("softmax (64,1024,768), RENDERED from its blueprint, static shape", lambda: its["compiled_object"](None, by, bx)))
     for name, fn in items:
         us = _time(lib, fn)
         gbs = nbytes / (us * 1e-6) / 1e9

@@ -24,16 +24,21 @@ def _glob(id_, arg_type, nrank, dtype="float32"):
     return {"type": "DEFINE-GLOBAL", "id": id_, "dtype": dtype, "pointer_p": nrank > 0, "arg_type": arg_type, "nrank": nrank}
 
 
-def softmax_rows(name: str = "fused_softmax") -> dict:
+def softmax_rows(name: str = "fused_softmax", rows: int | None = None, n: int | None = None) -> dict:
     """softmax over the last axis of (rows, n): max, sum of exp2((x - max) * 1/ln2), normalise
-    (nn/activations.lisp:59-62,107-119).  Arguments: val_y, rows, n, val_x."""
-    idx = _add(_mul("n", "_gid0"), "_gid1")
+    (nn/activations.lisp:59-62,107-119).  With `rows` and `n` given the shape is static, as for a tensor made
+    with a fixed shape: the bounds are literals and the arguments are val_y, val_x; otherwise they are the
+    dynamic-shape arguments val_y, rows, n, val_x."""
+    static = rows is not None and n is not None
+    R, N = (rows, n) if static else ("rows", "n")
+    idx = _add(_mul(N, "_gid0"), "_gid1")
     ex = {"op": "EXP2", "args": [_mul(_add(_A("val_x", idx), {"op": "NEG", "args": ["m"]}), 1.442695)]}
-    loop = {"type": "FOR", "idx": "_gid1", "upfrom": 0, "below": _lt("_gid1", "n"), "by": 1}
+    loop = {"type": "FOR", "idx": "_gid1", "upfrom": 0, "below": _lt("_gid1", N), "by": 1}
     end = {"type": "ENDFOR", "idx": "_gid1"}
+    shapes = [] if static else [_glob("rows", "shape", 0, "int64"), _glob("n", "shape", 0, "int64")]
     return {"name": name, "blueprint": [
-        _glob("val_y", "output", 2), _glob("rows", "shape", 0, "int64"), _glob("n", "shape", 0, "int64"), _glob("val_x", "input", 2),
-        {"type": "FOR", "idx": "_gid0", "upfrom": 0, "below": _lt("_gid0", "rows"), "by": 1},
+        _glob("val_y", "output", 2), *shapes, _glob("val_x", "input", 2),
+        {"type": "FOR", "idx": "_gid0", "upfrom": 0, "below": _lt("_gid0", R), "by": 1},
         {"type": "EXPR", "writes": [_A("m", None)], "expr": float("-inf"), "declare_type": True, "dtype": "float32"},
         dict(loop),
         {"type": "EXPR", "writes": [_A("m", None)], "expr": {"op": "MAX", "args": ["m", _A("val_x", idx)]}, "dtype": "float32", "reduction": True},

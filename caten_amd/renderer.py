@@ -372,21 +372,36 @@ class HipRenderer(Renderer):
                 out.append(f"{pad()}const int {f['idx'].lower()} = (int)(_t % (long long)({bs})); _t /= (long long)({bs});")
             body = body[npar:len(body) - npar]
         depth = 0
+        closers: List[str] = []  # what ends each open loop
         for pos, n in enumerate(body):
             t = n["type"]
             if t == "FOR":
                 if wave_red is not None:  # the lanes of the row's wavefront stride this axis together
-                    out.append(f"{pad()}for (int {n['idx'].lower()}=({self.render_expr(n['upfrom'], 'int64')})+_lane; "
-                               f"{self.render_expr(n['below'], 'int64')}; {n['idx'].lower()}+=64) {{")
+                    lo, hi = self._const_value(n["upfrom"]), self._const_value(self._upper_bound(n))
+                    idx = n["idx"].lower()
+                    if lo is not None and hi is not None and float(lo).is_integer() and float(hi).is_integer() \
+                            and 0 < (int(hi) - int(lo) + 63) // 64 <= 32:
+                        # a static row of at most 32 elements per lane: a counted loop, unrolled, so that the loops
+                        # over the same row share their loads (inputs are __restrict__) and the row is read once
+                        lo, hi = int(lo), int(hi)
+                        out.append(f"{pad()}#pragma unroll")
+                        out.append(f"{pad()}for (int {idx}_i=0; {idx}_i<{(hi - lo + 63) // 64}; {idx}_i++) {{ "
+                                   f"const int {idx}={lo}+_lane+64*{idx}_i;" + (f" if ({idx}<{hi}) {{" if (hi - lo) % 64 else ""))
+                        closers.append("}}" if (hi - lo) % 64 else "}")
+                    else:
+                        out.append(f"{pad()}for (int {idx}=({self.render_expr(n['upfrom'], 'int64')})+_lane; "
+                                   f"{self.render_expr(n['below'], 'int64')}; {idx}+=64) {{")
+                        closers.append("}")
                 else:
                     out.append(f"{pad()}for (int {n['idx'].lower()}={self.render_expr(n['upfrom'], 'int64')}; "
                                f"{self.render_expr(n['below'], 'int64')}; {n['idx'].lower()}+={self.render_expr(n.get('by', 1), 'int64')}) {{")
+                    closers.append("}")
                 indent += 2
                 depth += 1
             elif t == "ENDFOR":
                 indent -= 2
                 depth -= 1
-                out.append(f"{pad()}}}")
+                out.append(f"{pad()}{closers.pop()}")
                 if wave_red is not None:
                     for var, op in wave_red.get(pos, []):
                         out.append(f"{pad()}{var} = ct_wave_{op}_f({var});")

@@ -258,3 +258,30 @@ def test_rendered_rowwise_kernels_match_oracle(oracle):
         assert np.max(np.abs(got - want)) < 2e-5
         assert np.allclose(transfer_into_array(bufs["mean"]), x.mean(axis=1), rtol=1e-5, atol=1e-5)
         assert np.allclose(transfer_into_array(bufs["o"]), 2.5 + x.sum(axis=1, dtype=np.float64), rtol=1e-5, atol=1e-4)
+
+
+@pytest.mark.parametrize("n", [768, 700, 64, 5])
+def test_rendered_softmax_static_shape(oracle, n):
+    """A static-shape row reduction is rendered as counted, unrolled lane-strided loops (ragged rows get a guard on
+    the element index); the result must equal the dynamic-shape kernel's, i.e. the oracle's softmax."""
+    import caten_amd as ca
+    from caten_amd import blueprints
+    from caten_amd.buffer import HipBuffer, make_buffer, open_buffer, transfer_from_array, transfer_into_array
+    rows = 130
+    item = blueprints.softmax_rows("fused_softmax_static", rows, n)
+    rt = ca.HipRuntime()
+    r = ca.HipRenderer()
+    src = r.render_kernel(item)
+    trips = (n + 63) // 64
+    assert src.count("#pragma unroll") == 3 and src.count(f"_gid1_i<{trips};") == 3
+    assert (f"if (_gid1<{n})" in src) == (n % 64 != 0)
+    r.compile_kernel([item])
+    x = np.random.default_rng(n).normal(0, 3, (rows, n)).astype(np.float32)
+    bx = make_buffer([rows, n], [n, 1], "float32", device=HipBuffer)
+    by = make_buffer([rows, n], [n, 1], "float32", device=HipBuffer)
+    open_buffer(rt, bx)
+    open_buffer(rt, by)
+    transfer_from_array(rt, bx, x)
+    item["compiled_object"](None, by, bx)
+    got = transfer_into_array(by).reshape(rows, n)
+    assert np.max(np.abs(got - oracle.softmax(x))) < 1e-6

@@ -346,13 +346,15 @@ def test_matmul_degenerate(ops):
 
 
 @pytest.mark.parametrize("kind", ["q8_0", "q4_0"])
-def test_linear_many_rows_quantised(ops, oracle, kind):
-    """130 input rows x 4100 weight rows, ragged tile edges in both directions: the integer plane times the block
-    scales (quantised MFMA path) must match the product with the dequantised weights."""
+@pytest.mark.parametrize("rows,cols,m", [(4100, 256, 130), (333, 160, 70), (200, 4160, 40), (70, 12352, 9)])
+def test_linear_many_rows_quantised(ops, oracle, kind, rows, cols, m):
+    """Several input rows on the quantised MFMA path (integer plane times the block scales) against the product
+    with the dequantised weights: ragged tile edges in both directions; a row width whose scale rows are not
+    16-byte aligned; reductions longer than one scale tile (2048) with a partial last tile and a partial last
+    period of steps; a reduction long enough to be split over several workgroups per tile."""
     from caten_amd import _lib
     from caten_amd.llm import Tensor
     rng = np.random.default_rng(62)
-    rows, cols, m = 4100, 256, 130
     w = rng.normal(0, 0.02, (rows, cols)).astype(np.float32)
     x = rng.normal(0, 1, (m, cols)).astype(np.float32)
     b = rng.normal(0, 0.02, rows).astype(np.float32)

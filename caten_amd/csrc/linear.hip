@@ -782,7 +782,7 @@ int launch_gemv(const WMat *w, GemvArgs a, int m) {
   // generic path: prologue into a temporary, then wave-per-row
   float *tmp = nullptr;
   if (a.pro != CTHIP_PRO_NONE) {
-    int rc = cthip_alloc((void **)&tmp, sizeof(float) * (size_t)a.cols * m);
+    int rc = alloc_scratch((void **)&tmp, sizeof(float) * (size_t)a.cols * m);  // fully written below
     if (rc) return rc;
     hipLaunchKernelGGL(k_prologue, dim3(m), dim3(256), 0, s.stream, tmp, a.x, a.cols, a.pro, a.norm_g, a.norm_b, a.eps,
                        a.x_stride);
@@ -936,7 +936,7 @@ int cthip_linear(float *y, const void *wmat, const float *x, int m, const float 
     float *tmp = nullptr;
     int rc;
     if (prologue != CTHIP_PRO_NONE) {
-      if ((rc = cthip_alloc((void **)&tmp, sizeof(float) * (size_t)w->cols * m))) return rc;
+      if ((rc = alloc_scratch((void **)&tmp, sizeof(float) * (size_t)w->cols * m))) return rc;  // fully written below
       hipLaunchKernelGGL(k_prologue, dim3(m), dim3(256), 0, state().stream, tmp, x, (int)w->cols, prologue, norm_g, norm_b,
                          eps, (int64_t)(prologue == CTHIP_PRO_SWIGLU ? 2 * w->cols : w->cols));
       CTHIP_LAUNCH_CHECK();

@@ -83,14 +83,17 @@ def test_gpt2_long_context_attention(oracle):
 
 
 @pytest.mark.parametrize("kind", ["q4_0", "q8_0"])
-def test_gpt2_wide_model_folded_layernorm(oracle, kind):
-    """d_model 1024 (GPT-2 medium's width): the 4-bit decode GEMVs stage the input per workgroup, with the
-    folded LayerNorm's statistics computed there."""
-    print(f"case: gpt2 d1024 {kind}", flush=True)
+@pytest.mark.parametrize("dim,heads,ffn,plen", [(1024, 16, 2048, 5), (1280, 20, 5120, 5), (1600, 25, 6400, 12)])
+def test_gpt2_wide_model_folded_layernorm(oracle, kind, dim, heads, ffn, plen):
+    """The widths of GPT-2 medium / large / xl (apps/gpt2/gpt2.lisp:36-48), two layers each: from 1024 features on
+    the 4-bit decode GEMVs stage the input per workgroup, with the folded LayerNorm's statistics computed there;
+    1280 and 1600 features leave lanes of the row groups without a chunk; the 12-token prompt goes through the
+    batched prefill."""
+    print(f"case: gpt2 d{dim} {kind} prompt {plen}", flush=True)
     from caten_amd import synth, llm
-    cfg = dict(n_layers=2, n_heads=16, dim=1024, ffn=2048, vocab=700, max_seq=48, eps=1e-5)
+    cfg = dict(n_layers=2, n_heads=heads, dim=dim, ffn=ffn, vocab=700, max_seq=48, eps=1e-5)
     w = synth.gpt2_weights(cfg, seed=8)
-    prompt = synth.prompt(cfg["vocab"], 5, seed=8)
+    prompt = synth.prompt(cfg["vocab"], plen, seed=8)
     ref = oracle.GPT2(cfg, _dequantised(oracle, w, synth.GPT2_LINEAR_KEYS + ("lm_head",), kind))
     want_tokens, want_logits = ref.generate(prompt, 8, keep_logits=True)
     model = llm.make_gpt2(cfg, llm.gpt2_state_dict(w, kind))

@@ -20,6 +20,7 @@ struct State {
   int compute_units = 0;
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   int gemm_precision = GEMM_BF16X3_DEFAULT;  // option "gemm_precision" (GEMM_*) of m > 1 Linear launches
+  int gemv_stream = -1;  // option "gemv_stream_weights": -1 = per matrix (WMat::stream), 0 / 1 = never / always
 };
 State &state();
 // cthip_alloc without the zero fill, for temporaries that are fully written before they are read
@@ -55,7 +56,12 @@ struct WMat {
   void *q;          // quant plane: Q8_0 int8[rows][cols]; Q4_0 u8[rows][cols/2]; F32 float; F16 half
   void *d;          // scale plane: fp16[rows][cols/32] (quantised types), else NULL
   int64_t q_bytes, d_bytes;
+  // the single-row kernels request this matrix with the non-temporal hint: set for a matrix that cannot stay in
+  // the Infinity Cache between two uses (too large by itself, or one of a model's that together are too large)
+  bool stream;
 };
+// gfx950: 256 MB of Infinity Cache in front of HBM
+static const int64_t kInfinityCacheBytes = 256ll << 20;
 
 // Arguments of one fused Linear launch:
 //   y = act(prologue(x) . W^T + bias) + residual

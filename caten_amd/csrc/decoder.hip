@@ -299,6 +299,17 @@ static int finalize(Decoder *d) {
   TRY(dev_alloc(d, (void **)&d->am_val, sizeof(float) * kGemvMaxWaves));
   TRY(dev_alloc(d, (void **)&d->am_idx, sizeof(int) * kGemvMaxWaves));
 
+  {
+    // A step reads every weight once.  Past the Infinity Cache (three quarters of it: the KV cache and the
+    // activations live there too) nothing of that stream survives to the next step, so it is requested
+    // non-temporally and stops evicting what the step does reuse.
+    std::vector<WMat *> ws = {d->lm_head};
+    for (Layer &L : d->layers) ws.insert(ws.end(), {L.attn, L.proj, L.fc, L.fc2});
+    int64_t total = 0;
+    for (WMat *w : ws) total += w ? w->q_bytes + w->d_bytes : 0;
+    for (WMat *w : ws)
+      if (w) w->stream = total > kInfinityCacheBytes / 4 * 3;
+  }
   const char *ng = getenv("CTHIP_NO_GRAPH");
   if (ng && *ng && *ng != '0') d->use_graph = false;
   if (d->use_graph) {

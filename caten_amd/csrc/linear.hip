@@ -385,7 +385,10 @@ __device__ __forceinline__ void coop_fold(const GemvArgs &a, const float *__rest
 
 // PD = weight tiles a wavefront keeps in flight: 1 for the small, latency-bound launches (one tile
 // per wavefront), 4 for the large ones, whose throughput is bytes-in-flight / memory latency.
-template <int TYPE, int G, int KC, int PD>
+// NT: the weights are requested with the non-temporal hint.  A model whose weights exceed the 256 MB Infinity
+// Cache streams all of them from HBM every step whatever the hint; without it the stream also evicts the
+// vectors, fold terms and KV rows that the step does reuse.
+template <int TYPE, int G, int KC, int PD, bool NT>
 __global__ __launch_bounds__(256) void k_gemv(GemvArgs a) {
   constexpr int XPC = Fmt<TYPE>::XPC;
   constexpr int RPW = 64 / G;  // rows per wavefront per iteration
@@ -423,7 +426,17 @@ __global__ __launch_bounds__(256) void k_gemv(GemvArgs a) {
     for (int j = 0; j < KC; j++) {
       const int c = l + G * j;
       const bool ok = rok && c < nchunks;
-      w[j] = ok ? qp[(int64_t)row * row_chunks + c] : make_uint4(0u, 0u, 0u, 0u);
+      if (NT) {
+        uint4 t = make_uint4(0u, 0u, 0u, 0u);
+        if (ok) {
+          const uint4 *src = &qp[(int64_t)row * row_chunks + c];
+          t = make_uint4(__builtin_nontemporal_load(&src->x), __builtin_nontemporal_load(&src->y),
+                         __builtin_nontemporal_load(&src->z), __builtin_nontemporal_load(&src->w));
+        }
+        w[j] = t;
+      } else {
+        w[j] = ok ? qp[(int64_t)row * row_chunks + c] : make_uint4(0u, 0u, 0u, 0u);
+      }
       if (QUANT) {
         const int sidx = (TYPE == CTHIP_Q8_0) ? (c >> 1) : c;
         s[j] = ok ? a.d[(int64_t)row * scales_per_row + sidx] : (unsigned short)0;
@@ -633,11 +646,14 @@ __global__ __launch_bounds__(256) void k_prologue(float *__restrict__ out, const
 typedef void (*gemv_fn)(GemvArgs);
 struct GemvVariant {
   int type, G, KC;
-  gemv_fn fn;       // large launches
-  gemv_fn fn_small; // small, latency-bound launches
+  gemv_fn fn[2];       // large launches: [0] cached weights, [1] streamed (non-temporal) weights
+  gemv_fn fn_small[2]; // small, latency-bound launches
 };
 // large launches keep about 12 sixteen-byte loads per lane in flight
-#define V(T, G, KC) {T, G, KC, k_gemv<T, G, KC, (KC >= 12 ? 1 : KC >= 6 ? 2 : 4)>, k_gemv<T, G, KC, 1>}
+#define PD_OF(KC) (KC >= 12 ? 1 : KC >= 6 ? 2 : 4)
+#define V(T, G, KC)                                                                           \
+  {T, G, KC, {k_gemv<T, G, KC, PD_OF(KC), false>, k_gemv<T, G, KC, PD_OF(KC), true>},         \
+   {k_gemv<T, G, KC, 1, false>, k_gemv<T, G, KC, 1, true>}}
 static const GemvVariant kVariants[] = {
     V(CTHIP_Q8_0, 16, 1), V(CTHIP_Q8_0, 16, 2), V(CTHIP_Q8_0, 16, 3), V(CTHIP_Q8_0, 16, 4),
     V(CTHIP_Q8_0, 32, 3), V(CTHIP_Q8_0, 32, 4), V(CTHIP_Q8_0, 64, 3), V(CTHIP_Q8_0, 64, 4),
@@ -650,6 +666,7 @@ static const GemvVariant kVariants[] = {
     V(CTHIP_F16, 64, 6), V(CTHIP_F16, 64, 8), V(CTHIP_F16, 64, 12),
 };
 #undef V
+#undef PD_OF
 
 static int xpc_of(int type) {
   switch (type) {
@@ -751,7 +768,7 @@ int launch_gemv(const WMat *w, GemvArgs a, int m) {
       const int vi = (int)(v - kVariants);
       if (occ_cache[vi] == 0) {
         int nb = 0;
-        CTHIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, v->fn, 256, 16 * 1024));
+        CTHIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, v->fn[0], 256, 16 * 1024));
         occ_cache[vi] = nb > 0 ? nb : 1;
       }
       block = dim3(256);
@@ -771,7 +788,8 @@ int launch_gemv(const WMat *w, GemvArgs a, int m) {
     const int nwaves = (int)(grid.x * (block.x / 64));
     if (a.am_val && nwaves > kGemvMaxWaves)
       return fail(CTHIP_E_UNSUPPORTED, "gemv: %d wavefronts exceed the argmax scratch", nwaves);
-    hipLaunchKernelGGL(small ? v->fn_small : v->fn, grid, block, lds, s.stream, a);
+    const int nt = s.gemv_stream < 0 ? (w->stream ? 1 : 0) : s.gemv_stream;
+    hipLaunchKernelGGL(small ? v->fn_small[nt] : v->fn[nt], grid, block, lds, s.stream, a);
     CTHIP_LAUNCH_CHECK();
     if (a.am_val) {
       hipLaunchKernelGGL(k_argmax_finish, dim3(1), dim3(256), 0, s.stream, a, nwaves);
@@ -845,6 +863,7 @@ int wmat_create_impl(WMat **out, int type, const void *raw, int64_t rows, int64_
     }
     CTHIP_CHECK(hipMemcpyAsync(w->q, raw, (size_t)w->q_bytes, hipMemcpyDeviceToDevice, s.stream));
   }
+  w->stream = w->q_bytes + w->d_bytes > kInfinityCacheBytes;  // cannot stay cached between two uses by itself
   *out = w;
   return 0;
 }
@@ -966,6 +985,11 @@ int cthip_set_option(const char *name, int value) {
   if (!strcmp(name, "gemm_precision")) {
     if (value < GEMM_FP32 || value > GEMM_BF16X6) return fail(CTHIP_E_BAD_ARG, "cthip_set_option: gemm_precision is 0..3");
     state().gemm_precision = value;
+    return 0;
+  }
+  if (!strcmp(name, "gemv_stream_weights")) {
+    if (value < -1 || value > 1) return fail(CTHIP_E_BAD_ARG, "cthip_set_option: gemv_stream_weights is -1, 0 or 1");
+    state().gemv_stream = value;
     return 0;
   }
   if (!strcmp(name, "gemm_bf16")) {  // 1 = operands rounded to bf16, 0 = back to the default

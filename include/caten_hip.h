@@ -159,7 +159,11 @@ int cthip_linear(float *y, const void *wmat, const float *x, int m, const float 
  *   per product, fp32 accumulation (2^-16 of a product is lost); 3 = three terms, six MFMAs per
  *   product: all 24 bits of an fp32 operand; 0 = fp32 MFMA operands; 1 = operands rounded to bf16
  *   (rtol/atol 1e-2).
- * "gemm_bf16": 1 = shorthand for gemm_precision 1, 0 = back to the default. */
+ * "gemm_bf16": 1 = shorthand for gemm_precision 1, 0 = back to the default.
+ * "gemv_stream_weights": whether the single-row Linear kernels request the weights with the non-temporal
+ *   hint: -1 (default) = per matrix -- a matrix larger than the 256 MB Infinity Cache, and every matrix of a
+ *   decoder session whose weights together exceed three quarters of it; 0 = never; 1 = always.  Results do
+ *   not depend on it.  A decoder session picks its kernels when it first runs. */
 int cthip_set_option(const char *name, int value);
 
 /* !relu(!matmul A B) (api/high-level-ops.lisp:76-99; fused per test-scheduler.lisp:140-163):

@@ -104,6 +104,36 @@ def test_gpt2_wide_model_folded_layernorm(oracle, kind, dim, heads, ffn, plen):
     model.close()
 
 
+@pytest.mark.parametrize("arch", ["gpt2", "llama"])
+def test_streamed_weights_decode_identical(arch):
+    """A session whose kernels request the weights non-temporally (the policy for models past the Infinity Cache,
+    forced here on a small one) generates the same tokens and bit-identical logits as the default session."""
+    print(f"case: streamed weights {arch}", flush=True)
+    from caten_amd import _lib, synth, llm
+    lib = _lib.load()
+    if arch == "gpt2":
+        cfg = synth.GPT2_CONFIGS["gpt2-tiny"]
+        sd = llm.gpt2_state_dict(synth.gpt2_weights(cfg, seed=5), "q8_0")
+        make, gen = llm.make_gpt2, llm.gpt2_generate
+    else:
+        cfg = synth.LLAMA_CONFIGS["llama-tiny"]
+        sd = llm.llama_state_dict(synth.llama_weights(cfg, seed=5), "q4_0")
+        make, gen = llm.make_llama, llm.gpt2_generate  # the loop is the same for both architectures
+    prompt = synth.prompt(cfg["vocab"], 6, seed=5)
+    runs = []
+    try:
+        for mode in (0, 1):
+            _lib.check(lib.cthip_set_option(b"gemv_stream_weights", mode))
+            model = make(cfg, sd)
+            runs.append(gen(model, prompt, 10, on_device=False, keep_logits=True))
+            model.close()
+    finally:
+        _lib.check(lib.cthip_set_option(b"gemv_stream_weights", -1))
+    assert runs[0][0] == runs[1][0]
+    for a, b in zip(runs[0][1], runs[1][1]):
+        assert np.array_equal(a, b)
+
+
 def test_gpt2_prompt_lengths_and_restart(oracle):
     from caten_amd import synth, llm
     cfg = synth.GPT2_CONFIGS["gpt2-tiny"]

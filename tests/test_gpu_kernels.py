@@ -186,6 +186,33 @@ def test_gemv_wide_input_with_norms(ops, oracle, kind):
         close(ops.linear(x, wm), oracle.linear(x, wd))
 
 
+@pytest.mark.parametrize("kind", ["q4_0", "q8_0", "f16", "f32"])
+def test_gemv_streamed_weights_give_the_same_bits(ops, kind):
+    """The non-temporal request of the weights (what models past the Infinity Cache get) changes the cache policy
+    of the loads and nothing else: outputs are bit-identical to the cached-weights kernels, on a one-tile-per-
+    wavefront launch and on a looping one, with and without a staged input."""
+    from caten_amd import _lib
+    from caten_amd.llm import Tensor
+    rng = np.random.default_rng(27)
+    lib = _lib.load()
+    for rows, cols in ((300, 768), (9000, 768), (2560, 2048)):
+        w = rng.normal(0, 0.02, (rows, cols)).astype(np.float32)
+        x = rng.normal(0.1, 1.0, cols).astype(np.float32)
+        g = rng.normal(1, 0.05, cols).astype(np.float32)
+        wm = ops.WeightMatrix(kind, Tensor.from_f32(w, kind).raw, rows, cols)
+        outs = {}
+        try:
+            for mode in (0, 1):
+                _lib.check(lib.cthip_set_option(b"gemv_stream_weights", mode))
+                outs[mode] = (ops.linear(x, wm), ops.linear(x, wm, prologue="rmsnorm", norm_g=g))
+        finally:
+            _lib.check(lib.cthip_set_option(b"gemv_stream_weights", -1))
+        for a, b in zip(outs[0], outs[1]):
+            assert np.array_equal(a, b)
+    with pytest.raises(_lib.HipError):
+        _lib.check(lib.cthip_set_option(b"gemv_stream_weights", 2))
+
+
 def test_gemv_fallback_shapes_with_prologue(ops, oracle):
     from caten_amd.llm import Tensor
     rng = np.random.default_rng(22)

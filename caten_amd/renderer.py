@@ -168,6 +168,14 @@ class HipRenderer(Renderer):
             return f"(({CDTYPE[e['dtype']]}){r(a[-1])})"
         if op == "WHERE":
             return f"({r(a[0])} ? {r(a[1])} : {r(a[2])})"
+        if op == "INDEX-COMPONENTS":
+            # expr-index-components (renderer.lisp:194-221): the linear index of the element being computed,
+            # sum of stride * gid over the axes of the iteration space; an axis of size 1 contributes 0
+            terms = [{"op": "MUL", "args": [st, it]} for sz, st, it in zip(e["shape"], e["strides"], e["iterations"])
+                     if not (isinstance(sz, (int, np.integer)) and int(sz) == 1)]
+            if not terms:
+                return "0"
+            return self.render_expr(terms[0] if len(terms) == 1 else {"op": "ADD", "args": terms}, "int64")
         raise NotImplementedError(f"Hip-Renderer: no %render-node method for :{op}")
 
     def render_aref(self, e: dict, fdtype: str = "float32") -> str:
@@ -209,8 +217,10 @@ class HipRenderer(Renderer):
             if e.get("index") is not None and HipRenderer._uses(e["index"], sym):
                 return True
             sp = e.get("space")
-            if sp:
-                return any(HipRenderer._uses(x, sym) for x in sp["iterations"])
+            if sp and any(HipRenderer._uses(x, sym) for x in sp["iterations"]):
+                return True
+            if e.get("op") == "INDEX-COMPONENTS":
+                return any(HipRenderer._uses(x, sym) for x in list(e["iterations"]) + list(e["strides"]))
         return False
 
     def _parallel_prefix(self, body: List[dict]) -> int:
@@ -287,7 +297,7 @@ class HipRenderer(Renderer):
             elif t in ("IF", "ENDIF"):
                 return None
             elif t == "EXPR":
-                if n.get("dtype", "float32") != "float32" or len(n["writes"]) != 1:
+                if len(n["writes"]) != 1:
                     return None
                 w = n["writes"][0]
                 scalar = w.get("index") is None and "space" not in w
@@ -300,6 +310,8 @@ class HipRenderer(Renderer):
                     if scalar:
                         return None  # a loop-carried scalar that is not a reduction cannot be split over lanes
                     continue
+                if n.get("dtype", "float32") != "float32":
+                    return None  # the lane butterflies are fp32
                 e = n["expr"]
                 if not (scalar and isinstance(e, dict) and e.get("op", "").upper() in self._IDENTITY and len(e.get("args", [])) == 2):
                     return None
@@ -309,7 +321,9 @@ class HipRenderer(Renderer):
                            and x["id"].lower() == name and x.get("index") is None and "space" not in x for x in args]
                 if sum(selfref) != 1 or self._uses(args[1 - selfref.index(True)], name):
                     return None
-                if init.get(name) != ident:  # lane partials only combine when each starts at the identity
+                # lane partials combine when each starts at the identity; max / min are idempotent, so there any
+                # start value that all lanes share (a scalar set before the loop) will do
+                if init.get(name) != ident and not (op in ("max", "min") and name in init):
                     return None
                 loop_red.append((name, op))
         return found or None

@@ -285,3 +285,55 @@ def test_rendered_softmax_static_shape(oracle, n):
     item["compiled_object"](None, by, bx)
     got = transfer_into_array(by).reshape(rows, n)
     assert np.max(np.abs(got - oracle.softmax(x))) < 1e-6
+
+
+def test_rendered_argmax_with_index_components(oracle):
+    """ArgMax as Caten lowers it (high-level-ops.lisp:314-343): the row maximum, then the maximum over the row of
+    where(x == max, (N - 1) - index, 0) with the index from :INDEX-COMPONENTS, and N - that - 1 cast to int64 --
+    the lowest index among ties.  Rendered, compiled, run; checked against the oracle's argmax."""
+    import caten_amd as ca
+    from caten_amd.buffer import HipBuffer, make_buffer, open_buffer, transfer_from_array, transfer_into_array
+    A = lambda id_, idx: {"op": "AREF", "id": id_, "index": idx}  # noqa: E731
+    add = lambda *a: {"op": "ADD", "args": list(a)}  # noqa: E731
+    mul = lambda *a: {"op": "MUL", "args": list(a)}  # noqa: E731
+    lt = lambda a, b: {"op": "<", "args": [a, b]}  # noqa: E731
+    neg = lambda a: {"op": "NEG", "args": [a]}  # noqa: E731
+    rows, n = 37, 500
+    idx = add(mul(n, "_gid0"), "_gid1")
+    # the column index of the element: the row axis has stride 0 in this index space
+    col = {"op": "CAST", "dtype": "float32",
+           "args": [None, {"op": "INDEX-COMPONENTS", "shape": [rows, n], "strides": [0, 1], "iterations": ["_gid0", "_gid1"]}]}
+    eq = {"op": "NOT", "args": [{"op": "!=", "args": [None, A("val_x", idx), "m"]}]}
+    item = {"name": "fused_argmax", "blueprint": [
+        {"type": "DEFINE-GLOBAL", "id": "val_out", "dtype": "int64", "pointer_p": True, "arg_type": "output", "nrank": 1},
+        {"type": "DEFINE-GLOBAL", "id": "val_x", "dtype": "float32", "pointer_p": True, "arg_type": "input", "nrank": 2},
+        {"type": "FOR", "idx": "_gid0", "upfrom": 0, "below": lt("_gid0", rows), "by": 1},
+        {"type": "EXPR", "writes": [A("m", None)], "expr": float("-inf"), "declare_type": True, "dtype": "float32"},
+        {"type": "FOR", "idx": "_gid1", "upfrom": 0, "below": lt("_gid1", n), "by": 1},
+        {"type": "EXPR", "writes": [A("m", None)], "expr": {"op": "MAX", "args": ["m", A("val_x", idx)]}, "dtype": "float32", "reduction": True},
+        {"type": "ENDFOR", "idx": "_gid1"},
+        {"type": "EXPR", "writes": [A("best", None)], "expr": 0.0, "declare_type": True, "dtype": "float32"},
+        {"type": "FOR", "idx": "_gid1", "upfrom": 0, "below": lt("_gid1", n), "by": 1},
+        {"type": "EXPR", "writes": [A("best", None)], "dtype": "float32", "reduction": True,
+         "expr": {"op": "MAX", "args": ["best", {"op": "WHERE", "args": [eq, add(float(n - 1), neg(col)), 0.0]}]}},
+        {"type": "ENDFOR", "idx": "_gid1"},
+        {"type": "EXPR", "writes": [A("val_out", "_gid0")], "dtype": "int64",
+         "expr": {"op": "CAST", "dtype": "int64", "args": [None, add(add(float(n), neg("best")), -1.0)]}},
+        {"type": "ENDFOR", "idx": "_gid0"},
+    ]}
+    rt = ca.HipRuntime()
+    r = ca.HipRenderer()
+    src = r.render_kernel(item)
+    assert "(1*_gid1)" in src and "ct_wave_max_f(best)" in src  # index components; both reductions one wavefront per row
+    r.compile_kernel([item])
+    rng = np.random.default_rng(3)
+    x = rng.integers(-5, 6, (rows, n)).astype(np.float32)  # many ties: the lowest index must win
+    bx = make_buffer([rows, n], [n, 1], "float32", device=HipBuffer)
+    bo = make_buffer([rows], [1], "int64", device=HipBuffer)
+    open_buffer(rt, bx)
+    open_buffer(rt, bo)
+    transfer_from_array(rt, bx, x)
+    item["compiled_object"](None, bo, bx)
+    got = transfer_into_array(bo).reshape(rows)
+    assert np.array_equal(got, np.argmax(x, axis=1))
+    assert np.array_equal(got, np.asarray([oracle.argmax(row) for row in x]).reshape(rows))

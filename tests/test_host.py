@@ -133,6 +133,10 @@ def test_renderer_spellings():
     aref = {"op": "AREF", "id": "V", "space": {"strides": [12, 1, 0], "views": [None, (2, 9, 3, False), (0, 4, 1, True)],
                                                 "iterations": ["i", "j", "k"]}}
     assert r.render_expr(aref) == "v[((12*i)+(1*(2+(3*j))))]"
+    # renderer.lisp:194-221: the index of the element being computed; size-1 axes contribute nothing
+    ic = {"op": "INDEX-COMPONENTS", "shape": [4, 1, "n"], "strides": ["n", "n", 1], "iterations": ["_gid0", "_gid1", "_gid2"]}
+    assert r.render_expr(ic) == "((n*_gid0)+(1*_gid2))"
+    assert r.render_expr({"op": "INDEX-COMPONENTS", "shape": [1], "strides": [1], "iterations": ["_gid0"]}) == "0"
     with pytest.raises(NotImplementedError):
         r.render_expr({"op": "NOPE", "args": []})
 

@@ -726,7 +726,7 @@ __global__ __launch_bounds__(256) void k_splitk_reduce(GemmArgs a) {
   }
 }
 
-// precision: GEMM_FP32 = fp32 MFMA operands (k_gemm), GEMM_BF16 = operands rounded to bf16,
+// precision: GEMM_FP32 = fp32 MFMA operands (k_gemm_f32), GEMM_BF16 = operands rounded to bf16,
 // GEMM_BF16X3 / GEMM_BF16X6 = operands split in two / three bf16 terms.  Q8_0 / Q4_0 weights take k_gemm_q
 // (integer plane exact in bf16, block scales applied to the partial sums) with 1 / 2 / 3 activation terms.
 int launch_gemm(GemmArgs a, int bmode, int precision) {

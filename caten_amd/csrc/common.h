@@ -101,6 +101,12 @@ struct GemvArgs {
   int *am_pos;
   long long *am_hist;
   int *am_hist_n;
+  // the block that settles the token also gathers the next step's input, nx_out[d] = nx_wte[token][d] +
+  // nx_wpe[position + 1][d] (the Embedding items of the next forward), so that a device-resident loop needs no
+  // embedding launch between steps.  nx_out null = off; nx_wpe null = no position table.
+  float *nx_out;
+  const float *nx_wte, *nx_wpe;
+  int nx_dim, nx_vocab, nx_max_pos;
 };
 // most wavefronts any GEMV launch uses (sizes the am_val / am_idx scratch)
 constexpr int kGemvMaxWaves = 16384;

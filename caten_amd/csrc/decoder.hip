@@ -192,7 +192,7 @@ static int to_wmat(Decoder *d, const std::vector<std::string> &keys, int64_t wan
   return 0;
 }
 
-static int queue_step(Decoder *d, bool with_head);
+static int queue_step(Decoder *d, bool with_head, bool embed = true);
 static int queue_head(Decoder *d);
 
 // S = W.gamma and C = W.beta + bias for a LayerNorm that precedes the Linear W
@@ -319,8 +319,9 @@ static int finalize(Decoder *d) {
     for (int pass = 0; pass < 3; pass++) {
       hipGraph_t g = nullptr;
       CTHIP_CHECK(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
-      rc = queue_step(d, pass != 1);
-      for (int k = 1; pass == 2 && k < kStepsPerGraph && !rc; k++) rc = queue_step(d, true);
+      // the device-resident loop (pass 2) only ever follows a head, which leaves the next input in place
+      rc = queue_step(d, pass != 1, pass != 2);
+      for (int k = 1; pass == 2 && k < kStepsPerGraph && !rc; k++) rc = queue_step(d, true, false);
       hipError_t e = hipStreamEndCapture(st, &g);
       if (rc) {
         if (g) (void)hipGraphDestroy(g);
@@ -340,7 +341,7 @@ static int finalize(Decoder *d) {
 }
 
 // queues one decode step on the stream; token and position are read from d->tokpos
-static int queue_step(Decoder *d, bool with_head) {
+static int queue_step(Decoder *d, bool with_head, bool embed) {
   const cthip_decoder_config &c = d->cfg;
   const int D = c.dim, F = c.ffn, V = c.vocab, KD = kv_dim(c), Dh = c.dim / c.n_heads;
   const int *tok = d->tokpos, *pos = d->tokpos + 1;
@@ -348,7 +349,8 @@ static int queue_step(Decoder *d, bool with_head) {
 #define TRY(e) \
   if ((rc = (e))) return rc
   const bool gpt2 = c.arch == CTHIP_ARCH_GPT2;
-  TRY(launch_embedding(d->x, d->wte, nullptr, tok, 1, V, D, gpt2 ? d->wpe : nullptr, pos, c.max_seq));
+  // embed = false: the previous step's head has already gathered this step's input (queue_head)
+  if (embed) TRY(launch_embedding(d->x, d->wte, nullptr, tok, 1, V, D, gpt2 ? d->wpe : nullptr, pos, c.max_seq));
   for (int l = 0; l < c.n_layers; l++) {
     Layer &L = d->layers[l];
     GemvArgs a = {};
@@ -443,6 +445,13 @@ static int queue_head(Decoder *d) {
   o.am_pos = d->tokpos + 1;
   o.am_hist = (long long *)d->history;
   o.am_hist_n = d->hist_n;
+  // ... and its embedding rows become the next step's input, in the block that settles the token
+  o.nx_out = d->x;
+  o.nx_wte = d->wte;
+  o.nx_wpe = gpt2 ? d->wpe : nullptr;
+  o.nx_dim = c.dim;
+  o.nx_vocab = c.vocab;
+  o.nx_max_pos = c.max_seq;
   return launch_gemv(d->lm_head, o, 1);
 }
 

@@ -233,6 +233,7 @@ __device__ __forceinline__ void gemv_argmax_tail(const GemvArgs &a, int wave, in
 __global__ __launch_bounds__(256) void k_argmax_finish(GemvArgs a, int nparts) {
   __shared__ float sv[4];
   __shared__ int si[4];
+  __shared__ int next_tok, next_pos;
   // the loop state is requested up front so its latency overlaps the reduction
   int hist_n = 0, pos = 0;
   if (threadIdx.x == 0) {
@@ -259,6 +260,18 @@ __global__ __launch_bounds__(256) void k_argmax_finish(GemvArgs a, int nparts) {
       *a.am_hist_n = hist_n + 1;
     }
     if (a.am_pos) *a.am_pos = pos + 1;
+    next_tok = bi;
+    next_pos = pos + 1;
+  }
+  if (a.nx_out) {  // same values as the embedding launch of the next forward would write
+    __syncthreads();
+    const int id = next_tok, p = next_pos;
+    const bool hit = id >= 0 && id < a.nx_vocab, phit = p >= 0 && p < a.nx_max_pos;
+    for (int d = threadIdx.x; d < a.nx_dim; d += 256) {
+      float v = hit ? a.nx_wte[(int64_t)id * a.nx_dim + d] : 0.0f;
+      if (a.nx_wpe) v += phit ? a.nx_wpe[(int64_t)p * a.nx_dim + d] : 0.0f;
+      a.nx_out[d] = v;
+    }
   }
 }
 

@@ -172,7 +172,8 @@ def main():
                                f"h{cfg['n_heads']} ffn{cfg['ffn']} "
                                f"vocab{cfg['vocab']}), GGUF-{args.kind.upper()} linear weights, fp32 embeddings/norms/KV, "
                                f"{args.prompt}-token prompt, batch-1 greedy decode, positions {min(positions)}..{max(positions)}",
-                   "model": args.model, "weights": args.kind, "batch": 1},
+                   "shape": args.model, "weight_format": args.kind, "prompt_tokens": args.prompt,
+                   "positions": f"{min(positions)}..{max(positions)}"},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": TRAFFIC_BYTES.get((args.model, args.kind)),
                      "kernel": f"cthip::k_gemv<{args.kind}> on lm_head ({V}x{D}) with the ln_f prologue",

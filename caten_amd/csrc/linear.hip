@@ -753,13 +753,15 @@ int launch_gemv(const WMat *w, GemvArgs a, int m) {
     const int nrq = (a.rows + rpw - 1) / rpw;
     dim3 grid, block;
     const bool folded = (a.pro == CTHIP_PRO_RMSNORM) || (a.pro == CTHIP_PRO_LAYERNORM && a.fold_s != nullptr);
+    const bool quantised = w->type == CTHIP_Q8_0 || w->type == CTHIP_Q4_0;
     // The input vector goes through LDS once per workgroup when it must be normalised or gated first,
     // or when it is large next to a weight tile (a 4-bit tile multiplies 8 input bytes per weight byte):
-    // then four wavefronts share one copy and every wavefront takes several tiles.  A looping 8-bit launch
-    // with a folded norm (lm_head) stages too: its 48-float slice and statistics per wavefront cost more
-    // than the barrier (fp32 weights, 12 floats per lane, measured the other way round).
+    // then four wavefronts share one copy and every wavefront takes several tiles.  Quantised launches with a
+    // folded norm stage at every size: a lane's slice is 48-64 floats, and gamma * x plus the statistics once
+    // per workgroup beat once per wavefront (GPT-2 decode: Q8_0 284.6 -> 280.3 us / step, Q4_0 339 -> 308;
+    // fp32 / fp16 weights, 12-24 floats per lane, measured the other way round: 354 -> 369, 328 -> 347).
     const bool stage = (a.pro != CTHIP_PRO_NONE && !folded) || (w->type == CTHIP_Q4_0 && a.cols >= 1024) ||
-                       (folded && (a.cols >= 2048 || (nrq > 2048 && w->type == CTHIP_Q8_0)));
+                       (folded && (a.cols >= 2048 || quantised));
     const size_t lds = stage ? sizeof(float) * (size_t)a.cols : 0;
     if (lds > 64 * 1024) return fail(CTHIP_E_UNSUPPORTED, "gemv: %d input features exceed the LDS staging buffer", a.cols);
     a.stage_x = stage ? 1 : 0;

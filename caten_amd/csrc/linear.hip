@@ -773,9 +773,14 @@ int launch_gemv(const WMat *w, GemvArgs a, int m) {
       block = dim3(64);
       grid = dim3(nrq, m);
     } else if (stage && nrq <= s.compute_units * 4) {
+      // one tile per wavefront, as many wavefronts per workgroup (at most four) as leave about one workgroup
+      // per compute unit: fewer workgroups repeat the staging less, but idle units stream nothing
+      // (GPT-2 c_attn / c_fc, 576 / 768 tiles: 3 per workgroup 279.9 us / step, 4: 283.1, 2: 286.8, 1: 289.1)
       small = true;
-      block = dim3(256);
-      grid = dim3((nrq + 3) / 4, m);
+      int wpb = (nrq + s.compute_units - 1) / s.compute_units;
+      wpb = wpb < 1 ? 1 : wpb > 4 ? 4 : wpb;
+      block = dim3(64 * wpb);
+      grid = dim3((nrq + wpb - 1) / wpb, m);
     } else {
       // larger matrices: at least one wavefront per SIMD, more (up to what the register budget keeps
       // resident) once every wavefront has four tiles; all loop over the same number of tiles (an

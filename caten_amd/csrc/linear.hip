@@ -267,10 +267,19 @@ __global__ __launch_bounds__(256) void k_argmax_finish(GemvArgs a, int nparts) {
     __syncthreads();
     const int id = next_tok, p = next_pos;
     const bool hit = id >= 0 && id < a.nx_vocab, phit = p >= 0 && p < a.nx_max_pos;
-    for (int d = threadIdx.x; d < a.nx_dim; d += 256) {
-      float v = hit ? a.nx_wte[(int64_t)id * a.nx_dim + d] : 0.0f;
-      if (a.nx_wpe) v += phit ? a.nx_wpe[(int64_t)p * a.nx_dim + d] : 0.0f;
-      a.nx_out[d] = v;
+    if ((a.nx_dim & 3) == 0) {  // rows are 16-byte aligned: four floats per request
+      const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+      for (int d = threadIdx.x; d < (a.nx_dim >> 2); d += 256) {
+        const float4 e = hit ? ((const float4 *)(a.nx_wte + (int64_t)id * a.nx_dim))[d] : zero;
+        const float4 w = (a.nx_wpe && phit) ? ((const float4 *)(a.nx_wpe + (int64_t)p * a.nx_dim))[d] : zero;
+        ((float4 *)a.nx_out)[d] = a.nx_wpe ? make_float4(e.x + w.x, e.y + w.y, e.z + w.z, e.w + w.w) : e;
+      }
+    } else {
+      for (int d = threadIdx.x; d < a.nx_dim; d += 256) {
+        float v = hit ? a.nx_wte[(int64_t)id * a.nx_dim + d] : 0.0f;
+        if (a.nx_wpe) v += phit ? a.nx_wpe[(int64_t)p * a.nx_dim + d] : 0.0f;
+        a.nx_out[d] = v;
+      }
     }
   }
 }

@@ -765,7 +765,10 @@ int launch_gemm(GemmArgs a, int bmode, int precision) {
     grid.x = 8u * (unsigned)a.rm * (unsigned)a.rn;
     // too few tiles to occupy the chip and a long reduction axis: split K over several workgroups per tile
     const int nsteps = (a.K + 63) / 64;  // K-steps of 64 (two of the fp32 kernel's)
-    int ks = (int)((cus * 3 / 2) / tiles);
+    // workgroups aimed at: two per compute unit where the tiles fill less than half the chip (GPT-2 / Llama
+    // prefill 1.47 / 3.29 -> 1.44 / 3.18 ms against 1.5; three per unit: 1.55 / 3.18), else 1.5 (a 1024^3
+    // product, one tile per unit, loses 10-30 % when it is split in two)
+    int ks = (int)((tiles * 2 <= cus ? cus * 2 : cus * 3 / 2) / tiles);
     if (ks > nsteps / 6) ks = nsteps / 6;
     if (ks > 16) ks = 16;
     if (ks > 1) {

@@ -804,9 +804,12 @@ int launch_gemv(const WMat *w, GemvArgs a, int m) {
       }
       block = dim3(256);
       const int base = s.compute_units * 4;
-      int wanted = (nrq + 3) / 4;
+      // unstaged: a wavefront per tile up to three resident wavefronts per SIMD (fp32 GPT-2 decode with every large
+      // launch at 1024 / 2048 / 3072 / 4096 wavefronts: 369 / 343 / 334 / 343 us per step)
+      int wanted = stage ? (nrq + 3) / 4 : nrq;
       if (wanted < base) wanted = base;
-      if (wanted > base * occ_cache[vi]) wanted = base * occ_cache[vi];
+      const int cap = base * (stage || occ_cache[vi] < 3 ? occ_cache[vi] : 3);
+      if (wanted > cap) wanted = cap;
       // staged launches pay the input staging once per workgroup: whole workgroups per compute unit, two
       // when there is work for more than one (measured best; a third does not fit beside the first two)
       if (stage && wanted > base && occ_cache[vi] >= 2) wanted = 2 * base;

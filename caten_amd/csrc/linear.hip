@@ -781,13 +781,15 @@ int launch_gemv(const WMat *w, GemvArgs a, int m) {
       small = true;
       block = dim3(64);
       grid = dim3(nrq, m);
-    } else if (stage && nrq <= s.compute_units * 4) {
-      // one tile per wavefront, as many wavefronts per workgroup (at most four) as leave about one workgroup
+    } else if (stage && nrq <= s.compute_units * 3) {
+      // one tile per wavefront, as many wavefronts per workgroup (at most three) as leave about one workgroup
       // per compute unit: fewer workgroups repeat the staging less, but idle units stream nothing
-      // (GPT-2 c_attn / c_fc, 576 / 768 tiles: 3 per workgroup 279.9 us / step, 4: 283.1, 2: 286.8, 1: 289.1)
+      // (GPT-2 c_attn / c_fc, 576 / 768 tiles: 3 per workgroup 279.9 us / step, 4: 283.1, 2: 286.8, 1: 289.1).
+      // Beyond three tiles per compute unit the looping launch below is ahead (TinyLlama wo, 1024 tiles:
+      // 0.780 -> 0.772 ms / step; with the limit at two, GPT-2 loses 1 %)
       small = true;
       int wpb = (nrq + s.compute_units - 1) / s.compute_units;
-      wpb = wpb < 1 ? 1 : wpb > 4 ? 4 : wpb;
+      wpb = wpb < 1 ? 1 : wpb > 3 ? 3 : wpb;
       block = dim3(64 * wpb);
       grid = dim3((nrq + wpb - 1) / wpb, m);
     } else {

@@ -165,7 +165,7 @@ int cthip_gguf_open(void **out, const char *path) {
     v.key = c.str();
     v.type = c.get<uint32_t>();
     if (!c.ok || !skip_value(c, v.type, &v)) return bail("truncated or malformed metadata");
-    if (v.key == "general.alignment" && scalar_size(v.type) >= 1) {
+    if (v.key == "general.alignment" && v.type != 6 && v.type != 7 && v.type != 12 && scalar_size(v.type) >= 1) {
       uint64_t a = 0;
       memcpy(&a, v.data, scalar_size(v.type));
       if (a == 0 || (a & (a - 1))) return bail("general.alignment is not a power of two");
@@ -180,12 +180,16 @@ int cthip_gguf_open(void **out, const char *path) {
     if (!c.ok || t.n_dims > 4) return bail("malformed tensor info");
     uint64_t n = 1;
     for (uint32_t d = 0; d < t.n_dims; d++) {
-      t.dims[d] = (int64_t)c.get<uint64_t>();
-      n *= (uint64_t)t.dims[d];
+      const uint64_t dim = c.get<uint64_t>();
+      // an element count beyond what the file could hold is a malformed header, not a size to multiply on with
+      if (dim > (uint64_t)INT64_MAX || __builtin_mul_overflow(n, dim, &n) || n > (uint64_t)g->size * 32)
+        return bail("implausible tensor dimensions");
+      t.dims[d] = (int64_t)dim;
     }
     t.type = c.get<uint32_t>();
     t.rel_offset = c.get<uint64_t>();
     if (!c.ok) return bail("truncated tensor info");
+    if (t.rel_offset > g->size) return bail("tensor offset lies past the end of the file");
     t.nbytes = tensor_nbytes(t.type, n);
     g->tensors.push_back(t);
   }
@@ -194,7 +198,7 @@ int cthip_gguf_open(void **out, const char *path) {
   for (GGUFTensor &t : g->tensors) {
     const uint64_t off = start + t.rel_offset;
     t.abs_offset = off + (g->alignment - off % g->alignment) % g->alignment;
-    if (t.nbytes && t.abs_offset + t.nbytes > g->size) return bail("tensor data runs past the end of the file");
+    if (t.abs_offset > g->size || t.nbytes > g->size - t.abs_offset) return bail("tensor data runs past the end of the file");
   }
   *out = g;
   return 0;

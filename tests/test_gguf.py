@@ -84,6 +84,18 @@ def test_reader_rejects_malformed_files(tmp_gguf, tmp_path):
     open(tmp_gguf, "wb").write(blob[:40])
     with pytest.raises(HipError):
         gguf.GGUF(tmp_gguf)  # metadata truncated
+    def one_tensor(dims, ggml_type, offset):
+        name = b"t"
+        info = struct.pack("<Q", len(name)) + name + struct.pack("<I", len(dims)) + b"".join(struct.pack("<Q", d) for d in dims)
+        return b"GGUF" + struct.pack("<IQQ", 3, 1, 0) + info + struct.pack("<IQ", ggml_type, offset) + b"\0" * 64
+    for dims, off in [((1 << 62, 8), 0), ((1 << 63,), 0), ((1 << 40,), 0), ((8,), (1 << 64) - 16), ((8,), 1 << 20)]:
+        open(tmp_gguf, "wb").write(one_tensor(dims, 0, off))
+        with pytest.raises(HipError):
+            gguf.GGUF(tmp_gguf)  # element counts / offsets that overflow or leave the file
+    open(tmp_gguf, "wb").write(one_tensor((8,), 0, 0))
+    g = gguf.GGUF(tmp_gguf)
+    assert g.tensor_info[0].shape == (8,)
+    g.close()
     open(tmp_gguf, "wb").write(b"GGUF" + struct.pack("<IQQ", 3, 0, 0))
     g = gguf.GGUF(tmp_gguf)  # empty but valid
     assert len(g.tensor_info) == 0 and g.metadata_kv_count == 0

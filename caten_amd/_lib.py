@@ -66,6 +66,7 @@ PROTOTYPES = {
     "cthip_wmat_destroy": (_i, [_vp]),
     "cthip_wmat_nbytes": (_i64, [_vp]),
     "cthip_wmat_dequant": (_i, [_vp, _vp]),
+    "cthip_wmat_fold_layernorm": (_i, [_vp, _vp, _vp, _vp]),
     "cthip_linear": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _i, _i, _vp, _vp, _f]),
     "cthip_set_option": (_i, [C.c_char_p, _i]),
     "cthip_matmul": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i]),

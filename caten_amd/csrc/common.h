@@ -59,6 +59,10 @@ struct WMat {
   // the single-row kernels request this matrix with the non-temporal hint: set for a matrix that cannot stay in
   // the Infinity Cache between two uses (too large by itself, or one of a model's that together are too large)
   bool stream;
+  // a LayerNorm folded through the product (cthip_wmat_fold_layernorm): fold_s = W.gamma, fold_c = W.beta + bias,
+  // valid for exactly these gamma / beta / bias vectors
+  const float *fold_g = nullptr, *fold_b = nullptr, *fold_bias = nullptr;
+  float *fold_s = nullptr, *fold_c = nullptr;
 };
 // gfx950: 256 MB of Infinity Cache in front of HBM
 static const int64_t kInfinityCacheBytes = 256ll << 20;
@@ -84,6 +88,9 @@ struct GemvArgs {
   // LayerNorm folded through the product (see k_gemv): fold_s[r] = sum_k W[r,k]*gamma[k]; the caller
   // passes sum_k W[r,k]*beta[k] + b[r] as `bias`.  Null = normalise the input first.
   const float *fold_s;
+  // with fold_s: the Linear's own bias (may be null), so that a launch that prefers to normalise the staged
+  // input itself can undo the folding (fold_s = null, bias = bias0)
+  const float *bias0;
   // rows 2r / 2r+1 are a (gate, up) pair: the launch writes silu(gate_r) * up_r to y[r] (rows/2 outputs)
   // instead of the two products.  Needs a variant with at least two rows per wavefront.
   int pair_swiglu;

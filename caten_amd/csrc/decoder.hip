@@ -361,6 +361,7 @@ static int queue_step(Decoder *d, bool with_head, bool embed) {
     a.eps = c.eps;
     a.bias = gpt2 ? L.attn_c : L.attn_b;
     a.fold_s = L.attn_s;
+    a.bias0 = L.attn_b;
     a.y = d->q;
     a.split1 = D;
     a.split2 = D + KD;
@@ -401,6 +402,7 @@ static int queue_step(Decoder *d, bool with_head, bool embed) {
     f.eps = c.eps;
     f.bias = gpt2 ? L.fc_c : L.fc_b;
     f.fold_s = L.fc_s;
+    f.bias0 = L.fc_b;
     f.act = gpt2 ? CTHIP_ACT_GELU : CTHIP_ACT_NONE;
     f.pair_swiglu = L.fc_pairs ? 1 : 0;
     f.y = d->h;
@@ -434,6 +436,7 @@ static int queue_head(Decoder *d) {
   o.eps = c.eps;
   o.bias = d->lm_c;
   o.fold_s = d->lm_s;
+  o.bias0 = nullptr;
   o.y = d->logits;
   o.x_stride = c.dim;
   o.y_stride = c.vocab;

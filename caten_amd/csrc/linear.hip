@@ -405,18 +405,362 @@ __device__ __forceinline__ void coop_fold(const GemvArgs &a, const float *__rest
   s2_out = block_sum(s2);  // its barriers also publish xs
 }
 
+// Sixteen bytes that stay zero: lanes with nothing to fetch point their requests here, so that every
+// lane issues the same loads and no request sits behind a branch (the compiler can then wait for
+// exactly the tile it needs instead of for everything in flight).  Not const: a select between a
+// kernel-argument pointer and a constant would be addressed through the flat aperture.
+__device__ __align__(16) unsigned g_gemv_zeros[4];
+
+template <bool NT>
+__device__ __forceinline__ uint4 load_chunk(const uint4 *src) {
+  if (NT)
+    return make_uint4(__builtin_nontemporal_load(&src->x), __builtin_nontemporal_load(&src->y),
+                      __builtin_nontemporal_load(&src->z), __builtin_nontemporal_load(&src->w));
+  return *src;
+}
+
+// The looping launches (PD > 1 tiles in flight per wavefront).  The kernel is a stream: its time is the
+// first-byte latency plus bytes / bandwidth only if a new tile is requested whenever one has been
+// consumed, so (i) every request is unconditional -- rows past the end repeat the last row and are never
+// stored, chunks past the end of a row read the zero block -- and the loop body is the same on every
+// pass (a separate last pass requests nothing), which lets the wait before tile p count exactly the
+// PD - 1 tiles requested after it; (ii) the input side (vector, gamma or the gate's partner) is
+// requested BEFORE the weight ring: loads return in order, so a vector requested behind four tiles
+// would hold back the first product until all four had arrived.
+template <int TYPE, int G, int KC, int PD, bool NT, bool EPI, bool DIRECT>
+__device__ __forceinline__ void gemv_ring(const GemvArgs &a, float *xs_lds, float *red) {
+  constexpr int XPC = Fmt<TYPE>::XPC;
+  constexpr int RPW = 64 / G;
+  constexpr bool QUANT = (TYPE == CTHIP_Q8_0 || TYPE == CTHIP_Q4_0);
+  constexpr int SG = 4;  // float4 per thread of the staged vector that are requested ahead of the weights
+  constexpr int nthr = 256;  // what the looping launches use (reading blockDim would cost a memory round trip up front)
+  constexpr int waves_per_block = nthr >> 6;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int g = lane / G, l = lane % G;
+  const int wave = blockIdx.x * waves_per_block + (tid >> 6);
+  const int total_waves = gridDim.x * waves_per_block;
+  const int nchunks = a.cols / XPC;
+  const int m = blockIdx.y;
+  const float *__restrict__ x = a.x + (int64_t)m * a.x_stride;
+  const uint4 *__restrict__ qp = (const uint4 *)a.q;
+  const int64_t row_chunks = nchunks;
+  const int scales_per_row = a.cols >> 5;
+  const int nrq = (a.rows + RPW - 1) / RPW;
+  const float *zf = (const float *)g_gemv_zeros;
+  const uint4 *z16 = (const uint4 *)g_gemv_zeros;
+  const unsigned short *zh = (const unsigned short *)g_gemv_zeros;
+  const bool folded = (a.pro == CTHIP_PRO_RMSNORM) || (a.pro == CTHIP_PRO_LAYERNORM && a.fold_s != nullptr);
+  const bool swiglu = a.pro == CTHIP_PRO_SWIGLU;
+  const bool coop = a.stage_x != 0;
+  const int posv = a.pos ? a.pos[0] : 0;
+  const bool layernorm = a.pro == CTHIP_PRO_LAYERNORM;
+  const int n4 = a.cols >> 2;
+  // a LayerNorm that is not folded is applied while staging, when a thread's share of the vector stays in registers
+  const bool direct = DIRECT && coop && layernorm && !a.fold_s && n4 <= SG * nthr;
+  // staged inputs whose first SG * blockDim float4 are requested ahead of the weights
+  const bool early = coop && (folded || swiglu || a.pro == CTHIP_PRO_NONE || direct);
+
+  // ---- (1) the input side ----
+  float4 sv[SG], su[SG], sb[SG];
+  float xr[KC][XPC];
+  float gr[QUANT ? 1 : KC][QUANT ? 1 : XPC];  // gamma of an unstaged folded norm (fp32 / fp16 weights)
+  const float4 *x4 = (const float4 *)x;
+  // the second operand of the staging: the gate's partner, gamma, or (unused) the vector again
+  const float4 *u4 = swiglu ? (const float4 *)(x + a.cols) : (layernorm || folded) && a.norm_g ? (const float4 *)a.norm_g : x4;
+  const float4 *b4 = (direct && a.norm_b) ? (const float4 *)a.norm_b : x4;  // beta of a LayerNorm applied here
+  if (early) {
+#pragma unroll
+    for (int k = 0; k < SG; k++) {
+      int i = tid + k * nthr;
+      i = i < n4 ? i : n4 - 1;
+      sv[k] = x4[i];
+      su[k] = u4[i];
+      if constexpr (DIRECT) sb[k] = b4[i];  // unconditional (the vector again when unused): a request behind a branch would make every later wait a wait for everything
+    }
+  } else if (!coop) {
+#pragma unroll
+    for (int j = 0; j < KC; j++) {
+      const int c = l + G * j;
+      const bool ok = c < nchunks;
+#pragma unroll
+      for (int t = 0; t < XPC / 4; t++) {
+        const float4 v = *(ok ? (const float4 *)(x + (int64_t)c * XPC + 4 * t) : (const float4 *)g_gemv_zeros);
+        xr[j][4 * t + 0] = v.x;
+        xr[j][4 * t + 1] = v.y;
+        xr[j][4 * t + 2] = v.z;
+        xr[j][4 * t + 3] = v.w;
+        if (!QUANT) {
+          const float4 gv = *((ok && folded && a.norm_g) ? (const float4 *)(a.norm_g + (int64_t)c * XPC + 4 * t)
+                                                         : (const float4 *)g_gemv_zeros);
+          gr[QUANT ? 0 : j][QUANT ? 0 : 4 * t + 0] = gv.x;
+          gr[QUANT ? 0 : j][QUANT ? 0 : 4 * t + 1] = gv.y;
+          gr[QUANT ? 0 : j][QUANT ? 0 : 4 * t + 2] = gv.z;
+          gr[QUANT ? 0 : j][QUANT ? 0 : 4 * t + 3] = gv.w;
+        }
+      }
+    }
+  }
+
+  // ---- (2) the weight ring ----
+  auto request = [&](int rq, uint4 *w, unsigned short *s, float &epi) {
+    int row = rq * RPW + g;
+    row = row < a.rows ? row : a.rows - 1;
+#pragma unroll
+    for (int j = 0; j < KC; j++) {
+      const int c = l + G * j;
+      const bool ok = c < nchunks;
+      w[j] = load_chunk<NT>(ok ? qp + (int64_t)row * row_chunks + c : z16);
+      if (QUANT) {
+        const int sidx = (TYPE == CTHIP_Q8_0) ? (c >> 1) : c;
+        s[j] = *(ok ? a.d + (int64_t)row * scales_per_row + sidx : zh);
+      }
+    }
+    // the epilogue operands of the row travel with its weights, in ONE request: the first three lanes of the
+    // row's group fetch bias, residual and fold term, and the group's first lane collects them with two lane
+    // shifts when it stores.  Lanes with nothing to fetch repeat a neighbour's address: a common dummy line
+    // would be re-fetched by every tile of every wavefront and its L2 channel would hold all of them up.
+    if (EPI) {
+      const float *pb = a.bias ? a.bias + row : nullptr;
+      const float *pr = a.residual ? a.residual + (int64_t)m * a.y_stride + row : nullptr;
+      const float *pf = a.fold_s ? a.fold_s + row : nullptr;
+      const float *any = pb ? pb : pr ? pr : pf;  // one of them exists, or the launcher takes the kernel without EPI
+      epi = *(l == 0 ? (pb ? pb : any) : l == 1 ? (pr ? pr : any) : l == 2 ? (pf ? pf : any) : any);
+    }
+  };
+  uint4 wt[PD][KC];
+  unsigned short st[PD][KC];
+  float epi_t[PD];
+#pragma unroll
+  for (int p = 0; p < PD; p++) epi_t[p] = 0.0f;
+  const int own = wave < nrq ? wave : nrq - 1;  // what a slot without a tile requests: lines this wavefront fetches anyway
+  // Only the first tile goes out before the staged input is picked up: requests are issued in program order and
+  // a compute unit accepts them no faster than earlier ones are answered, so the whole ring in front of the
+  // staging code would hold that code back until most of the ring had arrived.
+  constexpr int PRE = 1;
+#pragma unroll
+  for (int p = 0; p < PRE; p++) {
+    const int rq = wave + p * total_waves;
+    request(rq < nrq ? rq : own, wt[p], st[p], epi_t[p]);
+  }
+
+  // a norm that is not folded is applied by the whole workgroup (its own loads wait for the tile above as well)
+  if (coop && !early) coop_prologue(a, x, xs_lds, red, true);
+
+  // ---- (3) the input side arrives ----
+  // Statistics of a folded norm over a staged vector.  No value is shared up front (a common shift, say the
+  // first element, would be one more round trip in front of everything): every thread sums its own elements
+  // shifted by its own first one, and the (count, mean, squared deviation) triples are merged exactly,
+  // thread -> wavefront by lane shuffles, wavefront -> workgroup through LDS.
+  float mu = 0.0f, rstd = 1.0f;
+  if (early) {
+    float s1 = 0.0f, s2 = 0.0f, cnt = 0.0f;
+    const float pivot = layernorm ? sv[0].x : 0.0f;  // this thread's first element (threads without one sum nothing)
+    auto put = [&](int i, const float4 v, const float4 u) {
+      if (swiglu) {
+        ((float4 *)xs_lds)[i] = make_float4(ct_silu(v.x) * u.x, ct_silu(v.y) * u.y, ct_silu(v.z) * u.z, ct_silu(v.w) * u.w);
+      } else if (folded || direct) {
+        const float4 gm = a.norm_g ? u : make_float4(1.f, 1.f, 1.f, 1.f);
+        const float d0 = v.x - pivot, d1 = v.y - pivot, d2 = v.z - pivot, d3 = v.w - pivot;
+        s1 += (d0 + d1) + (d2 + d3);
+        s2 = fmaf(d0, d0, s2);
+        s2 = fmaf(d1, d1, s2);
+        s2 = fmaf(d2, d2, s2);
+        s2 = fmaf(d3, d3, s2);
+        cnt += 4.0f;
+        // (a norm applied here writes its values once the statistics are known)
+        if (!direct) ((float4 *)xs_lds)[i] = make_float4(v.x * gm.x, v.y * gm.y, v.z * gm.z, v.w * gm.w);
+      } else {
+        ((float4 *)xs_lds)[i] = v;
+      }
+    };
+#pragma unroll
+    for (int k = 0; k < SG; k++) {
+      const int i = tid + k * nthr;
+      if (i < n4) put(i, sv[k], su[k]);
+    }
+    // longer vectors: the rest is requested behind the first tiles
+    for (int i = tid + SG * nthr; i < n4; i += nthr) put(i, x4[i], u4[i]);
+    if ((folded || direct) && layernorm) {
+      const float inv = cnt > 0.0f ? 1.0f / cnt : 0.0f;
+      const float mean_t = cnt > 0.0f ? pivot + s1 * inv : 0.0f;
+      const float n_w = wave_sum(cnt);
+      const float mean_w = wave_sum(cnt * mean_t) / fmaxf(n_w, 1.0f);
+      const float dm = mean_t - mean_w;
+      const float m2_w = wave_sum(s2 - s1 * s1 * inv + cnt * dm * dm);
+      if (lane == 0) {
+        red[tid >> 6] = n_w;
+        red[8 + (tid >> 6)] = mean_w;
+        red[16 + (tid >> 6)] = m2_w;
+      }
+    } else if (folded) {  // RMSNorm: the plain sum of squares
+      s2 = wave_sum(s2);
+      if (lane == 0) red[tid >> 6] = s2;
+    }
+    __syncthreads();  // publishes the staged vector and the per-wavefront statistics
+    if (folded || direct) {
+      const float inv_n = 1.0f / (float)a.cols;
+      float m2 = 0.0f;
+      if (layernorm) {
+        float sum = 0.0f;
+        for (int w = 0; w < waves_per_block; w++) sum += red[w] * red[8 + w];
+        mu = sum * inv_n;
+        for (int w = 0; w < waves_per_block; w++) {
+          const float dw = red[8 + w] - mu;
+          m2 += red[16 + w] + red[w] * dw * dw;
+        }
+      } else {
+        for (int w = 0; w < waves_per_block; w++) m2 += red[w];
+      }
+      rstd = 1.0f / sqrtf(fmaxf(m2 * inv_n, 0.0f) + a.eps);
+    }
+    if (direct) {
+      // y = ((x - mean) * rstd) * gamma + beta, as the unfused LayerNorm item computes it; nothing is left for the epilogue
+#pragma unroll
+      for (int k = 0; k < SG; k++) {
+        const int i = tid + k * nthr;
+        if (i < n4) {
+          const float4 v = sv[k];
+          const float4 gm = a.norm_g ? su[k] : make_float4(1.f, 1.f, 1.f, 1.f);
+          const float4 bt = a.norm_b ? sb[k] : make_float4(0.f, 0.f, 0.f, 0.f);
+          ((float4 *)xs_lds)[i] = make_float4((v.x - mu) * rstd * gm.x + bt.x, (v.y - mu) * rstd * gm.y + bt.y,
+                                              (v.z - mu) * rstd * gm.z + bt.z, (v.w - mu) * rstd * gm.w + bt.w);
+        }
+      }
+      mu = 0.0f;
+      rstd = 1.0f;
+      __syncthreads();
+    }
+  }
+  if (coop) {
+#pragma unroll
+    for (int j = 0; j < KC; j++) {
+      const int c = l + G * j;
+      const bool ok = c < nchunks;
+#pragma unroll
+      for (int t = 0; t < XPC / 4; t++) {
+        const float4 v = ok ? *(const float4 *)(xs_lds + (int64_t)c * XPC + 4 * t) : make_float4(0.f, 0.f, 0.f, 0.f);
+        xr[j][4 * t + 0] = v.x;
+        xr[j][4 * t + 1] = v.y;
+        xr[j][4 * t + 2] = v.z;
+        xr[j][4 * t + 3] = v.w;
+      }
+    }
+  }
+#pragma unroll
+  for (int p = PRE; p < PD; p++) {
+    const int rq = wave + p * total_waves;
+    request(rq < nrq ? rq : own, wt[p], st[p], epi_t[p]);
+  }
+  if (folded && !coop) {
+    // every group of G lanes holds the whole vector in registers: mean, then squared deviations, then gamma
+    const float inv_n = 1.0f / (float)a.cols;
+    if (layernorm) {
+      float s1 = 0.0f;
+#pragma unroll
+      for (int j = 0; j < KC; j++)
+#pragma unroll
+        for (int e = 0; e < XPC; e++) s1 += xr[j][e];  // lanes past the end hold zeros
+      mu = group_sum<G>(s1) * inv_n;
+    }
+    float s2 = 0.0f;
+    {
+#pragma unroll
+      for (int j = 0; j < KC; j++) {
+        const int c = l + G * j;
+        const bool ok = c < nchunks;
+#pragma unroll
+        for (int t = 0; t < XPC / 4; t++) {
+          float gg[4] = {1.f, 1.f, 1.f, 1.f};
+          if (QUANT) {  // (the launcher stages quantised folded launches; kept for completeness)
+            if (ok && a.norm_g) {
+              const float4 gv = *(const float4 *)(a.norm_g + (int64_t)c * XPC + 4 * t);
+              gg[0] = gv.x, gg[1] = gv.y, gg[2] = gv.z, gg[3] = gv.w;
+            }
+          } else if (a.norm_g) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) gg[e] = gr[QUANT ? 0 : j][QUANT ? 0 : 4 * t + e];
+          }
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            const float d = ok ? xr[j][4 * t + e] - mu : 0.0f;
+            s2 = fmaf(d, d, s2);
+            xr[j][4 * t + e] *= gg[e];
+          }
+        }
+      }
+    }
+    rstd = 1.0f / sqrtf(group_sum<G>(s2) * inv_n + a.eps);
+  }
+  float xs[KC];
+#pragma unroll
+  for (int j = 0; j < KC; j++) {
+    float s = 0.0f;
+    if (TYPE == CTHIP_Q4_0) {
+#pragma unroll
+      for (int e = 0; e < XPC; e++) s += xr[j][e];
+    }
+    xs[j] = s;
+  }
+
+  // ---- (4) stream the rows: slot p of the ring holds tile base + p * total_waves ----
+  float best_v = -INFINITY;
+  int best_i = 0x7fffffff;
+  auto consume = [&](int p, int rq) {
+    float acc = 0.0f;
+#pragma unroll
+    for (int j = 0; j < KC; j++) {
+      const float scale = QUANT ? half_bits_to_float(st[p][j]) : 1.0f;
+      acc += chunk_dot<TYPE>(wt[p][j], scale, xr[j], xs[j]);
+    }
+    acc = group_sum<G>(acc);
+    // valid in the group's first lane, which is the one that stores
+    const float bias = (EPI && a.bias) ? epi_t[p] : 0.0f;
+    const float resid = (EPI && a.residual) ? dpp_f<0x101>(epi_t[p]) : 0.0f;  // row_shl:1
+    const float fs = (EPI && a.fold_s) ? dpp_f<0x102>(epi_t[p]) : 0.0f;       // row_shl:2
+    if (folded) acc = rstd * (acc - mu * fs);
+    const int row = rq * RPW + g;
+    if (RPW >= 2 && a.pair_swiglu) {
+      // SwiGLU across the (gate, up) row pair held by neighbouring lane groups
+      const float mine = acc + bias;
+      const float other = __shfl_xor(mine, G & 63, 64);
+      if (l == 0 && (g & 1) == 0 && row < a.rows) a.y[(int64_t)m * a.y_stride + (row >> 1)] = ct_silu(mine) * other;
+    } else if (l == 0 && row < a.rows) {
+      const float v = gemv_store(a, m, row, acc, posv, bias, resid);
+      argmax_merge(best_v, best_i, v, row);
+    }
+  };
+  const int stride = PD * total_waves;
+  int base = wave;
+  for (; base + stride < nrq; base += stride) {  // every slot holds a tile; slot 0 has a successor
+#pragma unroll
+    for (int p = 0; p < PD; p++) {
+      const int rq = base + p * total_waves;
+      consume(p, rq);
+      const int nxt = rq + stride;
+      request(nxt < nrq ? nxt : rq, wt[p], st[p], epi_t[p]);
+    }
+  }
+#pragma unroll
+  for (int p = 0; p < PD; p++) {
+    const int rq = base + p * total_waves;
+    if (rq < nrq) consume(p, rq);  // wavefront-uniform
+  }
+  if (a.am_val) gemv_argmax_tail(a, wave, lane, best_v, best_i);
+}
+
 // PD = weight tiles a wavefront keeps in flight: 1 for the small, latency-bound launches (one tile
 // per wavefront), 4 for the large ones, whose throughput is bytes-in-flight / memory latency.
 // NT: the weights are requested with the non-temporal hint.  A model whose weights exceed the 256 MB Infinity
 // Cache streams all of them from HBM every step whatever the hint; without it the stream also evicts the
 // vectors, fold terms and KV rows that the step does reuse.
-template <int TYPE, int G, int KC, int PD, bool NT>
+template <int TYPE, int G, int KC, int PD, bool NT, bool EPI = false, bool DIRECT = false>
 __global__ __launch_bounds__(256) void k_gemv(GemvArgs a) {
   constexpr int XPC = Fmt<TYPE>::XPC;
   constexpr int RPW = 64 / G;  // rows per wavefront per iteration
   constexpr bool QUANT = (TYPE == CTHIP_Q8_0 || TYPE == CTHIP_Q4_0);
   extern __shared__ float xs_lds[];  // a.cols floats when a prologue is fused
-  __shared__ float red[4];
+  __shared__ float red[24];
   const int lane = threadIdx.x & 63;
   const int g = lane / G, l = lane % G;
   const int waves_per_block = blockDim.x >> 6;
@@ -466,6 +810,10 @@ __global__ __launch_bounds__(256) void k_gemv(GemvArgs a) {
     }
   };
 
+  if constexpr (PD > 1) {
+    gemv_ring<TYPE, G, KC, PD, NT, EPI, DIRECT>(a, xs_lds, red);
+    return;
+  }
   // Everything this wavefront needs from memory is requested before any arithmetic so the
   // latencies overlap: position, the first weight tiles, then the input vector.
   const int posv = a.pos ? a.pos[0] : 0;
@@ -668,13 +1016,17 @@ __global__ __launch_bounds__(256) void k_prologue(float *__restrict__ out, const
 typedef void (*gemv_fn)(GemvArgs);
 struct GemvVariant {
   int type, G, KC;
-  gemv_fn fn[2];       // large launches: [0] cached weights, [1] streamed (non-temporal) weights
-  gemv_fn fn_small[2]; // small, latency-bound launches
+  gemv_fn fn[2];       // looping launches: [0] cached weights, [1] streamed (non-temporal) weights
+  gemv_fn fn_epi[2];   // the same with per-row epilogue operands (bias, residual, fold term) travelling in the ring
+  gemv_fn fn_direct[2];  // looping, no epilogue operands, a LayerNorm applied to the staged input
+  gemv_fn fn_small[2]; // one tile per wavefront: latency-bound launches
 };
 // large launches keep about 12 sixteen-byte loads per lane in flight
 #define PD_OF(KC) (KC >= 12 ? 1 : KC >= 6 ? 2 : 4)
 #define V(T, G, KC)                                                                           \
   {T, G, KC, {k_gemv<T, G, KC, PD_OF(KC), false>, k_gemv<T, G, KC, PD_OF(KC), true>},         \
+   {k_gemv<T, G, KC, PD_OF(KC), false, PD_OF(KC) != 1>, k_gemv<T, G, KC, PD_OF(KC), true, PD_OF(KC) != 1>}, \
+   {k_gemv<T, G, KC, PD_OF(KC), false, false, PD_OF(KC) != 1>, k_gemv<T, G, KC, PD_OF(KC), true, false, PD_OF(KC) != 1>}, \
    {k_gemv<T, G, KC, 1, false>, k_gemv<T, G, KC, 1, true>}}
 static const GemvVariant kVariants[] = {
     V(CTHIP_Q8_0, 16, 1), V(CTHIP_Q8_0, 16, 2), V(CTHIP_Q8_0, 16, 3), V(CTHIP_Q8_0, 16, 4),
@@ -774,7 +1126,7 @@ int launch_gemv(const WMat *w, GemvArgs a, int m) {
     const size_t lds = stage ? sizeof(float) * (size_t)a.cols : 0;
     if (lds > 64 * 1024) return fail(CTHIP_E_UNSUPPORTED, "gemv: %d input features exceed the LDS staging buffer", a.cols);
     a.stage_x = stage ? 1 : 0;
-    bool small;
+    bool small, direct = false;
     if (!stage && nrq <= 2048) {
       // small matrices are pure latency: one tile per wavefront, one wavefront per workgroup, spread
       // over as many compute units as there are tiles
@@ -820,12 +1172,24 @@ int launch_gemv(const WMat *w, GemvArgs a, int m) {
       const int iters = (nrq + wanted - 1) / wanted;
       const int waves = (nrq + iters - 1) / iters;
       grid = dim3((waves + 3) / 4, m);
+      // the ring requests all its slots unconditionally: a wavefront with a single tile takes the kernel without one
+      if (iters == 1) small = true;
+      // A looping launch normalises the staged vector itself rather than carrying the fold terms: two more
+      // operands per row in the weight ring hold the stream up more than the second barrier of the staging costs
+      // (GPT-2 lm_head: 11.0 us folded, 10.0 us with neither)
+      if (!small && stage && a.pro == CTHIP_PRO_LAYERNORM && a.fold_s && !a.bias0 && !a.residual && a.cols <= 4096) {
+        a.fold_s = nullptr;
+        a.bias = nullptr;
+      }
+      direct = !small && stage && a.pro == CTHIP_PRO_LAYERNORM && !a.fold_s && !a.bias && !a.residual && a.cols <= 4096;
     }
     const int nwaves = (int)(grid.x * (block.x / 64));
     if (a.am_val && nwaves > kGemvMaxWaves)
       return fail(CTHIP_E_UNSUPPORTED, "gemv: %d wavefronts exceed the argmax scratch", nwaves);
     const int nt = s.gemv_stream < 0 ? (w->stream ? 1 : 0) : s.gemv_stream;
-    hipLaunchKernelGGL(small ? v->fn_small[nt] : v->fn[nt], grid, block, lds, s.stream, a);
+    const bool epi = a.bias || a.residual || a.fold_s;
+    hipLaunchKernelGGL(small ? v->fn_small[nt] : epi ? v->fn_epi[nt] : direct ? v->fn_direct[nt] : v->fn[nt], grid, block, lds,
+                       s.stream, a);
     CTHIP_LAUNCH_CHECK();
     if (a.am_val) {
       hipLaunchKernelGGL(k_argmax_finish, dim3(1), dim3(256), 0, s.stream, a, nwaves);
@@ -956,7 +1320,37 @@ int cthip_wmat_destroy(void *wmat) {
   WMat *w = (WMat *)wmat;
   cthip_free(w->q);
   cthip_free(w->d);
+  if (w->fold_s) cthip_free(w->fold_s);
+  if (w->fold_c) cthip_free(w->fold_c);
   delete w;
+  return 0;
+}
+
+int cthip_wmat_fold_layernorm(void *wmat, const float *gamma, const float *beta, const float *bias) {
+  CTHIP_REQUIRE_INIT();
+  CTHIP_ARG(wmat != nullptr && gamma != nullptr && beta != nullptr);
+  WMat *w = (WMat *)wmat;
+  if (!gemv_is_direct(w)) return fail(CTHIP_E_UNSUPPORTED, "cthip_wmat_fold_layernorm: no single-row kernel covers %lld columns", (long long)w->cols);
+  int rc;
+  if (!w->fold_s && (rc = cthip_alloc((void **)&w->fold_s, sizeof(float) * (size_t)w->rows))) return rc;
+  if (!w->fold_c && (rc = cthip_alloc((void **)&w->fold_c, sizeof(float) * (size_t)w->rows))) return rc;
+  w->fold_g = w->fold_b = w->fold_bias = nullptr;  // not valid until both products are queued
+  GemvArgs s = {};  // S = W . gamma
+  s.x = gamma;
+  s.y = w->fold_s;
+  s.x_stride = w->cols;
+  s.y_stride = w->rows;
+  if ((rc = launch_gemv(w, s, 1))) return rc;
+  GemvArgs c = {};  // C = W . beta + bias
+  c.x = beta;
+  c.bias = bias;
+  c.y = w->fold_c;
+  c.x_stride = w->cols;
+  c.y_stride = w->rows;
+  if ((rc = launch_gemv(w, c, 1))) return rc;
+  w->fold_g = gamma;
+  w->fold_b = beta;
+  w->fold_bias = bias;
   return 0;
 }
 
@@ -1013,6 +1407,11 @@ int cthip_linear(float *y, const void *wmat, const float *x, int m, const float 
   a.eps = eps;
   a.x_stride = (prologue == CTHIP_PRO_SWIGLU) ? 2 * w->cols : w->cols;
   a.y_stride = w->rows;
+  if (prologue == CTHIP_PRO_LAYERNORM && w->fold_g && w->fold_g == norm_g && w->fold_b == norm_b && w->fold_bias == bias) {
+    a.fold_s = w->fold_s;  // the norm goes through the product: see k_gemv
+    a.bias = w->fold_c;
+    a.bias0 = bias;
+  }
   return launch_gemv(w, a, m);
 }
 

@@ -93,6 +93,25 @@ class WeightMatrix:
         _lib.check(_lib.load().cthip_wmat_dequant(self.handle, out.ptr))
         return out.numpy()
 
+    def fold_layernorm(self, gamma, beta, bias=None) -> None:
+        """cthip_wmat_fold_layernorm: keeps device copies of gamma / beta / bias (the fold is keyed on their
+        addresses) and prepares LayerNorm(gamma, beta) in front of this Linear to go through the product."""
+        self._fold = (_dev(np.ascontiguousarray(gamma, np.float32)), _dev(np.ascontiguousarray(beta, np.float32)),
+                      _dev(None if bias is None else np.ascontiguousarray(bias, np.float32)))
+        dg, db, dbias = self._fold
+        _lib.check(_lib.load().cthip_wmat_fold_layernorm(self.handle, dg.ptr, db.ptr, _p(dbias)))
+
+    def linear_folded(self, x, act=None, eps: float = 1e-5) -> np.ndarray:
+        """act(LayerNorm(x) @ W^T + bias) with the vectors given to fold_layernorm (fewer than 8 input rows)."""
+        dg, db, dbias = self._fold
+        x = np.ascontiguousarray(x, np.float32)
+        m = x.size // self.cols
+        dx = _dev(x)
+        y = DeviceArray(x.shape[:-1] + (self.rows,), np.float32)
+        _lib.check(_lib.load().cthip_linear(y.ptr, self.handle, dx.ptr, m, _p(dbias), None, _ACT[act],
+                                            _PRO["layernorm"], dg.ptr, db.ptr, eps))
+        return y.numpy()
+
     def free(self):
         if self.handle:
             _lib.load().cthip_wmat_destroy(self.handle)

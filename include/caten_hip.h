@@ -127,6 +127,14 @@ int cthip_wmat_destroy(void *wmat);
 int64_t cthip_wmat_nbytes(const void *wmat);
 /* Expands the packed planes to fp32 (rows*cols); bit-exact with cthip_dequant of the raw bytes. */
 int cthip_wmat_dequant(const void *wmat, float *out);
+/* Prepares a LayerNorm (source/nn/normalization.lisp:39-58) in front of this Linear (source/nn/linear.lisp:3-17)
+ * to be carried through the product:  W.(((x-mu)*rstd)*gamma + beta) + bias = rstd*(W.(gamma*x) - mu*S) + C  with
+ * S = W.gamma and C = W.beta + bias computed here, once (two products over the matrix, queued on the stream).
+ * Afterwards cthip_linear(m < 8, CTHIP_PRO_LAYERNORM) called with these SAME gamma / beta / bias pointers needs mu
+ * and rstd only in its epilogue, so the statistics overlap the weight stream; this is how a decoder session runs
+ * its c_attn, c_fc and lm_head.  The terms are a snapshot: call again after changing gamma, beta or bias
+ * (`bias` may be NULL).  Other argument combinations keep normalising the input first. */
+int cthip_wmat_fold_layernorm(void *wmat, const float *gamma, const float *beta, const float *bias);
 
 /* ================================================================== */
 /* Hand-written fused items (what Caten's Schedule-Items compute)      */

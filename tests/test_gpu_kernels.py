@@ -213,6 +213,31 @@ def test_gemv_streamed_weights_give_the_same_bits(ops, kind):
         _lib.check(lib.cthip_set_option(b"gemv_stream_weights", 2))
 
 
+@pytest.mark.parametrize("kind", ["q8_0", "q4_0", "f32", "f16"])
+def test_layernorm_folded_through_the_product(ops, oracle, kind):
+    """cthip_wmat_fold_layernorm: LayerNorm carried through the product (S = W.gamma, C = W.beta + bias) gives the
+    Linear of the normalised input, on one-tile-per-wavefront launches, on looping ones (which normalise the staged
+    vector themselves when no per-row operand is left) and with several input rows; a call with other vectors
+    keeps normalising first."""
+    from caten_amd.llm import Tensor
+    rng = np.random.default_rng(31)
+    for rows, cols, with_bias in ((2304, 768, True), (9000, 768, False), (9000, 768, True), (1500, 2048, True)):
+        w = rng.normal(0, 0.02, (rows, cols)).astype(np.float32)
+        g = rng.normal(1, 0.05, cols).astype(np.float32)
+        b = rng.normal(0, 0.05, cols).astype(np.float32)
+        bias = rng.normal(0, 0.1, rows).astype(np.float32) if with_bias else None
+        t = Tensor.from_f32(w, kind)
+        wd = oracle.dequant(kind, t.raw, w.size).reshape(rows, cols)
+        wm = ops.WeightMatrix(kind, t.raw, rows, cols)
+        wm.fold_layernorm(g, b, bias)
+        for m in (1, 3):
+            x = rng.normal(0.3, 1.5, (m, cols)).astype(np.float32)
+            want = oracle.linear(oracle.layernorm(x, g, b), wd, bias)
+            close(wm.linear_folded(x), want, rtol=2e-3, atol=2e-4)
+            close(ops.linear(x, wm, bias=bias, prologue="layernorm", norm_g=g, norm_b=b), want, rtol=2e-3, atol=2e-4)
+        wm.free()
+
+
 def test_gemv_fallback_shapes_with_prologue(ops, oracle):
     from caten_amd.llm import Tensor
     rng = np.random.default_rng(22)

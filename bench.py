@@ -26,7 +26,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # (profiles/), scaled by a copy kernel of known size; None where it has not been measured.
-TRAFFIC_BYTES = {("gpt2", "q8_0"): 41730519}  # profiles/gemv_q8_0_lm_head_pmc.txt
+TRAFFIC_BYTES = {("gpt2", "q8_0"): 41965322}  # profiles/gemv_q8_0_lm_head_pmc.txt
 
 
 def cpu_baseline(cfg, weights, prompt, budget_s, kind, llama):
@@ -149,18 +149,19 @@ def main():
     wm = ops.WeightMatrix(args.kind, t.raw, V, D)
     dx = ops.DeviceArray.from_numpy(np.random.default_rng(1).normal(size=D).astype(np.float32))
     dg = ops.DeviceArray.from_numpy(weights["norm_w" if llama else "lnf_g"])
-    db = ops.DeviceArray.from_numpy(np.zeros(D, np.float32) if llama else weights["lnf_b"])
+    db = None if llama else ops.DeviceArray.from_numpy(weights["lnf_b"])
+    pro = _lib.PRO_RMSNORM if llama else _lib.PRO_LAYERNORM  # the final norm of the model, fused as the decode step fuses it
     dy = ops.DeviceArray((V,), np.float32)
     reps = 200
     for _ in range(20):
-        _lib.check(lib.cthip_linear(dy.ptr, wm.handle, dx.ptr, 1, None, None, 0, _lib.PRO_LAYERNORM, dg.ptr, db.ptr, 1e-5))
+        _lib.check(lib.cthip_linear(dy.ptr, wm.handle, dx.ptr, 1, None, None, 0, pro, dg.ptr, db.ptr if db else None, 1e-5))
     _lib.check(lib.cthip_sync())
     _lib.check(lib.cthip_timer_start())
     for _ in range(reps):
-        _lib.check(lib.cthip_linear(dy.ptr, wm.handle, dx.ptr, 1, None, None, 0, _lib.PRO_LAYERNORM, dg.ptr, db.ptr, 1e-5))
+        _lib.check(lib.cthip_linear(dy.ptr, wm.handle, dx.ptr, 1, None, None, 0, pro, dg.ptr, db.ptr if db else None, 1e-5))
     _lib.check(lib.cthip_timer_stop(C.byref(ms)))
     gemv_us = ms.value * 1e3 / reps
-    gemv_bytes = wm.nbytes + 4 * (3 * D + V)  # packed weights + x, gamma, beta + logits
+    gemv_bytes = wm.nbytes + 4 * ((2 if llama else 3) * D + V)  # packed weights + x, gamma (, beta) + logits
     achieved = gemv_bytes / (gemv_us * 1e-6) / 1e9
 
     res = {
@@ -176,7 +177,7 @@ def main():
                    "positions": f"{min(positions)}..{max(positions)}"},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": TRAFFIC_BYTES.get((args.model, args.kind)),
-                     "kernel": f"cthip::k_gemv<{args.kind}> on lm_head ({V}x{D}) with the ln_f prologue",
+                     "kernel": f"cthip::k_gemv<{args.kind}> on lm_head ({V}x{D}) with the {'RMSNorm' if llama else 'ln_f'} prologue",
                      "bytes_per_launch": gemv_bytes, "us_per_launch": gemv_us,
                      "step": {"bytes": step_bytes, "us": step_us, "achieved": step_gbs,
                               "frac": step_gbs / HBM_PEAK_GBS,

@@ -128,7 +128,22 @@ __global__ __launch_bounds__(256) void k_argmax_finish(GemvArgs a, int nparts) {
   }
   float bv = -INFINITY;
   int bi = 0x7fffffff;
-  for (int i = threadIdx.x; i < nparts; i += 256) argmax_merge(bv, bi, a.am_val[i], a.am_idx[i]);
+  // eight partials per thread are requested together (clamped addresses, no request behind a branch), so the
+  // 1 800 partials of a GPT-2 lm_head cost one memory round trip instead of seven dependent ones
+  for (int base = 0; base < nparts; base += 8 * 256) {
+    float pv[8];
+    int pi[8];
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+      const int i = base + threadIdx.x + 256 * k;
+      const int ic = i < nparts ? i : nparts - 1;
+      pv[k] = a.am_val[ic];
+      pi[k] = a.am_idx[ic];
+    }
+#pragma unroll
+    for (int k = 0; k < 8; k++)
+      if (base + threadIdx.x + 256 * k < nparts) argmax_merge(bv, bi, pv[k], pi[k]);
+  }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) argmax_merge(bv, bi, __shfl_xor(bv, o, 64), __shfl_xor(bi, o, 64));
   if ((threadIdx.x & 63) == 0) {

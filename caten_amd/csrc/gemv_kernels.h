@@ -215,7 +215,7 @@ __device__ __forceinline__ void coop_prologue(const GemvArgs &a, const float *__
 
 // Folded norm with a staged input: the workgroup writes gamma * x into LDS once and reduces the
 // shifted sums  s1 = sum(x - pivot), s2 = sum((x - pivot)^2)  over the whole vector, so no wavefront
-// loads gamma or repeats the statistics.  xs must hold a.cols floats; blockDim.x <= 256.
+// loads gamma or repeats the statistics.  xs must hold a.cols floats, red 16; blockDim.x <= 256.
 __device__ __forceinline__ void coop_fold(const GemvArgs &a, const float *__restrict__ x, float *xs, float *red,
                                           float pivot, float &s1_out, float &s2_out) {
   const int tid = threadIdx.x, nthr = blockDim.x, nw = nthr >> 6;
@@ -232,17 +232,21 @@ __device__ __forceinline__ void coop_fold(const GemvArgs &a, const float *__rest
     s2 = fmaf(d3, d3, s2);
     ((float4 *)xs)[i] = make_float4(v.x * g.x, v.y * g.y, v.z * g.z, v.w * g.w);
   }
-  auto block_sum = [&](float v) {
-    v = wave_sum(v);
-    __syncthreads();
-    if ((tid & 63) == 0) red[tid >> 6] = v;
-    __syncthreads();
-    float t = 0.0f;
-    for (int w = 0; w < nw; w++) t += red[w];
-    return t;
-  };
-  s1_out = block_sum(s1);
-  s2_out = block_sum(s2);  // its barriers also publish xs
+  // both sums cross the workgroup behind ONE barrier, which also publishes xs (red holds 8 + 8 partials)
+  s1 = wave_sum(s1);
+  s2 = wave_sum(s2);
+  if ((tid & 63) == 0) {
+    red[tid >> 6] = s1;
+    red[8 + (tid >> 6)] = s2;
+  }
+  __syncthreads();
+  float t1 = 0.0f, t2 = 0.0f;
+  for (int w = 0; w < nw; w++) {
+    t1 += red[w];
+    t2 += red[8 + w];
+  }
+  s1_out = t1;
+  s2_out = t2;
 }
 
 // Sixteen bytes that stay zero: lanes with nothing to fetch point their requests here, so that every

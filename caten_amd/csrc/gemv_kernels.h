@@ -347,7 +347,7 @@ __device__ __forceinline__ void gemv_ring(const GemvArgs &a, float *xs_lds, floa
   }
 
   // ---- (2) the weight ring ----
-  auto request = [&](int rq, uint4 *w, unsigned short *s, float &epi) {
+  auto request = [&](int rq, uint4 *w, unsigned *s, float &epi) {
     int row = rq * RPW + g;
     row = row < a.rows ? row : a.rows - 1;
 #pragma unroll
@@ -373,7 +373,9 @@ __device__ __forceinline__ void gemv_ring(const GemvArgs &a, float *xs_lds, floa
     }
   };
   uint4 wt[PD][KC];
-  unsigned short st[PD][KC];
+  // (one 32-bit register per scale: 16-bit elements would be packed in pairs right behind their loads, and that
+  // use would make the wavefront wait for the tile before it has requested anything else)
+  unsigned st[PD][KC];
   float epi_t[PD];
 #pragma unroll
   for (int p = 0; p < PD; p++) epi_t[p] = 0.0f;
@@ -554,7 +556,7 @@ __device__ __forceinline__ void gemv_ring(const GemvArgs &a, float *xs_lds, floa
     float acc = 0.0f;
 #pragma unroll
     for (int j = 0; j < KC; j++) {
-      const float scale = QUANT ? half_bits_to_float(st[p][j]) : 1.0f;
+      const float scale = QUANT ? half_bits_to_float((unsigned short)st[p][j]) : 1.0f;
       acc += chunk_dot<TYPE>(wt[p][j], scale, xr[j], xs[j]);
     }
     acc = group_sum<G>(acc);
@@ -625,31 +627,25 @@ __global__ __launch_bounds__(256) void k_gemv(GemvArgs a) {
   // stream instead of preceding it.  RMSNorm has no mu / beta term and needs no precomputation.
   const bool folded = (a.pro == CTHIP_PRO_RMSNORM) || (a.pro == CTHIP_PRO_LAYERNORM && a.fold_s != nullptr);
   const bool coop = a.stage_x != 0;  // input staged (and normalised, unless folded) once per workgroup
-  auto load = [&](int rq, uint4 *w, unsigned short *s, float &bias, float &resid, float &fs) {
-    const int row = rq * RPW + g;
-    const bool rok = row < a.rows;
-    // the epilogue operands of the row travel with its weights
-    bias = (rok && a.bias) ? a.bias[row] : 0.0f;
-    resid = (rok && a.residual) ? a.residual[(int64_t)m * a.y_stride + row] : 0.0f;
-    fs = (rok && a.fold_s) ? a.fold_s[row] : 0.0f;
+  // Every request is unconditional (a row past the end repeats the last row and is never stored, a chunk past the
+  // end of a row reads the zero block, an absent epilogue operand reads the zero block): a load behind a branch
+  // leaves a copy of its result at the end of that branch, and the wavefront would wait there for the whole tile
+  // before it has even requested its input vector -- two memory round trips in a launch that is nothing but latency.
+  auto load = [&](int rq, uint4 *w, unsigned *s, float &bias, float &resid, float &fs) {
+    int row = rq * RPW + g;
+    row = row < a.rows ? row : a.rows - 1;
+    const float *zf = (const float *)g_gemv_zeros;
+    bias = *(a.bias ? a.bias + row : zf);
+    resid = *(a.residual ? a.residual + (int64_t)m * a.y_stride + row : zf);
+    fs = *(a.fold_s ? a.fold_s + row : zf);
 #pragma unroll
     for (int j = 0; j < KC; j++) {
       const int c = l + G * j;
-      const bool ok = rok && c < nchunks;
-      if (NT) {
-        uint4 t = make_uint4(0u, 0u, 0u, 0u);
-        if (ok) {
-          const uint4 *src = &qp[(int64_t)row * row_chunks + c];
-          t = make_uint4(__builtin_nontemporal_load(&src->x), __builtin_nontemporal_load(&src->y),
-                         __builtin_nontemporal_load(&src->z), __builtin_nontemporal_load(&src->w));
-        }
-        w[j] = t;
-      } else {
-        w[j] = ok ? qp[(int64_t)row * row_chunks + c] : make_uint4(0u, 0u, 0u, 0u);
-      }
+      const bool ok = c < nchunks;
+      w[j] = load_chunk<NT>(ok ? qp + (int64_t)row * row_chunks + c : (const uint4 *)g_gemv_zeros);
       if (QUANT) {
         const int sidx = (TYPE == CTHIP_Q8_0) ? (c >> 1) : c;
-        s[j] = ok ? a.d[(int64_t)row * scales_per_row + sidx] : (unsigned short)0;
+        s[j] = *(ok ? a.d + (int64_t)row * scales_per_row + sidx : (const unsigned short *)g_gemv_zeros);
       }
     }
   };
@@ -662,13 +658,14 @@ __global__ __launch_bounds__(256) void k_gemv(GemvArgs a) {
   // latencies overlap: position, the first weight tiles, then the input vector.
   const int posv = a.pos ? a.pos[0] : 0;
   uint4 wt[PD][KC];
-  unsigned short st[PD][KC];
+  // (one 32-bit register per scale: 16-bit elements would be packed in pairs right behind their loads, and that
+  // use would make the wavefront wait for the tile before it has requested anything else)
+  unsigned st[PD][KC];
   float bias_t[PD], resid_t[PD], fs_t[PD];
 #pragma unroll
   for (int p = 0; p < PD; p++) {
-    bias_t[p] = resid_t[p] = fs_t[p] = 0.0f;
     const int rq = wave + p * total_waves;
-    if (rq < nrq) load(rq, wt[p], st[p], bias_t[p], resid_t[p], fs_t[p]);
+    load(rq < nrq ? rq : nrq - 1, wt[p], st[p], bias_t[p], resid_t[p], fs_t[p]);
   }
 
   float xr[KC][XPC];
@@ -750,7 +747,7 @@ __global__ __launch_bounds__(256) void k_gemv(GemvArgs a) {
         float acc = 0.0f;
 #pragma unroll
         for (int j = 0; j < KC; j++) {
-          const float scale = QUANT ? half_bits_to_float(st[p][j]) : 1.0f;
+          const float scale = QUANT ? half_bits_to_float((unsigned short)st[p][j]) : 1.0f;
           acc += chunk_dot<TYPE>(wt[p][j], scale, xr[j], xs[j]);
         }
         acc = group_sum<G>(acc);

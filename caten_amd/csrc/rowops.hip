@@ -395,7 +395,8 @@ __device__ __forceinline__ float4 rope4(float4 x, int c, int DH, float log2_base
 }
 
 template <int DH, bool APPEND>
-__global__ __launch_bounds__(1024) void k_attn_cached(float *__restrict__ out, const float *__restrict__ q,
+__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)))
+void k_attn_cached(float *__restrict__ out, const float *__restrict__ q,
                                                       float *__restrict__ kc, float *__restrict__ vc,
                                                       int start_pos, const int *__restrict__ pos, int H, int Hkv,
                                                       const float *__restrict__ newkv, float log2_base) {

@@ -34,12 +34,32 @@ __global__ __launch_bounds__(256) void k_rowop(RowArgs a) {
   float4 *__restrict__ yp = (float4 *)(a.y + row * n);
   float v[VPL][4];
   bool ok[VPL];
+  // every request of the row (and of gamma / beta) goes out before anything is used, none behind a branch: lanes
+  // past the end repeat the last chunk and drop it.  A load inside `if (ok)` is waited for at the end of that block,
+  // which turns a row into one memory round trip per chunk.
+  constexpr bool NORM = MODE == ROW_LAYERNORM || MODE == ROW_RMSNORM || MODE == ROW_LN_SOFTMAX;
+  float4 t[VPL], gm[NORM ? VPL : 1], bt[NORM ? VPL : 1];
 #pragma unroll
   for (int j = 0; j < VPL; j++) {
     const int c = lane + 64 * j;
     ok[j] = c < n4;
-    float4 t = ok[j] ? xp[c] : make_float4(0.f, 0.f, 0.f, 0.f);
-    v[j][0] = t.x; v[j][1] = t.y; v[j][2] = t.z; v[j][3] = t.w;
+    t[j] = xp[ok[j] ? c : n4 - 1];
+  }
+  if (NORM) {
+    const float4 *g4 = a.g ? (const float4 *)a.g : xp, *b4 = a.b ? (const float4 *)a.b : xp;  // xp: unused stand-in
+#pragma unroll
+    for (int j = 0; j < VPL; j++) {
+      const int c = lane + 64 * j;
+      gm[NORM ? j : 0] = g4[ok[j] ? c : n4 - 1];
+      bt[NORM ? j : 0] = b4[ok[j] ? c : n4 - 1];
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < VPL; j++) {
+    v[j][0] = ok[j] ? t[j].x : 0.0f;
+    v[j][1] = ok[j] ? t[j].y : 0.0f;
+    v[j][2] = ok[j] ? t[j].z : 0.0f;
+    v[j][3] = ok[j] ? t[j].w : 0.0f;
   }
   if (MODE == ROW_LAYERNORM || MODE == ROW_RMSNORM || MODE == ROW_LN_SOFTMAX) {
     const float inv_n = 1.0f / (float)n;
@@ -65,13 +85,12 @@ __global__ __launch_bounds__(256) void k_rowop(RowArgs a) {
 #pragma unroll
     for (int j = 0; j < VPL; j++) {
       if (ok[j]) {
-        const int c = lane + 64 * j;
-        float4 gm = a.g ? ((const float4 *)a.g)[c] : make_float4(1.f, 1.f, 1.f, 1.f);
-        float4 bt = a.b ? ((const float4 *)a.b)[c] : make_float4(0.f, 0.f, 0.f, 0.f);
-        v[j][0] = v[j][0] * rstd * gm.x + bt.x;
-        v[j][1] = v[j][1] * rstd * gm.y + bt.y;
-        v[j][2] = v[j][2] * rstd * gm.z + bt.z;
-        v[j][3] = v[j][3] * rstd * gm.w + bt.w;
+        const float4 g = a.g ? gm[NORM ? j : 0] : make_float4(1.f, 1.f, 1.f, 1.f);
+        const float4 b = a.b ? bt[NORM ? j : 0] : make_float4(0.f, 0.f, 0.f, 0.f);
+        v[j][0] = v[j][0] * rstd * g.x + b.x;
+        v[j][1] = v[j][1] * rstd * g.y + b.y;
+        v[j][2] = v[j][2] * rstd * g.z + b.z;
+        v[j][3] = v[j][3] * rstd * g.w + b.w;
       }
     }
   }
@@ -402,7 +421,7 @@ void k_attn_cached(float *__restrict__ out, const float *__restrict__ q,
                                                       const float *__restrict__ newkv, float log2_base) {
   constexpr int LPK = DH / 4;      // lanes per key
   constexpr int KPW = 64 / LPK;    // keys per wavefront per pass
-  constexpr int KPT = 8;           // passes held in registers
+  constexpr int KPT = 4;           // passes held in registers
   constexpr int NW = 16;
   constexpr int TILE = NW * KPW * KPT;
   __shared__ float part[NW][DH];

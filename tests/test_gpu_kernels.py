@@ -238,6 +238,38 @@ def test_layernorm_folded_through_the_product(ops, oracle, kind):
         wm.free()
 
 
+@pytest.mark.parametrize("kind", ["q8_0", "q4_0"])
+def test_looping_launches_with_long_staged_inputs(ops, oracle, kind):
+    """Looping launches whose staged input is longer than what a thread requests ahead of the weights (4096 floats):
+    the rest of the vector is staged by a loop behind the first tile; a LayerNorm that is not folded and has a bias
+    beside it is applied by the workgroup before the stream starts.  RMSNorm, SwiGLU and plain inputs, with and
+    without residual."""
+    from caten_amd.llm import Tensor
+    rng = np.random.default_rng(33)
+    rows, cols = 5000, 6144
+    w = rng.normal(0, 0.02, (rows, cols)).astype(np.float32)
+    t = Tensor.from_f32(w, kind)
+    wd = oracle.dequant(kind, t.raw, w.size).reshape(rows, cols)
+    wm = ops.WeightMatrix(kind, t.raw, rows, cols)
+    x = rng.normal(0.2, 1.0, cols).astype(np.float32)
+    g = rng.normal(1, 0.05, cols).astype(np.float32)
+    b = rng.normal(0, 0.05, cols).astype(np.float32)
+    bias = rng.normal(0, 0.1, rows).astype(np.float32)
+    res = rng.normal(0, 1, rows).astype(np.float32)
+    tol = dict(rtol=2e-3, atol=3e-4)
+    close(ops.linear(x, wm, prologue="rmsnorm", norm_g=g), oracle.linear(oracle.rmsnorm(x, g), wd), **tol)
+    close(ops.linear(x, wm, residual=res, prologue="rmsnorm", norm_g=g), oracle.linear(oracle.rmsnorm(x, g), wd) + res, **tol)
+    close(ops.linear(x, wm, bias=bias, prologue="layernorm", norm_g=g, norm_b=b),
+          oracle.linear(oracle.layernorm(x, g, b), wd, bias), **tol)
+    close(ops.linear(x, wm, prologue="layernorm", norm_g=g, norm_b=b), oracle.linear(oracle.layernorm(x, g, b), wd), **tol)
+    close(ops.linear(x, wm, bias=bias, residual=res), oracle.linear(x, wd, bias) + res, **tol)
+    xu = rng.normal(0, 1, 2 * cols).astype(np.float32)
+    gate, up = xu[:cols].astype(np.float64), xu[cols:].astype(np.float64)
+    sw = (gate / (1 + np.exp(-gate)) * up).astype(np.float32)
+    close(ops.linear(xu, wm, residual=res, prologue="swiglu"), oracle.linear(sw, wd) + res, **tol)
+    wm.free()
+
+
 def test_gemv_fallback_shapes_with_prologue(ops, oracle):
     from caten_amd.llm import Tensor
     rng = np.random.default_rng(22)

@@ -716,12 +716,24 @@ __global__ __launch_bounds__(256) void k_gemm_f32(GemmArgs a) {
 // C = act(sum_z ws[z] + bias) + residual, z in ascending order (the result does not depend on timing)
 __global__ __launch_bounds__(256) void k_splitk_reduce(GemmArgs a) {
   const int64_t n = (int64_t)a.M * a.N;
+  // Up to eight partials, bias and residual are requested together, none behind a branch (absent ones re-read
+  // the first partial and are dropped): a `for (z...) v += ws[z]` loop is one dependent round trip per share.
+  // The shares are still added in ascending order, so the result does not depend on the launch.
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
-    float v = a.ws[i];
-    for (int z = 1; z < a.ksplit; z++) v += a.ws[(int64_t)z * n + i];
-    if (a.bias) v += a.bias[i % a.N];
+    const float bv = *(a.bias ? a.bias + i % a.N : a.ws + i);
+    const float rv = *(a.residual ? a.residual + i : a.ws + i);
+    float v = 0.0f;
+    for (int zb = 0; zb < a.ksplit; zb += 8) {
+      float t[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++) t[u] = a.ws[(int64_t)(zb + u < a.ksplit ? zb + u : 0) * n + i];
+#pragma unroll
+      for (int u = 0; u < 8; u++)
+        if (zb + u < a.ksplit) v = (zb + u == 0) ? t[u] : v + t[u];
+    }
+    if (a.bias) v += bv;
     v = apply_act(a.act, v);
-    if (a.residual) v += a.residual[i];
+    if (a.residual) v += rv;
     a.C[i] = v;
   }
 }

@@ -26,7 +26,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # (profiles/), scaled by a copy kernel of known size; None where it has not been measured.
-TRAFFIC_BYTES = {("gpt2", "q8_0"): 41965322}  # profiles/gemv_q8_0_lm_head_pmc.txt
+TRAFFIC_BYTES = {("gpt2", "q8_0"): 44608512}  # profiles/gemv_q8_0_lm_head_pmc.txt
 
 
 def cpu_baseline(cfg, weights, prompt, budget_s, kind, llama):

@@ -74,8 +74,6 @@ def main():
                     help="also run one 256 MiB device-to-device copy (a kernel of known traffic to scale "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings by)")
     args = ap.parse_args()
-    if args.no_graph:
-        os.environ["CTHIP_NO_GRAPH"] = "1"
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (batch-1 decode does not use a second); run with --gpus 1",
               file=sys.stderr)
@@ -92,6 +90,8 @@ def main():
         # the KV cache bounds how many tokens one sequence can hold: restart sequences as needed
         pass
     lib = _lib.init(0)
+    if args.no_graph:
+        _lib.check(lib.cthip_set_option(b"decoder_graph", 0))
     model = (llm.make_llama(cfg, llm.llama_state_dict(weights, args.kind)) if llama
              else llm.make_gpt2(cfg, llm.gpt2_state_dict(weights, args.kind)))
 

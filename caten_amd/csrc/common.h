@@ -21,6 +21,10 @@ struct State {
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   int gemm_precision = GEMM_BF16X3_DEFAULT;  // option "gemm_precision" (GEMM_*) of m > 1 Linear launches
   int gemv_stream = -1;  // option "gemv_stream_weights": -1 = per matrix (WMat::stream), 0 / 1 = never / always
+  // decoder sessions read these when they first run
+  int decoder_graph = 1;  // option "decoder_graph": 0 = the step's launches are issued one by one (kernel tracing)
+  int prefill_gemm = 1;   // option "prefill_gemm": 0 = prompts are fed row by row through the decode step
+  int decode_fused = 1;   // option "decode_fused": 0 = five launches per layer instead of three
 };
 State &state();
 // cthip_alloc without the zero fill, for temporaries that are fully written before they are read

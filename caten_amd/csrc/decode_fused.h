@@ -1,0 +1,60 @@
+// Argument blocks and launchers of the three-launch decode layer (decode_fused.hip).
+#pragma once
+#include "common.h"
+
+namespace cthip {
+
+constexpr int kDecXcds = 8;  // accelerator dies of gfx950; one MLP accumulator each
+
+// how a launch assembles its input vector: x = base + bias + partial vectors
+struct DecStage {
+  const float *base;        // D floats
+  const float *bias;        // D floats (unused when the launch takes the base alone)
+  const float *fparts;      // fp32 partial vectors, D floats each (one per head)
+  const long long *iparts;  // kDecXcds fixed-point (2^-32) accumulators, D each
+  const float *gamma;       // LayerNorm gamma of the Linear that follows
+  float *xout;              // block 0 stores the assembled vector here (may be null)
+  float eps;
+  int D;
+};
+
+struct DecQkvArgs {
+  DecStage st;
+  const void *wq;            // c_attn quant plane, int8 [3D][D]
+  const unsigned short *wd;  // c_attn scale plane, fp16 [3D][D/32]
+  const float *fold_s, *fold_c;  // W.gamma and W.beta + bias
+  float *q, *kc, *vc;        // q (D), K / V cache (max_seq, D)
+  const int *pos;
+  int rows;                  // 3D
+};
+
+struct DecAttnArgs {
+  const float *q, *kc, *vc;
+  const int *pos;
+  const void *pq;            // attn.c_proj by head: int8 [H][D][Dh]
+  const unsigned short *pd;  // fp16 [H][D][Dh/32]
+  float *part;               // out: fp32 [H][D], head h's share of the projection
+  void *zero;                // cleared here: the MLP accumulators
+  int64_t zero_n16;          // ... in 16-byte units
+};
+
+struct DecMlpArgs {
+  DecStage st;
+  const void *wq;            // c_fc quant plane, int8 [F][D]
+  const unsigned short *wd;  // fp16 [F][D/32]
+  const float *fold_s, *fold_c;
+  const void *pq;            // mlp.c_proj by 16-column slab: int8 [F/16][D][16]
+  const unsigned short *pd;  // fp16 [F/32][D]
+  long long *accum;          // [kDecXcds][D]
+};
+
+bool dec_fused_supported(int type_attn, int type_proj, int type_fc, int type_fc2, int D, int H, int F);
+int dec_xcd_probe(int *max_id);
+int dec_relay_heads(const WMat *w, int DH, void **pq, void **pd);
+int dec_relay_slabs(const WMat *w, void **pq, void **pd);
+int launch_dec_qkv(const DecQkvArgs &a, bool from_accum);
+int launch_dec_attn_proj(const DecAttnArgs &a, int H, int D);
+int launch_dec_mlp(const DecMlpArgs &a, int F, int H);
+int launch_dec_sum(const DecStage &s, float *out);
+
+}  // namespace cthip

@@ -1,0 +1,540 @@
+// Three launches per layer for one decode row of a GPT-2 shaped Transformer (external/llm/layers.lisp:35-71)
+// with Q8_0 weights, instead of five.  A decode step is bound by the number of DEPENDENT launches, not by
+// bytes, so two pairs of consecutive Linears are merged around the vector that sits between them:
+//
+//   k_dec_qkv        x -> LayerNorm1 -> c_attn (+bias): q to a buffer, k / v rows into the cache at `pos`
+//   k_dec_attn_proj  one workgroup per head: attention over cache rows 0..pos, then that head's 64 columns
+//                    of attn.c_proj applied to its 64 outputs -> one partial vector per head
+//   k_dec_mlp        one workgroup per 16 hidden units: LayerNorm2 -> those rows of c_fc (+bias, GELU) ->
+//                    their 16 columns of mlp.c_proj -> partial vector, added into one accumulator per XCD
+//
+// A Linear whose INPUT is split over workgroups produces one partial output vector per workgroup; the
+// consumer of the vector adds the partials while it stages its input, so the residual stream travels as
+// "base vector + bias + partials" and is materialised by whoever reads it next:
+//   * attention: H partial vectors of fp32, plain stores (Patt);
+//   * MLP: F/16 workgroups would be too many partials to re-read, so each workgroup adds its vector into the
+//     accumulator of the XCD it runs on (Pmlp[xcd][D]).  Atomics that carry no device-scope bits execute in
+//     the L2 of the issuing XCD, which all its compute units share, and an accumulator is only ever touched
+//     from its own XCD, so no traffic crosses the fabric; the lines are written back at the end of the
+//     kernel like any other store.  The accumulators are 64-bit fixed point (2^-32): integer addition is
+//     associative, so the sum does not depend on the order the workgroups arrive in.
+// Weights of the two "column" Linears are re-laid at load so that a workgroup's share is contiguous.
+#include <stdlib.h>
+
+#include "common.h"
+#include "gemv_kernels.h"
+#include "decode_fused.h"
+
+namespace cthip {
+
+constexpr float kFixScale = 4294967296.0f;             // 2^32
+constexpr float kFixInv = 2.3283064365386963e-10f;     // 2^-32
+
+__device__ __forceinline__ int xcd_id() {
+  // XCC_ID hardware register (id 20), bits 3:0: the XCD this wavefront runs on
+  return (int)__builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20) & (kDecXcds - 1);
+}
+
+__device__ __forceinline__ float4 f4add(float4 a, float4 b) { return make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w); }
+
+// Assembles the launch's input vector  x = base + bias + sum(partials)  (one float4 per thread, D <= 1024),
+// writes gamma * x to LDS and returns the LayerNorm statistics of x; block 0 also stores x to s.xout.
+// MODE 0: base only; 1: + bias + NP fp32 partial vectors; 2: + bias + kDecXcds fixed-point accumulators.
+// Every load is unconditional and issued before any use.  red holds 24 floats.  blockDim.x == 256.
+template <int MODE, int NP>
+__device__ __forceinline__ void dec_stage(const DecStage &s, float *xs, float *red, float &mu, float &rstd) {
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int n4 = s.D >> 2;
+  const bool active = tid < n4;
+  const int i = active ? tid : n4 - 1;
+  float4 v = ((const float4 *)s.base)[i];
+  const float4 g = ((const float4 *)s.gamma)[i];
+  if (MODE != 0) {
+    const float4 b = ((const float4 *)s.bias)[i];
+    if (MODE == 1) {
+      float4 p[NP];
+#pragma unroll
+      for (int k = 0; k < NP; k++) p[k] = ((const float4 *)(s.fparts + (int64_t)k * s.D))[i];
+      v = f4add(v, b);
+#pragma unroll
+      for (int k = 0; k < NP; k++) v = f4add(v, p[k]);
+    } else {
+      longlong2 lo[kDecXcds], hi[kDecXcds];
+#pragma unroll
+      for (int k = 0; k < kDecXcds; k++) {
+        const longlong2 *src = (const longlong2 *)(s.iparts + (int64_t)k * s.D) + 2 * i;
+        lo[k] = src[0];
+        hi[k] = src[1];
+      }
+      long long t0 = 0, t1 = 0, t2 = 0, t3 = 0;
+#pragma unroll
+      for (int k = 0; k < kDecXcds; k++) {
+        t0 += lo[k].x;
+        t1 += lo[k].y;
+        t2 += hi[k].x;
+        t3 += hi[k].y;
+      }
+      v = f4add(v, b);
+      v = f4add(v, make_float4(__ll2float_rn(t0) * kFixInv, __ll2float_rn(t1) * kFixInv, __ll2float_rn(t2) * kFixInv,
+                               __ll2float_rn(t3) * kFixInv));
+    }
+  }
+  // (count, mean, squared deviation) per thread, merged exactly: thread -> wavefront by lane reductions,
+  // wavefront -> workgroup through LDS behind the one barrier that also publishes the staged vector
+  const float cnt = active ? 4.0f : 0.0f;
+  const float mean_t = 0.25f * ((v.x + v.y) + (v.z + v.w));
+  const float d0 = v.x - mean_t, d1 = v.y - mean_t, d2 = v.z - mean_t, d3 = v.w - mean_t;
+  const float m2_t = active ? fmaf(d0, d0, fmaf(d1, d1, fmaf(d2, d2, d3 * d3))) : 0.0f;
+  const float n_w = wave_sum(cnt);
+  const float mean_w = wave_sum(cnt * mean_t) / fmaxf(n_w, 1.0f);
+  const float dm = mean_t - mean_w;
+  const float m2_w = wave_sum(m2_t + cnt * dm * dm);
+  if (active) {
+    ((float4 *)xs)[i] = make_float4(v.x * g.x, v.y * g.y, v.z * g.z, v.w * g.w);
+    if (blockIdx.x == 0 && s.xout) ((float4 *)s.xout)[i] = v;
+  }
+  if (lane == 0) {
+    red[wv] = n_w;
+    red[8 + wv] = mean_w;
+    red[16 + wv] = m2_w;
+  }
+  __syncthreads();
+  const float inv_n = 1.0f / (float)s.D;
+  float sum = 0.0f;
+#pragma unroll
+  for (int w = 0; w < 4; w++) sum += red[w] * red[8 + w];
+  mu = sum * inv_n;
+  float m2 = 0.0f;
+#pragma unroll
+  for (int w = 0; w < 4; w++) {
+    const float dw = red[8 + w] - mu;
+    m2 += red[16 + w] + red[w] * dw * dw;
+  }
+  rstd = 1.0f / sqrtf(fmaxf(m2 * inv_n, 0.0f) + s.eps);
+}
+
+// One row of 16 lanes x KC chunks of a Q8_0 plane against the staged vector (D = 256 * KC).
+template <int KC>
+__device__ __forceinline__ float dec_row_dot(const uint4 *w, const unsigned *sc, const float *xs, int l) {
+  float acc = 0.0f;
+#pragma unroll
+  for (int j = 0; j < KC; j++) {
+    const int c = l + 16 * j;
+    float xr[16];
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+      const float4 v = *(const float4 *)(xs + c * 16 + 4 * t);
+      xr[4 * t + 0] = v.x;
+      xr[4 * t + 1] = v.y;
+      xr[4 * t + 2] = v.z;
+      xr[4 * t + 3] = v.w;
+    }
+    acc += chunk_dot<CTHIP_Q8_0>(w[j], half_bits_to_float((unsigned short)sc[j]), xr, 0.0f);
+  }
+  return row16_sum(acc);
+}
+
+// ---- launch 1: LayerNorm1 folded through c_attn; 16 rows per workgroup ----
+template <int KC, int MODE>
+__global__ __launch_bounds__(256) void k_dec_qkv(DecQkvArgs a) {
+  __shared__ __align__(16) float xs[256 * KC];
+  __shared__ float red[24];
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int g = lane >> 4, l = lane & 15;
+  const int D = a.st.D;
+  int row = blockIdx.x * 16 + wv * 4 + g;
+  const bool row_ok = row < a.rows;
+  row = row_ok ? row : a.rows - 1;
+  uint4 w[KC];
+  unsigned sc[KC];
+  const uint4 *qp = (const uint4 *)a.wq + (int64_t)row * (16 * KC);
+  const unsigned short *dp = a.wd + (int64_t)row * (8 * KC);
+#pragma unroll
+  for (int j = 0; j < KC; j++) {
+    const int c = l + 16 * j;
+    w[j] = qp[c];
+    sc[j] = dp[c >> 1];
+  }
+  const float fs = a.fold_s[row], fc = a.fold_c[row];
+  const int posv = a.pos[0];
+  float mu, rstd;
+  dec_stage<MODE, 1>(a.st, xs, red, mu, rstd);
+  const float acc = dec_row_dot<KC>(w, sc, xs, l);
+  if (l == 0 && row_ok) {
+    // rstd * (W.(gamma x) - mu * W.gamma) + (W.beta + bias)  =  W.LayerNorm(x) + bias
+    const float v = rstd * (acc - mu * fs) + fc;
+    if (row < D) a.q[row] = v;
+    else if (row < 2 * D) a.kc[(int64_t)posv * D + (row - D)] = v;
+    else a.vc[(int64_t)posv * D + (row - 2 * D)] = v;
+  }
+}
+
+// ---- launch 2: attention of one query row per head, then that head's columns of attn.c_proj ----
+// Attention as in k_attn_cached (rowops.hip): a key row is read by DH/4 lanes as one float4 each, a wavefront
+// holds four passes of K and V in registers, per-wavefront online softmax, one meeting in LDS.  The head's
+// slab of the projection (D rows x DH columns, contiguous after the re-layout) does not depend on anything
+// computed here and is requested first, so it arrives while the keys are being processed.
+template <int DH, int JR>
+__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)))
+void k_dec_attn_proj(DecAttnArgs a) {
+  constexpr int LPK = DH / 4, KPW = 64 / LPK, KPT = 4, NW = 16, TILE = NW * KPW * KPT;
+  constexpr int CPR = DH / 16;          // 16-byte chunks of a projection row inside the slab
+  constexpr int RPP = 1024 / CPR;       // projection rows per pass of the workgroup
+  __shared__ float part[NW][DH];
+  __shared__ float pm[NW], pl[NW];
+  __shared__ __align__(16) float oh[DH];
+  const int h = blockIdx.x, H = gridDim.x, D = H * DH;
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int g = lane / LPK, c = lane % LPK;
+  // the projection slab of this head
+  const int pc = tid % CPR, pr0 = tid / CPR;
+  uint4 pw[JR];
+  unsigned ps[JR];
+#pragma unroll
+  for (int j = 0; j < JR; j++) {
+    int r = pr0 + RPP * j;
+    r = r < D ? r : D - 1;
+    pw[j] = ((const uint4 *)a.pq)[((int64_t)h * D + r) * CPR + pc];
+    ps[j] = a.pd[((int64_t)h * D + r) * (DH / 32) + (pc >> 1)];
+  }
+  const int T = a.pos[0] + 1;
+  const unsigned kvs4 = (unsigned)(D / 4);
+  const float4 q4 = *(const float4 *)(a.q + h * DH + 4 * c);
+  const float4 *__restrict__ kp = (const float4 *)(a.kc + h * DH) + c;
+  const float4 *__restrict__ vp = (const float4 *)(a.vc + h * DH) + c;
+  const float scale = 1.0f / sqrtf((float)DH);
+  // the accumulators of the MLP launch are cleared here: their last reader (this layer's k_dec_qkv) has finished
+  {
+    uint4 *z = (uint4 *)a.zero;
+    const uint4 zz = make_uint4(0u, 0u, 0u, 0u);
+    for (int64_t k = (int64_t)h * 1024 + tid; k < a.zero_n16; k += (int64_t)H * 1024) z[k] = zz;
+  }
+  float m = -INFINITY, lsum = 0.0f;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int t0 = 0; t0 < T; t0 += TILE) {
+    if (t0 + wv * KPT * KPW >= T) break;  // nothing left for this wavefront (uniform)
+    float4 kr[KPT], vr[KPT];
+#pragma unroll
+    for (int u = 0; u < KPT; u++) {
+      const int j = t0 + (wv * KPT + u) * KPW + g;
+      const unsigned jj = (unsigned)min(j, T - 1);  // clamped: masked below, never outside the cache
+      kr[u] = kp[jj * kvs4];
+      vr[u] = vp[jj * kvs4];
+    }
+    float sc[KPT];
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < KPT; u++) {
+      float d = q4.x * kr[u].x;
+      d = fmaf(q4.y, kr[u].y, d);
+      d = fmaf(q4.z, kr[u].z, d);
+      d = fmaf(q4.w, kr[u].w, d);
+#pragma unroll
+      for (int o = LPK / 2; o > 0; o >>= 1) d += __shfl_xor(d, o, 64);
+      const bool ok = (t0 + (wv * KPT + u) * KPW + g) < T;
+      sc[u] = ok ? d * scale : -INFINITY;
+      tmax = fmaxf(tmax, sc[u]);
+    }
+#pragma unroll
+    for (int o = LPK; o < 64; o <<= 1) tmax = fmaxf(tmax, __shfl_xor(tmax, o, 64));
+    const float m_new = fmaxf(m, tmax);
+    const float corr = ct_exp(m - m_new);
+    float psum = 0.0f;
+#pragma unroll
+    for (int k2 = 0; k2 < 4; k2++) acc[k2] *= corr;
+#pragma unroll
+    for (int u = 0; u < KPT; u++) {
+      const float p = ct_exp(sc[u] - m_new);
+      psum += p;
+      acc[0] = fmaf(p, vr[u].x, acc[0]);
+      acc[1] = fmaf(p, vr[u].y, acc[1]);
+      acc[2] = fmaf(p, vr[u].z, acc[2]);
+      acc[3] = fmaf(p, vr[u].w, acc[3]);
+    }
+#pragma unroll
+    for (int o = LPK; o < 64; o <<= 1) psum += __shfl_xor(psum, o, 64);
+    lsum = lsum * corr + psum;
+    m = m_new;
+  }
+#pragma unroll
+  for (int o = LPK; o < 64; o <<= 1) {
+#pragma unroll
+    for (int k2 = 0; k2 < 4; k2++) acc[k2] += __shfl_xor(acc[k2], o, 64);
+  }
+  if (lane < LPK) {
+#pragma unroll
+    for (int k2 = 0; k2 < 4; k2++) part[wv][4 * lane + k2] = acc[k2];
+  }
+  if (lane == 0) {
+    pm[wv] = m;
+    pl[wv] = lsum;
+  }
+  __syncthreads();
+  if (tid < DH) {
+    float M = pm[0];
+#pragma unroll
+    for (int w = 1; w < NW; w++) M = fmaxf(M, pm[w]);
+    float o = 0.0f, L = 0.0f;
+#pragma unroll
+    for (int w = 0; w < NW; w++) {
+      const float e = ct_exp(pm[w] - M);
+      o = fmaf(e, part[w][tid], o);
+      L = fmaf(e, pl[w], L);
+    }
+    oh[tid] = o / L;
+  }
+  __syncthreads();
+  // partial projection: row r of the slab times the head's outputs; CPR lanes share a row
+  float xr[16];
+#pragma unroll
+  for (int t = 0; t < 4; t++) {
+    const float4 v = *(const float4 *)(oh + pc * 16 + 4 * t);
+    xr[4 * t + 0] = v.x;
+    xr[4 * t + 1] = v.y;
+    xr[4 * t + 2] = v.z;
+    xr[4 * t + 3] = v.w;
+  }
+#pragma unroll
+  for (int j = 0; j < JR; j++) {
+    float s = chunk_dot<CTHIP_Q8_0>(pw[j], half_bits_to_float((unsigned short)ps[j]), xr, 0.0f);
+    if (CPR >= 2) s += dpp_f<0xB1>(s);  // quad_perm [1,0,3,2]
+    if (CPR >= 4) s += dpp_f<0x4E>(s);  // quad_perm [2,3,0,1]
+    if (CPR >= 8) s += dpp_f<0x141>(s);  // row_half_mirror
+    const int r = pr0 + RPP * j;
+    if (pc == 0 && r < D) a.part[(int64_t)h * D + r] = s;
+  }
+}
+
+// ---- launch 3: LayerNorm2 folded through 16 rows of c_fc, GELU, their 16 columns of mlp.c_proj ----
+template <int KC, int NP>
+__global__ __launch_bounds__(256) void k_dec_mlp(DecMlpArgs a) {
+  __shared__ __align__(16) float xs[256 * KC];
+  __shared__ float red[24];
+  __shared__ __align__(16) float hs[16];
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int g = lane >> 4, l = lane & 15;
+  const int D = a.st.D;
+  const int slab = blockIdx.x;
+  const int row = slab * 16 + wv * 4 + g;  // < F: the launcher requires F % 16 == 0
+  uint4 w[KC];
+  unsigned sc[KC];
+  const uint4 *qp = (const uint4 *)a.wq + (int64_t)row * (16 * KC);
+  const unsigned short *dp = a.wd + (int64_t)row * (8 * KC);
+#pragma unroll
+  for (int j = 0; j < KC; j++) {
+    const int c = l + 16 * j;
+    w[j] = qp[c];
+    sc[j] = dp[c >> 1];
+  }
+  const float fs = a.fold_s[row], fc = a.fold_c[row];
+  // this slab's 16 columns of the second Linear: row r = tid + 256 j (D = 256 * KC)
+  uint4 pw[KC];
+  unsigned ps[KC];
+#pragma unroll
+  for (int j = 0; j < KC; j++) {
+    const int r = tid + 256 * j;
+    pw[j] = ((const uint4 *)a.pq)[(int64_t)slab * D + r];
+    ps[j] = a.pd[(int64_t)(slab >> 1) * D + r];
+  }
+  float mu, rstd;
+  dec_stage<1, NP>(a.st, xs, red, mu, rstd);
+  const float acc = dec_row_dot<KC>(w, sc, xs, l);
+  if (l == 0) hs[wv * 4 + g] = ct_gelu(rstd * (acc - mu * fs) + fc);
+  __syncthreads();
+  float hr[16];
+#pragma unroll
+  for (int t = 0; t < 4; t++) {
+    const float4 v = *(const float4 *)(hs + 4 * t);
+    hr[4 * t + 0] = v.x;
+    hr[4 * t + 1] = v.y;
+    hr[4 * t + 2] = v.z;
+    hr[4 * t + 3] = v.w;
+  }
+  long long *accum = a.accum + (int64_t)xcd_id() * D;
+#pragma unroll
+  for (int j = 0; j < KC; j++) {
+    const float s = chunk_dot<CTHIP_Q8_0>(pw[j], half_bits_to_float((unsigned short)ps[j]), hr, 0.0f);
+    // no device-scope bits: the addition happens in this XCD's L2
+    __hip_atomic_fetch_add(accum + tid + 256 * j, __float2ll_rn(s * kFixScale), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_WORKGROUP);
+  }
+}
+
+// the residual stream as one vector: x = base + bias + accumulators (in front of lm_head)
+__global__ __launch_bounds__(256) void k_dec_sum(DecStage s, float *out) {
+  const int n4 = s.D >> 2;
+  for (int i = threadIdx.x; i < n4; i += 256) {
+    float4 v = f4add(((const float4 *)s.base)[i], ((const float4 *)s.bias)[i]);
+    long long t[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int k = 0; k < kDecXcds; k++) {
+      const longlong2 *src = (const longlong2 *)(s.iparts + (int64_t)k * s.D) + 2 * i;
+      const longlong2 lo = src[0], hi = src[1];
+      t[0] += lo.x;
+      t[1] += lo.y;
+      t[2] += hi.x;
+      t[3] += hi.y;
+    }
+    v = f4add(v, make_float4(__ll2float_rn(t[0]) * kFixInv, __ll2float_rn(t[1]) * kFixInv, __ll2float_rn(t[2]) * kFixInv,
+                             __ll2float_rn(t[3]) * kFixInv));
+    ((float4 *)out)[i] = v;
+  }
+}
+
+// ---- re-layout at load ----
+// attn.c_proj (D x D): head h's columns [h*DH, (h+1)*DH) of every row, contiguous: pq[h][r][DH], pd[h][r][DH/32]
+__global__ void k_relay_heads(const uint4 *__restrict__ q, const unsigned short *__restrict__ d, uint4 *__restrict__ pq,
+                              unsigned short *__restrict__ pd, int D, int DH) {
+  const int cpr = DH / 16, spr = DH / 32, H = D / DH;
+  const int64_t nq = (int64_t)H * D * cpr, ns = (int64_t)H * D * spr;
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < nq) {
+    const int cc = (int)(i % cpr);
+    const int64_t hr = i / cpr;
+    const int r = (int)(hr % D), h = (int)(hr / D);
+    pq[i] = q[(int64_t)r * (D / 16) + h * cpr + cc];
+  }
+  if (i < ns) {
+    const int bb = (int)(i % spr);
+    const int64_t hr = i / spr;
+    const int r = (int)(hr % D), h = (int)(hr / D);
+    pd[i] = d[(int64_t)r * (D / 32) + h * spr + bb];
+  }
+}
+// mlp.c_proj (D x F): 16 columns per slab: pq[s][r] = chunk s of row r, pd[b][r] = scale of 32-block b of row r
+__global__ void k_relay_slabs(const uint4 *__restrict__ q, const unsigned short *__restrict__ d, uint4 *__restrict__ pq,
+                              unsigned short *__restrict__ pd, int D, int F) {
+  const int64_t nq = (int64_t)(F / 16) * D, ns = (int64_t)(F / 32) * D;
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < nq) {
+    const int r = (int)(i % D), s = (int)(i / D);
+    pq[i] = q[(int64_t)r * (F / 16) + s];
+  }
+  if (i < ns) {
+    const int r = (int)(i % D), b = (int)(i / D);
+    pd[i] = d[(int64_t)r * (F / 32) + b];
+  }
+}
+
+__global__ void k_xcd_probe(int *out) {
+  if (threadIdx.x == 0) {
+    const int id = (int)__builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20);
+    atomicMax(out, id);
+  }
+}
+
+// ------------------------------------------------------------------ host side
+bool dec_fused_supported(int type_attn, int type_proj, int type_fc, int type_fc2, int D, int H, int F) {
+  if (type_attn != CTHIP_Q8_0 || type_proj != CTHIP_Q8_0 || type_fc != CTHIP_Q8_0 || type_fc2 != CTHIP_Q8_0) return false;
+  if (D % 256 || D < 256 || D > 1024) return false;
+  if (H <= 0 || D % H || D / H != 64) return false;
+  if (H != 4 && H != 8 && H != 12 && H != 16) return false;
+  if (F % 32 || F <= 0) return false;
+  return true;
+}
+
+int dec_xcd_probe(int *max_id) {
+  int *dev = nullptr;
+  int rc = cthip_alloc((void **)&dev, 256);
+  if (rc) return rc;
+  hipLaunchKernelGGL(k_xcd_probe, dim3(4096), dim3(64), 0, state().stream, dev);
+  hipError_t e = hipGetLastError();
+  if (e == hipSuccess) rc = cthip_d2h(max_id, dev, sizeof(int));
+  cthip_free(dev);
+  if (e != hipSuccess) return fail((int)e, "decoder: XCD probe -> %s", hipGetErrorString(e));
+  return rc;
+}
+
+int dec_relay_heads(const WMat *w, int DH, void **pq, void **pd) {
+  const int D = (int)w->rows;
+  int rc;
+  if ((rc = cthip_alloc(pq, (size_t)D * D))) return rc;
+  if ((rc = cthip_alloc(pd, (size_t)D * (D / 32) * 2))) return rc;
+  const int64_t n = (int64_t)D * D / 16;
+  hipLaunchKernelGGL(k_relay_heads, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, state().stream, (const uint4 *)w->q,
+                     (const unsigned short *)w->d, (uint4 *)*pq, (unsigned short *)*pd, D, DH);
+  CTHIP_LAUNCH_CHECK();
+  return 0;
+}
+
+int dec_relay_slabs(const WMat *w, void **pq, void **pd) {
+  const int D = (int)w->rows, F = (int)w->cols;
+  int rc;
+  if ((rc = cthip_alloc(pq, (size_t)D * F))) return rc;
+  if ((rc = cthip_alloc(pd, (size_t)D * (F / 32) * 2))) return rc;
+  const int64_t n = (int64_t)D * F / 16;
+  hipLaunchKernelGGL(k_relay_slabs, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, state().stream, (const uint4 *)w->q,
+                     (const unsigned short *)w->d, (uint4 *)*pq, (unsigned short *)*pd, D, F);
+  CTHIP_LAUNCH_CHECK();
+  return 0;
+}
+
+int launch_dec_qkv(const DecQkvArgs &a, bool from_accum) {
+  const int D = a.st.D, KC = D / 256;
+  if (D % 256 || KC < 1 || KC > 4 || a.rows != 3 * D) return fail(CTHIP_E_BAD_ARG, "decoder: fused qkv launch with D = %d, rows = %d", D, a.rows);
+  dim3 grid((a.rows + 15) / 16), block(256);
+  hipStream_t st = state().stream;
+#define GO(KC_)                                                                        \
+  case KC_:                                                                            \
+    if (from_accum) hipLaunchKernelGGL((k_dec_qkv<KC_, 2>), grid, block, 0, st, a);    \
+    else hipLaunchKernelGGL((k_dec_qkv<KC_, 0>), grid, block, 0, st, a);               \
+    break
+  switch (KC) {
+    GO(1);
+    GO(2);
+    GO(3);
+    GO(4);
+  }
+#undef GO
+  CTHIP_LAUNCH_CHECK();
+  return 0;
+}
+
+int launch_dec_attn_proj(const DecAttnArgs &a, int H, int D) {
+  if (D != H * 64 || D > 1024) return fail(CTHIP_E_BAD_ARG, "decoder: fused attention launch with D = %d, H = %d", D, H);
+  dim3 grid(H), block(1024);
+  hipStream_t st = state().stream;
+  // rows of the projection slab per thread: D / (1024 / 4)
+  switch ((D + 255) / 256) {
+    case 1: hipLaunchKernelGGL((k_dec_attn_proj<64, 1>), grid, block, 0, st, a); break;
+    case 2: hipLaunchKernelGGL((k_dec_attn_proj<64, 2>), grid, block, 0, st, a); break;
+    case 3: hipLaunchKernelGGL((k_dec_attn_proj<64, 3>), grid, block, 0, st, a); break;
+    default: hipLaunchKernelGGL((k_dec_attn_proj<64, 4>), grid, block, 0, st, a); break;
+  }
+  CTHIP_LAUNCH_CHECK();
+  return 0;
+}
+
+int launch_dec_mlp(const DecMlpArgs &a, int F, int H) {
+  const int D = a.st.D, KC = D / 256;
+  if (D % 256 || KC < 1 || KC > 4 || F % 32) return fail(CTHIP_E_BAD_ARG, "decoder: fused MLP launch with D = %d, F = %d", D, F);
+  dim3 grid(F / 16), block(256);
+  hipStream_t st = state().stream;
+#define GO2(KC_, NP_) hipLaunchKernelGGL((k_dec_mlp<KC_, NP_>), grid, block, 0, st, a)
+#define GO(KC_)                   \
+  case KC_:                       \
+    if (H == 4) GO2(KC_, 4);      \
+    else if (H == 8) GO2(KC_, 8); \
+    else if (H == 12) GO2(KC_, 12); \
+    else if (H == 16) GO2(KC_, 16); \
+    else return fail(CTHIP_E_BAD_ARG, "decoder: fused MLP launch with %d heads", H); \
+    break
+  switch (KC) {
+    GO(1);
+    GO(2);
+    GO(3);
+    GO(4);
+  }
+#undef GO
+#undef GO2
+  CTHIP_LAUNCH_CHECK();
+  return 0;
+}
+
+int launch_dec_sum(const DecStage &s, float *out) {
+  hipLaunchKernelGGL(k_dec_sum, dim3(1), dim3(256), 0, state().stream, s, out);
+  CTHIP_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // namespace cthip

@@ -29,6 +29,7 @@
 #include <vector>
 
 #include "common.h"
+#include "decode_fused.h"
 
 namespace cthip {
 
@@ -61,6 +62,8 @@ struct Layer {
   // Llama: attn = wq|wk|wv, proj = wo, fc = gate|up, fc2 = down, ln1_g/ln2_g = rms weights
   bool fc_pairs = false;  // gate / up rows interleaved, SwiGLU in the gate|up launch
   float *k_cache = nullptr, *v_cache = nullptr;
+  // three-launch decode layer: attn.c_proj by head and mlp.c_proj by 16-column slab (quant / scale planes)
+  void *proj_hq = nullptr, *proj_hd = nullptr, *fc2_sq = nullptr, *fc2_sd = nullptr;
 };
 
 struct Decoder {
@@ -85,6 +88,11 @@ struct Decoder {
   int position = 0;
   bool primed = false;  // a forward has left token/position on the device
   bool use_graph = true;
+  // the three-launch decode layer (decode_fused.hip): second residual buffer, per-head partials of the
+  // attention projection, per-XCD accumulators of the MLP projection
+  bool fused = false;
+  float *x2 = nullptr, *patt = nullptr;
+  long long *pmlp = nullptr;
   hipGraphExec_t g_step = nullptr, g_body = nullptr, g_multi = nullptr;
   int64_t weight_bytes = 0, vector_bytes = 0;
   std::vector<void *> owned;  // device blocks to free
@@ -310,8 +318,31 @@ static int finalize(Decoder *d) {
     for (WMat *w : ws)
       if (w) w->stream = total > kInfinityCacheBytes / 4 * 3;
   }
-  const char *ng = getenv("CTHIP_NO_GRAPH");
-  if (ng && *ng && *ng != '0') d->use_graph = false;
+  if (c.arch == CTHIP_ARCH_GPT2 && state().decode_fused &&
+      dec_fused_supported(d->layers[0].attn->type, d->layers[0].proj->type, d->layers[0].fc->type,
+                          d->layers[0].fc2->type, D, c.n_heads, F)) {
+    // the per-XCD accumulators assume what gfx950 has: XCD ids 0..7
+    int max_id = -1;
+    TRY(dec_xcd_probe(&max_id));
+    d->fused = max_id >= 0 && max_id < kDecXcds;
+    for (int l = 0; l < c.n_layers && d->fused; l++) {
+      Layer &L = d->layers[l];
+      if (L.attn->type != CTHIP_Q8_0 || L.proj->type != CTHIP_Q8_0 || L.fc->type != CTHIP_Q8_0 || L.fc2->type != CTHIP_Q8_0)
+        d->fused = false;
+    }
+    if (d->fused) {
+      for (int l = 0; l < c.n_layers; l++) {
+        Layer &L = d->layers[l];
+        TRY(dec_relay_heads(L.proj, D / c.n_heads, &L.proj_hq, &L.proj_hd));
+        TRY(dec_relay_slabs(L.fc2, &L.fc2_sq, &L.fc2_sd));
+        d->owned.insert(d->owned.end(), {L.proj_hq, L.proj_hd, L.fc2_sq, L.fc2_sd});
+      }
+      TRY(dev_alloc(d, (void **)&d->x2, sizeof(float) * D));
+      TRY(dev_alloc(d, (void **)&d->patt, sizeof(float) * (size_t)c.n_heads * D));
+      TRY(dev_alloc(d, (void **)&d->pmlp, sizeof(long long) * (size_t)kDecXcds * D));
+    }
+  }
+  if (!state().decoder_graph) d->use_graph = false;
   if (d->use_graph) {
     hipStream_t st = state().stream;
     // 0: one step with the head; 1: one step without (prompt rows fed one by one); 2: kStepsPerGraph steps
@@ -351,6 +382,66 @@ static int queue_step(Decoder *d, bool with_head, bool embed) {
   const bool gpt2 = c.arch == CTHIP_ARCH_GPT2;
   // embed = false: the previous step's head has already gathered this step's input (queue_head)
   if (embed) TRY(launch_embedding(d->x, d->wte, nullptr, tok, 1, V, D, gpt2 ? d->wpe : nullptr, pos, c.max_seq));
+  if (d->fused) {
+    // Three launches per layer.  The residual stream alternates between d->x and d->x2 as "base + bias +
+    // partials": each launch adds up what its predecessor left and block 0 stores the sum for the launch after.
+    for (int l = 0; l < c.n_layers; l++) {
+      Layer &L = d->layers[l];
+      DecQkvArgs qa = {};
+      qa.st.base = d->x;
+      qa.st.bias = l ? d->layers[l - 1].fc2_b : nullptr;
+      qa.st.iparts = d->pmlp;
+      qa.st.gamma = L.ln1_g;
+      qa.st.xout = d->x2;
+      qa.st.eps = c.eps;
+      qa.st.D = D;
+      qa.wq = L.attn->q;
+      qa.wd = (const unsigned short *)L.attn->d;
+      qa.fold_s = L.attn_s;
+      qa.fold_c = L.attn_c;
+      qa.q = d->q;
+      qa.kc = L.k_cache;
+      qa.vc = L.v_cache;
+      qa.pos = pos;
+      qa.rows = 3 * D;
+      TRY(launch_dec_qkv(qa, l > 0));
+      DecAttnArgs aa = {};
+      aa.q = d->q;
+      aa.kc = L.k_cache;
+      aa.vc = L.v_cache;
+      aa.pos = pos;
+      aa.pq = L.proj_hq;
+      aa.pd = (const unsigned short *)L.proj_hd;
+      aa.part = d->patt;
+      aa.zero = d->pmlp;
+      aa.zero_n16 = (int64_t)kDecXcds * D * 8 / 16;
+      TRY(launch_dec_attn_proj(aa, c.n_heads, D));
+      DecMlpArgs ma = {};
+      ma.st.base = d->x2;
+      ma.st.bias = L.proj_b;
+      ma.st.fparts = d->patt;
+      ma.st.gamma = L.ln2_g;
+      ma.st.xout = d->x;
+      ma.st.eps = c.eps;
+      ma.st.D = D;
+      ma.wq = L.fc->q;
+      ma.wd = (const unsigned short *)L.fc->d;
+      ma.fold_s = L.fc_s;
+      ma.fold_c = L.fc_c;
+      ma.pq = L.fc2_sq;
+      ma.pd = (const unsigned short *)L.fc2_sd;
+      ma.accum = d->pmlp;
+      TRY(launch_dec_mlp(ma, F, c.n_heads));
+    }
+    DecStage fin = {};
+    fin.base = d->x;
+    fin.bias = d->layers[c.n_layers - 1].fc2_b;
+    fin.iparts = d->pmlp;
+    fin.D = D;
+    TRY(launch_dec_sum(fin, d->x));
+    if (with_head) TRY(queue_head(d));
+    return 0;
+  }
   for (int l = 0; l < c.n_layers; l++) {
     Layer &L = d->layers[l];
     GemvArgs a = {};
@@ -642,8 +733,7 @@ int cthip_decoder_forward(void *dec, const float *tokens, int s, int n, int64_t 
     const float tf = tokens[i];
     ids[i] = (tf >= 0.0f && tf < (float)c.vocab && (float)(int)tf == tf) ? (int)tf : -1;
   }
-  const char *np = getenv("CTHIP_NO_PREFILL_GEMM");
-  if (s >= kPrefillMin && !(np && *np && *np != '0')) {
+  if (s >= kPrefillMin && state().prefill_gemm) {
     if ((rc = prefill(d, ids.data(), s, n))) return rc;
   } else {
     for (int i = 0; i < s; i++) {

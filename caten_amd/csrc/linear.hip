@@ -406,8 +406,6 @@ int launch_gemv(const WMat *w, GemvArgs a, int m) {
       // staged launches pay the input staging once per workgroup: whole workgroups per compute unit, two
       // when there is work for more than one (measured best; a third does not fit beside the first two)
       if (stage && wanted > base && occ_cache[vi] >= 2) wanted = 2 * base;
-      static const char *ovr = getenv("CTHIP_GEMV_WAVES");  // tuning aid: overrides the wavefront count
-      if (ovr && atoi(ovr) > 0) wanted = atoi(ovr);
       const int iters = (nrq + wanted - 1) / wanted;
       // every resident wavefront slot is used even if some wavefronts then loop once more than others: with equal
       // iteration counts (12 565 tiles of the GPT-2 lm_head on 1 795 wavefronts of seven) a quarter of the compute units
@@ -667,6 +665,13 @@ int cthip_set_option(const char *name, int value) {
   if (!strcmp(name, "gemv_stream_weights")) {
     if (value < -1 || value > 1) return fail(CTHIP_E_BAD_ARG, "cthip_set_option: gemv_stream_weights is -1, 0 or 1");
     state().gemv_stream = value;
+    return 0;
+  }
+  if (!strcmp(name, "decoder_graph") || !strcmp(name, "prefill_gemm") || !strcmp(name, "decode_fused")) {
+    if (value != 0 && value != 1) return fail(CTHIP_E_BAD_ARG, "cthip_set_option: %s is 0 or 1", name);
+    if (!strcmp(name, "decoder_graph")) state().decoder_graph = value;
+    else if (!strcmp(name, "prefill_gemm")) state().prefill_gemm = value;
+    else state().decode_fused = value;
     return 0;
   }
   if (!strcmp(name, "gemm_bf16")) {  // 1 = operands rounded to bf16, 0 = back to the default

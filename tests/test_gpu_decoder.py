@@ -134,6 +134,33 @@ def test_streamed_weights_decode_identical(arch):
         assert np.array_equal(a, b)
 
 
+@pytest.mark.parametrize("name,plen", [("gpt2-tiny", 5), ("gpt2-mini", 40)])
+def test_three_launch_layer_equals_five_launch_layer(name, plen):
+    """The decode layer as three launches (attention + its projection, and the whole MLP, one launch each, partial
+    vectors added up by the consumer) and as five launches (one per Linear) are the same function: identical greedy
+    tokens, logits inside the fp32 band, and -- the per-XCD accumulators being integers -- bit-identical logits
+    from one run of the three-launch layer to the next."""
+    print(f"case: three-launch vs five-launch layer {name}", flush=True)
+    from caten_amd import _lib, synth, llm
+    lib = _lib.load()
+    cfg = synth.GPT2_CONFIGS[name]
+    sd = llm.gpt2_state_dict(synth.gpt2_weights(cfg, seed=11), "q8_0")
+    prompt = synth.prompt(cfg["vocab"], plen, seed=11)
+    runs = []
+    try:
+        for mode in (1, 0, 1):
+            _lib.check(lib.cthip_set_option(b"decode_fused", mode))
+            model = llm.make_gpt2(cfg, sd)
+            runs.append(llm.gpt2_generate(model, prompt, 20, on_device=False, keep_logits=True))
+            model.close()
+    finally:
+        _lib.check(lib.cthip_set_option(b"decode_fused", 1))
+    assert runs[0][0] == runs[1][0] == runs[2][0]
+    for a, b, c in zip(*[r[1] for r in runs]):
+        close(a, b)
+        assert np.array_equal(a, c)
+
+
 def test_gpt2_prompt_lengths_and_restart(oracle):
     from caten_amd import synth, llm
     cfg = synth.GPT2_CONFIGS["gpt2-tiny"]
@@ -209,7 +236,6 @@ def test_prefill_batch_equals_token_by_token(oracle):
     """A prompt pushed through one forward as a batch (MFMA GEMMs) and the same prompt fed row by row
     through the decode step are the same function: identical greedy tokens, logits and cache rows
     within the fp32 band; with bf16 MFMA operands within the 1e-2 band."""
-    import os
     from caten_amd import synth, llm, _lib
     cfg = synth.GPT2_CONFIGS["gpt2-mini"]
     w = synth.gpt2_weights(cfg, seed=2)
@@ -218,12 +244,13 @@ def test_prefill_batch_equals_token_by_token(oracle):
     x = [float(t) for t in prompt]
     m1 = llm.make_gpt2(cfg, sd)
     tok1, lg1 = m1.forward(x, len(x), 0, return_logits=True)
-    os.environ["CTHIP_NO_PREFILL_GEMM"] = "1"
+    lib = _lib.load()
+    _lib.check(lib.cthip_set_option(b"prefill_gemm", 0))
     try:
         m2 = llm.make_gpt2(cfg, sd)
         tok2, lg2 = m2.forward(x, len(x), 0, return_logits=True)
     finally:
-        del os.environ["CTHIP_NO_PREFILL_GEMM"]
+        _lib.check(lib.cthip_set_option(b"prefill_gemm", 1))
     assert tok1 == tok2
     close(lg1, lg2)
     close(m1.peek("k_cache.2")[:100 * cfg["dim"]], m2.peek("k_cache.2")[:100 * cfg["dim"]])
@@ -233,11 +260,11 @@ def test_prefill_batch_equals_token_by_token(oracle):
     # prefill appended to an existing sequence (n > 0)
     more = [float(t) for t in synth.prompt(cfg["vocab"], 9, seed=4)]
     ta, la = m1.forward(more, 9, m1.position, return_logits=True)
-    os.environ["CTHIP_NO_PREFILL_GEMM"] = "1"
+    _lib.check(lib.cthip_set_option(b"prefill_gemm", 0))
     try:
         tb, lb = m2.forward(more, 9, m2.position, return_logits=True)
     finally:
-        del os.environ["CTHIP_NO_PREFILL_GEMM"]
+        _lib.check(lib.cthip_set_option(b"prefill_gemm", 1))
     assert ta == tb
     close(la, lb)
     m1.close()

@@ -3,14 +3,14 @@
 
 A "step" is one decode step (one token).  Weights, KV cache, token and position are resident in
 HBM before the timed region; the timed region is K back-to-back steps of the device-resident loop
-(cthip_decoder_generate), bracketed by stream synchronisation, host wall clock.  `roofline` is
-the dominant kernel of a step -- the dequant-in-register GEMV, on its largest launch (lm_head,
-50257x768, 31 % of a step's bytes) -- measured with HIP events on the library's stream:
-algorithmic bytes (packed weights + input + output) over the average launch duration, against
-8 TB/s; `roofline.step` gives the same ratio for the whole step (one hipGraph replay: packed
-weights + norms/biases + embedding rows + KV rows).  `cpu_baseline` times the CPU oracle (a single-thread C
-restatement of Caten's BACKEND=CLANG kernels, incl. its one-hot embedding and 3-reduction argmax)
-on the host cores, on a bounded sample of the same workload.
+(cthip_decoder_generate), bracketed by stream synchronisation, host wall clock.  `roofline` is the
+whole step: algorithmic bytes of one token (packed weights + norms/biases + embedding rows + KV rows)
+over the step time measured with HIP events on the library's stream, against 8 TB/s; its `lm_head`
+entry gives the step's largest launch (50257x768, 31 % of the bytes) alone, once back to back on one
+matrix (which then sits in the Infinity Cache) and once rotating over enough copies that every launch
+streams from HBM.  `cpu_baseline` times the CPU oracle (a single-thread C restatement of Caten's
+BACKEND=CLANG kernels, incl. its one-hot embedding and 3-reduction argmax) on the host cores, on a
+bounded sample of the same workload.
 """
 import argparse
 import json
@@ -24,9 +24,20 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
-# (profiles/), scaled by a copy kernel of known size; None where it has not been measured.
-TRAFFIC_BYTES = {("gpt2", "q8_0"): 44608512}  # profiles/gemv_q8_0_lm_head_pmc.txt
+
+
+def profile_traffic(model, kind):
+    """HBM-side bytes of one decode step (FETCH_SIZE + WRITE_SIZE summed over the step's dispatches, scaled by a copy
+    of known size) as recorded in the committed rocprofv3 --pmc summary of this workload; None if there is none."""
+    path = os.path.join(ROOT, "profiles", f"decode_{model}_{kind}_step_pmc.txt")
+    try:
+        with open(path) as f:
+            for line in f:
+                if line.startswith("step_traffic_bytes:"):
+                    return int(float(line.split(":", 1)[1].split()[0]))
+    except OSError:
+        pass
+    return None
 
 
 def cpu_baseline(cfg, weights, prompt, budget_s, kind, llama):
@@ -70,6 +81,8 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU baseline budget (0 disables)")
     ap.add_argument("--no-graph", action="store_true",
                     help="launch the step's kernels one by one instead of replaying the hipGraph (for kernel tracing)")
+    ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
+                    help="library option set before the model is built (cthip_set_option), e.g. decode_fused=0")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (a kernel of known traffic to scale "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings by)")
@@ -92,6 +105,9 @@ def main():
     lib = _lib.init(0)
     if args.no_graph:
         _lib.check(lib.cthip_set_option(b"decoder_graph", 0))
+    for kv in args.option:
+        name, value = kv.split("=")
+        _lib.check(lib.cthip_set_option(name.encode(), int(value)))
     model = (llm.make_llama(cfg, llm.llama_state_dict(weights, args.kind)) if llama
              else llm.make_gpt2(cfg, llm.gpt2_state_dict(weights, args.kind)))
 
@@ -141,28 +157,40 @@ def main():
     step_bytes = float(np.mean([model.step_bytes(t + 1) for t in range(pos0, pos0 + k)]))
     step_gbs = step_bytes / (step_us * 1e-6) / 1e9
 
-    # ---- the dominant kernel on its largest launch: ln_f -> lm_head GEMV (+ per-wavefront argmax partials) ----
+    # ---- the largest single launch of a step: ln_f -> lm_head GEMV (+ per-wavefront argmax partials) ----
+    # "warm": the same matrix back to back -- 41 MB stay in the 256 MB Infinity Cache, so this is a cache-fed figure;
+    # "cold": the launches rotate over enough copies of the matrix (> 256 MB together) that every one streams from HBM.
     from caten_amd import ops
     from caten_amd.llm import Tensor
     V, D = cfg["vocab"], cfg["dim"]
     t = Tensor.from_f32(weights["lm_head"], args.kind)
-    wm = ops.WeightMatrix(args.kind, t.raw, V, D)
+    wm0 = ops.WeightMatrix(args.kind, t.raw, V, D)
+    ncopies = max(2, int(np.ceil(1.25 * (256 << 20) / wm0.nbytes)))
+    wms = [wm0] + [ops.WeightMatrix(args.kind, t.raw, V, D) for _ in range(ncopies - 1)]
     dx = ops.DeviceArray.from_numpy(np.random.default_rng(1).normal(size=D).astype(np.float32))
     dg = ops.DeviceArray.from_numpy(weights["norm_w" if llama else "lnf_g"])
     db = None if llama else ops.DeviceArray.from_numpy(weights["lnf_b"])
     pro = _lib.PRO_RMSNORM if llama else _lib.PRO_LAYERNORM  # the final norm of the model, fused as the decode step fuses it
     dy = ops.DeviceArray((V,), np.float32)
-    reps = 200
-    for _ in range(20):
-        _lib.check(lib.cthip_linear(dy.ptr, wm.handle, dx.ptr, 1, None, None, 0, pro, dg.ptr, db.ptr if db else None, 1e-5))
-    _lib.check(lib.cthip_sync())
-    _lib.check(lib.cthip_timer_start())
-    for _ in range(reps):
-        _lib.check(lib.cthip_linear(dy.ptr, wm.handle, dx.ptr, 1, None, None, 0, pro, dg.ptr, db.ptr if db else None, 1e-5))
-    _lib.check(lib.cthip_timer_stop(C.byref(ms)))
-    gemv_us = ms.value * 1e3 / reps
-    gemv_bytes = wm.nbytes + 4 * ((2 if llama else 3) * D + V)  # packed weights + x, gamma (, beta) + logits
-    achieved = gemv_bytes / (gemv_us * 1e-6) / 1e9
+    gemv_bytes = wm0.nbytes + 4 * ((2 if llama else 3) * D + V)  # packed weights + x, gamma (, beta) + logits
+
+    def time_lm_head(mats, reps):
+        for i in range(2 * len(mats)):
+            _lib.check(lib.cthip_linear(dy.ptr, mats[i % len(mats)].handle, dx.ptr, 1, None, None, 0, pro, dg.ptr,
+                                        db.ptr if db else None, 1e-5))
+        _lib.check(lib.cthip_sync())
+        _lib.check(lib.cthip_timer_start())
+        for i in range(reps):
+            _lib.check(lib.cthip_linear(dy.ptr, mats[i % len(mats)].handle, dx.ptr, 1, None, None, 0, pro, dg.ptr,
+                                        db.ptr if db else None, 1e-5))
+        _lib.check(lib.cthip_timer_stop(C.byref(ms)))
+        us = ms.value * 1e3 / reps
+        gbs = gemv_bytes / (us * 1e-6) / 1e9
+        return {"us_per_launch": us, "achieved": gbs, "frac": gbs / HBM_PEAK_GBS}
+    lm_warm = time_lm_head(wms[:1], 200)
+    lm_cold = time_lm_head(wms, 25 * len(wms))
+    lm_cold["copies"] = len(wms)
+    traffic = profile_traffic(args.model, args.kind)
 
     res = {
         "metric": "decode tokens/sec at batch 1 on 1 MI355X; fused-kernel HBM GB/s vs peak",
@@ -175,13 +203,15 @@ def main():
                                f"{args.prompt}-token prompt, batch-1 greedy decode, positions {min(positions)}..{max(positions)}",
                    "shape": args.model, "weight_format": args.kind, "prompt_tokens": args.prompt,
                    "positions": f"{min(positions)}..{max(positions)}"},
-        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": TRAFFIC_BYTES.get((args.model, args.kind)),
-                     "kernel": f"cthip::k_gemv<{args.kind}> on lm_head ({V}x{D}) with the {'RMSNorm' if llama else 'ln_f'} prologue",
-                     "bytes_per_launch": gemv_bytes, "us_per_launch": gemv_us,
-                     "step": {"bytes": step_bytes, "us": step_us, "achieved": step_gbs,
-                              "frac": step_gbs / HBM_PEAK_GBS,
-                              "what": "one decode step = one hipGraph replay of every fused launch"}},
+        # the whole decode step: every launch of one token, HIP events on the library's stream around K steps
+        "roofline": {"bound": "hbm", "achieved": step_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": step_gbs / HBM_PEAK_GBS, "traffic": traffic,
+                     "kernel": "one decode step = one replay of the step's launches (the dequant-in-register Linear "
+                               "kernels, attention, argmax), packed weights + norms / biases + embedding rows + KV rows",
+                     "bytes_per_launch": step_bytes, "us_per_launch": step_us,
+                     "lm_head": {"kernel": f"cthip::k_gemv<{args.kind}> on lm_head ({V}x{D}) with the "
+                                           f"{'RMSNorm' if llama else 'ln_f'} prologue, the step's largest launch",
+                                 "bytes_per_launch": gemv_bytes, "warm_infinity_cache": lm_warm, "cold_hbm": lm_cold}},
     }
     if args.calibrate_copy:
         n = 256 << 20

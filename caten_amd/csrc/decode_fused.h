@@ -53,7 +53,7 @@ int dec_xcd_probe(int *max_id);
 int dec_relay_heads(const WMat *w, int DH, void **pq, void **pd);
 int dec_relay_slabs(const WMat *w, void **pq, void **pd);
 int launch_dec_qkv(const DecQkvArgs &a, bool from_accum);
-int launch_dec_attn_proj(const DecAttnArgs &a, int H, int D);
+int launch_dec_attn_proj(const DecAttnArgs &a, int H, int D, int replicas);
 int launch_dec_mlp(const DecMlpArgs &a, int F, int H);
 int launch_dec_sum(const DecStage &s, float *out);
 

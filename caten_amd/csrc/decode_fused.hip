@@ -3,8 +3,8 @@
 // bytes, so two pairs of consecutive Linears are merged around the vector that sits between them:
 //
 //   k_dec_qkv        x -> LayerNorm1 -> c_attn (+bias): q to a buffer, k / v rows into the cache at `pos`
-//   k_dec_attn_proj  one workgroup per head: attention over cache rows 0..pos, then that head's 64 columns
-//                    of attn.c_proj applied to its 64 outputs -> one partial vector per head
+//   k_dec_attn_proj  four workgroups per head: attention over cache rows 0..pos, then a quarter of the rows of
+//                    that head's 64 columns of attn.c_proj applied to its 64 outputs -> one partial vector per head
 //   k_dec_mlp        one workgroup per 16 hidden units: LayerNorm2 -> those rows of c_fc (+bias, GELU) ->
 //                    their 16 columns of mlp.c_proj -> partial vector, added into one accumulator per XCD
 //
@@ -39,7 +39,7 @@ __device__ __forceinline__ float4 f4add(float4 a, float4 b) { return make_float4
 
 // Assembles the launch's input vector  x = base + bias + sum(partials)  (one float4 per thread, D <= 1024),
 // writes gamma * x to LDS and returns the LayerNorm statistics of x; block 0 also stores x to s.xout.
-// MODE 0: base only; 1: + bias + NP fp32 partial vectors; 2: + bias + kDecXcds fixed-point accumulators.
+// MODE 0: base only; 1: + bias + NP fp32 partial vectors; 2: + bias + NP fixed-point accumulators.
 // Every load is unconditional and issued before any use.  red holds 24 floats.  blockDim.x == 256.
 template <int MODE, int NP>
 __device__ __forceinline__ void dec_stage(const DecStage &s, float *xs, float *red, float &mu, float &rstd) {
@@ -59,16 +59,16 @@ __device__ __forceinline__ void dec_stage(const DecStage &s, float *xs, float *r
 #pragma unroll
       for (int k = 0; k < NP; k++) v = f4add(v, p[k]);
     } else {
-      longlong2 lo[kDecXcds], hi[kDecXcds];
+      longlong2 lo[NP], hi[NP];
 #pragma unroll
-      for (int k = 0; k < kDecXcds; k++) {
+      for (int k = 0; k < NP; k++) {
         const longlong2 *src = (const longlong2 *)(s.iparts + (int64_t)k * s.D) + 2 * i;
         lo[k] = src[0];
         hi[k] = src[1];
       }
       long long t0 = 0, t1 = 0, t2 = 0, t3 = 0;
 #pragma unroll
-      for (int k = 0; k < kDecXcds; k++) {
+      for (int k = 0; k < NP; k++) {
         t0 += lo[k].x;
         t1 += lo[k].y;
         t2 += hi[k].x;
@@ -135,7 +135,7 @@ __device__ __forceinline__ float dec_row_dot(const uint4 *w, const unsigned *sc,
 }
 
 // ---- launch 1: LayerNorm1 folded through c_attn; 16 rows per workgroup ----
-template <int KC, int MODE>
+template <int KC, int MODE, int NP>
 __global__ __launch_bounds__(256) void k_dec_qkv(DecQkvArgs a) {
   __shared__ __align__(16) float xs[256 * KC];
   __shared__ float red[24];
@@ -158,7 +158,7 @@ __global__ __launch_bounds__(256) void k_dec_qkv(DecQkvArgs a) {
   const float fs = a.fold_s[row], fc = a.fold_c[row];
   const int posv = a.pos[0];
   float mu, rstd;
-  dec_stage<MODE, 1>(a.st, xs, red, mu, rstd);
+  dec_stage<MODE, NP>(a.st, xs, red, mu, rstd);
   const float acc = dec_row_dot<KC>(w, sc, xs, l);
   if (l == 0 && row_ok) {
     // rstd * (W.(gamma x) - mu * W.gamma) + (W.beta + bias)  =  W.LayerNorm(x) + bias
@@ -186,14 +186,16 @@ void k_dec_attn_proj(DecAttnArgs a) {
   const int h = blockIdx.x, H = gridDim.x, D = H * DH;
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int g = lane / LPK, c = lane % LPK;
-  // the projection slab of this head
+  // The projection slab of this head.  gridDim.y workgroups per head repeat the head's attention and share the
+  // slab's rows: what one compute unit has to fetch bounds the launch, and the slab is most of it.
+  const int rr = D / (int)gridDim.y, rbase = (int)blockIdx.y * rr;  // this workgroup's rows of the slab
   const int pc = tid % CPR, pr0 = tid / CPR;
   uint4 pw[JR];
   unsigned ps[JR];
 #pragma unroll
   for (int j = 0; j < JR; j++) {
     int r = pr0 + RPP * j;
-    r = r < D ? r : D - 1;
+    r = rbase + (r < rr ? r : rr - 1);
     pw[j] = ((const uint4 *)a.pq)[((int64_t)h * D + r) * CPR + pc];
     ps[j] = a.pd[((int64_t)h * D + r) * (DH / 32) + (pc >> 1)];
   }
@@ -207,7 +209,8 @@ void k_dec_attn_proj(DecAttnArgs a) {
   {
     uint4 *z = (uint4 *)a.zero;
     const uint4 zz = make_uint4(0u, 0u, 0u, 0u);
-    for (int64_t k = (int64_t)h * 1024 + tid; k < a.zero_n16; k += (int64_t)H * 1024) z[k] = zz;
+    const int64_t nthr = (int64_t)H * gridDim.y * 1024;
+    for (int64_t k = ((int64_t)blockIdx.y * H + h) * 1024 + tid; k < a.zero_n16; k += nthr) z[k] = zz;
   }
   float m = -INFINITY, lsum = 0.0f;
   float acc[4] = {0.f, 0.f, 0.f, 0.f};
@@ -301,7 +304,7 @@ void k_dec_attn_proj(DecAttnArgs a) {
     if (CPR >= 4) s += dpp_f<0x4E>(s);  // quad_perm [2,3,0,1]
     if (CPR >= 8) s += dpp_f<0x141>(s);  // row_half_mirror
     const int r = pr0 + RPP * j;
-    if (pc == 0 && r < D) a.part[(int64_t)h * D + r] = s;
+    if (pc == 0 && r < rr) a.part[(int64_t)h * D + rbase + r] = s;
   }
 }
 
@@ -354,7 +357,8 @@ __global__ __launch_bounds__(256) void k_dec_mlp(DecMlpArgs a) {
 #pragma unroll
   for (int j = 0; j < KC; j++) {
     const float s = chunk_dot<CTHIP_Q8_0>(pw[j], half_bits_to_float((unsigned short)ps[j]), hr, 0.0f);
-    // no device-scope bits: the addition happens in this XCD's L2
+    // no device-scope bits: the addition happens in this XCD's L2.  (One device-wide accumulator instead of
+    // one per XCD costs the 192 workgroups more in contention than the seven arrays cost the reader.)
     __hip_atomic_fetch_add(accum + tid + 256 * j, __float2ll_rn(s * kFixScale), __ATOMIC_RELAXED,
                            __HIP_MEMORY_SCOPE_WORKGROUP);
   }
@@ -474,10 +478,10 @@ int launch_dec_qkv(const DecQkvArgs &a, bool from_accum) {
   if (D % 256 || KC < 1 || KC > 4 || a.rows != 3 * D) return fail(CTHIP_E_BAD_ARG, "decoder: fused qkv launch with D = %d, rows = %d", D, a.rows);
   dim3 grid((a.rows + 15) / 16), block(256);
   hipStream_t st = state().stream;
-#define GO(KC_)                                                                        \
-  case KC_:                                                                            \
-    if (from_accum) hipLaunchKernelGGL((k_dec_qkv<KC_, 2>), grid, block, 0, st, a);    \
-    else hipLaunchKernelGGL((k_dec_qkv<KC_, 0>), grid, block, 0, st, a);               \
+#define GO(KC_)                                                                                  \
+  case KC_:                                                                                      \
+    if (from_accum) hipLaunchKernelGGL((k_dec_qkv<KC_, 2, kDecXcds>), grid, block, 0, st, a);    \
+    else hipLaunchKernelGGL((k_dec_qkv<KC_, 0, 1>), grid, block, 0, st, a);                      \
     break
   switch (KC) {
     GO(1);
@@ -490,12 +494,13 @@ int launch_dec_qkv(const DecQkvArgs &a, bool from_accum) {
   return 0;
 }
 
-int launch_dec_attn_proj(const DecAttnArgs &a, int H, int D) {
-  if (D != H * 64 || D > 1024) return fail(CTHIP_E_BAD_ARG, "decoder: fused attention launch with D = %d, H = %d", D, H);
-  dim3 grid(H), block(1024);
+int launch_dec_attn_proj(const DecAttnArgs &a, int H, int D, int replicas) {
+  if (D != H * 64 || D > 1024 || replicas < 1 || D % replicas)
+    return fail(CTHIP_E_BAD_ARG, "decoder: fused attention launch with D = %d, H = %d, %d workgroups per head", D, H, replicas);
+  dim3 grid(H, replicas), block(1024);
   hipStream_t st = state().stream;
-  // rows of the projection slab per thread: D / (1024 / 4)
-  switch ((D + 255) / 256) {
+  // rows of the projection slab per thread: (D / replicas) rows of 4 chunks over 1024 threads
+  switch ((D / replicas + 255) / 256) {
     case 1: hipLaunchKernelGGL((k_dec_attn_proj<64, 1>), grid, block, 0, st, a); break;
     case 2: hipLaunchKernelGGL((k_dec_attn_proj<64, 2>), grid, block, 0, st, a); break;
     case 3: hipLaunchKernelGGL((k_dec_attn_proj<64, 3>), grid, block, 0, st, a); break;
@@ -511,10 +516,10 @@ int launch_dec_mlp(const DecMlpArgs &a, int F, int H) {
   dim3 grid(F / 16), block(256);
   hipStream_t st = state().stream;
 #define GO2(KC_, NP_) hipLaunchKernelGGL((k_dec_mlp<KC_, NP_>), grid, block, 0, st, a)
-#define GO(KC_)                   \
-  case KC_:                       \
-    if (H == 4) GO2(KC_, 4);      \
-    else if (H == 8) GO2(KC_, 8); \
+#define GO(KC_)                     \
+  case KC_:                         \
+    if (H == 4) GO2(KC_, 4);        \
+    else if (H == 8) GO2(KC_, 8);   \
     else if (H == 12) GO2(KC_, 12); \
     else if (H == 16) GO2(KC_, 16); \
     else return fail(CTHIP_E_BAD_ARG, "decoder: fused MLP launch with %d heads", H); \

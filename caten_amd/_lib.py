@@ -70,6 +70,7 @@ PROTOTYPES = {
     "cthip_linear": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _i, _i, _vp, _vp, _f]),
     "cthip_set_option": (_i, [C.c_char_p, _i]),
     "cthip_matmul": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i]),
+    "cthip_matmul_noalloc": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i]),
     "cthip_softmax": (_i, [_vp, _vp, _i64, _i]),
     "cthip_layernorm": (_i, [_vp, _vp, _vp, _vp, _f, _i64, _i]),
     "cthip_rmsnorm": (_i, [_vp, _vp, _vp, _f, _i64, _i]),

@@ -140,6 +140,8 @@ int launch_argmax(int64_t *out, const float *x, int64_t rows, int n, int *tok_ou
 enum { GEMM_FP32 = 0, GEMM_BF16 = 1, GEMM_BF16X3 = 2, GEMM_BF16X6 = 3 };
 int launch_linear_gemm(float *y, const WMat *w, const float *x, int m, const float *bias, const float *residual,
                        int act, int precision);
+// takes the device address of the static split-K scratch of cthip_matmul_noalloc (once per device, that device current)
+int matmul_scratch_init(int device);
 // gate|up rows (m, 2*cols) -> silu(gate)*up (m, cols), or a norm, as a launch of its own
 int launch_prologue(float *out, const float *x, int cols, int pro, const float *g, const float *b, float eps,
                     int64_t x_stride, int m);

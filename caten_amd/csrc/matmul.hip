@@ -741,7 +741,26 @@ __global__ __launch_bounds__(256) void k_splitk_reduce(GemmArgs a) {
 // precision: GEMM_FP32 = fp32 MFMA operands (k_gemm_f32), GEMM_BF16 = operands rounded to bf16,
 // GEMM_BF16X3 / GEMM_BF16X6 = operands split in two / three bf16 terms.  Q8_0 / Q4_0 weights take k_gemm_q
 // (integer plane exact in bf16, block scales applied to the partial sums) with 1 / 2 / 3 activation terms.
-int launch_gemm(GemmArgs a, int bmode, int precision) {
+// Split-K partial tiles of the entry point that allocates nothing (cthip_matmul_noalloc): one array per device,
+// held until the process ends.  In host code the name below is only a stand-in; the device address is taken
+// once per device with hipGetSymbolAddress (matmul_scratch_init, called by cthip_init) and kept in g_scratch_ptr.
+constexpr size_t kScratchBytes = 4ull << 20;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+constexpr int kMaxDevices = 64;
+static float *g_scratch_ptr[kMaxDevices] = {};
+
+int matmul_scratch_init(int device) {
+  if (device < 0 || device >= kMaxDevices) return fail(CTHIP_E_BAD_ARG, "cthip_init: device %d is beyond the %d this library keeps scratch for", device, kMaxDevices);
+  if (g_scratch_ptr[device]) return 0;
+  void *p = nullptr;
+  CTHIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+  g_scratch_ptr[device] = (float *)p;
+  return 0;
+}
+
+// static_ws: null = split-K partials come from the caching allocator; otherwise they go to this buffer of
+// static_ws_bytes bytes and nothing is allocated or freed
+int launch_gemm(GemmArgs a, int bmode, int precision, float *static_ws, size_t static_ws_bytes) {
   if (a.M == 0 || a.N == 0) return 0;
   hipStream_t st = state().stream;
   const int cus = state().compute_units;
@@ -788,8 +807,16 @@ int launch_gemm(GemmArgs a, int bmode, int precision) {
       a.kper = steps_per * 64;
       a.ksplit = (nsteps + steps_per - 1) / steps_per;
       if (a.ksplit > 1) {
-        int rc = alloc_scratch((void **)&a.ws, sizeof(float) * (size_t)a.ksplit * a.M * a.N);
-        if (rc) return rc;
+        const size_t need = sizeof(float) * (size_t)a.ksplit * a.M * a.N;
+        if (static_ws) {
+          if (need > static_ws_bytes)
+            return fail(CTHIP_E_UNSUPPORTED, "cthip_matmul_noalloc: (%d,%d,%d) splits its reduction %d ways and needs %zu bytes of partial "
+                        "tiles; the static scratch holds %zu (use cthip_matmul)", a.M, a.N, a.K, a.ksplit, need, static_ws_bytes);
+          a.ws = static_ws;  // every element of every share is written before the reduction reads it
+        } else {
+          int rc = alloc_scratch((void **)&a.ws, need);
+          if (rc) return rc;
+        }
         grid.y = a.ksplit;
       } else {
         a.kper = a.K;
@@ -847,7 +874,7 @@ int launch_gemm(GemmArgs a, int bmode, int precision) {
   }
   hipError_t le = hipGetLastError();
   if (le != hipSuccess) {
-    if (a.ws) cthip_free(a.ws);
+    if (a.ws && !static_ws) cthip_free(a.ws);
     return fail((int)le, "gemm: launch -> %s", hipGetErrorString(le));
   }
   if (a.ksplit > 1) {
@@ -855,7 +882,7 @@ int launch_gemm(GemmArgs a, int bmode, int precision) {
     if (blocks > 4096) blocks = 4096;
     hipLaunchKernelGGL(k_splitk_reduce, dim3((unsigned)blocks), dim3(256), 0, st, a);
     le = hipGetLastError();
-    int rc = cthip_free(a.ws);  // stream-ordered: the block is reused only by later work on the same stream
+    int rc = static_ws ? 0 : cthip_free(a.ws);  // stream-ordered: the block is reused only by later work on the same stream
     if (le != hipSuccess) return fail((int)le, "gemm: launch -> %s", hipGetErrorString(le));
     return rc;
   }
@@ -877,14 +904,14 @@ int launch_linear_gemm(float *y, const WMat *w, const float *x, int m, const flo
   a.N = (int)w->rows;
   a.K = (int)w->cols;
   a.act = act;
-  return launch_gemm(a, B_WMAT, precision);
+  return launch_gemm(a, B_WMAT, precision, nullptr, 0);
 }
 
 }  // namespace cthip
 
 using namespace cthip;
 
-extern "C" int cthip_matmul(float *C, const float *A, const float *B, int M, int N, int K, int act, int precision) {
+static int matmul_entry(float *C, const float *A, const float *B, int M, int N, int K, int act, int precision, bool noalloc) {
   CTHIP_REQUIRE_INIT();
   CTHIP_ARG(M >= 0 && N >= 0 && K >= 0);
   CTHIP_ARG((int64_t)M * N == 0 || (C != nullptr && (K == 0 || (A != nullptr && B != nullptr))));
@@ -898,5 +925,16 @@ extern "C" int cthip_matmul(float *C, const float *A, const float *B, int M, int
   a.N = N;
   a.K = K;
   a.act = act;
-  return launch_gemm(a, B_ROWMAJOR, precision);
+  if (!noalloc) return launch_gemm(a, B_ROWMAJOR, precision, nullptr, 0);
+  float *ws = g_scratch_ptr[state().device];
+  if (!ws) return fail(CTHIP_E_STATE, "cthip_matmul_noalloc: no scratch address for device %d", state().device);
+  return launch_gemm(a, B_ROWMAJOR, precision, ws, kScratchBytes);
+}
+
+extern "C" int cthip_matmul(float *C, const float *A, const float *B, int M, int N, int K, int act, int precision) {
+  return matmul_entry(C, A, B, M, N, K, act, precision, false);
+}
+
+extern "C" int cthip_matmul_noalloc(float *C, const float *A, const float *B, int M, int N, int K, int act, int precision) {
+  return matmul_entry(C, A, B, M, N, K, act, precision, true);
 }

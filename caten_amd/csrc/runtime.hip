@@ -130,6 +130,10 @@ int cthip_init(int device) {
     CTHIP_CHECK(hipEventCreateWithFlags(&st.ev[i], hipEventDisableTiming));
     st.used[i] = false;
   }
+  {
+    int rc = matmul_scratch_init(device);
+    if (rc) return rc;
+  }
   s.device = device;
   s.inited = true;
   return 0;

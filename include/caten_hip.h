@@ -180,6 +180,13 @@ int cthip_set_option(const char *name, int value);
  * (2^-16 of a product is lost), 1 = bf16 MFMA operands (rtol/atol 1e-2); fp32 accumulation
  * in every mode. */
 int cthip_matmul(float *C, const float *A, const float *B, int M, int N, int K, int act, int precision);
+/* cthip_matmul for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): same arguments, same kernels, same results, but the partial tiles of
+ * a split reduction go to a 4 MiB array that is part of the library's code object instead of a block of the
+ * caching allocator, and no allocation or release happens during the call.  A shape whose split needs more
+ * (split count x M x N x 4 bytes) returns CTHIP_E_UNSUPPORTED.  All calls on one GPU share that array: calls
+ * that overlap on one GPU (two host threads, two streams) race.  It has no counterpart in the reference. */
+int cthip_matmul_noalloc(float *C, const float *A, const float *B, int M, int N, int K, int act, int precision);
 
 /* Row ops over the last axis, fp32, rows x n contiguous. */
 int cthip_softmax(float *y, const float *x, int64_t rows, int n);   /* nn/activations.lisp:59-62,107-119 */

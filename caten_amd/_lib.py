@@ -59,6 +59,15 @@ PROTOTYPES = {
     "cthip_module_unload": (_i, [_vp]),
     "cthip_get_function": (_i, [_vpp, _vp, C.c_char_p]),
     "cthip_launch": (_i, [_vp, C.POINTER(C.c_uint), C.POINTER(C.c_uint), C.c_uint, _vpp, _i]),
+    "cthip_render_header": (C.c_char_p, []),
+    "cthip_program_create": (_i, [_vpp, C.c_char_p]),
+    "cthip_program_destroy": (_i, [_vp]),
+    "cthip_program_source": (C.c_char_p, [_vp]),
+    "cthip_program_name": (C.c_char_p, [_vp]),
+    "cthip_program_route": (C.c_char_p, [_vp]),
+    "cthip_program_last_route": (C.c_char_p, [_vp]),
+    "cthip_program_bind": (_i, [_vp, _vp]),
+    "cthip_program_launch": (_i, [_vp, C.POINTER(C.c_void_p), _i]),
     "cthip_timer_start": (_i, []),
     "cthip_timer_stop": (_i, [C.POINTER(_f)]),
     "cthip_dequant": (_i, [_i, _vp, _i64, _vp]),
@@ -110,6 +119,8 @@ PROTOTYPES = {
     "cthip_bpe_encode": (_i, [_vp, C.c_char_p, _sz, C.POINTER(_i), _sz, C.POINTER(_sz)]),
     "cthip_bpe_decode": (_i, [_vp, C.POINTER(_i), _sz, C.c_char_p, _sz, C.POINTER(_sz)]),
 }
+
+E_NOT_INIT, E_BAD_ARG, E_UNSUPPORTED, E_COMPILE, E_STATE = -1, -2, -3, -4, -5  # include/caten_hip.h
 
 _lib = None
 _inited = False

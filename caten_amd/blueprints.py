@@ -52,3 +52,79 @@ def softmax_rows(name: str = "fused_softmax", rows: int | None = None, n: int | 
         dict(end),
         {"type": "ENDFOR", "idx": "_gid0"},
     ]}
+
+
+def matmul(name: str = "fused_matmul", relu: bool = False, bias: bool = False, transposed_b: bool = False) -> dict:
+    """(caten (!matmul a b)) with symbolic m n k as the reference lowers it (test-scheduler.lisp:126-135):
+    out[n*i+j] = epilogue(sum_k a[kk*i+k] * b[..]); `transposed_b`: b is (n, kk) read through a transposed view,
+    i.e. Linear's x @ W^T (nn/linear.lisp:3-17); `bias`: + bias[j]; `relu`: max(., 0) (test-scheduler.lisp:140-163).
+    Arguments: val_out, m, n, kk, val_a, val_b [, val_bias]."""
+    b_idx = _add(_mul("kk", "_gid1"), "_gid2") if transposed_b else _add("_gid1", _mul("n", "_gid2"))
+    e = "acc"
+    if bias:
+        e = _add("acc", _A("val_bias", "_gid1"))
+    if relu:
+        e = {"op": "MAX", "args": [e, 0.0]}
+    return {"name": name, "blueprint": [
+        _glob("val_out", "output", 2), _glob("m", "shape", 0, "int64"), _glob("n", "shape", 0, "int64"),
+        _glob("kk", "shape", 0, "int64"), _glob("val_a", "input", 2), _glob("val_b", "input", 2),
+        *([_glob("val_bias", "input", 1)] if bias else []),
+        {"type": "FOR", "idx": "_gid0", "upfrom": 0, "below": _lt("_gid0", "m"), "by": 1},
+        {"type": "FOR", "idx": "_gid1", "upfrom": 0, "below": _lt("_gid1", "n"), "by": 1},
+        {"type": "EXPR", "writes": [_A("acc", None)], "expr": 0.0, "declare_type": True, "dtype": "float32"},
+        {"type": "FOR", "idx": "_gid2", "upfrom": 0, "below": _lt("_gid2", "kk"), "by": 1},
+        {"type": "EXPR", "writes": [_A("acc", None)], "dtype": "float32", "reduction": True,
+         "expr": _add("acc", _mul(_A("val_a", _add(_mul("kk", "_gid0"), "_gid2")), _A("val_b", b_idx)))},
+        {"type": "ENDFOR", "idx": "_gid2"},
+        {"type": "EXPR", "writes": [_A("val_out", _add(_mul("n", "_gid0"), "_gid1"))], "dtype": "float32", "expr": e},
+        {"type": "ENDFOR", "idx": "_gid1"},
+        {"type": "ENDFOR", "idx": "_gid0"},
+    ]}
+
+
+def embedding_onehot(name: str = "fused_embedding") -> dict:
+    """Embedding as the reference computes it (nn/embedding.lisp:13-25): out[t, d] = sum_v where(v == idx[t], W[v, d], 0),
+    the vocabulary index compared as a float (index-components cast to the table's dtype), `==` spelled not(!=).
+    Arguments: val_out, t, d, v, val_idx, val_w."""
+    eq = {"op": "NOT", "args": [{"op": "!=", "args": [{"op": "CAST", "dtype": "float32", "args": ["_gid2"]}, _A("val_idx", "_gid0")]}]}
+    return {"name": name, "blueprint": [
+        _glob("val_out", "output", 2), _glob("t", "shape", 0, "int64"), _glob("d", "shape", 0, "int64"),
+        _glob("v", "shape", 0, "int64"), _glob("val_idx", "input", 1), _glob("val_w", "input", 2),
+        {"type": "FOR", "idx": "_gid0", "upfrom": 0, "below": _lt("_gid0", "t"), "by": 1},
+        {"type": "FOR", "idx": "_gid1", "upfrom": 0, "below": _lt("_gid1", "d"), "by": 1},
+        {"type": "EXPR", "writes": [_A("acc", None)], "expr": 0.0, "declare_type": True, "dtype": "float32"},
+        {"type": "FOR", "idx": "_gid2", "upfrom": 0, "below": _lt("_gid2", "v"), "by": 1},
+        {"type": "EXPR", "writes": [_A("acc", None)], "dtype": "float32", "reduction": True,
+         "expr": _add("acc", {"op": "WHERE", "args": [eq, _A("val_w", _add(_mul("d", "_gid2"), "_gid1")), 0.0]})},
+        {"type": "ENDFOR", "idx": "_gid2"},
+        {"type": "EXPR", "writes": [_A("val_out", _add(_mul("d", "_gid0"), "_gid1"))], "dtype": "float32", "expr": "acc"},
+        {"type": "ENDFOR", "idx": "_gid1"},
+        {"type": "ENDFOR", "idx": "_gid0"},
+    ]}
+
+
+def argmax_rows(name: str = "fused_argmax") -> dict:
+    """ArgMaxNode over the last axis (api/high-level-ops.lisp:314-325): m = max(x); g = max(where(x == m, (n-1) - i, 0));
+    out = cast_int64(n - g - 1) -- the lowest index among ties.  Arguments: val_out (int64), rows, n, val_x."""
+    x = _A("val_x", _add(_mul("n", "_gid0"), "_gid1"))
+    eq = {"op": "NOT", "args": [{"op": "!=", "args": [x, "m"]}]}
+    rev = {"op": "CAST", "dtype": "float32", "args": [_add(_add("n", {"op": "NEG", "args": [1]}), _mul("_gid1", -1))]}
+    loop = {"type": "FOR", "idx": "_gid1", "upfrom": 0, "below": _lt("_gid1", "n"), "by": 1}
+    end = {"type": "ENDFOR", "idx": "_gid1"}
+    return {"name": name, "blueprint": [
+        _glob("val_out", "output", 1, "int64"), _glob("rows", "shape", 0, "int64"), _glob("n", "shape", 0, "int64"),
+        _glob("val_x", "input", 2),
+        {"type": "FOR", "idx": "_gid0", "upfrom": 0, "below": _lt("_gid0", "rows"), "by": 1},
+        {"type": "EXPR", "writes": [_A("m", None)], "expr": float("-inf"), "declare_type": True, "dtype": "float32"},
+        dict(loop),
+        {"type": "EXPR", "writes": [_A("m", None)], "expr": {"op": "MAX", "args": ["m", x]}, "dtype": "float32", "reduction": True},
+        dict(end),
+        {"type": "EXPR", "writes": [_A("g", None)], "expr": 0.0, "declare_type": True, "dtype": "float32"},
+        dict(loop),
+        {"type": "EXPR", "writes": [_A("g", None)], "dtype": "float32", "reduction": True,
+         "expr": {"op": "MAX", "args": ["g", {"op": "WHERE", "args": [eq, rev, 0.0]}]}},
+        dict(end),
+        {"type": "EXPR", "writes": [_A("val_out", "_gid0")], "dtype": "int64",
+         "expr": {"op": "CAST", "dtype": "int64", "args": [_add(_add("n", {"op": "NEG", "args": ["g"]}), {"op": "NEG", "args": [1]})]}},
+        {"type": "ENDFOR", "idx": "_gid0"},
+    ]}

@@ -10,7 +10,6 @@ from __future__ import annotations
 
 import copy
 import ctypes as C
-from dataclasses import dataclass, field
 from typing import Any, List, Optional
 
 import numpy as np
@@ -29,18 +28,51 @@ def dtype_size(dtype: str) -> int:
     return np.dtype(DTYPES[dtype]).itemsize
 
 
-@dataclass
 class AbstractBuffer:
-    shape: List[int] = field(default_factory=list)
-    stride: List[int] = field(default_factory=list)
-    dtype: str = "float32"
-    views: List[Optional[tuple]] = field(default_factory=list)  # (from, to, by, broadcast-p) or None
-    nrank: int = 0
-    value: Any = None  # device pointer (int) for rank > 0, a host number for rank 0
+    """Slots of source/runtime/buffer.lisp:46-53.  `value` is the device pointer (int) for rank > 0, a host number
+    for rank 0.
+
+    copy-buffer (buffer.lisp:60-68) shares the storage between the copy and the original, and the reference leaves
+    the rest to the garbage collector.  Device storage has to be released exactly once, so here a copy does not own
+    it: it keeps a reference to the buffer that opened the storage (`base`) and reads the pointer through it.  A view
+    of a pool that has been closed therefore holds no pointer at all instead of one the allocator may have handed to
+    a new owner, and only the opening buffer ever frees."""
+
+    def __init__(self, shape=None, stride=None, dtype="float32", views=None, nrank=0, value=None):
+        self.shape: List[int] = list(shape) if shape is not None else []
+        self.stride: List[int] = list(stride) if stride is not None else []
+        self.dtype = dtype
+        self.views: List[Optional[tuple]] = list(views) if views is not None else []  # (from, to, by, broadcast-p) or None
+        self.nrank = nrank
+        self.base: Optional["AbstractBuffer"] = None  # the buffer whose storage this one shares (views, copies)
+        self._value = value
+
+    @property
+    def value(self):
+        return self.base.value if self.base is not None else self._value
+
+    @value.setter
+    def value(self, v):
+        # storage of its own from here on (open-buffer on a copy, a scalar cast to a tensor)
+        self.base = None
+        self._value = v
+
+    @property
+    def owns_storage(self) -> bool:
+        return self.base is None
 
     def copy(self) -> "AbstractBuffer":
-        """copy-buffer (buffer.lisp:60-68): a shallow copy sharing the storage."""
-        return copy.copy(self)
+        """copy-buffer (buffer.lisp:60-68): a shallow copy sharing the storage; the copy does not own it."""
+        c = copy.copy(self)
+        c.shape, c.stride, c.views = list(self.shape), list(self.stride), list(self.views)
+        if self.nrank > 0 or self.base is not None:
+            c.base = self.base if self.base is not None else self
+            c._value = None
+        return c
+
+    def __repr__(self):
+        return (f"<{type(self).__name__} :shape {self.shape} :stride {self.stride} :dtype {self.dtype} "
+                f":views {self.views} :nrank {self.nrank} :value {self.value}>")
 
 
 class HipBuffer(AbstractBuffer):
@@ -84,7 +116,11 @@ def open_buffer(runtime, buffer: HipBuffer) -> HipBuffer:
 
 def close_buffer(runtime, buffer: HipBuffer) -> None:
     """close-buffer: idempotent (metal.lisp:123-126)."""
-    if buffer.nrank > 0 and isinstance(buffer.value, int) and buffer.value:
+    if buffer.nrank > 0 and not buffer.owns_storage:
+        buffer.base = None  # a view or copy: the storage belongs to the buffer that opened it
+        buffer._value = None
+        return
+    if buffer.nrank > 0 and isinstance(buffer.value, int) and not isinstance(buffer.value, bool) and buffer.value:
         _lib.check(_lib.load().cthip_free(buffer.value))
     if buffer.nrank > 0:
         buffer.value = None

@@ -25,6 +25,7 @@ struct State {
   int decoder_graph = 1;  // option "decoder_graph": 0 = the step's launches are issued one by one (kernel tracing)
   int prefill_gemm = 1;   // option "prefill_gemm": 0 = prompts are fed row by row through the decode step
   int decode_fused = 1;   // option "decode_fused": 0 = five launches per layer instead of three
+  int render_routes = 1;  // option "render_routes": 0 = every program runs its rendered kernel, none a hand-written one
 };
 State &state();
 // cthip_alloc without the zero fill, for temporaries that are fully written before they are read

@@ -229,6 +229,35 @@ __global__ __launch_bounds__(256) void k_gemv_generic(GemvArgs a) {
   if (a.am_val) gemv_argmax_tail(a, wave, lane, best_v, best_i);
 }
 
+// fp32 / fp16 rows whose width is no multiple of a 16-byte chunk: rows start at any element, so the lanes of a
+// wavefront stride the row element by element.  `x` must already carry the prologue.
+template <int TYPE>
+__global__ __launch_bounds__(256) void k_gemv_elements(GemvArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int wave = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int total_waves = gridDim.x * (blockDim.x >> 6);
+  const int m = blockIdx.y;
+  const float *__restrict__ x = a.x + (int64_t)m * a.x_stride;
+  const int posv = a.pos ? a.pos[0] : 0;
+  float best_v = -INFINITY;
+  int best_i = 0x7fffffff;
+  for (int row = wave; row < a.rows; row += total_waves) {
+    float acc = 0.0f;
+    for (int c = lane; c < a.cols; c += 64) {
+      const int64_t e = (int64_t)row * a.cols + c;
+      const float w = TYPE == CTHIP_F16 ? half_bits_to_float(((const unsigned short *)a.q)[e]) : ((const float *)a.q)[e];
+      acc = fmaf(w, x[c], acc);
+    }
+    acc = wave_sum(acc);
+    if (lane == 0) {
+      const float v = gemv_store(a, m, row, acc, posv, a.bias ? a.bias[row] : 0.0f,
+                                 a.residual ? a.residual[(int64_t)m * a.y_stride + row] : 0.0f);
+      argmax_merge(best_v, best_i, v, row);
+    }
+  }
+  if (a.am_val) gemv_argmax_tail(a, wave, lane, best_v, best_i);
+}
+
 // prologue as a kernel of its own, for the generic fallback: one block per input vector
 __global__ __launch_bounds__(256) void k_prologue(float *__restrict__ out, const float *__restrict__ x, int cols,
                                                   int pro, const float *__restrict__ g,
@@ -453,11 +482,20 @@ int launch_gemv(const WMat *w, GemvArgs a, int m) {
   int cap = s.compute_units * 8;
   if (cap * 4 > kGemvMaxWaves) cap = kGemvMaxWaves / 4;
   dim3 grid(blocks < cap ? blocks : cap, m), block(256);
+  // rows that are whole 16-byte chunks are read chunk by chunk; any other width (fp32 / fp16 only: quantised rows
+  // are multiples of 32) element by element
+  const bool chunks = a.cols % xpc_of(w->type) == 0;
   switch (w->type) {
     case CTHIP_Q8_0: hipLaunchKernelGGL(k_gemv_generic<CTHIP_Q8_0>, grid, block, 0, s.stream, a); break;
     case CTHIP_Q4_0: hipLaunchKernelGGL(k_gemv_generic<CTHIP_Q4_0>, grid, block, 0, s.stream, a); break;
-    case CTHIP_F16: hipLaunchKernelGGL(k_gemv_generic<CTHIP_F16>, grid, block, 0, s.stream, a); break;
-    default: hipLaunchKernelGGL(k_gemv_generic<CTHIP_F32>, grid, block, 0, s.stream, a); break;
+    case CTHIP_F16:
+      if (chunks) hipLaunchKernelGGL(k_gemv_generic<CTHIP_F16>, grid, block, 0, s.stream, a);
+      else hipLaunchKernelGGL(k_gemv_elements<CTHIP_F16>, grid, block, 0, s.stream, a);
+      break;
+    default:
+      if (chunks) hipLaunchKernelGGL(k_gemv_generic<CTHIP_F32>, grid, block, 0, s.stream, a);
+      else hipLaunchKernelGGL(k_gemv_elements<CTHIP_F32>, grid, block, 0, s.stream, a);
+      break;
   }
   CTHIP_LAUNCH_CHECK();
   if (a.am_val) {
@@ -667,10 +705,12 @@ int cthip_set_option(const char *name, int value) {
     state().gemv_stream = value;
     return 0;
   }
-  if (!strcmp(name, "decoder_graph") || !strcmp(name, "prefill_gemm") || !strcmp(name, "decode_fused")) {
+  if (!strcmp(name, "decoder_graph") || !strcmp(name, "prefill_gemm") || !strcmp(name, "decode_fused") ||
+      !strcmp(name, "render_routes")) {
     if (value != 0 && value != 1) return fail(CTHIP_E_BAD_ARG, "cthip_set_option: %s is 0 or 1", name);
     if (!strcmp(name, "decoder_graph")) state().decoder_graph = value;
     else if (!strcmp(name, "prefill_gemm")) state().prefill_gemm = value;
+    else if (!strcmp(name, "render_routes")) state().render_routes = value;
     else state().decode_fused = value;
     return 0;
   }

@@ -907,6 +907,42 @@ int launch_linear_gemm(float *y, const WMat *w, const float *x, int m, const flo
   return launch_gemm(a, B_WMAT, precision, nullptr, 0);
 }
 
+// A matmul-shaped Schedule-Item routed here by the renderer: C (M,N) = act(A (M,K) . B + bias), B either (K,N)
+// row-major or (N,K) rows read through a transposed view (Linear, source/nn/linear.lisp:3-17); fp32-grade operands.
+int matmul_routed(float *C, const float *A, const float *B, int M, int N, int K, int act, const float *bias, bool b_is_nk) {
+  if (b_is_nk && M < 8) {  // a few rows of a Linear: the single-row kernels stream the weights once per row
+    WMat w = {};
+    w.type = CTHIP_F32;
+    w.rows = N;
+    w.cols = K;
+    w.q = const_cast<float *>(B);
+    w.q_bytes = (int64_t)N * K * 4;
+    GemvArgs g = {};
+    g.y = C;
+    g.x = A;
+    g.bias = bias;
+    g.act = act;
+    g.x_stride = K;
+    g.y_stride = N;
+    return launch_gemv(&w, g, M);
+  }
+  GemmArgs a = {};
+  a.C = C;
+  a.A = A;
+  a.bias = bias;
+  a.M = M;
+  a.N = N;
+  a.K = K;
+  a.act = act;
+  if (b_is_nk) {
+    a.wq = B;
+    a.wtype = CTHIP_F32;
+    return launch_gemm(a, B_WMAT, GEMM_BF16X6, nullptr, 0);
+  }
+  a.B = B;
+  return launch_gemm(a, B_ROWMAJOR, GEMM_BF16X6, nullptr, 0);
+}
+
 }  // namespace cthip
 
 using namespace cthip;

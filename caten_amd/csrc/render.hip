@@ -1,0 +1,1095 @@
+// Hip-Renderer behind the C ABI: a Schedule-Item's blueprint, printed as an s-expression, becomes a PROGRAM --
+// HIP source with gfx950-aware work distribution for the item, plus, where the item is one of the shapes a
+// hand-written kernel covers, a route to that kernel.  Caten's renderer protocol (`%render-kernel` /
+// `%compile-kernel`, source/codegen/renderer.lisp:30-34) is implemented by Lisp classes; the Lisp side of this
+// backend (and the Python mirror the tests drive) only prints the blueprint and calls the entry points below, so
+// both get the same kernels.
+//
+// Interchange text (case-insensitive; what a Lisp `format` of the Render-IR nodes of renderer.lisp:36-92 and
+// aasm/attrs.lisp:298-318 gives):
+//   (item NAME node...)
+//   node := (define-global ID DTYPE POINTER-P input|output|shape NRANK)
+//         | (for IDX UPFROM BELOW BY [local|global]) | (endfor IDX) | (if COND) | (endif)
+//         | (expr (WRITE...) RHS :dtype DTYPE [:declare t] [:reduction t])
+//   WRITE, expr := number | inf | -inf | nan | t | nil | SYMBOL | (aref ID [INDEX]) | (const VALUE DTYPE)
+//         | (cast DTYPE expr) | (space block|thread RANK) | (OP expr...)     OP = the aasm instruction set
+// BELOW is the loop condition, e.g. (< _gid0 n) (source/byoc/clang.lisp:58-73); an aref's INDEX is the flat element
+// index sum_d stride_d * (from_d + by_d * gid_d) the reference renders (clang.lisp:82-97).
+//
+// Work distribution of rendered kernels (the reference leaves every loop serial at OPTIMIZE=1, so its Metal
+// kernels run in one thread, source/byoc/metal.lisp:341-345): the outermost perfectly nested loops whose index
+// appears in every global write below them are data-parallel and become one flat thread id, innermost fastest, in
+// 256-thread workgroups; row reductions (a parallel prefix whose body is scalar statements and loops over one
+// more axis, some of them reductions into scalars that start at the operation's identity) get one WAVEFRONT per
+// row: the 64 lanes stride the axis together, partials meet in a __shfl_xor butterfly, lane 0 stores per-row
+// scalars; a row of static length becomes counted, unrolled loops so that the row is read once.
+//
+// Routes (checked again at every launch against the actual shapes; anything that does not fit runs the rendered
+// kernel): the matmul nest ADD(reduction) o MUL of source/test-suite/test-scheduler.lisp:126-135 with an
+// optional bias / ReLU epilogue -> the MFMA GEMM (B row-major, or read through a transposed view as Linear does,
+// source/nn/linear.lisp:3-17; fewer than eight rows of a Linear -> the single-row kernels); the one-hot masked sum
+// of Embedding (source/nn/embedding.lisp:13-25) -> a row gather; ArgMaxNode's two reductions
+// (source/api/high-level-ops.lisp:314-325) -> the argmax kernel; softmax rows (source/nn/activations.lisp:107-119)
+// -> the row kernel.
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <map>
+#include <string>
+#include <vector>
+
+#include "common.h"
+
+namespace cthip {
+
+// ------------------------------------------------------------------ s-expressions
+struct Sx {
+  enum Kind { LIST, SYM, INT, FLT, STR } kind = LIST;
+  std::string s;       // SYM (lower case) / STR
+  long long i = 0;     // INT
+  double f = 0.0;      // FLT
+  std::vector<Sx> v;   // LIST
+  bool is_sym(const char *name) const { return kind == SYM && s == name; }
+  bool is_list() const { return kind == LIST; }
+  bool is_num() const { return kind == INT || kind == FLT; }
+  const Sx &head() const { return v[0]; }
+  bool call(const char *op) const { return kind == LIST && !v.empty() && v[0].is_sym(op); }
+  size_t n() const { return v.size(); }
+};
+static Sx sx_sym(const std::string &s) { Sx x; x.kind = Sx::SYM; x.s = s; return x; }
+static Sx sx_int(long long i) { Sx x; x.kind = Sx::INT; x.i = i; return x; }
+static Sx sx_list(std::vector<Sx> v) { Sx x; x.kind = Sx::LIST; x.v = std::move(v); return x; }
+
+struct Parser {
+  const char *p;
+  std::string err;
+  void skip() {
+    for (;;) {
+      while (*p == ' ' || *p == '\n' || *p == '\t' || *p == '\r') p++;
+      if (*p == ';') while (*p && *p != '\n') p++;
+      else break;
+    }
+  }
+  bool parse(Sx &out) {
+    skip();
+    if (!*p) return err = "unexpected end of text", false;
+    if (*p == '(') {
+      p++;
+      out = Sx();
+      for (;;) {
+        skip();
+        if (!*p) return err = "unbalanced '('", false;
+        if (*p == ')') { p++; return true; }
+        Sx e;
+        if (!parse(e)) return false;
+        out.v.push_back(std::move(e));
+      }
+    }
+    if (*p == ')') return err = "unexpected ')'", false;
+    if (*p == '"') {
+      p++;
+      out = Sx();
+      out.kind = Sx::STR;
+      while (*p && *p != '"') {
+        if (*p == '\\' && p[1]) p++;
+        out.s.push_back(*p++);
+      }
+      if (*p != '"') return err = "unterminated string", false;
+      p++;
+      return true;
+    }
+    std::string tok;
+    while (*p && *p != ' ' && *p != '\n' && *p != '\t' && *p != '\r' && *p != '(' && *p != ')') tok.push_back(*p++);
+    if (!tok.empty() && tok[0] == ':') tok = tok.substr(1);  // keywords and symbols are the same thing here
+    std::string low;
+    for (char c : tok) low.push_back((char)tolower((unsigned char)c));
+    // numbers: integers, floats (Lisp prints 1.0d0 / 1.0f0 / 1.0e-5 exponent markers)
+    std::string num = low;
+    for (char &c : num) if (c == 'd' || c == 'f') c = 'e';
+    char *end = nullptr;
+    out = Sx();
+    if (low == "inf" || low == "+inf") { out.kind = Sx::FLT; out.f = INFINITY; return true; }
+    if (low == "-inf") { out.kind = Sx::FLT; out.f = -INFINITY; return true; }
+    if (low == "nan") { out.kind = Sx::FLT; out.f = NAN; return true; }
+    const bool numeric_start = !num.empty() && (isdigit((unsigned char)num[0]) || ((num[0] == '-' || num[0] == '+' || num[0] == '.') && num.size() > 1 && (isdigit((unsigned char)num[1]) || num[1] == '.')));
+    if (numeric_start) {
+      long long iv = strtoll(num.c_str(), &end, 10);
+      if (end && !*end) { out.kind = Sx::INT; out.i = iv; return true; }
+      double fv = strtod(num.c_str(), &end);
+      if (end && !*end) { out.kind = Sx::FLT; out.f = fv; return true; }
+    }
+    out.kind = Sx::SYM;
+    out.s = low;
+    return true;
+  }
+};
+
+// ------------------------------------------------------------------ blueprint
+struct Global {
+  std::string id, dtype, type;  // type: input / output / shape
+  bool pointer = false;
+  int nrank = 0;
+};
+struct BpNode {
+  enum T { FOR, ENDFOR, IF, ENDIF, EXPR } t = EXPR;
+  std::string idx;              // FOR / ENDFOR
+  Sx upfrom, below, by;         // FOR
+  bool global_scope = false;    // FOR
+  Sx cond;                      // IF
+  std::vector<Sx> writes;       // EXPR
+  Sx rhs;
+  bool declare = false, reduction = false;
+  std::string dtype = "float32";
+};
+struct Item {
+  std::string name;
+  std::vector<Global> globals;
+  std::vector<BpNode> body;
+};
+
+static const std::map<std::string, std::string> &cdtypes() {  // ->cdtype (source/codegen/helpers.lisp:101-113)
+  static const std::map<std::string, std::string> m = {
+      {"bool", "bool"}, {"float64", "double"}, {"float32", "float"}, {"float16", "_Float16"},
+      {"uint64", "unsigned long long"}, {"int64", "long long"}, {"uint32", "unsigned int"}, {"int32", "int"},
+      {"uint16", "unsigned short"}, {"int16", "short"}, {"uint8", "unsigned char"}, {"int8", "signed char"}};
+  return m;
+}
+static size_t dtype_bytes(const std::string &d) {
+  if (d == "float64" || d == "uint64" || d == "int64") return 8;
+  if (d == "float32" || d == "uint32" || d == "int32") return 4;
+  if (d == "float16" || d == "uint16" || d == "int16") return 2;
+  return 1;
+}
+
+static bool truthy(const Sx &x) { return !(x.is_sym("nil") || (x.kind == Sx::LIST && x.v.empty())); }
+
+static bool build_item(const Sx &top, Item &it, std::string &err) {
+  if (!top.call("item") || top.n() < 2) return err = "expected (item NAME node...)", false;
+  it.name = top.v[1].s;
+  for (char &c : it.name) c = (char)tolower((unsigned char)c);
+  if (it.name.empty()) return err = "the item has no name", false;
+  int depth = 0, ifs = 0;
+  for (size_t k = 2; k < top.n(); k++) {
+    const Sx &n = top.v[k];
+    if (!n.is_list() || n.v.empty() || n.v[0].kind != Sx::SYM) return err = "a blueprint node must be a list headed by its type", false;
+    const std::string &ty = n.v[0].s;
+    if (ty == "define-global") {
+      if (n.n() != 6) return err = "(define-global ID DTYPE POINTER-P TYPE NRANK)", false;
+      Global g;
+      g.id = n.v[1].s;
+      g.dtype = n.v[2].s;
+      g.pointer = truthy(n.v[3]);
+      g.type = n.v[4].s;
+      g.nrank = (int)n.v[5].i;
+      if (!cdtypes().count(g.dtype)) return err = "define-global: unknown dtype " + g.dtype, false;
+      if (g.type != "input" && g.type != "output" && g.type != "shape") return err = "define-global: type is input, output or shape", false;
+      it.globals.push_back(g);
+    } else if (ty == "for") {
+      if (n.n() < 5) return err = "(for IDX UPFROM BELOW BY [SCOPE])", false;
+      BpNode b;
+      b.t = BpNode::FOR;
+      b.idx = n.v[1].s;
+      b.upfrom = n.v[2];
+      b.below = n.v[3];
+      b.by = n.v[4];
+      b.global_scope = n.n() > 5 && n.v[5].is_sym("global");
+      it.body.push_back(b);
+      depth++;
+    } else if (ty == "endfor") {
+      BpNode b;
+      b.t = BpNode::ENDFOR;
+      b.idx = n.n() > 1 ? n.v[1].s : "";
+      it.body.push_back(b);
+      if (--depth < 0) return err = "endfor without for", false;
+    } else if (ty == "if") {
+      if (n.n() != 2) return err = "(if COND)", false;
+      BpNode b;
+      b.t = BpNode::IF;
+      b.cond = n.v[1];
+      it.body.push_back(b);
+      ifs++;
+    } else if (ty == "endif") {
+      BpNode b;
+      b.t = BpNode::ENDIF;
+      it.body.push_back(b);
+      if (--ifs < 0) return err = "endif without if", false;
+    } else if (ty == "expr") {
+      if (n.n() < 3 || !n.v[1].is_list()) return err = "(expr (WRITE...) RHS :dtype DTYPE [:declare t] [:reduction t])", false;
+      BpNode b;
+      b.t = BpNode::EXPR;
+      b.writes = n.v[1].v;
+      b.rhs = n.v[2];
+      for (size_t q = 3; q + 1 < n.n(); q += 2) {
+        if (n.v[q].is_sym("dtype")) b.dtype = n.v[q + 1].s;
+        else if (n.v[q].is_sym("declare") || n.v[q].is_sym("declare-type")) b.declare = truthy(n.v[q + 1]);
+        else if (n.v[q].is_sym("reduction")) b.reduction = truthy(n.v[q + 1]);
+      }
+      if (b.writes.empty()) return err = "expr: no write", false;
+      if (!cdtypes().count(b.dtype)) return err = "expr: unknown dtype " + b.dtype, false;
+      it.body.push_back(b);
+    } else {
+      return err = "unknown blueprint node :" + ty, false;
+    }
+  }
+  if (depth || ifs) return err = "unbalanced for / if", false;
+  return true;
+}
+
+// ------------------------------------------------------------------ expressions -> HIP
+struct Rend {
+  std::string err;
+
+  static std::string fmt_float(double v, bool f64) {
+    if (isinf(v)) return v > 0 ? "_infinity" : "_negative_infinity";
+    if (isnan(v)) return "_nan";
+    char buf[64];
+    if (f64) {
+      snprintf(buf, sizeof(buf), "%.17g", v);
+      std::string s = buf;
+      if (s.find('.') == std::string::npos && s.find('e') == std::string::npos) s += ".0";
+      return s;
+    }
+    // the shortest decimal that reads back as the same float, in positional notation (as Caten's ~f prints)
+    const float fv = (float)v;
+    int prec = 0;
+    for (; prec <= 8; prec++) {
+      snprintf(buf, sizeof(buf), "%.*e", prec, (double)fv);
+      if (strtof(buf, nullptr) == fv) break;
+    }
+    std::string m = buf;  // [-]d.ddde[+-]xx
+    const bool negative = m[0] == '-';
+    if (negative) m = m.substr(1);
+    const size_t ep = m.find('e');
+    const int ex = atoi(m.c_str() + ep + 1);
+    std::string digits;
+    for (size_t k = 0; k < ep; k++)
+      if (m[k] != '.') digits.push_back(m[k]);
+    while (digits.size() > 1 && digits.back() == '0') digits.pop_back();
+    std::string s;
+    if (ex >= 0) {
+      while ((int)digits.size() < ex + 1) digits.push_back('0');
+      s = digits.substr(0, (size_t)ex + 1) + "." + ((int)digits.size() > ex + 1 ? digits.substr((size_t)ex + 1) : "0");
+    } else {
+      s = "0." + std::string((size_t)(-ex - 1), '0') + digits;
+    }
+    return (negative ? "-" : "") + s + "f";
+  }
+
+  // %render-const (renderer.lisp:319-329)
+  std::string constant(const Sx &v, const std::string &dtype) {
+    if (v.is_sym("t")) return "true";
+    if (v.is_sym("nil")) return "false";
+    const bool fl = dtype.rfind("float", 0) == 0;
+    if (v.kind == Sx::FLT || (fl && v.kind == Sx::INT)) return fmt_float(v.kind == Sx::FLT ? v.f : (double)v.i, dtype == "float64");
+    if (v.kind == Sx::INT) return std::to_string(v.i);
+    if (v.kind == Sx::SYM) return v.s;
+    err = "cannot render a constant";
+    return "0";
+  }
+
+  std::string aref(const Sx &e) {
+    if (e.n() < 2) { err = "(aref ID [INDEX])"; return "0"; }
+    const std::string &name = e.v[1].s;
+    if (e.n() == 2 || e.v[2].is_sym("nil")) return name;
+    return name + "[" + expr(e.v[2], "int64") + "]";
+  }
+
+  // render-expr / %render-node dispatch (renderer.lisp:331-411)
+  std::string expr(const Sx &e, const std::string &fd) {
+    if (e.kind == Sx::INT) return std::to_string(e.i);
+    if (e.kind == Sx::FLT) return fmt_float(e.f, fd == "float64");
+    if (e.kind == Sx::SYM) return e.is_sym("t") ? "true" : e.is_sym("nil") ? "false" : e.s;
+    if (e.kind == Sx::STR) return e.s;
+    if (e.v.empty() || e.v[0].kind != Sx::SYM) { err = "an expression must be headed by its operation"; return "0"; }
+    const std::string &op = e.v[0].s;
+    const bool f64 = fd == "float64";
+    auto r = [&](size_t k) { return expr(e.v[k], fd); };
+    const size_t na = e.n() - 1;
+    auto need = [&](size_t k) {
+      if (na < k) { err = "too few arguments for :" + op; return false; }
+      return true;
+    };
+    if (op == "const") return need(1) ? constant(e.v[1], na >= 2 ? e.v[2].s : fd) : "0";
+    if (op == "aref") return aref(e);
+    if (op == "space") {  // metal.lisp:173-176 -> blockIdx / threadIdx
+      if (!need(2)) return "0";
+      const char *xyz[3] = {"x", "y", "z"};
+      const long long rank = e.v[2].i;
+      if (rank < 0 || rank > 2) { err = "space: rank is 0, 1 or 2"; return "0"; }
+      return std::string(e.v[1].is_sym("block") ? "blockIdx." : "threadIdx.") + xyz[rank];
+    }
+    static const std::map<std::string, std::string> infix = {{"add", "+"}, {"mul", "*"}, {"mod", "%"}, {"idiv", "/"}, {"and", " & "}, {"or", " | "}, {"xor", " ^ "}};
+    auto inf = infix.find(op);
+    if (inf != infix.end()) {
+      if (!need(1)) return "0";
+      std::string s = "(";
+      for (size_t k = 1; k <= na; k++) s += (k > 1 ? inf->second : "") + r(k);
+      return s + ")";
+    }
+    if (op == "wmma") return need(3) ? "(" + r(1) + "+" + r(2) + "*" + r(3) + ")" : "0";
+    if (op == "max") return need(2) ? "ct_max(" + r(1) + ", " + r(2) + ")" : "0";
+    if (op == "neg") return need(1) ? "(-" + r(1) + ")" : "0";
+    if (op == "not") return need(1) ? "(!" + r(1) + ")" : "0";
+    if (op == "sin" || op == "log2" || op == "exp2" || op == "sqrt") return need(1) ? op + (f64 ? "" : "f") + "(" + r(1) + ")" : "0";
+    if (op == "recip") {
+      if (!need(1)) return "0";
+      if (fd.rfind("float", 0) == 0) return std::string(f64 ? "(1.0" : "(1.0f") + "/(" + r(1) + "))";
+      return "(1/(" + r(1) + "))";
+    }
+    if (op == "!=" || op == "<") return need(2) ? "(" + r(na - 1) + op + r(na) + ")" : "0";
+    if (op == "move" || op == "store") return need(1) ? r(na) : "0";
+    if (op == "cast") {
+      if (!need(2)) return "0";
+      auto ct = cdtypes().find(e.v[1].s);
+      if (ct == cdtypes().end()) { err = "cast: unknown dtype " + e.v[1].s; return "0"; }
+      return "((" + ct->second + ")" + r(na) + ")";
+    }
+    if (op == "where") return need(3) ? "(" + r(1) + " ? " + r(2) + " : " + r(3) + ")" : "0";
+    err = "Hip-Renderer: no %render-node method for :" + op;
+    return "0";
+  }
+};
+
+static bool uses(const Sx &e, const std::string &sym) {
+  if (e.kind == Sx::SYM) return e.s == sym;
+  if (e.kind != Sx::LIST) return false;
+  for (size_t k = (e.call("aref") || e.call("cast") || e.call("const")) ? 1 : 0; k < e.n(); k++)
+    if (uses(e.v[k], sym)) return true;
+  return false;
+}
+static bool is_scalar_ref(const Sx &w) { return w.kind == Sx::SYM || (w.call("aref") && (w.n() == 2 || w.v[2].is_sym("nil"))); }
+static std::string ref_name(const Sx &w) { return w.kind == Sx::SYM ? w.s : (w.call("aref") && w.n() >= 2 ? w.v[1].s : std::string()); }
+static bool const_value(const Sx &e, double &out) {
+  if (e.kind == Sx::INT) { out = (double)e.i; return true; }
+  if (e.kind == Sx::FLT) { out = e.f; return true; }
+  if (e.call("const") && e.n() >= 2) return const_value(e.v[1], out);
+  if (e.call("neg") && e.n() == 2 && const_value(e.v[1], out)) { out = -out; return true; }
+  return false;
+}
+static bool is_zero(const Sx &e) {
+  double v;
+  return const_value(e, v) && v == 0.0;
+}
+static bool is_one(const Sx &e) {
+  double v;
+  return const_value(e, v) && v == 1.0;
+}
+// `below` is the condition (idx < N); returns N when it has that shape and by == 1
+static const Sx *upper_bound(const BpNode &f) {
+  if (!is_one(f.by)) return nullptr;
+  if (f.below.call("<") && f.below.n() >= 3) {
+    const Sx &x = f.below.v[f.below.n() - 2], &y = f.below.v[f.below.n() - 1];
+    if (x.kind == Sx::SYM && x.s == f.idx) return &y;
+  }
+  return nullptr;
+}
+static int match_end(const std::vector<BpNode> &b, int i) {  // index of the ENDFOR that closes the FOR at i
+  int lvl = 0;
+  for (int j = i; j < (int)b.size(); j++) {
+    if (b[j].t == BpNode::FOR) lvl++;
+    else if (b[j].t == BpNode::ENDFOR && --lvl == 0) return j;
+  }
+  return -1;
+}
+
+// integer expressions over the by-value arguments (grid sizes, route shapes)
+static bool eval_int(const Sx &e, const std::map<std::string, long long> &env, long long &out) {
+  if (e.kind == Sx::INT) { out = e.i; return true; }
+  if (e.kind == Sx::FLT) { out = (long long)e.f; return e.f == (double)out; }
+  if (e.kind == Sx::SYM) {
+    auto it = env.find(e.s);
+    if (it == env.end()) return false;
+    out = it->second;
+    return true;
+  }
+  if (e.kind != Sx::LIST || e.v.empty() || e.v[0].kind != Sx::SYM) return false;
+  const std::string &op = e.v[0].s;
+  if (op == "const") return e.n() >= 2 && eval_int(e.v[1], env, out);
+  if (op == "cast") return e.n() >= 3 && eval_int(e.v[2], env, out);
+  std::vector<long long> a;
+  for (size_t k = 1; k < e.n(); k++) {
+    long long v;
+    if (!eval_int(e.v[k], env, v)) return false;
+    a.push_back(v);
+  }
+  if (a.empty()) return false;
+  if (op == "add") { out = 0; for (long long v : a) out += v; return true; }
+  if (op == "mul") { out = 1; for (long long v : a) out *= v; return true; }
+  if (op == "neg") { out = -a[0]; return true; }
+  if (op == "max" && a.size() == 2) { out = a[0] > a[1] ? a[0] : a[1]; return true; }
+  if (op == "idiv" && a.size() == 2 && a[1]) { out = a[0] / a[1]; return true; }
+  if (op == "mod" && a.size() == 2 && a[1]) { out = a[0] % a[1]; return true; }
+  if (op == "move" || op == "store") { out = a.back(); return true; }
+  return false;
+}
+
+// ------------------------------------------------------------------ routes to hand-written kernels
+// An index expression as an affine function of (up to three) loop indices, found by evaluation: base and one
+// coefficient per index, confirmed on a probe point.  Whatever way the scheduler spelled the index, a matrix
+// laid out row-major gives the same numbers.
+struct Affine {
+  long long base = 0, c[3] = {0, 0, 0};
+};
+static bool affine_of(const Sx &index, const std::string idx[3], int nidx, std::map<std::string, long long> env, Affine &out) {
+  auto at = [&](long long a, long long b, long long c, long long &v) {
+    const long long p[3] = {a, b, c};
+    for (int k = 0; k < nidx; k++) env[idx[k]] = p[k];
+    return eval_int(index, env, v);
+  };
+  long long v0, v;
+  if (!at(0, 0, 0, v0)) return false;
+  out.base = v0;
+  for (int k = 0; k < nidx; k++) {
+    if (!at(k == 0, k == 1, k == 2, v)) return false;
+    out.c[k] = v - v0;
+  }
+  if (!at(2, 3, 5, v)) return false;
+  return v == v0 + 2 * out.c[0] + (nidx > 1 ? 3 * out.c[1] : 0) + (nidx > 2 ? 5 * out.c[2] : 0);
+}
+
+enum RouteKind { R_NONE = 0, R_MATMUL, R_EMBEDDING, R_ARGMAX, R_SOFTMAX };
+struct Route {
+  RouteKind kind = R_NONE;
+  int out = -1, a = -1, b = -1, bias = -1;  // argument positions
+  Sx out_idx, a_idx, b_idx, bias_idx;       // index expressions over the loop indices
+  std::string idx[3];                       // loop indices: (i, j, k) / (t, d, v) / (row, col)
+  Sx bound[3];                              // their upper bounds
+  int act = CTHIP_ACT_NONE;
+};
+
+struct Program {
+  Item item;
+  std::string source, route_name = "rendered", last_route = "none";
+  std::vector<Sx> grid_bounds;
+  int rows_per_block = 256;
+  bool parallel = false;
+  Route route;
+  hipFunction_t fn = nullptr;
+};
+
+static int arg_pos(const Item &it, const std::string &id) {
+  for (size_t k = 0; k < it.globals.size(); k++)
+    if (it.globals[k].id == id) return (int)k;
+  return -1;
+}
+static bool is_ref_to(const Sx &e, const std::string &name) { return is_scalar_ref(e) && ref_name(e) == name; }
+
+// acc = acc + X  /  acc = X + acc  /  (wmma acc a b); returns X (for wmma: (mul a b))
+static bool reduction_term(const BpNode &n, const std::string &acc, const char *op, Sx &term) {
+  if (n.t != BpNode::EXPR || n.writes.size() != 1 || !is_ref_to(n.writes[0], acc)) return false;
+  const Sx &e = n.rhs;
+  if (!strcmp(op, "add") && e.call("wmma") && e.n() == 4 && is_ref_to(e.v[1], acc)) {
+    term = sx_list({sx_sym("mul"), e.v[2], e.v[3]});
+    return true;
+  }
+  if (!e.call(op) || e.n() != 3) return false;
+  if (is_ref_to(e.v[1], acc) && !uses(e.v[2], acc)) { term = e.v[2]; return true; }
+  if (is_ref_to(e.v[2], acc) && !uses(e.v[1], acc)) { term = e.v[1]; return true; }
+  return false;
+}
+static bool is_global_aref(const Item &it, const Sx &e, int &pos) {
+  if (!e.call("aref") || e.n() < 3) return false;
+  pos = arg_pos(it, e.v[1].s);
+  return pos >= 0 && it.globals[pos].pointer && it.globals[pos].dtype == "float32";
+}
+
+// for i < M: for j < N: { acc = 0; for k < K: acc += A[..] * B[..]; out[..] = epilogue(acc) }
+static bool match_matmul(const Item &it, Route &r) {
+  const std::vector<BpNode> &b = it.body;
+  if (b.size() != 9) return false;
+  if (b[0].t != BpNode::FOR || b[1].t != BpNode::FOR || b[2].t != BpNode::EXPR || b[3].t != BpNode::FOR || b[4].t != BpNode::EXPR ||
+      b[5].t != BpNode::ENDFOR || b[6].t != BpNode::EXPR || b[7].t != BpNode::ENDFOR || b[8].t != BpNode::ENDFOR)
+    return false;
+  const int fors[3] = {0, 1, 3};
+  for (int q = 0; q < 3; q++) {
+    const Sx *ub = upper_bound(b[fors[q]]);
+    if (!ub || !is_zero(b[fors[q]].upfrom)) return false;
+    r.idx[q] = b[fors[q]].idx;
+    r.bound[q] = *ub;
+  }
+  if (!b[2].declare || b[2].writes.size() != 1 || !is_scalar_ref(b[2].writes[0]) || !is_zero(b[2].rhs) || b[2].dtype != "float32") return false;
+  const std::string acc = ref_name(b[2].writes[0]);
+  Sx term;
+  if (!reduction_term(b[4], acc, "add", term) || !term.call("mul") || term.n() != 3) return false;
+  if (!is_global_aref(it, term.v[1], r.a) || !is_global_aref(it, term.v[2], r.b)) return false;
+  r.a_idx = term.v[1].v[2];
+  r.b_idx = term.v[2].v[2];
+  // the epilogue: acc, max(acc + bias, 0), acc + bias, max(acc, 0)
+  if (b[6].writes.size() != 1 || !is_global_aref(it, b[6].writes[0], r.out) || it.globals[r.out].type != "output") return false;
+  r.out_idx = b[6].writes[0].v[2];
+  Sx e = b[6].rhs;
+  r.act = CTHIP_ACT_NONE;
+  if (e.call("max") && e.n() == 3 && (is_zero(e.v[2]) || is_zero(e.v[1]))) {
+    const Sx inner = is_zero(e.v[2]) ? e.v[1] : e.v[2];  // (a copy: e's own element cannot be assigned to e)
+    e = inner;
+    r.act = CTHIP_ACT_RELU;
+  }
+  if (e.call("add") && e.n() == 3) {
+    const int ai = is_ref_to(e.v[1], acc) ? 1 : is_ref_to(e.v[2], acc) ? 2 : 0;
+    if (!ai || !is_global_aref(it, e.v[3 - ai], r.bias)) return false;
+    r.bias_idx = e.v[3 - ai].v[2];
+  } else if (!is_ref_to(e, acc)) {
+    return false;
+  }
+  if (r.out == r.a || r.out == r.b) return false;
+  r.kind = R_MATMUL;
+  return true;
+}
+
+// for t < T: for d < D: { acc = 0; for v < V: acc += where(eq(v, idx[t]), W[v, d], 0); out[t, d] = acc }
+// (eq is spelled not(!=), source/api/function.lisp; the compared index may be cast to the table's dtype)
+static const Sx &strip_cast(const Sx &e) { return (e.call("cast") && e.n() == 3) ? strip_cast(e.v[2]) : e; }
+static bool match_embedding(const Item &it, Route &r) {
+  const std::vector<BpNode> &b = it.body;
+  if (b.size() != 9) return false;
+  if (b[0].t != BpNode::FOR || b[1].t != BpNode::FOR || b[2].t != BpNode::EXPR || b[3].t != BpNode::FOR || b[4].t != BpNode::EXPR ||
+      b[5].t != BpNode::ENDFOR || b[6].t != BpNode::EXPR || b[7].t != BpNode::ENDFOR || b[8].t != BpNode::ENDFOR)
+    return false;
+  const int fors[3] = {0, 1, 3};
+  for (int q = 0; q < 3; q++) {
+    const Sx *ub = upper_bound(b[fors[q]]);
+    if (!ub || !is_zero(b[fors[q]].upfrom)) return false;
+    r.idx[q] = b[fors[q]].idx;
+    r.bound[q] = *ub;
+  }
+  if (!b[2].declare || b[2].writes.size() != 1 || !is_scalar_ref(b[2].writes[0]) || !is_zero(b[2].rhs)) return false;
+  const std::string acc = ref_name(b[2].writes[0]);
+  Sx term;
+  if (!reduction_term(b[4], acc, "add", term) || !term.call("where") || term.n() != 4 || !is_zero(term.v[3])) return false;
+  const Sx &cond = term.v[1];
+  if (!cond.call("not") || cond.n() != 2 || !cond.v[1].call("!=") || cond.v[1].n() < 3) return false;
+  const Sx &x = strip_cast(cond.v[1].v[cond.v[1].n() - 2]), &y = strip_cast(cond.v[1].v[cond.v[1].n() - 1]);
+  // one side is the vocabulary index (any spelling of it, checked by evaluation at launch), the other the token
+  // id read from the input
+  const Sx *vside = nullptr, *tside = nullptr;
+  int dummy;
+  if (uses(x, r.idx[2]) && !is_global_aref(it, x, dummy)) vside = &x, tside = &y;
+  else if (uses(y, r.idx[2]) && !is_global_aref(it, y, dummy)) vside = &y, tside = &x;
+  if (!vside || !is_global_aref(it, *tside, r.b) || uses(tside->v[2], r.idx[2]) || uses(tside->v[2], r.idx[1])) return false;
+  r.b_idx = tside->v[2];
+  r.bias_idx = *vside;
+  if (!is_global_aref(it, term.v[2], r.a)) return false;
+  r.a_idx = term.v[2].v[2];
+  if (b[6].writes.size() != 1 || !is_global_aref(it, b[6].writes[0], r.out) || !is_ref_to(b[6].rhs, acc)) return false;
+  r.out_idx = b[6].writes[0].v[2];
+  r.kind = R_EMBEDDING;
+  return true;
+}
+
+// for r < R: { m = -inf; for i < N: m = max(m, x[r, i]); g = 0; for i < N: g = max(g, where(eq(x[r, i], m), (N - 1) - i, 0));
+//              out[r] = cast(N - g - 1) }      -- ArgMaxNode, lowest index among ties
+static bool match_argmax(const Item &it, Route &r) {
+  const std::vector<BpNode> &b = it.body;
+  if (b.size() != 11) return false;
+  const BpNode::T want[11] = {BpNode::FOR, BpNode::EXPR, BpNode::FOR, BpNode::EXPR, BpNode::ENDFOR, BpNode::EXPR, BpNode::FOR,
+                              BpNode::EXPR, BpNode::ENDFOR, BpNode::EXPR, BpNode::ENDFOR};
+  for (int k = 0; k < 11; k++)
+    if (b[k].t != want[k]) return false;
+  const Sx *rows = upper_bound(b[0]), *n1 = upper_bound(b[2]), *n2 = upper_bound(b[6]);
+  if (!rows || !n1 || !n2 || !is_zero(b[0].upfrom) || !is_zero(b[2].upfrom) || !is_zero(b[6].upfrom)) return false;
+  r.idx[0] = b[0].idx;
+  r.idx[1] = b[2].idx;
+  r.bound[0] = *rows;
+  r.bound[1] = *n1;
+  double v;
+  if (!b[1].declare || !const_value(b[1].rhs, v) || !(isinf(v) && v < 0) || !is_scalar_ref(b[1].writes[0])) return false;
+  const std::string m = ref_name(b[1].writes[0]);
+  Sx term;
+  if (!reduction_term(b[3], m, "max", term) || !is_global_aref(it, term, r.a)) return false;
+  r.a_idx = term.v[2];
+  if (!b[5].declare || !is_zero(b[5].rhs) || !is_scalar_ref(b[5].writes[0])) return false;
+  const std::string g = ref_name(b[5].writes[0]);
+  Sx t2;
+  if (!reduction_term(b[7], g, "max", t2) || !t2.call("where") || t2.n() != 4 || !is_zero(t2.v[3])) return false;
+  const Sx &cond = t2.v[1];
+  if (!cond.call("not") || cond.n() != 2 || !cond.v[1].call("!=") || cond.v[1].n() < 3) return false;
+  const Sx &x = cond.v[1].v[cond.v[1].n() - 2], &y = cond.v[1].v[cond.v[1].n() - 1];
+  int xa = -1;
+  if (!((is_global_aref(it, x, xa) && is_ref_to(y, m)) || (is_global_aref(it, y, xa) && is_ref_to(x, m))) || xa != r.a) return false;
+  // the value kept is (N - 1) - i, in any spelling: checked by evaluation at launch
+  r.b_idx = strip_cast(t2.v[2]);
+  if (b[6].idx != r.idx[1]) r.idx[2] = b[6].idx;  // the second loop's own index name: evaluation binds both
+  int op = -1;
+  if (b[9].writes.size() != 1 || !b[9].writes[0].call("aref") || (op = arg_pos(it, b[9].writes[0].v[1].s)) < 0) return false;
+  if (it.globals[op].dtype != "int64" || !it.globals[op].pointer) return false;
+  r.out = op;
+  r.out_idx = b[9].writes[0].n() > 2 ? b[9].writes[0].v[2] : sx_int(0);
+  r.bias_idx = strip_cast(b[9].rhs);  // N - g - 1, checked by evaluation at launch
+  r.idx[2] = r.idx[2].empty() ? r.idx[1] : r.idx[2];
+  r.kind = R_ARGMAX;
+  r.bound[2] = sx_sym(g);  // the name of the kept maximum: the launch evaluates the final expression over it
+  return true;
+}
+
+// for r < R: { m = -inf; for i: m = max(m, x); s = 0; for i: s += exp2((x - m) * c); for i: y = exp2((x - m) * c) * recip(s) }
+static bool is_exp_of_shifted(const Item &it, const Sx &e, const std::string &m, int &xpos, Sx &xidx) {
+  if (!e.call("exp2") || e.n() != 2) return false;
+  const Sx &mul = e.v[1];
+  if (!mul.call("mul") || mul.n() != 3) return false;
+  double c;
+  const Sx *sh = nullptr;
+  if (const_value(mul.v[2], c)) sh = &mul.v[1];
+  else if (const_value(mul.v[1], c)) sh = &mul.v[2];
+  if (!sh || fabs(c - 1.4426950408889634) > 1e-5) return false;
+  if (!sh->call("add") || sh->n() != 3) return false;
+  const Sx *xa = nullptr, *neg = nullptr;
+  if (sh->v[2].call("neg")) xa = &sh->v[1], neg = &sh->v[2];
+  else if (sh->v[1].call("neg")) xa = &sh->v[2], neg = &sh->v[1];
+  if (!xa || neg->n() != 2 || !is_ref_to(neg->v[1], m) || !is_global_aref(it, *xa, xpos)) return false;
+  xidx = xa->v[2];
+  return true;
+}
+static bool match_softmax(const Item &it, Route &r) {
+  const std::vector<BpNode> &b = it.body;
+  if (b.size() != 13) return false;
+  const BpNode::T want[13] = {BpNode::FOR, BpNode::EXPR, BpNode::FOR, BpNode::EXPR, BpNode::ENDFOR, BpNode::EXPR, BpNode::FOR,
+                              BpNode::EXPR, BpNode::ENDFOR, BpNode::FOR, BpNode::EXPR, BpNode::ENDFOR, BpNode::ENDFOR};
+  for (int k = 0; k < 13; k++)
+    if (b[k].t != want[k]) return false;
+  const Sx *rows = upper_bound(b[0]), *n1 = upper_bound(b[2]), *n2 = upper_bound(b[6]), *n3 = upper_bound(b[9]);
+  if (!rows || !n1 || !n2 || !n3 || !is_zero(b[0].upfrom) || !is_zero(b[2].upfrom) || !is_zero(b[6].upfrom) || !is_zero(b[9].upfrom)) return false;
+  if (b[2].idx != b[6].idx || b[2].idx != b[9].idx) return false;
+  r.idx[0] = b[0].idx;
+  r.idx[1] = b[2].idx;
+  r.bound[0] = *rows;
+  r.bound[1] = *n1;
+  double v;
+  if (!b[1].declare || !const_value(b[1].rhs, v) || !(isinf(v) && v < 0) || !is_scalar_ref(b[1].writes[0])) return false;
+  const std::string m = ref_name(b[1].writes[0]);
+  Sx term;
+  if (!reduction_term(b[3], m, "max", term) || !is_global_aref(it, term, r.a)) return false;
+  r.a_idx = term.v[2];
+  if (!b[5].declare || !is_zero(b[5].rhs) || !is_scalar_ref(b[5].writes[0])) return false;
+  const std::string s = ref_name(b[5].writes[0]);
+  Sx t2, xi;
+  int xp = -1;
+  if (!reduction_term(b[7], s, "add", t2) || !is_exp_of_shifted(it, t2, m, xp, xi) || xp != r.a) return false;
+  const Sx &e = b[10].rhs;
+  if (!e.call("mul") || e.n() != 3) return false;
+  const Sx *ex = nullptr, *rc = nullptr;
+  if (e.v[2].call("recip")) ex = &e.v[1], rc = &e.v[2];
+  else if (e.v[1].call("recip")) ex = &e.v[2], rc = &e.v[1];
+  if (!ex || rc->n() != 2 || !is_ref_to(rc->v[1], s) || !is_exp_of_shifted(it, *ex, m, xp, xi) || xp != r.a) return false;
+  if (b[10].writes.size() != 1 || !is_global_aref(it, b[10].writes[0], r.out) || r.out == r.a) return false;
+  r.out_idx = b[10].writes[0].v[2];
+  r.kind = R_SOFTMAX;
+  return true;
+}
+
+// ------------------------------------------------------------------ rendering a kernel
+static const char *kHeader =
+    "\n#define _infinity __builtin_inff()\n"
+    "#define _negative_infinity (-__builtin_inff())\n"
+    "#define _nan __builtin_nanf(\"\")\n"
+    "#define ct_max(a, b) ((a) > (b) ? (a) : (b))\n"
+    "#define ct_min(a, b) ((a) < (b) ? (a) : (b))\n"
+    "// reductions over the 64 lanes of a wavefront (every lane gets the result)\n"
+    "#define CT_WAVE_REDUCE(name, T, OP)                                        \\\n"
+    "  static __device__ __forceinline__ T name(T v) {                          \\\n"
+    "    for (int o = 32; o > 0; o >>= 1) { T w = __shfl_xor(v, o, 64); v = OP; } \\\n"
+    "    return v;                                                              \\\n"
+    "  }\n"
+    "CT_WAVE_REDUCE(ct_wave_add_f, float, v + w)\n"
+    "CT_WAVE_REDUCE(ct_wave_max_f, float, ct_max(v, w))\n"
+    "CT_WAVE_REDUCE(ct_wave_min_f, float, ct_min(v, w))\n"
+    "CT_WAVE_REDUCE(ct_wave_mul_f, float, v * w)\n";
+
+struct KernelRenderer {
+  const Item &it;
+  Rend R;
+  std::map<std::string, bool> locals;
+  explicit KernelRenderer(const Item &item) : it(item) {
+    for (const BpNode &n : it.body)
+      if (n.t == BpNode::EXPR && n.declare)
+        for (const Sx &w : n.writes) locals[ref_name(w)] = true;
+  }
+
+  // how many leading FOR nodes of the body (a perfect nest) are data-parallel
+  int parallel_prefix() {
+    const std::vector<BpNode> &b = it.body;
+    int depth = 0;
+    while (depth < (int)b.size() && b[depth].t == BpNode::FOR) {
+      const BpNode &f = b[depth];
+      const int j = match_end(b, depth);
+      if (j != (int)b.size() - 1 - depth) break;
+      bool ok = true;
+      if (!f.global_scope) {
+        for (int q = depth + 1; q < j && ok; q++) {
+          const BpNode &n = b[q];
+          if (n.t != BpNode::EXPR) continue;
+          for (const Sx &w : n.writes) {
+            const bool local = n.declare || is_scalar_ref(w) || locals.count(ref_name(w));
+            if (!local && !uses(w, f.idx)) ok = false;
+          }
+        }
+        if (!(is_zero(f.upfrom) && upper_bound(f))) ok = false;
+      } else if (!upper_bound(f) || !is_zero(f.upfrom)) {
+        ok = false;
+      }
+      if (!ok) break;
+      depth++;
+    }
+    return depth;
+  }
+
+  // Row-reduction pattern inside the parallel prefix: {position of an ENDFOR: scalars to combine across lanes}.
+  // found == false: the row stays in one thread.
+  bool wave_reductions(int lo, int hi, std::map<int, std::vector<std::pair<std::string, std::string>>> &out) {
+    const std::vector<BpNode> &b = it.body;
+    int depth = 0;
+    std::map<std::string, std::pair<bool, double>> init;  // scalar -> (is a constant, its value)
+    std::vector<std::pair<std::string, std::string>> loop_red;
+    std::vector<std::string> loop_reduced;  // targets of reductions in the loop being walked
+    bool pending_bad = false;
+    for (int pos = lo; pos < hi; pos++) {
+      const BpNode &n = b[pos];
+      if (n.t == BpNode::FOR) {
+        if (++depth > 1 || n.global_scope || !is_one(n.by)) return false;
+        loop_red.clear();
+        loop_reduced.clear();
+        pending_bad = false;
+      } else if (n.t == BpNode::ENDFOR) {
+        depth--;
+        if (pending_bad) return false;
+        if (!loop_red.empty()) out[pos] = loop_red;
+        loop_red.clear();
+      } else if (n.t == BpNode::IF || n.t == BpNode::ENDIF) {
+        return false;
+      } else {
+        if (n.writes.size() != 1) return false;
+        const Sx &w = n.writes[0];
+        const bool scalar = is_scalar_ref(w);
+        const std::string name = ref_name(w);
+        if (depth == 0) {
+          if (scalar) {
+            double v;
+            const bool c = const_value(n.rhs, v);
+            init[name] = {c, c ? v : 0.0};
+          }
+          continue;
+        }
+        if (!n.reduction) {
+          if (scalar) return false;  // a loop-carried scalar that is not a reduction cannot be split over lanes
+          // an array store that reads a scalar reduced in this same loop (a running sum) would see a lane's
+          // partial: such a row stays in one thread
+          for (const std::string &t : loop_reduced)
+            if (uses(n.rhs, t)) return false;
+          // ... also when the reduction comes later in the loop body
+          continue;
+        }
+        if (n.dtype != "float32") return false;  // the lane butterflies are fp32
+        static const std::map<std::string, std::pair<std::string, double>> ident = {
+            {"add", {"add", 0.0}}, {"max", {"max", -INFINITY}}, {"min", {"min", INFINITY}}, {"mul", {"mul", 1.0}}};
+        const Sx &e = n.rhs;
+        if (!scalar || !e.is_list() || e.n() != 3 || e.v[0].kind != Sx::SYM || !ident.count(e.v[0].s)) return false;
+        const auto &id = ident.at(e.v[0].s);
+        const bool s1 = is_ref_to(e.v[1], name), s2 = is_ref_to(e.v[2], name);
+        if (s1 == s2 || uses(e.v[s1 ? 2 : 1], name)) return false;
+        // lane partials combine when each starts at the identity; max / min are idempotent, so there any start
+        // value that all lanes share (a scalar set before the loop) will do
+        auto in = init.find(name);
+        const bool at_identity = in != init.end() && in->second.first && in->second.second == id.second;
+        if (!at_identity && !((id.first == "max" || id.first == "min") && in != init.end())) return false;
+        loop_red.push_back({name, id.first});
+        loop_reduced.push_back(name);
+        // array stores earlier in this loop that read the scalar
+        for (int q = pos - 1; q >= lo && b[q].t != BpNode::FOR; q--)
+          if (b[q].t == BpNode::EXPR && !b[q].reduction && uses(b[q].rhs, name)) pending_bad = true;
+      }
+    }
+    return !out.empty();
+  }
+
+  bool render(Program &pg, std::string &err) {
+    const std::vector<BpNode> &b = it.body;
+    std::string o;
+    std::string params;
+    for (const Global &g : it.globals) {
+      const std::string &ct = cdtypes().at(g.dtype);
+      if (!params.empty()) params += ", ";
+      if (g.pointer) params += std::string(g.type == "input" ? "const " : "") + ct + "*" + (g.type == "input" ? " __restrict__ " : " ") + g.id;
+      else params += "const " + ct + " " + g.id;
+    }
+    o += "extern \"C\" __global__ void __launch_bounds__(256) " + it.name + "(" + params + ") {\n";
+    const int npar = parallel_prefix();
+    std::map<int, std::vector<std::pair<std::string, std::string>>> wave_red;
+    const int lo = npar, hi = (int)b.size() - npar;
+    const bool wave = npar > 0 && wave_reductions(lo, hi, wave_red);
+    pg.rows_per_block = wave ? 4 : 256;
+    pg.parallel = npar > 0;
+    int indent = 2;
+    auto pad = [&]() { return std::string((size_t)indent, ' '); };
+    if (npar) {
+      std::string total;
+      for (int q = 0; q < npar; q++) {
+        const Sx *ub = upper_bound(b[q]);
+        pg.grid_bounds.push_back(*ub);
+        total += std::string(q ? "*" : "") + "(long long)(" + R.expr(*ub, "int64") + ")";
+      }
+      o += pad() + "const long long _total = " + total + ";\n";
+      if (wave) {
+        o += pad() + "long long _t = ((long long)blockIdx.x * 256 + threadIdx.x) >> 6;  // one wavefront per row\n";
+        o += pad() + "const int _lane = threadIdx.x & 63;\n";
+      } else {
+        o += pad() + "long long _t = (long long)blockIdx.x * 256 + threadIdx.x;\n";
+      }
+      o += pad() + "if (_t >= _total) return;\n";
+      for (int q = npar - 1; q >= 0; q--) {  // innermost loop varies fastest
+        const std::string bs = R.expr(*upper_bound(b[q]), "int64");
+        o += pad() + "const int " + b[q].idx + " = (int)(_t % (long long)(" + bs + ")); _t /= (long long)(" + bs + ");\n";
+      }
+    }
+    int depth = 0;
+    std::vector<std::string> closers;
+    for (int pos = lo; pos < hi; pos++) {
+      const BpNode &n = b[pos];
+      if (n.t == BpNode::FOR) {
+        bool done = false;
+        if (wave) {  // the lanes of the row's wavefront stride this axis together
+          double flo, fhi;
+          const Sx *ub = upper_bound(n);
+          if (ub && const_value(n.upfrom, flo) && const_value(*ub, fhi) && flo == floor(flo) && fhi == floor(fhi)) {
+            const long long l = (long long)flo, h = (long long)fhi, per = (h - l + 63) / 64;
+            if (per > 0 && per <= 32) {
+              // a static row of at most 32 elements per lane: a counted loop, unrolled, so that the loops over the
+              // same row share their loads (inputs are __restrict__) and the row is read once
+              const bool ragged = (h - l) % 64 != 0;
+              o += pad() + "#pragma unroll\n";
+              o += pad() + "for (int " + n.idx + "_i=0; " + n.idx + "_i<" + std::to_string(per) + "; " + n.idx + "_i++) { const int " +
+                   n.idx + "=" + std::to_string(l) + "+_lane+64*" + n.idx + "_i;" + (ragged ? " if (" + n.idx + "<" + std::to_string(h) + ") {" : "") + "\n";
+              closers.push_back(ragged ? "}}" : "}");
+              done = true;
+            }
+          }
+          if (!done) {
+            o += pad() + "for (int " + n.idx + "=(" + R.expr(n.upfrom, "int64") + ")+_lane; " + R.expr(n.below, "int64") + "; " + n.idx + "+=64) {\n";
+            closers.push_back("}");
+          }
+        } else {
+          o += pad() + "for (int " + n.idx + "=" + R.expr(n.upfrom, "int64") + "; " + R.expr(n.below, "int64") + "; " + n.idx + "+=" +
+               R.expr(n.by, "int64") + ") {\n";
+          closers.push_back("}");
+        }
+        indent += 2;
+        depth++;
+      } else if (n.t == BpNode::ENDFOR) {
+        indent -= 2;
+        depth--;
+        o += pad() + closers.back() + "\n";
+        closers.pop_back();
+        if (wave && wave_red.count(pos))
+          for (const auto &vr : wave_red[pos]) o += pad() + vr.first + " = ct_wave_" + vr.second + "_f(" + vr.first + ");\n";
+      } else if (n.t == BpNode::IF) {
+        o += pad() + "if (" + R.expr(n.cond, "int64") + ") {\n";
+        indent += 2;
+      } else if (n.t == BpNode::ENDIF) {
+        indent -= 2;
+        o += pad() + "}\n";
+      } else {
+        std::string lhs;
+        for (size_t k = 0; k < n.writes.size(); k++) lhs += std::string(k ? ", " : "") + (n.writes[k].kind == Sx::SYM ? n.writes[k].s : R.aref(n.writes[k]));
+        std::string stmt = (n.declare ? cdtypes().at(n.dtype) + " " : "") + lhs + " = " + R.expr(n.rhs, n.dtype) + ";";
+        bool global_write = false;
+        for (const Sx &w : n.writes)
+          if (!locals.count(ref_name(w))) global_write = true;
+        if (wave && depth == 0 && !n.declare && global_write) stmt = "if (_lane == 0) { " + stmt + " }";  // every lane holds the value; one stores it
+        o += pad() + stmt + "\n";
+      }
+    }
+    o += "}\n";
+    if (!R.err.empty()) return err = R.err, false;
+    pg.source = o;
+    return true;
+  }
+};
+
+// entry points of the hand-written kernels the routes use (matmul.hip, linear.hip, rowops.hip)
+int matmul_routed(float *C, const float *A, const float *B, int M, int N, int K, int act, const float *bias, bool b_is_nk);
+
+static bool launch_route(Program &pg, void **args, const std::map<std::string, long long> &env, int &rc) {
+  Route &r = pg.route;
+  rc = 0;
+  auto ptr = [&](int pos) { return *(void **)args[pos]; };
+  auto bound = [&](int q, long long &v) { return eval_int(r.bound[q], env, v) && v >= 0 && v <= 0x7fffffff; };
+  if (r.kind == R_MATMUL) {
+    long long M, N, K;
+    if (!bound(0, M) || !bound(1, N) || !bound(2, K)) return false;
+    Affine ao, aa, ab, abias;
+    if (!affine_of(r.out_idx, r.idx, 3, env, ao) || !affine_of(r.a_idx, r.idx, 3, env, aa) || !affine_of(r.b_idx, r.idx, 3, env, ab)) return false;
+    // C (M,N) row-major, A (M,K) row-major
+    if (ao.base || ao.c[0] != N || ao.c[1] != 1 || ao.c[2] != 0) return false;
+    if (aa.base || aa.c[0] != K || aa.c[1] != 0 || aa.c[2] != 1) return false;
+    bool b_nk;
+    if (ab.base == 0 && ab.c[0] == 0 && ab.c[1] == 1 && ab.c[2] == N) b_nk = false;       // B (K,N) row-major
+    else if (ab.base == 0 && ab.c[0] == 0 && ab.c[1] == K && ab.c[2] == 1) b_nk = true;   // W (N,K) read through a transposed view
+    else return false;
+    const float *bias = nullptr;
+    if (r.bias >= 0) {
+      if (!affine_of(r.bias_idx, r.idx, 3, env, abias) || abias.base || abias.c[0] || abias.c[1] != 1 || abias.c[2]) return false;
+      bias = (const float *)ptr(r.bias);
+    }
+    if (M == 0 || N == 0) return true;
+    rc = matmul_routed((float *)ptr(r.out), (const float *)ptr(r.a), (const float *)ptr(r.b), (int)M, (int)N, (int)K, r.act, bias, b_nk);
+    pg.last_route = b_nk ? "cthip_linear" : "cthip_matmul";
+    return true;
+  }
+  if (r.kind == R_EMBEDDING) {
+    long long T, D, V;
+    if (!bound(0, T) || !bound(1, D) || !bound(2, V)) return false;
+    Affine ao, aw, ai;
+    if (!affine_of(r.out_idx, r.idx, 3, env, ao) || !affine_of(r.a_idx, r.idx, 3, env, aw) || !affine_of(r.b_idx, r.idx, 3, env, ai)) return false;
+    if (ao.base || ao.c[0] != D || ao.c[1] != 1 || ao.c[2]) return false;  // out (T, D)
+    if (aw.base || aw.c[0] || aw.c[1] != 1 || aw.c[2] != D) return false;  // W (V, D)
+    if (ai.base || ai.c[0] != 1 || ai.c[1] || ai.c[2]) return false;       // idx (T)
+    Affine av;
+    if (!affine_of(r.bias_idx, r.idx, 3, env, av) || av.base || av.c[0] || av.c[1] || av.c[2] != 1) return false;  // compared with v itself
+    if (T == 0 || D == 0) return true;
+    rc = cthip_embedding((float *)ptr(r.out), (const float *)ptr(r.a), (const float *)ptr(r.b), (int)T, (int)V, (int)D);
+    pg.last_route = "cthip_embedding";
+    return true;
+  }
+  if (r.kind == R_ARGMAX) {
+    long long Rn, N;
+    if (!bound(0, Rn) || !bound(1, N) || N < 1) return false;
+    Affine ax, ao;
+    if (!affine_of(r.a_idx, r.idx, 2, env, ax) || ax.base || ax.c[0] != N || ax.c[1] != 1) return false;
+    const std::string oi[3] = {r.idx[0], "", ""};
+    if (!affine_of(r.out_idx, oi, 1, env, ao) || ao.base || (ao.c[0] != 1 && Rn > 1)) return false;
+    // kept value (N - 1) - i and result N - g - 1, whatever their spelling
+    std::map<std::string, long long> e2 = env;
+    for (long long i : {0ll, 1ll, N - 1}) {
+      e2[r.idx[1]] = i;
+      e2[r.idx[2]] = i;
+      long long v;
+      if (!eval_int(r.b_idx, e2, v) || v != (N - 1) - i) return false;
+    }
+    for (long long g : {0ll, N - 1}) {
+      e2[r.bound[2].s] = g;
+      long long v;
+      if (!eval_int(r.bias_idx, e2, v) || v != N - g - 1) return false;
+    }
+    if (Rn == 0) return true;
+    rc = cthip_argmax((int64_t *)ptr(r.out), (const float *)ptr(r.a), Rn, (int)N);
+    pg.last_route = "cthip_argmax";
+    return true;
+  }
+  if (r.kind == R_SOFTMAX) {
+    long long Rn, N;
+    if (!bound(0, Rn) || !bound(1, N) || N < 1) return false;
+    Affine ax, ao;
+    if (!affine_of(r.a_idx, r.idx, 2, env, ax) || ax.base || ax.c[0] != N || ax.c[1] != 1) return false;
+    if (!affine_of(r.out_idx, r.idx, 2, env, ao) || ao.base || ao.c[0] != N || ao.c[1] != 1) return false;
+    if (Rn == 0) return true;
+    rc = cthip_softmax((float *)ptr(r.out), (const float *)ptr(r.a), Rn, (int)N);
+    pg.last_route = "cthip_softmax";
+    return true;
+  }
+  return false;
+}
+
+}  // namespace cthip
+
+using namespace cthip;
+
+extern "C" {
+
+const char *cthip_render_header(void) { return kHeader; }
+
+int cthip_program_create(void **program, const char *blueprint) {
+  CTHIP_ARG(program != nullptr && blueprint != nullptr);
+  Parser ps{blueprint, {}};
+  Sx top;
+  if (!ps.parse(top)) return fail(CTHIP_E_BAD_ARG, "cthip_program_create: %s", ps.err.c_str());
+  Program *pg = new Program();
+  std::string err;
+  if (!build_item(top, pg->item, err)) {
+    delete pg;
+    return fail(CTHIP_E_BAD_ARG, "cthip_program_create: %s", err.c_str());
+  }
+  KernelRenderer kr(pg->item);
+  if (!kr.render(*pg, err)) {
+    delete pg;
+    return fail(CTHIP_E_UNSUPPORTED, "cthip_program_create: %s", err.c_str());
+  }
+  Route r;
+  if (match_matmul(pg->item, r)) pg->route = r, pg->route_name = "matmul";
+  else if ((r = Route(), match_embedding(pg->item, r))) pg->route = r, pg->route_name = "embedding";
+  else if ((r = Route(), match_argmax(pg->item, r))) pg->route = r, pg->route_name = "argmax";
+  else if ((r = Route(), match_softmax(pg->item, r))) pg->route = r, pg->route_name = "softmax";
+  *program = pg;
+  return 0;
+}
+
+int cthip_program_destroy(void *program) {
+  delete (Program *)program;
+  return 0;
+}
+
+const char *cthip_program_source(const void *program) { return program ? ((const Program *)program)->source.c_str() : ""; }
+const char *cthip_program_name(const void *program) { return program ? ((const Program *)program)->item.name.c_str() : ""; }
+const char *cthip_program_route(const void *program) { return program ? ((const Program *)program)->route_name.c_str() : ""; }
+const char *cthip_program_last_route(const void *program) { return program ? ((const Program *)program)->last_route.c_str() : ""; }
+
+int cthip_program_bind(void *program, void *module) {
+  CTHIP_REQUIRE_INIT();
+  CTHIP_ARG(program != nullptr && module != nullptr);
+  Program *pg = (Program *)program;
+  void *fn = nullptr;
+  int rc = cthip_get_function(&fn, module, pg->item.name.c_str());
+  if (rc) return rc;
+  pg->fn = (hipFunction_t)fn;
+  return 0;
+}
+
+int cthip_program_launch(void *program, void **args, int nargs) {
+  CTHIP_REQUIRE_INIT();
+  CTHIP_ARG(program != nullptr && (nargs == 0 || args != nullptr));
+  Program *pg = (Program *)program;
+  const Item &it = pg->item;
+  if (nargs != (int)it.globals.size())
+    return fail(CTHIP_E_BAD_ARG, "HIP: %s takes %zu arguments, got %d", it.name.c_str(), it.globals.size(), nargs);
+  std::map<std::string, long long> env;
+  for (int k = 0; k < nargs; k++) {
+    const Global &g = it.globals[k];
+    if (!args[k]) return fail(CTHIP_E_BAD_ARG, "HIP: %s: argument %s is null", it.name.c_str(), g.id.c_str());
+    if (g.pointer) {
+      if (!*(void **)args[k]) return fail(CTHIP_E_BAD_ARG, "HIP: please transfer the buffer %s to the device first", g.id.c_str());
+      continue;
+    }
+    long long v = 0;
+    if (g.dtype == "int64" || g.dtype == "uint64") v = *(long long *)args[k];
+    else if (g.dtype == "int32") v = *(int *)args[k];
+    else if (g.dtype == "uint32") v = *(unsigned *)args[k];
+    else if (g.dtype == "int16") v = *(short *)args[k];
+    else if (g.dtype == "uint16") v = *(unsigned short *)args[k];
+    else if (g.dtype == "int8") v = *(signed char *)args[k];
+    else if (g.dtype == "uint8" || g.dtype == "bool") v = *(unsigned char *)args[k];
+    else continue;  // floating-point scalars do not size anything
+    env[g.id] = v;
+  }
+  if (pg->route.kind != R_NONE && state().render_routes) {
+    int rc = 0;
+    if (launch_route(*pg, args, env, rc)) return rc;
+  }
+  if (!pg->fn) return fail(CTHIP_E_STATE, "HIP: %s has not been bound to a compiled module (cthip_program_bind)", it.name.c_str());
+  long long total = 1;
+  for (const Sx &b : pg->grid_bounds) {
+    long long v;
+    if (!eval_int(b, env, v)) return fail(CTHIP_E_UNSUPPORTED, "HIP: %s: a loop bound is not an expression of the shape arguments", it.name.c_str());
+    total *= v > 0 ? v : 0;
+  }
+  unsigned grid[3] = {1, 1, 1}, block[3] = {1, 1, 1};
+  if (pg->parallel) {
+    const long long per = pg->rows_per_block;
+    const long long nb = (total + per - 1) / per;
+    if (nb > 0x7fffffffll) return fail(CTHIP_E_UNSUPPORTED, "HIP: %s: %lld workgroups exceed the grid", it.name.c_str(), nb);
+    if (nb == 0) return 0;
+    grid[0] = (unsigned)nb;
+    block[0] = 256;
+  }
+  pg->last_route = "rendered";
+  return cthip_launch(pg->fn, grid, block, 0, args, nargs);
+}
+
+}  // extern "C"

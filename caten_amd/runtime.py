@@ -82,6 +82,7 @@ class GraphRuntime:
         self.pc = 0
         self.profile = os.environ.get("PROFILE", "0") == "1"
         self.times = {"kernel": 0.0, "vm": 0.0, "allocate": 0.0}
+        self._casts: List[AbstractBuffer] = []  # storage opened by :View nodes that cast a scalar to an array
 
     # runtime-setvar / runtime-getvar (runtime.lisp:66-74)
     def setvar(self, var, value):
@@ -128,9 +129,13 @@ class GraphRuntime:
 
     def free(self):
         """free-runtime (runtime.lisp:76-81)"""
+        # views and copies are closed like the rest but own nothing: every block goes back exactly once
         for v in self.variables.values():
             if isinstance(v, AbstractBuffer):
                 close_buffer(self, v)
+        for b in self._casts:
+            close_buffer(self, b)
+        self._casts.clear()
         for n in self.graph:
             pool = n.attrs.get("pool")
             if isinstance(pool, AbstractBuffer):
@@ -180,9 +185,17 @@ class GraphRuntime:
         shape, v1, v2, v3, stride = (rest[i * nrank:(i + 1) * nrank] for i in range(5))
         bc = node.attrs.get("broadcast", [False] * nrank)
         buf = base.copy()
+        initial = buf.value
+        scalar_to_tensor = nrank > 0 and isinstance(initial, (bool, int, float, np.number)) and base.nrank == 0
         buf.shape, buf.stride = [int(s) for s in shape], [int(s) for s in stride]
         buf.views = [(int(a), int(b), int(c), bool(d)) for a, b, c, d in zip(v1, v2, v3, bc)]
         buf.nrank = nrank
+        if scalar_to_tensor:
+            # casting a scalar to an array: storage of its own, every element the scalar (runtime.lisp:274-283)
+            open_buffer(self, buf)
+            n = int(np.prod([1 if b else int(s) for b, s in zip(bc, shape)])) if nrank else 1
+            transfer_from_array(self, buf, np.full(n, initial, DTYPES[buf.dtype]))
+            self._casts.append(buf)
         return buf
 
     def realize_jit_kernel(self, node: Node, args):

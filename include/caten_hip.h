@@ -101,6 +101,33 @@ int cthip_get_function(void **fn, void *module, const char *name);
 int cthip_launch(void *fn, const unsigned grid[3], const unsigned block[3], unsigned lds_bytes,
                  void **args, int nargs);
 
+/* ---- Hip-Renderer: %render-kernel / invoke behind the C ABI ----
+ * The renderer protocol (source/codegen/renderer.lisp:30-34) is a Lisp class; its work for this backend -- HIP
+ * source with gfx950-aware work distribution for a Schedule-Item, and the choice of a hand-written kernel where
+ * the item is a matmul / Linear / one-hot Embedding / ArgMax / softmax-row shape -- is done here, so the Lisp
+ * Hip-Renderer only prints the blueprint as an s-expression (grammar: header of caten_amd/csrc/render.hip).
+ *   %render-kernel  = cthip_program_create + cthip_program_source   (CLANG: clang.lisp:21-110; METAL: metal.lisp:178-250)
+ *   %compile-kernel = cthip_render_header + every program's source -> cthip_compile -> cthip_module_load ->
+ *                     cthip_program_bind per item                   (clang.lisp:207-226, metal.lisp:326-345)
+ *   invoke          = cthip_program_launch: args[i] points at the i-th argument value (a device pointer or a
+ *                     by-value scalar) in Caten's order outputs -> dynamic shapes -> inputs
+ *                     (rewriting-rules.lisp:207-231; metal.lisp:288-322).  The grid comes from the item's
+ *                     data-parallel loops and the shape arguments.  A program with a route checks the actual
+ *                     layout at every launch and falls back to its rendered kernel when it does not fit.
+ * cthip_program_route: "rendered", or the shape recognised at creation ("matmul", "embedding", "argmax",
+ * "softmax"); cthip_program_last_route: what the last launch ran ("rendered", "cthip_matmul", "cthip_linear",
+ * "cthip_embedding", "cthip_argmax", "cthip_softmax").  Strings stay valid until the program is destroyed.
+ * Option "render_routes" 0 makes every program run its rendered kernel. */
+const char *cthip_render_header(void);
+int cthip_program_create(void **program, const char *blueprint);
+int cthip_program_destroy(void *program);
+const char *cthip_program_source(const void *program);
+const char *cthip_program_name(const void *program);
+const char *cthip_program_route(const void *program);
+const char *cthip_program_last_route(const void *program);
+int cthip_program_bind(void *program, void *module);
+int cthip_program_launch(void *program, void **args, int nargs);
+
 /* Event timing on the library's stream (PROFILE=1 in the reference times each
  * JIT kernel on the host clock, source/codegen/runner.lisp:7-31). */
 int cthip_timer_start(void);

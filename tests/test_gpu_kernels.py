@@ -126,8 +126,6 @@ SHAPES = [(768, 768), (2304, 768), (3072, 768), (768, 3072), (5003, 768), (1000,
 @pytest.mark.parametrize("kind", ["q8_0", "q4_0", "f32", "f16"])
 @pytest.mark.parametrize("rows,cols", SHAPES)
 def test_gemv_plain(ops, oracle, kind, rows, cols):
-    if kind in ("f32", "f16") and rows > 6000:
-        pytest.skip("large fp32 case covered by the decoder test")
     print(f"case: gemv {kind} ({rows},{cols})", flush=True)
     from caten_amd.llm import Tensor
     rng = np.random.default_rng(rows * 7 + cols)
@@ -137,6 +135,28 @@ def test_gemv_plain(ops, oracle, kind, rows, cols):
     wd = oracle.dequant(kind, t.raw, w.size).reshape(rows, cols)
     wm = ops.WeightMatrix(kind, t.raw, rows, cols)
     close(ops.linear(x, wm), oracle.linear(x, wd))
+
+
+@pytest.mark.parametrize("kind,cols", [("f32", 10), ("f32", 1023), ("f16", 12), ("f16", 770)])
+@pytest.mark.parametrize("m", [1, 5])
+def test_gemv_rows_that_are_not_whole_chunks(ops, oracle, kind, cols, m):
+    """fp32 / fp16 weight rows whose width is no multiple of four / eight elements: rows start at any element and the
+    last columns count (every column gets a weight that a dropped tail or a wrong row stride would miss)."""
+    print(f"case: gemv {kind} cols {cols} m {m}", flush=True)
+    from caten_amd.llm import Tensor
+    rows = 37
+    rng = np.random.default_rng(cols * 3 + m)
+    w = rng.normal(0, 0.5, (rows, cols)).astype(np.float32)
+    w[:, -1] += 3.0
+    x = rng.normal(0, 1, (m, cols)).astype(np.float32)
+    b = rng.normal(0, 1, rows).astype(np.float32)
+    t = Tensor.from_f32(w, kind)
+    wd = oracle.dequant(kind, t.raw, w.size).reshape(rows, cols)
+    wm = ops.WeightMatrix(kind, t.raw, rows, cols)
+    got = ops.linear(x, wm, bias=b, act="relu")
+    close(got, oracle.relu(oracle.linear(x, wd, b)))
+    ref = np.maximum(x.astype(np.float64) @ wd.astype(np.float64).T + b, 0.0)
+    close(got, ref)
 
 
 @pytest.mark.parametrize("kind", ["q8_0", "q4_0", "f32"])

@@ -124,6 +124,15 @@ def test_vm_view_and_errors():
     v = rt.forward(("x", x))
     assert v.shape == [2, 3] and v.value == x.value  # a view moves no data (runtime.lisp:261-284)
     assert buffer_ref(v, 0, 0) == 4.0 and buffer_ref(v, 1, 2) == 10.0  # rows from 1, by 1
+    # free-runtime with the buffer and its view both in the variable table: the block goes back once
+    import ctypes as C
+    lib = ca._lib.load()
+    live0, live1 = C.c_size_t(), C.c_size_t()
+    ca._lib.check(lib.cthip_cache_stats(C.byref(live0), None, None))
+    rt.free()
+    ca._lib.check(lib.cthip_cache_stats(C.byref(live1), None, None))
+    assert live0.value - live1.value == 256 and v.value is None and x.value is None
+    rt.free()
     # a wrong argument count surfaces as a runtime-error carrying the pc (cf. metal.lisp:289)
     vm = _relu_matmul_graph(ca, 0, 0, 0)
     vm.graph[3].reads = ["out", "m", "n", "a", "b"]
@@ -337,3 +346,177 @@ def test_rendered_argmax_with_index_components(oracle):
     got = transfer_into_array(bo).reshape(rows)
     assert np.array_equal(got, np.argmax(x, axis=1))
     assert np.array_equal(got, np.asarray([oracle.argmax(row) for row in x]).reshape(rows))
+
+
+# ------------------------------------------------------------------ programs routed to the hand-written kernels
+def _run_item(ca, item, arg_values):
+    """render -> compile -> call one Schedule-Item the way realize-node :JIT_KERNEL does; arg_values in DEFINE-GLOBAL
+    order, arrays become device buffers.  Returns (outputs as arrays, the program)."""
+    from caten_amd.buffer import make_buffer, HipBuffer, open_buffer, transfer_from_array, transfer_into_array, close_buffer
+    rt = ca.HipRuntime()
+    r = ca.HipRenderer()
+    r.render_kernel(item)
+    r.compile_kernel([item])
+    prog = item["compiled_object"]
+    args, bufs = [], []
+    globs = [n for n in item["blueprint"] if n["type"] == "DEFINE-GLOBAL"]
+    for g, v in zip(globs, arg_values):
+        if isinstance(v, np.ndarray):
+            shape = list(v.shape)
+            stride = [int(np.prod(shape[k + 1:])) for k in range(len(shape))]
+            b = make_buffer(shape, stride, g["dtype"], device=HipBuffer)
+            open_buffer(rt, b)
+            transfer_from_array(rt, b, v.ravel())
+            bufs.append(b)
+            args.append(b)
+        else:
+            args.append(v)
+    prog(None, *args)
+    outs = [transfer_into_array(b).reshape(b.shape) for g, b in zip(globs, args) if g["arg_type"] == "output" and hasattr(b, "shape") and b.nrank > 0]
+    for b in bufs:
+        close_buffer(rt, b)
+    return outs, prog
+
+
+def test_matmul_item_runs_the_mfma_gemm(oracle):
+    """BASELINE config 1 through the plug-in path: the blueprint of (caten (!relu (!matmul a b))) at 1024^3 is
+    recognised and the launch goes to the MFMA GEMM, not to the rendered thread-per-output kernel; the result is
+    the oracle's (rtol 1e-3 / atol 1e-4); with routes switched off the rendered kernel gives the same."""
+    import caten_amd as ca
+    from caten_amd import blueprints as bp, _lib
+    rng = np.random.default_rng(0)
+    M = N = K = 1024
+    A = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+    B = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    out0 = np.zeros((M, N), np.float32)
+    print("case: routed matmul 1024^3", flush=True)
+    (got,), prog = _run_item(ca, bp.matmul(relu=True), [out0, M, N, K, A, B])
+    assert prog.last_route == "cthip_matmul"
+    want = np.maximum(A.astype(np.float64) @ B.astype(np.float64), 0.0)
+    assert np.all(np.abs(got - want) <= 1e-4 + 1e-3 * np.abs(want))
+    sub = oracle.matmul(A[:16], B, relu=True)  # the oracle's serial fp32 accumulation on a few rows
+    assert np.all(np.abs(got[:16] - sub) <= 1e-4 + 1e-3 * np.abs(sub))
+    # the rendered kernel (routes off) on a smaller case, same function
+    lib = _lib.load()
+    _lib.check(lib.cthip_set_option(b"render_routes", 0))
+    try:
+        (g2,), prog2 = _run_item(ca, bp.matmul(relu=True), [np.zeros((70, 50), np.float32), 70, 50, 33, A[:70, :33].copy(), B[:33, :50].copy()])
+        assert prog2.last_route == "rendered"
+    finally:
+        _lib.check(lib.cthip_set_option(b"render_routes", 1))
+    (g3,), prog3 = _run_item(ca, bp.matmul(relu=True), [np.zeros((70, 50), np.float32), 70, 50, 33, A[:70, :33].copy(), B[:33, :50].copy()])
+    assert prog3.last_route == "cthip_matmul"
+    assert np.all(np.abs(g2 - g3) <= 1e-4 + 1e-3 * np.abs(g3))
+
+
+@pytest.mark.parametrize("M", [1, 5, 64, 130])
+def test_linear_item_through_a_transposed_view(oracle, M):
+    """x @ W^T + b with W (out, in) read through a transposed view (nn/linear.lisp:3-17), ReLU fused
+    (test-scheduler.lisp:140-163): fewer than eight rows go to the single-row kernels, more to the GEMM."""
+    import caten_amd as ca
+    from caten_amd import blueprints as bp
+    print(f"case: routed linear m={M}", flush=True)
+    rng = np.random.default_rng(M)
+    N, K = 300, 768
+    X = rng.normal(0, 1, (M, K)).astype(np.float32)
+    W = rng.normal(0, 0.05, (N, K)).astype(np.float32)
+    b = rng.normal(0, 1, N).astype(np.float32)
+    (got,), prog = _run_item(ca, bp.matmul(bias=True, relu=True, transposed_b=True), [np.zeros((M, N), np.float32), M, N, K, X, W, b])
+    assert prog.last_route == "cthip_linear"
+    want = oracle.relu(oracle.linear(X, W, b))
+    assert np.all(np.abs(got - want) <= 1e-4 + 1e-3 * np.abs(want))
+
+
+def test_matmul_item_with_another_layout_falls_back_to_its_rendered_kernel(oracle):
+    """The route is checked against the actual index arithmetic at every launch: an A that is read with a row
+    stride of 2*k (every other row of a taller matrix) is not what the GEMM takes, so the rendered kernel runs."""
+    import caten_amd as ca
+    from caten_amd import blueprints as bp
+    item = bp.matmul()
+    red = item["blueprint"][-5]["expr"]["args"][1]["args"][0]  # the aref of val_a
+    red["index"] = {"op": "ADD", "args": [{"op": "MUL", "args": [{"op": "MUL", "args": [2, "kk"]}, "_gid0"]}, "_gid2"]}
+    rng = np.random.default_rng(3)
+    M, N, K = 20, 30, 40
+    A2 = rng.uniform(-1, 1, (2 * M, K)).astype(np.float32)
+    B = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    (got,), prog = _run_item(ca, item, [np.zeros((M, N), np.float32), M, N, K, A2, B])
+    assert item["route"] == "matmul" and prog.last_route == "rendered"
+    assert np.allclose(got, oracle.matmul(A2[::2].copy(), B), rtol=1e-3, atol=1e-4)
+
+
+def test_embedding_item_becomes_a_gather(oracle):
+    """The one-hot masked sum over the vocabulary (nn/embedding.lisp:13-25) is launched as a row gather; ids that
+    equal no row (out of range, fractional) select nothing, as in the sum."""
+    import caten_amd as ca
+    from caten_amd import blueprints as bp
+    rng = np.random.default_rng(5)
+    V, D = 5003, 96
+    W = rng.normal(0, 1, (V, D)).astype(np.float32)
+    idx = np.array([0, 17, 5002, 4, 4, 5003, -1, 2.5, 1234], np.float32)
+    (got,), prog = _run_item(ca, bp.embedding_onehot(), [np.zeros((idx.size, D), np.float32), idx.size, D, V, idx, W])
+    assert prog.last_route == "cthip_embedding"
+    assert np.array_equal(got, oracle.embedding_onehot(W, idx))
+
+
+def test_argmax_item(oracle):
+    """ArgMaxNode (high-level-ops.lisp:314-325) routed to the argmax kernel: lowest index among ties, int64 result;
+    the rendered two-reduction kernel agrees."""
+    import caten_amd as ca
+    from caten_amd import blueprints as bp, _lib
+    rng = np.random.default_rng(9)
+    R, N = 7, 50257
+    x = rng.normal(0, 1, (R, N)).astype(np.float32)
+    x[1, 777] = x[1, 40000] = 9.0   # a tie: the lower index wins
+    x[2, 0] = 11.0
+    x[3, N - 1] = 11.0
+    (got,), prog = _run_item(ca, bp.argmax_rows(), [np.zeros(R, np.int64), R, N, x])
+    assert prog.last_route == "cthip_argmax"
+    want = np.array([int(oracle.argmax(row)) for row in x], np.int64)
+    assert np.array_equal(got, want) and got[1] == 777 and got[2] == 0 and got[3] == N - 1
+    lib = _lib.load()
+    _lib.check(lib.cthip_set_option(b"render_routes", 0))
+    try:
+        (g2,), prog2 = _run_item(ca, bp.argmax_rows(), [np.zeros(R, np.int64), R, N, x])
+    finally:
+        _lib.check(lib.cthip_set_option(b"render_routes", 1))
+    assert prog2.last_route == "rendered" and np.array_equal(g2, want)
+
+
+def test_softmax_item_with_dynamic_shape(oracle):
+    import caten_amd as ca
+    from caten_amd import blueprints as bp
+    rng = np.random.default_rng(2)
+    x = (10 + 100 * rng.normal(0, 1, (300, 777))).astype(np.float32)
+    (got,), prog = _run_item(ca, bp.softmax_rows(), [np.zeros_like(x), 300, 777, x])
+    assert prog.last_route == "cthip_softmax"
+    want = oracle.softmax(x)
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-5) and np.allclose(got.sum(-1), 1.0, atol=1e-5)
+
+
+def test_rank0_output_passed_by_pointer_is_written_back():
+    """A rank-0 OUTPUT is declared as a pointer (rewriting-rules.lisp:207-231); CLANG boxes the Lisp number in a
+    one-element foreign object and stores the result back into the buffer (clang.lisp:166-185).  Here the box is a
+    device cell: the kernel writes it, the caller reads it back into the buffer's value."""
+    import caten_amd as ca
+    from caten_amd import blueprints as bp
+    from caten_amd.buffer import make_buffer, HipBuffer, open_buffer, transfer_from_array, close_buffer
+    A = lambda id_, idx: {"op": "AREF", "id": id_, "index": idx}  # noqa: E731
+    item = {"name": "sum_all", "blueprint": [
+        bp._glob("val_s", "output", 0) | {"pointer_p": True}, bp._glob("n", "shape", 0, "int64"), bp._glob("val_x", "input", 1),
+        {"type": "EXPR", "writes": [A("acc", None)], "expr": 0.0, "declare_type": True, "dtype": "float32"},
+        {"type": "FOR", "idx": "_gid0", "upfrom": 0, "below": bp._lt("_gid0", "n"), "by": 1},
+        {"type": "EXPR", "writes": [A("acc", None)], "expr": {"op": "ADD", "args": ["acc", A("val_x", "_gid0")]}, "dtype": "float32", "reduction": True},
+        {"type": "ENDFOR", "idx": "_gid0"},
+        {"type": "EXPR", "writes": [A("val_s", 0)], "expr": {"op": "ADD", "args": ["acc", A("val_s", 0)]}, "dtype": "float32"},
+    ]}
+    rt = ca.HipRuntime()
+    r = ca.HipRenderer()
+    r.render_kernel(item)
+    r.compile_kernel([item])
+    x = make_buffer([100], [1], "float32", device=HipBuffer)
+    open_buffer(rt, x)
+    transfer_from_array(rt, x, np.arange(100, dtype=np.float32))
+    s = make_buffer([], [], "float32", value=0.5, device=HipBuffer)
+    item["compiled_object"](None, s, 100, x)
+    assert s.value == 4950.5  # the incoming value went in, the result came back
+    close_buffer(rt, x)

@@ -57,6 +57,94 @@ def test_buffer_storage_size_and_views():
         make_buffer([3], [1, 1], "float32")
 
 
+class _StubLib:
+    """Stands in for the C ABI's allocator and copies: hands out fake addresses, records every free and upload."""
+
+    def __init__(self):
+        self.next = 0x1000
+        self.live = set()
+        self.freed = []
+        self.uploads = {}
+
+    def cthip_alloc(self, out, nbytes):
+        p = self.next
+        self.next += 0x1000
+        self.live.add(p)
+        out._obj.value = p
+        return 0
+
+    def cthip_free(self, p):
+        assert p in self.live, f"freeing {p:#x}, which is not a live block (double free or stale pointer)"
+        self.live.discard(p)
+        self.freed.append(p)
+        return 0
+
+    def cthip_h2d(self, dst, src, nbytes):
+        self.uploads[dst] = bytes((ctypes.c_char * nbytes).from_address(src))
+        return 0
+
+
+@pytest.fixture
+def stub_lib(monkeypatch):
+    from caten_amd import _lib
+    stub = _StubLib()
+    monkeypatch.setattr(_lib, "load", lambda: stub)
+    monkeypatch.setattr(_lib, "init", lambda device=0: stub)
+    monkeypatch.setattr(_lib, "check", lambda status: None if status == 0 else (_ for _ in ()).throw(AssertionError(status)))
+    return stub
+
+
+def _view_node(nrank, shape, stride, broadcast=None):
+    from caten_amd.runtime import Node
+    reads = ["base"] + list(shape) + [0] * nrank + list(shape) + [1] * nrank + list(stride)
+    return Node("View", ["v"], reads, {"nrank": nrank, "broadcast": broadcast or [False] * nrank})
+
+
+def test_views_do_not_own_storage(stub_lib):
+    """A :View shares its base's storage (copy-buffer, buffer.lisp:60-68): free-runtime releases every block once,
+    and a view of a pool that a dynamic shape closed holds no pointer a later owner could lose."""
+    from caten_amd.runtime import GraphRuntime, Node
+    from caten_amd.buffer import HipBuffer
+
+    class RT(GraphRuntime):
+        buffer_type = HipBuffer
+
+    alloc = Node("Allocate", ["base"], ["n", 4, 4, 1], {"nrank": 2, "dtype": "float32"})
+    rt = RT([alloc, _view_node(2, ["n", 4], [4, 1])], ["v"])
+    v = rt.forward(("n", 3))
+    base = rt.getvar("base")
+    assert v.value == base.value and not v.owns_storage and base.owns_storage
+    first = base.value
+    # the dynamic shape changes: the pool is closed and re-opened; the old view points nowhere
+    v2 = rt.forward(("n", 5))
+    assert stub_lib.freed == [first]
+    assert v.value is None
+    assert v2.value == rt.getvar("base").value != first
+    rt.free()  # the base and its view are both in the variable table: one block, one free
+    assert len(stub_lib.freed) == 2 and not stub_lib.live
+    rt.free()  # idempotent
+    assert len(stub_lib.freed) == 2
+
+
+def test_view_casts_a_scalar_to_an_array(stub_lib):
+    """realize-node :View on a buffer holding a number with nrank > 0 opens storage and fills it with the number,
+    sized by the non-broadcast axes (runtime.lisp:274-283)."""
+    from caten_amd.runtime import GraphRuntime
+    from caten_amd.buffer import HipBuffer, make_buffer
+
+    class RT(GraphRuntime):
+        buffer_type = HipBuffer
+
+    scalar = make_buffer([], [], "float32", value=2.5, device=HipBuffer)
+    rt = RT([_view_node(2, [3, 4], [0, 1], broadcast=[True, False])], ["v"], {"base": scalar})
+    v = rt.forward()
+    assert v.nrank == 2 and isinstance(v.value, int) and v.owns_storage
+    assert np.frombuffer(stub_lib.uploads[v.value], np.float32).tolist() == [2.5] * 4
+    assert scalar.value == 2.5
+    rt.free()
+    assert not stub_lib.live
+
+
 def test_remap_key():
     from caten_amd.llm import remap_key
     assert remap_key("blk.3.attn_qkv.weight") == "h.3.attn.c_attn.weight"
@@ -109,6 +197,77 @@ def test_renderer_emits_and_hiprtc_compiles_for_gfx950():
     assert "ct_max(acc, 0.0f)" in src
     r.compile_kernel([item])
     assert r.code_object[:4] == b"\x7fELF"
+
+
+def test_programs_recognise_the_shapes_hand_written_kernels_cover():
+    """cthip_program_create: the matmul nest (test-scheduler.lisp:126-135) with its epilogues, Linear's transposed
+    read, the one-hot Embedding (nn/embedding.lisp:13-25), ArgMaxNode (high-level-ops.lisp:314-325) and softmax rows
+    get a route next to their rendered source; anything else is rendered only."""
+    from caten_amd import HipRenderer, blueprints as bp
+    r = HipRenderer()
+    cases = [(bp.matmul(), "matmul"), (bp.matmul(relu=True), "matmul"), (bp.matmul(bias=True, relu=True, transposed_b=True), "matmul"),
+             (_matmul_item(), "matmul"), (bp.embedding_onehot(), "embedding"), (bp.argmax_rows(), "argmax"),
+             (bp.softmax_rows(), "softmax"), (bp.softmax_rows(rows=8, n=40), "softmax")]
+    for item, want in cases:
+        src = r.render_kernel(item)
+        assert item["route"] == want, (item["name"], item["route"])
+        assert 'extern "C" __global__' in src  # the rendered kernel is always there to fall back on
+    # a GELU epilogue is not one of the epilogues the GEMM applies: rendered
+    gelu = bp.matmul()
+    gelu["blueprint"][-3]["expr"] = {"op": "MUL", "args": ["acc", {"op": "RECIP", "args": [{"op": "ADD", "args": [1.0, {"op": "EXP2", "args": ["acc"]}]}]}]}
+    r.render_kernel(gelu)
+    assert gelu["route"] == "rendered"
+    # the reduction multiplies by something that is not an array element: rendered
+    odd = bp.matmul()
+    odd["blueprint"][-5]["expr"]["args"][1]["args"][1] = "m"
+    r.render_kernel(odd)
+    assert odd["route"] == "rendered"
+
+
+def test_row_with_a_running_sum_stays_in_one_thread():
+    """s += x[i]; y[i] = s inside one loop is a scan, not a reduction: splitting the loop over the lanes of a
+    wavefront would store every lane's partial, so such a row keeps one thread (no lane-strided loop)."""
+    from caten_amd import HipRenderer, blueprints as bp
+    A = lambda id_, idx: {"op": "AREF", "id": id_, "index": idx}  # noqa: E731
+    add = lambda *a: {"op": "ADD", "args": list(a)}  # noqa: E731
+    mul = lambda *a: {"op": "MUL", "args": list(a)}  # noqa: E731
+    idx = add(mul("n", "_gid0"), "_gid1")
+    for order in (0, 1):
+        red = {"type": "EXPR", "writes": [A("s", None)], "expr": add("s", A("val_x", idx)), "dtype": "float32", "reduction": True}
+        store = {"type": "EXPR", "writes": [A("val_y", idx)], "expr": "s", "dtype": "float32"}
+        item = {"name": "running_sum", "blueprint": [
+            bp._glob("val_y", "output", 2), bp._glob("rows", "shape", 0, "int64"), bp._glob("n", "shape", 0, "int64"),
+            bp._glob("val_x", "input", 2),
+            {"type": "FOR", "idx": "_gid0", "upfrom": 0, "below": bp._lt("_gid0", "rows"), "by": 1},
+            {"type": "EXPR", "writes": [A("s", None)], "expr": 0.0, "declare_type": True, "dtype": "float32"},
+            {"type": "FOR", "idx": "_gid1", "upfrom": 0, "below": bp._lt("_gid1", "n"), "by": 1},
+            *([red, store] if order == 0 else [store, red]),
+            {"type": "ENDFOR", "idx": "_gid1"},
+            {"type": "ENDFOR", "idx": "_gid0"},
+        ]}
+        src = HipRenderer().render_kernel(item)
+        assert "+=64" not in src and "ct_wave_" not in src and "_lane" not in src
+    # the plain reduction next to it does get a wavefront per row
+    src = HipRenderer().render_kernel(bp.softmax_rows())
+    assert "+=64" in src and "ct_wave_max_f" in src and "ct_wave_add_f" in src
+
+
+def test_program_text_errors_are_reported():
+    from caten_amd import _lib, HipError
+    lib = _lib.load()
+    p = ctypes.c_void_p()
+    for text, what in [(b"(item k (for i 0", b"unbalanced"), (b"(item k (frobnicate 1))", b"unknown blueprint node"),
+                       (b"(item k (for i 0 (< i 4) 1))", b"unbalanced for"), (b"(kernel k)", b"expected (item"),
+                       (b"(item k (define-global a float33 t input 1))", b"unknown dtype")]:
+        assert lib.cthip_program_create(ctypes.byref(p), text) != 0
+        assert what in lib.cthip_last_error(), lib.cthip_last_error()
+    # an instruction the renderer has no spelling for
+    assert lib.cthip_program_create(ctypes.byref(p), b"(item k (expr (y) (frob x) :dtype float32))") == _lib.E_UNSUPPORTED
+    assert b"no %render-node method for :frob" in lib.cthip_last_error()
+    # Lisp float syntax and keywords are read: 1.0d0, 1.0f0, :dtype, upper case
+    assert lib.cthip_program_create(ctypes.byref(p), b"(ITEM K (EXPR ((AREF Y 0)) (ADD 1.5d0 2.0f0 1.0e-5) :DTYPE :FLOAT32))") == 0
+    assert b"y[0] = (1.5f+2.0f+0.00001f);" in lib.cthip_program_source(p)
+    lib.cthip_program_destroy(p)
 
 
 def test_renderer_reports_compile_errors():

@@ -1,8 +1,11 @@
-"""Prefill timing on one MI355X (`python -m caten_amd.bench_prefill`): a 512-token prompt through the
+#!/usr/bin/env python3
+"""Prefill timing on one MI355X (`python bench_prefill.py`): a 512-token prompt through the
 GPT-2-small shaped Q8_0 model as one batch (the prefill leg of the GPT-2 Q8_0 benchmark configuration; `--model llama-1.1b
 --kind q4_0 --tokens 128` is the Llama-1.1B Q4_0 configuration's): MFMA GEMMs over the
 rows with the weights dequantised while staged.  Reports the wall time of `forward` (synchronous) and
-the linear-layer FLOP rate against the MFMA peak of the operand type."""
+the linear-layer FLOP rate against the MFMA peak of the operand type.  The logits of every operand format are checked
+against the fp32-operand run (fp32-grade formats: rtol 1e-3 / atol 1e-4 per logit; bf16: 5e-2 of the vector's norm) and the greedy token must agree
+before a figure is printed."""
 from __future__ import annotations
 
 import json
@@ -10,7 +13,12 @@ import time
 
 import numpy as np
 
-from . import _lib, llm, synth
+import os
+import sys
+
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+
+from caten_amd import _lib, llm, synth  # noqa: E402
 
 
 def main(model="gpt2", kind="q8_0", s=512):
@@ -28,9 +36,22 @@ def main(model="gpt2", kind="q8_0", s=512):
         lin_flop = 2.0 * s * L * (3 * D * D + D * D + 2 * D * F) + 2.0 * V * D  # lm_head on the last row only
     att_flop = 2.0 * 2.0 * L * cfg["n_heads"] * (D // cfg["n_heads"]) * s * (s + 1) / 2
     names = {0: "fp32", 3: "3-term split bf16 (6 MFMAs per product)", 2: "2-term split bf16 (3 MFMAs per product)", 1: "bf16"}
+    ref_tok = ref_logits = None
     for mode, peak in ((0, 157.3), (3, 2500.0), (2, 2500.0), (1, 2500.0)):
         _lib.check(lib.cthip_set_option(b"gemm_precision", mode))
-        m.forward(prompt, s, 0)
+        tok, logits = m.forward(prompt, s, 0, return_logits=True)
+        if ref_logits is None:
+            ref_tok, ref_logits = tok, logits.astype(np.float64)
+        else:
+            if mode == 1:
+                # operands rounded to bf16 through every layer: checked as a whole (relative error of the logits vector)
+                rel = np.linalg.norm(logits - ref_logits) / np.linalg.norm(ref_logits)
+                bad = np.array([not rel < 5e-2])
+            else:
+                bad = np.abs(logits - ref_logits) > 1e-4 + 1e-3 * np.abs(ref_logits)
+            if bad.any() or (tok != ref_tok and mode != 1):
+                raise SystemExit(f"bench_prefill: {names[mode]}: {int(bad.sum())} logits differ from the fp32-operand run "
+                                 f"(token {tok} vs {ref_tok}); no figure is reported for a wrong result")
         ts = []
         for _ in range(5):
             t0 = time.perf_counter()

@@ -3,6 +3,7 @@
 // variants x 8 kernels compile in parallel instead of in one three-minute unit.
 #pragma once
 #include "common.h"
+#include "gemv_plan.h"
 
 namespace cthip {
 
@@ -779,15 +780,11 @@ struct GemvVariant {
   gemv_fn fn_direct[2];  // looping, no epilogue operands, a LayerNorm applied to the staged input
   gemv_fn fn_small[2]; // one tile per wavefront: latency-bound launches
 };
-// looping launches keep about 12 sixteen-byte loads per lane in flight; the widest 4-bit variants (96+ input floats per
-// lane in registers) keep two tiles, which leaves room for a second wavefront per SIMD (TinyLlama down projection:
-// 0.720 -> 0.707 ms per decode step)
-#define PD_OF_T(T, KC) (KC >= 12 ? 1 : (KC >= 6 || ((T) == CTHIP_Q4_0 && KC >= 3)) ? 2 : 4)
 #define V(T, G, KC)                                                                           \
   {T, G, KC, {k_gemv<T, G, KC, PD_OF_T(T, KC), false>, k_gemv<T, G, KC, PD_OF_T(T, KC), true>},         \
    {k_gemv<T, G, KC, PD_OF_T(T, KC), false, PD_OF_T(T, KC) != 1>, k_gemv<T, G, KC, PD_OF_T(T, KC), true, PD_OF_T(T, KC) != 1>}, \
    {k_gemv<T, G, KC, PD_OF_T(T, KC), false, false, PD_OF_T(T, KC) != 1>, k_gemv<T, G, KC, PD_OF_T(T, KC), true, false, PD_OF_T(T, KC) != 1>}, \
-   {k_gemv<T, G, KC, 1, false>, k_gemv<T, G, KC, 1, true>}}
+   {k_gemv<T, G, KC, 1, false>, k_gemv<T, G, KC, 1, true>}},
 // defined in gemv_q8.hip, gemv_q4.hip, gemv_f32.hip, gemv_f16.hip
 extern const GemvVariant kGemvQ8[], kGemvQ4[], kGemvF32[], kGemvF16[];
 extern const int kGemvQ8Count, kGemvQ4Count, kGemvF32Count, kGemvF16Count;

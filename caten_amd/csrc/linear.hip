@@ -27,6 +27,7 @@
 
 #include "common.h"
 #include "gemv_kernels.h"
+#include "gemv_plan.h"
 
 namespace cthip {
 
@@ -311,31 +312,17 @@ static const std::vector<GemvVariant> &all_variants() {
   return all;
 }
 
-static int xpc_of(int type) {
-  switch (type) {
-    case CTHIP_Q8_0: return 16;
-    case CTHIP_Q4_0: return 32;
-    case CTHIP_F16: return 8;
-    default: return 4;
-  }
-}
+static int xpc_of(int type) { return gemv_xpc(type); }
 
-static const GemvVariant *pick_variant(int type, int cols) {
-  const int xpc = xpc_of(type);
-  if (cols % xpc) return nullptr;
-  const int nchunks = cols / xpc;
-  const GemvVariant *best = nullptr;
-  int best_waste = 1 << 30;
-  for (const GemvVariant &v : all_variants()) {
-    if (v.type != type || v.G * v.KC < nchunks) continue;
-    int waste = v.G * v.KC - nchunks;
-    if (waste < best_waste || (waste == best_waste && best && v.G < best->G)) {
-      best = &v;
-      best_waste = waste;
-    }
-  }
-  return best;
+// the kernels of the variant the plan names (the tables of the per-type translation units are in gemv_shapes() order)
+static const GemvVariant *variant_of(int shape) {
+  if (shape < 0) return nullptr;
+  const std::vector<GemvVariant> &all = all_variants();
+  const GemvShape &sh = gemv_shapes()[shape];
+  const GemvVariant &v = all[(size_t)shape];
+  return (v.type == sh.type && v.G == sh.G && v.KC == sh.KC) ? &v : nullptr;
 }
+static const GemvVariant *pick_variant(int type, int cols) { return variant_of(gemv_pick_shape(type, cols)); }
 
 int launch_prologue(float *out, const float *x, int cols, int pro, const float *g, const float *b, float eps,
                     int64_t x_stride, int m) {
@@ -379,89 +366,49 @@ int launch_gemv(const WMat *w, GemvArgs a, int m) {
   if (a.pair_swiglu && (!v || v->G > 32 || (a.rows & 1) || a.am_val || a.residual || a.split1 != a.rows))
     return fail(CTHIP_E_UNSUPPORTED, "gemv: the paired SwiGLU epilogue needs two rows per wavefront and plain outputs");
   if (v) {
-    const int rpw = 64 / v->G;
-    const int nrq = (a.rows + rpw - 1) / rpw;
-    dim3 grid, block;
-    const bool folded = (a.pro == CTHIP_PRO_RMSNORM) || (a.pro == CTHIP_PRO_LAYERNORM && a.fold_s != nullptr);
-    const bool quantised = w->type == CTHIP_Q8_0 || w->type == CTHIP_Q4_0;
-    // The input vector goes through LDS once per workgroup when it must be normalised or gated first,
-    // or when it is large next to a weight tile (a 4-bit tile multiplies 8 input bytes per weight byte):
-    // then four wavefronts share one copy and every wavefront takes several tiles.  Quantised launches with a
-    // folded norm stage at every size: a lane's slice is 48-64 floats, and gamma * x plus the statistics once
-    // per workgroup beat once per wavefront (GPT-2 decode: Q8_0 284.6 -> 280.3 us / step, Q4_0 339 -> 308;
-    // fp32 / fp16 weights, 12-24 floats per lane, measured the other way round: 354 -> 369, 328 -> 347).
-    const bool stage = (a.pro != CTHIP_PRO_NONE && !folded) || (w->type == CTHIP_Q4_0 && a.cols >= 1024) ||
-                       (folded && (a.cols >= 2048 || quantised));
-    const size_t lds = stage ? sizeof(float) * (size_t)a.cols : 0;
-    if (lds > 64 * 1024) return fail(CTHIP_E_UNSUPPORTED, "gemv: %d input features exceed the LDS staging buffer", a.cols);
-    a.stage_x = stage ? 1 : 0;
-    bool small, direct = false;
-    if (!stage && nrq <= 2048) {
-      // small matrices are pure latency: one tile per wavefront, one wavefront per workgroup, spread
-      // over as many compute units as there are tiles
-      small = true;
-      block = dim3(64);
-      grid = dim3(nrq, m);
-    } else if (stage && nrq <= s.compute_units * 3) {
-      // one tile per wavefront, as many wavefronts per workgroup (at most three) as leave about one workgroup
-      // per compute unit: fewer workgroups repeat the staging less, but idle units stream nothing
-      // (GPT-2 c_attn / c_fc, 576 / 768 tiles: 3 per workgroup 279.9 us / step, 4: 283.1, 2: 286.8, 1: 289.1).
-      // Beyond three tiles per compute unit the looping launch below is ahead (TinyLlama wo, 1024 tiles:
-      // 0.780 -> 0.772 ms / step; with the limit at two, GPT-2 loses 1 %)
-      small = true;
-      int wpb = (nrq + s.compute_units - 1) / s.compute_units;
-      wpb = wpb < 1 ? 1 : wpb > 3 ? 3 : wpb;
-      block = dim3(64 * wpb);
-      grid = dim3((nrq + wpb - 1) / wpb, m);
-    } else {
-      // larger matrices: at least one wavefront per SIMD, more (up to what the register budget keeps
-      // resident) once every wavefront has four tiles
-      small = false;
-      static std::vector<int> occ_cache(all_variants().size(), 0);
-      const int vi = (int)(v - all_variants().data());
+    const int vi = (int)(v - all_variants().data());
+    static std::vector<int> occ_cache(all_variants().size(), 0);
+    GemvPlanIn in = {};
+    in.type = w->type;
+    in.rows = a.rows;
+    in.cols = a.cols;
+    in.m = m;
+    in.pro = a.pro;
+    in.fold = a.fold_s != nullptr;
+    in.bias = a.bias != nullptr;
+    in.bias0 = a.bias0 != nullptr;
+    in.residual = a.residual != nullptr;
+    in.argmax = a.am_val != nullptr;
+    in.compute_units = s.compute_units;
+    in.occupancy = 1;
+    GemvPlan p = gemv_plan(in);
+    if (!p.error && p.kernel != GEMV_K_SMALL) {  // a looping launch: how many of its workgroups a compute unit holds
       if (occ_cache[vi] == 0) {
         int nb = 0;
         CTHIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, v->fn[0], 256, 16 * 1024));
         occ_cache[vi] = nb > 0 ? nb : 1;
       }
-      block = dim3(256);
-      const int base = s.compute_units * 4;
-      // unstaged: a wavefront per tile up to three resident wavefronts per SIMD (fp32 GPT-2 decode with every large
-      // launch at 1024 / 2048 / 3072 / 4096 wavefronts: 369 / 343 / 334 / 343 us per step)
-      int wanted = stage ? (nrq + 3) / 4 : nrq;
-      if (wanted < base) wanted = base;
-      const int cap = base * (stage || occ_cache[vi] < 3 ? occ_cache[vi] : 3);
-      if (wanted > cap) wanted = cap;
-      // staged launches pay the input staging once per workgroup: whole workgroups per compute unit, two
-      // when there is work for more than one (measured best; a third does not fit beside the first two)
-      if (stage && wanted > base && occ_cache[vi] >= 2) wanted = 2 * base;
-      const int iters = (nrq + wanted - 1) / wanted;
-      // every resident wavefront slot is used even if some wavefronts then loop once more than others: with equal
-      // iteration counts (12 565 tiles of the GPT-2 lm_head on 1 795 wavefronts of seven) a quarter of the compute units
-      // would run one workgroup where the others run two (10.3 -> 10.0 us)
-      const int waves = wanted < nrq ? wanted : nrq;
-      grid = dim3((waves + 3) / 4, m);
-      // the ring requests all its slots unconditionally: a wavefront with a single tile takes the kernel without one
-      if (iters == 1) small = true;
-      // A looping launch normalises the staged vector itself rather than carrying the fold terms: two more
-      // operands per row in the weight ring hold the stream up more than the second barrier of the staging costs
-      // (GPT-2 lm_head: 11.0 us folded, 10.0 us with neither)
-      if (!small && stage && a.pro == CTHIP_PRO_LAYERNORM && a.fold_s && !a.bias0 && !a.residual && a.cols <= 4096) {
-        a.fold_s = nullptr;
-        a.bias = nullptr;
-      }
-      direct = !small && stage && a.pro == CTHIP_PRO_LAYERNORM && !a.fold_s && !a.bias && !a.residual && a.cols <= 4096;
+      in.occupancy = occ_cache[vi];
+      p = gemv_plan(in);
     }
-    const int nwaves = (int)(grid.x * (block.x / 64));
-    if (a.am_val && nwaves > kGemvMaxWaves)
-      return fail(CTHIP_E_UNSUPPORTED, "gemv: %d wavefronts exceed the argmax scratch", nwaves);
+    if (p.error) return fail(CTHIP_E_UNSUPPORTED, "gemv: (%d, %d): %s", a.rows, a.cols, p.error);
+    a.stage_x = p.stage ? 1 : 0;
+    if (p.unfold) {
+      a.fold_s = nullptr;
+      a.bias = nullptr;
+    }
+    if (a.am_val && p.nwaves > kGemvMaxWaves)
+      return fail(CTHIP_E_UNSUPPORTED, "gemv: %d wavefronts exceed the argmax scratch", p.nwaves);
     const int nt = s.gemv_stream < 0 ? (w->stream ? 1 : 0) : s.gemv_stream;
-    const bool epi = a.bias || a.residual || a.fold_s;
-    hipLaunchKernelGGL(small ? v->fn_small[nt] : epi ? v->fn_epi[nt] : direct ? v->fn_direct[nt] : v->fn[nt], grid, block, lds,
-                       s.stream, a);
+    // the looping kernel with per-row operands in its ring dereferences one of them unconditionally
+    if (p.kernel == GEMV_K_LOOP_EPI && !a.bias && !a.residual && !a.fold_s)
+      return fail(CTHIP_E_STATE, "gemv: a launch with epilogue operands in its ring has none");
+    const gemv_fn fn = p.kernel == GEMV_K_SMALL ? v->fn_small[nt] : p.kernel == GEMV_K_LOOP_EPI ? v->fn_epi[nt]
+                     : p.kernel == GEMV_K_LOOP_DIRECT ? v->fn_direct[nt] : v->fn[nt];
+    hipLaunchKernelGGL(fn, dim3(p.grid_x, p.grid_y), dim3(p.block), p.lds, s.stream, a);
     CTHIP_LAUNCH_CHECK();
     if (a.am_val) {
-      hipLaunchKernelGGL(k_argmax_finish, dim3(1), dim3(256), 0, s.stream, a, nwaves);
+      hipLaunchKernelGGL(k_argmax_finish, dim3(1), dim3(256), 0, s.stream, a, p.nwaves);
       CTHIP_LAUNCH_CHECK();
     }
     return 0;

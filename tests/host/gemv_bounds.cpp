@@ -1,0 +1,253 @@
+// CPU bounds harness for the single-row Linear launches.  For every weight type x matrix shape x prologue /
+// epilogue combination x occupancy the launcher can see, it takes the launch plan the library itself computes
+// (caten_amd/csrc/gemv_plan.h, the code launch_gemv runs) and walks every workgroup, wavefront and lane of that
+// plan through a transcription of the kernels' index arithmetic (k_gemv / gemv_ring / coop_prologue / coop_fold of
+// caten_amd/csrc/gemv_kernels.h), asserting for each access that the pointer it dereferences exists and that the
+// bytes lie inside the operand: quant plane, scale plane, input vector(s), gamma / beta, bias / residual / fold
+// terms, output, argmax partials, the LDS staging buffer and the `red` array.  Prints the number of launches and
+// accesses checked and every violation; exit status 1 if there is any.
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <string>
+
+#include "../../caten_amd/csrc/gemv_plan.h"
+
+using namespace cthip;
+
+static long long g_checked = 0, g_violations = 0, g_launches = 0;
+static std::string g_case;
+
+struct Region {
+  const char *name;
+  bool present;
+  long long bytes;
+};
+static void touch(const Region &r, long long off, long long n, const char *what) {
+  g_checked++;
+  if (!r.present) {
+    if (g_violations++ < 40) printf("VIOLATION %s: %s dereferences %s, which is null\n", g_case.c_str(), what, r.name);
+    return;
+  }
+  if (off < 0 || off + n > r.bytes || (off % n) != 0) {
+    if (g_violations++ < 40) printf("VIOLATION %s: %s touches %s[%lld..%lld) of %lld bytes\n", g_case.c_str(), what, r.name, off, off + n, r.bytes);
+  }
+}
+
+struct Case {
+  int type, rows, cols, m, pro;
+  bool fold, bias, bias0, residual, argmax, pair;
+  int cus, occ;
+};
+
+static void walk(const Case &c) {
+  GemvPlanIn in = {};
+  in.type = c.type; in.rows = c.rows; in.cols = c.cols; in.m = c.m; in.pro = c.pro; in.fold = c.fold; in.bias = c.bias;
+  in.bias0 = c.bias0; in.residual = c.residual; in.argmax = c.argmax; in.compute_units = c.cus; in.occupancy = c.occ;
+  GemvPlan p = gemv_plan(in);
+  char buf[256];
+  snprintf(buf, sizeof(buf), "type %d (%d,%d) m %d pro %d fold %d bias %d bias0 %d resid %d argmax %d pair %d cus %d occ %d", c.type, c.rows, c.cols,
+           c.m, c.pro, c.fold, c.bias, c.bias0, c.residual, c.argmax, c.pair, c.cus, c.occ);
+  g_case = buf;
+  if (p.shape < 0 || p.error) return;  // generic fallback / refused: not these kernels
+  g_launches++;
+  const GemvShape &v = gemv_shapes()[p.shape];
+  const int G = v.G, KC = v.KC, XPC = gemv_xpc(c.type), RPW = 64 / G;
+  const int PD = p.kernel == GEMV_K_SMALL ? 1 : PD_OF_T(c.type, KC);
+  const bool QUANT = c.type == CTHIP_Q8_0 || c.type == CTHIP_Q4_0;
+  bool fold = c.fold, bias = c.bias;
+  if (p.unfold) fold = false, bias = false;
+  const bool swiglu = c.pro == CTHIP_PRO_SWIGLU, layernorm = c.pro == CTHIP_PRO_LAYERNORM;
+  const bool folded = c.pro == CTHIP_PRO_RMSNORM || (layernorm && fold);
+  const bool coop = p.stage;
+  const int in_cols = swiglu ? 2 * c.cols : c.cols;
+  const long long x_stride = in_cols, out_rows = c.pair ? c.rows / 2 : c.rows, y_stride = out_rows;
+  const long long row_bytes = c.type == CTHIP_Q8_0 ? c.cols : c.type == CTHIP_Q4_0 ? c.cols / 2 : c.type == CTHIP_F16 ? 2ll * c.cols : 4ll * c.cols;
+  Region Q = {"quant plane", true, row_bytes * c.rows}, D = {"scale plane", QUANT, 2ll * (c.cols / 32) * c.rows};
+  Region X = {"x", true, 4 * x_stride * c.m}, NG = {"norm_g", c.pro == CTHIP_PRO_LAYERNORM || c.pro == CTHIP_PRO_RMSNORM, 4ll * c.cols};
+  Region NB = {"norm_b", layernorm, 4ll * c.cols}, B = {"bias", bias, 4ll * c.rows}, R = {"residual", c.residual, 4 * y_stride * c.m};
+  Region FS = {"fold_s", fold, 4ll * c.rows}, Y = {"y", true, 4 * y_stride * c.m}, AM = {"argmax partials", c.argmax, 4ll * 16384};
+  Region LDS = {"LDS staging buffer", p.lds > 0, (long long)p.lds}, RED = {"red", true, 4 * 24};
+  const int nchunks = c.cols / XPC, nrq = (c.rows + RPW - 1) / RPW, n4 = c.cols >> 2;
+  const int nthr = (int)p.block, wpb = nthr >> 6, total_waves = (int)p.grid_x * wpb;
+  const int scales_per_row = c.cols >> 5;
+  const bool ring = PD > 1;
+  if (ring && nthr != 256) { g_violations++; printf("VIOLATION %s: the looping kernel is compiled for 256 threads, launched with %d\n", g_case.c_str(), nthr); }
+  const bool epi_kernel = p.kernel == GEMV_K_LOOP_EPI, direct_kernel = p.kernel == GEMV_K_LOOP_DIRECT;
+  for (int m = 0; m < c.m; m++)
+    for (unsigned bx = 0; bx < p.grid_x; bx++)
+      for (int tid = 0; tid < nthr; tid++) {
+        const int lane = tid & 63, g = lane / G, l = lane % G, wave = (int)bx * wpb + (tid >> 6);
+        const long long xoff = 4 * x_stride * m;
+        auto tile = [&](int rq, const char *what) {
+          int row = rq * RPW + g;
+          row = row < c.rows ? row : c.rows - 1;
+          for (int j = 0; j < KC; j++) {
+            const int cc = l + G * j;
+            if (cc >= nchunks) continue;  // reads the zero block
+            touch(Q, ((long long)row * nchunks + cc) * 16, 16, what);
+            if (QUANT) touch(D, 2 * ((long long)row * scales_per_row + (c.type == CTHIP_Q8_0 ? (cc >> 1) : cc)), 2, what);
+          }
+          return row;
+        };
+        auto epi_operands = [&](int row, bool in_ring) {
+          if (in_ring) {  // gemv_ring: one request by the first three lanes; `any` must exist
+            if (!bias && !c.residual && !fold) { g_violations++; printf("VIOLATION %s: the ring's epilogue request has no operand\n", g_case.c_str()); return; }
+            if (bias) touch(B, 4ll * row, 4, "epilogue request");
+            if (c.residual) touch(R, 4 * (y_stride * m + row), 4, "epilogue request");
+            if (fold) touch(FS, 4ll * row, 4, "epilogue request");
+          } else {
+            if (bias) touch(B, 4ll * row, 4, "bias");
+            if (c.residual) touch(R, 4 * (y_stride * m + row), 4, "residual");
+            if (fold) touch(FS, 4ll * row, 4, "fold term");
+          }
+        };
+        auto store = [&](int rq) {
+          const int row = rq * RPW + g;
+          if (row >= c.rows) return;
+          if (c.pair) { if (l == 0 && (g & 1) == 0) touch(Y, 4 * (y_stride * m + (row >> 1)), 4, "paired store"); }
+          else if (l == 0) touch(Y, 4 * (y_stride * m + row), 4, "store");
+        };
+        auto x_slice = [&](bool from_lds) {
+          for (int j = 0; j < KC; j++) {
+            const int cc = l + G * j;
+            if (cc >= nchunks) continue;
+            for (int t = 0; t < XPC / 4; t++) {
+              if (from_lds) touch(LDS, 4ll * (cc * XPC + 4 * t), 16, "staged slice");
+              else touch(X, xoff + 4ll * (cc * XPC + 4 * t), 16, "input slice");
+            }
+          }
+        };
+        auto gamma_slice = [&]() {
+          for (int j = 0; j < KC; j++) {
+            const int cc = l + G * j;
+            if (cc >= nchunks) continue;
+            for (int t = 0; t < XPC / 4; t++) touch(NG, 4ll * (cc * XPC + 4 * t), 16, "gamma slice");
+          }
+        };
+        auto coop_prologue = [&](bool normalise) {
+          if (!swiglu && !normalise) { for (int i = tid; i < n4; i += nthr) touch(X, xoff + 16ll * i, 16, "copy"), touch(LDS, 16ll * i, 16, "copy"); return; }
+          if (swiglu) { for (int i = tid; i < n4; i += nthr) touch(X, xoff + 16ll * i, 16, "gate"), touch(X, xoff + 4ll * c.cols + 16ll * i, 16, "up"), touch(LDS, 16ll * i, 16, "swiglu"); return; }
+          for (int i = tid; i < n4; i += nthr) {
+            touch(X, xoff + 16ll * i, 16, "norm input");
+            touch(NG, 16ll * i, 16, "norm gamma");
+            if (layernorm) touch(NB, 16ll * i, 16, "norm beta");
+            touch(LDS, 16ll * i, 16, "normalised");
+          }
+          touch(RED, 4 * (tid >> 6), 4, "red");
+          if (wpb > 8) { g_violations++; printf("VIOLATION %s: %d wavefronts overflow red\n", g_case.c_str(), wpb); }
+        };
+        if (!ring) {
+          // ---- k_gemv, one tile in flight ----
+          const int rq0 = wave < nrq ? wave : nrq - 1;
+          epi_operands(tile(rq0, "first tile"), false);
+          if (folded && layernorm) touch(X, xoff, 4, "pivot");
+          if (coop) {
+            if (folded) {
+              for (int i = tid; i < n4; i += nthr) touch(X, xoff + 16ll * i, 16, "fold input"), touch(NG, 16ll * i, 16, "fold gamma"), touch(LDS, 16ll * i, 16, "fold stage");
+              touch(RED, 4 * (tid >> 6), 4, "red"), touch(RED, 4 * (8 + (tid >> 6)), 4, "red");
+            } else coop_prologue(c.pro != CTHIP_PRO_NONE);
+          }
+          x_slice(coop);
+          if (folded && !coop) gamma_slice();
+          for (int base = wave; base < nrq; base += total_waves) {
+            store(base);
+            if (base + total_waves < nrq) epi_operands(tile(base + total_waves, "next tile"), false);
+          }
+        } else {
+          // ---- gemv_ring ----
+          const bool direct = direct_kernel && coop && layernorm && !fold && n4 <= 4 * 256;
+          const bool early = coop && (folded || swiglu || c.pro == CTHIP_PRO_NONE || direct);
+          if (early) {
+            for (int k = 0; k < 4; k++) {
+              int i = tid + k * 256;
+              i = i < n4 ? i : n4 - 1;
+              touch(X, xoff + 16ll * i, 16, "early input");
+              if (swiglu) touch(X, xoff + 4ll * c.cols + 16ll * i, 16, "early up");
+              else if ((layernorm || folded) && NG.present) touch(NG, 16ll * i, 16, "early gamma");
+              if (direct_kernel && direct) touch(NB, 16ll * i, 16, "early beta");
+            }
+          } else if (!coop) {
+            x_slice(false);
+            if (!QUANT && folded) gamma_slice();
+          }
+          const int own = wave < nrq ? wave : nrq - 1;
+          auto request = [&](int rq) { const int row = tile(rq, "ring tile"); if (epi_kernel) epi_operands(row, true); };
+          request(wave < nrq ? wave : own);
+          if (coop && !early) coop_prologue(true);
+          if (early) {
+            for (int i = tid; i < n4; i += 256) {
+              if (i >= tid + 4 * 256) { touch(X, xoff + 16ll * i, 16, "late input"); if (swiglu) touch(X, xoff + 4ll * c.cols + 16ll * i, 16, "late up"); else if (NG.present) touch(NG, 16ll * i, 16, "late gamma"); }
+              touch(LDS, 16ll * i, 16, "stage");
+            }
+            touch(RED, 4 * (tid >> 6), 4, "red"), touch(RED, 4 * (8 + (tid >> 6)), 4, "red"), touch(RED, 4 * (16 + (tid >> 6)), 4, "red");
+          }
+          if (coop) x_slice(true);
+          for (int pp = 1; pp < PD; pp++) { const int rq = wave + pp * total_waves; request(rq < nrq ? rq : own); }
+          if (folded && !coop && QUANT) gamma_slice();
+          const int stride = PD * total_waves;
+          int base = wave;
+          for (; base + stride < nrq; base += stride)
+            for (int pp = 0; pp < PD; pp++) { const int rq = base + pp * total_waves; store(rq); const int nxt = rq + stride; request(nxt < nrq ? nxt : rq); }
+          for (int pp = 0; pp < PD; pp++) { const int rq = base + pp * total_waves; if (rq < nrq) store(rq); }
+        }
+        if (c.argmax && lane == 0) touch(AM, 4ll * wave, 4, "argmax partial");
+      }
+}
+
+int main(int argc, char **argv) {
+  // default: a few seconds (every shape, the flag combinations thinned out on the large ones); "full": everything
+  const bool full = argc > 1 && !strcmp(argv[1], "full");
+  const int types[] = {CTHIP_Q8_0, CTHIP_Q4_0, CTHIP_F32, CTHIP_F16};
+  // widths: each variant's exact width, one chunk less, the smallest, and the model widths
+  const int rowsv[] = {1, 2, 3, 5, 17, 64, 767, 768, 2304, 3072, 5003, 32000, 50257};
+  for (int type : types) {
+    const int xpc = gemv_xpc(type);
+    std::vector<int> colsv = {xpc, 2 * xpc, 768, 1024, 1280, 1600, 2048, 3072, 4096, 5632, 8192};
+    for (const GemvShape &s : gemv_shapes())
+      if (s.type == type) colsv.push_back(s.G * s.KC * xpc), colsv.push_back((s.G * s.KC - 1) * xpc);
+    for (int cols : colsv) {
+      if (cols <= 0 || cols % xpc || ((type == CTHIP_Q8_0 || type == CTHIP_Q4_0) && cols % 32)) continue;
+      for (int rows : rowsv) {
+        if ((long long)rows * cols > 50257ll * 1024) continue;
+        for (int pro = 0; pro <= 3; pro++)
+          for (int flags = 0; flags < 32; flags++) {
+            Case c = {};
+            c.type = type; c.rows = rows; c.cols = cols; c.m = (rows < 100 ? 3 : 1); c.pro = pro;
+            c.fold = (flags & 1) && pro == CTHIP_PRO_LAYERNORM;
+            c.bias = (flags & 2) || c.fold;  // a folded launch always carries W.beta + bias
+            c.bias0 = c.fold && (flags & 4);
+            c.residual = flags & 8;
+            c.argmax = (flags & 16) && c.m == 1;
+            if ((flags & 16) && c.m != 1) continue;
+            if ((flags & 4) && !c.fold) continue;
+            if ((flags & 1) && pro != CTHIP_PRO_LAYERNORM) continue;
+            // very large walks: one occupancy only
+            const long long cost = (long long)rows * cols;
+            const bool big = cost > 8000000;
+            // (flags: 1 fold, 2 bias, 4 the Linear's own bias beside the fold, 8 residual, 16 argmax; 17 = what lm_head launches)
+            if (!full && cost > 20000 && flags != 0 && flags != 2 && flags != 11 && flags != 15 && flags != 17 && flags != 24) continue;
+            if (!full && cost > 1000000 && (pro == 3 || (flags != 0 && flags != 11 && flags != 17))) continue;
+            if (!full && cost > 20000000 && !(pro == 1 && flags == 17) && !(pro == 0 && flags == 0)) continue;
+            for (int occ = 1; occ <= (big ? 2 : 4); occ++) {
+              if (big && (flags & ~25)) continue;
+              if (!full && cost > 20000 && occ != 2) continue;
+              c.cus = 256; c.occ = occ;
+              walk(c);
+            }
+            if (!big && (full || cost <= 20000)) { c.cus = 64; c.occ = 2; walk(c); }
+          }
+        // gate / up pairs: two rows per wavefront, even row count, no residual
+        if (rows % 2 == 0) {
+          Case c = {};
+          c.type = type; c.rows = rows; c.cols = cols; c.m = 1; c.pro = CTHIP_PRO_RMSNORM; c.pair = true; c.cus = 256; c.occ = 2;
+          const int sh = gemv_pick_shape(type, cols);
+          if (sh >= 0 && gemv_shapes()[sh].G <= 32) walk(c);
+        }
+      }
+    }
+  }
+  printf("gemv bounds: %lld launches, %lld accesses checked, %lld violations\n", g_launches, g_checked, g_violations);
+  return g_violations ? 1 : 0;
+}

@@ -95,6 +95,7 @@ PROTOTYPES = {
     "cthip_decoder_missing": (_i, [_vp]),
     "cthip_decoder_forward": (_i, [_vp, _vp, _i, _i, C.POINTER(_i64), _vp]),
     "cthip_decoder_generate": (_i, [_vp, _i, _vp]),
+    "cthip_decoder_generate_until": (_i, [_vp, _i, _i64, _vp, C.POINTER(_i)]),
     "cthip_decoder_position": (_i, [_vp]),
     "cthip_decoder_step_bytes": (_i64, [_vp, _i]),
     "cthip_decoder_peek": (_i, [_vp, C.c_char_p, _vpp, C.POINTER(_i64)]),

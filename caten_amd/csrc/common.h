@@ -113,6 +113,10 @@ struct GemvArgs {
   int *am_pos;
   long long *am_hist;
   int *am_hist_n;
+  // stop condition of a device-resident loop: am_ctrl[0] = a token id that ends the sequence (-1 = none),
+  // am_ctrl[1] = set to 1 by the step that produced it; from then on the steps still queued change nothing
+  // (token, position and history stay as they are).  Null = no stop condition.
+  int *am_ctrl;
   // the block that settles the token also gathers the next step's input, nx_out[d] = nx_wte[token][d] +
   // nx_wpe[position + 1][d] (the Embedding items of the next forward), so that a device-resident loop needs no
   // embedding launch between steps.  nx_out null = off; nx_wpe null = no position table.

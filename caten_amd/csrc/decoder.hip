@@ -82,6 +82,9 @@ struct Decoder {
   int64_t *token64 = nullptr;
   int64_t *history = nullptr;
   int *hist_n = nullptr;
+  int *ctrl = nullptr;        // [0] = token id that ends a sequence (-1 = none), [1] = the sequence has ended
+  int *ctrl_host = nullptr;   // pinned copy of ctrl the host polls between graph launches
+  hipEvent_t ctrl_ev = nullptr;
   // scratch of the argmax fused behind lm_head: one partial per wavefront
   float *am_val = nullptr;
   int *am_idx = nullptr;
@@ -304,6 +307,13 @@ static int finalize(Decoder *d) {
   TRY(dev_alloc(d, (void **)&d->token64, 256));
   TRY(dev_alloc(d, (void **)&d->history, sizeof(int64_t) * (size_t)(c.max_seq + 1)));
   TRY(dev_alloc(d, (void **)&d->hist_n, 256));
+  TRY(dev_alloc(d, (void **)&d->ctrl, 256));
+  {
+    const int none[2] = {-1, 0};
+    TRY(cthip_h2d(d->ctrl, none, sizeof(none)));
+    CTHIP_CHECK(hipHostMalloc((void **)&d->ctrl_host, 256, hipHostMallocDefault));
+    CTHIP_CHECK(hipEventCreateWithFlags(&d->ctrl_ev, hipEventDisableTiming));
+  }
   TRY(dev_alloc(d, (void **)&d->am_val, sizeof(float) * kGemvMaxWaves));
   TRY(dev_alloc(d, (void **)&d->am_idx, sizeof(int) * kGemvMaxWaves));
 
@@ -542,6 +552,7 @@ static int queue_head(Decoder *d) {
   o.am_pos = d->tokpos + 1;
   o.am_hist = (long long *)d->history;
   o.am_hist_n = d->hist_n;
+  o.am_ctrl = d->ctrl;
   // ... and its embedding rows become the next step's input, in the block that settles the token
   o.nx_out = d->x;
   o.nx_wte = d->wte;
@@ -663,6 +674,8 @@ int cthip_decoder_destroy(void *dec) {
   if (d->g_step) (void)hipGraphExecDestroy(d->g_step);
   if (d->g_body) (void)hipGraphExecDestroy(d->g_body);
   if (d->g_multi) (void)hipGraphExecDestroy(d->g_multi);
+  if (d->ctrl_host) (void)hipHostFree(d->ctrl_host);
+  if (d->ctrl_ev) (void)hipEventDestroy(d->ctrl_ev);
   for (auto &kv : d->raw) cthip_free(kv.second.dev);
   for (void *p : d->owned) cthip_free(p);
   for (Layer &L : d->layers) {
@@ -730,6 +743,10 @@ int cthip_decoder_forward(void *dec, const float *tokens, int s, int n, int64_t 
   if (rc) return rc;
   int zero = 0;
   if ((rc = cthip_h2d(d->hist_n, &zero, sizeof(int)))) return rc;
+  {
+    const int none[2] = {-1, 0};
+    if ((rc = cthip_h2d(d->ctrl, none, sizeof(none)))) return rc;
+  }
   // ids arrive as floats (gpt2.lisp:95); one that equals no vocabulary index selects no row
   std::vector<int> ids(s);
   for (int i = 0; i < s; i++) {
@@ -752,26 +769,62 @@ int cthip_decoder_forward(void *dec, const float *tokens, int s, int n, int64_t 
   return 0;
 }
 
-int cthip_decoder_generate(void *dec, int steps, int64_t *tokens_out) {
-  CTHIP_REQUIRE_INIT();
-  CTHIP_ARG(dec != nullptr && steps >= 0 && (steps == 0 || tokens_out != nullptr));
-  Decoder *d = (Decoder *)dec;
+// the loop behind cthip_decoder_generate / cthip_decoder_generate_until
+static int generate_impl(Decoder *d, int steps, int eos, int64_t *tokens_out, int *n_generated) {
   if (!d->primed)
     return fail(CTHIP_E_STATE, "cthip_decoder_generate: run cthip_decoder_forward on a prompt first");
   if (d->position + steps > d->cfg.max_seq)
     return fail(CTHIP_E_BAD_ARG, "cthip_decoder_generate: %d more tokens from position %d overflow max_seq %d", steps,
                 d->position, d->cfg.max_seq);
+  if (n_generated) *n_generated = 0;
   if (steps == 0) return 0;
   int rc, zero = 0;
   if ((rc = cthip_h2d(d->hist_n, &zero, sizeof(int)))) return rc;
+  const int ctrl[2] = {eos, 0};
+  if ((rc = cthip_h2d(d->ctrl, ctrl, sizeof(ctrl)))) return rc;
+  hipStream_t st = state().stream;
+  d->ctrl_host[1] = 0;
+  bool copy_pending = false;
   int i = 0;
+  auto ended = [&]() {
+    // Looks at the last copy of the flag that has ARRIVED; never waits.  A step that runs after the sequence
+    // has ended changes nothing, so launching a batch too many costs time only.
+    if (eos < 0) return false;
+    if (copy_pending && hipEventQuery(d->ctrl_ev) == hipSuccess) copy_pending = false;
+    if (!copy_pending) {
+      if (d->ctrl_host[1]) return true;
+      if (hipMemcpyAsync(d->ctrl_host, d->ctrl, 2 * sizeof(int), hipMemcpyDeviceToHost, st) == hipSuccess &&
+          hipEventRecord(d->ctrl_ev, st) == hipSuccess)
+        copy_pending = true;
+    }
+    return false;
+  };
   if (d->use_graph)
-    for (; i + kStepsPerGraph <= steps; i += kStepsPerGraph) CTHIP_CHECK(hipGraphLaunch(d->g_multi, state().stream));
-  for (; i < steps; i++)
+    for (; i + kStepsPerGraph <= steps && !ended(); i += kStepsPerGraph) CTHIP_CHECK(hipGraphLaunch(d->g_multi, st));
+  for (; i < steps && !ended(); i++)
     if ((rc = run_step(d, true))) return rc;
-  if ((rc = cthip_d2h(tokens_out, d->history, sizeof(int64_t) * (size_t)steps))) return rc;
-  d->position += steps;
+  int n = 0;
+  if ((rc = cthip_d2h(&n, d->hist_n, sizeof(int)))) return rc;  // synchronises
+  if (n < 0 || n > steps) return fail(CTHIP_E_STATE, "cthip_decoder_generate: the device reports %d tokens for %d steps", n, steps);
+  if (n && (rc = cthip_d2h(tokens_out, d->history, sizeof(int64_t) * (size_t)n))) return rc;
+  d->position += n;
+  if (n_generated) *n_generated = n;
   return 0;
+}
+
+int cthip_decoder_generate(void *dec, int steps, int64_t *tokens_out) {
+  CTHIP_REQUIRE_INIT();
+  CTHIP_ARG(dec != nullptr && steps >= 0 && (steps == 0 || tokens_out != nullptr));
+  return generate_impl((Decoder *)dec, steps, -1, tokens_out, nullptr);
+}
+
+int cthip_decoder_generate_until(void *dec, int max_steps, int64_t eos_token, int64_t *tokens_out, int *n_generated) {
+  CTHIP_REQUIRE_INIT();
+  CTHIP_ARG(dec != nullptr && max_steps >= 0 && (max_steps == 0 || tokens_out != nullptr) && n_generated != nullptr);
+  Decoder *d = (Decoder *)dec;
+  if (eos_token < 0 || eos_token >= d->cfg.vocab)
+    return fail(CTHIP_E_BAD_ARG, "cthip_decoder_generate_until: token %lld is not in the vocabulary of %d", (long long)eos_token, d->cfg.vocab);
+  return generate_impl(d, max_steps, (int)eos_token, tokens_out, n_generated);
 }
 
 int cthip_decoder_position(const void *dec) { return dec ? ((const Decoder *)dec)->position : -1; }

@@ -122,10 +122,15 @@ __global__ __launch_bounds__(256) void k_argmax_finish(GemvArgs a, int nparts) {
   __shared__ int si[4];
   __shared__ int next_tok, next_pos;
   // the loop state is requested up front so its latency overlaps the reduction
-  int hist_n = 0, pos = 0;
+  int hist_n = 0, pos = 0, eos = -1, stopped = 0, cur_tok = 0;
   if (threadIdx.x == 0) {
     if (a.am_hist) hist_n = *a.am_hist_n;
     if (a.am_pos) pos = *a.am_pos;
+    if (a.am_ctrl) {
+      eos = a.am_ctrl[0];
+      stopped = a.am_ctrl[1];
+      cur_tok = a.am_tok ? *a.am_tok : 0;
+    }
   }
   float bv = -INFINITY;
   int bi = 0x7fffffff;
@@ -155,15 +160,22 @@ __global__ __launch_bounds__(256) void k_argmax_finish(GemvArgs a, int nparts) {
   if (threadIdx.x == 0) {
     for (int k = 1; k < 4; k++) argmax_merge(bv, bi, sv[k], si[k]);
     if (bi == 0x7fffffff) bi = 0;  // no comparable value (all NaN)
-    *a.am_token64 = bi;
-    if (a.am_tok) *a.am_tok = bi;
-    if (a.am_hist) {
-      a.am_hist[hist_n] = bi;
-      *a.am_hist_n = hist_n + 1;
+    if (stopped) {
+      // the sequence has ended: this step (queued before the host could know) leaves the loop state as it is
+      next_tok = cur_tok;
+      next_pos = pos;
+    } else {
+      *a.am_token64 = bi;
+      if (a.am_tok) *a.am_tok = bi;
+      if (a.am_hist) {
+        a.am_hist[hist_n] = bi;
+        *a.am_hist_n = hist_n + 1;
+      }
+      if (a.am_pos) *a.am_pos = pos + 1;
+      if (a.am_ctrl && bi == eos) a.am_ctrl[1] = 1;
+      next_tok = bi;
+      next_pos = pos + 1;
     }
-    if (a.am_pos) *a.am_pos = pos + 1;
-    next_tok = bi;
-    next_pos = pos + 1;
   }
   if (a.nx_out) {  // same values as the embedding launch of the next forward would write
     __syncthreads();

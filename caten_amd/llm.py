@@ -122,6 +122,14 @@ class Transformer:
                                                   logits.ctypes.data if return_logits else None))
         return (int(tok.value), logits) if return_logits else int(tok.value)
 
+    def generate_until(self, max_steps: int, eos_token: int) -> List[int]:
+        """Greedy tokens from the device-resident loop until `eos_token` has been produced (it is the last element)
+        or `max_steps` tokens exist; the stop condition is evaluated on the device."""
+        out = np.empty(max(max_steps, 1), np.int64)
+        n = C.c_int()
+        _lib.check(self.lib.cthip_decoder_generate_until(self.handle, max_steps, int(eos_token), out.ctypes.data, C.byref(n)))
+        return [int(t) for t in out[:n.value]]
+
     def generate_on_device(self, steps: int) -> List[int]:
         """Continues greedily for `steps` tokens without returning to the host in between."""
         out = np.empty(max(steps, 1), np.int64)

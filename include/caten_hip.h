@@ -280,6 +280,12 @@ int cthip_decoder_forward(void *dec, const float *tokens, int s, int n, int64_t 
  * without host round trips and writes their greedy tokens to tokens_out (host).
  * Synchronous at the end only. */
 int cthip_decoder_generate(void *dec, int steps, int64_t *tokens_out);
+/* The same loop with a stop condition checked ON THE DEVICE (the reference's loop has none, apps/gpt2/gpt2.lisp:102:
+ * it always runs max-length forwards): the step that produces `eos_token` ends the sequence -- the steps already
+ * queued behind it leave token, position and history untouched, and the host, which looks at the flag between
+ * graph launches without waiting for it, stops queuing.  tokens_out receives the tokens up to and including
+ * eos_token (or max_steps of them), *n_generated their number; the position advances by that number. */
+int cthip_decoder_generate_until(void *dec, int max_steps, int64_t eos_token, int64_t *tokens_out, int *n_generated);
 /* Current position (tokens in the KV cache). */
 int cthip_decoder_position(const void *dec);
 /* Bytes of HBM one decode step must read at position t (weights + norms/biases + KV rows). */

@@ -331,3 +331,39 @@ def test_llama_1b_width_q4_0_matches_oracle(oracle):
     T = len(prompt) + steps - 1
     close(model.peek("k_cache.1")[:T * kd], ref.k_cache[1].ravel()[:T * kd])
     model.close()
+
+
+@pytest.mark.parametrize("name", ["gpt2-tiny", "gpt2-mini"])
+def test_generate_until_stops_on_the_device(name):
+    """The device-resident loop with a stop condition: the step that produces the end token is the last one that
+    changes anything (token, position, history), however many steps were already queued behind it; what comes out
+    is the unconditional loop's sequence cut after that token, and generation can go on from there."""
+    print(f"case: generate_until {name}", flush=True)
+    from caten_amd import synth, llm, HipError
+    cfg = synth.GPT2_CONFIGS[name]
+    sd = llm.gpt2_state_dict(synth.gpt2_weights(cfg, seed=4), "q8_0")
+    prompt = synth.prompt(cfg["vocab"], 9, seed=4)
+    model = llm.make_gpt2(cfg, sd)
+    first = model.forward([float(t) for t in prompt], len(prompt), 0)
+    free = model.generate_on_device(40)
+    model.close()
+    # an end token that first appears somewhere in the middle (and one that appears at the very first step)
+    for k in (0, 5, 17, 30):
+        eos = free[k]
+        k = free.index(eos)
+        model = llm.make_gpt2(cfg, sd)
+        assert model.forward([float(t) for t in prompt], len(prompt), 0) == first
+        got = model.generate_until(40, eos)
+        assert got == free[:k + 1]
+        assert model.position == len(prompt) + k + 1
+        # the loop state is where the end token left it: going on reproduces the unconditional sequence
+        assert model.generate_on_device(3) == free[k + 1:k + 4]
+        model.close()
+    # a token that never comes: all max_steps tokens
+    model = llm.make_gpt2(cfg, sd)
+    model.forward([float(t) for t in prompt], len(prompt), 0)
+    never = next(t for t in range(cfg["vocab"]) if t not in free)
+    assert model.generate_until(40, never) == free
+    with pytest.raises(HipError):
+        model.generate_until(5, cfg["vocab"])
+    model.close()

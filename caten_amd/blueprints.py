@@ -128,3 +128,91 @@ def argmax_rows(name: str = "fused_argmax") -> dict:
          "expr": {"op": "CAST", "dtype": "int64", "args": [_add(_add("n", {"op": "NEG", "args": ["g"]}), {"op": "NEG", "args": [1]})]}},
         {"type": "ENDFOR", "idx": "_gid0"},
     ]}
+
+
+def _sub(a, b):
+    return _add(a, {"op": "NEG", "args": [b]})
+
+
+def add_global_2d(name: str = "fused_add_global", local=(16, 8)) -> dict:
+    """z = x + y over (rows, n) after the auto-scheduler's GLOBAL directive (directive.lisp:94-117): each loop has
+    become `idx = blockIdx.d * local + threadIdx.d` (an EXPR carrying its ExprGrid) and a bounds IF; the grid size is
+    spelled the way astfor-mutate-global spells it.  Arguments: val_z, rows, n, val_x, val_y."""
+    def bind(idx, rank, upper, loc):
+        size = {"op": "CAST", "dtype": "float32", "args": [upper]}
+        gs = {"op": "CAST", "dtype": "int64",
+              "args": [_add(_mul(size, {"op": "RECIP", "args": [float(loc)]}), (loc - 1) / float(loc))]}  # ceil(size / local)
+        sp = lambda lv: {"op": "SPACE", "level": lv, "rank": rank}  # noqa: E731
+        return {"type": "EXPR", "writes": [_A(idx, None)], "declare_type": True, "dtype": "int64",
+                "expr": _add(_mul(sp("block"), loc), sp("thread")), "grid": {"rank": rank, "global": gs, "local": loc}}
+    idx = _add(_mul("n", "_gid0"), "_gid1")
+    return {"name": name, "blueprint": [
+        _glob("val_z", "output", 2), _glob("rows", "shape", 0, "int64"), _glob("n", "shape", 0, "int64"),
+        _glob("val_x", "input", 2), _glob("val_y", "input", 2),
+        bind("_gid0", 1, "rows", local[1]),
+        {"type": "IF", "condition": _lt("_gid0", "rows")},
+        bind("_gid1", 0, "n", local[0]),
+        {"type": "IF", "condition": _lt("_gid1", "n")},
+        {"type": "EXPR", "writes": [_A("val_z", idx)], "expr": _add(_A("val_x", idx), _A("val_y", idx)), "dtype": "float32"},
+        {"type": "ENDIF"},
+        {"type": "ENDIF"},
+    ]}
+
+
+def conv2d_relu(N, C, H, W, K, R, S, name: str = "fused_conv2d") -> dict:
+    """relu(conv2d(x, w) + b), NCHW, stride 1, no padding, static shapes: the seven-loop nest the reference lowers a
+    ConvND to (nn/conv.lisp: im2col-free windowed views, one reduction nest over c, r, s).  Arguments: val_y, val_x, val_w, val_b."""
+    OH, OW = H - R + 1, W - S + 1
+    loops = [("_gid0", N), ("_gid1", K), ("_gid2", OH), ("_gid3", OW)]
+    red = [("_gid4", C), ("_gid5", R), ("_gid6", S)]
+    xi = _add(_mul(C * H * W, "_gid0"), _mul(H * W, "_gid4"), _mul(W, _add("_gid2", "_gid5")), _add("_gid3", "_gid6"))
+    wi = _add(_mul(C * R * S, "_gid1"), _mul(R * S, "_gid4"), _mul(S, "_gid5"), "_gid6")
+    yi = _add(_mul(K * OH * OW, "_gid0"), _mul(OH * OW, "_gid1"), _mul(OW, "_gid2"), "_gid3")
+    bp = [_glob("val_y", "output", 4), _glob("val_x", "input", 4), _glob("val_w", "input", 4), _glob("val_b", "input", 1)]
+    bp += [{"type": "FOR", "idx": i, "upfrom": 0, "below": _lt(i, n), "by": 1} for i, n in loops]
+    bp.append({"type": "EXPR", "writes": [_A("acc", None)], "expr": 0.0, "declare_type": True, "dtype": "float32"})
+    bp += [{"type": "FOR", "idx": i, "upfrom": 0, "below": _lt(i, n), "by": 1} for i, n in red]
+    bp.append({"type": "EXPR", "writes": [_A("acc", None)], "dtype": "float32", "reduction": True,
+               "expr": _add("acc", _mul(_A("val_x", xi), _A("val_w", wi)))})
+    bp += [{"type": "ENDFOR", "idx": i} for i, _ in reversed(red)]
+    bp.append({"type": "EXPR", "writes": [_A("val_y", yi)], "dtype": "float32",
+               "expr": {"op": "MAX", "args": [_add("acc", _A("val_b", "_gid1")), 0.0]}})
+    bp += [{"type": "ENDFOR", "idx": i} for i, _ in reversed(loops)]
+    return {"name": name, "blueprint": bp}
+
+
+def maxpool2x2(N, C, H, W, name: str = "fused_maxpool") -> dict:
+    """MaxPool 2x2 stride 2 over NCHW (nn/pool.lisp): max-reduction over the window.  Arguments: val_y, val_x."""
+    OH, OW = H // 2, W // 2
+    loops = [("_gid0", N * C), ("_gid1", OH), ("_gid2", OW)]
+    xi = _add(_mul(H * W, "_gid0"), _mul(W, _add(_mul(2, "_gid1"), "_gid3")), _add(_mul(2, "_gid2"), "_gid4"))
+    yi = _add(_mul(OH * OW, "_gid0"), _mul(OW, "_gid1"), "_gid2")
+    bp = [_glob("val_y", "output", 4), _glob("val_x", "input", 4)]
+    bp += [{"type": "FOR", "idx": i, "upfrom": 0, "below": _lt(i, n), "by": 1} for i, n in loops]
+    bp.append({"type": "EXPR", "writes": [_A("m", None)], "expr": float("-inf"), "declare_type": True, "dtype": "float32"})
+    bp += [{"type": "FOR", "idx": i, "upfrom": 0, "below": _lt(i, 2), "by": 1} for i in ("_gid3", "_gid4")]
+    bp.append({"type": "EXPR", "writes": [_A("m", None)], "dtype": "float32", "reduction": True, "expr": {"op": "MAX", "args": ["m", _A("val_x", xi)]}})
+    bp += [{"type": "ENDFOR", "idx": i} for i in ("_gid4", "_gid3")]
+    bp.append({"type": "EXPR", "writes": [_A("val_y", yi)], "dtype": "float32", "expr": "m"})
+    bp += [{"type": "ENDFOR", "idx": i} for i, _ in reversed(loops)]
+    return {"name": name, "blueprint": bp}
+
+
+def linear_relu_backward(name: str = "fused_relu_bias_backward") -> dict:
+    """A backward item of y = relu(x @ W^T + b): dz = dy * (y > 0) written back, and db[j] = sum_i dz[i, j] -- a
+    reduction over the FIRST axis, so the parallel loop is the feature axis and the batch loop stays serial inside a
+    thread.  Arguments: val_dz, val_db, m, n, val_dy, val_y."""
+    idx = _add(_mul("n", "_gid1"), "_gid0")
+    gate = {"op": "WHERE", "args": [_lt(0.0, _A("val_y", idx)), _A("val_dy", idx), 0.0]}
+    return {"name": name, "blueprint": [
+        _glob("val_dz", "output", 2), _glob("val_db", "output", 1), _glob("m", "shape", 0, "int64"), _glob("n", "shape", 0, "int64"),
+        _glob("val_dy", "input", 2), _glob("val_y", "input", 2),
+        {"type": "FOR", "idx": "_gid0", "upfrom": 0, "below": _lt("_gid0", "n"), "by": 1},
+        {"type": "EXPR", "writes": [_A("acc", None)], "expr": 0.0, "declare_type": True, "dtype": "float32"},
+        {"type": "FOR", "idx": "_gid1", "upfrom": 0, "below": _lt("_gid1", "m"), "by": 1},
+        {"type": "EXPR", "writes": [_A("val_dz", idx)], "expr": gate, "dtype": "float32"},
+        {"type": "EXPR", "writes": [_A("acc", None)], "expr": _add("acc", gate), "dtype": "float32", "reduction": True},
+        {"type": "ENDFOR", "idx": "_gid1"},
+        {"type": "EXPR", "writes": [_A("val_db", "_gid0")], "expr": "acc", "dtype": "float32"},
+        {"type": "ENDFOR", "idx": "_gid0"},
+    ]}

@@ -10,9 +10,11 @@
 //   (item NAME node...)
 //   node := (define-global ID DTYPE POINTER-P input|output|shape NRANK)
 //         | (for IDX UPFROM BELOW BY [local|global]) | (endfor IDX) | (if COND) | (endif)
-//         | (expr (WRITE...) RHS :dtype DTYPE [:declare t] [:reduction t])
+//         | (expr (WRITE...) RHS :dtype DTYPE [:declare t] [:reduction t] [:grid (RANK GLOBAL-SIZE LOCAL-SIZE)])
 //   WRITE, expr := number | inf | -inf | nan | t | nil | SYMBOL | (aref ID [INDEX]) | (const VALUE DTYPE)
 //         | (cast DTYPE expr) | (space block|thread RANK) | (OP expr...)     OP = the aasm instruction set
+// :grid marks the statement that binds an index to (space block RANK) * LOCAL-SIZE + (space thread RANK) after the
+// auto-scheduler's GLOBAL directive (its ExprGrid); such an item is launched with exactly those sizes.
 // BELOW is the loop condition, e.g. (< _gid0 n) (source/byoc/clang.lisp:58-73); an aref's INDEX is the flat element
 // index sum_d stride_d * (from_d + by_d * gid_d) the reference renders (clang.lisp:82-97).
 //
@@ -141,6 +143,11 @@ struct BpNode {
   Sx rhs;
   bool declare = false, reduction = false;
   std::string dtype = "float32";
+  // an index bound to blockIdx / threadIdx by the auto-scheduler's GLOBAL directive carries the launch size of
+  // its axis (ExprGrid: source/codegen/auto-scheduler/directive.lisp:94-117, gathered by blueprint-gather-grids,
+  // source/codegen/blueprint.lisp:726-737): rank 0..2, workgroups along it, threads per workgroup along it
+  int grid_rank = -1;
+  Sx grid_global, grid_local;
 };
 struct Item {
   std::string name;
@@ -224,6 +231,14 @@ static bool build_item(const Sx &top, Item &it, std::string &err) {
         if (n.v[q].is_sym("dtype")) b.dtype = n.v[q + 1].s;
         else if (n.v[q].is_sym("declare") || n.v[q].is_sym("declare-type")) b.declare = truthy(n.v[q + 1]);
         else if (n.v[q].is_sym("reduction")) b.reduction = truthy(n.v[q + 1]);
+        else if (n.v[q].is_sym("grid")) {
+          const Sx &g = n.v[q + 1];
+          if (!g.is_list() || g.n() != 3 || g.v[0].kind != Sx::INT || g.v[0].i < 0 || g.v[0].i > 2)
+            return err = "expr: :grid (RANK GLOBAL-SIZE LOCAL-SIZE) with rank 0, 1 or 2", false;
+          b.grid_rank = (int)g.v[0].i;
+          b.grid_global = g.v[1];
+          b.grid_local = g.v[2];
+        }
       }
       if (b.writes.empty()) return err = "expr: no write", false;
       if (!cdtypes().count(b.dtype)) return err = "expr: unknown dtype " + b.dtype, false;
@@ -393,35 +408,66 @@ static int match_end(const std::vector<BpNode> &b, int i) {  // index of the END
   return -1;
 }
 
-// integer expressions over the by-value arguments (grid sizes, route shapes)
-static bool eval_int(const Sx &e, const std::map<std::string, long long> &env, long long &out) {
-  if (e.kind == Sx::INT) { out = e.i; return true; }
-  if (e.kind == Sx::FLT) { out = (long long)e.f; return e.f == (double)out; }
+// Expressions over the by-value arguments (grid sizes, route shapes), evaluated on the host.  Integer arithmetic is
+// exact (loop bounds, strides); the float instructions cover how the GLOBAL directive spells a grid size,
+// cast_int(ceil-ish(float(upper - from) / float(by)) / local-size) (directive.lisp:97-100).
+static bool eval_num(const Sx &e, const std::map<std::string, long long> &env, double &out, bool &is_int) {
+  if (e.kind == Sx::INT) { out = (double)e.i; is_int = true; return true; }
+  if (e.kind == Sx::FLT) { out = e.f; is_int = false; return true; }
   if (e.kind == Sx::SYM) {
     auto it = env.find(e.s);
     if (it == env.end()) return false;
-    out = it->second;
+    out = (double)it->second;
+    is_int = true;
     return true;
   }
   if (e.kind != Sx::LIST || e.v.empty() || e.v[0].kind != Sx::SYM) return false;
   const std::string &op = e.v[0].s;
-  if (op == "const") return e.n() >= 2 && eval_int(e.v[1], env, out);
-  if (op == "cast") return e.n() >= 3 && eval_int(e.v[2], env, out);
-  std::vector<long long> a;
+  if (op == "const") {
+    if (e.n() < 2 || !eval_num(e.v[1], env, out, is_int)) return false;
+    if (e.n() >= 3 && e.v[2].kind == Sx::SYM && e.v[2].s.rfind("float", 0) == 0) is_int = false;
+    return true;
+  }
+  if (op == "cast") {
+    if (e.n() < 3 || !eval_num(e.v[e.n() - 1], env, out, is_int)) return false;
+    const bool to_float = e.v[1].kind == Sx::SYM && e.v[1].s.rfind("float", 0) == 0;
+    if (!to_float) out = trunc(out);  // a C cast to an integer type
+    is_int = !to_float;
+    return true;
+  }
+  std::vector<double> a;
+  bool all_int = true;
   for (size_t k = 1; k < e.n(); k++) {
-    long long v;
-    if (!eval_int(e.v[k], env, v)) return false;
+    if (e.v[k].is_sym("nil")) continue;  // the placeholder read of :< / :!=
+    double v;
+    bool vi;
+    if (!eval_num(e.v[k], env, v, vi)) return false;
     a.push_back(v);
+    all_int = all_int && vi;
   }
   if (a.empty()) return false;
-  if (op == "add") { out = 0; for (long long v : a) out += v; return true; }
-  if (op == "mul") { out = 1; for (long long v : a) out *= v; return true; }
+  is_int = all_int;
+  if (op == "add") { out = 0; for (double v : a) out += v; return true; }
+  if (op == "mul") { out = 1; for (double v : a) out *= v; return true; }
   if (op == "neg") { out = -a[0]; return true; }
   if (op == "max" && a.size() == 2) { out = a[0] > a[1] ? a[0] : a[1]; return true; }
-  if (op == "idiv" && a.size() == 2 && a[1]) { out = a[0] / a[1]; return true; }
-  if (op == "mod" && a.size() == 2 && a[1]) { out = a[0] % a[1]; return true; }
+  if (op == "recip") {
+    if (a[0] == 0) return false;
+    if (all_int) out = trunc(1.0 / a[0]);
+    else out = 1.0 / a[0];
+    return true;
+  }
+  if (op == "idiv" && a.size() == 2 && a[1] != 0) { out = all_int ? trunc(a[0] / a[1]) : a[0] / a[1]; return true; }
+  if (op == "mod" && a.size() == 2 && a[1] != 0 && all_int) { out = (double)((long long)a[0] % (long long)a[1]); return true; }
   if (op == "move" || op == "store") { out = a.back(); return true; }
   return false;
+}
+static bool eval_int(const Sx &e, const std::map<std::string, long long> &env, long long &out) {
+  double v;
+  bool is_int;
+  if (!eval_num(e, env, v, is_int) || v != trunc(v) || fabs(v) > 9e15) return false;
+  out = (long long)v;
+  return true;
 }
 
 // ------------------------------------------------------------------ routes to hand-written kernels
@@ -464,6 +510,8 @@ struct Program {
   std::vector<Sx> grid_bounds;
   int rows_per_block = 256;
   bool parallel = false;
+  bool explicit_grid = false;  // the blueprint carries its own launch sizes (ExprGrid)
+  Sx grid_global[3], grid_local[3];
   Route route;
   hipFunction_t fn = nullptr;
 };
@@ -811,8 +859,17 @@ struct KernelRenderer {
       if (g.pointer) params += std::string(g.type == "input" ? "const " : "") + ct + "*" + (g.type == "input" ? " __restrict__ " : " ") + g.id;
       else params += "const " + ct + " " + g.id;
     }
-    o += "extern \"C\" __global__ void __launch_bounds__(256) " + it.name + "(" + params + ") {\n";
-    const int npar = parallel_prefix();
+    for (const BpNode &n : b)
+      if (n.t == BpNode::EXPR && n.grid_rank >= 0) {
+        if (!pg.explicit_grid)
+          for (int q = 0; q < 3; q++) pg.grid_global[q] = pg.grid_local[q] = sx_int(1);
+        pg.explicit_grid = true;
+        pg.grid_global[n.grid_rank] = n.grid_global;
+        pg.grid_local[n.grid_rank] = n.grid_local;
+      }
+    o += std::string("extern \"C\" __global__ void __launch_bounds__(") + (pg.explicit_grid ? "1024" : "256") + ") " + it.name + "(" + params + ") {\n";
+    // an item that brings its own grid keeps its loops as they are: the scheduler has distributed it already
+    const int npar = pg.explicit_grid ? 0 : parallel_prefix();
     std::map<int, std::vector<std::pair<std::string, std::string>>> wave_red;
     const int lo = npar, hi = (int)b.size() - npar;
     const bool wave = npar > 0 && wave_reductions(lo, hi, wave_red);
@@ -1080,6 +1137,22 @@ int cthip_program_launch(void *program, void **args, int nargs) {
     total *= v > 0 ? v : 0;
   }
   unsigned grid[3] = {1, 1, 1}, block[3] = {1, 1, 1};
+  if (pg->explicit_grid) {
+    long long threads = 1;
+    for (int q = 0; q < 3; q++) {
+      long long g, l;
+      if (!eval_int(pg->grid_global[q], env, g) || !eval_int(pg->grid_local[q], env, l))
+        return fail(CTHIP_E_UNSUPPORTED, "HIP: %s: a grid size is not an expression of the shape arguments", it.name.c_str());
+      if (g < 0 || l < 1 || g > 0x7fffffffll || l > 1024) return fail(CTHIP_E_BAD_ARG, "HIP: %s: grid %lld x %lld along axis %d", it.name.c_str(), g, l, q);
+      if (g == 0) return 0;
+      grid[q] = (unsigned)g;
+      block[q] = (unsigned)l;
+      threads *= l;
+    }
+    if (threads > 1024) return fail(CTHIP_E_BAD_ARG, "HIP: %s: %lld threads per workgroup", it.name.c_str(), threads);
+    pg->last_route = "rendered";
+    return cthip_launch(pg->fn, grid, block, 0, args, nargs);
+  }
   if (pg->parallel) {
     const long long per = pg->rows_per_block;
     const long long nb = (total + per - 1) / per;

@@ -13,7 +13,9 @@ Blueprints are authored as plain dicts (so a fixture needs no Lisp image).  A Sc
   {"type": "DEFINE-GLOBAL", "id", "dtype", "pointer_p", "arg_type": "output"|"shape"|"input", "nrank"}
   {"type": "FOR", "idx", "upfrom": expr, "below": expr, "by": expr, "scope": "local"|"global"}
   {"type": "ENDFOR", "idx"}            {"type": "IF", "condition": expr}      {"type": "ENDIF"}
-  {"type": "EXPR", "writes": [aref], "expr": expr, "declare_type": bool, "dtype": str, "reduction": bool}
+  {"type": "EXPR", "writes": [aref], "expr": expr, "declare_type": bool, "dtype": str, "reduction": bool,
+   "grid": {"rank": 0|1|2, "global": expr, "local": expr}}     (grid: only on the statement that binds an index to
+                                                                 blockIdx / threadIdx, its ExprGrid, directive.lisp:94-117)
 
   expr := number | "symbol" | aref | {"op": OP, "args": [expr...]}            (OP = aasm instruction set)
         | {"op": "CAST", "dtype": str, "args": [expr]} | {"op": "CONST", "value": v, "dtype": str}
@@ -132,6 +134,9 @@ def item_sexp(item: dict) -> str:
                 flags += " :declare t"
             if n.get("reduction"):
                 flags += " :reduction t"
+            if n.get("grid") is not None:  # ExprGrid of an index bound to blockIdx / threadIdx (directive.lisp:94-117)
+                g = n["grid"]
+                flags += f" :grid ({int(g['rank'])} {sexp(g['global'])} {sexp(g['local'])})"
             out.append(f"  (expr ({' '.join(sexp(w) for w in n['writes'])}) {sexp(n['expr'])}{flags})")
         else:
             out.append(f"  ({t.lower()})")  # the library reports the unknown node type

@@ -206,12 +206,18 @@
     (:EXPR
      (let ((iterations (getattr bp :iterations))
            (type (read-type-relay bp)))
-       (format out "  (expr (~{~a~^ ~}) ~a :dtype ~(~a~)~a~a)~%"
+       (format out "  (expr (~{~a~^ ~}) ~a :dtype ~(~a~)~a~a~a)~%"
                (map 'list #'(lambda (x y z) (write-sexp x y z iterations)) (node-writes bp) (relay-writes type) (relay-write-iters type))
                (sexp (getattr bp :EXPR) iterations)
                (buffer-dtype (car (relay-writes type)))
                (if (car (getattr bp :declare-type)) " :declare t" "")
-               (if (getattr bp :reduction :allow-undefined t) " :reduction t" ""))))))
+               (if (getattr bp :reduction :allow-undefined t) " :reduction t" "")
+               ;; an index the GLOBAL directive bound to blockIdx / threadIdx brings the launch size of its axis
+               ;; (source/codegen/auto-scheduler/directive.lisp:94-117; Metal gathers them with blueprint-gather-grids)
+               (let ((meta (getattr bp :meta :allow-undefined t)))
+                 (if (typep meta 'ExprGrid)
+                     (format nil " :grid (~a ~a ~a)" (exprgrid-rank meta) (sexp (exprgrid-global-size meta)) (sexp (exprgrid-local-size meta)))
+                     "")))))))
 
 (defclass Hip-Program ()
   ((name :initarg :name :accessor hp-name)

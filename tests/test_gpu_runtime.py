@@ -520,3 +520,56 @@ def test_rank0_output_passed_by_pointer_is_written_back():
     item["compiled_object"](None, s, 100, x)
     assert s.value == 4950.5  # the incoming value went in, the result came back
     close_buffer(rt, x)
+
+
+@pytest.mark.parametrize("rows,n", [(1, 1), (37, 1000), (256, 64)])
+def test_item_with_an_explicit_grid_launches_on_that_grid(rows, n):
+    """An item the auto-scheduler marked GLOBAL (directive.lisp:94-117): indices are blockIdx * local + threadIdx with
+    a bounds IF, the launch takes ceil(size / local) blocks from the ExprGrid expressions (2-D here)."""
+    import caten_amd as ca
+    from caten_amd import blueprints as bp
+    print(f"case: explicit grid {rows}x{n}", flush=True)
+    rng = np.random.default_rng(rows)
+    x = rng.standard_normal((rows, n)).astype(np.float32)
+    y = rng.standard_normal((rows, n)).astype(np.float32)
+    (got,), prog = _run_item(ca, bp.add_global_2d(), [np.full((rows, n), np.nan, np.float32), rows, n, x, y])
+    assert prog.last_route == "rendered"
+    assert np.array_equal(got, x + y)
+
+
+def test_conv2d_and_maxpool_items(oracle):
+    """relu(conv2d + bias) (nn/conv.lisp) and 2x2 max-pool (nn/pool.lisp) as their static loop nests: output
+    positions across threads, window reductions serial in the thread; against NumPy in fp64."""
+    import caten_amd as ca
+    from caten_amd import blueprints as bp
+    print("case: conv2d / maxpool items", flush=True)
+    rng = np.random.default_rng(0)
+    N, Cc, H, W, K, R, S = 3, 5, 17, 19, 7, 3, 4
+    x = rng.standard_normal((N, Cc, H, W)).astype(np.float32)
+    w = (0.2 * rng.standard_normal((K, Cc, R, S))).astype(np.float32)
+    b = rng.standard_normal(K).astype(np.float32)
+    OH, OW = H - R + 1, W - S + 1
+    (got,), _ = _run_item(ca, bp.conv2d_relu(N, Cc, H, W, K, R, S), [np.zeros((N, K, OH, OW), np.float32), x, w, b])
+    win = np.lib.stride_tricks.sliding_window_view(x.astype(np.float64), (R, S), axis=(2, 3))  # N C OH OW R S
+    want = np.maximum(np.einsum("nchwrs,kcrs->nkhw", win, w.astype(np.float64)) + b[None, :, None, None], 0.0)
+    assert np.all(np.abs(got - want) <= 1e-4 + 1e-3 * np.abs(want))
+    H2, W2 = 16, 18
+    xp = rng.standard_normal((N, Cc, H2, W2)).astype(np.float32)
+    (gp,), _ = _run_item(ca, bp.maxpool2x2(N, Cc, H2, W2), [np.zeros((N, Cc, H2 // 2, W2 // 2), np.float32), xp])
+    assert np.array_equal(gp, xp.reshape(N, Cc, H2 // 2, 2, W2 // 2, 2).max(axis=(3, 5)))
+
+
+@pytest.mark.parametrize("m,n", [(1, 5), (130, 300), (1000, 64)])
+def test_backward_item_with_a_first_axis_reduction(m, n):
+    """The backward of relu(x W^T + b) with respect to the pre-activation and the bias: dz = dy * (y > 0) and
+    db = dz.sum(axis 0) in one item; the batch loop is the reduction, taken by the lanes of a wavefront."""
+    import caten_amd as ca
+    from caten_amd import blueprints as bp
+    print(f"case: relu/bias backward {m}x{n}", flush=True)
+    rng = np.random.default_rng(m)
+    y = np.maximum(rng.standard_normal((m, n)), 0).astype(np.float32)
+    dy = rng.standard_normal((m, n)).astype(np.float32)
+    (dz, db), _ = _run_item(ca, bp.linear_relu_backward(), [np.zeros((m, n), np.float32), np.zeros(n, np.float32), m, n, dy, y])
+    want = np.where(y > 0, dy, 0).astype(np.float32)
+    assert np.array_equal(dz, want)
+    assert np.allclose(db, want.astype(np.float64).sum(0), rtol=1e-4, atol=1e-4)

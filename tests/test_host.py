@@ -315,3 +315,25 @@ def test_runtime_vm_semantics_on_host_scalars():
     s = make_buffer([], [], "int64")
     s.value = 7
     assert coerce_dtyped_buffer(s, "float32") == 7.0 and coerce_dtyped_buffer(3.9, "int64") == 3
+
+
+def test_explicit_grid_item_keeps_its_own_indexing():
+    """An item whose indices are bound from blockIdx / threadIdx (ExprGrid) gets no second work distribution from the
+    renderer, and the text of its grid sizes is carried into the program."""
+    from caten_amd import HipRenderer, blueprints as bp
+    it = bp.add_global_2d(local=(16, 8))
+    src = HipRenderer().render_kernel(it)
+    assert "_total" not in src and "__launch_bounds__(1024)" in src
+    assert "((blockIdx.y*8)+threadIdx.y)" in src and "((blockIdx.x*16)+threadIdx.x)" in src
+    assert "if ((_gid1<n))" in src
+
+
+def test_conv_pool_and_backward_items_render():
+    from caten_amd import HipRenderer, blueprints as bp
+    r = HipRenderer()
+    conv = r.render_kernel(bp.conv2d_relu(2, 3, 8, 8, 4, 3, 3))
+    assert "(long long)(2)*(long long)(4)*(long long)(6)*(long long)(6)" in conv and conv.count("for (int") == 3
+    pool = r.render_kernel(bp.maxpool2x2(2, 3, 8, 8))
+    assert "_negative_infinity" in pool and "ct_max(m," in pool
+    bwd = r.render_kernel(bp.linear_relu_backward())
+    assert "ct_wave_add_f(acc)" in bwd and "_gid1+=64" in bwd

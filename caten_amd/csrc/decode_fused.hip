@@ -27,57 +27,72 @@
 
 namespace cthip {
 
-constexpr float kFixScale = 4294967296.0f;             // 2^32
-constexpr float kFixInv = 2.3283064365386963e-10f;     // 2^-32
+// The registers a launch's input vector  x = base + bias + sum(partials)  is requested into (one float4 per thread,
+// D <= 1024).  MODE 0: base only; 1: + bias + NP fp32 partial vectors; 2: + bias + NP fixed-point accumulators.
+template <int MODE, int NP>
+struct DecStageRegs {
+  float4 v, g, b;
+  float4 p[MODE == 1 ? NP : 1];
+  longlong2 lo[MODE == 2 ? NP : 1], hi[MODE == 2 ? NP : 1];
+  int i;
+  bool active;
+};
 
-__device__ __forceinline__ int xcd_id() {
-  // XCC_ID hardware register (id 20), bits 3:0: the XCD this wavefront runs on
-  return (int)__builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20) & (kDecXcds - 1);
+// Requests only, every one unconditional.  A launch issues these FIRST, then its weight requests, then fences the
+// scheduler: answers come back in request order, so the vector is staged while the weights are still arriving,
+// and no use of an answer (the compiler likes to start adding partials early, to save registers) ends up in
+// front of a later request, where it would hold that request back by a memory round trip.
+template <int MODE, int NP>
+__device__ __forceinline__ void dec_stage_request(const DecStage &s, DecStageRegs<MODE, NP> &r) {
+  const int tid = threadIdx.x;
+  const int n4 = s.D >> 2;
+  r.active = tid < n4;
+  const int i = r.active ? tid : n4 - 1;
+  r.i = i;
+  r.v = ((const float4 *)s.base)[i];
+  r.g = ((const float4 *)s.gamma)[i];
+  if (MODE != 0) r.b = ((const float4 *)s.bias)[i];
+  if (MODE == 1) {
+#pragma unroll
+    for (int k = 0; k < NP; k++) r.p[k] = ((const float4 *)(s.fparts + (int64_t)k * s.D))[i];
+  }
+  if (MODE == 2) {
+#pragma unroll
+    for (int k = 0; k < NP; k++) {
+      const longlong2 *src = (const longlong2 *)(s.iparts + (int64_t)k * s.D) + 2 * i;
+      r.lo[k] = src[0];
+      r.hi[k] = src[1];
+    }
+  }
 }
 
-__device__ __forceinline__ float4 f4add(float4 a, float4 b) { return make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w); }
-
-// Assembles the launch's input vector  x = base + bias + sum(partials)  (one float4 per thread, D <= 1024),
-// writes gamma * x to LDS and returns the LayerNorm statistics of x; block 0 also stores x to s.xout.
-// MODE 0: base only; 1: + bias + NP fp32 partial vectors; 2: + bias + NP fixed-point accumulators.
-// Every load is unconditional and issued before any use.  red holds 24 floats.  blockDim.x == 256.
+// Adds the answers up, writes gamma * x to LDS and returns the LayerNorm statistics of x; block 0 also stores x to
+// s.xout.  red holds 24 floats.  blockDim.x == 256.
 template <int MODE, int NP>
-__device__ __forceinline__ void dec_stage(const DecStage &s, float *xs, float *red, float &mu, float &rstd) {
+__device__ __forceinline__ void dec_stage_finish(const DecStage &s, DecStageRegs<MODE, NP> &r, float *xs, float *red,
+                                                 float &mu, float &rstd) {
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
-  const int n4 = s.D >> 2;
-  const bool active = tid < n4;
-  const int i = active ? tid : n4 - 1;
-  float4 v = ((const float4 *)s.base)[i];
-  const float4 g = ((const float4 *)s.gamma)[i];
-  if (MODE != 0) {
-    const float4 b = ((const float4 *)s.bias)[i];
-    if (MODE == 1) {
-      float4 p[NP];
+  const bool active = r.active;
+  const int i = r.i;
+  float4 v = r.v;
+  const float4 g = r.g;
+  if (MODE == 1) {
+    v = f4add(v, r.b);
 #pragma unroll
-      for (int k = 0; k < NP; k++) p[k] = ((const float4 *)(s.fparts + (int64_t)k * s.D))[i];
-      v = f4add(v, b);
+    for (int k = 0; k < NP; k++) v = f4add(v, r.p[k]);
+  }
+  if (MODE == 2) {
+    long long t0 = 0, t1 = 0, t2 = 0, t3 = 0;
 #pragma unroll
-      for (int k = 0; k < NP; k++) v = f4add(v, p[k]);
-    } else {
-      longlong2 lo[NP], hi[NP];
-#pragma unroll
-      for (int k = 0; k < NP; k++) {
-        const longlong2 *src = (const longlong2 *)(s.iparts + (int64_t)k * s.D) + 2 * i;
-        lo[k] = src[0];
-        hi[k] = src[1];
-      }
-      long long t0 = 0, t1 = 0, t2 = 0, t3 = 0;
-#pragma unroll
-      for (int k = 0; k < NP; k++) {
-        t0 += lo[k].x;
-        t1 += lo[k].y;
-        t2 += hi[k].x;
-        t3 += hi[k].y;
-      }
-      v = f4add(v, b);
-      v = f4add(v, make_float4(__ll2float_rn(t0) * kFixInv, __ll2float_rn(t1) * kFixInv, __ll2float_rn(t2) * kFixInv,
-                               __ll2float_rn(t3) * kFixInv));
+    for (int k = 0; k < NP; k++) {
+      t0 += r.lo[k].x;
+      t1 += r.lo[k].y;
+      t2 += r.hi[k].x;
+      t3 += r.hi[k].y;
     }
+    v = f4add(v, r.b);
+    v = f4add(v, make_float4(__ll2float_rn(t0) * kFixInv, __ll2float_rn(t1) * kFixInv, __ll2float_rn(t2) * kFixInv,
+                             __ll2float_rn(t3) * kFixInv));
   }
   // (count, mean, squared deviation) per thread, merged exactly: thread -> wavefront by lane reductions,
   // wavefront -> workgroup through LDS behind the one barrier that also publishes the staged vector
@@ -145,6 +160,10 @@ __global__ __launch_bounds__(256) void k_dec_qkv(DecQkvArgs a) {
   int row = blockIdx.x * 16 + wv * 4 + g;
   const bool row_ok = row < a.rows;
   row = row_ok ? row : a.rows - 1;
+  DecStageRegs<MODE, NP> sr;
+  dec_stage_request(a.st, sr);
+  const int posv = a.pos[0];
+  __builtin_amdgcn_sched_barrier(0);
   uint4 w[KC];
   unsigned sc[KC];
   const uint4 *qp = (const uint4 *)a.wq + (int64_t)row * (16 * KC);
@@ -156,9 +175,9 @@ __global__ __launch_bounds__(256) void k_dec_qkv(DecQkvArgs a) {
     sc[j] = dp[c >> 1];
   }
   const float fs = a.fold_s[row], fc = a.fold_c[row];
-  const int posv = a.pos[0];
+  __builtin_amdgcn_sched_barrier(0);
   float mu, rstd;
-  dec_stage<MODE, NP>(a.st, xs, red, mu, rstd);
+  dec_stage_finish(a.st, sr, xs, red, mu, rstd);
   const float acc = dec_row_dot<KC>(w, sc, xs, l);
   if (l == 0 && row_ok) {
     // rstd * (W.(gamma x) - mu * W.gamma) + (W.beta + bias)  =  W.LayerNorm(x) + bias
@@ -319,6 +338,9 @@ __global__ __launch_bounds__(256) void k_dec_mlp(DecMlpArgs a) {
   const int D = a.st.D;
   const int slab = blockIdx.x;
   const int row = slab * 16 + wv * 4 + g;  // < F: the launcher requires F % 16 == 0
+  DecStageRegs<1, NP> sr;
+  dec_stage_request(a.st, sr);
+  __builtin_amdgcn_sched_barrier(0);
   uint4 w[KC];
   unsigned sc[KC];
   const uint4 *qp = (const uint4 *)a.wq + (int64_t)row * (16 * KC);
@@ -339,8 +361,9 @@ __global__ __launch_bounds__(256) void k_dec_mlp(DecMlpArgs a) {
     pw[j] = ((const uint4 *)a.pq)[(int64_t)slab * D + r];
     ps[j] = a.pd[(int64_t)(slab >> 1) * D + r];
   }
+  __builtin_amdgcn_sched_barrier(0);
   float mu, rstd;
-  dec_stage<1, NP>(a.st, xs, red, mu, rstd);
+  dec_stage_finish(a.st, sr, xs, red, mu, rstd);
   const float acc = dec_row_dot<KC>(w, sc, xs, l);
   if (l == 0) hs[wv * 4 + g] = ct_gelu(rstd * (acc - mu * fs) + fc);
   __syncthreads();
@@ -368,7 +391,8 @@ __global__ __launch_bounds__(256) void k_dec_mlp(DecMlpArgs a) {
 __global__ __launch_bounds__(256) void k_dec_sum(DecStage s, float *out) {
   const int n4 = s.D >> 2;
   for (int i = threadIdx.x; i < n4; i += 256) {
-    float4 v = f4add(((const float4 *)s.base)[i], ((const float4 *)s.bias)[i]);
+    float4 v = ((const float4 *)s.base)[i];
+    if (s.bias) v = f4add(v, ((const float4 *)s.bias)[i]);
     long long t[4] = {0, 0, 0, 0};
 #pragma unroll
     for (int k = 0; k < kDecXcds; k++) {

@@ -96,6 +96,9 @@ struct Decoder {
   bool fused = false;
   float *x2 = nullptr, *patt = nullptr;
   long long *pmlp = nullptr;
+  // grouped-query layers (decode_gqa.hip): the attention projection has an accumulator set of its own
+  bool fused_gqa = false;
+  long long *pattn = nullptr;
   hipGraphExec_t g_step = nullptr, g_body = nullptr, g_multi = nullptr;
   int64_t weight_bytes = 0, vector_bytes = 0;
   std::vector<void *> owned;  // device blocks to free
@@ -352,6 +355,30 @@ static int finalize(Decoder *d) {
       TRY(dev_alloc(d, (void **)&d->pmlp, sizeof(long long) * (size_t)kDecXcds * D));
     }
   }
+  if (c.arch == CTHIP_ARCH_LLAMA && state().decode_fused &&
+      gqa_fused_supported(d->layers[0].attn->type, d->layers[0].proj->type, d->layers[0].fc->type, d->layers[0].fc2->type,
+                          D, c.n_heads, c.n_kv_heads, F)) {
+    int max_id = -1;
+    TRY(dec_xcd_probe(&max_id));
+    d->fused_gqa = max_id >= 0 && max_id < kDecXcds;
+    for (int l = 0; l < c.n_layers && d->fused_gqa; l++) {
+      Layer &L = d->layers[l];
+      if (L.attn->type != CTHIP_Q4_0 || L.proj->type != CTHIP_Q4_0 || L.fc->type != CTHIP_Q4_0 || L.fc2->type != CTHIP_Q4_0)
+        d->fused_gqa = false;
+    }
+    if (d->fused_gqa) {
+      for (int l = 0; l < c.n_layers; l++) {
+        Layer &L = d->layers[l];
+        TRY(gqa_relay_groups(L.proj, D / c.n_heads, &L.proj_hq, &L.proj_hd));
+        TRY(gqa_relay_slabs(L.fc2, &L.fc2_sq, &L.fc2_sd));
+        d->owned.insert(d->owned.end(), {L.proj_hq, L.proj_hd, L.fc2_sq, L.fc2_sd});
+      }
+      TRY(dev_alloc(d, (void **)&d->x2, sizeof(float) * D));
+      TRY(dev_alloc(d, (void **)&d->pattn, sizeof(long long) * (size_t)kDecXcds * D));
+      TRY(dev_alloc(d, (void **)&d->pmlp, sizeof(long long) * (size_t)kDecXcds * D));
+      TRY(cthip_memset(d->pattn, 0, sizeof(long long) * (size_t)kDecXcds * D));
+    }
+  }
   if (!state().decoder_graph) d->use_graph = false;
   if (d->use_graph) {
     hipStream_t st = state().stream;
@@ -449,6 +476,72 @@ static int queue_step(Decoder *d, bool with_head, bool embed) {
     DecStage fin = {};
     fin.base = d->x;
     fin.bias = d->layers[c.n_layers - 1].fc2_b;
+    fin.iparts = d->pmlp;
+    fin.D = D;
+    TRY(launch_dec_sum(fin, d->x));
+    if (with_head) TRY(queue_head(d));
+    return 0;
+  }
+  if (d->fused_gqa) {
+    // The same three launches for grouped-query layers.  Both column Linears add into per-XCD accumulators:
+    // pattn (attention projection, cleared by the qkv launch) and pmlp (down projection, cleared by the attention
+    // launch); the residual stream alternates between d->x and d->x2 as "base + accumulators".
+    const int replicas = 4;
+    const int64_t acc16 = (int64_t)kDecXcds * D * 8 / 16;
+    for (int l = 0; l < c.n_layers; l++) {
+      Layer &L = d->layers[l];
+      GqaQkvArgs qa = {};
+      qa.st.base = d->x;
+      qa.st.iparts = d->pmlp;
+      qa.st.gamma = L.ln1_g;
+      qa.st.xout = d->x2;
+      qa.st.eps = c.eps;
+      qa.st.D = D;
+      qa.wq = L.attn->q;
+      qa.wd = (const unsigned short *)L.attn->d;
+      qa.q = d->q;
+      qa.kc = L.k_cache;
+      qa.vc = L.v_cache;
+      qa.pos = pos;
+      qa.rows = D + 2 * KD;
+      qa.KD = KD;
+      qa.DH = Dh;
+      qa.log2_base = log2f(c.rope_base);
+      qa.zero = d->pattn;
+      qa.zero_n16 = acc16;
+      TRY(launch_gqa_qkv(qa, l > 0));
+      GqaAttnArgs aa = {};
+      aa.q = d->q;
+      aa.kc = L.k_cache;
+      aa.vc = L.v_cache;
+      aa.pos = pos;
+      aa.pq = L.proj_hq;
+      aa.pd = (const unsigned short *)L.proj_hd;
+      aa.accum = d->pattn;
+      aa.zero = d->pmlp;
+      aa.zero_n16 = acc16;
+      aa.D = D;
+      aa.KD = KD;
+      TRY(launch_gqa_attn_proj(aa, c.n_heads, c.n_kv_heads, replicas));
+      GqaMlpArgs ma = {};
+      ma.st.base = d->x2;
+      ma.st.iparts = d->pattn;
+      ma.st.gamma = L.ln2_g;
+      ma.st.xout = d->x;
+      ma.st.eps = c.eps;
+      ma.st.D = D;
+      ma.wq = L.fc->q;
+      ma.wd = (const unsigned short *)L.fc->d;
+      ma.gate_stride = L.fc_pairs ? 2 : 1;
+      ma.up_off = L.fc_pairs ? 1 : F;
+      ma.pq = L.fc2_sq;
+      ma.pd = (const unsigned short *)L.fc2_sd;
+      ma.accum = d->pmlp;
+      TRY(launch_gqa_mlp(ma, F, c.n_kv_heads));
+    }
+    DecStage fin = {};
+    fin.base = d->x;
+    fin.bias = nullptr;
     fin.iparts = d->pmlp;
     fin.D = D;
     TRY(launch_dec_sum(fin, d->x));

@@ -394,25 +394,6 @@ __global__ __launch_bounds__(256) void k_qkv_split(float *__restrict__ q, float 
 // (positional-encoding.lisp:3-64 at position pos), uses them for key T-1, and the first query head of each
 // kv group stores the rotated key and the value into cache row T-1 -- the rotation and the `!assign` into
 // the cache (layers.lisp:13-33) need no launches of their own.
-__device__ __forceinline__ float4 rope4(float4 x, int c, int DH, float log2_base, int at) {
-  // lane c holds elements 4c..4c+3 = pairs 2c and 2c+1 of the head; same arithmetic as k_rope
-  float o[4] = {x.x, x.y, x.z, x.w};
-#pragma unroll
-  for (int t = 0; t < 2; t++) {
-    const int i = 2 * c + t;
-    const float expo = (float)(2 * i) / (float)DH;
-    const float logb = log2_base * 0.6931472f;
-    const float theta = exp2f(-(expo * logb) * 1.442695f);
-    const float ang = (float)at * theta;
-    float sn, cs;
-    sincosf(ang, &sn, &cs);
-    const float x0 = o[2 * t], x1 = o[2 * t + 1];
-    o[2 * t] = x0 * cs - x1 * sn;
-    o[2 * t + 1] = x0 * sn + x1 * cs;
-  }
-  return make_float4(o[0], o[1], o[2], o[3]);
-}
-
 template <int DH, bool APPEND>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)))
 void k_attn_cached(float *__restrict__ out, const float *__restrict__ q,

@@ -161,6 +161,42 @@ def test_three_launch_layer_equals_five_launch_layer(name, plen):
         assert np.array_equal(a, c)
 
 
+@pytest.mark.parametrize("plen", [3, 40])
+def test_three_launch_grouped_query_layer_equals_five_launch_layer(plen):
+    """The same for RMSNorm / RoPE / grouped-query / SwiGLU layers with Q4_0 weights at the width the three-launch
+    layer is built for (d 2048, 32 query / 4 key-value heads, SwiGLU 5632; 2 layers, small vocabulary): both column
+    Linears add into per-XCD integer accumulators.  Identical greedy tokens and cache rows inside the fp32 band
+    against the five-launch layer, bit-identical logits between two runs."""
+    print(f"case: three-launch vs five-launch grouped-query layer, prompt {plen}", flush=True)
+    from caten_amd import _lib, synth, llm
+    lib = _lib.load()
+    cfg = dict(synth.LLAMA_CONFIGS["llama-1.1b"], n_layers=2, max_seq=96, vocab=2000)
+    sd = llm.llama_state_dict(synth.llama_weights(cfg, seed=13), "q4_0")
+    prompt = synth.prompt(cfg["vocab"], plen, seed=13)
+    kd = cfg["dim"] // cfg["n_heads"] * cfg["n_kv_heads"]
+    runs, caches = [], []
+    try:
+        for mode in (1, 0, 1):
+            _lib.check(lib.cthip_set_option(b"decode_fused", mode))
+            model = llm.make_llama(cfg, sd)
+            runs.append(llm.gpt2_generate(model, prompt, 20, on_device=False, keep_logits=True))
+            caches.append([model.peek(f"{n}.{l}")[:(plen + 19) * kd] for n in ("k_cache", "v_cache") for l in (0, 1)])
+            model.close()
+    finally:
+        _lib.check(lib.cthip_set_option(b"decode_fused", 1))
+    assert runs[0][0] == runs[1][0] == runs[2][0]
+    for a, b, c in zip(*[r[1] for r in runs]):
+        close(a, b)
+        assert np.array_equal(a, c)
+    for a, b, c in zip(*caches):
+        close(a, b)
+        assert np.array_equal(a, c)
+    # the device-resident loop (graphs of several steps) gives the host-driven loop's tokens
+    model = llm.make_llama(cfg, sd)
+    assert llm.gpt2_generate(model, prompt, 20, on_device=True) == runs[0][0]
+    model.close()
+
+
 def test_gpt2_prompt_lengths_and_restart(oracle):
     from caten_amd import synth, llm
     cfg = synth.GPT2_CONFIGS["gpt2-tiny"]

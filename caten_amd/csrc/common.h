@@ -232,6 +232,32 @@ __device__ __forceinline__ float apply_act(int act, float v) {
   }
 }
 
+// byte N of a dword as a float in one instruction.  Written out because the compiler, seeing the nibble mask,
+// narrows every extract to a 4-bit field extract followed by a byte-0 conversion: two instructions per weight.
+#define CTHIP_UBYTE(N)                                                  \
+  __device__ __forceinline__ float ubyte##N##_f32(uint32_t v) {         \
+    float f;                                                            \
+    asm("v_cvt_f32_ubyte" #N " %0, %1" : "=v"(f) : "v"(v));             \
+    return f;                                                           \
+  }
+CTHIP_UBYTE(0)
+CTHIP_UBYTE(1)
+CTHIP_UBYTE(2)
+CTHIP_UBYTE(3)
+#undef CTHIP_UBYTE
+// the same for a signed byte: the conversion sign-extends the selected byte itself (otherwise a field extract first)
+#define CTHIP_SBYTE(N)                                                                                          \
+  __device__ __forceinline__ float sbyte##N##_f32(uint32_t v) {                                                 \
+    float f;                                                                                                    \
+    asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_" #N : "=v"(f) : "v"(v)); \
+    return f;                                                                                                   \
+  }
+CTHIP_SBYTE(0)
+CTHIP_SBYTE(1)
+CTHIP_SBYTE(2)
+CTHIP_SBYTE(3)
+#undef CTHIP_SBYTE
+
 // RoPE of four consecutive elements of a head (positional-encoding.lisp:3-64) at position `at`
 __device__ __forceinline__ float4 rope4(float4 x, int c, int DH, float log2_base, int at) {
   // lane c holds elements 4c..4c+3 = pairs 2c and 2c+1 of the head; same arithmetic as k_rope

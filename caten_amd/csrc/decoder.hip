@@ -243,8 +243,10 @@ static int finalize(Decoder *d) {
     snprintf(b, sizeof(b), c.arch == CTHIP_ARCH_GPT2 ? "h.%d.%s" : "layers.%d.%s", l, s);
     return std::string(b);
   };
-#define TRY(e) \
-  if ((rc = (e))) return rc
+#define TRY(e)                 \
+  do {                         \
+    if ((rc = (e))) return rc; \
+  } while (0)
   if (c.arch == CTHIP_ARCH_GPT2) {
     TRY(to_f32(d, "wte.weight", (int64_t)V * D, &d->wte));
     TRY(to_f32(d, "wpe.weight", (int64_t)c.max_seq * D, &d->wpe));
@@ -414,8 +416,10 @@ static int queue_step(Decoder *d, bool with_head, bool embed) {
   const int D = c.dim, F = c.ffn, V = c.vocab, KD = kv_dim(c), Dh = c.dim / c.n_heads;
   const int *tok = d->tokpos, *pos = d->tokpos + 1;
   int rc;
-#define TRY(e) \
-  if ((rc = (e))) return rc
+#define TRY(e)                 \
+  do {                         \
+    if ((rc = (e))) return rc; \
+  } while (0)
   const bool gpt2 = c.arch == CTHIP_ARCH_GPT2;
   // embed = false: the previous step's head has already gathered this step's input (queue_head)
   if (embed) TRY(launch_embedding(d->x, d->wte, nullptr, tok, 1, V, D, gpt2 ? d->wpe : nullptr, pos, c.max_seq));

@@ -45,20 +45,6 @@ __device__ __forceinline__ float chunk_dot<CTHIP_Q8_0>(const uint4 w, float scal
   return s * scale;
 }
 
-// byte N of a dword as a float in one instruction.  Written out because the compiler, seeing the nibble mask,
-// narrows every extract to a 4-bit field extract followed by a byte-0 conversion: two instructions per weight.
-#define CTHIP_UBYTE(N)                                                  \
-  __device__ __forceinline__ float ubyte##N##_f32(uint32_t v) {         \
-    float f;                                                            \
-    asm("v_cvt_f32_ubyte" #N " %0, %1" : "=v"(f) : "v"(v));             \
-    return f;                                                           \
-  }
-CTHIP_UBYTE(0)
-CTHIP_UBYTE(1)
-CTHIP_UBYTE(2)
-CTHIP_UBYTE(3)
-#undef CTHIP_UBYTE
-
 template <>
 __device__ __forceinline__ float chunk_dot<CTHIP_Q4_0>(const uint4 w, float scale, const float *__restrict__ x, float xsum) {
   const uint32_t dw[4] = {w.x, w.y, w.z, w.w};

@@ -4,9 +4,10 @@
 //
 // One 256-thread workgroup (4 wavefronts, 2x2) owns a 64x64 tile of C; each wavefront accumulates a
 // 32x32 sub-tile in 16 accumulator registers, with v_mfma_f32_32x32x2_f32 (k_gemm_f32, fp32 operands)
-// or v_mfma_f32_32x32x16_bf16 (k_gemm_split / k_gemm_q, operands split into bf16 terms, fp32
-// accumulation).  Operands are staged through two LDS buffers with three K-steps of global loads in
-// flight; 1024x1024 outputs give 256 workgroups = one per compute unit.
+// or v_mfma_f32_32x32x16_bf16 (k_gemm_split, operands split into bf16 terms, fp32 accumulation).  Operands are
+// staged through two LDS buffers with three K-steps of global loads in flight; 1024x1024 outputs give 256
+// workgroups = one per compute unit.  Quantised weights take k_gemm_qpc: 64x128 tiles, 512 threads, half of
+// them staging and half multiplying.  Finished tiles leave through LDS as whole rows (store_tile).
 #include <hip/hip_bf16.h>
 
 #include "common.h"
@@ -54,7 +55,7 @@ struct GemmArgs {
 // holds them k-contiguous per row in bf16, 16-byte chunks swizzled by row so that neither the operand
 // reads nor the staging writes collide on banks.  Two LDS buffers and three register sets keep the
 // global loads three K-steps ahead of the MFMAs with one barrier per step.
-enum { W_ROWMAJOR = 0, W_F32 = 1, W_F16 = 2, W_Q4 = 3, W_Q8 = 4 };  // W_Q4 / W_Q8: k_gemm_q only
+enum { W_ROWMAJOR = 0, W_F32 = 1, W_F16 = 2, W_Q4 = 3, W_Q8 = 4 };  // W_Q4 / W_Q8: k_gemm_qpc only
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
 typedef float v2f __attribute__((ext_vector_type(2)));
@@ -112,12 +113,63 @@ struct BRegs {  // one K-step of B held by a thread between its request and its 
 // staging and the row-wise A writes over all banks.
 __device__ __forceinline__ int swz(int row) { return (row ^ (row >> 3)) & 7; }
 
+// Row-wise stores of a finished BM x BN tile that the multiplying wavefronts have put into LDS (Cs, row pitch
+// BN + 4 floats): all NT threads of the workgroup take 16-byte pieces of whole rows, so a store instruction covers
+// 512 contiguous bytes per 32 lanes and bias / residual are read the same way.  (Stores straight from the
+// accumulator layout are 16 or 32 scalar stores per lane and keep a workgroup busy for microseconds.)
+// Split-K shares go to their slice of a.ws untouched.  Call after a barrier that follows the writes to Cs.
+template <int BM, int BN, int NT>
+__device__ __forceinline__ void store_tile(const GemmArgs &a, const float *Cs, int m0, int n0, int tid) {
+  constexpr int LDC = BN + 4, F4 = BN / 4;
+  const int M = a.M, N = a.N;
+  const bool plain = a.ksplit > 1;
+  float *dst = plain ? a.ws + (int64_t)blockIdx.y * M * N : a.C;
+  const bool vec = (N & 3) == 0;
+#pragma unroll
+  for (int j = 0; j < BM * F4 / NT; j++) {
+    const int f = tid + NT * j, lr = f / F4, c4 = f % F4;
+    const int row = m0 + lr, col = n0 + 4 * c4;
+    if (row >= M || col >= N) continue;
+    const float4 v4 = *(const float4 *)(Cs + lr * LDC + 4 * c4);
+    float v[4] = {v4.x, v4.y, v4.z, v4.w};
+    float *o = dst + (int64_t)row * N + col;
+    if (vec) {
+      if (!plain) {
+        if (a.bias) {
+          const float4 bb = *(const float4 *)(a.bias + col);
+          v[0] += bb.x, v[1] += bb.y, v[2] += bb.z, v[3] += bb.w;
+        }
+#pragma unroll
+        for (int t = 0; t < 4; t++) v[t] = apply_act(a.act, v[t]);
+        if (a.residual) {
+          const float4 rr = *(const float4 *)(a.residual + (int64_t)row * N + col);
+          v[0] += rr.x, v[1] += rr.y, v[2] += rr.z, v[3] += rr.w;
+        }
+      }
+      *(float4 *)o = make_float4(v[0], v[1], v[2], v[3]);
+    } else {
+      for (int t = 0; t < 4 && col + t < N; t++) {
+        float x = v[t];
+        if (!plain) {
+          x = apply_act(a.act, x + (a.bias ? a.bias[col + t] : 0.0f));
+          if (a.residual) x += a.residual[(int64_t)row * N + col + t];
+        }
+        o[t] = x;
+      }
+    }
+  }
+}
+
 template <int BMODE, int NS, bool AL>
 __global__ __launch_bounds__(256) void k_gemm_split(GemmArgs a) {
   constexpr int BM = 64, BN = 64, BK = 64, LDK = BK, NP = (NS == 1) ? 1 : (NS == 3) ? 2 : 3;
   constexpr int NSET = 3;  // register sets = K-steps of global loads in flight
-  __shared__ __align__(16) unsigned short As[2][NP][BM][LDK];
-  __shared__ __align__(16) unsigned short Bs[2][NP][BN][LDK];
+  constexpr int kOpBytes = 2 * NP * BM * LDK * 2, kCBytes = BM * (BN + 4) * 4;
+  // both operand buffers; after the last step the same memory holds the output tile (store_tile)
+  __shared__ __align__(16) unsigned char smem[2 * kOpBytes > kCBytes ? 2 * kOpBytes : kCBytes];
+  typedef unsigned short(*OpT)[NP][BM][LDK];
+  OpT As = (OpT)smem, Bs = (OpT)(smem + kOpBytes);
+  float *Cs = (float *)smem;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
@@ -301,28 +353,12 @@ __global__ __launch_bounds__(256) void k_gemm_split(GemmArgs a) {
     if (i + 1 < nsteps) step(i + 1, ra2, rb2);
   }
   // ---- epilogue: acc[r] is C[row = 8*(r/4) + 4*(l/32) + r%4][col = l%32] of the 32x32 sub-tile ----
-  const int col = n0 + 32 * wn + (lane & 31);
-  if (col < N) {
-    if (a.ksplit > 1) {
-      float *ws = a.ws + (int64_t)blockIdx.y * M * N;
+  // (the last step ended with a barrier: nobody reads the operand buffers any more)
 #pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const int row = m0 + 32 * wm + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-        if (row < M) ws[(int64_t)row * N + col] = acc[r];
-      }
-      return;
-    }
-    const float bias = a.bias ? a.bias[col] : 0.0f;
-#pragma unroll
-    for (int r = 0; r < 16; r++) {
-      const int row = m0 + 32 * wm + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-      if (row < M) {
-        float v = apply_act(a.act, acc[r] + bias);
-        if (a.residual) v += a.residual[(int64_t)row * N + col];
-        a.C[(int64_t)row * N + col] = v;
-      }
-    }
-  }
+  for (int r = 0; r < 16; r++)
+    Cs[(32 * wm + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * (BN + 4) + 32 * wn + (lane & 31)] = acc[r];
+  __syncthreads();
+  store_tile<BM, BN, 256>(a, Cs, m0, n0, tid);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -336,30 +372,54 @@ __global__ __launch_bounds__(256) void k_gemm_split(GemmArgs a) {
 // Against dequantising to fp32 and splitting both operands this needs a third fewer MFMAs, an eighth
 // of the conversion work on the weight side, and is more accurate (no rounding of q * d).
 //
-// One 256-thread workgroup owns 64*MB x 64 of the output (a wavefront accumulates MB 32x32 blocks; MB = 1 is
-// what the launcher uses), walks K in steps of 64 = two quant blocks, same LDS layout / swizzle / prefetch
-// depth / XCD regions / split-K as k_gemm_split.
+// K is walked in steps of 64 = two quant blocks, with the LDS layout / swizzle / prefetch depth / XCD regions /
+// split-K of k_gemm_split.
 template <int MB>
 struct ARegsQ {  // one K-step of A held by a thread: rows ar + 16 i, i < 4 * MB
   float4 v[4 * MB];
 };
-struct BRegsQ {
-  uint4 v;           // Q8_0: 16 int8; Q4_0: the 16 bytes of a 32-weight block
-  unsigned short d;  // fp16 scale bits (threads tid < 128: row tid >> 1, block tid & 1 of the step)
-};
 
 // two small integers (as floats, exact) -> packed bf16 pair, x0 in the low half
 __device__ __forceinline__ unsigned pack_int_bf16(float x0, float x1) {
-  return (__float_as_uint(x1) & 0xffff0000u) | (__float_as_uint(x0) >> 16);
+  return __builtin_amdgcn_perm(__float_as_uint(x1), __float_as_uint(x0), 0x07060302u);  // high halves of both
 }
 
-template <int WT, int NPA, int MB>
-__global__ __launch_bounds__(256) void k_gemm_q(GemmArgs a) {
-  constexpr int BM = 64 * MB, BN = 64, BK = 64, LDK = BK;
-  __shared__ __align__(16) unsigned short As[2][NPA][BM][LDK];
-  __shared__ __align__(16) unsigned short Bs[2][BN][LDK];
+// ---------------------------------------------------------------------------------------------
+// The two halves of a K-step are done by different wavefronts of a 512-thread workgroup.
+//
+// When every wavefront stages (conversions on the vector ALU, LDS writes), then multiplies (LDS reads, matrix
+// cores, block scales on the vector ALU), then meets the others at a barrier, nothing overlaps with one or two
+// wavefronts per SIMD: a step of 64 took 0.7-1.1 us and the matrix cores were busy an eighth of the time.
+// Here wavefronts 4..7 only stage the NEXT step (and request the one three further on) while wavefronts 0..3
+// only multiply the CURRENT one out of the other LDS buffer, so every SIMD holds one of each and the waits of
+// one half are filled by the other.  (Measured with in-kernel timestamps on 512 x 3072 x 768: matrix
+// instructions and vector instructions of a SIMD do not issue side by side, so a step costs the sum of both
+// halves' instructions, about 0.95 us; what the split removes is the exposed latency between the phases.)
+// The tile is 64 x 128 (a multiplying wavefront owns 32 x 64 = two accumulator blocks against one A operand),
+// which keeps both halves about equally long and gives the prefill shapes no more workgroups than compute units.
+// Weight bytes become floats with one sign-extending conversion each (sbyteN_f32) and pairs of them bf16 with
+// one byte permute.
+struct BRegsQ2 {
+  uint4 v[2];        // rows wr and wr + 64 of the tile
+  unsigned short d;  // fp16 scale bits: row ptid >> 1, block ptid & 1 of the step
+};
+
+template <int WT, int NPA>
+__global__ __launch_bounds__(512) void k_gemm_qpc(GemmArgs a) {
+  constexpr int BM = 64, BN = 128, BK = 64, LDK = BK, LDC = BN + 4;
+  constexpr int kABytes = 2 * NPA * BM * LDK * 2, kBBytes = 2 * BN * LDK * 2, kCBytes = BM * LDC * 4;
+  // the operand buffers; after the last step the same memory holds the output tile for the row-wise stores
+  __shared__ __align__(16) unsigned char smem[(kABytes + kBBytes > kCBytes) ? kABytes + kBBytes : kCBytes];
   __shared__ float Ss[2][BN][2];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  typedef unsigned short(*AsT)[NPA][BM][LDK];
+  typedef unsigned short(*BsT)[BN][LDK];
+  AsT As = (AsT)smem;
+  BsT Bs = (BsT)(smem + kABytes);
+  float(*Cs)[LDC] = (float(*)[LDC])smem;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const bool producer = tid >= 256;
+  const int ptid = tid & 255;            // staging role: index among the staging threads
+  const int wave = (tid >> 6) & 3;       // multiplying role: 2 x 2 wavefronts of 32 x 64
   const int wm = wave >> 1, wn = wave & 1;
   const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
   if (local >= a.rm * a.rn) return;
@@ -369,35 +429,37 @@ __global__ __launch_bounds__(256) void k_gemm_q(GemmArgs a) {
   const int M = a.M, N = a.N, ldk = a.K;
   const int kbeg = blockIdx.y * a.kper;
   const int K = min(a.K, kbeg + a.kper);
-  v16f acc[MB];
+  v16f acc[2];
 #pragma unroll
-  for (int b = 0; b < MB; b++)
+  for (int b = 0; b < 2; b++)
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[b][r] = 0.0f;
 
-  const int ar = tid >> 4, akq = tid & 15;  // A: rows ar + 16 i, k = 4 akq .. +3
-  const int wr = tid >> 2, wkc = tid & 3;   // B: weight row wr, k = 16 wkc .. +15
-  const int sr = (tid & 127) >> 1, sb = tid & 1;  // scales: row sr, quant block sb of the step (threads < 128 stage them)
+  const int ar = ptid >> 4, akq = ptid & 15;  // A: rows ar + 16 i, k = 4 akq .. +3
+  const int wr = ptid >> 2, wkc = ptid & 3;   // B: weight rows wr and wr + 64, k = 16 wkc .. +15
+  const int sr = ptid >> 1, sb = ptid & 1;    // scales: row sr, quant block sb of the step
   const int blocks_per_row = ldk >> 5;
 
-  // requests without branches (see load4; quantised rows are a multiple of 32 wide, so always aligned)
-  auto fetch = [&](int k0, ARegsQ<MB> &ra, BRegsQ &rb) {  // k0 counts from kbeg
+  auto fetch = [&](int k0, ARegsQ<1> &ra, BRegsQ2 &rb) {  // k0 counts from kbeg; requests without branches
 #pragma unroll
-    for (int i = 0; i < 4 * MB; i++) {
+    for (int i = 0; i < 4; i++) {
       const int row = m0 + ar + 16 * i, k = kbeg + k0 + 4 * akq;
       ra.v[i] = load4<true>(a.A + (int64_t)row * ldk + k, row < M ? clamp04(K - k) : 0);
     }
-    // a 16-wide chunk / a quant block is inside the row or past this share's end
-    const int n = n0 + wr, k = kbeg + k0 + 16 * wkc;
-    const int64_t e = (int64_t)n * ldk + k;
-    const uint8_t *q = (const uint8_t *)a.wq + (WT == W_Q8 ? e : ((e >> 5) << 4));
-    rb.v = *((n < N && k < K) ? (const uint4 *)q : (const uint4 *)g_zeros);
-    const int ns = n0 + sr, ks = kbeg + k0 + 32 * sb;  // threads 128.. ask for the same scales again: same cache lines
+    const int k = kbeg + k0 + 16 * wkc;
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      const int n = n0 + wr + 64 * j;
+      const int64_t e = (int64_t)n * ldk + k;
+      const uint8_t *q = (const uint8_t *)a.wq + (WT == W_Q8 ? e : ((e >> 5) << 4));
+      rb.v[j] = *((n < N && k < K) ? (const uint4 *)q : (const uint4 *)g_zeros);
+    }
+    const int ns = n0 + sr, ks = kbeg + k0 + 32 * sb;
     rb.d = *((ns < N && ks < K) ? a.wd + (int64_t)ns * blocks_per_row + (ks >> 5) : (const unsigned short *)g_zeros);
   };
-  auto stage = [&](const ARegsQ<MB> &ra, const BRegsQ &rb, int buf) {
+  auto stage = [&](const ARegsQ<1> &ra, const BRegsQ2 &rb, int buf) {
 #pragma unroll
-    for (int i = 0; i < 4 * MB; i++) {
+    for (int i = 0; i < 4; i++) {
       const float x[4] = {ra.v[i].x, ra.v[i].y, ra.v[i].z, ra.v[i].w};
       uint2 pl[NPA];
       split4<NPA>(x, pl);
@@ -405,76 +467,91 @@ __global__ __launch_bounds__(256) void k_gemm_q(GemmArgs a) {
 #pragma unroll
       for (int p = 0; p < NPA; p++) *(uint2 *)&As[buf][p][row][8 * ((akq >> 1) ^ swz(row)) + 4 * (akq & 1)] = pl[p];
     }
-    float q[16];
-    const unsigned dw[4] = {rb.v.x, rb.v.y, rb.v.z, rb.v.w};
-    if (WT == W_Q8) {
 #pragma unroll
-      for (int t = 0; t < 4; t++) {
-        const int v = (int)dw[t];
-        q[4 * t + 0] = (float)(int)(int8_t)(v);
-        q[4 * t + 1] = (float)(int)(int8_t)(v >> 8);
-        q[4 * t + 2] = (float)(int)(int8_t)(v >> 16);
-        q[4 * t + 3] = (float)(v >> 24);
+    for (int jr = 0; jr < 2; jr++) {
+      float q[16];
+      const unsigned dw[4] = {rb.v[jr].x, rb.v[jr].y, rb.v[jr].z, rb.v[jr].w};
+      if (WT == W_Q8) {
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+          q[4 * t + 0] = sbyte0_f32(dw[t]);
+          q[4 * t + 1] = sbyte1_f32(dw[t]);
+          q[4 * t + 2] = sbyte2_f32(dw[t]);
+          q[4 * t + 3] = sbyte3_f32(dw[t]);
+        }
+      } else {
+        // chunks 0, 2 of the step are the low nibbles of their block, 1, 3 the high
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+          const unsigned nb = ((wkc & 1) ? dw[t] >> 4 : dw[t]) & 0x0f0f0f0fu;
+          q[4 * t + 0] = ubyte0_f32(nb) - 8.0f;
+          q[4 * t + 1] = ubyte1_f32(nb) - 8.0f;
+          q[4 * t + 2] = ubyte2_f32(nb) - 8.0f;
+          q[4 * t + 3] = ubyte3_f32(nb) - 8.0f;
+        }
       }
-    } else {
-      const int sh = (wkc & 1) ? 4 : 0;  // chunks 0, 2 of the step are the low nibbles of their block, 1, 3 the high
+      const int row = wr + 64 * jr;
 #pragma unroll
-      for (int t = 0; t < 16; t++) q[t] = (float)((int)((dw[t >> 2] >> (8 * (t & 3) + sh)) & 0xf) - 8);
+      for (int j = 0; j < 2; j++)
+        *(uint4 *)&Bs[buf][row][8 * ((2 * wkc + j) ^ swz(row))] =
+            make_uint4(pack_int_bf16(q[8 * j + 0], q[8 * j + 1]), pack_int_bf16(q[8 * j + 2], q[8 * j + 3]),
+                       pack_int_bf16(q[8 * j + 4], q[8 * j + 5]), pack_int_bf16(q[8 * j + 6], q[8 * j + 7]));
     }
-#pragma unroll
-    for (int j = 0; j < 2; j++)
-      *(uint4 *)&Bs[buf][wr][8 * ((2 * wkc + j) ^ swz(wr))] =
-          make_uint4(pack_int_bf16(q[8 * j + 0], q[8 * j + 1]), pack_int_bf16(q[8 * j + 2], q[8 * j + 3]),
-                     pack_int_bf16(q[8 * j + 4], q[8 * j + 5]), pack_int_bf16(q[8 * j + 6], q[8 * j + 7]));
-    if (tid < 128) Ss[buf][sr][sb] = half_bits_to_float(rb.d);
+    Ss[buf][sr][sb] = half_bits_to_float(rb.d);
   };
   auto mma = [&](int buf) {
-    const int rowb = 32 * wn + (lane & 31);
+    const int rowa = 32 * wm + (lane & 31);
 #pragma unroll
     for (int kb = 0; kb < 2; kb++) {  // the two quant blocks of the step
-      v16f tmp[MB];
+      v16f tmp[2];
 #pragma unroll
-      for (int b = 0; b < MB; b++)
+      for (int b = 0; b < 2; b++)
 #pragma unroll
         for (int r = 0; r < 16; r++) tmp[b][r] = 0.0f;
 #pragma unroll
       for (int s2 = 0; s2 < 2; s2++) {
         const int ch = 4 * kb + 2 * s2 + (lane >> 5);
-        const v8bf bv = __builtin_bit_cast(v8bf, *(const uint4 *)&Bs[buf][rowb][8 * (ch ^ swz(rowb))]);
+        v8bf av[NPA];
 #pragma unroll
-        for (int b = 0; b < MB; b++) {
-          const int rowa = 32 * MB * wm + 32 * b + (lane & 31);
+        for (int p = 0; p < NPA; p++) av[p] = __builtin_bit_cast(v8bf, *(const uint4 *)&As[buf][p][rowa][8 * (ch ^ swz(rowa))]);
 #pragma unroll
-          for (int p = NPA - 1; p >= 0; p--) {
-            const v8bf av = __builtin_bit_cast(v8bf, *(const uint4 *)&As[buf][p][rowa][8 * (ch ^ swz(rowa))]);
-            tmp[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv, tmp[b], 0, 0, 0);
-          }
+        for (int b = 0; b < 2; b++) {
+          const int rowb = 64 * wn + 32 * b + (lane & 31);
+          const v8bf bv = __builtin_bit_cast(v8bf, *(const uint4 *)&Bs[buf][rowb][8 * (ch ^ swz(rowb))]);
+#pragma unroll
+          for (int p = NPA - 1; p >= 0; p--) tmp[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[p], bv, tmp[b], 0, 0, 0);
         }
       }
-      const float d = Ss[buf][rowb][kb];  // scale of this lane's output column for this block
 #pragma unroll
-      for (int b = 0; b < MB; b++)
+      for (int b = 0; b < 2; b++) {
+        const float d = Ss[buf][64 * wn + 32 * b + (lane & 31)][kb];  // scale of this lane's output column for this block
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[b][r] = fmaf(d, tmp[b][r], acc[b][r]);
+      }
     }
   };
 
-  ARegsQ<MB> ra0, ra1, ra2;
-  BRegsQ rb0, rb1, rb2;
+  ARegsQ<1> ra0, ra1, ra2;
+  BRegsQ2 rb0, rb1, rb2;
   const int nsteps = K > kbeg ? (K - kbeg + BK - 1) / BK : 0;
-  // no conditions inside a step and no exit inside the loop, as in k_gemm_split
-  auto step = [&](int i, ARegsQ<MB> &ran, BRegsQ &rbn) {
-    stage(ran, rbn, (i + 1) & 1);
-    fetch((i + 4) * BK, ran, rbn);
-    mma(i & 1);
+  // one barrier per step; the branch on the role is uniform over a wavefront
+  auto step = [&](int i, ARegsQ<1> &ran, BRegsQ2 &rbn) {
+    if (producer) {
+      stage(ran, rbn, (i + 1) & 1);
+      fetch((i + 4) * BK, ran, rbn);
+    } else {
+      mma(i & 1);
+    }
     __syncthreads();
   };
   if (nsteps > 0) {
-    fetch(0, ra0, rb0);
-    fetch(BK, ra1, rb1);
-    fetch(2 * BK, ra2, rb2);
-    stage(ra0, rb0, 0);
-    fetch(3 * BK, ra0, rb0);
+    if (producer) {
+      fetch(0, ra0, rb0);
+      fetch(BK, ra1, rb1);
+      fetch(2 * BK, ra2, rb2);
+      stage(ra0, rb0, 0);
+      fetch(3 * BK, ra0, rb0);
+    }
     __syncthreads();
     int i = 0;
     for (; i + 3 <= nsteps; i += 3) {
@@ -485,26 +562,18 @@ __global__ __launch_bounds__(256) void k_gemm_q(GemmArgs a) {
     if (i < nsteps) step(i, ra1, rb1);
     if (i + 1 < nsteps) step(i + 1, ra2, rb2);
   }
-  // ---- epilogue: acc[b][r] is C[row = 8*(r/4) + 4*(l/32) + r%4][col = l%32] of the wavefront's block b ----
-  const int col = n0 + 32 * wn + (lane & 31);
-  if (col >= N) return;
-  const float bias = (a.ksplit > 1 || !a.bias) ? 0.0f : a.bias[col];
-  float *dst = a.ksplit > 1 ? a.ws + (int64_t)blockIdx.y * M * N : a.C;
+  // ---- epilogue: acc[b][r] is C[row = 8*(r/4) + 4*(l/32) + r%4][col = l%32] of the wavefront's block b.  The
+  // tile goes through LDS (the operand buffers are free after the last barrier) so that all 512 threads store
+  // whole rows: 16-byte stores, bias and residual read the same way.
+  if (!producer) {
 #pragma unroll
-  for (int b = 0; b < MB; b++) {
+    for (int b = 0; b < 2; b++)
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-      const int row = m0 + 32 * MB * wm + 32 * b + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-      if (row < M) {
-        float v = acc[b][r];
-        if (a.ksplit <= 1) {
-          v = apply_act(a.act, v + bias);
-          if (a.residual) v += a.residual[(int64_t)row * N + col];
-        }
-        dst[(int64_t)row * N + col] = v;
-      }
-    }
+      for (int r = 0; r < 16; r++)
+        Cs[32 * wm + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)][64 * wn + 32 * b + (lane & 31)] = acc[b][r];
   }
+  __syncthreads();
+  store_tile<BM, BN, 512>(a, &Cs[0][0], m0, n0, tid);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -528,8 +597,11 @@ __global__ __launch_bounds__(256) void k_gemm_f32(GemmArgs a) {
   // row pitches: odd where the staging writes are transposing scalar writes (k varies fastest over the lanes,
   // so k * pitch has to spread over the banks), a multiple of 4 where they are float4 rows
   constexpr int BM = 64, BN = 64, BK = 32, LDA = BM + 1, LDB = BMODE == B_ROWMAJOR ? BN + 4 : BN + 1;
-  __shared__ __align__(16) float As[2][BK][LDA];
-  __shared__ __align__(16) float Bs[2][BK][LDB];
+  constexpr int kABytes = 2 * BK * LDA * 4, kBBytes = 2 * BK * LDB * 4, kCBytes = BM * (BN + 4) * 4;
+  __shared__ __align__(16) unsigned char smem[kABytes + kBBytes > kCBytes ? kABytes + kBBytes : kCBytes];
+  float(*As)[BK][LDA] = (float(*)[BK][LDA])smem;
+  float(*Bs)[BK][LDB] = (float(*)[BK][LDB])(smem + kABytes);
+  float *Cs = (float *)smem;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
@@ -695,22 +767,12 @@ __global__ __launch_bounds__(256) void k_gemm_f32(GemmArgs a) {
     if (i + 1 < nsteps) step(i + 1, ra2, rb2);
   }
   // ---- epilogue: acc[r] is C[row = 8*(r/4) + 4*(l/32) + r%4][col = l%32] of the 32x32 sub-tile ----
-  const int col = n0 + 32 * wn + (lane & 31);
-  if (col >= N) return;
-  const float bias = (a.ksplit > 1 || !a.bias) ? 0.0f : a.bias[col];
-  float *dst = a.ksplit > 1 ? a.ws + (int64_t)blockIdx.y * M * N : a.C;
+  // (the last step ended with a barrier: nobody reads the operand buffers any more)
 #pragma unroll
-  for (int r = 0; r < 16; r++) {
-    const int row = m0 + 32 * wm + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-    if (row < M) {
-      float v = acc[r];
-      if (a.ksplit <= 1) {
-        v = apply_act(a.act, v + bias);
-        if (a.residual) v += a.residual[(int64_t)row * N + col];
-      }
-      dst[(int64_t)row * N + col] = v;
-    }
-  }
+  for (int r = 0; r < 16; r++)
+    Cs[(32 * wm + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * (BN + 4) + 32 * wn + (lane & 31)] = acc[r];
+  __syncthreads();
+  store_tile<BM, BN, 256>(a, Cs, m0, n0, tid);
 }
 
 // C = act(sum_z ws[z] + bias) + residual, z in ascending order (the result does not depend on timing)
@@ -739,7 +801,7 @@ __global__ __launch_bounds__(256) void k_splitk_reduce(GemmArgs a) {
 }
 
 // precision: GEMM_FP32 = fp32 MFMA operands (k_gemm_f32), GEMM_BF16 = operands rounded to bf16,
-// GEMM_BF16X3 / GEMM_BF16X6 = operands split in two / three bf16 terms.  Q8_0 / Q4_0 weights take k_gemm_q
+// GEMM_BF16X3 / GEMM_BF16X6 = operands split in two / three bf16 terms.  Q8_0 / Q4_0 weights take k_gemm_qpc
 // (integer plane exact in bf16, block scales applied to the partial sums) with 1 / 2 / 3 activation terms.
 // Split-K partial tiles of the entry point that allocates nothing (cthip_matmul_noalloc): one array per device,
 // held until the process ends.  In host code the name below is only a stand-in; the device address is taken
@@ -771,7 +833,8 @@ int launch_gemm(GemmArgs a, int bmode, int precision, float *static_ws, size_t s
   // 64 output rows per workgroup.  (128-row tiles -- two accumulator blocks per wavefront, half the weight-side
   // staging -- measured slower on every prefill shape: one workgroup per compute unit and 32 KB of A per step.)
   const int bm = 64;
-  const int64_t tiles = (int64_t)((a.M + bm - 1) / bm) * ((a.N + 63) / 64);
+  const int bn = quant ? 128 : 64;  // k_gemm_qpc owns 64 x 128
+  const int64_t tiles = (int64_t)((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn);
   if (tiles > 0x7fffffff / 16) return fail(CTHIP_E_BAD_ARG, "gemm: too many tiles");
   dim3 grid((unsigned)tiles), block(256);
   a.ksplit = 1;
@@ -780,7 +843,7 @@ int launch_gemm(GemmArgs a, int bmode, int precision, float *static_ws, size_t s
   {
     // one region of tiles per XCD: the split with the fewest tiles per XCD, then the least operand bytes per L2
     a.tm = (a.M + bm - 1) / bm;
-    a.tn = (a.N + 63) / 64;
+    a.tn = (a.N + bn - 1) / bn;
     const double sza = 4.0 * bm / 64, szb = bmode == B_ROWMAJOR ? 4.0 : a.wtype == CTHIP_Q8_0 ? 1.0625 : a.wtype == CTHIP_Q4_0 ? 0.5625 : a.wtype == CTHIP_F16 ? 2.0 : 4.0;
     double best = -1.0;
     for (int rx = 1; rx <= 8; rx *= 2) {
@@ -799,7 +862,8 @@ int launch_gemm(GemmArgs a, int bmode, int precision, float *static_ws, size_t s
     // workgroups aimed at: two per compute unit where the tiles fill less than half the chip (GPT-2 / Llama
     // prefill 1.47 / 3.29 -> 1.44 / 3.18 ms against 1.5; three per unit: 1.55 / 3.18), else 1.5 (a 1024^3
     // product, one tile per unit, loses 10-30 % when it is split in two)
-    int ks = (int)((tiles * 2 <= cus ? cus * 2 : cus * 3 / 2) / tiles);
+    // (the 512-thread workgroups of k_gemm_qpc sit one to a compute unit: aim at one each)
+    int ks = quant ? (int)(cus / tiles) : (int)((tiles * 2 <= cus ? cus * 2 : cus * 3 / 2) / tiles);
     if (ks > nsteps / 6) ks = nsteps / 6;
     if (ks > 16) ks = 16;
     if (ks > 1) {
@@ -835,7 +899,7 @@ int launch_gemm(GemmArgs a, int bmode, int precision, float *static_ws, size_t s
     }
   } else if (quant) {
     const int npa = precision == GEMM_BF16X6 ? 3 : precision == GEMM_BF16X3 ? 2 : 1;
-#define QG(WT, NPA, MB) hipLaunchKernelGGL((k_gemm_q<WT, NPA, MB>), grid, block, 0, st, a)
+#define QG(WT, NPA, MB) hipLaunchKernelGGL((k_gemm_qpc<WT, NPA>), grid, dim3(512), 0, st, a)
 #define QSEL(WT)                  \
   if (npa == 3) QG(WT, 3, 1);     \
   else if (npa == 2) QG(WT, 2, 1); \

@@ -21,6 +21,8 @@
 // Weights of the two "column" Linears are re-laid at load so that a workgroup's share is contiguous.
 #include <stdlib.h>
 
+#include <type_traits>
+
 #include "common.h"
 #include "gemv_kernels.h"
 #include "decode_fused.h"
@@ -233,27 +235,30 @@ void k_dec_attn_proj(DecAttnArgs a) {
   }
   float m = -INFINITY, lsum = 0.0f;
   float acc[4] = {0.f, 0.f, 0.f, 0.f};
-  for (int t0 = 0; t0 < T; t0 += TILE) {
-    if (t0 + wv * KPT * KPW >= T) break;  // nothing left for this wavefront (uniform)
-    float4 kr[KPT], vr[KPT];
+  // One tile = NP key passes per wavefront, all requested together: wavefront wv owns keys t0 + (wv*NP + u)*KPW + g.
+  // Up to 16*KPW*KPT keys that is KPT passes; a longer context takes tiles of twice as many passes, so that
+  // positions up to twice as far still cost ONE memory round trip instead of two.
+  auto tile = [&](auto np_tag, int t0) {
+    constexpr int NP = decltype(np_tag)::value;
+    float4 kr[NP], vr[NP];
 #pragma unroll
-    for (int u = 0; u < KPT; u++) {
-      const int j = t0 + (wv * KPT + u) * KPW + g;
+    for (int u = 0; u < NP; u++) {
+      const int j = t0 + (wv * NP + u) * KPW + g;
       const unsigned jj = (unsigned)min(j, T - 1);  // clamped: masked below, never outside the cache
       kr[u] = kp[jj * kvs4];
       vr[u] = vp[jj * kvs4];
     }
-    float sc[KPT];
+    float sc[NP];
     float tmax = -INFINITY;
 #pragma unroll
-    for (int u = 0; u < KPT; u++) {
+    for (int u = 0; u < NP; u++) {
       float d = q4.x * kr[u].x;
       d = fmaf(q4.y, kr[u].y, d);
       d = fmaf(q4.z, kr[u].z, d);
       d = fmaf(q4.w, kr[u].w, d);
 #pragma unroll
       for (int o = LPK / 2; o > 0; o >>= 1) d += __shfl_xor(d, o, 64);
-      const bool ok = (t0 + (wv * KPT + u) * KPW + g) < T;
+      const bool ok = (t0 + (wv * NP + u) * KPW + g) < T;
       sc[u] = ok ? d * scale : -INFINITY;
       tmax = fmaxf(tmax, sc[u]);
     }
@@ -265,7 +270,7 @@ void k_dec_attn_proj(DecAttnArgs a) {
 #pragma unroll
     for (int k2 = 0; k2 < 4; k2++) acc[k2] *= corr;
 #pragma unroll
-    for (int u = 0; u < KPT; u++) {
+    for (int u = 0; u < NP; u++) {
       const float p = ct_exp(sc[u] - m_new);
       psum += p;
       acc[0] = fmaf(p, vr[u].x, acc[0]);
@@ -277,6 +282,14 @@ void k_dec_attn_proj(DecAttnArgs a) {
     for (int o = LPK; o < 64; o <<= 1) psum += __shfl_xor(psum, o, 64);
     lsum = lsum * corr + psum;
     m = m_new;
+  };
+  if (T <= TILE) {
+    if (wv * KPT * KPW < T) tile(std::integral_constant<int, KPT>(), 0);  // (uniform per wavefront)
+  } else {
+    for (int t0 = 0; t0 < T; t0 += 2 * TILE) {
+      if (t0 + wv * 2 * KPT * KPW >= T) break;  // nothing left for this wavefront (uniform)
+      tile(std::integral_constant<int, 2 * KPT>(), t0);
+    }
   }
 #pragma unroll
   for (int o = LPK; o < 64; o <<= 1) {

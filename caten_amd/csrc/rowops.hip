@@ -7,6 +7,7 @@
 // once; the reductions are 64-lane shuffles, no LDS.  Rows longer than
 // 64*4*8 = 2048 floats fall back to one 256-thread block per row that re-reads
 // the row through L2.
+#include <type_traits>
 #include "common.h"
 
 namespace cthip {
@@ -430,13 +431,15 @@ void k_attn_cached(float *__restrict__ out, const float *__restrict__ q,
   }
   float m = -INFINITY, l = 0.0f;
   float acc[4] = {0.f, 0.f, 0.f, 0.f};
-  // wavefront wv owns keys t0 + (wv*KPT + u)*KPW + g
-  for (int t0 = 0; t0 < T; t0 += TILE) {
-    if (t0 + wv * KPT * KPW >= T) break;  // nothing left for this wavefront (uniform)
-    float4 kr[KPT], vr[KPT];
+  // One tile = NP key passes per wavefront, all requested together: wavefront wv owns keys t0 + (wv*NP + u)*KPW + g.
+  // Up to TILE keys that is KPT passes; a longer context takes tiles of twice as many passes, so that positions up
+  // to twice as far still cost one memory round trip instead of two.
+  auto tile = [&](auto np_tag, int t0) {
+    constexpr int NP = decltype(np_tag)::value;
+    float4 kr[NP], vr[NP];
 #pragma unroll
-    for (int u = 0; u < KPT; u++) {
-      const int j = t0 + (wv * KPT + u) * KPW + g;
+    for (int u = 0; u < NP; u++) {
+      const int j = t0 + (wv * NP + u) * KPW + g;
       // clamp: masked below, never out of the cache; APPEND: row T-1 comes from the registers
       const unsigned jj = (unsigned)min(j, APPEND ? max(T - 2, 0) : T - 1);
       kr[u] = kp[jj * kvs4];
@@ -446,17 +449,17 @@ void k_attn_cached(float *__restrict__ out, const float *__restrict__ q,
         vr[u] = vn;
       }
     }
-    float sc[KPT];
+    float sc[NP];
     float tmax = -INFINITY;
 #pragma unroll
-    for (int u = 0; u < KPT; u++) {
+    for (int u = 0; u < NP; u++) {
       float d = q4.x * kr[u].x;
       d = fmaf(q4.y, kr[u].y, d);
       d = fmaf(q4.z, kr[u].z, d);
       d = fmaf(q4.w, kr[u].w, d);
 #pragma unroll
       for (int o = LPK / 2; o > 0; o >>= 1) d += __shfl_xor(d, o, 64);
-      const bool ok = (t0 + (wv * KPT + u) * KPW + g) < T;
+      const bool ok = (t0 + (wv * NP + u) * KPW + g) < T;
       sc[u] = ok ? d * scale : -INFINITY;
       tmax = fmaxf(tmax, sc[u]);
     }
@@ -468,7 +471,7 @@ void k_attn_cached(float *__restrict__ out, const float *__restrict__ q,
 #pragma unroll
     for (int k2 = 0; k2 < 4; k2++) acc[k2] *= corr;
 #pragma unroll
-    for (int u = 0; u < KPT; u++) {
+    for (int u = 0; u < NP; u++) {
       const float p = ct_exp(sc[u] - m_new);  // exp2(-inf) = 0 for masked keys
       ps += p;
       acc[0] = fmaf(p, vr[u].x, acc[0]);
@@ -480,6 +483,14 @@ void k_attn_cached(float *__restrict__ out, const float *__restrict__ q,
     for (int o = LPK; o < 64; o <<= 1) ps += __shfl_xor(ps, o, 64);  // every lane of a key holds the same p
     l = l * corr + ps;
     m = m_new;
+  };
+  if (T <= TILE) {
+    if (wv * KPT * KPW < T) tile(std::integral_constant<int, KPT>(), 0);  // (uniform per wavefront)
+  } else {
+    for (int t0 = 0; t0 < T; t0 += 2 * TILE) {
+      if (t0 + wv * 2 * KPT * KPW >= T) break;  // nothing left for this wavefront (uniform)
+      tile(std::integral_constant<int, 2 * KPT>(), t0);
+    }
   }
   // combine the key groups inside the wavefront, then the wavefronts through LDS
 #pragma unroll

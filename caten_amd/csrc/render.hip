@@ -897,7 +897,34 @@ struct KernelRenderer {
         o += pad() + "const int " + b[q].idx + " = (int)(_t % (long long)(" + bs + ")); _t /= (long long)(" + bs + ");\n";
       }
     }
+    // row loops of the wavefront path whose length is only known at run time (from 0, step 1)
+    std::map<int, bool> dyn_rows;
+    std::string dyn_cond, dyn_nonempty;
+    bool dyn_ok = true;
+    if (wave) {
+      for (int pos = lo; pos < hi; pos++) {
+        const BpNode &n = b[pos];
+        if (n.t != BpNode::FOR) continue;
+        double v;
+        const Sx *ub = upper_bound(n);
+        if (!ub || const_value(*ub, v) || !is_zero(n.upfrom)) continue;
+        bool inner = false;  // only loops directly inside the row (depth 0 of the body)
+        int d = 0;
+        for (int q = lo; q < pos; q++) d += b[q].t == BpNode::FOR ? 1 : b[q].t == BpNode::ENDFOR ? -1 : 0;
+        inner = d == 0;
+        if (!inner) continue;
+        dyn_rows[pos] = true;
+        const std::string c = "(" + R.expr(*ub, "int64") + ") <= 2048", c0 = "(" + R.expr(*ub, "int64") + ") > 0";
+        if (dyn_cond.find(c) == std::string::npos) dyn_cond += std::string(dyn_cond.empty() ? "" : " && ") + c;
+        if (dyn_nonempty.find(c0) == std::string::npos) dyn_nonempty += std::string(dyn_nonempty.empty() ? "" : " && ") + c0;
+      }
+    }
+    // bounded: row loops of dynamic length are emitted as 32 counted, unrolled, guarded passes (the caller has
+    // checked at run time that the row has at most 64 * 32 elements), so that, as for a static row, the loops
+    // over the same row can share their loads and the row is read once
+    auto emit_body = [&](int bounded) {  // 0: lane-strided loops; N: dynamic rows as N counted passes
     int depth = 0;
+    std::string guard;  // inside a counted pass of a dynamic row: the name of its "this element exists" flag
     std::vector<std::string> closers;
     for (int pos = lo; pos < hi; pos++) {
       const BpNode &n = b[pos];
@@ -919,6 +946,17 @@ struct KernelRenderer {
               done = true;
             }
           }
+          if (!done && bounded && dyn_rows.count(pos)) {
+            // every pass reads unconditionally (the index is clamped to the row's last element) and only its
+            // effects are guarded: the loads of the loops over one row are then the same expressions and are shared
+            const std::string ub_s = R.expr(*upper_bound(n), "int64");
+            o += pad() + "#pragma unroll\n";
+            o += pad() + "for (int " + n.idx + "_i=0; " + n.idx + "_i<" + std::to_string(bounded) + "; " + n.idx + "_i++) { const bool " + n.idx +
+                 "_ok=_lane+64*" + n.idx + "_i<(" + ub_s + "); const int " + n.idx + "=" + n.idx + "_ok ? _lane+64*" + n.idx + "_i : (int)(" + ub_s + ")-1;\n";
+            closers.push_back("}");
+            guard = n.idx + "_ok";
+            done = true;
+          }
           if (!done) {
             o += pad() + "for (int " + n.idx + "=(" + R.expr(n.upfrom, "int64") + ")+_lane; " + R.expr(n.below, "int64") + "; " + n.idx + "+=64) {\n";
             closers.push_back("}");
@@ -933,6 +971,7 @@ struct KernelRenderer {
       } else if (n.t == BpNode::ENDFOR) {
         indent -= 2;
         depth--;
+        if (depth == 0) guard.clear();
         o += pad() + closers.back() + "\n";
         closers.pop_back();
         if (wave && wave_red.count(pos))
@@ -951,8 +990,42 @@ struct KernelRenderer {
         for (const Sx &w : n.writes)
           if (!locals.count(ref_name(w))) global_write = true;
         if (wave && depth == 0 && !n.declare && global_write) stmt = "if (_lane == 0) { " + stmt + " }";  // every lane holds the value; one stores it
+        if (depth == 1 && !guard.empty()) {
+          // the value is computed outside the guard, on the clamped index the other loops use, so that it is shared
+          if (global_write && n.writes.size() == 1)
+            stmt = "{ const " + cdtypes().at(n.dtype) + " _w = " + R.expr(n.rhs, n.dtype) + "; if (" + guard + ") { " + lhs + " = _w; } }";
+          else if (global_write) stmt = "if (" + guard + ") { " + stmt + " }";
+          else if (!n.declare && n.writes.size() == 1) stmt = lhs + " = " + guard + " ? (" + R.expr(n.rhs, n.dtype) + ") : " + lhs + ";";
+        }
         o += pad() + stmt + "\n";
       }
+    }
+    };
+    if (dyn_rows.size() < 2) dyn_rows.clear();  // a row that is walked once gains nothing from being held
+    for (const auto &kv : dyn_rows) {            // row loops with nothing but statements inside, and a non-empty row
+      for (int q = kv.first + 1; q < hi && b[q].t != BpNode::ENDFOR; q++)
+        if (b[q].t != BpNode::EXPR || b[q].declare) dyn_ok = false;
+    }
+    if (!dyn_rows.empty() && dyn_ok) {
+      // copies of the body for rows of up to 256 ... 2048 elements (4 ... 32 passes: a pass beyond the row still
+      // computes on the clamped element), then the loops
+      const int passes[6] = {4, 8, 12, 16, 24, 32};
+      for (int k = 0; k < 6; k++) {
+        std::string c = dyn_cond;
+        for (size_t at = c.find("<= 2048"); at != std::string::npos; at = c.find("<= 2048", at + 1)) c.replace(at, 7, "<= " + std::to_string(64 * passes[k]));
+        o += pad() + (k ? "} else if (" : "if (") + dyn_nonempty + " && " + c + ") {\n";
+        indent += 2;
+        emit_body(passes[k]);
+        indent -= 2;
+      }
+      o += pad() + "} else {\n";
+      indent += 2;
+      emit_body(0);
+      indent -= 2;
+      o += pad() + "}\n";
+    } else {
+      dyn_rows.clear();
+      emit_body(0);
     }
     o += "}\n";
     if (!R.err.empty()) return err = R.err, false;

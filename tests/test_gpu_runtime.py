@@ -177,8 +177,9 @@ def test_rendered_rowwise_kernels_match_oracle(oracle):
     rt = ca.HipRuntime()
     r = ca.HipRenderer()
     src = r.render_kernel(item)
-    # rows became wavefronts: the three row loops are strided by the 64 lanes, the two reductions end in a butterfly
-    assert src.count("for (int") == 3 and src.count("+=64") == 3 and "blockIdx.x" in src
+    # rows became wavefronts: the three row loops are strided by the 64 lanes, the two reductions end in a butterfly;
+    # rows of at most 256 ... 2048 elements take copies of the body with 4 ... 32 counted passes
+    assert src.count("for (int") == 21 and src.count("+=64") == 3 and "blockIdx.x" in src and "(n) <= 2048" in src
     assert "m = ct_wave_max_f(m);" in src and "s = ct_wave_add_f(s);" in src
     r.compile_kernel([item])
     rows, n = 300, 77
@@ -245,7 +246,7 @@ def test_rendered_rowwise_kernels_match_oracle(oracle):
     ]}
     r2 = ca.HipRenderer()
     src_ln, src_off = r2.render_kernel(ln), r2.render_kernel(off)
-    assert src_ln.count("+=64") == 3 and "if (_lane == 0) { val_mean[_gid0] = u; }" in src_ln
+    assert src_ln.count("+=64") == 3 and src_ln.count("if (_lane == 0) { val_mean[_gid0] = u; }") == 7
     assert "_lane" not in src_off and "+=64" not in src_off
     r2.compile_kernel([ln, off])
     for rows, n in ((300, 77), (5, 768), (64, 1)):
@@ -293,7 +294,8 @@ def test_rendered_softmax_static_shape(oracle, n):
     transfer_from_array(rt, bx, x)
     item["compiled_object"](None, by, bx)
     got = transfer_into_array(by).reshape(rows, n)
-    assert np.max(np.abs(got - oracle.softmax(x))) < 1e-6
+    # the reference's own softmax tolerance (test-llm.lisp:64-80): the lanes add a 5000-element row in another order
+    assert np.allclose(got, oracle.softmax(x), atol=1e-5, rtol=1e-6)
 
 
 def test_rendered_argmax_with_index_components(oracle):
@@ -573,3 +575,25 @@ def test_backward_item_with_a_first_axis_reduction(m, n):
     want = np.where(y > 0, dy, 0).astype(np.float32)
     assert np.array_equal(dz, want)
     assert np.allclose(db, want.astype(np.float64).sum(0), rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("rows,n", [(300, 77), (4, 256), (4, 257), (7, 512), (7, 513), (6, 768), (6, 769), (9, 1024), (9, 1025),
+                                     (3, 1536), (3, 1537), (5, 2048), (3, 2049), (2, 5000), (64, 1)])
+def test_rendered_softmax_dynamic_rows_short_and_long(oracle, rows, n):
+    """The softmax blueprint RENDERED (routes switched off) with a row length known only at launch: rows of at most
+    256 ... 2048 elements run a copy of the body whose row loops are 4 ... 32 counted passes with clamped,
+    unconditional reads and guarded effects (the row is read once), longer rows the lane-strided loops; all against
+    the oracle, on both sides of every boundary."""
+    import caten_amd as ca
+    from caten_amd import _lib, blueprints as bp
+    print(f"case: rendered dynamic softmax {rows}x{n}", flush=True)
+    lib = _lib.load()
+    x = np.random.default_rng(n).normal(0, 3, (rows, n)).astype(np.float32)
+    _lib.check(lib.cthip_set_option(b"render_routes", 0))
+    try:
+        (got,), prog = _run_item(ca, bp.softmax_rows(), [np.zeros((rows, n), np.float32), rows, n, x])
+        assert prog.last_route == "rendered"
+    finally:
+        _lib.check(lib.cthip_set_option(b"render_routes", 1))
+    # the reference's own softmax tolerance (test-llm.lisp:64-80): the lanes add a 5000-element row in another order
+    assert np.allclose(got, oracle.softmax(x), atol=1e-5, rtol=1e-6)

@@ -30,8 +30,8 @@ struct DecStage {
 
 struct DecQkvArgs {
   DecStage st;
-  const void *wq;            // c_attn quant plane, int8 [3D][D]
-  const unsigned short *wd;  // c_attn scale plane, fp16 [3D][D/32]
+  const void *wq;            // c_attn weights [3D][D] (int8 / fp16 / fp32)
+  const unsigned short *wd;  // Q8_0: scale plane, fp16 [3D][D/32]
   const float *fold_s, *fold_c;  // W.gamma and W.beta + bias
   float *q, *kc, *vc;        // q (D), K / V cache (max_seq, D)
   const int *pos;
@@ -41,8 +41,8 @@ struct DecQkvArgs {
 struct DecAttnArgs {
   const float *q, *kc, *vc;
   const int *pos;
-  const void *pq;            // attn.c_proj by head: int8 [H][D][Dh]
-  const unsigned short *pd;  // fp16 [H][D][Dh/32]
+  const void *pq;            // attn.c_proj by head: [H][D][Dh]
+  const unsigned short *pd;  // Q8_0: fp16 [H][D][Dh/32]
   float *part;               // out: fp32 [H][D], head h's share of the projection
   void *zero;                // cleared here: the MLP accumulators
   int64_t zero_n16;          // ... in 16-byte units
@@ -50,11 +50,11 @@ struct DecAttnArgs {
 
 struct DecMlpArgs {
   DecStage st;
-  const void *wq;            // c_fc quant plane, int8 [F][D]
-  const unsigned short *wd;  // fp16 [F][D/32]
+  const void *wq;            // c_fc weights [F][D]
+  const unsigned short *wd;  // Q8_0: fp16 [F][D/32]
   const float *fold_s, *fold_c;
-  const void *pq;            // mlp.c_proj by 16-column slab: int8 [F/16][D][16]
-  const unsigned short *pd;  // fp16 [F/32][D]
+  const void *pq;            // mlp.c_proj by 16-column slab: [F/16][D][16]
+  const unsigned short *pd;  // Q8_0: fp16 [F/32][D]
   long long *accum;          // [kDecXcds][D]
 };
 
@@ -62,9 +62,9 @@ bool dec_fused_supported(int type_attn, int type_proj, int type_fc, int type_fc2
 int dec_xcd_probe(int *max_id);
 int dec_relay_heads(const WMat *w, int DH, void **pq, void **pd);
 int dec_relay_slabs(const WMat *w, void **pq, void **pd);
-int launch_dec_qkv(const DecQkvArgs &a, bool from_accum);
-int launch_dec_attn_proj(const DecAttnArgs &a, int H, int D, int replicas);
-int launch_dec_mlp(const DecMlpArgs &a, int F, int H);
+int launch_dec_qkv(const DecQkvArgs &a, int type, bool from_accum);
+int launch_dec_attn_proj(const DecAttnArgs &a, int type, int H, int D, int replicas);
+int launch_dec_mlp(const DecMlpArgs &a, int type, int F, int H);
 int launch_dec_sum(const DecStage &s, float *out);
 
 }  // namespace cthip

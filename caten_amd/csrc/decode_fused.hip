@@ -1,5 +1,5 @@
 // Three launches per layer for one decode row of a GPT-2 shaped Transformer (external/llm/layers.lisp:35-71)
-// with Q8_0 weights, instead of five.  A decode step is bound by the number of DEPENDENT launches, not by
+// with Q8_0, fp32 or fp16 weights (template argument TYPE), instead of five.  A decode step is bound by the number of DEPENDENT launches, not by
 // bytes, so two pairs of consecutive Linears are merged around the vector that sits between them:
 //
 //   k_dec_qkv        x -> LayerNorm1 -> c_attn (+bias): q to a buffer, k / v rows into the cache at `pos`
@@ -130,29 +130,59 @@ __device__ __forceinline__ void dec_stage_finish(const DecStage &s, DecStageRegs
   rstd = 1.0f / sqrtf(fmaxf(m2 * inv_n, 0.0f) + s.eps);
 }
 
-// One row of 16 lanes x KC chunks of a Q8_0 plane against the staged vector (D = 256 * KC).
-template <int KC>
-__device__ __forceinline__ float dec_row_dot(const uint4 *w, const unsigned *sc, const float *xs, int l) {
-  float acc = 0.0f;
+// Weight formats of the fused launches: a 16-byte chunk holds XPC weights (Q8_0: 16 int8, fp16: 8, fp32: 4); only
+// Q8_0 has a scale plane (one fp16 per 32 weights).
+template <int TYPE>
+struct DecFmt {
+  static constexpr int XPC = Fmt<TYPE>::XPC;
+  static constexpr bool QUANT = TYPE == CTHIP_Q8_0;
+};
+
+// XPC consecutive floats of a vector in LDS
+template <int XPC>
+__device__ __forceinline__ void lds_floats(const float *p, float *xr) {
 #pragma unroll
-  for (int j = 0; j < KC; j++) {
-    const int c = l + 16 * j;
-    float xr[16];
-#pragma unroll
-    for (int t = 0; t < 4; t++) {
-      const float4 v = *(const float4 *)(xs + c * 16 + 4 * t);
-      xr[4 * t + 0] = v.x;
-      xr[4 * t + 1] = v.y;
-      xr[4 * t + 2] = v.z;
-      xr[4 * t + 3] = v.w;
-    }
-    acc += chunk_dot<CTHIP_Q8_0>(w[j], half_bits_to_float((unsigned short)sc[j]), xr, 0.0f);
+  for (int t = 0; t < XPC / 4; t++) {
+    const float4 v = *(const float4 *)(p + 4 * t);
+    xr[4 * t + 0] = v.x;
+    xr[4 * t + 1] = v.y;
+    xr[4 * t + 2] = v.z;
+    xr[4 * t + 3] = v.w;
   }
-  return row16_sum(acc);
+}
+
+// One row of D = 256 * KC weights against the staged vector: 16 lanes per row, lane l owns chunks l + 16 j.  Two
+// running sums: a chain of dependent FMAs issues at half rate when the SIMD holds one wavefront.
+template <int TYPE, int KC>
+__device__ __forceinline__ float dec_row_dot(const uint4 *w, const unsigned *sc, const float *xs, int l) {
+  constexpr int XPC = DecFmt<TYPE>::XPC, NCL = KC * 16 / XPC;
+  float acc[2] = {0.0f, 0.0f};
+#pragma unroll
+  for (int j = 0; j < NCL; j++) {
+    const int c = l + 16 * j;
+    float xr[XPC];
+    lds_floats<XPC>(xs + c * XPC, xr);
+    acc[j & 1] += chunk_dot<TYPE>(w[j], DecFmt<TYPE>::QUANT ? half_bits_to_float((unsigned short)sc[j]) : 1.0f, xr, 0.0f);
+  }
+  return row16_sum(acc[0] + acc[1]);
+}
+
+// requests of one row's chunks (and block scales) for dec_row_dot
+template <int TYPE, int KC>
+__device__ __forceinline__ void dec_row_request(const void *wq, const unsigned short *wd, int64_t row, int l, uint4 *w, unsigned *sc) {
+  constexpr int XPC = DecFmt<TYPE>::XPC, NCL = KC * 16 / XPC;
+  const uint4 *qp = (const uint4 *)wq + row * (16 * NCL);
+#pragma unroll
+  for (int j = 0; j < NCL; j++) {
+    const int c = l + 16 * j;
+    w[j] = qp[c];
+    if (DecFmt<TYPE>::QUANT) sc[j] = wd[row * (8 * KC) + ((c * XPC) >> 5)];
+    else sc[j] = 0;
+  }
 }
 
 // ---- launch 1: LayerNorm1 folded through c_attn; 16 rows per workgroup ----
-template <int KC, int MODE, int NP>
+template <int TYPE, int KC, int MODE, int NP>
 __global__ __launch_bounds__(256) void k_dec_qkv(DecQkvArgs a) {
   __shared__ __align__(16) float xs[256 * KC];
   __shared__ float red[24];
@@ -166,21 +196,15 @@ __global__ __launch_bounds__(256) void k_dec_qkv(DecQkvArgs a) {
   dec_stage_request(a.st, sr);
   const int posv = a.pos[0];
   __builtin_amdgcn_sched_barrier(0);
-  uint4 w[KC];
-  unsigned sc[KC];
-  const uint4 *qp = (const uint4 *)a.wq + (int64_t)row * (16 * KC);
-  const unsigned short *dp = a.wd + (int64_t)row * (8 * KC);
-#pragma unroll
-  for (int j = 0; j < KC; j++) {
-    const int c = l + 16 * j;
-    w[j] = qp[c];
-    sc[j] = dp[c >> 1];
-  }
+  constexpr int NCL = KC * 16 / DecFmt<TYPE>::XPC;
+  uint4 w[NCL];
+  unsigned sc[NCL];
+  dec_row_request<TYPE, KC>(a.wq, a.wd, row, l, w, sc);
   const float fs = a.fold_s[row], fc = a.fold_c[row];
   __builtin_amdgcn_sched_barrier(0);
   float mu, rstd;
   dec_stage_finish(a.st, sr, xs, red, mu, rstd);
-  const float acc = dec_row_dot<KC>(w, sc, xs, l);
+  const float acc = dec_row_dot<TYPE, KC>(w, sc, xs, l);
   if (l == 0 && row_ok) {
     // rstd * (W.(gamma x) - mu * W.gamma) + (W.beta + bias)  =  W.LayerNorm(x) + bias
     const float v = rstd * (acc - mu * fs) + fc;
@@ -195,11 +219,12 @@ __global__ __launch_bounds__(256) void k_dec_qkv(DecQkvArgs a) {
 // holds four passes of K and V in registers, per-wavefront online softmax, one meeting in LDS.  The head's
 // slab of the projection (D rows x DH columns, contiguous after the re-layout) does not depend on anything
 // computed here and is requested first, so it arrives while the keys are being processed.
-template <int DH, int JR>
+template <int TYPE, int DH, int JR>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)))
 void k_dec_attn_proj(DecAttnArgs a) {
   constexpr int LPK = DH / 4, KPW = 64 / LPK, KPT = 4, NW = 16, TILE = NW * KPW * KPT;
-  constexpr int CPR = DH / 16;          // 16-byte chunks of a projection row inside the slab
+  constexpr int XPC = DecFmt<TYPE>::XPC;
+  constexpr int CPR = DH / XPC;         // 16-byte chunks of a projection row inside the slab
   constexpr int RPP = 1024 / CPR;       // projection rows per pass of the workgroup
   __shared__ float part[NW][DH];
   __shared__ float pm[NW], pl[NW];
@@ -218,7 +243,7 @@ void k_dec_attn_proj(DecAttnArgs a) {
     int r = pr0 + RPP * j;
     r = rbase + (r < rr ? r : rr - 1);
     pw[j] = ((const uint4 *)a.pq)[((int64_t)h * D + r) * CPR + pc];
-    ps[j] = a.pd[((int64_t)h * D + r) * (DH / 32) + (pc >> 1)];
+    ps[j] = DecFmt<TYPE>::QUANT ? a.pd[((int64_t)h * D + r) * (DH / 32) + ((pc * XPC) >> 5)] : 0;
   }
   const int T = a.pos[0] + 1;
   const unsigned kvs4 = (unsigned)(D / 4);
@@ -320,28 +345,22 @@ void k_dec_attn_proj(DecAttnArgs a) {
   }
   __syncthreads();
   // partial projection: row r of the slab times the head's outputs; CPR lanes share a row
-  float xr[16];
-#pragma unroll
-  for (int t = 0; t < 4; t++) {
-    const float4 v = *(const float4 *)(oh + pc * 16 + 4 * t);
-    xr[4 * t + 0] = v.x;
-    xr[4 * t + 1] = v.y;
-    xr[4 * t + 2] = v.z;
-    xr[4 * t + 3] = v.w;
-  }
+  float xr[XPC];
+  lds_floats<XPC>(oh + pc * XPC, xr);
 #pragma unroll
   for (int j = 0; j < JR; j++) {
-    float s = chunk_dot<CTHIP_Q8_0>(pw[j], half_bits_to_float((unsigned short)ps[j]), xr, 0.0f);
-    if (CPR >= 2) s += dpp_f<0xB1>(s);  // quad_perm [1,0,3,2]
-    if (CPR >= 4) s += dpp_f<0x4E>(s);  // quad_perm [2,3,0,1]
-    if (CPR >= 8) s += dpp_f<0x141>(s);  // row_half_mirror
+    float s = chunk_dot<TYPE>(pw[j], DecFmt<TYPE>::QUANT ? half_bits_to_float((unsigned short)ps[j]) : 1.0f, xr, 0.0f);
+    if (CPR >= 2) s += dpp_f<0xB1>(s);    // quad_perm [1,0,3,2]
+    if (CPR >= 4) s += dpp_f<0x4E>(s);    // quad_perm [2,3,0,1]
+    if (CPR >= 8) s += dpp_f<0x141>(s);   // row_half_mirror
+    if (CPR >= 16) s += dpp_f<0x140>(s);  // row_mirror
     const int r = pr0 + RPP * j;
     if (pc == 0 && r < rr) a.part[(int64_t)h * D + rbase + r] = s;
   }
 }
 
 // ---- launch 3: LayerNorm2 folded through 16 rows of c_fc, GELU, their 16 columns of mlp.c_proj ----
-template <int KC, int NP>
+template <int TYPE, int KC, int NP>
 __global__ __launch_bounds__(256) void k_dec_mlp(DecMlpArgs a) {
   __shared__ __align__(16) float xs[256 * KC];
   __shared__ float red[24];
@@ -354,30 +373,25 @@ __global__ __launch_bounds__(256) void k_dec_mlp(DecMlpArgs a) {
   DecStageRegs<1, NP> sr;
   dec_stage_request(a.st, sr);
   __builtin_amdgcn_sched_barrier(0);
-  uint4 w[KC];
-  unsigned sc[KC];
-  const uint4 *qp = (const uint4 *)a.wq + (int64_t)row * (16 * KC);
-  const unsigned short *dp = a.wd + (int64_t)row * (8 * KC);
-#pragma unroll
-  for (int j = 0; j < KC; j++) {
-    const int c = l + 16 * j;
-    w[j] = qp[c];
-    sc[j] = dp[c >> 1];
-  }
+  constexpr int XPC = DecFmt<TYPE>::XPC, NCL = KC * 16 / XPC, SCH = 16 / XPC;
+  uint4 w[NCL];
+  unsigned sc[NCL];
+  dec_row_request<TYPE, KC>(a.wq, a.wd, row, l, w, sc);
   const float fs = a.fold_s[row], fc = a.fold_c[row];
-  // this slab's 16 columns of the second Linear: row r = tid + 256 j (D = 256 * KC)
-  uint4 pw[KC];
+  // this slab's 16 columns (SCH chunks) of the second Linear: row r = tid + 256 j (D = 256 * KC)
+  uint4 pw[KC][SCH];
   unsigned ps[KC];
 #pragma unroll
   for (int j = 0; j < KC; j++) {
     const int r = tid + 256 * j;
-    pw[j] = ((const uint4 *)a.pq)[(int64_t)slab * D + r];
-    ps[j] = a.pd[(int64_t)(slab >> 1) * D + r];
+#pragma unroll
+    for (int k = 0; k < SCH; k++) pw[j][k] = ((const uint4 *)a.pq)[((int64_t)slab * D + r) * SCH + k];
+    ps[j] = DecFmt<TYPE>::QUANT ? a.pd[(int64_t)(slab >> 1) * D + r] : 0;
   }
   __builtin_amdgcn_sched_barrier(0);
   float mu, rstd;
   dec_stage_finish(a.st, sr, xs, red, mu, rstd);
-  const float acc = dec_row_dot<KC>(w, sc, xs, l);
+  const float acc = dec_row_dot<TYPE, KC>(w, sc, xs, l);
   if (l == 0) hs[wv * 4 + g] = ct_gelu(rstd * (acc - mu * fs) + fc);
   __syncthreads();
   float hr[16];
@@ -392,7 +406,10 @@ __global__ __launch_bounds__(256) void k_dec_mlp(DecMlpArgs a) {
   long long *accum = a.accum + (int64_t)xcd_id() * D;
 #pragma unroll
   for (int j = 0; j < KC; j++) {
-    const float s = chunk_dot<CTHIP_Q8_0>(pw[j], half_bits_to_float((unsigned short)ps[j]), hr, 0.0f);
+    float s = 0.0f;
+#pragma unroll
+    for (int k = 0; k < SCH; k++)
+      s += chunk_dot<TYPE>(pw[j][k], DecFmt<TYPE>::QUANT ? half_bits_to_float((unsigned short)ps[j]) : 1.0f, hr + XPC * k, 0.0f);
     // no device-scope bits: the addition happens in this XCD's L2.  (One device-wide accumulator instead of
     // one per XCD costs the 192 workgroups more in contention than the seven arrays cost the reader.)
     __hip_atomic_fetch_add(accum + tid + 256 * j, __float2ll_rn(s * kFixScale), __ATOMIC_RELAXED,
@@ -423,38 +440,27 @@ __global__ __launch_bounds__(256) void k_dec_sum(DecStage s, float *out) {
 }
 
 // ---- re-layout at load ----
-// attn.c_proj (D x D): head h's columns [h*DH, (h+1)*DH) of every row, contiguous: pq[h][r][DH], pd[h][r][DH/32]
-__global__ void k_relay_heads(const uint4 *__restrict__ q, const unsigned short *__restrict__ d, uint4 *__restrict__ pq,
-                              unsigned short *__restrict__ pd, int D, int DH) {
-  const int cpr = DH / 16, spr = DH / 32, H = D / DH;
-  const int64_t nq = (int64_t)H * D * cpr, ns = (int64_t)H * D * spr;
+// A "column" Linear keeps a copy in which a workgroup's share is contiguous.  In 16-byte chunks: in[r][cpr] ->
+// out[g][r][cpg] (group g = head or 16-column slab, cpr = groups * cpg); Q8_0 scales (one per 32 columns):
+// ds[r][spr] -> out[g / gps][r][spg] with gps groups sharing a scale (heads: gps = 1, spg = Dh / 32; slabs of 16
+// columns: gps = 2, spg = 1).
+__global__ void k_relay_chunks(const uint4 *__restrict__ q, uint4 *__restrict__ pq, int rows, int cpr, int cpg) {
+  const int64_t n = (int64_t)rows * cpr;
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < nq) {
-    const int cc = (int)(i % cpr);
-    const int64_t hr = i / cpr;
-    const int r = (int)(hr % D), h = (int)(hr / D);
-    pq[i] = q[(int64_t)r * (D / 16) + h * cpr + cc];
-  }
-  if (i < ns) {
-    const int bb = (int)(i % spr);
-    const int64_t hr = i / spr;
-    const int r = (int)(hr % D), h = (int)(hr / D);
-    pd[i] = d[(int64_t)r * (D / 32) + h * spr + bb];
-  }
+  if (i >= n) return;
+  const int cc = (int)(i % cpg);
+  const int64_t gr = i / cpg;
+  const int r = (int)(gr % rows), g = (int)(gr / rows);
+  pq[i] = q[(int64_t)r * cpr + (int64_t)g * cpg + cc];
 }
-// mlp.c_proj (D x F): 16 columns per slab: pq[s][r] = chunk s of row r, pd[b][r] = scale of 32-block b of row r
-__global__ void k_relay_slabs(const uint4 *__restrict__ q, const unsigned short *__restrict__ d, uint4 *__restrict__ pq,
-                              unsigned short *__restrict__ pd, int D, int F) {
-  const int64_t nq = (int64_t)(F / 16) * D, ns = (int64_t)(F / 32) * D;
+__global__ void k_relay_scales(const unsigned short *__restrict__ d, unsigned short *__restrict__ pd, int rows, int spr, int spg) {
+  const int64_t n = (int64_t)rows * spr;
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < nq) {
-    const int r = (int)(i % D), s = (int)(i / D);
-    pq[i] = q[(int64_t)r * (F / 16) + s];
-  }
-  if (i < ns) {
-    const int r = (int)(i % D), b = (int)(i / D);
-    pd[i] = d[(int64_t)r * (F / 32) + b];
-  }
+  if (i >= n) return;
+  const int bb = (int)(i % spg);
+  const int64_t gr = i / spg;
+  const int r = (int)(gr % rows), g = (int)(gr / rows);
+  pd[i] = d[(int64_t)r * spr + (int64_t)g * spg + bb];
 }
 
 __global__ void k_xcd_probe(int *out) {
@@ -465,8 +471,11 @@ __global__ void k_xcd_probe(int *out) {
 }
 
 // ------------------------------------------------------------------ host side
+static int type_xpc(int type) { return type == CTHIP_Q8_0 ? 16 : type == CTHIP_F16 ? 8 : type == CTHIP_F32 ? 4 : 0; }
+
 bool dec_fused_supported(int type_attn, int type_proj, int type_fc, int type_fc2, int D, int H, int F) {
-  if (type_attn != CTHIP_Q8_0 || type_proj != CTHIP_Q8_0 || type_fc != CTHIP_Q8_0 || type_fc2 != CTHIP_Q8_0) return false;
+  if (type_attn != type_proj || type_attn != type_fc || type_attn != type_fc2) return false;
+  if (type_attn != CTHIP_Q8_0 && type_attn != CTHIP_F32 && type_attn != CTHIP_F16) return false;
   if (D % 256 || D < 256 || D > 1024) return false;
   if (H <= 0 || D % H || D / H != 64) return false;
   if (H != 4 && H != 8 && H != 12 && H != 16) return false;
@@ -486,87 +495,111 @@ int dec_xcd_probe(int *max_id) {
   return rc;
 }
 
-int dec_relay_heads(const WMat *w, int DH, void **pq, void **pd) {
-  const int D = (int)w->rows;
+// group_cols columns per group; scales (Q8_0): groups_per_scale groups share the 32-column block of a scale
+static int relay(const WMat *w, int group_cols, void **pq, void **pd) {
+  const int xpc = type_xpc(w->type);
+  if (!xpc || w->cols % group_cols || group_cols % xpc)
+    return fail(CTHIP_E_BAD_ARG, "decoder: cannot re-lay a %lld x %lld matrix of type %d by groups of %d columns",
+                (long long)w->rows, (long long)w->cols, w->type, group_cols);
+  const int rows = (int)w->rows, cpr = (int)(w->cols / xpc), cpg = group_cols / xpc;
   int rc;
-  if ((rc = cthip_alloc(pq, (size_t)D * D))) return rc;
-  if ((rc = cthip_alloc(pd, (size_t)D * (D / 32) * 2))) return rc;
-  const int64_t n = (int64_t)D * D / 16;
-  hipLaunchKernelGGL(k_relay_heads, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, state().stream, (const uint4 *)w->q,
-                     (const unsigned short *)w->d, (uint4 *)*pq, (unsigned short *)*pd, D, DH);
+  *pd = nullptr;
+  if ((rc = cthip_alloc(pq, (size_t)rows * cpr * 16))) return rc;
+  const int64_t n = (int64_t)rows * cpr;
+  hipLaunchKernelGGL(k_relay_chunks, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, state().stream, (const uint4 *)w->q,
+                     (uint4 *)*pq, rows, cpr, cpg);
   CTHIP_LAUNCH_CHECK();
+  if (w->type == CTHIP_Q8_0) {
+    const int spr = (int)(w->cols / 32), spg = group_cols >= 32 ? group_cols / 32 : 1;
+    if ((rc = cthip_alloc(pd, (size_t)rows * spr * 2))) return rc;
+    const int64_t ns = (int64_t)rows * spr;
+    hipLaunchKernelGGL(k_relay_scales, dim3((unsigned)((ns + 255) / 256)), dim3(256), 0, state().stream,
+                       (const unsigned short *)w->d, (unsigned short *)*pd, rows, spr, spg);
+    CTHIP_LAUNCH_CHECK();
+  }
   return 0;
 }
 
-int dec_relay_slabs(const WMat *w, void **pq, void **pd) {
-  const int D = (int)w->rows, F = (int)w->cols;
-  int rc;
-  if ((rc = cthip_alloc(pq, (size_t)D * F))) return rc;
-  if ((rc = cthip_alloc(pd, (size_t)D * (F / 32) * 2))) return rc;
-  const int64_t n = (int64_t)D * F / 16;
-  hipLaunchKernelGGL(k_relay_slabs, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, state().stream, (const uint4 *)w->q,
-                     (const unsigned short *)w->d, (uint4 *)*pq, (unsigned short *)*pd, D, F);
-  CTHIP_LAUNCH_CHECK();
-  return 0;
-}
+int dec_relay_heads(const WMat *w, int DH, void **pq, void **pd) { return relay(w, DH, pq, pd); }
+int dec_relay_slabs(const WMat *w, void **pq, void **pd) { return relay(w, 16, pq, pd); }
 
-int launch_dec_qkv(const DecQkvArgs &a, bool from_accum) {
+#define DEC_TYPES(GO_T)                 \
+  switch (type) {                       \
+    case CTHIP_Q8_0: GO_T(CTHIP_Q8_0); break; \
+    case CTHIP_F32: GO_T(CTHIP_F32); break;   \
+    case CTHIP_F16: GO_T(CTHIP_F16); break;   \
+    default: return fail(CTHIP_E_BAD_ARG, "decoder: the three-launch layer has no kernels for weight type %d", type); \
+  }
+
+int launch_dec_qkv(const DecQkvArgs &a, int type, bool from_accum) {
   const int D = a.st.D, KC = D / 256;
   if (D % 256 || KC < 1 || KC > 4 || a.rows != 3 * D) return fail(CTHIP_E_BAD_ARG, "decoder: fused qkv launch with D = %d, rows = %d", D, a.rows);
   dim3 grid((a.rows + 15) / 16), block(256);
   hipStream_t st = state().stream;
-#define GO(KC_)                                                                                  \
-  case KC_:                                                                                      \
-    if (from_accum) hipLaunchKernelGGL((k_dec_qkv<KC_, 2, kDecXcds>), grid, block, 0, st, a);    \
-    else hipLaunchKernelGGL((k_dec_qkv<KC_, 0, 1>), grid, block, 0, st, a);                      \
+#define GO(T, KC_)                                                                                  \
+  case KC_:                                                                                         \
+    if (from_accum) hipLaunchKernelGGL((k_dec_qkv<T, KC_, 2, kDecXcds>), grid, block, 0, st, a);    \
+    else hipLaunchKernelGGL((k_dec_qkv<T, KC_, 0, 1>), grid, block, 0, st, a);                      \
     break
-  switch (KC) {
-    GO(1);
-    GO(2);
-    GO(3);
-    GO(4);
+#define GO_T(T) \
+  switch (KC) { \
+    GO(T, 1);   \
+    GO(T, 2);   \
+    GO(T, 3);   \
+    GO(T, 4);   \
   }
+  DEC_TYPES(GO_T)
+#undef GO_T
 #undef GO
   CTHIP_LAUNCH_CHECK();
   return 0;
 }
 
-int launch_dec_attn_proj(const DecAttnArgs &a, int H, int D, int replicas) {
-  if (D != H * 64 || D > 1024 || replicas < 1 || D % replicas)
+int launch_dec_attn_proj(const DecAttnArgs &a, int type, int H, int D, int replicas) {
+  const int xpc = type_xpc(type);
+  if (D != H * 64 || D > 1024 || replicas < 1 || D % replicas || !xpc)
     return fail(CTHIP_E_BAD_ARG, "decoder: fused attention launch with D = %d, H = %d, %d workgroups per head", D, H, replicas);
   dim3 grid(H, replicas), block(1024);
   hipStream_t st = state().stream;
-  // rows of the projection slab per thread: (D / replicas) rows of 4 chunks over 1024 threads
-  switch ((D / replicas + 255) / 256) {
-    case 1: hipLaunchKernelGGL((k_dec_attn_proj<64, 1>), grid, block, 0, st, a); break;
-    case 2: hipLaunchKernelGGL((k_dec_attn_proj<64, 2>), grid, block, 0, st, a); break;
-    case 3: hipLaunchKernelGGL((k_dec_attn_proj<64, 3>), grid, block, 0, st, a); break;
-    default: hipLaunchKernelGGL((k_dec_attn_proj<64, 4>), grid, block, 0, st, a); break;
+  // passes over the slab rows: (D / replicas) rows of 64 / xpc chunks over 1024 threads
+  const int rpp = 1024 / (64 / xpc), jr = (D / replicas + rpp - 1) / rpp;
+  if (jr > 4) return fail(CTHIP_E_BAD_ARG, "decoder: fused attention launch needs %d passes over its slab", jr);
+#define GO_T(T)                                                                              \
+  switch (jr) {                                                                              \
+    case 1: hipLaunchKernelGGL((k_dec_attn_proj<T, 64, 1>), grid, block, 0, st, a); break;   \
+    case 2: hipLaunchKernelGGL((k_dec_attn_proj<T, 64, 2>), grid, block, 0, st, a); break;   \
+    case 3: hipLaunchKernelGGL((k_dec_attn_proj<T, 64, 3>), grid, block, 0, st, a); break;   \
+    default: hipLaunchKernelGGL((k_dec_attn_proj<T, 64, 4>), grid, block, 0, st, a); break;  \
   }
+  DEC_TYPES(GO_T)
+#undef GO_T
   CTHIP_LAUNCH_CHECK();
   return 0;
 }
 
-int launch_dec_mlp(const DecMlpArgs &a, int F, int H) {
+int launch_dec_mlp(const DecMlpArgs &a, int type, int F, int H) {
   const int D = a.st.D, KC = D / 256;
   if (D % 256 || KC < 1 || KC > 4 || F % 32) return fail(CTHIP_E_BAD_ARG, "decoder: fused MLP launch with D = %d, F = %d", D, F);
+  if (H != 4 && H != 8 && H != 12 && H != 16) return fail(CTHIP_E_BAD_ARG, "decoder: fused MLP launch with %d heads", H);
   dim3 grid(F / 16), block(256);
   hipStream_t st = state().stream;
-#define GO2(KC_, NP_) hipLaunchKernelGGL((k_dec_mlp<KC_, NP_>), grid, block, 0, st, a)
-#define GO(KC_)                     \
-  case KC_:                         \
-    if (H == 4) GO2(KC_, 4);        \
-    else if (H == 8) GO2(KC_, 8);   \
-    else if (H == 12) GO2(KC_, 12); \
-    else if (H == 16) GO2(KC_, 16); \
-    else return fail(CTHIP_E_BAD_ARG, "decoder: fused MLP launch with %d heads", H); \
+#define GO2(T, KC_, NP_) hipLaunchKernelGGL((k_dec_mlp<T, KC_, NP_>), grid, block, 0, st, a)
+#define GO(T, KC_)                     \
+  case KC_:                            \
+    if (H == 4) GO2(T, KC_, 4);        \
+    else if (H == 8) GO2(T, KC_, 8);   \
+    else if (H == 12) GO2(T, KC_, 12); \
+    else GO2(T, KC_, 16);              \
     break
-  switch (KC) {
-    GO(1);
-    GO(2);
-    GO(3);
-    GO(4);
+#define GO_T(T) \
+  switch (KC) { \
+    GO(T, 1);   \
+    GO(T, 2);   \
+    GO(T, 3);   \
+    GO(T, 4);   \
   }
+  DEC_TYPES(GO_T)
+#undef GO_T
 #undef GO
 #undef GO2
   CTHIP_LAUNCH_CHECK();

@@ -342,7 +342,7 @@ static int finalize(Decoder *d) {
     d->fused = max_id >= 0 && max_id < kDecXcds;
     for (int l = 0; l < c.n_layers && d->fused; l++) {
       Layer &L = d->layers[l];
-      if (L.attn->type != CTHIP_Q8_0 || L.proj->type != CTHIP_Q8_0 || L.fc->type != CTHIP_Q8_0 || L.fc2->type != CTHIP_Q8_0)
+      if (L.attn->type != d->layers[0].attn->type || L.proj->type != L.attn->type || L.fc->type != L.attn->type || L.fc2->type != L.attn->type)
         d->fused = false;
     }
     if (d->fused) {
@@ -350,7 +350,8 @@ static int finalize(Decoder *d) {
         Layer &L = d->layers[l];
         TRY(dec_relay_heads(L.proj, D / c.n_heads, &L.proj_hq, &L.proj_hd));
         TRY(dec_relay_slabs(L.fc2, &L.fc2_sq, &L.fc2_sd));
-        d->owned.insert(d->owned.end(), {L.proj_hq, L.proj_hd, L.fc2_sq, L.fc2_sd});
+        for (void *p : {L.proj_hq, L.proj_hd, L.fc2_sq, L.fc2_sd})
+          if (p) d->owned.push_back(p);
       }
       TRY(dev_alloc(d, (void **)&d->x2, sizeof(float) * D));
       TRY(dev_alloc(d, (void **)&d->patt, sizeof(float) * (size_t)c.n_heads * D));
@@ -448,7 +449,7 @@ static int queue_step(Decoder *d, bool with_head, bool embed) {
       qa.vc = L.v_cache;
       qa.pos = pos;
       qa.rows = 3 * D;
-      TRY(launch_dec_qkv(qa, l > 0));
+      TRY(launch_dec_qkv(qa, L.attn->type, l > 0));
       DecAttnArgs aa = {};
       aa.q = d->q;
       aa.kc = L.k_cache;
@@ -459,7 +460,7 @@ static int queue_step(Decoder *d, bool with_head, bool embed) {
       aa.part = d->patt;
       aa.zero = d->pmlp;
       aa.zero_n16 = (int64_t)kDecXcds * D * 8 / 16;
-      TRY(launch_dec_attn_proj(aa, c.n_heads, D, replicas));
+      TRY(launch_dec_attn_proj(aa, L.attn->type, c.n_heads, D, replicas));
       DecMlpArgs ma = {};
       ma.st.base = d->x2;
       ma.st.bias = L.proj_b;
@@ -475,7 +476,7 @@ static int queue_step(Decoder *d, bool with_head, bool embed) {
       ma.pq = L.fc2_sq;
       ma.pd = (const unsigned short *)L.fc2_sd;
       ma.accum = d->pmlp;
-      TRY(launch_dec_mlp(ma, F, c.n_heads));
+      TRY(launch_dec_mlp(ma, L.attn->type, F, c.n_heads));
     }
     DecStage fin = {};
     fin.base = d->x;

@@ -134,17 +134,18 @@ def test_streamed_weights_decode_identical(arch):
         assert np.array_equal(a, b)
 
 
-@pytest.mark.parametrize("name,plen", [("gpt2-tiny", 5), ("gpt2-mini", 40)])
-def test_three_launch_layer_equals_five_launch_layer(name, plen):
+@pytest.mark.parametrize("name,plen,kind", [("gpt2-tiny", 5, "q8_0"), ("gpt2-mini", 40, "q8_0"), ("gpt2-tiny", 5, "f32"),
+                                            ("gpt2-mini", 40, "f32"), ("gpt2-tiny", 5, "f16"), ("gpt2-mini", 40, "f16")])
+def test_three_launch_layer_equals_five_launch_layer(name, plen, kind):
     """The decode layer as three launches (attention + its projection, and the whole MLP, one launch each, partial
     vectors added up by the consumer) and as five launches (one per Linear) are the same function: identical greedy
     tokens, logits inside the fp32 band, and -- the per-XCD accumulators being integers -- bit-identical logits
     from one run of the three-launch layer to the next."""
-    print(f"case: three-launch vs five-launch layer {name}", flush=True)
+    print(f"case: three-launch vs five-launch layer {name} {kind}", flush=True)
     from caten_amd import _lib, synth, llm
     lib = _lib.load()
     cfg = synth.GPT2_CONFIGS[name]
-    sd = llm.gpt2_state_dict(synth.gpt2_weights(cfg, seed=11), "q8_0")
+    sd = llm.gpt2_state_dict(synth.gpt2_weights(cfg, seed=11), kind)
     prompt = synth.prompt(cfg["vocab"], plen, seed=11)
     runs = []
     try:

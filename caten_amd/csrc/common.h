@@ -143,8 +143,20 @@ int launch_argmax(int64_t *out, const float *x, int64_t rows, int n, int *tok_ou
 // Linear over m rows on the MFMA path (weights dequantised while staged).  precision: fp32 MFMA operands,
 // operands rounded to bf16, or operands split in two / three bf16 terms (2^-16 / fp32-grade).
 enum { GEMM_FP32 = 0, GEMM_BF16 = 1, GEMM_BF16X3 = 2, GEMM_BF16X6 = 3 };
+// A split-K launch whose reduction the caller takes over (launch_reduce_norm): the raw partial tiles ws[z][m][n]
+struct GemmDeferred {
+  float *ws = nullptr;  // null: the launch did not split K, y is complete
+  int ksplit = 0;
+};
+// defer: non-null = when the launch splits K, leave the partial tiles (bias / residual NOT applied) and hand them
+// over instead of reducing them; the caller releases defer->ws with cthip_free after queuing its reduction
 int launch_linear_gemm(float *y, const WMat *w, const float *x, int m, const float *bias, const float *residual,
-                       int act, int precision);
+                       int act, int precision, GemmDeferred *defer = nullptr);
+bool reduce_norm_supported(int n, int nparts);
+// C (m, n) = sum_z ws[z] + bias + residual for partial tiles handed over through GemmDeferred
+int launch_splitk_reduce(float *C, float *ws, int ksplit, int m, int n, const float *bias, const float *residual);
+int launch_reduce_norm(float *y, float *xout, const float *parts, int nparts, int64_t part_stride, const float *bias,
+                       const float *resid, const float *g, const float *b, float eps, int64_t rows, int n, bool rms);
 // takes the device address of the static split-K scratch of cthip_matmul_noalloc (once per device, that device current)
 int matmul_scratch_init(int device);
 // gate|up rows (m, 2*cols) -> silu(gate)*up (m, cols), or a norm, as a launch of its own

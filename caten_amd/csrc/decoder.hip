@@ -698,24 +698,48 @@ static int prefill(Decoder *d, const int *ids, int s, int n) {
     TRY(cthip_h2d(d->tokpos, tp, sizeof(tp)));
   }
   TRY(launch_embedding(X, d->wte, nullptr, ids_dev, s, V, D, gpt2 ? d->wpe : nullptr, d->tokpos + 1, c.max_seq));
-  for (int l = 0; l < c.n_layers; l++) {
-    Layer &L = d->layers[l];
-    if (gpt2) TRY(cthip_layernorm(XN, X, L.ln1_g, L.ln1_b, c.eps, s, D));
-    else TRY(cthip_rmsnorm(XN, X, L.ln1_g, c.eps, s, D));
-    TRY(launch_linear_gemm(QKV, L.attn, XN, s, L.attn_b, nullptr, CTHIP_ACT_NONE, prec));
-    TRY(launch_qkv_split(Q, L.k_cache, L.v_cache, QKV, s, n, c.n_heads, c.n_kv_heads, Dh, gpt2 ? 0.0f : c.rope_base));
-    TRY(launch_attn(ATT, Q, L.k_cache, L.v_cache, s, n, nullptr, n + s, c.n_heads, c.n_kv_heads, Dh));
-    TRY(launch_linear_gemm(X, L.proj, ATT, s, L.proj_b, X, CTHIP_ACT_NONE, prec));
-    if (gpt2) TRY(cthip_layernorm(XN, X, L.ln2_g, L.ln2_b, c.eps, s, D));
-    else TRY(cthip_rmsnorm(XN, X, L.ln2_g, c.eps, s, D));
-    TRY(launch_linear_gemm(Hb, L.fc, XN, s, L.fc_b, nullptr, gpt2 ? CTHIP_ACT_GELU : CTHIP_ACT_NONE, prec));
-    const float *hin = Hb;
-    if (!gpt2) {
-      if (L.fc_pairs) TRY(launch_swiglu_pairs(G, Hb, (int64_t)s * F));
-      else TRY(launch_prologue(G, Hb, F, CTHIP_PRO_SWIGLU, nullptr, nullptr, 0.0f, 2 * (int64_t)F, s));
-      hin = G;
+  {
+    // A row-split Linear (attention projection, second MLP Linear) whose reduction axis was shared among several
+    // workgroups per tile leaves partial tiles; what follows it is the residual add and the next norm, so one pass
+    // over the rows does all three (launch_reduce_norm) instead of a reduction launch and a norm launch.
+    auto norm = [&](float *y, const float *x, const float *g, const float *b) {
+      return gpt2 ? cthip_layernorm(y, x, g, b, c.eps, s, D) : cthip_rmsnorm(y, x, g, c.eps, s, D);
+    };
+    // X += W.in + bias, then XN = norm(X) with (g, b); g == nullptr: no norm follows (after the last layer)
+    auto linear_residual_norm = [&](const WMat *w, const float *in, const float *bias, const float *g, const float *b) {
+      GemmDeferred df;
+      const bool fuse = g != nullptr && reduce_norm_supported(D, 1);
+      int r = launch_linear_gemm(X, w, in, s, bias, X, CTHIP_ACT_NONE, prec, fuse ? &df : nullptr);
+      if (r) return r;
+      if (df.ws) {
+        if (reduce_norm_supported(D, df.ksplit)) {
+          r = launch_reduce_norm(XN, X, df.ws, df.ksplit, (int64_t)s * D, bias, X, g, b, c.eps, s, D, !gpt2);
+        } else {  // too many shares of too wide a row to hold at once: reduce, then normalise
+          r = launch_splitk_reduce(X, df.ws, df.ksplit, s, D, bias, X);
+          if (!r) r = norm(XN, X, g, b);
+        }
+        const int r2 = cthip_free(df.ws);  // stream-ordered: reused only by later work on this stream
+        return r ? r : r2;
+      }
+      return g ? norm(XN, X, g, b) : 0;
+    };
+    TRY(norm(XN, X, d->layers[0].ln1_g, d->layers[0].ln1_b));
+    for (int l = 0; l < c.n_layers; l++) {
+      Layer &L = d->layers[l];
+      TRY(launch_linear_gemm(QKV, L.attn, XN, s, L.attn_b, nullptr, CTHIP_ACT_NONE, prec));
+      TRY(launch_qkv_split(Q, L.k_cache, L.v_cache, QKV, s, n, c.n_heads, c.n_kv_heads, Dh, gpt2 ? 0.0f : c.rope_base));
+      TRY(launch_attn(ATT, Q, L.k_cache, L.v_cache, s, n, nullptr, n + s, c.n_heads, c.n_kv_heads, Dh));
+      TRY(linear_residual_norm(L.proj, ATT, L.proj_b, L.ln2_g, L.ln2_b));
+      TRY(launch_linear_gemm(Hb, L.fc, XN, s, L.fc_b, nullptr, gpt2 ? CTHIP_ACT_GELU : CTHIP_ACT_NONE, prec));
+      const float *hin = Hb;
+      if (!gpt2) {
+        if (L.fc_pairs) TRY(launch_swiglu_pairs(G, Hb, (int64_t)s * F));
+        else TRY(launch_prologue(G, Hb, F, CTHIP_PRO_SWIGLU, nullptr, nullptr, 0.0f, 2 * (int64_t)F, s));
+        hin = G;
+      }
+      const bool last = l + 1 == c.n_layers;
+      TRY(linear_residual_norm(L.fc2, hin, L.fc2_b, last ? nullptr : d->layers[l + 1].ln1_g, last ? nullptr : d->layers[l + 1].ln1_b));
     }
-    TRY(launch_linear_gemm(X, L.fc2, hin, s, L.fc2_b, X, CTHIP_ACT_NONE, prec));
   }
   // the last row continues through the decode-step head
   TRY(cthip_d2d(d->x, X + (size_t)(s - 1) * D, sizeof(float) * D));

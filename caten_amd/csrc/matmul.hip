@@ -822,7 +822,7 @@ int matmul_scratch_init(int device) {
 
 // static_ws: null = split-K partials come from the caching allocator; otherwise they go to this buffer of
 // static_ws_bytes bytes and nothing is allocated or freed
-int launch_gemm(GemmArgs a, int bmode, int precision, float *static_ws, size_t static_ws_bytes) {
+int launch_gemm(GemmArgs a, int bmode, int precision, float *static_ws, size_t static_ws_bytes, GemmDeferred *defer) {
   if (a.M == 0 || a.N == 0) return 0;
   hipStream_t st = state().stream;
   const int cus = state().compute_units;
@@ -941,6 +941,11 @@ int launch_gemm(GemmArgs a, int bmode, int precision, float *static_ws, size_t s
     if (a.ws && !static_ws) cthip_free(a.ws);
     return fail((int)le, "gemm: launch -> %s", hipGetErrorString(le));
   }
+  if (a.ksplit > 1 && defer && !static_ws && a.act == CTHIP_ACT_NONE) {  // the caller reduces (and owns the tiles)
+    defer->ws = a.ws;
+    defer->ksplit = a.ksplit;
+    return 0;
+  }
   if (a.ksplit > 1) {
     int64_t blocks = ((int64_t)a.M * a.N + 255) / 256;
     if (blocks > 4096) blocks = 4096;
@@ -954,8 +959,25 @@ int launch_gemm(GemmArgs a, int bmode, int precision, float *static_ws, size_t s
 }
 
 // Linear over m rows with packed weights: y (m, rows) = act(x (m, cols) @ W^T + bias) + residual
+int launch_splitk_reduce(float *C, float *ws, int ksplit, int m, int n, const float *bias, const float *residual) {
+  GemmArgs a = {};
+  a.C = C;
+  a.ws = ws;
+  a.ksplit = ksplit;
+  a.M = m;
+  a.N = n;
+  a.bias = bias;
+  a.residual = residual;
+  a.act = CTHIP_ACT_NONE;
+  int64_t blocks = ((int64_t)m * n + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(k_splitk_reduce, dim3((unsigned)blocks), dim3(256), 0, state().stream, a);
+  CTHIP_LAUNCH_CHECK();
+  return 0;
+}
+
 int launch_linear_gemm(float *y, const WMat *w, const float *x, int m, const float *bias, const float *residual,
-                       int act, int precision) {
+                       int act, int precision, GemmDeferred *defer) {
   GemmArgs a = {};
   a.C = y;
   a.A = x;
@@ -968,7 +990,7 @@ int launch_linear_gemm(float *y, const WMat *w, const float *x, int m, const flo
   a.N = (int)w->rows;
   a.K = (int)w->cols;
   a.act = act;
-  return launch_gemm(a, B_WMAT, precision, nullptr, 0);
+  return launch_gemm(a, B_WMAT, precision, nullptr, 0, defer);
 }
 
 // A matmul-shaped Schedule-Item routed here by the renderer: C (M,N) = act(A (M,K) . B + bias), B either (K,N)
@@ -1001,10 +1023,10 @@ int matmul_routed(float *C, const float *A, const float *B, int M, int N, int K,
   if (b_is_nk) {
     a.wq = B;
     a.wtype = CTHIP_F32;
-    return launch_gemm(a, B_WMAT, GEMM_BF16X6, nullptr, 0);
+    return launch_gemm(a, B_WMAT, GEMM_BF16X6, nullptr, 0, nullptr);
   }
   a.B = B;
-  return launch_gemm(a, B_ROWMAJOR, GEMM_BF16X6, nullptr, 0);
+  return launch_gemm(a, B_ROWMAJOR, GEMM_BF16X6, nullptr, 0, nullptr);
 }
 
 }  // namespace cthip
@@ -1025,10 +1047,10 @@ static int matmul_entry(float *C, const float *A, const float *B, int M, int N, 
   a.N = N;
   a.K = K;
   a.act = act;
-  if (!noalloc) return launch_gemm(a, B_ROWMAJOR, precision, nullptr, 0);
+  if (!noalloc) return launch_gemm(a, B_ROWMAJOR, precision, nullptr, 0, nullptr);
   float *ws = g_scratch_ptr[state().device];
   if (!ws) return fail(CTHIP_E_STATE, "cthip_matmul_noalloc: no scratch address for device %d", state().device);
-  return launch_gemm(a, B_ROWMAJOR, precision, ws, kScratchBytes);
+  return launch_gemm(a, B_ROWMAJOR, precision, ws, kScratchBytes, nullptr);
 }
 
 extern "C" int cthip_matmul(float *C, const float *A, const float *B, int M, int N, int K, int act, int precision) {

@@ -123,6 +123,124 @@ __global__ __launch_bounds__(256) void k_rowop(RowArgs a) {
     if (ok[j]) yp[lane + 64 * j] = make_float4(v[j][0], v[j][1], v[j][2], v[j][3]);
 }
 
+// Split-K reduction, residual update and the following norm in one pass over the rows (prompt batches): a row-split
+// Linear whose reduction axis was shared among `nparts` workgroups per tile leaves raw partial tiles; the next thing
+// that happens to its output is the residual add and a LayerNorm / RMSNorm.  One wavefront per row:
+//   x = sum_z parts[z][row] (ascending z, as k_splitk_reduce adds them) + bias + resid   -> xout[row]
+//   y[row] = norm(x)                                                                    (arithmetic of k_rowop)
+struct ReduceNormArgs {
+  float *y, *xout;
+  const float *parts;
+  int nparts;
+  int64_t part_stride;  // floats between two partial matrices
+  const float *bias, *resid, *g, *b;
+  float eps;
+  int64_t rows;
+  int n;
+};
+
+template <int MODE, int VPL, int NZ>
+__global__ __launch_bounds__(256) void k_reduce_norm(ReduceNormArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (row >= a.rows) return;
+  const int n = a.n, n4 = n >> 2;
+  float4 t[VPL][NZ], bs[VPL], rs[VPL], gm[VPL], bt[VPL];
+  bool ok[VPL];
+  // every request first, none behind a branch: shares past nparts repeat share 0 and are dropped
+#pragma unroll
+  for (int j = 0; j < VPL; j++) {
+    const int c = lane + 64 * j;
+    ok[j] = c < n4;
+    const int cc = ok[j] ? c : n4 - 1;
+#pragma unroll
+    for (int z = 0; z < NZ; z++) t[j][z] = ((const float4 *)(a.parts + (int64_t)(z < a.nparts ? z : 0) * a.part_stride + row * n))[cc];
+    bs[j] = ((const float4 *)(a.bias ? a.bias : a.parts))[cc];
+    rs[j] = ((const float4 *)((a.resid ? a.resid : a.parts) + row * n))[cc];
+    gm[j] = ((const float4 *)(a.g ? a.g : a.parts))[cc];
+    bt[j] = ((const float4 *)(a.b ? a.b : a.parts))[cc];
+  }
+  float v[VPL][4];
+#pragma unroll
+  for (int j = 0; j < VPL; j++) {
+    float x[4] = {t[j][0].x, t[j][0].y, t[j][0].z, t[j][0].w};
+#pragma unroll
+    for (int z = 1; z < NZ; z++)
+      if (z < a.nparts) x[0] += t[j][z].x, x[1] += t[j][z].y, x[2] += t[j][z].z, x[3] += t[j][z].w;
+    if (a.bias) x[0] += bs[j].x, x[1] += bs[j].y, x[2] += bs[j].z, x[3] += bs[j].w;
+    if (a.resid) x[0] += rs[j].x, x[1] += rs[j].y, x[2] += rs[j].z, x[3] += rs[j].w;
+    if (ok[j]) ((float4 *)(a.xout + row * n))[lane + 64 * j] = make_float4(x[0], x[1], x[2], x[3]);
+#pragma unroll
+    for (int e = 0; e < 4; e++) v[j][e] = ok[j] ? x[e] : 0.0f;
+  }
+  const float inv_n = 1.0f / (float)n;
+  float mean = 0.0f;
+  if (MODE != ROW_RMSNORM) {
+    float s = 0.0f;
+#pragma unroll
+    for (int j = 0; j < VPL; j++)
+#pragma unroll
+      for (int e = 0; e < 4; e++) s += v[j][e];
+    mean = wave_sum(s) * inv_n;
+  }
+  float q = 0.0f;
+#pragma unroll
+  for (int j = 0; j < VPL; j++)
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      float d = ok[j] ? v[j][e] - mean : 0.0f;
+      v[j][e] = d;
+      q = fmaf(d, d, q);
+    }
+  const float rstd = 1.0f / sqrtf(wave_sum(q) * inv_n + a.eps);
+#pragma unroll
+  for (int j = 0; j < VPL; j++) {
+    if (ok[j]) {
+      const float4 g = a.g ? gm[j] : make_float4(1.f, 1.f, 1.f, 1.f);
+      const float4 b = a.b ? bt[j] : make_float4(0.f, 0.f, 0.f, 0.f);
+      ((float4 *)(a.y + row * n))[lane + 64 * j] = make_float4(v[j][0] * rstd * g.x + b.x, v[j][1] * rstd * g.y + b.y,
+                                                             v[j][2] * rstd * g.z + b.z, v[j][3] * rstd * g.w + b.w);
+    }
+  }
+}
+
+// true if the fused pass can take this shape (otherwise the caller reduces and normalises in two launches)
+bool reduce_norm_supported(int n, int nparts) {
+  if (n % 4 || n > 2048 || nparts < 1 || nparts > 16) return false;
+  // the shares of a row are all requested at once: VPL x NZ float4 per lane have to stay in registers
+  const int vpl = (n / 4 + 63) / 64, nz = nparts <= 2 ? 2 : nparts <= 4 ? 4 : nparts <= 8 ? 8 : 16;
+  return vpl * nz <= 32;
+}
+
+int launch_reduce_norm(float *y, float *xout, const float *parts, int nparts, int64_t part_stride, const float *bias,
+                       const float *resid, const float *g, const float *b, float eps, int64_t rows, int n, bool rms) {
+  if (rows == 0 || n == 0) return 0;
+  if (!reduce_norm_supported(n, nparts)) return fail(CTHIP_E_BAD_ARG, "reduce + norm: rows of %d with %d shares", n, nparts);
+  ReduceNormArgs a = {y, xout, parts, nparts, part_stride, bias, resid, g, b, eps, rows, n};
+  const int vpl = (n / 4 + 63) / 64;
+  dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+  hipStream_t st = state().stream;
+#define RN3(MODE, V, Z) hipLaunchKernelGGL((k_reduce_norm<MODE, V, Z>), grid, block, 0, st, a)
+#define RN2(MODE, V)               \
+  if (nparts <= 2) RN3(MODE, V, 2); \
+  else if (nparts <= 4) RN3(MODE, V, 4); \
+  else if (nparts <= 8) RN3(MODE, V, 8); \
+  else RN3(MODE, V, 16)
+#define RN1(MODE)                  \
+  if (vpl <= 1) { RN2(MODE, 1); }  \
+  else if (vpl <= 2) { RN2(MODE, 2); } \
+  else if (vpl <= 3) { RN2(MODE, 3); } \
+  else if (vpl <= 4) { RN2(MODE, 4); } \
+  else if (vpl <= 6) { RN2(MODE, 6); } \
+  else { RN2(MODE, 8); }
+  if (rms) { RN1(ROW_RMSNORM) } else { RN1(ROW_LAYERNORM) }
+#undef RN1
+#undef RN2
+#undef RN3
+  CTHIP_LAUNCH_CHECK();
+  return 0;
+}
+
 // any n: one block per row, three passes through L2
 template <int MODE>
 __global__ __launch_bounds__(256) void k_rowop_generic(RowArgs a) {

@@ -770,8 +770,8 @@ __global__ __launch_bounds__(256) void k_attn_rows(float *__restrict__ out, cons
 // NW wavefronts take the 32-key tiles of the visible cache round-robin, each with its own online softmax
 // for all 32 rows, and meet once in LDS.  fp32 MFMA operands (v_mfma_f32_32x32x2_f32): the products are the
 // reference's fp32 products, only the summation order differs.
-//   S^T = K Q^T : lane l feeds K[key l%32][d = 2s + l/32] (from a d-major LDS copy of the key tile) and
-//                 Q[query l%32][d = 2s + l/32] (registers), so a lane ends up with 16 keys of ONE query;
+//   S^T = K Q^T : lane l feeds K[key l%32][d = (l/32) DH/2 + s] (from a d-major LDS copy of the key tile) and
+//                 Q[query l%32][the same d] (registers), so a lane ends up with 16 keys of ONE query;
 //   softmax     : per lane over its 16 registers + one exchange with lane l^32;
 //   O^T += V^T P^T : lane l feeds V[key of register s][d = l%32 (+32 per block)] straight from the cache
 //                 (128 contiguous bytes per half-wavefront) and P = its own register s: the output stays
@@ -784,8 +784,11 @@ __global__ __launch_bounds__(64 * NW) void k_attn_mfma(float *__restrict__ out, 
                                                    int start_pos, int H, int Hkv) {
   constexpr int NS = DH / 2;   // k-steps of K Q^T
   constexpr int DB = DH / 32;  // 32-wide blocks of the head dimension
-  __shared__ float Kt[NW][DH][33];        // per wavefront: its key tile, d-major
-  __shared__ float Co[NW][DB * 16][64];   // per wavefront: unnormalised outputs for the final combine
+  // per wavefront: its key tile, d-major; once its tiles are done, its unnormalised outputs for the combine
+  __shared__ union {
+    float Kt[DH][33];
+    float Co[DB * 16][64];
+  } W[NW];
   __shared__ float Cm[NW][64], Cl[NW][64];
   const int h = blockIdx.x, i0 = (gridDim.y - 1 - blockIdx.y) * 32;  // the longest groups are dispatched first
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
@@ -796,16 +799,6 @@ __global__ __launch_bounds__(64 * NW) void k_attn_mfma(float *__restrict__ out, 
   const int Tmax = start_pos + min(i0 + 32, S);
   const int ntiles = (Tmax + 31) / 32;
   const float scale = 1.0f / sqrtf((float)DH);
-  float qreg[NS];
-#pragma unroll
-  for (int s = 0; s < NS; s++) qreg[s] = q[((int64_t)qrow * H + h) * DH + 2 * s + half];
-  float m = -INFINITY, l = 0.0f;
-  v16f_t o[DB];
-#pragma unroll
-  for (int b = 0; b < DB; b++)
-#pragma unroll
-    for (int r = 0; r < 16; r++) o[b][r] = 0.0f;
-
   // the key tile of a pass is requested one pass ahead, its values at the start of the pass: both are in
   // registers by the time the matrix cores need them
   float4 kreg[DH / 8];
@@ -818,16 +811,41 @@ __global__ __launch_bounds__(64 * NW) void k_attn_mfma(float *__restrict__ out, 
     }
   };
   if (wv < ntiles) load_k(wv);
+  // The block's 32 query rows go through LDS (the memory of the key tiles, before they are written): whole
+  // rows in 16-byte pieces, one request per cache line and block.  (Every wavefront fetching its own operand
+  // registers straight from memory asked for each line 128 times: 4 us of a 512-token launch.)
+  constexpr int QP = DH + 4;  // row pitch: 16-byte reads of 8 consecutive rows spread over all banks
+  static_assert(32 * QP * 4 <= sizeof(W), "the query rows fit the key tile memory");
+  float(*Qs)[QP] = reinterpret_cast<float(*)[QP]>(&W[0]);
+  for (int f = tid; f < 8 * DH; f += 64 * NW) {
+    const int row = f / (DH / 4), c4 = f % (DH / 4);
+    *(float4 *)&Qs[row][4 * c4] = *(const float4 *)(q + ((int64_t)min(i0 + row, S - 1) * H + h) * DH + 4 * c4);
+  }
+  __syncthreads();
+  float qreg[NS];  // k-step s of this lane: d = half * NS + s
+#pragma unroll
+  for (int j = 0; j < NS / 4; j++) {
+    const float4 t = *(const float4 *)&Qs[col][half * NS + 4 * j];
+    qreg[4 * j + 0] = t.x, qreg[4 * j + 1] = t.y, qreg[4 * j + 2] = t.z, qreg[4 * j + 3] = t.w;
+  }
+  __syncthreads();  // the key tiles may overwrite the rows now
+  float m = -INFINITY, l = 0.0f;
+  v16f_t o[DB];
+#pragma unroll
+  for (int b = 0; b < DB; b++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) o[b][r] = 0.0f;
+
   for (int t = wv; t < ntiles; t += NW) {
     const int kb = t * 32;
     // the key tile, transposed into LDS
 #pragma unroll
     for (int u = 0; u < DH / 8; u++) {
       const int f = lane + 64 * u, key = f / (DH / 4), d4 = f % (DH / 4);
-      Kt[wv][4 * d4 + 0][key] = kreg[u].x;
-      Kt[wv][4 * d4 + 1][key] = kreg[u].y;
-      Kt[wv][4 * d4 + 2][key] = kreg[u].z;
-      Kt[wv][4 * d4 + 3][key] = kreg[u].w;
+      W[wv].Kt[4 * d4 + 0][key] = kreg[u].x;
+      W[wv].Kt[4 * d4 + 1][key] = kreg[u].y;
+      W[wv].Kt[4 * d4 + 2][key] = kreg[u].z;
+      W[wv].Kt[4 * d4 + 3][key] = kreg[u].w;
     }
     float vreg[DB][16];
 #pragma unroll
@@ -843,7 +861,7 @@ __global__ __launch_bounds__(64 * NW) void k_attn_mfma(float *__restrict__ out, 
 #pragma unroll
     for (int r = 0; r < 16; r++) sacc[r] = 0.0f;
 #pragma unroll
-    for (int s = 0; s < NS; s++) sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(Kt[wv][2 * s + half][col], qreg[s], sacc, 0, 0, 0);
+    for (int s = 0; s < NS; s++) sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(W[wv].Kt[half * NS + s][col], qreg[s], sacc, 0, 0, 0);
     __builtin_amdgcn_wave_barrier();
     // sacc[r] = score of key kb + 8*(r/4) + 4*half + r%4 against query `col`
     float tmax = -INFINITY;
@@ -883,7 +901,7 @@ __global__ __launch_bounds__(64 * NW) void k_attn_mfma(float *__restrict__ out, 
 #pragma unroll
   for (int b = 0; b < DB; b++)
 #pragma unroll
-    for (int r = 0; r < 16; r++) Co[wv][b * 16 + r][lane] = o[b][r];
+    for (int r = 0; r < 16; r++) W[wv].Co[b * 16 + r][lane] = o[b][r];
   __syncthreads();
   float M = Cm[0][lane];
 #pragma unroll
@@ -904,7 +922,7 @@ __global__ __launch_bounds__(64 * NW) void k_attn_mfma(float *__restrict__ out, 
       const int R = wv * RPW + k, b = R >> 4, r = R & 15;
       float v = 0.0f;
 #pragma unroll
-      for (int w = 0; w < NW; w++) v = fmaf(e[w], Co[w][R][lane], v);
+      for (int w = 0; w < NW; w++) v = fmaf(e[w], W[w].Co[R][lane], v);
       orow[32 * b + 8 * (r >> 2) + 4 * half + (r & 3)] = v * inv;
     }
   }

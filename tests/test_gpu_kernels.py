@@ -397,8 +397,13 @@ def test_rope(ops, oracle):
                                              (16, 0, 4, 4, 64), (37, 5, 8, 2, 64), (130, 0, 2, 2, 64), (21, 200, 2, 1, 128),
                                              (19, 3, 2, 2, 32), (512, 0, 2, 2, 64),
                                              # 32 rows and more: the matrix-core kernel (ragged last group, GQA, other head sizes)
-                                             (32, 0, 2, 2, 64), (33, 7, 4, 2, 64), (70, 100, 2, 1, 128), (45, 2, 2, 2, 32)])
+                                             (32, 0, 2, 2, 64), (33, 7, 4, 2, 64), (70, 100, 2, 1, 128), (45, 2, 2, 2, 32),
+                                             # several tiles per wavefront, tiles whose keys some rows do not see
+                                             # (start not a multiple of 32)
+                                             (300, 21, 4, 2, 64), (200, 150, 2, 1, 128), (1100, 0, 1, 1, 32),
+                                             (40, 2100, 2, 1, 64)])
 def test_sdpa_cached(ops, oracle, S, start, H, Hkv, Dh):
+    print(f"case: sdpa_cached S={S} start={start} H={H}/{Hkv} Dh={Dh}", flush=True)
     rng = np.random.default_rng(S + start)
     T = start + S
     maxlen = T + 5

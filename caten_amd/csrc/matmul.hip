@@ -60,9 +60,11 @@ typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
 typedef float v2f __attribute__((ext_vector_type(2)));
 
-__device__ __forceinline__ unsigned pack_bf16(float x0, float x1) {  // round to nearest even, x0 in the low half
-  const unsigned lo = __builtin_bit_cast(unsigned short, (__bf16)x0), hi = __builtin_bit_cast(unsigned short, (__bf16)x1);
-  return lo | (hi << 16);
+// round to nearest even, x0 in the low half: as a vector conversion this is ONE v_cvt_pk_bf16_f32 (two scalar
+// conversions are two of them, each with an idle half, plus a shift and an or)
+__device__ __forceinline__ unsigned pack_bf16(float x0, float x1) {
+  const v2f v = {x0, x1};
+  return __builtin_bit_cast(unsigned, __builtin_convertvector(v, v2bf));
 }
 // 4 consecutive k -> NP planes of 4 bf16: plane 0 = bf16(x), plane p = bf16(what planes 0..p-1 miss)
 template <int NP>
@@ -126,10 +128,10 @@ __device__ __forceinline__ void store_tile(const GemmArgs &a, const float *Cs, i
   float *dst = plain ? a.ws + (int64_t)blockIdx.y * M * N : a.C;
   const bool vec = (N & 3) == 0;
 #pragma unroll
-  for (int j = 0; j < BM * F4 / NT; j++) {
+  for (int j = 0; j < (BM * F4 + NT - 1) / NT; j++) {
     const int f = tid + NT * j, lr = f / F4, c4 = f % F4;
     const int row = m0 + lr, col = n0 + 4 * c4;
-    if (row >= M || col >= N) continue;
+    if (f >= BM * F4 || row >= M || col >= N) continue;
     const float4 v4 = *(const float4 *)(Cs + lr * LDC + 4 * c4);
     float v[4] = {v4.x, v4.y, v4.z, v4.w};
     float *o = dst + (int64_t)row * N + col;
@@ -374,9 +376,9 @@ __global__ __launch_bounds__(256) void k_gemm_split(GemmArgs a) {
 //
 // K is walked in steps of 64 = two quant blocks, with the LDS layout / swizzle / prefetch depth / XCD regions /
 // split-K of k_gemm_split.
-template <int MB>
-struct ARegsQ {  // one K-step of A held by a thread: rows ar + 16 i, i < 4 * MB
-  float4 v[4 * MB];
+template <int NA>
+struct ARegsQ {  // one K-step of A held by a staging thread: NA 16-byte pieces
+  float4 v[NA];
 };
 
 // two small integers (as floats, exact) -> packed bf16 pair, x0 in the low half
@@ -399,13 +401,16 @@ __device__ __forceinline__ unsigned pack_int_bf16(float x0, float x1) {
 // which keeps both halves about equally long and gives the prefill shapes no more workgroups than compute units.
 // Weight bytes become floats with one sign-extending conversion each (sbyteN_f32) and pairs of them bf16 with
 // one byte permute.
+template <int NB>
 struct BRegsQ2 {
-  uint4 v[2];        // rows wr and wr + 64 of the tile
+  uint4 v[NB];       // 16 weights each: units ptid + PT j of the tile's 128 rows x 4 pieces
   unsigned short d;  // fp16 scale bits: row ptid >> 1, block ptid & 1 of the step
 };
 
-template <int WT, int NPA>
-__global__ __launch_bounds__(512) void k_gemm_qpc(GemmArgs a) {
+template <int WT, int NPA, int NPW>
+__global__ __launch_bounds__(256 + 64 * NPW) void k_gemm_qpc(GemmArgs a) {
+  constexpr int PT = 64 * NPW, NT = 256 + PT;  // staging threads, all threads
+  constexpr int NA = 1024 / PT, NB = 512 / PT;  // 16-byte pieces of A / of the weights per staging thread and step
   constexpr int BM = 64, BN = 128, BK = 64, LDK = BK, LDC = BN + 4;
   constexpr int kABytes = 2 * NPA * BM * LDK * 2, kBBytes = 2 * BN * LDK * 2, kCBytes = BM * LDC * 4;
   // the operand buffers; after the last step the same memory holds the output tile for the row-wise stores
@@ -417,8 +422,8 @@ __global__ __launch_bounds__(512) void k_gemm_qpc(GemmArgs a) {
   BsT Bs = (BsT)(smem + kABytes);
   float(*Cs)[LDC] = (float(*)[LDC])smem;
   const int tid = threadIdx.x, lane = tid & 63;
-  const bool producer = tid >= 256;
-  const int ptid = tid & 255;            // staging role: index among the staging threads
+  const bool producer = __builtin_amdgcn_readfirstlane(tid) >= 256;  // uniform over a wavefront, and known to be
+  const int ptid = producer ? tid - 256 : tid;  // staging role: index among the staging threads
   const int wave = (tid >> 6) & 3;       // multiplying role: 2 x 2 wavefronts of 32 x 64
   const int wm = wave >> 1, wn = wave & 1;
   const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
@@ -435,21 +440,24 @@ __global__ __launch_bounds__(512) void k_gemm_qpc(GemmArgs a) {
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[b][r] = 0.0f;
 
-  const int ar = ptid >> 4, akq = ptid & 15;  // A: rows ar + 16 i, k = 4 akq .. +3
-  const int wr = ptid >> 2, wkc = ptid & 3;   // B: weight rows wr and wr + 64, k = 16 wkc .. +15
-  const int sr = ptid >> 1, sb = ptid & 1;    // scales: row sr, quant block sb of the step
+  const int ar = ptid >> 4, akq = ptid & 15;  // A: rows ar + (PT / 16) i, k = 4 akq .. +3
+  const int wr = ptid >> 2, wkc = ptid & 3;   // B: weight rows wr + (PT / 4) j, k = 16 wkc .. +15
+  const int sr = (ptid & 255) >> 1, sb = ptid & 1;  // scales: row sr, quant block sb of the step (first 256 stagers)
+  const bool scaler = ptid < 256;
   const int blocks_per_row = ldk >> 5;
 
-  auto fetch = [&](int k0, ARegsQ<1> &ra, BRegsQ2 &rb) {  // k0 counts from kbeg; requests without branches
+  typedef ARegsQ<NA> ARg;
+  typedef BRegsQ2<NB> BRg;
+  auto fetch = [&](int k0, ARg &ra, BRg &rb) {  // k0 counts from kbeg; requests without branches
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const int row = m0 + ar + 16 * i, k = kbeg + k0 + 4 * akq;
+    for (int i = 0; i < NA; i++) {
+      const int row = m0 + ar + (PT / 16) * i, k = kbeg + k0 + 4 * akq;
       ra.v[i] = load4<true>(a.A + (int64_t)row * ldk + k, row < M ? clamp04(K - k) : 0);
     }
     const int k = kbeg + k0 + 16 * wkc;
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-      const int n = n0 + wr + 64 * j;
+    for (int j = 0; j < NB; j++) {
+      const int n = n0 + wr + (PT / 4) * j;
       const int64_t e = (int64_t)n * ldk + k;
       const uint8_t *q = (const uint8_t *)a.wq + (WT == W_Q8 ? e : ((e >> 5) << 4));
       rb.v[j] = *((n < N && k < K) ? (const uint4 *)q : (const uint4 *)g_zeros);
@@ -457,18 +465,18 @@ __global__ __launch_bounds__(512) void k_gemm_qpc(GemmArgs a) {
     const int ns = n0 + sr, ks = kbeg + k0 + 32 * sb;
     rb.d = *((ns < N && ks < K) ? a.wd + (int64_t)ns * blocks_per_row + (ks >> 5) : (const unsigned short *)g_zeros);
   };
-  auto stage = [&](const ARegsQ<1> &ra, const BRegsQ2 &rb, int buf) {
+  auto stage = [&](const ARg &ra, const BRg &rb, int buf) {
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
+    for (int i = 0; i < NA; i++) {
       const float x[4] = {ra.v[i].x, ra.v[i].y, ra.v[i].z, ra.v[i].w};
       uint2 pl[NPA];
       split4<NPA>(x, pl);
-      const int row = ar + 16 * i;
+      const int row = ar + (PT / 16) * i;
 #pragma unroll
       for (int p = 0; p < NPA; p++) *(uint2 *)&As[buf][p][row][8 * ((akq >> 1) ^ swz(row)) + 4 * (akq & 1)] = pl[p];
     }
 #pragma unroll
-    for (int jr = 0; jr < 2; jr++) {
+    for (int jr = 0; jr < NB; jr++) {
       float q[16];
       const unsigned dw[4] = {rb.v[jr].x, rb.v[jr].y, rb.v[jr].z, rb.v[jr].w};
       if (WT == W_Q8) {
@@ -490,14 +498,14 @@ __global__ __launch_bounds__(512) void k_gemm_qpc(GemmArgs a) {
           q[4 * t + 3] = ubyte3_f32(nb) - 8.0f;
         }
       }
-      const int row = wr + 64 * jr;
+      const int row = wr + (PT / 4) * jr;
 #pragma unroll
       for (int j = 0; j < 2; j++)
         *(uint4 *)&Bs[buf][row][8 * ((2 * wkc + j) ^ swz(row))] =
             make_uint4(pack_int_bf16(q[8 * j + 0], q[8 * j + 1]), pack_int_bf16(q[8 * j + 2], q[8 * j + 3]),
                        pack_int_bf16(q[8 * j + 4], q[8 * j + 5]), pack_int_bf16(q[8 * j + 6], q[8 * j + 7]));
     }
-    Ss[buf][sr][sb] = half_bits_to_float(rb.d);
+    if (scaler) Ss[buf][sr][sb] = half_bits_to_float(rb.d);  // uniform over a wavefront
   };
   auto mma = [&](int buf) {
     const int rowa = 32 * wm + (lane & 31);
@@ -531,19 +539,14 @@ __global__ __launch_bounds__(512) void k_gemm_qpc(GemmArgs a) {
     }
   };
 
-  ARegsQ<1> ra0, ra1, ra2;
-  BRegsQ2 rb0, rb1, rb2;
+  ARg ra0, ra1, ra2;
+  BRg rb0, rb1, rb2;
   const int nsteps = K > kbeg ? (K - kbeg + BK - 1) / BK : 0;
-  // one barrier per step; the branch on the role is uniform over a wavefront
-  auto step = [&](int i, ARegsQ<1> &ran, BRegsQ2 &rbn) {
-    if (producer) {
-      stage(ran, rbn, (i + 1) & 1);
-      fetch((i + 4) * BK, ran, rbn);
-    } else {
-      mma(i & 1);
-    }
-    __syncthreads();
-  };
+  // One barrier per step.  Each role runs its own loop, so the staging loop has no branch around its requests:
+  // with the role tested inside a shared loop the compiler has to assume the path on which a step's requests
+  // were skipped, waits for ALL but the last requests before every use, and the three-steps-ahead prefetch
+  // degenerates into one step ahead (each step then costs a memory round trip).  Every wavefront passes the
+  // same number of barriers on either path.
   if (nsteps > 0) {
     if (producer) {
       fetch(0, ra0, rb0);
@@ -551,16 +554,27 @@ __global__ __launch_bounds__(512) void k_gemm_qpc(GemmArgs a) {
       fetch(2 * BK, ra2, rb2);
       stage(ra0, rb0, 0);
       fetch(3 * BK, ra0, rb0);
+      __syncthreads();
+      auto step = [&](int i, ARg &ran, BRg &rbn) {
+        stage(ran, rbn, (i + 1) & 1);
+        fetch((i + 4) * BK, ran, rbn);
+        __syncthreads();
+      };
+      int i = 0;
+      for (; i + 3 <= nsteps; i += 3) {
+        step(i, ra1, rb1);
+        step(i + 1, ra2, rb2);
+        step(i + 2, ra0, rb0);
+      }
+      if (i < nsteps) step(i, ra1, rb1);
+      if (i + 1 < nsteps) step(i + 1, ra2, rb2);
+    } else {
+      __syncthreads();
+      for (int i = 0; i < nsteps; i++) {
+        mma(i & 1);
+        __syncthreads();
+      }
     }
-    __syncthreads();
-    int i = 0;
-    for (; i + 3 <= nsteps; i += 3) {
-      step(i, ra1, rb1);
-      step(i + 1, ra2, rb2);
-      step(i + 2, ra0, rb0);
-    }
-    if (i < nsteps) step(i, ra1, rb1);
-    if (i + 1 < nsteps) step(i + 1, ra2, rb2);
   }
   // ---- epilogue: acc[b][r] is C[row = 8*(r/4) + 4*(l/32) + r%4][col = l%32] of the wavefront's block b.  The
   // tile goes through LDS (the operand buffers are free after the last barrier) so that all 512 threads store
@@ -573,7 +587,7 @@ __global__ __launch_bounds__(512) void k_gemm_qpc(GemmArgs a) {
         Cs[32 * wm + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)][64 * wn + 32 * b + (lane & 31)] = acc[b][r];
   }
   __syncthreads();
-  store_tile<BM, BN, 512>(a, &Cs[0][0], m0, n0, tid);
+  store_tile<BM, BN, NT>(a, &Cs[0][0], m0, n0, tid);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -899,7 +913,9 @@ int launch_gemm(GemmArgs a, int bmode, int precision, float *static_ws, size_t s
     }
   } else if (quant) {
     const int npa = precision == GEMM_BF16X6 ? 3 : precision == GEMM_BF16X3 ? 2 : 1;
-#define QG(WT, NPA, MB) hipLaunchKernelGGL((k_gemm_qpc<WT, NPA>), grid, dim3(512), 0, st, a)
+#define QG(WT, NPA, MB)                                                                       \
+  if (getenv("QPC_NPW4")) hipLaunchKernelGGL((k_gemm_qpc<WT, NPA, 4>), grid, dim3(512), 0, st, a); \
+  else hipLaunchKernelGGL((k_gemm_qpc<WT, NPA, 8>), grid, dim3(768), 0, st, a)
 #define QSEL(WT)                  \
   if (npa == 3) QG(WT, 3, 1);     \
   else if (npa == 2) QG(WT, 2, 1); \

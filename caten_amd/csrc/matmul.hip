@@ -407,7 +407,11 @@ struct BRegsQ2 {
   unsigned short d;  // fp16 scale bits: row ptid >> 1, block ptid & 1 of the step
 };
 
-template <int WT, int NPA, int NPW>
+// FULL: every tile and every K-step of the launch lies inside the operands and their byte offsets fit 32 bits
+// (the launcher checks).  The requests of a step are then a scalar base, advanced per step on the scalar unit,
+// plus per-thread offsets computed once -- no address arithmetic, bounds tests or selects on the vector unit,
+// which the staging wavefronts share with the scale multiplications of the multiplying ones.
+template <int WT, int NPA, int NPW, bool FULL>
 __global__ __launch_bounds__(256 + 64 * NPW) void k_gemm_qpc(GemmArgs a) {
   constexpr int PT = 64 * NPW, NT = 256 + PT;  // staging threads, all threads
   constexpr int NA = 1024 / PT, NB = 512 / PT;  // 16-byte pieces of A / of the weights per staging thread and step
@@ -445,10 +449,32 @@ __global__ __launch_bounds__(256 + 64 * NPW) void k_gemm_qpc(GemmArgs a) {
   const int sr = (ptid & 255) >> 1, sb = ptid & 1;  // scales: row sr, quant block sb of the step (first 256 stagers)
   const bool scaler = ptid < 256;
   const int blocks_per_row = ldk >> 5;
+  const int nsteps = K > kbeg ? (K - kbeg + BK - 1) / BK : 0;
+  unsigned aoff[NA], boff[NB], soff;  // FULL: byte offsets of this thread's pieces from the step's bases
+#pragma unroll
+  for (int i = 0; i < NA; i++) aoff[i] = 4u * ((unsigned)(m0 + ar + (PT / 16) * i) * (unsigned)ldk + 4u * akq);
+#pragma unroll
+  for (int j = 0; j < NB; j++) {
+    const unsigned e = (unsigned)(n0 + wr + (PT / 4) * j) * (unsigned)ldk;
+    boff[j] = WT == W_Q8 ? e + 16u * wkc : ((e >> 5) << 4) + ((wkc >> 1) << 4);
+  }
+  soff = 2u * ((unsigned)(n0 + sr) * (unsigned)blocks_per_row + sb);
 
   typedef ARegsQ<NA> ARg;
   typedef BRegsQ2<NB> BRg;
   auto fetch = [&](int k0, ARg &ra, BRg &rb) {  // k0 counts from kbeg; requests without branches
+    if constexpr (FULL) {
+      const int kk = kbeg + min(k0, (nsteps - 1) * BK);  // steps past the end ask for the last one again
+      const char *ab = (const char *)(a.A + kk);
+      const char *bb = (const char *)a.wq + (WT == W_Q8 ? kk : ((kk >> 5) << 4));
+      const char *sbase = (const char *)a.wd + ((kk >> 5) << 1);
+#pragma unroll
+      for (int i = 0; i < NA; i++) ra.v[i] = *(const float4 *)(ab + aoff[i]);
+#pragma unroll
+      for (int j = 0; j < NB; j++) rb.v[j] = *(const uint4 *)(bb + boff[j]);
+      rb.d = *(const unsigned short *)(sbase + soff);
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < NA; i++) {
       const int row = m0 + ar + (PT / 16) * i, k = kbeg + k0 + 4 * akq;
@@ -541,7 +567,6 @@ __global__ __launch_bounds__(256 + 64 * NPW) void k_gemm_qpc(GemmArgs a) {
 
   ARg ra0, ra1, ra2;
   BRg rb0, rb1, rb2;
-  const int nsteps = K > kbeg ? (K - kbeg + BK - 1) / BK : 0;
   // One barrier per step.  Each role runs its own loop, so the staging loop has no branch around its requests:
   // with the role tested inside a shared loop the compiler has to assume the path on which a step's requests
   // were skipped, waits for ALL but the last requests before every use, and the three-steps-ahead prefetch
@@ -913,9 +938,12 @@ int launch_gemm(GemmArgs a, int bmode, int precision, float *static_ws, size_t s
     }
   } else if (quant) {
     const int npa = precision == GEMM_BF16X6 ? 3 : precision == GEMM_BF16X3 ? 2 : 1;
-#define QG(WT, NPA, MB)                                                                       \
-  if (getenv("QPC_NPW4")) hipLaunchKernelGGL((k_gemm_qpc<WT, NPA, 4>), grid, dim3(512), 0, st, a); \
-  else hipLaunchKernelGGL((k_gemm_qpc<WT, NPA, 8>), grid, dim3(768), 0, st, a)
+    // whole tiles, whole steps, 32-bit byte offsets: the kernel's addressing without bounds tests
+    const bool full = a.M % 64 == 0 && a.N % 128 == 0 && a.K % 64 == 0 && a.kper % 64 == 0 &&
+                      (int64_t)a.M * a.K * 4 < (1ll << 32) && (int64_t)a.N * a.K < (1ll << 32);
+#define QG(WT, NPA, MB)                                                                    \
+  if (full) hipLaunchKernelGGL((k_gemm_qpc<WT, NPA, 8, true>), grid, dim3(768), 0, st, a); \
+  else hipLaunchKernelGGL((k_gemm_qpc<WT, NPA, 8, false>), grid, dim3(768), 0, st, a)
 #define QSEL(WT)                  \
   if (npa == 3) QG(WT, 3, 1);     \
   else if (npa == 2) QG(WT, 2, 1); \

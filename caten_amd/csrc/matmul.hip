@@ -533,8 +533,32 @@ __global__ __launch_bounds__(256 + 64 * NPW) void k_gemm_qpc(GemmArgs a) {
     }
     if (scaler) Ss[buf][sr][sb] = half_bits_to_float(rb.d);  // uniform over a wavefront
   };
+  // The operand reads of a whole step are issued before its first matrix instruction (left to itself the
+  // compiler puts each read right before its use, and every pair of matrix instructions then waits out an LDS
+  // round trip): the matrix cores start when the first operands arrive and the rest come in behind them.
   auto mma = [&](int buf) {
     const int rowa = 32 * wm + (lane & 31);
+    v8bf av[2][2][NPA], bv[2][2][2];  // [quant block][k-slice][term / accumulator block]
+    float d[2][2];
+#pragma unroll
+    for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+      for (int s2 = 0; s2 < 2; s2++) {
+        const int ch = 4 * kb + 2 * s2 + (lane >> 5);
+#pragma unroll
+        for (int p = 0; p < NPA; p++) av[kb][s2][p] = __builtin_bit_cast(v8bf, *(const uint4 *)&As[buf][p][rowa][8 * (ch ^ swz(rowa))]);
+#pragma unroll
+        for (int b = 0; b < 2; b++) {
+          const int rowb = 64 * wn + 32 * b + (lane & 31);
+          bv[kb][s2][b] = __builtin_bit_cast(v8bf, *(const uint4 *)&Bs[buf][rowb][8 * (ch ^ swz(rowb))]);
+        }
+      }
+#pragma unroll
+    for (int b = 0; b < 2; b++) {
+      const float2 dd = *(const float2 *)&Ss[buf][64 * wn + 32 * b + (lane & 31)][0];  // this lane's output column
+      d[0][b] = dd.x, d[1][b] = dd.y;
+    }
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int kb = 0; kb < 2; kb++) {  // the two quant blocks of the step
       v16f tmp[2];
@@ -543,25 +567,15 @@ __global__ __launch_bounds__(256 + 64 * NPW) void k_gemm_qpc(GemmArgs a) {
 #pragma unroll
         for (int r = 0; r < 16; r++) tmp[b][r] = 0.0f;
 #pragma unroll
-      for (int s2 = 0; s2 < 2; s2++) {
-        const int ch = 4 * kb + 2 * s2 + (lane >> 5);
-        v8bf av[NPA];
+      for (int s2 = 0; s2 < 2; s2++)
 #pragma unroll
-        for (int p = 0; p < NPA; p++) av[p] = __builtin_bit_cast(v8bf, *(const uint4 *)&As[buf][p][rowa][8 * (ch ^ swz(rowa))]);
+        for (int b = 0; b < 2; b++)
 #pragma unroll
-        for (int b = 0; b < 2; b++) {
-          const int rowb = 64 * wn + 32 * b + (lane & 31);
-          const v8bf bv = __builtin_bit_cast(v8bf, *(const uint4 *)&Bs[buf][rowb][8 * (ch ^ swz(rowb))]);
+          for (int p = NPA - 1; p >= 0; p--) tmp[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[kb][s2][p], bv[kb][s2][b], tmp[b], 0, 0, 0);
 #pragma unroll
-          for (int p = NPA - 1; p >= 0; p--) tmp[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[p], bv, tmp[b], 0, 0, 0);
-        }
-      }
+      for (int b = 0; b < 2; b++)
 #pragma unroll
-      for (int b = 0; b < 2; b++) {
-        const float d = Ss[buf][64 * wn + 32 * b + (lane & 31)][kb];  // scale of this lane's output column for this block
-#pragma unroll
-        for (int r = 0; r < 16; r++) acc[b][r] = fmaf(d, tmp[b][r], acc[b][r]);
-      }
+        for (int r = 0; r < 16; r++) acc[b][r] = fmaf(d[kb][b], tmp[b][r], acc[b][r]);
     }
   };
 

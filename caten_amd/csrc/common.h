@@ -2,6 +2,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
+#include <limits.h>
 #include <stdint.h>
 #include <stdio.h>
 #include <string>
@@ -150,8 +151,18 @@ struct GemmDeferred {
 };
 // defer: non-null = when the launch splits K, leave the partial tiles (bias / residual NOT applied) and hand them
 // over instead of reducing them; the caller releases defer->ws with cthip_free after queuing its reduction
+// Output columns routed to up to three destinations (a fused q/k/v projection whose thirds go to the query rows
+// and to the cache rows of the two caches): columns [c0[i], c0[i + 1]) land in dst[i] with row pitch ld[i],
+// first column at offset 0.  c0[0] = 0; every c0 is a multiple of 128 (whole tiles are routed); an unused
+// third part has c0 = INT_MAX.
+struct GemmRoute {
+  float *dst[3];
+  int c0[3];
+  int ld[3];
+};
+// route: non-null = y is ignored, the columns go where the route says; K is not split then.
 int launch_linear_gemm(float *y, const WMat *w, const float *x, int m, const float *bias, const float *residual,
-                       int act, int precision, GemmDeferred *defer = nullptr);
+                       int act, int precision, GemmDeferred *defer = nullptr, const GemmRoute *route = nullptr);
 bool reduce_norm_supported(int n, int nparts);
 // C (m, n) = sum_z ws[z] + bias + residual for partial tiles handed over through GemmDeferred
 int launch_splitk_reduce(float *C, float *ws, int ksplit, int m, int n, const float *bias, const float *residual);

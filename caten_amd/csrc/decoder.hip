@@ -726,8 +726,14 @@ static int prefill(Decoder *d, const int *ids, int s, int n) {
     TRY(norm(XN, X, d->layers[0].ln1_g, d->layers[0].ln1_b));
     for (int l = 0; l < c.n_layers; l++) {
       Layer &L = d->layers[l];
-      TRY(launch_linear_gemm(QKV, L.attn, XN, s, L.attn_b, nullptr, CTHIP_ACT_NONE, prec));
-      TRY(launch_qkv_split(Q, L.k_cache, L.v_cache, QKV, s, n, c.n_heads, c.n_kv_heads, Dh, gpt2 ? 0.0f : c.rope_base));
+      if (gpt2 && D % 128 == 0 && KD % 128 == 0) {
+        // no rotation: the thirds of the fused projection go straight to the query rows and the cache rows
+        const GemmRoute rt = {{Q, L.k_cache + (int64_t)n * KD, L.v_cache + (int64_t)n * KD}, {0, D, D + KD}, {D, KD, KD}};
+        TRY(launch_linear_gemm(nullptr, L.attn, XN, s, L.attn_b, nullptr, CTHIP_ACT_NONE, prec, nullptr, &rt));
+      } else {
+        TRY(launch_linear_gemm(QKV, L.attn, XN, s, L.attn_b, nullptr, CTHIP_ACT_NONE, prec));
+        TRY(launch_qkv_split(Q, L.k_cache, L.v_cache, QKV, s, n, c.n_heads, c.n_kv_heads, Dh, gpt2 ? 0.0f : c.rope_base));
+      }
       TRY(launch_attn(ATT, Q, L.k_cache, L.v_cache, s, n, nullptr, n + s, c.n_heads, c.n_kv_heads, Dh));
       TRY(linear_residual_norm(L.proj, ATT, L.proj_b, L.ln2_g, L.ln2_b));
       TRY(launch_linear_gemm(Hb, L.fc, XN, s, L.fc_b, nullptr, gpt2 ? CTHIP_ACT_GELU : CTHIP_ACT_NONE, prec));

@@ -38,6 +38,8 @@ struct GemmArgs {
   // rm x rn tiles, one per XCD (workgroup i is dispatched to XCD i % 8), so that every L2 holds only
   // its region's rows of A and columns of B
   int tm, tn, rx, rm, rn;
+  int routed;       // 1: whole tiles go to route.dst[...] instead of C (see GemmRoute)
+  GemmRoute route;
 };
 
 // ---------------------------------------------------------------------------------------------
@@ -126,7 +128,12 @@ __device__ __forceinline__ void store_tile(const GemmArgs &a, const float *Cs, i
   const int M = a.M, N = a.N;
   const bool plain = a.ksplit > 1;
   float *dst = plain ? a.ws + (int64_t)blockIdx.y * M * N : a.C;
-  const bool vec = (N & 3) == 0;
+  int ldd = N, cbase = 0;  // row pitch of the destination and the column its first element stands for
+  if (a.routed) {
+    const int part = n0 >= a.route.c0[2] ? 2 : n0 >= a.route.c0[1] ? 1 : 0;  // uniform over the workgroup
+    dst = a.route.dst[part], ldd = a.route.ld[part], cbase = a.route.c0[part];
+  }
+  const bool vec = (N & 3) == 0 && (ldd & 3) == 0;
 #pragma unroll
   for (int j = 0; j < (BM * F4 + NT - 1) / NT; j++) {
     const int f = tid + NT * j, lr = f / F4, c4 = f % F4;
@@ -134,7 +141,7 @@ __device__ __forceinline__ void store_tile(const GemmArgs &a, const float *Cs, i
     if (f >= BM * F4 || row >= M || col >= N) continue;
     const float4 v4 = *(const float4 *)(Cs + lr * LDC + 4 * c4);
     float v[4] = {v4.x, v4.y, v4.z, v4.w};
-    float *o = dst + (int64_t)row * N + col;
+    float *o = dst + (int64_t)row * ldd + (col - cbase);
     if (vec) {
       if (!plain) {
         if (a.bias) {
@@ -919,6 +926,7 @@ int launch_gemm(GemmArgs a, int bmode, int precision, float *static_ws, size_t s
     int ks = quant ? (int)(cus / tiles) : (int)((tiles * 2 <= cus ? cus * 2 : cus * 3 / 2) / tiles);
     if (ks > nsteps / 6) ks = nsteps / 6;
     if (ks > 16) ks = 16;
+    if (a.routed) ks = 1;  // routed tiles are stored by the workgroup that computed them
     if (ks > 1) {
       const int steps_per = (nsteps + ks - 1) / ks;
       a.kper = steps_per * 64;
@@ -1035,7 +1043,7 @@ int launch_splitk_reduce(float *C, float *ws, int ksplit, int m, int n, const fl
 }
 
 int launch_linear_gemm(float *y, const WMat *w, const float *x, int m, const float *bias, const float *residual,
-                       int act, int precision, GemmDeferred *defer) {
+                       int act, int precision, GemmDeferred *defer, const GemmRoute *route) {
   GemmArgs a = {};
   a.C = y;
   a.A = x;
@@ -1048,6 +1056,14 @@ int launch_linear_gemm(float *y, const WMat *w, const float *x, int m, const flo
   a.N = (int)w->rows;
   a.K = (int)w->cols;
   a.act = act;
+  if (route) {
+    for (int i = 0; i < 3; i++)
+      if (route->c0[i] != INT_MAX && (route->c0[i] % 128 != 0 || !route->dst[i] || route->ld[i] <= 0))
+        return fail(CTHIP_E_BAD_ARG, "launch_linear_gemm: route part %d starts at column %d (whole 128-column tiles are routed)", i, route->c0[i]);
+    if (route->c0[0] != 0 || residual) return fail(CTHIP_E_BAD_ARG, "launch_linear_gemm: a route starts at column 0 and takes no residual");
+    a.routed = 1;
+    a.route = *route;
+  }
   return launch_gemm(a, B_WMAT, precision, nullptr, 0, defer);
 }
 

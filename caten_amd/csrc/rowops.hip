@@ -218,7 +218,9 @@ int launch_reduce_norm(float *y, float *xout, const float *parts, int nparts, in
   if (!reduce_norm_supported(n, nparts)) return fail(CTHIP_E_BAD_ARG, "reduce + norm: rows of %d with %d shares", n, nparts);
   ReduceNormArgs a = {y, xout, parts, nparts, part_stride, bias, resid, g, b, eps, rows, n};
   const int vpl = (n / 4 + 63) / 64;
-  dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+  // a row per wavefront; few rows (a prompt) go one to a workgroup so that they spread over the compute units
+  const int wpb = rows <= 4096 ? 1 : 4;
+  dim3 grid((unsigned)((rows + wpb - 1) / wpb)), block(64 * wpb);
   hipStream_t st = state().stream;
 #define RN3(MODE, V, Z) hipLaunchKernelGGL((k_reduce_norm<MODE, V, Z>), grid, block, 0, st, a)
 #define RN2(MODE, V)               \

@@ -170,7 +170,8 @@ __device__ __forceinline__ void store_tile(const GemmArgs &a, const float *Cs, i
 }
 
 template <int BMODE, int NS, bool AL>
-__global__ __launch_bounds__(256) void k_gemm_split(GemmArgs a) {
+__global__ __launch_bounds__(NS == 1 ? 256 : 768) void k_gemm_split(GemmArgs a) {
+  constexpr bool ROLES = NS != 1;  // one bf16 term per operand: too little to multiply per step to pay for the roles
   constexpr int BM = 64, BN = 64, BK = 64, LDK = BK, NP = (NS == 1) ? 1 : (NS == 3) ? 2 : 3;
   constexpr int NSET = 3;  // register sets = K-steps of global loads in flight
   constexpr int kOpBytes = 2 * NP * BM * LDK * 2, kCBytes = BM * (BN + 4) * 4;
@@ -179,8 +180,15 @@ __global__ __launch_bounds__(256) void k_gemm_split(GemmArgs a) {
   typedef unsigned short(*OpT)[NP][BM][LDK];
   OpT As = (OpT)smem, Bs = (OpT)(smem + kOpBytes);
   float *Cs = (float *)smem;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+  // ROLES: twelve wavefronts in three roles, one of each per SIMD: 0..3 multiply the current step out of one LDS
+  // buffer, 4..7 stage the next step's A into the other (and request the step three further on), 8..11 do the same
+  // for B.  Each role runs its own loop (same number of barriers on every path), so a stager's waits count the
+  // younger requests of ITS loop and the conversions run under the other wavefronts' matrix instructions.
+  // Otherwise four wavefronts that each stage, request and multiply in turn.
+  const int ltid = threadIdx.x, lane = ltid & 63;
+  const int role = ROLES ? __builtin_amdgcn_readfirstlane(ltid) >> 8 : 0;  // uniform over a wavefront, and known to be
+  const int tid = ltid & 255;                                  // index within the role
+  const int wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
   const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
   if (local >= a.rm * a.rn) return;
   const int mi = (xcd % a.rx) * a.rm + local % a.rm, ni = (xcd / a.rx) * a.rn + local / a.rm;
@@ -201,8 +209,8 @@ __global__ __launch_bounds__(256) void k_gemm_split(GemmArgs a) {
   const int wr = tid >> 2, wkc = tid & 3;
 
   // requests without branches (see load4): outside the operands they read zeros
-  auto fetch_a = [&](int k0, ARegs &ra) {  // k0 counts from kbeg
-    auto ld = [&](int i) {
+  auto fetch_a = [&](int k0, ARegs &ra) __attribute__((always_inline)) {  // k0 counts from kbeg
+    auto ld = [&](int i) __attribute__((always_inline)) {
       const int row = m0 + ar + 16 * i, k = kbeg + k0 + 4 * akq;
       return load4<AL>(a.A + (int64_t)row * ldk + k, row < M ? clamp04(K - k) : 0);
     };
@@ -211,9 +219,9 @@ __global__ __launch_bounds__(256) void k_gemm_split(GemmArgs a) {
     ra.v2 = ld(2);
     ra.v3 = ld(3);
   };
-  auto fetch_b = [&](int k0, BRegs<BMODE> &rb) {
+  auto fetch_b = [&](int k0, BRegs<BMODE> &rb) __attribute__((always_inline)) {
     if (BMODE == W_ROWMAJOR) {
-      auto ld = [&](int j) {
+      auto ld = [&](int j) __attribute__((always_inline)) {
         const int k = kbeg + k0 + 4 * bkq + j, n = n0 + 4 * bnq;
         const float4 v = load4<AL>(a.B + (int64_t)k * N + n, k < K ? clamp04(N - n) : 0);
         return make_uint4(__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z), __float_as_uint(v.w));
@@ -242,8 +250,8 @@ __global__ __launch_bounds__(256) void k_gemm_split(GemmArgs a) {
       }
     }
   };
-  auto stage_a = [&](const ARegs &ra, int buf) {
-    auto put = [&](int i, const float4 v) {
+  auto stage_a = [&](const ARegs &ra, int buf) __attribute__((always_inline)) {
+    auto put = [&](int i, const float4 v) __attribute__((always_inline)) {
       const float x[4] = {v.x, v.y, v.z, v.w};
       uint2 pl[NP];
       split4<NP>(x, pl);
@@ -256,10 +264,10 @@ __global__ __launch_bounds__(256) void k_gemm_split(GemmArgs a) {
     put(2, ra.v2);
     put(3, ra.v3);
   };
-  auto stage_b = [&](const BRegs<BMODE> &rb, int buf) {
+  auto stage_b = [&](const BRegs<BMODE> &rb, int buf) __attribute__((always_inline)) {
     if (BMODE == W_ROWMAJOR) {
       // column 4 bnq + i gets its 4 consecutive k: a 4x4 transpose in registers
-      auto put = [&](int i, unsigned x0, unsigned x1, unsigned x2, unsigned x3) {
+      auto put = [&](int i, unsigned x0, unsigned x1, unsigned x2, unsigned x3) __attribute__((always_inline)) {
         const float x[4] = {__uint_as_float(x0), __uint_as_float(x1), __uint_as_float(x2), __uint_as_float(x3)};
         uint2 pl[NP];
         split4<NP>(x, pl);
@@ -305,42 +313,48 @@ __global__ __launch_bounds__(256) void k_gemm_split(GemmArgs a) {
       }
     }
   };
-  auto mma = [&](int buf) {
+  // all operand reads of a step are issued before its first matrix instruction: the matrix cores start when the
+  // first operands arrive and the rest come in behind them (read-then-use pairs each wait out an LDS round trip)
+  auto mma = [&](int buf) __attribute__((always_inline)) {
     // 32x32x16: lane l holds A[i = l%32][k = 8*(l/32) .. +7] and B[k = 8*(l/32) .. +7][j = l%32]
+    const int rowa = 32 * wm + (lane & 31), rowb = 32 * wn + (lane & 31);
+    v8bf av[BK / 16][NP], bv[BK / 16][NP];
 #pragma unroll
     for (int s = 0; s < BK / 16; s++) {
-      const int ch = 2 * s + (lane >> 5), rowa = 32 * wm + (lane & 31), rowb = 32 * wn + (lane & 31);
-      v8bf av[NP], bv[NP];
+      const int ch = 2 * s + (lane >> 5);
 #pragma unroll
       for (int p = 0; p < NP; p++) {
-        av[p] = __builtin_bit_cast(v8bf, *(const uint4 *)&As[buf][p][rowa][8 * (ch ^ swz(rowa))]);
-        bv[p] = __builtin_bit_cast(v8bf, *(const uint4 *)&Bs[buf][p][rowb][8 * (ch ^ swz(rowb))]);
+        av[s][p] = __builtin_bit_cast(v8bf, *(const uint4 *)&As[buf][p][rowa][8 * (ch ^ swz(rowa))]);
+        bv[s][p] = __builtin_bit_cast(v8bf, *(const uint4 *)&Bs[buf][p][rowb][8 * (ch ^ swz(rowb))]);
       }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int s = 0; s < BK / 16; s++) {
       // every pair of planes whose product is above 2^-8(NP) of the leading one, smallest first
 #pragma unroll
       for (int t = NP - 1; t >= 0; t--) {
 #pragma unroll
-        for (int p = 0; p <= t; p++) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[p], bv[t - p], acc, 0, 0, 0);
+        for (int p = 0; p <= t; p++) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[s][p], bv[s][t - p], acc, 0, 0, 0);
       }
     }
   };
-
-  ARegs ra0, ra1, ra2;  // separate objects with named members: every set stays in registers
-  BRegs<BMODE> rb0, rb1, rb2;
   const int nsteps = K > kbeg ? (K - kbeg + BK - 1) / BK : 0;
   // step i: LDS buffer i%2 holds it; register set (i+1) % NSET holds step i+1, requested NSET steps ago.
-  // No conditions inside a step (past the last one the requests read zeros and stage them) and no exit
-  // inside the loop: the waits before a set is staged then count on a known number of younger requests.
-  auto step = [&](int i, ARegs &ran, BRegs<BMODE> &rbn) {
-    stage_a(ran, (i + 1) & 1);
-    stage_b(rbn, (i + 1) & 1);
-    fetch_a((i + 1 + NSET) * BK, ran);
-    fetch_b((i + 1 + NSET) * BK, rbn);
-    mma(i & 1);
-    __syncthreads();
-  };
-  static_assert(NSET == 3, "the loop below is unrolled by hand over the register sets");
-  if (nsteps > 0) {  // K = 0 comes without operands
+  // No conditions inside a staging step (past the last one the requests read zeros and stage them) and no exit
+  // inside the loops: the waits before a set is staged then count on a known number of younger requests.
+  static_assert(NSET == 3, "the loops below are unrolled by hand over the register sets");
+  if (nsteps > 0 && !ROLES) {
+    ARegs ra0, ra1, ra2;  // separate objects with named members: every set stays in registers
+    BRegs<BMODE> rb0, rb1, rb2;
+    auto step = [&](int i, ARegs &ran, BRegs<BMODE> &rbn) {
+      stage_a(ran, (i + 1) & 1);
+      stage_b(rbn, (i + 1) & 1);
+      fetch_a((i + 1 + NSET) * BK, ran);
+      fetch_b((i + 1 + NSET) * BK, rbn);
+      mma(i & 1);
+      __syncthreads();
+    };
     fetch_a(0, ra0);
     fetch_b(0, rb0);
     fetch_a(BK, ra1);
@@ -360,14 +374,66 @@ __global__ __launch_bounds__(256) void k_gemm_split(GemmArgs a) {
     }
     if (i < nsteps) step(i, ra1, rb1);
     if (i + 1 < nsteps) step(i + 1, ra2, rb2);
+  } else if (nsteps > 0) {  // K = 0 comes without operands
+    if (role == 0) {
+      __syncthreads();
+      for (int i = 0; i < nsteps; i++) {
+        mma(i & 1);
+        __syncthreads();
+      }
+    } else if (role == 1) {
+      ARegs ra0, ra1, ra2;  // separate objects with named members: every set stays in registers
+      fetch_a(0, ra0);
+      fetch_a(BK, ra1);
+      fetch_a(2 * BK, ra2);
+      stage_a(ra0, 0);
+      fetch_a(3 * BK, ra0);
+      __syncthreads();
+      auto step = [&](int i, ARegs &ran) __attribute__((always_inline)) {
+        stage_a(ran, (i + 1) & 1);
+        fetch_a((i + 1 + NSET) * BK, ran);
+        __syncthreads();
+      };
+      int i = 0;
+      for (; i + NSET <= nsteps; i += NSET) {
+        step(i, ra1);
+        step(i + 1, ra2);
+        step(i + 2, ra0);
+      }
+      if (i < nsteps) step(i, ra1);
+      if (i + 1 < nsteps) step(i + 1, ra2);
+    } else {
+      BRegs<BMODE> rb0, rb1, rb2;
+      fetch_b(0, rb0);
+      fetch_b(BK, rb1);
+      fetch_b(2 * BK, rb2);
+      stage_b(rb0, 0);
+      fetch_b(3 * BK, rb0);
+      __syncthreads();
+      auto step = [&](int i, BRegs<BMODE> &rbn) __attribute__((always_inline)) {
+        stage_b(rbn, (i + 1) & 1);
+        fetch_b((i + 1 + NSET) * BK, rbn);
+        __syncthreads();
+      };
+      int i = 0;
+      for (; i + NSET <= nsteps; i += NSET) {
+        step(i, rb1);
+        step(i + 1, rb2);
+        step(i + 2, rb0);
+      }
+      if (i < nsteps) step(i, rb1);
+      if (i + 1 < nsteps) step(i + 1, rb2);
+    }
   }
   // ---- epilogue: acc[r] is C[row = 8*(r/4) + 4*(l/32) + r%4][col = l%32] of the 32x32 sub-tile ----
   // (the last step ended with a barrier: nobody reads the operand buffers any more)
+  if (role == 0) {
 #pragma unroll
-  for (int r = 0; r < 16; r++)
-    Cs[(32 * wm + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * (BN + 4) + 32 * wn + (lane & 31)] = acc[r];
+    for (int r = 0; r < 16; r++)
+      Cs[(32 * wm + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * (BN + 4) + 32 * wn + (lane & 31)] = acc[r];
+  }
   __syncthreads();
-  store_tile<BM, BN, 256>(a, Cs, m0, n0, tid);
+  store_tile<BM, BN, ROLES ? 768 : 256>(a, Cs, m0, n0, ltid);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -981,9 +1047,9 @@ int launch_gemm(GemmArgs a, int bmode, int precision, float *static_ws, size_t s
     int wm = W_ROWMAJOR;
     if (bmode == B_WMAT) wm = a.wtype == CTHIP_F16 ? W_F16 : W_F32;
 #define SPLIT3(MODE, AL)                                                                                      \
-  if (precision == GEMM_BF16X6) hipLaunchKernelGGL((k_gemm_split<MODE, 6, AL>), grid, block, 0, st, a);      \
-  else if (precision == GEMM_BF16X3) hipLaunchKernelGGL((k_gemm_split<MODE, 3, AL>), grid, block, 0, st, a); \
-  else hipLaunchKernelGGL((k_gemm_split<MODE, 1, AL>), grid, block, 0, st, a)
+  if (precision == GEMM_BF16X6) hipLaunchKernelGGL((k_gemm_split<MODE, 6, AL>), grid, dim3(768), 0, st, a);      \
+  else if (precision == GEMM_BF16X3) hipLaunchKernelGGL((k_gemm_split<MODE, 3, AL>), grid, dim3(768), 0, st, a); \
+  else hipLaunchKernelGGL((k_gemm_split<MODE, 1, AL>), grid, dim3(256), 0, st, a)
 #define SPLIT(MODE)      \
   case MODE:             \
     if (al) {            \

@@ -54,6 +54,83 @@ def softmax_rows(name: str = "fused_softmax", rows: int | None = None, n: int | 
     ]}
 
 
+def _neg(a):
+    return {"op": "NEG", "args": [a]}
+
+
+def _rstd(q, N, eps):
+    """1 / sqrt(q / n + eps), the division spelled recip(cast(n)) as the simplifier leaves it"""
+    n = {"op": "CAST", "dtype": "float32", "args": [N]} if isinstance(N, str) else float(N)
+    return {"op": "RECIP", "args": [{"op": "SQRT", "args": [_add(_mul(q, {"op": "RECIP", "args": [n]}), eps)]}]}
+
+
+def layernorm_rows(name: str = "fused_layernorm", affine: bool = True, eps: float = 1e-5, rows: int | None = None,
+                   n: int | None = None) -> dict:
+    """LayerNorm over the last axis of (rows, n) as one kernel (nn/normalization.lisp:39-58): the mean, the biased
+    variance of the centred row, then (x - mean) * rstd [* gamma + beta].  Arguments: val_y, [rows, n,] val_x
+    [, val_g, val_b]."""
+    static = rows is not None and n is not None
+    R, N = (rows, n) if static else ("rows", "n")
+    idx = _add(_mul(N, "_gid0"), "_gid1")
+    xi = _A("val_x", idx)
+    nf = {"op": "CAST", "dtype": "float32", "args": [N]} if not static else float(N)
+    loop = {"type": "FOR", "idx": "_gid1", "upfrom": 0, "below": _lt("_gid1", N), "by": 1}
+    end = {"type": "ENDFOR", "idx": "_gid1"}
+    shapes = [] if static else [_glob("rows", "shape", 0, "int64"), _glob("n", "shape", 0, "int64")]
+    params = [_glob("val_g", "input", 1), _glob("val_b", "input", 1)] if affine else []
+    centred = _add(xi, _neg("u"))
+    y = _mul(centred, "r")
+    if affine:
+        y = _add(_mul(y, _A("val_g", "_gid1")), _A("val_b", "_gid1"))
+    return {"name": name, "blueprint": [
+        _glob("val_y", "output", 2), *shapes, _glob("val_x", "input", 2), *params,
+        {"type": "FOR", "idx": "_gid0", "upfrom": 0, "below": _lt("_gid0", R), "by": 1},
+        {"type": "EXPR", "writes": [_A("s", None)], "expr": 0.0, "declare_type": True, "dtype": "float32"},
+        dict(loop),
+        {"type": "EXPR", "writes": [_A("s", None)], "expr": _add("s", xi), "dtype": "float32", "reduction": True},
+        dict(end),
+        {"type": "EXPR", "writes": [_A("u", None)], "expr": _mul("s", {"op": "RECIP", "args": [nf]}), "declare_type": True, "dtype": "float32"},
+        {"type": "EXPR", "writes": [_A("q", None)], "expr": 0.0, "declare_type": True, "dtype": "float32"},
+        dict(loop),
+        {"type": "EXPR", "writes": [_A("q", None)], "expr": _add("q", _mul(centred, centred)), "dtype": "float32", "reduction": True},
+        dict(end),
+        {"type": "EXPR", "writes": [_A("r", None)], "expr": _rstd("q", N, eps), "declare_type": True, "dtype": "float32"},
+        dict(loop),
+        {"type": "EXPR", "writes": [_A("val_y", idx)], "expr": y, "dtype": "float32"},
+        dict(end),
+        {"type": "ENDFOR", "idx": "_gid0"},
+    ]}
+
+
+def rmsnorm_rows(name: str = "fused_rmsnorm", weight: bool = True, eps: float = 1e-5, rows: int | None = None,
+                 n: int | None = None) -> dict:
+    """RMSNorm over the last axis of (rows, n) (nn/normalization.lisp:78-92): x / sqrt(mean(x^2) + eps) [* w].
+    Arguments: val_y, [rows, n,] val_x [, val_w]."""
+    static = rows is not None and n is not None
+    R, N = (rows, n) if static else ("rows", "n")
+    idx = _add(_mul(N, "_gid0"), "_gid1")
+    xi = _A("val_x", idx)
+    loop = {"type": "FOR", "idx": "_gid1", "upfrom": 0, "below": _lt("_gid1", N), "by": 1}
+    end = {"type": "ENDFOR", "idx": "_gid1"}
+    shapes = [] if static else [_glob("rows", "shape", 0, "int64"), _glob("n", "shape", 0, "int64")]
+    y = _mul(xi, "r")
+    if weight:
+        y = _mul(_A("val_w", "_gid1"), y)
+    return {"name": name, "blueprint": [
+        _glob("val_y", "output", 2), *shapes, _glob("val_x", "input", 2), *([_glob("val_w", "input", 1)] if weight else []),
+        {"type": "FOR", "idx": "_gid0", "upfrom": 0, "below": _lt("_gid0", R), "by": 1},
+        {"type": "EXPR", "writes": [_A("q", None)], "expr": 0.0, "declare_type": True, "dtype": "float32"},
+        dict(loop),
+        {"type": "EXPR", "writes": [_A("q", None)], "expr": _add(_mul(xi, xi), "q"), "dtype": "float32", "reduction": True},
+        dict(end),
+        {"type": "EXPR", "writes": [_A("r", None)], "expr": _rstd("q", N, eps), "declare_type": True, "dtype": "float32"},
+        dict(loop),
+        {"type": "EXPR", "writes": [_A("val_y", idx)], "expr": y, "dtype": "float32"},
+        dict(end),
+        {"type": "ENDFOR", "idx": "_gid0"},
+    ]}
+
+
 def matmul(name: str = "fused_matmul", relu: bool = False, bias: bool = False, transposed_b: bool = False) -> dict:
     """(caten (!matmul a b)) with symbolic m n k as the reference lowers it (test-scheduler.lisp:126-135):
     out[n*i+j] = epilogue(sum_k a[kk*i+k] * b[..]); `transposed_b`: b is (n, kk) read through a transposed view,

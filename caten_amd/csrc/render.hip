@@ -37,6 +37,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <algorithm>
 #include <map>
 #include <string>
 #include <vector>
@@ -494,7 +495,7 @@ static bool affine_of(const Sx &index, const std::string idx[3], int nidx, std::
   return v == v0 + 2 * out.c[0] + (nidx > 1 ? 3 * out.c[1] : 0) + (nidx > 2 ? 5 * out.c[2] : 0);
 }
 
-enum RouteKind { R_NONE = 0, R_MATMUL, R_EMBEDDING, R_ARGMAX, R_SOFTMAX };
+enum RouteKind { R_NONE = 0, R_MATMUL, R_EMBEDDING, R_ARGMAX, R_SOFTMAX, R_LAYERNORM, R_RMSNORM };
 struct Route {
   RouteKind kind = R_NONE;
   int out = -1, a = -1, b = -1, bias = -1;  // argument positions
@@ -502,6 +503,7 @@ struct Route {
   std::string idx[3];                       // loop indices: (i, j, k) / (t, d, v) / (row, col)
   Sx bound[3];                              // their upper bounds
   int act = CTHIP_ACT_NONE;
+  double eps = 0.0;                         // LayerNorm / RMSNorm: read off the item by evaluation
 };
 
 struct Program {
@@ -722,6 +724,241 @@ static bool match_softmax(const Item &it, Route &r) {
   if (b[10].writes.size() != 1 || !is_global_aref(it, b[10].writes[0], r.out) || r.out == r.a) return false;
   r.out_idx = b[10].writes[0].v[2];
   r.kind = R_SOFTMAX;
+  return true;
+}
+
+// ---- LayerNorm / RMSNorm rows (source/nn/normalization.lisp:39-58,78-92) ----
+// The scalar statements between the loops (mean = s / n, rstd = 1 / sqrt(q / n + eps)) and the per-element
+// expressions come in whatever spelling the simplifier left (recip of a cast, a folded constant, operands in any
+// order), so they are recognised by VALUE: evaluated on probe numbers and compared with what the norm computes.
+struct Probe {
+  const Item *it = nullptr;
+  std::map<std::string, double> scalars;  // temporaries and by-value arguments
+  std::map<int, double> arrays;           // argument position of a global array -> what any element of it reads as
+  std::map<int, Sx> index;                // the index expression each array was read with
+};
+static bool sx_equal(const Sx &a, const Sx &b) {
+  if (a.kind != b.kind) return false;
+  if (a.kind == Sx::LIST) {
+    if (a.n() != b.n()) return false;
+    for (size_t k = 0; k < a.n(); k++)
+      if (!sx_equal(a.v[k], b.v[k])) return false;
+    return true;
+  }
+  return a.s == b.s && a.i == b.i && a.f == b.f;
+}
+static bool probe(const Sx &e, Probe &p, double &out) {
+  if (e.kind == Sx::INT) { out = (double)e.i; return true; }
+  if (e.kind == Sx::FLT) { out = e.f; return true; }
+  if (e.kind == Sx::SYM) {
+    auto f = p.scalars.find(e.s);
+    if (f == p.scalars.end()) return false;
+    out = f->second;
+    return true;
+  }
+  if (e.kind != Sx::LIST || e.v.empty() || e.v[0].kind != Sx::SYM) return false;
+  const std::string &op = e.v[0].s;
+  if (op == "aref") {
+    if (is_scalar_ref(e)) {
+      auto f = p.scalars.find(ref_name(e));
+      if (f == p.scalars.end()) return false;
+      out = f->second;
+      return true;
+    }
+    int pos;
+    if (!is_global_aref(*p.it, e, pos)) return false;
+    auto f = p.arrays.find(pos);
+    if (f == p.arrays.end()) return false;
+    auto seen = p.index.find(pos);
+    if (seen == p.index.end()) p.index[pos] = e.v[2];
+    else if (!sx_equal(seen->second, e.v[2])) return false;  // one element of each array per iteration
+    out = f->second;
+    return true;
+  }
+  if (op == "const") return e.n() >= 2 && probe(e.v[1], p, out);
+  if (op == "cast") {
+    if (e.n() < 3 || e.v[1].kind != Sx::SYM || e.v[1].s.rfind("float", 0) != 0) return false;
+    return probe(e.v[e.n() - 1], p, out);
+  }
+  std::vector<double> a;
+  for (size_t k = 1; k < e.n(); k++) {
+    double v;
+    if (!probe(e.v[k], p, v)) return false;
+    a.push_back(v);
+  }
+  if (a.empty()) return false;
+  if (op == "add") { out = 0; for (double v : a) out += v; return true; }
+  if (op == "mul") { out = 1; for (double v : a) out *= v; return true; }
+  if (op == "neg" && a.size() == 1) { out = -a[0]; return true; }
+  if (op == "recip" && a.size() == 1 && a[0] != 0) { out = 1.0 / a[0]; return true; }
+  if (op == "sqrt" && a.size() == 1 && a[0] >= 0) { out = sqrt(a[0]); return true; }
+  return false;
+}
+static bool near(double a, double b) { return fabs(a - b) <= 1e-9 * (1.0 + fabs(b)); }
+static void global_arefs(const Item &it, const Sx &e, std::vector<int> &out) {
+  int pos;
+  if (e.call("aref")) {
+    if (is_global_aref(it, e, pos) && std::find(out.begin(), out.end(), pos) == out.end()) out.push_back(pos);
+    return;
+  }
+  if (e.kind == Sx::LIST)
+    for (const Sx &c : e.v) global_arefs(it, c, out);
+}
+// the row length as the probes see it: a literal bound is itself, a symbolic one is bound to 7
+static bool probe_row_length(const Sx &bound, Probe &p, double &n) {
+  if (const_value(bound, n)) return n >= 1;
+  if (bound.kind != Sx::SYM) return false;
+  p.scalars[bound.s] = n = 7.0;
+  return true;
+}
+// rr = 1 / sqrt(q / n + eps): eps is what the statement gives at q = 0, confirmed at a second point
+static bool probe_rstd(const BpNode &st, const std::string &q, Probe &p, double n, double &eps) {
+  if (st.t != BpNode::EXPR || !st.declare || st.writes.size() != 1 || !is_scalar_ref(st.writes[0])) return false;
+  double v0, v1;
+  p.scalars[q] = 0.0;
+  if (!probe(st.rhs, p, v0) || !(v0 > 1.0) || !std::isfinite(v0)) return false;
+  eps = 1.0 / (v0 * v0);
+  p.scalars[q] = 2.0 * n;
+  return probe(st.rhs, p, v1) && near(v1, 1.0 / sqrt(2.0 + eps)) && eps > 1e-14 && eps < 1.0;
+}
+// y[r, i] = t * gamma[i] + beta[i] with t the normalised element; gamma / beta optional.  `set_t` puts the probe
+// values that make t = 3 (and a second time t = -0.5).
+template <typename F>
+static bool probe_affine_store(const Item &it, const BpNode &st, Probe &p, Route &r, F set_t) {
+  if (st.t != BpNode::EXPR || st.writes.size() != 1 || !is_global_aref(it, st.writes[0], r.out) || r.out == r.a) return false;
+  r.out_idx = st.writes[0].v[2];
+  std::vector<int> arrs;
+  global_arefs(it, st.rhs, arrs);
+  std::vector<int> extra;
+  for (int a : arrs)
+    if (a != r.a) extra.push_back(a);
+  if (extra.size() > 2 || std::find(extra.begin(), extra.end(), r.out) != extra.end()) return false;
+  auto value = [&](double t, double g, double b, int gpos, int bpos, double &out) {
+    p.arrays.clear();
+    p.index.clear();
+    set_t(t);
+    if (gpos >= 0) p.arrays[gpos] = g;
+    if (bpos >= 0) p.arrays[bpos] = b;
+    return probe(st.rhs, p, out);
+  };
+  auto fits = [&](int gpos, int bpos) {
+    double v;
+    const double g = gpos >= 0 ? 1.5 : 1.0, b = bpos >= 0 ? 0.25 : 0.0;
+    if (!value(3.0, g, b, gpos, bpos, v) || !near(v, 3.0 * g + b)) return false;
+    const double g2 = gpos >= 0 ? -0.75 : 1.0, b2 = bpos >= 0 ? 2.0 : 0.0;
+    if (!value(-0.5, g2, b2, gpos, bpos, v) || !near(v, -0.5 * g2 + b2)) return false;
+    r.b = gpos, r.bias = bpos;
+    if (gpos >= 0) r.b_idx = p.index[gpos];
+    if (bpos >= 0) r.bias_idx = p.index[bpos];
+    r.a_idx = p.index.count(r.a) ? p.index[r.a] : r.a_idx;
+    return true;
+  };
+  if (extra.empty()) return fits(-1, -1);
+  if (extra.size() == 1) return fits(extra[0], -1) || fits(-1, extra[0]);
+  return fits(extra[0], extra[1]) || fits(extra[1], extra[0]);
+}
+static bool rownorm_loops(const std::vector<BpNode> &b, const int *fors, int nfors, Route &r) {
+  const Sx *rows = upper_bound(b[0]);
+  if (!rows || !is_zero(b[0].upfrom)) return false;
+  r.idx[0] = b[0].idx;
+  r.bound[0] = *rows;
+  for (int k = 0; k < nfors; k++) {
+    const BpNode &f = b[fors[k]];
+    const Sx *n = upper_bound(f);
+    if (!n || !is_zero(f.upfrom) || (k && (f.idx != r.idx[1] || !sx_equal(*n, r.bound[1])))) return false;
+    if (!k) r.idx[1] = f.idx, r.bound[1] = *n;
+  }
+  return true;
+}
+// for r: { s = 0; for i: s += x; u = s / n; q = 0; for i: q += (x - u)^2; rr = 1 / sqrt(q / n + eps);
+//          for i: y = (x - u) * rr [* gamma[i]] [+ beta[i]] }
+static bool match_layernorm(const Item &it, Route &r) {
+  const std::vector<BpNode> &b = it.body;
+  if (b.size() != 15) return false;
+  const BpNode::T want[15] = {BpNode::FOR, BpNode::EXPR, BpNode::FOR, BpNode::EXPR, BpNode::ENDFOR, BpNode::EXPR, BpNode::EXPR,
+                              BpNode::FOR, BpNode::EXPR, BpNode::ENDFOR, BpNode::EXPR, BpNode::FOR, BpNode::EXPR,
+                              BpNode::ENDFOR, BpNode::ENDFOR};
+  for (int k = 0; k < 15; k++)
+    if (b[k].t != want[k]) return false;
+  const int fors[3] = {2, 7, 11};
+  if (!rownorm_loops(b, fors, 3, r)) return false;
+  if (!b[1].declare || !is_zero(b[1].rhs) || !is_scalar_ref(b[1].writes[0])) return false;
+  const std::string s = ref_name(b[1].writes[0]);
+  Sx term;
+  if (!reduction_term(b[3], s, "add", term) || !is_global_aref(it, term, r.a)) return false;
+  r.a_idx = term.v[2];
+  Probe p;
+  p.it = &it;
+  double n, v;
+  if (!probe_row_length(r.bound[1], p, n)) return false;
+  // the mean
+  if (!b[5].declare || b[5].writes.size() != 1 || !is_scalar_ref(b[5].writes[0])) return false;
+  const std::string u = ref_name(b[5].writes[0]);
+  p.scalars[s] = 3.5 * n;
+  if (!probe(b[5].rhs, p, v) || !near(v, 3.5)) return false;
+  p.scalars[s] = -n;
+  if (!probe(b[5].rhs, p, v) || !near(v, -1.0)) return false;
+  // the sum of squared deviations
+  if (!b[6].declare || !is_zero(b[6].rhs) || !is_scalar_ref(b[6].writes[0])) return false;
+  const std::string q = ref_name(b[6].writes[0]);
+  if (!reduction_term(b[8], q, "add", term)) return false;
+  const double xs[2] = {3.0, 0.5}, us[2] = {1.0, 2.0};
+  for (int k = 0; k < 2; k++) {
+    p.arrays.clear();
+    p.index.clear();
+    p.arrays[r.a] = xs[k];
+    p.scalars[u] = us[k];
+    if (!probe(term, p, v) || !near(v, (xs[k] - us[k]) * (xs[k] - us[k])) || !sx_equal(p.index[r.a], r.a_idx)) return false;
+  }
+  if (!probe_rstd(b[10], q, p, n, r.eps)) return false;
+  const std::string rr = ref_name(b[10].writes[0]);
+  auto set_t = [&](double t) {  // (x - u) * rr = t
+    p.arrays[r.a] = 2.0 * t + 1.0;
+    p.scalars[u] = 1.0;
+    p.scalars[rr] = 0.5;
+  };
+  if (!probe_affine_store(it, b[12], p, r, set_t)) return false;
+  r.kind = R_LAYERNORM;
+  return true;
+}
+// for r: { q = 0; for i: q += x * x; rr = 1 / sqrt(q / n + eps); for i: y = x * rr [* w[i]] }
+static bool match_rmsnorm(const Item &it, Route &r) {
+  const std::vector<BpNode> &b = it.body;
+  if (b.size() != 10) return false;
+  const BpNode::T want[10] = {BpNode::FOR, BpNode::EXPR, BpNode::FOR, BpNode::EXPR, BpNode::ENDFOR, BpNode::EXPR,
+                              BpNode::FOR, BpNode::EXPR, BpNode::ENDFOR, BpNode::ENDFOR};
+  for (int k = 0; k < 10; k++)
+    if (b[k].t != want[k]) return false;
+  const int fors[2] = {2, 6};
+  if (!rownorm_loops(b, fors, 2, r)) return false;
+  if (!b[1].declare || !is_zero(b[1].rhs) || !is_scalar_ref(b[1].writes[0])) return false;
+  const std::string q = ref_name(b[1].writes[0]);
+  Sx term;
+  if (!reduction_term(b[3], q, "add", term)) return false;
+  std::vector<int> arrs;
+  global_arefs(it, term, arrs);
+  if (arrs.size() != 1) return false;
+  r.a = arrs[0];
+  Probe p;
+  p.it = &it;
+  double n, v;
+  if (!probe_row_length(r.bound[1], p, n)) return false;
+  const double xs[2] = {3.0, -2.0};
+  for (int k = 0; k < 2; k++) {
+    p.arrays.clear();
+    p.index.clear();
+    p.arrays[r.a] = xs[k];
+    if (!probe(term, p, v) || !near(v, xs[k] * xs[k])) return false;
+  }
+  r.a_idx = p.index[r.a];
+  if (!probe_rstd(b[5], q, p, n, r.eps)) return false;
+  const std::string rr = ref_name(b[5].writes[0]);
+  auto set_t = [&](double t) {  // x * rr = t
+    p.arrays[r.a] = 2.0 * t;
+    p.scalars[rr] = 0.5;
+  };
+  if (!probe_affine_store(it, b[7], p, r, set_t) || r.bias >= 0) return false;
+  r.kind = R_RMSNORM;
   return true;
 }
 
@@ -1115,6 +1352,26 @@ static bool launch_route(Program &pg, void **args, const std::map<std::string, l
     pg.last_route = "cthip_softmax";
     return true;
   }
+  if (r.kind == R_LAYERNORM || r.kind == R_RMSNORM) {
+    long long Rn, N;
+    if (!bound(0, Rn) || !bound(1, N) || N < 1) return false;
+    Affine ax, ao, ag;
+    if (!affine_of(r.a_idx, r.idx, 2, env, ax) || ax.base || ax.c[0] != N || ax.c[1] != 1) return false;
+    if (!affine_of(r.out_idx, r.idx, 2, env, ao) || ao.base || ao.c[0] != N || ao.c[1] != 1) return false;
+    // gamma / beta are read by column, whatever the row
+    if (r.b >= 0 && (!affine_of(r.b_idx, r.idx, 2, env, ag) || ag.base || ag.c[0] != 0 || ag.c[1] != 1)) return false;
+    if (r.bias >= 0 && (!affine_of(r.bias_idx, r.idx, 2, env, ag) || ag.base || ag.c[0] != 0 || ag.c[1] != 1)) return false;
+    if (Rn == 0) return true;
+    const float *g = r.b >= 0 ? (const float *)ptr(r.b) : nullptr, *bt = r.bias >= 0 ? (const float *)ptr(r.bias) : nullptr;
+    if (r.kind == R_LAYERNORM) {
+      rc = cthip_layernorm((float *)ptr(r.out), (const float *)ptr(r.a), g, bt, (float)r.eps, Rn, (int)N);
+      pg.last_route = "cthip_layernorm";
+    } else {
+      rc = cthip_rmsnorm((float *)ptr(r.out), (const float *)ptr(r.a), g, (float)r.eps, Rn, (int)N);
+      pg.last_route = "cthip_rmsnorm";
+    }
+    return true;
+  }
   return false;
 }
 
@@ -1147,6 +1404,8 @@ int cthip_program_create(void **program, const char *blueprint) {
   else if ((r = Route(), match_embedding(pg->item, r))) pg->route = r, pg->route_name = "embedding";
   else if ((r = Route(), match_argmax(pg->item, r))) pg->route = r, pg->route_name = "argmax";
   else if ((r = Route(), match_softmax(pg->item, r))) pg->route = r, pg->route_name = "softmax";
+  else if ((r = Route(), match_layernorm(pg->item, r))) pg->route = r, pg->route_name = "layernorm";
+  else if ((r = Route(), match_rmsnorm(pg->item, r))) pg->route = r, pg->route_name = "rmsnorm";
   *program = pg;
   return 0;
 }

@@ -495,6 +495,59 @@ def test_softmax_item_with_dynamic_shape(oracle):
     assert np.allclose(got, want, rtol=1e-5, atol=1e-5) and np.allclose(got.sum(-1), 1.0, atol=1e-5)
 
 
+@pytest.mark.parametrize("static", [False, True])
+def test_layernorm_and_rmsnorm_items_are_routed(oracle, static):
+    """LayerNorm / RMSNorm rows lowered as one kernel each (nn/normalization.lisp:39-58,78-92) go to the row
+    kernels; eps is read off the item.  The same items with routing switched off run their rendered kernels, and
+    an item that also stores the row mean is not a LayerNorm the row kernel can stand in for."""
+    import copy
+    import caten_amd as ca
+    from caten_amd import blueprints as bp, _lib
+    rows, n = 37, 768
+    rng = np.random.default_rng(9)
+    x = rng.normal(0.5, 3, (rows, n)).astype(np.float32)
+    g = rng.normal(1, 0.1, n).astype(np.float32)
+    b = rng.normal(0, 0.1, n).astype(np.float32)
+    shape = dict(rows=rows, n=n) if static else {}
+    dyn = [] if static else [rows, n]
+    y0 = np.zeros_like(x)
+    cases = [
+        (bp.layernorm_rows(eps=1e-5, **shape), [y0, *dyn, x, g, b], "cthip_layernorm", oracle.layernorm(x, g, b, eps=1e-5)),
+        (bp.layernorm_rows(affine=False, eps=1e-3, **shape), [y0, *dyn, x], "cthip_layernorm",
+         oracle.layernorm(x, np.ones(n, np.float32), np.zeros(n, np.float32), eps=1e-3)),
+        (bp.rmsnorm_rows(eps=1e-6, **shape), [y0, *dyn, x, g], "cthip_rmsnorm", oracle.rmsnorm(x, g, eps=1e-6)),
+        (bp.rmsnorm_rows(weight=False, eps=1e-5, **shape), [y0, *dyn, x], "cthip_rmsnorm",
+         oracle.rmsnorm(x, np.ones(n, np.float32), eps=1e-5)),
+    ]
+    lib = _lib.load()
+    for item, args, route, want in cases:
+        (got,), prog = _run_item(ca, copy.deepcopy(item), args)
+        assert prog.last_route == route, (item["name"], prog.last_route)
+        assert np.max(np.abs(got - want)) < 2e-5
+        _lib.check(lib.cthip_set_option(b"render_routes", 0))
+        try:
+            (got2,), prog2 = _run_item(ca, copy.deepcopy(item), args)
+        finally:
+            _lib.check(lib.cthip_set_option(b"render_routes", 1))
+        assert prog2.last_route == "rendered" and np.max(np.abs(got2 - want)) < 2e-5
+    # variations that are not the norm: the mean is also stored / the variance is not of the centred row
+    ln = bp.layernorm_rows(**shape)
+    k = next(i for i, nd in enumerate(ln["blueprint"]) if nd.get("writes") and nd["writes"][0]["id"] == "q")
+    ln["blueprint"].insert(k, {"type": "EXPR", "writes": [{"op": "AREF", "id": "val_y", "index": "_gid0"}], "expr": "u", "dtype": "float32"})
+    r = ca.HipRenderer()
+    r.render_kernel(ln)
+    r.compile_kernel([ln])
+    assert ln["route"] == "rendered"
+    bad = bp.layernorm_rows(**shape)
+    for nd in bad["blueprint"]:
+        if nd.get("reduction") and nd["writes"][0]["id"] == "q":
+            xi = nd["expr"]["args"][1]["args"][0]["args"][0]
+            nd["expr"] = {"op": "ADD", "args": ["q", {"op": "MUL", "args": [xi, xi]}]}  # sum of x^2, not of (x - u)^2
+    r.render_kernel(bad)
+    r.compile_kernel([bad])
+    assert bad["route"] == "rendered"
+
+
 def test_rank0_output_passed_by_pointer_is_written_back():
     """A rank-0 OUTPUT is declared as a pointer (rewriting-rules.lisp:207-231); CLANG boxes the Lisp number in a
     one-element foreign object and stores the result back into the buffer (clang.lisp:166-185).  Here the box is a

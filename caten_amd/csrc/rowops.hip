@@ -930,6 +930,200 @@ __global__ __launch_bounds__(64 * NW) void k_attn_mfma(float *__restrict__ out, 
   }
 }
 
+// The same prompt attention with bf16 matrix instructions (v_mfma_f32_32x32x16_bf16, 16 times the rate of the
+// fp32-operand one): every operand is written as hi + lo bf16 terms and each product as hi*hi + hi*lo + lo*hi, so
+// what is dropped is below 2^-16 of a product -- the "two terms" grade of the GEMMs (gemm_precision 2).  With
+// fp32 operands the matrix instructions alone are 4096 cycles of a 32-key tile; here they are 768 and the tile is
+// bound by the conversions.
+//   S^T = K Q^T : lane l feeds K[key l%32][d = 16 s + 8 (l/32) .. +7] (16 bytes of the row-major bf16 copy of
+//                 the key tile in LDS) and Q[query l%32][the same d] (registers): 16 keys of ONE query per lane,
+//                 key of register r = 8 (r/4) + 4 (l/32) + r%4 as in the fp32 kernel;
+//   O^T += V^T P^T : registers 8 t .. 8 t + 7 of a lane are exactly the 8 keys it has to supply for the t-th
+//                 16-key slice, so P is packed from its own registers and V[those keys][d = l%32 (+32 per block)]
+//                 comes straight from the cache as before.
+typedef __bf16 v8bf_t __attribute__((ext_vector_type(8)));
+typedef __bf16 v2bf_t __attribute__((ext_vector_type(2)));
+typedef float v2f_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ unsigned pk_bf16(float x0, float x1) {  // one v_cvt_pk_bf16_f32, x0 in the low half
+  const v2f_t v = {x0, x1};
+  return __builtin_bit_cast(unsigned, __builtin_convertvector(v, v2bf_t));
+}
+// 8 floats -> their bf16 leading terms and the bf16 of what those miss, packed for one matrix operand each
+__device__ __forceinline__ void split8(const float *x, v8bf_t &hi, v8bf_t &lo) {
+  unsigned h[4], l[4];
+#pragma unroll
+  for (int k = 0; k < 4; k++) {
+    h[k] = pk_bf16(x[2 * k], x[2 * k + 1]);
+    l[k] = pk_bf16(x[2 * k] - __uint_as_float(h[k] << 16), x[2 * k + 1] - __uint_as_float(h[k] & 0xffff0000u));
+  }
+  hi = __builtin_bit_cast(v8bf_t, make_uint4(h[0], h[1], h[2], h[3]));
+  lo = __builtin_bit_cast(v8bf_t, make_uint4(l[0], l[1], l[2], l[3]));
+}
+
+template <int DH, int NW>
+__global__ __launch_bounds__(64 * NW) void k_attn_mfma_bf(float *__restrict__ out, const float *__restrict__ q,
+                                                      const float *__restrict__ kc, const float *__restrict__ vc, int S,
+                                                      int start_pos, int H, int Hkv) {
+  constexpr int NSL = DH / 16;  // 16-wide slices of the head dimension in K Q^T
+  constexpr int DB = DH / 32;   // 32-wide blocks of the head dimension
+  constexpr int KP = DH + 8;    // row pitch of the bf16 key tile: 16-byte reads of 8 consecutive rows hit all banks
+  // per wavefront: its key tile (hi and lo planes, row-major); once its tiles are done, its unnormalised outputs
+  __shared__ union {
+    unsigned short K[2][32][KP];
+    float Co[DB * 16][64];
+  } W[NW];
+  __shared__ float Cm[NW][64], Cl[NW][64];
+  const int h = blockIdx.x, i0 = (gridDim.y - 1 - blockIdx.y) * 32;  // the longest groups are dispatched first
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int half = lane >> 5, col = lane & 31;
+  const int hk = h / (H / Hkv), KD = Hkv * DH;
+  const int qrow = min(i0 + col, S - 1);  // rows past the end repeat the last one and are not stored
+  const int Tq = start_pos + qrow + 1;    // keys this lane's query sees
+  const int Tmax = start_pos + min(i0 + 32, S);
+  const int ntiles = (Tmax + 31) / 32;
+  const float scale = 1.0f / sqrtf((float)DH);
+  // the key tile of a pass is requested one pass ahead, its values at the start of the pass
+  float4 kreg[DH / 8];
+  auto load_k = [&](int t) {
+#pragma unroll
+    for (int u = 0; u < DH / 8; u++) {
+      const int f = lane + 64 * u, key = f / (DH / 4), d4 = f % (DH / 4);
+      const int kr = min(t * 32 + key, Tmax - 1);  // rows clamped to the last visible one: masked below
+      kreg[u] = *(const float4 *)(kc + (int64_t)kr * KD + hk * DH + 4 * d4);
+    }
+  };
+  if (wv < ntiles) load_k(wv);
+  // the block's 32 query rows through LDS (the memory of the key tiles, before they are written), see k_attn_mfma
+  constexpr int QP = DH + 4;
+  static_assert(32 * QP * 4 <= sizeof(W), "the query rows fit the key tile memory");
+  float(*Qs)[QP] = reinterpret_cast<float(*)[QP]>(&W[0]);
+  for (int f = tid; f < 8 * DH; f += 64 * NW) {
+    const int row = f / (DH / 4), c4 = f % (DH / 4);
+    *(float4 *)&Qs[row][4 * c4] = *(const float4 *)(q + ((int64_t)min(i0 + row, S - 1) * H + h) * DH + 4 * c4);
+  }
+  __syncthreads();
+  v8bf_t qh[NSL], ql[NSL];  // slice s of this lane: d = 16 s + 8 half .. +7
+#pragma unroll
+  for (int s = 0; s < NSL; s++) {
+    const float4 t0 = *(const float4 *)&Qs[col][16 * s + 8 * half], t1 = *(const float4 *)&Qs[col][16 * s + 8 * half + 4];
+    const float x[8] = {t0.x, t0.y, t0.z, t0.w, t1.x, t1.y, t1.z, t1.w};
+    split8(x, qh[s], ql[s]);
+  }
+  __syncthreads();  // the key tiles may overwrite the rows now
+  float m = -INFINITY, l = 0.0f;
+  v16f_t o[DB];
+#pragma unroll
+  for (int b = 0; b < DB; b++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) o[b][r] = 0.0f;
+
+  for (int t = wv; t < ntiles; t += NW) {
+    const int kb = t * 32;
+    // the key tile, split, into LDS
+#pragma unroll
+    for (int u = 0; u < DH / 8; u++) {
+      const int f = lane + 64 * u, key = f / (DH / 4), d4 = f % (DH / 4);
+      const unsigned h0 = pk_bf16(kreg[u].x, kreg[u].y), h1 = pk_bf16(kreg[u].z, kreg[u].w);
+      const unsigned l0 = pk_bf16(kreg[u].x - __uint_as_float(h0 << 16), kreg[u].y - __uint_as_float(h0 & 0xffff0000u));
+      const unsigned l1 = pk_bf16(kreg[u].z - __uint_as_float(h1 << 16), kreg[u].w - __uint_as_float(h1 & 0xffff0000u));
+      *(uint2 *)&W[wv].K[0][key][4 * d4] = make_uint2(h0, h1);
+      *(uint2 *)&W[wv].K[1][key][4 * d4] = make_uint2(l0, l1);
+    }
+    float vreg[DB][16];
+#pragma unroll
+    for (int s = 0; s < 16; s++) {
+      const int kr = min(kb + 8 * (s >> 2) + 4 * half + (s & 3), Tmax - 1);
+      const float *vrow = vc + (int64_t)kr * KD + hk * DH + col;
+#pragma unroll
+      for (int b = 0; b < DB; b++) vreg[b][s] = vrow[32 * b];
+    }
+    if (t + NW < ntiles) load_k(t + NW);
+    __builtin_amdgcn_wave_barrier();
+    v16f_t sacc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) sacc[r] = 0.0f;
+#pragma unroll
+    for (int s = 0; s < NSL; s++) {
+      const v8bf_t kh = __builtin_bit_cast(v8bf_t, *(const uint4 *)&W[wv].K[0][col][16 * s + 8 * half]);
+      const v8bf_t kl = __builtin_bit_cast(v8bf_t, *(const uint4 *)&W[wv].K[1][col][16 * s + 8 * half]);
+      sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kl, qh[s], sacc, 0, 0, 0);  // smallest products first
+      sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kh, ql[s], sacc, 0, 0, 0);
+      sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kh, qh[s], sacc, 0, 0, 0);
+    }
+    __builtin_amdgcn_wave_barrier();
+    // sacc[r] = score of key kb + 8*(r/4) + 4*half + r%4 against query `col`
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int key = kb + 8 * (r >> 2) + 4 * half + (r & 3);
+      const float sc = (key < Tq) ? sacc[r] * scale : -INFINITY;
+      sacc[r] = sc;
+      tmax = fmaxf(tmax, sc);
+    }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float m_new = fmaxf(m, tmax);
+    const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;  // no key of this tile visible to this query yet
+    const float corr = ct_exp(m - m_use);
+    float ps = 0.0f, pr[16];
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      pr[r] = ct_exp(sacc[r] - m_use);
+      ps += pr[r];
+    }
+    ps += __shfl_xor(ps, 32, 64);
+    l = l * corr + ps;
+    m = m_new;
+#pragma unroll
+    for (int b = 0; b < DB; b++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) o[b][r] *= corr;
+#pragma unroll
+    for (int t2 = 0; t2 < 2; t2++) {  // the two 16-key slices of the tile
+      v8bf_t ph, pl;
+      split8(pr + 8 * t2, ph, pl);
+#pragma unroll
+      for (int b = 0; b < DB; b++) {
+        v8bf_t vh, vl;
+        split8(&vreg[b][8 * t2], vh, vl);
+        o[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vl, ph, o[b], 0, 0, 0);
+        o[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vh, pl, o[b], 0, 0, 0);
+        o[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vh, ph, o[b], 0, 0, 0);
+      }
+    }
+  }
+  // o[b][r] = unnormalised output element d = 32b + 8*(r/4) + 4*half + r%4 of query `col`
+  __builtin_amdgcn_wave_barrier();
+  Cm[wv][lane] = m;
+  Cl[wv][lane] = l;
+#pragma unroll
+  for (int b = 0; b < DB; b++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) W[wv].Co[b * 16 + r][lane] = o[b][r];
+  __syncthreads();
+  float M = Cm[0][lane];
+#pragma unroll
+  for (int w = 1; w < NW; w++) M = fmaxf(M, Cm[w][lane]);  // finite: the wavefront holding key 0 saw it
+  float e[NW], L = 0.0f;
+#pragma unroll
+  for (int w = 0; w < NW; w++) {
+    e[w] = (Cm[w][lane] == -INFINITY) ? 0.0f : ct_exp(Cm[w][lane] - M);
+    L = fmaf(e[w], Cl[w][lane], L);
+  }
+  const float inv = 1.0f / L;
+  if (i0 + col < S) {
+    float *orow = out + ((int64_t)(i0 + col) * H + h) * DH;
+    constexpr int RPW = DB * 16 / NW;  // wavefront wv finishes registers wv * RPW .. of every lane
+#pragma unroll
+    for (int k = 0; k < RPW; k++) {
+      const int R = wv * RPW + k, b = R >> 4, r = R & 15;
+      float v = 0.0f;
+#pragma unroll
+      for (int w = 0; w < NW; w++) v = fmaf(e[w], W[w].Co[R][lane], v);
+      orow[32 * b + 8 * (r >> 2) + 4 * half + (r & 3)] = v * inv;
+    }
+  }
+}
+
 int launch_attn(float *out, const float *q, const float *kc, const float *vc, int S, int start_pos, const int *pos,
                 int max_T, int H, int Hkv, int Dh) {
   if (S == 0) return 0;
@@ -938,11 +1132,20 @@ int launch_attn(float *out, const float *q, const float *kc, const float *vc, in
   if (S >= 32 && pos == nullptr) {  // prompt rows on the matrix cores
     // eight wavefronts per block where their LDS tiles fit (head_dim <= 64), four otherwise
     dim3 grid(H, (S + 31) / 32);
-    switch (Dh) {
-      case 32: hipLaunchKernelGGL((k_attn_mfma<32, 8>), grid, dim3(512), 0, st, out, q, kc, vc, S, start_pos, H, Hkv); break;
-      case 64: hipLaunchKernelGGL((k_attn_mfma<64, 8>), grid, dim3(512), 0, st, out, q, kc, vc, S, start_pos, H, Hkv); break;
-      case 128: hipLaunchKernelGGL((k_attn_mfma<128, 4>), grid, dim3(256), 0, st, out, q, kc, vc, S, start_pos, H, Hkv); break;
-      default: return fail(CTHIP_E_UNSUPPORTED, "attention: head_dim %d (supported: 32, 64, 128)", Dh);
+    if (state().gemm_precision == 0) {  // fp32 operands asked for: the products are fp32 products
+      switch (Dh) {
+        case 32: hipLaunchKernelGGL((k_attn_mfma<32, 8>), grid, dim3(512), 0, st, out, q, kc, vc, S, start_pos, H, Hkv); break;
+        case 64: hipLaunchKernelGGL((k_attn_mfma<64, 8>), grid, dim3(512), 0, st, out, q, kc, vc, S, start_pos, H, Hkv); break;
+        case 128: hipLaunchKernelGGL((k_attn_mfma<128, 4>), grid, dim3(256), 0, st, out, q, kc, vc, S, start_pos, H, Hkv); break;
+        default: return fail(CTHIP_E_UNSUPPORTED, "attention: head_dim %d (supported: 32, 64, 128)", Dh);
+      }
+    } else {  // two bf16 terms per operand, whatever the GEMMs use
+      switch (Dh) {
+        case 32: hipLaunchKernelGGL((k_attn_mfma_bf<32, 8>), grid, dim3(512), 0, st, out, q, kc, vc, S, start_pos, H, Hkv); break;
+        case 64: hipLaunchKernelGGL((k_attn_mfma_bf<64, 8>), grid, dim3(512), 0, st, out, q, kc, vc, S, start_pos, H, Hkv); break;
+        case 128: hipLaunchKernelGGL((k_attn_mfma_bf<128, 4>), grid, dim3(256), 0, st, out, q, kc, vc, S, start_pos, H, Hkv); break;
+        default: return fail(CTHIP_E_UNSUPPORTED, "attention: head_dim %d (supported: 32, 64, 128)", Dh);
+      }
     }
     CTHIP_LAUNCH_CHECK();
     return 0;

@@ -413,6 +413,14 @@ def test_sdpa_cached(ops, oracle, S, start, H, Hkv, Dh):
     mask = oracle.triu_neginf(S, T, 1 + start)
     want = oracle.sdpa(q, np.ascontiguousarray(k[:T]), np.ascontiguousarray(v[:T]), mask)
     close(ops.sdpa_cached(q, k, v, start), want, 1e-4, 1e-5)
+    if S >= 32:  # the matrix-core kernel with fp32 operands instead of two bf16 terms per operand
+        from caten_amd import _lib
+        lib = _lib.load()
+        _lib.check(lib.cthip_set_option(b"gemm_precision", 0))
+        try:
+            close(ops.sdpa_cached(q, k, v, start), want, 1e-4, 1e-5)
+        finally:
+            _lib.check(lib.cthip_set_option(b"gemm_precision", 2))
 
 
 # ------------------------------------------------------------------ matmul (MFMA)

@@ -990,7 +990,7 @@ int launch_gemm(GemmArgs a, int bmode, int precision, float *static_ws, size_t s
     // product, one tile per unit, loses 10-30 % when it is split in two)
     // (the 512-thread workgroups of k_gemm_qpc sit one to a compute unit: aim at one each)
     int ks = quant ? (int)(cus / tiles) : (int)((tiles * 2 <= cus ? cus * 2 : cus * 3 / 2) / tiles);
-    if (ks > nsteps / 6) ks = nsteps / 6;
+    if (ks > nsteps / 3) ks = nsteps / 3;
     if (ks > 16) ks = 16;
     if (a.routed) ks = 1;  // routed tiles are stored by the workgroup that computed them
     if (ks > 1) {

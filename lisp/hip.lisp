@@ -10,8 +10,8 @@
 ;;;; The renderer protocol is implemented by PRINTING: %render-kernel prints the Schedule-Item's blueprint as an
 ;;;; s-expression (the grammar is in the header of caten_amd/csrc/render.hip) and hands it to
 ;;;; cthip_program_create, which returns HIP source with gfx950-aware work distribution and, for the matmul /
-;;;; Linear / one-hot Embedding / ArgMax / softmax-row shapes, a route to a hand-written kernel; `invoke` is
-;;;; cthip_program_launch.  Nothing about work distribution lives on this side.
+;;;; Linear / one-hot Embedding / ArgMax / softmax / LayerNorm / RMSNorm row shapes, a route to a hand-written
+;;;; kernel; `invoke` is cthip_program_launch.  Nothing about work distribution lives on this side.
 ;;;;
 ;;;; This image has no Common Lisp implementation, so this file has not been loaded by a Lisp here;
 ;;;; the same C ABI, including the s-expression text, is exercised through the Python mirror in caten_amd/.

@@ -47,28 +47,28 @@ struct GqaStageRegs {
 // back in request order, so the vector can be staged while the weights are still arriving, and nothing that
 // uses an answer (the compiler would otherwise start adding accumulators early, to save registers) is moved in
 // front of a later request.
-template <int NV, bool ACC>
+template <int NT, int NV, bool ACC>
 __device__ __forceinline__ void gqa_stage_request(const GqaStage &s, GqaStageRegs<NV, ACC> &r) {
   const int tid = threadIdx.x;
 #pragma unroll
   for (int k = 0; k < NV; k++) {
-    r.v[k] = ((const float4 *)s.base)[tid + 256 * k];
-    r.g[k] = ((const float4 *)s.gamma)[tid + 256 * k];
+    r.v[k] = ((const float4 *)s.base)[tid + NT * k];
+    r.g[k] = ((const float4 *)s.gamma)[tid + NT * k];
   }
   if (ACC) {
 #pragma unroll
     for (int k = 0; k < NV; k++)
 #pragma unroll
       for (int x = 0; x < kDecXcds; x++) {
-        const longlong2 *src = (const longlong2 *)(s.iparts + (int64_t)x * s.D) + 2 * (tid + 256 * k);
+        const longlong2 *src = (const longlong2 *)(s.iparts + (int64_t)x * s.D) + 2 * (tid + NT * k);
         r.lo[k][x] = src[0];
         r.hi[k][x] = src[1];
       }
   }
 }
 
-// gamma * x to LDS (swizzled), 1 / rms(x) returned; block 0 stores x to s.xout.  red holds 4 floats.
-template <int NV, bool ACC>
+// gamma * x to LDS (swizzled), 1 / rms(x) returned; block 0 stores x to s.xout.  red holds NT / 64 floats.
+template <int NT, int NV, bool ACC>
 __device__ __forceinline__ float gqa_stage_finish(const GqaStage &s, GqaStageRegs<NV, ACC> &r, float *xs, float *red) {
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   if (ACC) {
@@ -91,13 +91,14 @@ __device__ __forceinline__ float gqa_stage_finish(const GqaStage &s, GqaStageReg
   for (int k = 0; k < NV; k++) {
     const float4 v = r.v[k], g = r.g[k];
     ss = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, fmaf(v.w, v.w, ss))));
-    ((float4 *)xs)[swz(tid + 256 * k)] = make_float4(v.x * g.x, v.y * g.y, v.z * g.z, v.w * g.w);
-    if (blockIdx.x == 0 && s.xout) ((float4 *)s.xout)[tid + 256 * k] = v;
+    ((float4 *)xs)[swz(tid + NT * k)] = make_float4(v.x * g.x, v.y * g.y, v.z * g.z, v.w * g.w);
+    if (blockIdx.x == 0 && s.xout) ((float4 *)s.xout)[tid + NT * k] = v;
   }
   ss = wave_sum(ss);
   if (lane == 0) red[wv] = ss;
   __syncthreads();
-  const float tot = (red[0] + red[1]) + (red[2] + red[3]);
+  float tot = (red[0] + red[1]) + (red[2] + red[3]);
+  if (NT == 512) tot += (red[4] + red[5]) + (red[6] + red[7]);
   return 1.0f / sqrtf(tot / (float)s.D + s.eps);
 }
 
@@ -117,21 +118,25 @@ __device__ __forceinline__ float read_block(const float *xs, int blk, float *xr)
 }
 
 // ---- launch 1: RMSNorm folded through wq|wk|wv; a wavefront produces four consecutive rows ----
-template <int KC, bool ACC>
-__global__ __launch_bounds__(256) void k_gqa_qkv(GqaQkvArgs a) {
+// NT threads per workgroup: with 512 every SIMD holds two wavefronts, and a wavefront issues a vector instruction
+// every 8 cycles at best whatever its instruction-level parallelism -- the 2.4 instructions per 4-bit weight and
+// the accumulator sums of one wavefront per SIMD are what a 256-thread launch spends its time on.
+template <int KC, bool ACC, int NT>
+__global__ __launch_bounds__(NT) void k_gqa_qkv(GqaQkvArgs a) {
+  constexpr int RW = 16 / (NT / 64);  // rows per wavefront
   __shared__ __align__(16) float xs[2048 * KC];
-  __shared__ float red[4];
+  __shared__ float red[NT / 64];
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int D = a.st.D;
-  const int r0 = blockIdx.x * 16 + wv * 4;  // < rows: the launcher requires rows % 16 == 0
-  GqaStageRegs<2 * KC, ACC> sr;
-  gqa_stage_request(a.st, sr);
+  const int r0 = blockIdx.x * 16 + wv * RW;  // < rows: the launcher requires rows % 16 == 0
+  GqaStageRegs<512 * KC / NT, ACC> sr;
+  gqa_stage_request<NT>(a.st, sr);
   const int posv = a.pos[0];
   __builtin_amdgcn_sched_barrier(0);
-  uint4 w[4][KC];
-  unsigned sc[4][KC];
+  uint4 w[RW][KC];
+  unsigned sc[RW][KC];
 #pragma unroll
-  for (int u = 0; u < 4; u++)
+  for (int u = 0; u < RW; u++)
 #pragma unroll
     for (int j = 0; j < KC; j++) {
       const int64_t idx = (int64_t)(r0 + u) * (64 * KC) + lane + 64 * j;
@@ -142,32 +147,40 @@ __global__ __launch_bounds__(256) void k_gqa_qkv(GqaQkvArgs a) {
   if (a.zero) {  // the attention launch's accumulators: read last by the previous layer's MLP launch
     uint4 *z = (uint4 *)a.zero;
     const uint4 zz = make_uint4(0u, 0u, 0u, 0u);
-    for (int64_t k = (int64_t)blockIdx.x * 256 + tid; k < a.zero_n16; k += (int64_t)gridDim.x * 256) z[k] = zz;
+    for (int64_t k = (int64_t)blockIdx.x * NT + tid; k < a.zero_n16; k += (int64_t)gridDim.x * NT) z[k] = zz;
   }
-  const float rstd = gqa_stage_finish(a.st, sr, xs, red);
-  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  const float rstd = gqa_stage_finish<NT>(a.st, sr, xs, red);
+  float acc[RW];
+#pragma unroll
+  for (int u = 0; u < RW; u++) acc[u] = 0.0f;
 #pragma unroll
   for (int j = 0; j < KC; j++) {
     float xr[32];
     const float xsum = read_block(xs, lane + 64 * j, xr);
 #pragma unroll
-    for (int u = 0; u < 4; u++) acc[u] += chunk_dot<CTHIP_Q4_0>(w[u][j], half_bits_to_float((unsigned short)sc[u][j]), xr, xsum);
+    for (int u = 0; u < RW; u++) acc[u] += chunk_dot<CTHIP_Q4_0>(w[u][j], half_bits_to_float((unsigned short)sc[u][j]), xr, xsum);
   }
 #pragma unroll
-  for (int u = 0; u < 4; u++) acc[u] = wave_sum(acc[u]) * rstd;
+  for (int u = 0; u < RW; u++) acc[u] = wave_sum(acc[u]) * rstd;
   if (lane == 0) {
-    float4 o = make_float4(acc[0], acc[1], acc[2], acc[3]);
+    // the wavefront's RW rows as (part of) a group of four consecutive rows = two rotation pairs
+    const int g0 = r0 & ~3;
+    const bool second = RW == 2 && (r0 & 2);
+    float4 o = RW == 4 ? make_float4(acc[0], acc[1], acc[RW - 2], acc[RW - 1])
+                       : (second ? make_float4(0.f, 0.f, acc[0], acc[1]) : make_float4(acc[0], acc[1], 0.f, 0.f));
     float *dst;
-    if (r0 < D) {
-      o = rope4(o, (r0 % a.DH) >> 2, a.DH, a.log2_base, posv);
-      dst = a.q + r0;
-    } else if (r0 < D + a.KD) {
-      o = rope4(o, ((r0 - D) % a.DH) >> 2, a.DH, a.log2_base, posv);
-      dst = a.kc + (int64_t)posv * a.KD + (r0 - D);
+    if (g0 < D) {
+      o = rope4(o, (g0 % a.DH) >> 2, a.DH, a.log2_base, posv);
+      dst = a.q + g0;
+    } else if (g0 < D + a.KD) {
+      o = rope4(o, ((g0 - D) % a.DH) >> 2, a.DH, a.log2_base, posv);
+      dst = a.kc + (int64_t)posv * a.KD + (g0 - D);
     } else {
-      dst = a.vc + (int64_t)posv * a.KD + (r0 - D - a.KD);
+      dst = a.vc + (int64_t)posv * a.KD + (g0 - D - a.KD);
     }
-    *(float4 *)dst = o;
+    if (RW == 4) *(float4 *)dst = o;
+    else if (second) *(float2 *)(dst + 2) = make_float2(o.z, o.w);
+    else *(float2 *)dst = make_float2(o.x, o.y);
   }
 }
 
@@ -320,22 +333,24 @@ void k_gqa_attn_proj(GqaAttnArgs a) {
 }
 
 // ---- launch 3: RMSNorm folded through 32 gate and 32 up rows, SwiGLU, one Q4_0 block per row of `down` ----
-template <int KC>
-__global__ __launch_bounds__(256) void k_gqa_mlp(GqaMlpArgs a) {
+template <int KC, int NT>
+__global__ __launch_bounds__(NT) void k_gqa_mlp(GqaMlpArgs a) {
+  constexpr int RW = 32 / (NT / 64);    // gate rows (and up rows) per wavefront
+  constexpr int PJ = 2048 * KC / NT;    // rows of the down projection per thread
   __shared__ __align__(16) float xs[2048 * KC];
-  __shared__ float red[4];
+  __shared__ float red[NT / 64];
   __shared__ __align__(16) float hs[32];
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int D = a.st.D;
   const int slab = blockIdx.x;
-  GqaStageRegs<2 * KC, true> sr;
-  gqa_stage_request(a.st, sr);
+  GqaStageRegs<512 * KC / NT, true> sr;
+  gqa_stage_request<NT>(a.st, sr);
   __builtin_amdgcn_sched_barrier(0);
-  uint4 wg[8][KC], wu[8][KC];
-  unsigned sg[8][KC], su[8][KC];
+  uint4 wg[RW][KC], wu[RW][KC];
+  unsigned sg[RW][KC], su[RW][KC];
 #pragma unroll
-  for (int u = 0; u < 8; u++) {
-    const int64_t gr = (int64_t)(slab * 32 + wv * 8 + u) * a.gate_stride, ur = gr + a.up_off;
+  for (int u = 0; u < RW; u++) {
+    const int64_t gr = (int64_t)(slab * 32 + wv * RW + u) * a.gate_stride, ur = gr + a.up_off;
 #pragma unroll
     for (int j = 0; j < KC; j++) {
       const int64_t gi = gr * (64 * KC) + lane + 64 * j, ui = ur * (64 * KC) + lane + 64 * j;
@@ -345,38 +360,38 @@ __global__ __launch_bounds__(256) void k_gqa_mlp(GqaMlpArgs a) {
       su[u][j] = a.wd[ui];
     }
   }
-  // this slab's block of every row of the down projection: row r = tid + 256 j (D = 2048 * KC)
-  uint4 pw[8 * KC];
-  unsigned ps[8 * KC];
+  // this slab's block of every row of the down projection: row r = tid + NT j (D = 2048 * KC)
+  uint4 pw[PJ];
+  unsigned ps[PJ];
 #pragma unroll
-  for (int j = 0; j < 8 * KC; j++) {
-    const int64_t idx = (int64_t)slab * D + tid + 256 * j;
+  for (int j = 0; j < PJ; j++) {
+    const int64_t idx = (int64_t)slab * D + tid + NT * j;
     pw[j] = ((const uint4 *)a.pq)[idx];
     ps[j] = a.pd[idx];
   }
   __builtin_amdgcn_sched_barrier(0);
-  const float rstd = gqa_stage_finish(a.st, sr, xs, red);
-  float ag[8], au[8];
+  const float rstd = gqa_stage_finish<NT>(a.st, sr, xs, red);
+  float ag[RW], au[RW];
 #pragma unroll
-  for (int u = 0; u < 8; u++) ag[u] = au[u] = 0.0f;
+  for (int u = 0; u < RW; u++) ag[u] = au[u] = 0.0f;
 #pragma unroll
   for (int j = 0; j < KC; j++) {
     float xr[32];
     const float xsum = read_block(xs, lane + 64 * j, xr);
 #pragma unroll
-    for (int u = 0; u < 8; u++) {
+    for (int u = 0; u < RW; u++) {
       ag[u] += chunk_dot<CTHIP_Q4_0>(wg[u][j], half_bits_to_float((unsigned short)sg[u][j]), xr, xsum);
       au[u] += chunk_dot<CTHIP_Q4_0>(wu[u][j], half_bits_to_float((unsigned short)su[u][j]), xr, xsum);
     }
   }
 #pragma unroll
-  for (int u = 0; u < 8; u++) {
+  for (int u = 0; u < RW; u++) {
     ag[u] = wave_sum(ag[u]);
     au[u] = wave_sum(au[u]);
   }
   if (lane == 0) {
 #pragma unroll
-    for (int u = 0; u < 8; u++) hs[wv * 8 + u] = ct_silu(rstd * ag[u]) * (rstd * au[u]);
+    for (int u = 0; u < RW; u++) hs[wv * RW + u] = ct_silu(rstd * ag[u]) * (rstd * au[u]);
   }
   __syncthreads();
   float hr[32], hsum;
@@ -395,9 +410,9 @@ __global__ __launch_bounds__(256) void k_gqa_mlp(GqaMlpArgs a) {
   }
   long long *accum = a.accum + (int64_t)xcd_id() * D;
 #pragma unroll
-  for (int j = 0; j < 8 * KC; j++) {
+  for (int j = 0; j < PJ; j++) {
     const float s = chunk_dot<CTHIP_Q4_0>(pw[j], half_bits_to_float((unsigned short)ps[j]), hr, hsum);
-    __hip_atomic_fetch_add(accum + tid + 256 * j, __float2ll_rn(s * kFixScale), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    __hip_atomic_fetch_add(accum + tid + NT * j, __float2ll_rn(s * kFixScale), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
   }
 }
 
@@ -447,10 +462,10 @@ int launch_gqa_qkv(const GqaQkvArgs &a, bool from_accum) {
   const int D = a.st.D;
   if (D != 2048 || a.rows % 16 || a.rows != D + 2 * a.KD || a.DH != 64 || a.KD % 64)
     return fail(CTHIP_E_BAD_ARG, "decoder: fused grouped-query qkv launch with D = %d, rows = %d, KD = %d", D, a.rows, a.KD);
-  dim3 grid(a.rows / 16), block(256);
+  dim3 grid(a.rows / 16), block(512);
   hipStream_t st = state().stream;
-  if (from_accum) hipLaunchKernelGGL((k_gqa_qkv<1, true>), grid, block, 0, st, a);
-  else hipLaunchKernelGGL((k_gqa_qkv<1, false>), grid, block, 0, st, a);
+  if (from_accum) hipLaunchKernelGGL((k_gqa_qkv<1, true, 512>), grid, block, 0, st, a);
+  else hipLaunchKernelGGL((k_gqa_qkv<1, false, 512>), grid, block, 0, st, a);
   CTHIP_LAUNCH_CHECK();
   return 0;
 }
@@ -475,9 +490,9 @@ int launch_gqa_mlp(const GqaMlpArgs &a, int F, int HKV) {
   (void)HKV;
   const int D = a.st.D;
   if (D != 2048 || F % 32) return fail(CTHIP_E_BAD_ARG, "decoder: fused SwiGLU launch with D = %d, F = %d", D, F);
-  dim3 grid(F / 32), block(256);
+  dim3 grid(F / 32), block(512);
   hipStream_t st = state().stream;
-  hipLaunchKernelGGL((k_gqa_mlp<1>), grid, block, 0, st, a);
+  hipLaunchKernelGGL((k_gqa_mlp<1, 512>), grid, block, 0, st, a);
   CTHIP_LAUNCH_CHECK();
   return 0;
 }

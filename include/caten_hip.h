@@ -104,8 +104,9 @@ int cthip_launch(void *fn, const unsigned grid[3], const unsigned block[3], unsi
 /* ---- Hip-Renderer: %render-kernel / invoke behind the C ABI ----
  * The renderer protocol (source/codegen/renderer.lisp:30-34) is a Lisp class; its work for this backend -- HIP
  * source with gfx950-aware work distribution for a Schedule-Item, and the choice of a hand-written kernel where
- * the item is a matmul / Linear / one-hot Embedding / ArgMax / softmax-row shape -- is done here, so the Lisp
- * Hip-Renderer only prints the blueprint as an s-expression (grammar: header of caten_amd/csrc/render.hip).
+ * the item is a matmul / Linear / one-hot Embedding / ArgMax / softmax / LayerNorm / RMSNorm row shape -- is done
+ * here, so the Lisp Hip-Renderer only prints the blueprint as an s-expression (grammar: header of
+ * caten_amd/csrc/render.hip).
  *   %render-kernel  = cthip_program_create + cthip_program_source   (CLANG: clang.lisp:21-110; METAL: metal.lisp:178-250)
  *   %compile-kernel = cthip_render_header + every program's source -> cthip_compile -> cthip_module_load ->
  *                     cthip_program_bind per item                   (clang.lisp:207-226, metal.lisp:326-345)
@@ -115,8 +116,9 @@ int cthip_launch(void *fn, const unsigned grid[3], const unsigned block[3], unsi
  *                     data-parallel loops and the shape arguments.  A program with a route checks the actual
  *                     layout at every launch and falls back to its rendered kernel when it does not fit.
  * cthip_program_route: "rendered", or the shape recognised at creation ("matmul", "embedding", "argmax",
- * "softmax"); cthip_program_last_route: what the last launch ran ("rendered", "cthip_matmul", "cthip_linear",
- * "cthip_embedding", "cthip_argmax", "cthip_softmax").  Strings stay valid until the program is destroyed.
+ * "softmax", "layernorm", "rmsnorm"); cthip_program_last_route: what the last launch ran ("rendered",
+ * "cthip_matmul", "cthip_linear", "cthip_embedding", "cthip_argmax", "cthip_softmax", "cthip_layernorm",
+ * "cthip_rmsnorm").  Strings stay valid until the program is destroyed.
  * Option "render_routes" 0 makes every program run its rendered kernel. */
 const char *cthip_render_header(void);
 int cthip_program_create(void **program, const char *blueprint);

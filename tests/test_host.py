@@ -207,7 +207,12 @@ def test_programs_recognise_the_shapes_hand_written_kernels_cover():
     r = HipRenderer()
     cases = [(bp.matmul(), "matmul"), (bp.matmul(relu=True), "matmul"), (bp.matmul(bias=True, relu=True, transposed_b=True), "matmul"),
              (_matmul_item(), "matmul"), (bp.embedding_onehot(), "embedding"), (bp.argmax_rows(), "argmax"),
-             (bp.softmax_rows(), "softmax"), (bp.softmax_rows(rows=8, n=40), "softmax")]
+             (bp.softmax_rows(), "softmax"), (bp.softmax_rows(rows=8, n=40), "softmax"),
+             # LayerNorm / RMSNorm rows (nn/normalization.lisp:39-58,78-92), recognised by the VALUE of their scalar
+             # statements and element expressions: with and without affine parameters, static and dynamic shape
+             (bp.layernorm_rows(), "layernorm"), (bp.layernorm_rows(affine=False, eps=1e-3), "layernorm"),
+             (bp.layernorm_rows(rows=8, n=40), "layernorm"), (bp.rmsnorm_rows(), "rmsnorm"),
+             (bp.rmsnorm_rows(weight=False, rows=4, n=96, eps=1e-6), "rmsnorm")]
     for item, want in cases:
         src = r.render_kernel(item)
         assert item["route"] == want, (item["name"], item["route"])
@@ -222,6 +227,25 @@ def test_programs_recognise_the_shapes_hand_written_kernels_cover():
     odd["blueprint"][-5]["expr"]["args"][1]["args"][1] = "m"
     r.render_kernel(odd)
     assert odd["route"] == "rendered"
+    # a "LayerNorm" whose variance is the mean of x^2 (not of the centred row), one whose output forgets the mean,
+    # and an RMSNorm that adds a bias: not what the row kernels compute, so rendered
+    ln = bp.layernorm_rows()
+    for nd in ln["blueprint"]:
+        if nd.get("reduction") and nd["writes"][0]["id"] == "q":
+            xi = nd["expr"]["args"][1]["args"][0]["args"][0]
+            nd["expr"] = {"op": "ADD", "args": ["q", {"op": "MUL", "args": [xi, xi]}]}
+    r.render_kernel(ln)
+    assert ln["route"] == "rendered"
+    ln2 = bp.layernorm_rows(affine=False)
+    st = next(nd for nd in ln2["blueprint"] if nd.get("writes") and nd["writes"][0]["id"] == "val_y")
+    st["expr"] = {"op": "MUL", "args": [st["expr"]["args"][0]["args"][0], "r"]}  # x * r instead of (x - u) * r
+    r.render_kernel(ln2)
+    assert ln2["route"] == "rendered"
+    rms = bp.rmsnorm_rows()
+    st = next(nd for nd in rms["blueprint"] if nd.get("writes") and nd["writes"][0]["id"] == "val_y")
+    st["expr"] = {"op": "ADD", "args": [st["expr"], 1.0]}
+    r.render_kernel(rms)
+    assert rms["route"] == "rendered"
 
 
 def test_row_with_a_running_sum_stays_in_one_thread():

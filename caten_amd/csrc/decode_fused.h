@@ -9,6 +9,19 @@ constexpr int kDecXcds = 8;  // accelerator dies of gfx950; one MLP accumulator 
 constexpr float kFixScale = 4294967296.0f;             // 2^32
 constexpr float kFixInv = 2.3283064365386963e-10f;     // 2^-32
 
+// Fixed-point (2^-32) <-> float in a handful of instructions each (the 64-bit conversions of the language are a
+// dozen): the integer part and the fraction are converted separately.  to_fix truncates the fraction below 2^-32
+// (the same on every run, which is what the accumulators are for); from_fix is within an ulp of the rounded value.
+// Magnitudes below 2^31.
+__device__ __forceinline__ long long to_fix(float s) {
+  const float fl = floorf(s);
+  const unsigned lo = (unsigned)((s - fl) * kFixScale);  // s - floor(s) is exact, in [0, 1)
+  return (long long)(((unsigned long long)(unsigned)(int)fl << 32) | lo);
+}
+__device__ __forceinline__ float from_fix(long long t) {
+  return fmaf((float)(unsigned)t, kFixInv, (float)(int)(t >> 32));
+}
+
 __device__ __forceinline__ int xcd_id() {
   // XCC_ID hardware register (id 20), bits 3:0: the XCD this wavefront runs on
   return (int)__builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20) & (kDecXcds - 1);

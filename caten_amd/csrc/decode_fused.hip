@@ -93,8 +93,8 @@ __device__ __forceinline__ void dec_stage_finish(const DecStage &s, DecStageRegs
       t3 += r.hi[k].y;
     }
     v = f4add(v, r.b);
-    v = f4add(v, make_float4(__ll2float_rn(t0) * kFixInv, __ll2float_rn(t1) * kFixInv, __ll2float_rn(t2) * kFixInv,
-                             __ll2float_rn(t3) * kFixInv));
+    v = f4add(v, make_float4(from_fix(t0), from_fix(t1), from_fix(t2),
+                             from_fix(t3)));
   }
   // (count, mean, squared deviation) per thread, merged exactly: thread -> wavefront by lane reductions,
   // wavefront -> workgroup through LDS behind the one barrier that also publishes the staged vector
@@ -412,7 +412,7 @@ __global__ __launch_bounds__(256) void k_dec_mlp(DecMlpArgs a) {
       s += chunk_dot<TYPE>(pw[j][k], DecFmt<TYPE>::QUANT ? half_bits_to_float((unsigned short)ps[j]) : 1.0f, hr + XPC * k, 0.0f);
     // no device-scope bits: the addition happens in this XCD's L2.  (One device-wide accumulator instead of
     // one per XCD costs the 192 workgroups more in contention than the seven arrays cost the reader.)
-    __hip_atomic_fetch_add(accum + tid + 256 * j, __float2ll_rn(s * kFixScale), __ATOMIC_RELAXED,
+    __hip_atomic_fetch_add(accum + tid + 256 * j, to_fix(s), __ATOMIC_RELAXED,
                            __HIP_MEMORY_SCOPE_WORKGROUP);
   }
 }
@@ -433,8 +433,8 @@ __global__ __launch_bounds__(256) void k_dec_sum(DecStage s, float *out) {
       t[2] += hi.x;
       t[3] += hi.y;
     }
-    v = f4add(v, make_float4(__ll2float_rn(t[0]) * kFixInv, __ll2float_rn(t[1]) * kFixInv, __ll2float_rn(t[2]) * kFixInv,
-                             __ll2float_rn(t[3]) * kFixInv));
+    v = f4add(v, make_float4(from_fix(t[0]), from_fix(t[1]), from_fix(t[2]),
+                             from_fix(t[3])));
     ((float4 *)out)[i] = v;
   }
 }

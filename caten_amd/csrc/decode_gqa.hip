@@ -82,8 +82,8 @@ __device__ __forceinline__ float gqa_stage_finish(const GqaStage &s, GqaStageReg
         t2 += r.hi[k][x].x;
         t3 += r.hi[k][x].y;
       }
-      r.v[k] = f4add(r.v[k], make_float4(__ll2float_rn(t0) * kFixInv, __ll2float_rn(t1) * kFixInv,
-                                         __ll2float_rn(t2) * kFixInv, __ll2float_rn(t3) * kFixInv));
+      r.v[k] = f4add(r.v[k], make_float4(from_fix(t0), from_fix(t1),
+                                         from_fix(t2), from_fix(t3)));
     }
   }
   float ss = 0.0f;
@@ -328,7 +328,7 @@ void k_gqa_attn_proj(GqaAttnArgs a) {
     s += dpp_f<0xB1>(s);  // the row's other block
     const int r = pr0 + 512 * j;
     if (pc == 0 && r < rr)
-      __hip_atomic_fetch_add(accum + rbase + r, __float2ll_rn(s * kFixScale), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      __hip_atomic_fetch_add(accum + rbase + r, to_fix(s), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
   }
 }
 
@@ -412,7 +412,7 @@ __global__ __launch_bounds__(NT) void k_gqa_mlp(GqaMlpArgs a) {
 #pragma unroll
   for (int j = 0; j < PJ; j++) {
     const float s = chunk_dot<CTHIP_Q4_0>(pw[j], half_bits_to_float((unsigned short)ps[j]), hr, hsum);
-    __hip_atomic_fetch_add(accum + tid + NT * j, __float2ll_rn(s * kFixScale), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    __hip_atomic_fetch_add(accum + tid + NT * j, to_fix(s), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
   }
 }
 

@@ -205,11 +205,86 @@ __global__ __launch_bounds__(256) void k_reduce_norm(ReduceNormArgs a) {
 }
 
 // true if the fused pass can take this shape (otherwise the caller reduces and normalises in two launches)
+// The same with four wavefronts per row (rows too wide, or with too many shares, for one wavefront's registers):
+// thread t of the row's 256 owns float4 t + 256 j, the row statistics meet in LDS.
+template <int MODE, int VPL, int NZ>
+__global__ __launch_bounds__(256) void k_reduce_norm_wide(ReduceNormArgs a) {
+  __shared__ float red[2][4];
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int64_t row = blockIdx.x;
+  const int n = a.n, n4 = n >> 2;
+  float4 t[VPL][NZ], bs[VPL], rs[VPL], gm[VPL], bt[VPL];
+  bool ok[VPL];
+  // every request first, none behind a branch: shares past nparts repeat share 0 and are dropped
+#pragma unroll
+  for (int j = 0; j < VPL; j++) {
+    const int c = tid + 256 * j;
+    ok[j] = c < n4;
+    const int cc = ok[j] ? c : n4 - 1;
+#pragma unroll
+    for (int z = 0; z < NZ; z++) t[j][z] = ((const float4 *)(a.parts + (int64_t)(z < a.nparts ? z : 0) * a.part_stride + row * n))[cc];
+    bs[j] = ((const float4 *)(a.bias ? a.bias : a.parts))[cc];
+    rs[j] = ((const float4 *)((a.resid ? a.resid : a.parts) + row * n))[cc];
+    gm[j] = ((const float4 *)(a.g ? a.g : a.parts))[cc];
+    bt[j] = ((const float4 *)(a.b ? a.b : a.parts))[cc];
+  }
+  float v[VPL][4];
+#pragma unroll
+  for (int j = 0; j < VPL; j++) {
+    float x[4] = {t[j][0].x, t[j][0].y, t[j][0].z, t[j][0].w};
+#pragma unroll
+    for (int z = 1; z < NZ; z++)
+      if (z < a.nparts) x[0] += t[j][z].x, x[1] += t[j][z].y, x[2] += t[j][z].z, x[3] += t[j][z].w;
+    if (a.bias) x[0] += bs[j].x, x[1] += bs[j].y, x[2] += bs[j].z, x[3] += bs[j].w;
+    if (a.resid) x[0] += rs[j].x, x[1] += rs[j].y, x[2] += rs[j].z, x[3] += rs[j].w;
+    if (ok[j]) ((float4 *)(a.xout + row * n))[tid + 256 * j] = make_float4(x[0], x[1], x[2], x[3]);
+#pragma unroll
+    for (int e = 0; e < 4; e++) v[j][e] = ok[j] ? x[e] : 0.0f;
+  }
+  const float inv_n = 1.0f / (float)n;
+  float mean = 0.0f;
+  if (MODE != ROW_RMSNORM) {
+    float s = 0.0f;
+#pragma unroll
+    for (int j = 0; j < VPL; j++)
+#pragma unroll
+      for (int e = 0; e < 4; e++) s += v[j][e];
+    s = wave_sum(s);
+    if (lane == 0) red[0][wv] = s;
+    __syncthreads();
+    mean = ((red[0][0] + red[0][1]) + (red[0][2] + red[0][3])) * inv_n;
+  }
+  float q = 0.0f;
+#pragma unroll
+  for (int j = 0; j < VPL; j++)
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      float d = ok[j] ? v[j][e] - mean : 0.0f;
+      v[j][e] = d;
+      q = fmaf(d, d, q);
+    }
+  q = wave_sum(q);
+  if (lane == 0) red[1][wv] = q;
+  __syncthreads();
+  const float rstd = 1.0f / sqrtf(((red[1][0] + red[1][1]) + (red[1][2] + red[1][3])) * inv_n + a.eps);
+#pragma unroll
+  for (int j = 0; j < VPL; j++) {
+    if (ok[j]) {
+      const float4 g = a.g ? gm[j] : make_float4(1.f, 1.f, 1.f, 1.f);
+      const float4 b = a.b ? bt[j] : make_float4(0.f, 0.f, 0.f, 0.f);
+      ((float4 *)(a.y + row * n))[tid + 256 * j] = make_float4(v[j][0] * rstd * g.x + b.x, v[j][1] * rstd * g.y + b.y,
+                                                             v[j][2] * rstd * g.z + b.z, v[j][3] * rstd * g.w + b.w);
+    }
+  }
+}
+
+static int reduce_norm_bucket(int nparts) { return nparts <= 2 ? 2 : nparts <= 4 ? 4 : nparts <= 8 ? 8 : 16; }
 bool reduce_norm_supported(int n, int nparts) {
-  if (n % 4 || n > 2048 || nparts < 1 || nparts > 16) return false;
-  // the shares of a row are all requested at once: VPL x NZ float4 per lane have to stay in registers
-  const int vpl = (n / 4 + 63) / 64, nz = nparts <= 2 ? 2 : nparts <= 4 ? 4 : nparts <= 8 ? 8 : 16;
-  return vpl * nz <= 32;
+  if (n % 4 || n > 8192 || nparts < 1 || nparts > 16) return false;
+  // the shares of a row are all requested at once: VPL x NZ float4 per lane have to stay in registers; one
+  // wavefront per row where that fits, four otherwise
+  const int nz = reduce_norm_bucket(nparts);
+  return ((n / 4 + 63) / 64) * nz <= 32 || ((n / 4 + 255) / 256) * nz <= 32;
 }
 
 int launch_reduce_norm(float *y, float *xout, const float *parts, int nparts, int64_t part_stride, const float *bias,
@@ -217,11 +292,32 @@ int launch_reduce_norm(float *y, float *xout, const float *parts, int nparts, in
   if (rows == 0 || n == 0) return 0;
   if (!reduce_norm_supported(n, nparts)) return fail(CTHIP_E_BAD_ARG, "reduce + norm: rows of %d with %d shares", n, nparts);
   ReduceNormArgs a = {y, xout, parts, nparts, part_stride, bias, resid, g, b, eps, rows, n};
+  hipStream_t st = state().stream;
+  if (((n / 4 + 63) / 64) * reduce_norm_bucket(nparts) > 32) {  // four wavefronts per row
+    const int vplw = (n / 4 + 255) / 256;
+    dim3 gridw((unsigned)rows), blockw(256);
+#define RW3(MODE, V, Z) hipLaunchKernelGGL((k_reduce_norm_wide<MODE, V, Z>), gridw, blockw, 0, st, a)
+#define RW2(MODE, V)                       \
+    if (nparts <= 2) RW3(MODE, V, 2);      \
+    else if (nparts <= 4) RW3(MODE, V, 4); \
+    else if (nparts <= 8) RW3(MODE, V, 8); \
+    else RW3(MODE, V, 16)
+#define RW1(MODE)                            \
+    if (vplw <= 1) { RW2(MODE, 1); }         \
+    else if (vplw <= 2) { RW2(MODE, 2); }    \
+    else if (vplw <= 4) { RW2(MODE, 4); }    \
+    else { RW2(MODE, 8); }
+    if (rms) { RW1(ROW_RMSNORM) } else { RW1(ROW_LAYERNORM) }
+#undef RW1
+#undef RW2
+#undef RW3
+    CTHIP_LAUNCH_CHECK();
+    return 0;
+  }
   const int vpl = (n / 4 + 63) / 64;
   // a row per wavefront; few rows (a prompt) go one to a workgroup so that they spread over the compute units
   const int wpb = rows <= 4096 ? 1 : 4;
   dim3 grid((unsigned)((rows + wpb - 1) / wpb)), block(64 * wpb);
-  hipStream_t st = state().stream;
 #define RN3(MODE, V, Z) hipLaunchKernelGGL((k_reduce_norm<MODE, V, Z>), grid, block, 0, st, a)
 #define RN2(MODE, V)               \
   if (nparts <= 2) RN3(MODE, V, 2); \

@@ -160,6 +160,9 @@ struct GemmRoute {
   int c0[3];
   int ld[3];
 };
+// act == kActSwigluPairs: the weight rows are (gate_j, up_j) pairs and y (m, rows / 2) gets silu(gate_j) * up_j
+// (SwiGLU, external/llm/layers.lisp:53-64, in the epilogue of the gate|up launch); K is not split then.
+constexpr int kActSwigluPairs = 64;
 // route: non-null = y is ignored, the columns go where the route says; K is not split then.
 int launch_linear_gemm(float *y, const WMat *w, const float *x, int m, const float *bias, const float *residual,
                        int act, int precision, GemmDeferred *defer = nullptr, const GemmRoute *route = nullptr);

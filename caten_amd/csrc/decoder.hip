@@ -739,12 +739,17 @@ static int prefill(Decoder *d, const int *ids, int s, int n) {
       }
       TRY(launch_attn(ATT, Q, L.k_cache, L.v_cache, s, n, nullptr, n + s, c.n_heads, c.n_kv_heads, Dh));
       TRY(linear_residual_norm(L.proj, ATT, L.proj_b, L.ln2_g, L.ln2_b));
-      TRY(launch_linear_gemm(Hb, L.fc, XN, s, L.fc_b, nullptr, gpt2 ? CTHIP_ACT_GELU : CTHIP_ACT_NONE, prec));
       const float *hin = Hb;
-      if (!gpt2) {
-        if (L.fc_pairs) TRY(launch_swiglu_pairs(G, Hb, (int64_t)s * F));
-        else TRY(launch_prologue(G, Hb, F, CTHIP_PRO_SWIGLU, nullptr, nullptr, 0.0f, 2 * (int64_t)F, s));
+      if (!gpt2 && L.fc_pairs && (2 * F) % 4 == 0) {  // SwiGLU in the epilogue of the gate|up launch
+        TRY(launch_linear_gemm(G, L.fc, XN, s, L.fc_b, nullptr, kActSwigluPairs, prec));
         hin = G;
+      } else {
+        TRY(launch_linear_gemm(Hb, L.fc, XN, s, L.fc_b, nullptr, gpt2 ? CTHIP_ACT_GELU : CTHIP_ACT_NONE, prec));
+        if (!gpt2) {
+          if (L.fc_pairs) TRY(launch_swiglu_pairs(G, Hb, (int64_t)s * F));
+          else TRY(launch_prologue(G, Hb, F, CTHIP_PRO_SWIGLU, nullptr, nullptr, 0.0f, 2 * (int64_t)F, s));
+          hin = G;
+        }
       }
       const bool last = l + 1 == c.n_layers;
       TRY(linear_residual_norm(L.fc2, hin, L.fc2_b, last ? nullptr : d->layers[l + 1].ln1_g, last ? nullptr : d->layers[l + 1].ln1_b));

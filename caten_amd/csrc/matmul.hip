@@ -38,6 +38,7 @@ struct GemmArgs {
   // rm x rn tiles, one per XCD (workgroup i is dispatched to XCD i % 8), so that every L2 holds only
   // its region's rows of A and columns of B
   int tm, tn, rx, rm, rn;
+  int pairs;        // 1: columns (2j, 2j + 1) are (gate, up) and C (M, N / 2) gets silu(gate) * up
   int routed;       // 1: whole tiles go to route.dst[...] instead of C (see GemmRoute)
   GemmRoute route;
 };
@@ -142,6 +143,15 @@ __device__ __forceinline__ void store_tile(const GemmArgs &a, const float *Cs, i
     const float4 v4 = *(const float4 *)(Cs + lr * LDC + 4 * c4);
     float v[4] = {v4.x, v4.y, v4.z, v4.w};
     float *o = dst + (int64_t)row * ldd + (col - cbase);
+    if (a.pairs) {  // N is a multiple of 4 and K is not split (the launcher sees to both)
+      if (a.bias) {
+        const float4 bb = *(const float4 *)(a.bias + col);
+        v[0] += bb.x, v[1] += bb.y, v[2] += bb.z, v[3] += bb.w;
+      }
+      *(float2 *)(a.C + (int64_t)row * (N >> 1) + (col >> 1)) =
+          make_float2(apply_act(CTHIP_ACT_SILU, v[0]) * v[1], apply_act(CTHIP_ACT_SILU, v[2]) * v[3]);
+      continue;
+    }
     if (vec) {
       if (!plain) {
         if (a.bias) {
@@ -992,7 +1002,7 @@ int launch_gemm(GemmArgs a, int bmode, int precision, float *static_ws, size_t s
     int ks = quant ? (int)(cus / tiles) : (int)((tiles * 2 <= cus ? cus * 2 : cus * 3 / 2) / tiles);
     if (ks > nsteps / 3) ks = nsteps / 3;
     if (ks > 16) ks = 16;
-    if (a.routed) ks = 1;  // routed tiles are stored by the workgroup that computed them
+    if (a.routed || a.pairs) ks = 1;  // routed / paired tiles are stored by the workgroup that computed them
     if (ks > 1) {
       const int steps_per = (nsteps + ks - 1) / ks;
       a.kper = steps_per * 64;
@@ -1122,6 +1132,11 @@ int launch_linear_gemm(float *y, const WMat *w, const float *x, int m, const flo
   a.N = (int)w->rows;
   a.K = (int)w->cols;
   a.act = act;
+  if (act == kActSwigluPairs) {
+    if (a.N % 4 || residual || route) return fail(CTHIP_E_BAD_ARG, "launch_linear_gemm: paired SwiGLU epilogue with %d rows, a residual or a route", a.N);
+    a.act = CTHIP_ACT_NONE;
+    a.pairs = 1;
+  }
   if (route) {
     for (int i = 0; i < 3; i++)
       if (route->c0[i] != INT_MAX && (route->c0[i] % 128 != 0 || !route->dst[i] || route->ld[i] <= 0))

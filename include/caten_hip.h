@@ -241,7 +241,9 @@ int cthip_rope(float *out, const float *x, int B, int S, int H, int Dh, float ba
 /* scaled-dot-product-attention (external/llm/layers.lisp:3-5) of S query rows
  * (S,H,Dh) at positions start_pos..start_pos+S-1 against a KV cache laid out
  * (max_len, Hkv, Dh) (layers.lisp:19-33) holding T = start_pos+S rows, with the
- * causal mask of layers.lisp:83 applied.  out (S,H,Dh). */
+ * causal mask of layers.lisp:83 applied.  out (S,H,Dh).  From 32 rows on the products run on the matrix cores:
+ * with two bf16 terms per operand (2^-16 of a product dropped), or with fp32 operands when option
+ * "gemm_precision" is 0. */
 int cthip_sdpa_cached(float *out, const float *q, const float *k_cache, const float *v_cache,
                       int S, int start_pos, int H, int Hkv, int Dh);
 

@@ -293,7 +293,9 @@ int launch_reduce_norm(float *y, float *xout, const float *parts, int nparts, in
   if (!reduce_norm_supported(n, nparts)) return fail(CTHIP_E_BAD_ARG, "reduce + norm: rows of %d with %d shares", n, nparts);
   ReduceNormArgs a = {y, xout, parts, nparts, part_stride, bias, resid, g, b, eps, rows, n};
   hipStream_t st = state().stream;
-  if (((n / 4 + 63) / 64) * reduce_norm_bucket(nparts) > 32) {  // four wavefronts per row
+  // four wavefronts per row where one cannot hold the row's shares, and for a prompt's few rows of some width: the
+  // pass is a single memory round trip, and four times the threads ask for it four times as wide
+  if (((n / 4 + 63) / 64) * reduce_norm_bucket(nparts) > 32 || (rows <= 2048 && n >= 512)) {
     const int vplw = (n / 4 + 255) / 256;
     dim3 gridw((unsigned)rows), blockw(256);
 #define RW3(MODE, V, Z) hipLaunchKernelGGL((k_reduce_norm_wide<MODE, V, Z>), gridw, blockw, 0, st, a)

@@ -1171,8 +1171,21 @@ struct KernelRenderer {
           double flo, fhi;
           const Sx *ub = upper_bound(n);
           if (ub && const_value(n.upfrom, flo) && const_value(*ub, fhi) && flo == floor(flo) && fhi == floor(fhi)) {
-            const long long l = (long long)flo, h = (long long)fhi, per = (h - l + 63) / 64;
-            if (per > 0 && per <= 32) {
+            const long long l = (long long)flo, h = (long long)fhi, per = (h - l + 63) / 64, quads = (h - l) / 4;
+            if ((h - l) % 4 == 0 && quads >= 64 && (quads + 63) / 64 <= 8) {
+              // a row of whole quads, at least one per lane: a lane owns 4 CONSECUTIVE elements per pass, so its four
+              // loads (and stores) of a stride-1 operand are one 128-bit access after the compiler has merged them
+              const long long per4 = (quads + 63) / 64;
+              const bool ragged = quads % 64 != 0;
+              o += pad() + "#pragma unroll\n";
+              o += pad() + "for (int " + n.idx + "_i=0; " + n.idx + "_i<" + std::to_string(per4) + "; " + n.idx + "_i++) {" +
+                   (ragged ? " const bool " + n.idx + "_q=_lane+64*" + n.idx + "_i<" + std::to_string(quads) + ";" : "") + "\n";
+              o += pad() + "#pragma unroll\n";
+              o += pad() + "for (int " + n.idx + "_k=0; " + n.idx + "_k<4; " + n.idx + "_k++) { const int " + n.idx + "=" + std::to_string(l) +
+                   "+4*(_lane+64*" + n.idx + "_i)+" + n.idx + "_k;" + (ragged ? " if (" + n.idx + "_q) {" : "") + "\n";
+              closers.push_back(ragged ? "}}}" : "}}");
+              done = true;
+            } else if (per > 0 && per <= 32) {
               // a static row of at most 32 elements per lane: a counted loop, unrolled, so that the loops over the
               // same row share their loads (inputs are __restrict__) and the row is read once
               const bool ragged = (h - l) % 64 != 0;

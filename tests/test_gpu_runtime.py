@@ -272,8 +272,10 @@ def test_rendered_rowwise_kernels_match_oracle(oracle):
 
 @pytest.mark.parametrize("n", [768, 700, 64, 5])
 def test_rendered_softmax_static_shape(oracle, n):
-    """A static-shape row reduction is rendered as counted, unrolled lane-strided loops (ragged rows get a guard on
-    the element index); the result must equal the dynamic-shape kernel's, i.e. the oracle's softmax."""
+    """A static-shape row reduction is rendered as counted, unrolled loops: a lane owns four consecutive elements per
+    pass when the row is whole quads, at least one per lane (the compiler merges them into 128-bit accesses), one
+    element per pass otherwise; ragged rows get a guard.  The result must equal the dynamic-shape kernel's, i.e.
+    the oracle's softmax."""
     import caten_amd as ca
     from caten_amd import blueprints
     from caten_amd.buffer import HipBuffer, make_buffer, open_buffer, transfer_from_array, transfer_into_array
@@ -282,9 +284,15 @@ def test_rendered_softmax_static_shape(oracle, n):
     rt = ca.HipRuntime()
     r = ca.HipRenderer()
     src = r.render_kernel(item)
-    trips = (n + 63) // 64
-    assert src.count("#pragma unroll") == 3 and src.count(f"_gid1_i<{trips};") == 3
-    assert (f"if (_gid1<{n})" in src) == (n % 64 != 0)
+    if n % 4 == 0 and n // 4 >= 64:
+        quads = n // 4
+        trips = (quads + 63) // 64
+        assert src.count("#pragma unroll") == 6 and src.count(f"_gid1_i<{trips};") == 3 and src.count("_gid1_k<4;") == 3
+        assert (f"_gid1_q=_lane+64*_gid1_i<{quads};" in src) == (quads % 64 != 0)
+    else:
+        trips = (n + 63) // 64
+        assert src.count("#pragma unroll") == 3 and src.count(f"_gid1_i<{trips};") == 3
+        assert (f"if (_gid1<{n})" in src) == (n % 64 != 0)
     r.compile_kernel([item])
     x = np.random.default_rng(n).normal(0, 3, (rows, n)).astype(np.float32)
     bx = make_buffer([rows, n], [n, 1], "float32", device=HipBuffer)

@@ -1,7 +1,8 @@
 #!/usr/bin/env python3
 """Timings of the single fused items on one MI355X (`python bench_items.py`):
 the benchmark configurations `!relu(!matmul A B)` at 1024^3 fp32 and the row ops (LayerNorm -> softmax and
-GELU(tanh) over fp32 (64,1024,768)), each against the roofline that bounds it.  HIP events on the
+GELU(tanh) over fp32 (64,1024,768)), each against the roofline that bounds it; the row ops also against a
+device-to-device copy of the same array, the streaming rate this box actually reaches.  HIP events on the
 library's stream; inputs resident on the device.  Every timed item's output is checked on sampled rows against an
 fp64 NumPy evaluation of the same formula before its figure is printed."""
 from __future__ import annotations
@@ -119,13 +120,20 @@ def main():
         return run
     items.append(("softmax (64,1024,768), RENDERED from its blueprint, dynamic shape", rendered(it, by, rows, d, bx)))
     items.append(("softmax (64,1024,768), RENDERED from its blueprint, static shape", rendered(its, by, bx)))
+    # the streaming ceiling of this box: a device-to-device copy of the same array (the same bytes read and written)
+    copy_us = _time(lib, lambda: _lib.check(lib.cthip_d2d(y.ptr, x.ptr, rows * d * 4)))
+    if not np.array_equal(y.numpy()[rs], xh[rs]):
+        raise SystemExit("bench_items: the device-to-device copy did not copy")
+    copy_gbs = nbytes / (copy_us * 1e-6) / 1e9
+    out.append({"item": "device-to-device copy (64,1024,768): the measured streaming ceiling", "us": copy_us, "achieved": copy_gbs,
+                "unit": "GB/s", "peak": 8000.0, "frac": copy_gbs / 8000.0, "bytes": nbytes})
     for name, fn in items:
         us = _time(lib, fn)
         key = [k for k in want if name.startswith(k)]
         _check(name, y.numpy()[rs], want[key[0]] if key else want["softmax ("], 1e-3, 1e-5)
         gbs = nbytes / (us * 1e-6) / 1e9
         out.append({"item": name, "us": us, "achieved": gbs, "unit": "GB/s", "peak": 8000.0, "frac": gbs / 8000.0,
-                    "bytes": nbytes})
+                    "frac_of_copy": gbs / copy_gbs, "bytes": nbytes})
     for o in out:
         print(json.dumps(o))
 

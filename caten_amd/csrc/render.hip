@@ -38,6 +38,7 @@
 #include <string.h>
 
 #include <algorithm>
+#include <functional>
 #include <map>
 #include <string>
 #include <vector>
@@ -304,11 +305,16 @@ struct Rend {
     return "0";
   }
 
+  // element reads that the kernel holds in registers: the rendered reference -> the register that has it
+  std::map<std::string, std::string> held;
+
   std::string aref(const Sx &e) {
     if (e.n() < 2) { err = "(aref ID [INDEX])"; return "0"; }
     const std::string &name = e.v[1].s;
     if (e.n() == 2 || e.v[2].is_sym("nil")) return name;
-    return name + "[" + expr(e.v[2], "int64") + "]";
+    const std::string ref = name + "[" + expr(e.v[2], "int64") + "]";
+    auto h = held.find(ref);
+    return h == held.end() ? ref : h->second;
   }
 
   // render-expr / %render-node dispatch (renderer.lisp:331-411)
@@ -1159,7 +1165,46 @@ struct KernelRenderer {
     // bounded: row loops of dynamic length are emitted as 32 counted, unrolled, guarded passes (the caller has
     // checked at run time that the row has at most 64 * 32 elements), so that, as for a static row, the loops
     // over the same row can share their loads and the row is read once
+    // The loops over one dynamic row read the same elements.  The compiler merges equal loads only over a short
+    // distance, and a load that follows a store to an unqualified pointer is repeated, one round trip per
+    // element; so the elements that the row's loops read from the kernel's INPUT arrays (never written here) are
+    // loaded once, into registers, by a pass of their own in front of the first loop, and the loops read those.
+    // Only loops with the first one's index name and bound take part (their pass counters mean the same element).
+    auto hold_row = [&](int first, const std::string &head, const std::string &idx, const std::string &ub_s, int passes, std::string &out,
+                        const std::string &ind) {
+      std::vector<std::pair<std::string, std::string>> refs;  // rendered reference, element type
+      std::function<void(const Sx &)> walk = [&](const Sx &e) {
+        if (e.call("aref") && e.n() >= 3 && !e.v[2].is_sym("nil")) {
+          const int g = arg_pos(it, e.v[1].s);
+          if (g >= 0 && it.globals[g].pointer && it.globals[g].type == "input" && uses(e.v[2], idx)) {
+            const std::string ref = R.aref(e);
+            bool seen = false;
+            for (const auto &r : refs) seen = seen || r.first == ref;
+            if (!seen) refs.push_back({ref, cdtypes().at(it.globals[g].dtype)});
+          }
+          return;
+        }
+        if (e.kind == Sx::LIST)
+          for (const Sx &c : e.v) walk(c);
+      };
+      for (const auto &kv : dyn_rows) {
+        const BpNode &f = b[kv.first];
+        if (f.idx != idx) continue;
+        if (R.expr(*upper_bound(f), "int64") != ub_s) return;  // the same name over another range: hold nothing
+        for (int q = kv.first + 1; q < hi && b[q].t != BpNode::ENDFOR; q++)
+          if (b[q].t == BpNode::EXPR) walk(b[q].rhs);
+      }
+      (void)first;
+      if (refs.empty() || refs.size() > 4) return;
+      for (size_t k = 0; k < refs.size(); k++) out += ind + refs[k].second + " _h" + std::to_string(k) + "[" + std::to_string(passes) + "];\n";
+      out += ind + "#pragma unroll\n";
+      out += ind + head;
+      for (size_t k = 0; k < refs.size(); k++) out += " _h" + std::to_string(k) + "[" + idx + "_i] = " + refs[k].first + ";";
+      out += " }\n";
+      for (size_t k = 0; k < refs.size(); k++) R.held[refs[k].first] = "_h" + std::to_string(k) + "[" + idx + "_i]";
+    };
     auto emit_body = [&](int bounded) {  // 0: lane-strided loops; N: dynamic rows as N counted passes
+    R.held.clear();
     int depth = 0;
     std::string guard;  // inside a counted pass of a dynamic row: the name of its "this element exists" flag
     std::vector<std::string> closers;
@@ -1200,9 +1245,11 @@ struct KernelRenderer {
             // every pass reads unconditionally (the index is clamped to the row's last element) and only its
             // effects are guarded: the loads of the loops over one row are then the same expressions and are shared
             const std::string ub_s = R.expr(*upper_bound(n), "int64");
+            const std::string head = "for (int " + n.idx + "_i=0; " + n.idx + "_i<" + std::to_string(bounded) + "; " + n.idx + "_i++) { const bool " + n.idx +
+                                     "_ok=_lane+64*" + n.idx + "_i<(" + ub_s + "); const int " + n.idx + "=" + n.idx + "_ok ? _lane+64*" + n.idx + "_i : (int)(" + ub_s + ")-1;";
+            if (pos == dyn_rows.begin()->first) hold_row(pos, head, n.idx, ub_s, bounded, o, pad());
             o += pad() + "#pragma unroll\n";
-            o += pad() + "for (int " + n.idx + "_i=0; " + n.idx + "_i<" + std::to_string(bounded) + "; " + n.idx + "_i++) { const bool " + n.idx +
-                 "_ok=_lane+64*" + n.idx + "_i<(" + ub_s + "); const int " + n.idx + "=" + n.idx + "_ok ? _lane+64*" + n.idx + "_i : (int)(" + ub_s + ")-1;\n";
+            o += pad() + head + "\n";
             closers.push_back("}");
             guard = n.idx + "_ok";
             done = true;
@@ -1242,14 +1289,21 @@ struct KernelRenderer {
         if (wave && depth == 0 && !n.declare && global_write) stmt = "if (_lane == 0) { " + stmt + " }";  // every lane holds the value; one stores it
         if (depth == 1 && !guard.empty()) {
           // the value is computed outside the guard, on the clamped index the other loops use, so that it is shared
-          if (global_write && n.writes.size() == 1)
+          if (global_write && n.writes.size() == 1 && !uses(n.rhs, ref_name(n.writes[0]))) {
+            // a pass beyond the row repeats the store of the row's last element, with the same value: no guard at
+            // all (a guarded store takes the loads it depends on into its branch, one round trip each)
+          } else if (global_write && n.writes.size() == 1)
             stmt = "{ const " + cdtypes().at(n.dtype) + " _w = " + R.expr(n.rhs, n.dtype) + "; if (" + guard + ") { " + lhs + " = _w; } }";
           else if (global_write) stmt = "if (" + guard + ") { " + stmt + " }";
-          else if (!n.declare && n.writes.size() == 1) stmt = lhs + " = " + guard + " ? (" + R.expr(n.rhs, n.dtype) + ") : " + lhs + ";";
+          else if (!n.declare && n.writes.size() == 1)
+            // (as a statement of its own: inside the conditional operator the reads would be conditional as well, and a
+            // conditional load waits for its answer before the next one is asked for)
+            stmt = "{ const " + cdtypes().at(n.dtype) + " _w = " + R.expr(n.rhs, n.dtype) + "; " + lhs + " = " + guard + " ? _w : " + lhs + "; }";
         }
         o += pad() + stmt + "\n";
       }
     }
+    R.held.clear();
     };
     if (dyn_rows.size() < 2) dyn_rows.clear();  // a row that is walked once gains nothing from being held
     for (const auto &kv : dyn_rows) {            // row loops with nothing but statements inside, and a non-empty row

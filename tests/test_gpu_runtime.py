@@ -178,8 +178,10 @@ def test_rendered_rowwise_kernels_match_oracle(oracle):
     r = ca.HipRenderer()
     src = r.render_kernel(item)
     # rows became wavefronts: the three row loops are strided by the 64 lanes, the two reductions end in a butterfly;
-    # rows of at most 256 ... 2048 elements take copies of the body with 4 ... 32 counted passes
-    assert src.count("for (int") == 21 and src.count("+=64") == 3 and "blockIdx.x" in src and "(n) <= 2048" in src
+    # rows of at most 256 ... 2048 elements take copies of the body with 4 ... 32 counted passes, each behind a pass
+    # that loads the row's elements of the input into registers once (the three loops then read those)
+    assert src.count("for (int") == 27 and src.count("+=64") == 3 and "blockIdx.x" in src and "(n) <= 2048" in src
+    assert src.count("_h0[_gid1_i] = val_x[((n*_gid0)+_gid1)];") == 6 and src.count("val_x[") == 6 + 3
     assert "m = ct_wave_max_f(m);" in src and "s = ct_wave_add_f(s);" in src
     r.compile_kernel([item])
     rows, n = 300, 77
@@ -658,3 +660,53 @@ def test_rendered_softmax_dynamic_rows_short_and_long(oracle, rows, n):
         _lib.check(lib.cthip_set_option(b"render_routes", 1))
     # the reference's own softmax tolerance (test-llm.lisp:64-80): the lanes add a 5000-element row in another order
     assert np.allclose(got, oracle.softmax(x), atol=1e-5, rtol=1e-6)
+
+
+@pytest.mark.parametrize("rows,n", [(5, 77), (3, 256), (4, 300), (2, 2048), (2, 2100)])
+def test_rendered_dynamic_rows_with_an_update_in_place_and_two_inputs(rows, n):
+    """Two loops over a row of run-time length: s = sum_j x[j] * g[j], then y[j] = y[j] + s * x[j].  The counted
+    passes hold x and g in registers (loaded once), and the second loop's store reads the array it writes, so it
+    has to stay guarded: a pass beyond the row must not add to the row's last element a second time."""
+    import caten_amd as ca
+    from caten_amd import _lib
+    print(f"case: rendered dynamic update in place {rows}x{n}", flush=True)
+    A = lambda id_, idx: {"op": "AREF", "id": id_, "index": idx}  # noqa: E731
+    add = lambda *a: {"op": "ADD", "args": list(a)}  # noqa: E731
+    mul = lambda *a: {"op": "MUL", "args": list(a)}  # noqa: E731
+    lt = lambda a, b: {"op": "<", "args": [a, b]}  # noqa: E731
+    idx = add(mul("n", "_gid0"), "_gid1")
+    item = {"name": "fused_axpy_rows", "blueprint": [
+        {"type": "DEFINE-GLOBAL", "id": "val_y", "dtype": "float32", "pointer_p": True, "arg_type": "output", "nrank": 2},
+        {"type": "DEFINE-GLOBAL", "id": "rows", "dtype": "int64", "pointer_p": False, "arg_type": "shape", "nrank": 0},
+        {"type": "DEFINE-GLOBAL", "id": "n", "dtype": "int64", "pointer_p": False, "arg_type": "shape", "nrank": 0},
+        {"type": "DEFINE-GLOBAL", "id": "val_x", "dtype": "float32", "pointer_p": True, "arg_type": "input", "nrank": 2},
+        {"type": "DEFINE-GLOBAL", "id": "val_g", "dtype": "float32", "pointer_p": True, "arg_type": "input", "nrank": 1},
+        {"type": "FOR", "idx": "_gid0", "upfrom": 0, "below": lt("_gid0", "rows"), "by": 1},
+        {"type": "EXPR", "writes": [A("s", None)], "expr": 0.0, "declare_type": True, "dtype": "float32"},
+        {"type": "FOR", "idx": "_gid1", "upfrom": 0, "below": lt("_gid1", "n"), "by": 1},
+        {"type": "EXPR", "writes": [A("s", None)], "expr": add("s", mul(A("val_x", idx), A("val_g", "_gid1"))), "dtype": "float32",
+         "reduction": True},
+        {"type": "ENDFOR", "idx": "_gid1"},
+        {"type": "FOR", "idx": "_gid1", "upfrom": 0, "below": lt("_gid1", "n"), "by": 1},
+        {"type": "EXPR", "writes": [A("val_y", idx)], "expr": add(A("val_y", idx), mul("s", A("val_x", idx))), "dtype": "float32"},
+        {"type": "ENDFOR", "idx": "_gid1"},
+        {"type": "ENDFOR", "idx": "_gid0"},
+    ]}
+    src = ca.HipRenderer().render_kernel(item)
+    # both inputs held, the output (read and written) not; its store keeps the guard in the counted passes
+    assert src.count("_h0[_gid1_i] = val_x[") == 6 and src.count("_h1[_gid1_i] = val_g[") == 6
+    assert src.count("if (_gid1_ok) { val_y[") == 6
+    rng = np.random.default_rng(n)
+    x = rng.normal(0, 1, (rows, n)).astype(np.float32)
+    g = rng.normal(0, 1, n).astype(np.float32)
+    y0 = rng.normal(0, 1, (rows, n)).astype(np.float32)
+    lib = _lib.load()
+    _lib.check(lib.cthip_set_option(b"render_routes", 0))
+    try:
+        (got,), prog = _run_item(ca, item, [y0.copy(), rows, n, x, g])
+        assert prog.last_route == "rendered"
+    finally:
+        _lib.check(lib.cthip_set_option(b"render_routes", 1))
+    s = (x.astype(np.float64) * g).sum(-1, keepdims=True)
+    want = y0 + s * x
+    assert np.allclose(got, want, rtol=1e-4, atol=1e-4)

@@ -714,25 +714,26 @@ __global__ __launch_bounds__(256 + 64 * NPW) void k_gemm_qpc(GemmArgs a) {
 
 // ---------------------------------------------------------------------------------------------
 // fp32-operand MFMA GEMM (v_mfma_f32_32x32x2_f32): the products are fp32 products, only the summation
-// order differs from a scalar loop.  Same skeleton as k_gemm_split -- 64x64 tile per 256-thread workgroup,
-// 2x2 wavefronts, two LDS buffers, three register sets of global loads in flight, one barrier per step,
-// XCD regions, split-K -- with K-steps of 32 and the operands kept as fp32 in LDS, k-major ([k][m], [k][n]):
+// order differs from a scalar loop.  This kernel takes PACKED WEIGHTS (N rows x K, any of the five formats,
+// dequantised to fp32 while staging); a (K,N) fp32 matrix takes k_gemm_f32pc below.  64x64 tile per 256-thread
+// workgroup, 2x2 wavefronts, two LDS buffers, three register sets of global loads in flight, one barrier per
+// step, XCD regions, split-K, K-steps of 32, the operands kept as fp32 in LDS, k-major ([k][m], [k][n]):
 // lane l of a wavefront reads A[row l%32][k = 2s + l/32] and B[k = 2s + l/32][col l%32], i.e. 32
-// consecutive floats per half-wavefront.  A (and packed weights) arrive k-contiguous and are transposed by
-// the staging writes; a (K,N) row-major B is copied as it is.
+// consecutive floats per half-wavefront.  A and the weights arrive k-contiguous and are transposed by
+// the staging writes.
 struct FRegsA {
   float4 v0, v1;  // units tid and tid + 256 of the 64 x 8 float4 of a K-step
 };
 struct FRegsB {
-  uint4 r0, r1;      // row-major B: two float4; packed weights: the raw bytes of 8 consecutive k of one row
+  uint4 r0, r1;      // packed weights: the raw bytes of 8 consecutive k of one row; row-major B: two float4 (rows k, k + 2)
   unsigned short d;  // block scale (quantised weights)
 };
 
-template <int BMODE, bool AL>
+template <bool AL>
 __global__ __launch_bounds__(256) void k_gemm_f32(GemmArgs a) {
-  // row pitches: odd where the staging writes are transposing scalar writes (k varies fastest over the lanes,
-  // so k * pitch has to spread over the banks), a multiple of 4 where they are float4 rows
-  constexpr int BM = 64, BN = 64, BK = 32, LDA = BM + 1, LDB = BMODE == B_ROWMAJOR ? BN + 4 : BN + 1;
+  // odd row pitches: the staging writes are transposing scalar writes (k varies fastest over the lanes, so
+  // k * pitch has to spread over the banks)
+  constexpr int BM = 64, BN = 64, BK = 32, LDA = BM + 1, LDB = BN + 1;
   constexpr int kABytes = 2 * BK * LDA * 4, kBBytes = 2 * BK * LDB * 4, kCBytes = BM * (BN + 4) * 4;
   __shared__ __align__(16) unsigned char smem[kABytes + kBBytes > kCBytes ? kABytes + kBBytes : kCBytes];
   float(*As)[BK][LDA] = (float(*)[BK][LDA])smem;
@@ -756,20 +757,12 @@ __global__ __launch_bounds__(256) void k_gemm_f32(GemmArgs a) {
     const int row = m0 + (u >> 3), k = kbeg + k0 + 4 * (u & 7);
     return load4<AL>(a.A + (int64_t)row * ldk + k, row < M ? clamp04(K - k) : 0);
   };
-  auto load_b_rows = [&](int u, int k0) {  // row-major B, unit u: k = u / 16, n = 4 (u % 16) .. +3
-    const int k = kbeg + k0 + (u >> 4), n = n0 + 4 * (u & 15);
-    const float4 v = load4<AL>(a.B + (int64_t)k * N + n, k < K ? clamp04(N - n) : 0);
-    return make_uint4(__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z), __float_as_uint(v.w));
-  };
   auto fetch = [&](int k0, FRegsA &ra, FRegsB &rb) {
     ra.v0 = load_a(tid, k0);
     ra.v1 = load_a(tid + 256, k0);
     rb.r0 = rb.r1 = make_uint4(0u, 0u, 0u, 0u);
     rb.d = 0;
-    if (BMODE == B_ROWMAJOR) {
-      rb.r0 = load_b_rows(tid, k0);
-      rb.r1 = load_b_rows(tid + 256, k0);
-    } else {
+    {
       // packed weights: weight row tid / 4, k = 8 (tid % 4) .. +7 of the step.  AL: rows are a multiple of 8
       // wide (quantised rows always are), so the 8 are inside the row or past its end
       const int n = n0 + (tid >> 2), k = kbeg + k0 + 8 * (tid & 3);
@@ -818,10 +811,7 @@ __global__ __launch_bounds__(256) void k_gemm_f32(GemmArgs a) {
   auto stage = [&](const FRegsA &ra, const FRegsB &rb, int buf) {
     put_a(tid, ra.v0, buf);
     put_a(tid + 256, ra.v1, buf);
-    if (BMODE == B_ROWMAJOR) {
-      *(uint4 *)&Bs[buf][tid >> 4][4 * (tid & 15)] = rb.r0;
-      *(uint4 *)&Bs[buf][(tid + 256) >> 4][4 * (tid & 15)] = rb.r1;
-    } else {
+    {
       float w0, w1, w2, w3, w4, w5, w6, w7;
       if (a.wtype == CTHIP_F32) {
         w0 = __uint_as_float(rb.r0.x), w1 = __uint_as_float(rb.r0.y), w2 = __uint_as_float(rb.r0.z), w3 = __uint_as_float(rb.r0.w);
@@ -909,6 +899,203 @@ __global__ __launch_bounds__(256) void k_gemm_f32(GemmArgs a) {
     Cs[(32 * wm + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * (BN + 4) + 32 * wn + (lane & 31)] = acc[r];
   __syncthreads();
   store_tile<BM, BN, 256>(a, Cs, m0, n0, tid);
+}
+
+// ---------------------------------------------------------------------------------------------
+// The same product with the roles of a step split over wavefronts, as in k_gemm_split: 768 threads, wavefronts
+// 0..3 only multiply, 4..7 only stage A, 8..11 only stage B (one loop per role, one barrier per step).
+//
+// One wavefront per SIMD issues an instruction every 8 cycles or so: with every wavefront staging, requesting and
+// multiplying, a step's hundred-odd other instructions did not fit behind its 16 matrix instructions (64 cycles
+// each) and a step took 1950 cycles instead of 1024.  Here a multiplying wavefront issues nothing but its matrix
+// instructions and the operand reads of the NEXT step (a second register set; the operands of an fp32 matrix
+// instruction are one register each), which needs three LDS buffers: in step i the staging wavefronts fill
+// buffer (i + 2) % 3 while the multiplying ones read buffer (i + 1) % 3 and compute from registers.
+//
+// LDS layout: plane p = 2 (k / 4) + (k % 2) holds, for every row, the PAIR (k, k + 2) -- what a lane (row l % 32,
+// half l / 32) feeds to the two matrix instructions 2j, 2j + 1 of a step is the 8 bytes [plane 2j + l / 32][row],
+// and a staging thread that holds 4 consecutive k of a row writes two such pairs.
+//
+// FULL (the launcher checks): every tile and every K-step of the launch lies inside the operands and their byte
+// offsets fit 32 bits.  A step's requests are then a scalar base, advanced on the scalar unit, plus per-thread
+// offsets computed once -- no address arithmetic, bounds tests or selects on the vector unit, which the staging
+// wavefronts share with the multiplying one of their SIMD.  B is (K,N) row-major here; packed weights (N,K) keep
+// k_gemm_f32, which measured faster on the prompt shapes.
+template <bool AL, bool FULL>
+__global__ __launch_bounds__(768) void k_gemm_f32pc(GemmArgs a) {
+  constexpr int BM = 64, BN = 64, BK = 32, NP = BK / 2;
+  // plane pitches in floats: a multiple of 4 where the staging writes are 16 bytes (B), else 8-byte aligned
+  constexpr int PA = 2 * BM + 2, PB = 2 * BN + 4;
+  constexpr int kABuf = NP * PA * 4, kBBuf = NP * PB * 4;  // bytes per buffer
+  constexpr int kABytes = 3 * kABuf, kBBytes = 3 * kBBuf, kCBytes = BM * (BN + 4) * 4;
+  __shared__ __align__(16) unsigned char smem[kABytes + kBBytes > kCBytes ? kABytes + kBBytes : kCBytes];
+  float *Cs = (float *)smem;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int role = __builtin_amdgcn_readfirstlane(tid) >> 8;  // 0 multiply, 1 stage A, 2 stage B: uniform over a wavefront
+  const int t = tid & 255;                                    // index within the role
+  const int wave = t >> 6, wm = wave >> 1, wn = wave & 1;
+  const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+  if (local >= a.rm * a.rn) return;
+  const int mi = (xcd % a.rx) * a.rm + local % a.rm, ni = (xcd / a.rx) * a.rn + local / a.rm;
+  if (mi >= a.tm || ni >= a.tn) return;
+  const int m0 = mi * BM, n0 = ni * BN;
+  const int M = a.M, N = a.N, ldk = a.K;
+  const int kbeg = blockIdx.y * a.kper;
+  const int K = min(a.K, kbeg + a.kper);
+  const int nsteps = K > kbeg ? (K - kbeg + BK - 1) / BK : 0;
+  v16f acc;
+#pragma unroll
+  for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+
+  if (nsteps > 0) {  // K = 0 comes without operands
+    if (role == 0) {
+      // ---- multiply: registers of step i were read during step i - 1
+      const unsigned abase = 4u * (unsigned)((lane >> 5) * PA + 2 * (32 * wm + (lane & 31)));
+      const unsigned bbase = (unsigned)kABytes + 4u * (unsigned)((lane >> 5) * PB + 2 * (32 * wn + (lane & 31)));
+      auto rd = [&](int buf, float2(&av)[8], float2(&bv)[8]) __attribute__((always_inline)) {
+        const unsigned char *pa = smem + abase + (unsigned)buf * kABuf, *pb = smem + bbase + (unsigned)buf * kBBuf;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+          av[j] = *(const float2 *)(pa + j * (2 * PA * 4));
+          bv[j] = *(const float2 *)(pb + j * (2 * PB * 4));
+        }
+      };
+      // the next step's reads are spread between this step's pairs of matrix instructions
+      auto step = [&](int nbuf, const float2(&av)[8], const float2(&bv)[8], float2(&an)[8], float2(&bn)[8]) __attribute__((always_inline)) {
+        const unsigned char *pa = smem + abase + (unsigned)nbuf * kABuf, *pb = smem + bbase + (unsigned)nbuf * kBBuf;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+          an[j] = *(const float2 *)(pa + j * (2 * PA * 4));
+          bn[j] = *(const float2 *)(pb + j * (2 * PB * 4));
+          __builtin_amdgcn_sched_barrier(0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[j].x, bv[j].x, acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[j].y, bv[j].y, acc, 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        __syncthreads();
+      };
+      float2 a0[8], b0[8], a1[8], b1[8];
+      __syncthreads();  // steps 0 and 1 are staged
+      rd(0, a0, b0);
+      int nb = 1;  // buffer of the step after the current one
+      int i = 0;
+      for (; i + 2 <= nsteps; i += 2) {
+        step(nb, a0, b0, a1, b1);
+        nb = nb == 2 ? 0 : nb + 1;
+        step(nb, a1, b1, a0, b0);
+        nb = nb == 2 ? 0 : nb + 1;
+      }
+      if (i < nsteps) step(nb, a0, b0, a1, b1);
+    } else if (role == 1) {
+      // ---- stage A: units t and t + 256 of the 64 rows x 8 groups of 4 consecutive k
+      unsigned aoff[2];
+#pragma unroll
+      for (int h = 0; h < 2; h++) aoff[h] = 4u * ((unsigned)(m0 + ((t + 256 * h) >> 3)) * (unsigned)ldk + 4u * (unsigned)(t & 7));
+      auto fetch = [&](int k0, FRegsA &ra) __attribute__((always_inline)) {
+        if constexpr (FULL) {
+          const char *ab = (const char *)(a.A + kbeg + min(k0, (nsteps - 1) * BK));  // steps past the end ask for the last one again
+          ra.v0 = *(const float4 *)(ab + aoff[0]);
+          ra.v1 = *(const float4 *)(ab + aoff[1]);
+          return;
+        }
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+          const int u = t + 256 * h, row = m0 + (u >> 3), k = kbeg + k0 + 4 * (u & 7);
+          const float4 v = load4<AL>(a.A + (int64_t)row * ldk + k, row < M ? clamp04(K - k) : 0);
+          if (h == 0) ra.v0 = v;
+          else ra.v1 = v;
+        }
+      };
+      auto stage = [&](const FRegsA &ra, int buf) __attribute__((always_inline)) {
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+          const int u = t + 256 * h, row = u >> 3, g = u & 7;
+          const float4 v = h == 0 ? ra.v0 : ra.v1;
+          float *p = (float *)(smem + buf * kABuf) + 2 * g * PA + 2 * row;
+          *(float2 *)p = make_float2(v.x, v.z);         // k = 4g, 4g + 2
+          *(float2 *)(p + PA) = make_float2(v.y, v.w);  // k = 4g + 1, 4g + 3
+        }
+      };
+      FRegsA r0, r1, r2;
+      fetch(0, r0);
+      fetch(BK, r1);
+      fetch(2 * BK, r2);
+      stage(r0, 0);
+      fetch(3 * BK, r0);
+      stage(r1, 1);
+      fetch(4 * BK, r1);
+      __syncthreads();
+      // step i stages step i + 2 (register set and buffer (i + 2) % 3) and requests step i + 5
+      auto step = [&](int i, FRegsA &rs, int buf) __attribute__((always_inline)) {
+        stage(rs, buf);
+        fetch((i + 5) * BK, rs);
+        __syncthreads();
+      };
+      int i = 0;
+      for (; i + 3 <= nsteps; i += 3) {
+        step(i, r2, 2);
+        step(i + 1, r0, 0);
+        step(i + 2, r1, 1);
+      }
+      if (i < nsteps) step(i, r2, 2);
+      if (i + 1 < nsteps) step(i + 1, r0, 0);
+    } else {
+      // ---- stage B
+      const unsigned boff = 4u * ((unsigned)(4 * (t >> 5) + ((t >> 4) & 1)) * (unsigned)N + (unsigned)(n0 + 4 * (t & 15)));
+      auto fetch = [&](int k0, FRegsB &rb) __attribute__((always_inline)) {
+        rb.d = 0;
+        if constexpr (FULL) {
+          const char *bb = (const char *)(a.B + (int64_t)(kbeg + min(k0, (nsteps - 1) * BK)) * N);
+          rb.r0 = *(const uint4 *)(bb + boff);
+          rb.r1 = *(const uint4 *)(bb + boff + 8u * (unsigned)N);  // two rows further on
+          return;
+        }
+        // thread (g, h, nq): rows k = 4g + h and 4g + 2 + h of the step, columns 4 nq .. + 3
+        const int g = t >> 5, h = (t >> 4) & 1, n = n0 + 4 * (t & 15);
+        const int k1 = kbeg + k0 + 4 * g + h, k2 = k1 + 2;
+        const float4 v1 = load4<AL>(a.B + (int64_t)k1 * N + n, k1 < K ? clamp04(N - n) : 0);
+        const float4 v2 = load4<AL>(a.B + (int64_t)k2 * N + n, k2 < K ? clamp04(N - n) : 0);
+        rb.r0 = make_uint4(__float_as_uint(v1.x), __float_as_uint(v1.y), __float_as_uint(v1.z), __float_as_uint(v1.w));
+        rb.r1 = make_uint4(__float_as_uint(v2.x), __float_as_uint(v2.y), __float_as_uint(v2.z), __float_as_uint(v2.w));
+      };
+      auto stage = [&](const FRegsB &rb, int buf) __attribute__((always_inline)) {
+        float *p = (float *)(smem + kABytes + buf * kBBuf) + (t >> 4) * PB + 2 * 4 * (t & 15);  // plane 2g + h = t / 16
+        *(uint4 *)p = make_uint4(rb.r0.x, rb.r1.x, rb.r0.y, rb.r1.y);
+        *(uint4 *)(p + 4) = make_uint4(rb.r0.z, rb.r1.z, rb.r0.w, rb.r1.w);
+      };
+      FRegsB r0, r1, r2;
+      fetch(0, r0);
+      fetch(BK, r1);
+      fetch(2 * BK, r2);
+      stage(r0, 0);
+      fetch(3 * BK, r0);
+      stage(r1, 1);
+      fetch(4 * BK, r1);
+      __syncthreads();
+      auto step = [&](int i, FRegsB &rs, int buf) __attribute__((always_inline)) {
+        stage(rs, buf);
+        fetch((i + 5) * BK, rs);
+        __syncthreads();
+      };
+      int i = 0;
+      for (; i + 3 <= nsteps; i += 3) {
+        step(i, r2, 2);
+        step(i + 1, r0, 0);
+        step(i + 2, r1, 1);
+      }
+      if (i < nsteps) step(i, r2, 2);
+      if (i + 1 < nsteps) step(i + 1, r0, 0);
+    }
+  }
+  // ---- epilogue: acc[r] is C[row = 8*(r/4) + 4*(l/32) + r%4][col = l%32] of the 32x32 sub-tile ----
+  // (the last step ended with a barrier that every role passed: nobody reads or writes the operand buffers any more)
+  if (role == 0) {
+#pragma unroll
+    for (int r = 0; r < 16; r++)
+      Cs[(32 * wm + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * (BN + 4) + 32 * wn + (lane & 31)] = acc[r];
+  }
+  __syncthreads();
+  store_tile<BM, BN, 768>(a, Cs, m0, n0, tid);
 }
 
 // C = act(sum_z ws[z] + bias) + residual, z in ascending order (the result does not depend on timing)
@@ -1028,11 +1215,14 @@ int launch_gemm(GemmArgs a, int bmode, int precision, float *static_ws, size_t s
     // aligned: every 4 (8 for packed weights) consecutive operand elements a thread asks for are one aligned vector
     const bool al = bmode == B_ROWMAJOR ? (a.K % 4 == 0 && a.N % 4 == 0) : (a.K % 8 == 0);
     if (bmode == B_ROWMAJOR) {
-      if (al) hipLaunchKernelGGL((k_gemm_f32<B_ROWMAJOR, true>), grid, block, 0, st, a);
-      else hipLaunchKernelGGL((k_gemm_f32<B_ROWMAJOR, false>), grid, block, 0, st, a);
+      const bool full = al && a.M % 64 == 0 && a.N % 64 == 0 && a.K % 32 == 0 && a.kper % 32 == 0 && (int64_t)a.M * a.K * 4 < (1ll << 32) &&
+                        ((int64_t)64 * a.N + a.N) * 4 < (1ll << 32);
+      if (full) hipLaunchKernelGGL((k_gemm_f32pc<true, true>), grid, dim3(768), 0, st, a);
+      else if (al) hipLaunchKernelGGL((k_gemm_f32pc<true, false>), grid, dim3(768), 0, st, a);
+      else hipLaunchKernelGGL((k_gemm_f32pc<false, false>), grid, dim3(768), 0, st, a);
     } else {
-      if (al) hipLaunchKernelGGL((k_gemm_f32<B_WMAT, true>), grid, block, 0, st, a);
-      else hipLaunchKernelGGL((k_gemm_f32<B_WMAT, false>), grid, block, 0, st, a);
+      if (al) hipLaunchKernelGGL((k_gemm_f32<true>), grid, block, 0, st, a);
+      else hipLaunchKernelGGL((k_gemm_f32<false>), grid, block, 0, st, a);
     }
   } else if (quant) {
     const int npa = precision == GEMM_BF16X6 ? 3 : precision == GEMM_BF16X3 ? 2 : 1;

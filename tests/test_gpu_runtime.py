@@ -710,3 +710,52 @@ def test_rendered_dynamic_rows_with_an_update_in_place_and_two_inputs(rows, n):
     s = (x.astype(np.float64) * g).sum(-1, keepdims=True)
     want = y0 + s * x
     assert np.allclose(got, want, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("rows,n", [(1, 1), (5, 77), (3, 1024), (4, 256), (41, 25), (130, 300), (1, 1025)])
+@pytest.mark.parametrize("static", [False, True])
+def test_rendered_elementwise_items_four_elements_per_thread(rows, n, static):
+    """Element-wise items (no loop inside the parallel ones): a thread takes four elements 256 apart, whole blocks of
+    1024 without a test and the last one with; operands whose index is the row-major position are addressed by the
+    flat position, others (a bias along the row, a transposed read) through the indices taken apart.
+    y[i][j] = x[i][j] * 2 + b[j] + xt[j][i]."""
+    import caten_amd as ca
+    from caten_amd import _lib
+    print(f"case: rendered element-wise {rows}x{n} static={static}", flush=True)
+    A = lambda id_, idx: {"op": "AREF", "id": id_, "index": idx}  # noqa: E731
+    add = lambda *a: {"op": "ADD", "args": list(a)}  # noqa: E731
+    mul = lambda *a: {"op": "MUL", "args": list(a)}  # noqa: E731
+    lt = lambda a, b: {"op": "<", "args": [a, b]}  # noqa: E731
+    R, N = (rows, n) if static else ("rows", "n")
+    idx = add(mul(N, "_gid0"), "_gid1")
+    idx_t = add(mul(R, "_gid1"), "_gid0")
+    glob = lambda id_, ty, nr: {"type": "DEFINE-GLOBAL", "id": id_, "dtype": "float32", "pointer_p": True, "arg_type": ty, "nrank": nr}  # noqa: E731
+    shape = [] if static else [
+        {"type": "DEFINE-GLOBAL", "id": "rows", "dtype": "int64", "pointer_p": False, "arg_type": "shape", "nrank": 0},
+        {"type": "DEFINE-GLOBAL", "id": "n", "dtype": "int64", "pointer_p": False, "arg_type": "shape", "nrank": 0}]
+    item = {"name": "fused_affine_ew", "blueprint": [glob("val_y", "output", 2)] + shape + [
+        glob("val_x", "input", 2), glob("val_b", "input", 1), glob("val_xt", "input", 2),
+        {"type": "FOR", "idx": "_gid0", "upfrom": 0, "below": lt("_gid0", R), "by": 1},
+        {"type": "FOR", "idx": "_gid1", "upfrom": 0, "below": lt("_gid1", N), "by": 1},
+        {"type": "EXPR", "writes": [A("val_y", idx)], "expr": add(mul(A("val_x", idx), 2.0), A("val_b", "_gid1"), A("val_xt", idx_t)), "dtype": "float32"},
+        {"type": "ENDFOR", "idx": "_gid1"},
+        {"type": "ENDFOR", "idx": "_gid0"},
+    ]}
+    src = ca.HipRenderer().render_kernel(item)
+    assert "val_x[_t]" in src and "val_y[_t] =" in src
+    if rows > 1 and n > 1:  # (a 1 x n or n x 1 array read transposed IS read in row-major order)
+        assert "val_b[_gid1]" in src and "val_xt[_t]" not in src
+    assert "_e < 4" in src and "blockIdx.x * 1024" in src
+    rng = np.random.default_rng(rows * 1000 + n)
+    x = rng.normal(0, 1, (rows, n)).astype(np.float32)
+    bias = rng.normal(0, 1, n).astype(np.float32)
+    xt = rng.normal(0, 1, (n, rows)).astype(np.float32)
+    lib = _lib.load()
+    _lib.check(lib.cthip_set_option(b"render_routes", 0))
+    try:
+        args = [np.zeros((rows, n), np.float32)] + ([] if static else [rows, n]) + [x, bias, xt]
+        (got,), prog = _run_item(ca, item, args)
+        assert prog.last_route == "rendered"
+    finally:
+        _lib.check(lib.cthip_set_option(b"render_routes", 1))
+    assert np.array_equal(got, (x * np.float32(2.0) + bias) + xt.T)

@@ -127,6 +127,14 @@ def main():
     copy_gbs = nbytes / (copy_us * 1e-6) / 1e9
     out.append({"item": "device-to-device copy (64,1024,768): the measured streaming ceiling", "us": copy_us, "achieved": copy_gbs,
                 "unit": "GB/s", "peak": 8000.0, "frac": copy_gbs / 8000.0, "bytes": nbytes})
+    # GELU(tanh) as a RENDERED element-wise kernel (there is no route for it: this is what an item of that shape runs)
+    ig = blueprints.gelu_tanh()
+    igs = blueprints.gelu_tanh("fused_gelu_static", rows, d)
+    rr.render_kernel(ig)
+    rr.render_kernel(igs)
+    rr.compile_kernel([ig, igs])
+    items.append(("GELU(tanh) (64,1024,768), RENDERED from its blueprint, dynamic shape", lambda: ig["compiled_object"](None, by, rows, d, bx)))
+    items.append(("GELU(tanh) (64,1024,768), RENDERED from its blueprint, static shape", lambda: igs["compiled_object"](None, by, bx)))
     for name, fn in items:
         us = _time(lib, fn)
         key = [k for k in want if name.startswith(k)]

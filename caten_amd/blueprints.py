@@ -1,4 +1,4 @@
-"""Blueprints of row-wise Schedule-Items in the dict interchange format of renderer.py, shaped the way Caten
+"""Blueprints of row-wise and element-wise Schedule-Items in the dict interchange format of renderer.py, shaped the way Caten
 lowers them (one kernel, several loops over the row: source/test-suite/test-scheduler.lisp:37-45,
 test-activations.lisp:60-73).  Used by the item benchmark to time RENDERED kernels next to the hand-written ones."""
 from __future__ import annotations
@@ -56,6 +56,28 @@ def softmax_rows(name: str = "fused_softmax", rows: int | None = None, n: int | 
 
 def _neg(a):
     return {"op": "NEG", "args": [a]}
+
+
+def gelu_tanh(name: str = "fused_gelu", rows: int | None = None, n: int | None = None) -> dict:
+    """GELU(tanh) of every element of (rows, n), decomposed the way the reference does (nn/activations.lisp:202-215,
+    3-7; api/high-level-ops.lisp:112-117): 0.5 x (1 + tanh(u)) with u = sqrt(2/pi) (x + 0.044715 x^3),
+    tanh(u) = 2 sigmoid(2u) - 1, sigmoid(z) = recip(1 + exp2(z * -1/ln2)).  Static or dynamic shape as for
+    softmax_rows."""
+    static = rows is not None and n is not None
+    R, N = (rows, n) if static else ("rows", "n")
+    idx = _add(_mul(N, "_gid0"), "_gid1")
+    x = _A("val_x", idx)
+    u = _mul(0.7978845608, _add(x, _mul(0.044715, _mul(x, _mul(x, x)))))
+    sig = {"op": "RECIP", "args": [_add(1.0, {"op": "EXP2", "args": [_mul(_mul(2.0, u), -1.4426950408889634)]})]}
+    shapes = [] if static else [_glob("rows", "shape", 0, "int64"), _glob("n", "shape", 0, "int64")]
+    return {"name": name, "blueprint": [
+        _glob("val_y", "output", 2), *shapes, _glob("val_x", "input", 2),
+        {"type": "FOR", "idx": "_gid0", "upfrom": 0, "below": _lt("_gid0", R), "by": 1},
+        {"type": "FOR", "idx": "_gid1", "upfrom": 0, "below": _lt("_gid1", N), "by": 1},
+        {"type": "EXPR", "writes": [_A("val_y", idx)], "expr": _mul(_mul(0.5, x), _add(1.0, _add(_mul(2.0, sig), -1.0))), "dtype": "float32"},
+        {"type": "ENDFOR", "idx": "_gid1"},
+        {"type": "ENDFOR", "idx": "_gid0"},
+    ]}
 
 
 def _rstd(q, N, eps):

@@ -1205,8 +1205,11 @@ struct KernelRenderer {
     // element; so the elements that the row's loops read from the kernel's INPUT arrays (never written here) are
     // loaded once, into registers, by a pass of their own in front of the first loop, and the loops read those.
     // Only loops with the first one's index name and bound take part (their pass counters mean the same element).
-    auto hold_row = [&](int first, const std::string &head, const std::string &idx, const std::string &ub_s, int passes, std::string &out,
-                        const std::string &ind) {
+    // siblings: the row loops that take part; head / close: what opens and closes one pass over the row (the loops
+    // and any guard, as the row's own loops are opened); dims / slot: the shape of a register array that holds one
+    // value per element of the thread, and the element's place in it
+    auto hold_loops = [&](const std::vector<int> &siblings, const std::string &head, const std::string &close, const std::string &idx,
+                          const std::string &dims, const std::string &slot, int per_thread, std::string &out, const std::string &ind) {
       std::vector<std::pair<std::string, std::string>> refs;  // rendered reference, element type
       std::function<void(const Sx &)> walk = [&](const Sx &e) {
         if (e.call("aref") && e.n() >= 3 && !e.v[2].is_sym("nil")) {
@@ -1222,21 +1225,52 @@ struct KernelRenderer {
         if (e.kind == Sx::LIST)
           for (const Sx &c : e.v) walk(c);
       };
+      for (int f : siblings)
+        for (int q = f + 1; q < hi && b[q].t != BpNode::ENDFOR; q++) {
+          if (b[q].t != BpNode::EXPR) return;  // something else than statements in a row loop: hold nothing
+          walk(b[q].rhs);
+        }
+      if (refs.empty() || refs.size() > 4 || (int)refs.size() * per_thread > 96) return;
+      for (size_t k = 0; k < refs.size(); k++) out += ind + refs[k].second + " _h" + std::to_string(k) + dims + ";\n";
+      out += ind + "#pragma unroll\n";
+      out += ind + head;
+      for (size_t k = 0; k < refs.size(); k++) out += " _h" + std::to_string(k) + slot + " = " + refs[k].first + ";";
+      out += " " + close + "\n";
+      for (size_t k = 0; k < refs.size(); k++) R.held[refs[k].first] = "_h" + std::to_string(k) + slot;
+    };
+    // dynamic rows: the loops with the first one's index name; another range under the same name: hold nothing
+    auto hold_row = [&](int first, const std::string &head, const std::string &idx, const std::string &ub_s, int passes, std::string &out,
+                        const std::string &ind) {
+      std::vector<int> siblings;
       for (const auto &kv : dyn_rows) {
         const BpNode &f = b[kv.first];
         if (f.idx != idx) continue;
-        if (R.expr(*upper_bound(f), "int64") != ub_s) return;  // the same name over another range: hold nothing
-        for (int q = kv.first + 1; q < hi && b[q].t != BpNode::ENDFOR; q++)
-          if (b[q].t == BpNode::EXPR) walk(b[q].rhs);
+        if (R.expr(*upper_bound(f), "int64") != ub_s) return;
+        siblings.push_back(kv.first);
       }
       (void)first;
-      if (refs.empty() || refs.size() > 4) return;
-      for (size_t k = 0; k < refs.size(); k++) out += ind + refs[k].second + " _h" + std::to_string(k) + "[" + std::to_string(passes) + "];\n";
-      out += ind + "#pragma unroll\n";
-      out += ind + head;
-      for (size_t k = 0; k < refs.size(); k++) out += " _h" + std::to_string(k) + "[" + idx + "_i] = " + refs[k].first + ";";
-      out += " }\n";
-      for (size_t k = 0; k < refs.size(); k++) R.held[refs[k].first] = "_h" + std::to_string(k) + "[" + idx + "_i]";
+      hold_loops(siblings, head, "}", idx, "[" + std::to_string(passes) + "]", "[" + idx + "_i]", passes, out, ind);
+    };
+    // static rows: the loops directly inside the row with this loop's index name, which must all have its range;
+    // at least two of them (a row that is walked once gains nothing), and this one the first
+    auto static_siblings = [&](int pos, long long l, long long h) {
+      std::vector<int> sib;
+      int d = 0;
+      for (int q = lo; q < hi; q++) {
+        if (b[q].t == BpNode::FOR) {
+          if (d == 0 && b[q].idx == b[pos].idx) {
+            double fl, fh;
+            const Sx *ub = upper_bound(b[q]);
+            if (!ub || !const_value(b[q].upfrom, fl) || !const_value(*ub, fh) || (long long)fl != l || (long long)fh != h) return std::vector<int>();
+            sib.push_back(q);
+          }
+          d++;
+        } else if (b[q].t == BpNode::ENDFOR) {
+          d--;
+        }
+      }
+      if (sib.size() < 2 || sib[0] != pos) sib.clear();
+      return sib;
     };
     const std::vector<std::pair<std::string, std::string>> *held_flat = nullptr;   // element-wise items: reads held per element
     const std::vector<std::pair<std::string, std::string>> *flat_named = nullptr;  // ... and elements addressed by _t
@@ -1263,21 +1297,35 @@ struct KernelRenderer {
               // loads (and stores) of a stride-1 operand are one 128-bit access after the compiler has merged them
               const long long per4 = (quads + 63) / 64;
               const bool ragged = quads % 64 != 0;
+              const std::string h1 = "for (int " + n.idx + "_i=0; " + n.idx + "_i<" + std::to_string(per4) + "; " + n.idx + "_i++) {" +
+                                     (ragged ? " const bool " + n.idx + "_q=_lane+64*" + n.idx + "_i<" + std::to_string(quads) + ";" : "");
+              const std::string h2 = "for (int " + n.idx + "_k=0; " + n.idx + "_k<4; " + n.idx + "_k++) { const int " + n.idx + "=" + std::to_string(l) +
+                                     "+4*(_lane+64*" + n.idx + "_i)+" + n.idx + "_k;" + (ragged ? " if (" + n.idx + "_q) {" : "");
+              if (depth == 0) {
+                const std::vector<int> sib = static_siblings(pos, l, h);
+                if (!sib.empty())
+                  hold_loops(sib, h1 + "\n" + pad() + "#pragma unroll\n" + pad() + h2, ragged ? "}}}" : "}}", n.idx, "[" + std::to_string(per4) + "][4]",
+                             "[" + n.idx + "_i][" + n.idx + "_k]", (int)per4 * 4, o, pad());
+              }
               o += pad() + "#pragma unroll\n";
-              o += pad() + "for (int " + n.idx + "_i=0; " + n.idx + "_i<" + std::to_string(per4) + "; " + n.idx + "_i++) {" +
-                   (ragged ? " const bool " + n.idx + "_q=_lane+64*" + n.idx + "_i<" + std::to_string(quads) + ";" : "") + "\n";
+              o += pad() + h1 + "\n";
               o += pad() + "#pragma unroll\n";
-              o += pad() + "for (int " + n.idx + "_k=0; " + n.idx + "_k<4; " + n.idx + "_k++) { const int " + n.idx + "=" + std::to_string(l) +
-                   "+4*(_lane+64*" + n.idx + "_i)+" + n.idx + "_k;" + (ragged ? " if (" + n.idx + "_q) {" : "") + "\n";
+              o += pad() + h2 + "\n";
               closers.push_back(ragged ? "}}}" : "}}");
               done = true;
             } else if (per > 0 && per <= 32) {
               // a static row of at most 32 elements per lane: a counted loop, unrolled, so that the loops over the
               // same row share their loads (inputs are __restrict__) and the row is read once
               const bool ragged = (h - l) % 64 != 0;
+              const std::string h1 = "for (int " + n.idx + "_i=0; " + n.idx + "_i<" + std::to_string(per) + "; " + n.idx + "_i++) { const int " + n.idx + "=" +
+                                     std::to_string(l) + "+_lane+64*" + n.idx + "_i;" + (ragged ? " if (" + n.idx + "<" + std::to_string(h) + ") {" : "");
+              if (depth == 0) {
+                const std::vector<int> sib = static_siblings(pos, l, h);
+                if (!sib.empty())
+                  hold_loops(sib, h1, ragged ? "}}" : "}", n.idx, "[" + std::to_string(per) + "]", "[" + n.idx + "_i]", (int)per, o, pad());
+              }
               o += pad() + "#pragma unroll\n";
-              o += pad() + "for (int " + n.idx + "_i=0; " + n.idx + "_i<" + std::to_string(per) + "; " + n.idx + "_i++) { const int " +
-                   n.idx + "=" + std::to_string(l) + "+_lane+64*" + n.idx + "_i;" + (ragged ? " if (" + n.idx + "<" + std::to_string(h) + ") {" : "") + "\n";
+              o += pad() + h1 + "\n";
               closers.push_back(ragged ? "}}" : "}");
               done = true;
             }

@@ -289,12 +289,15 @@ def test_rendered_softmax_static_shape(oracle, n):
     if n % 4 == 0 and n // 4 >= 64:
         quads = n // 4
         trips = (quads + 63) // 64
-        assert src.count("#pragma unroll") == 6 and src.count(f"_gid1_i<{trips};") == 3 and src.count("_gid1_k<4;") == 3
+        # three loops over the row, behind one of the same shape that loads the row into registers
+        assert src.count("#pragma unroll") == 8 and src.count(f"_gid1_i<{trips};") == 4 and src.count("_gid1_k<4;") == 4
         assert (f"_gid1_q=_lane+64*_gid1_i<{quads};" in src) == (quads % 64 != 0)
+        assert src.count("_h0[_gid1_i][_gid1_k] = val_x[") == 1 and src.count("val_x[") == 1
     else:
         trips = (n + 63) // 64
-        assert src.count("#pragma unroll") == 3 and src.count(f"_gid1_i<{trips};") == 3
+        assert src.count("#pragma unroll") == 4 and src.count(f"_gid1_i<{trips};") == 4
         assert (f"if (_gid1<{n})" in src) == (n % 64 != 0)
+        assert src.count("_h0[_gid1_i] = val_x[") == 1 and src.count("val_x[") == 1
     r.compile_kernel([item])
     x = np.random.default_rng(n).normal(0, 3, (rows, n)).astype(np.float32)
     bx = make_buffer([rows, n], [n, 1], "float32", device=HipBuffer)

@@ -71,17 +71,16 @@ __device__ __forceinline__ unsigned pack_bf16(float x0, float x1) {
 }
 // 4 consecutive k -> NP planes of 4 bf16: plane 0 = bf16(x), plane p = bf16(what planes 0..p-1 miss)
 template <int NP>
-__device__ __forceinline__ void split4(const float x[4], uint2 *pl) {
-  float r[4] = {x[0], x[1], x[2], x[3]};
+__device__ __forceinline__ void split4(float r0, float r1, float r2, float r3, uint2 *pl) {
 #pragma unroll
   for (int p = 0; p < NP; p++) {
-    pl[p].x = pack_bf16(r[0], r[1]);
-    pl[p].y = pack_bf16(r[2], r[3]);
+    pl[p].x = pack_bf16(r0, r1);
+    pl[p].y = pack_bf16(r2, r3);
     if (p + 1 < NP) {  // exact: the difference of a float and its own leading bits
-      r[0] -= __uint_as_float(pl[p].x << 16);
-      r[1] -= __uint_as_float(pl[p].x & 0xffff0000u);
-      r[2] -= __uint_as_float(pl[p].y << 16);
-      r[3] -= __uint_as_float(pl[p].y & 0xffff0000u);
+      r0 -= __uint_as_float(pl[p].x << 16);
+      r1 -= __uint_as_float(pl[p].x & 0xffff0000u);
+      r2 -= __uint_as_float(pl[p].y << 16);
+      r3 -= __uint_as_float(pl[p].y & 0xffff0000u);
     }
   }
 }
@@ -262,9 +261,8 @@ __global__ __launch_bounds__(NS == 1 ? 256 : 768) void k_gemm_split(GemmArgs a) 
   };
   auto stage_a = [&](const ARegs &ra, int buf) __attribute__((always_inline)) {
     auto put = [&](int i, const float4 v) __attribute__((always_inline)) {
-      const float x[4] = {v.x, v.y, v.z, v.w};
       uint2 pl[NP];
-      split4<NP>(x, pl);
+      split4<NP>(v.x, v.y, v.z, v.w, pl);
 #pragma unroll
       for (int p = 0; p < NP; p++)
         *(uint2 *)&As[buf][p][ar + 16 * i][8 * ((akq >> 1) ^ swz(ar + 16 * i)) + 4 * (akq & 1)] = pl[p];
@@ -278,17 +276,17 @@ __global__ __launch_bounds__(NS == 1 ? 256 : 768) void k_gemm_split(GemmArgs a) 
     if (BMODE == W_ROWMAJOR) {
       // column 4 bnq + i gets its 4 consecutive k: a 4x4 transpose in registers
       auto put = [&](int i, unsigned x0, unsigned x1, unsigned x2, unsigned x3) __attribute__((always_inline)) {
-        const float x[4] = {__uint_as_float(x0), __uint_as_float(x1), __uint_as_float(x2), __uint_as_float(x3)};
         uint2 pl[NP];
-        split4<NP>(x, pl);
+        split4<NP>(__uint_as_float(x0), __uint_as_float(x1), __uint_as_float(x2), __uint_as_float(x3), pl);
 #pragma unroll
         for (int p = 0; p < NP; p++)
           *(uint2 *)&Bs[buf][p][4 * bnq + i][8 * ((bkq >> 1) ^ swz(4 * bnq + i)) + 4 * (bkq & 1)] = pl[p];
       };
-      put(0, rb.v[0].x, rb.v[1].x, rb.v[2].x, rb.v[3].x);
-      put(1, rb.v[0].y, rb.v[1].y, rb.v[2].y, rb.v[3].y);
-      put(2, rb.v[0].z, rb.v[1].z, rb.v[2].z, rb.v[3].z);
-      put(3, rb.v[0].w, rb.v[1].w, rb.v[2].w, rb.v[3].w);
+      const uint4 q0 = rb.v[0], q1 = rb.v[BRegs<BMODE>::NV > 1 ? 1 : 0], q2 = rb.v[BRegs<BMODE>::NV > 2 ? 2 : 0], q3 = rb.v[BRegs<BMODE>::NV > 3 ? 3 : 0];
+      put(0, q0.x, q1.x, q2.x, q3.x);
+      put(1, q0.y, q1.y, q2.y, q3.y);
+      put(2, q0.z, q1.z, q2.z, q3.z);
+      put(3, q0.w, q1.w, q2.w, q3.w);
     } else {
       float x[16];
       if (BMODE == W_F32) {
@@ -315,8 +313,8 @@ __global__ __launch_bounds__(NS == 1 ? 256 : 768) void k_gemm_split(GemmArgs a) 
 #pragma unroll
       for (int j = 0; j < 2; j++) {
         uint2 p0[NP], p1[NP];
-        split4<NP>(x + 8 * j, p0);
-        split4<NP>(x + 8 * j + 4, p1);
+        split4<NP>(x[8 * j], x[8 * j + 1], x[8 * j + 2], x[8 * j + 3], p0);
+        split4<NP>(x[8 * j + 4], x[8 * j + 5], x[8 * j + 6], x[8 * j + 7], p1);
 #pragma unroll
         for (int p = 0; p < NP; p++)
           *(uint4 *)&Bs[buf][p][wr][8 * ((2 * wkc + j) ^ swz(wr))] = make_uint4(p0[p].x, p0[p].y, p1[p].x, p1[p].y);
@@ -357,7 +355,7 @@ __global__ __launch_bounds__(NS == 1 ? 256 : 768) void k_gemm_split(GemmArgs a) 
   if (nsteps > 0 && !ROLES) {
     ARegs ra0, ra1, ra2;  // separate objects with named members: every set stays in registers
     BRegs<BMODE> rb0, rb1, rb2;
-    auto step = [&](int i, ARegs &ran, BRegs<BMODE> &rbn) {
+    auto step = [&](int i, ARegs &ran, BRegs<BMODE> &rbn) __attribute__((always_inline)) {
       stage_a(ran, (i + 1) & 1);
       stage_b(rbn, (i + 1) & 1);
       fetch_a((i + 1 + NSET) * BK, ran);
@@ -579,7 +577,7 @@ __global__ __launch_bounds__(256 + 64 * NPW) void k_gemm_qpc(GemmArgs a) {
     for (int i = 0; i < NA; i++) {
       const float x[4] = {ra.v[i].x, ra.v[i].y, ra.v[i].z, ra.v[i].w};
       uint2 pl[NPA];
-      split4<NPA>(x, pl);
+      split4<NPA>(x[0], x[1], x[2], x[3], pl);
       const int row = ar + (PT / 16) * i;
 #pragma unroll
       for (int p = 0; p < NPA; p++) *(uint2 *)&As[buf][p][row][8 * ((akq >> 1) ^ swz(row)) + 4 * (akq & 1)] = pl[p];

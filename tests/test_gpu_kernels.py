@@ -425,6 +425,7 @@ def test_sdpa_cached(ops, oracle, S, start, H, Hkv, Dh):
 
 # ------------------------------------------------------------------ matmul (MFMA)
 @pytest.mark.parametrize("M,N,K", [(256, 256, 256), (64, 64, 32), (3, 5, 7), (65, 33, 17), (100, 768, 1024), (1, 64, 64),
+                                   (128, 128, 64), (64, 128, 160), (70, 64, 128), (64, 192, 96),  # 2, 5, 4, 3 K-steps of 32
                                    (100, 70, 2000), (33, 65, 1030), (64, 64, 4096)])  # the last three split K
 def test_matmul_relu_vs_oracle(ops, oracle, M, N, K):
     print(f"case: matmul {M}x{N}x{K}", flush=True)

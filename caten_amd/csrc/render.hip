@@ -996,6 +996,17 @@ struct KernelRenderer {
         for (const Sx &w : n.writes) locals[ref_name(w)] = true;
   }
 
+  // an index made of loop indices, shape arguments and constants only: no temporary of the body (it may be set
+  // after the place a hoisted read would go) and no element read inside it
+  bool plain_index(const Sx &e) const {
+    if (e.kind == Sx::SYM) return !locals.count(e.s);
+    if (e.kind != Sx::LIST) return true;
+    if (e.call("aref")) return false;
+    for (size_t k = (e.call("cast") || e.call("const")) ? 2 : 1; k < e.n(); k++)
+      if (!plain_index(e.v[k])) return false;
+    return true;
+  }
+
   // how many leading FOR nodes of the body (a perfect nest) are data-parallel
   int parallel_prefix() {
     const std::vector<BpNode> &b = it.body;
@@ -1214,7 +1225,7 @@ struct KernelRenderer {
       std::function<void(const Sx &)> walk = [&](const Sx &e) {
         if (e.call("aref") && e.n() >= 3 && !e.v[2].is_sym("nil")) {
           const int g = arg_pos(it, e.v[1].s);
-          if (g >= 0 && it.globals[g].pointer && it.globals[g].type == "input" && uses(e.v[2], idx)) {
+          if (g >= 0 && it.globals[g].pointer && it.globals[g].type == "input" && uses(e.v[2], idx) && plain_index(e.v[2])) {
             const std::string ref = R.aref(e);
             bool seen = false;
             for (const auto &r : refs) seen = seen || r.first == ref;
@@ -1482,7 +1493,7 @@ struct KernelRenderer {
           if (e.call("where")) return;
           if (e.call("aref") && e.n() >= 3 && !e.v[2].is_sym("nil")) {
             const int g = arg_pos(it, e.v[1].s);
-            if (g >= 0 && it.globals[g].pointer && it.globals[g].type == "input") {
+            if (g >= 0 && it.globals[g].pointer && it.globals[g].type == "input" && plain_index(e.v[2])) {
               const std::string ref = R.aref(e);
               bool seen = false;
               for (const auto &r : refs) seen = seen || r.first == ref;

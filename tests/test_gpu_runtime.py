@@ -762,3 +762,44 @@ def test_rendered_elementwise_items_four_elements_per_thread(rows, n, static):
     finally:
         _lib.check(lib.cthip_set_option(b"render_routes", 1))
     assert np.array_equal(got, (x * np.float32(2.0) + bias) + xt.T)
+
+
+@pytest.mark.parametrize("ntok,d", [(5, 8), (300, 64), (17, 1000)])
+def test_rendered_gather_keeps_its_indexed_read_behind_the_index(ntok, d):
+    """An element-wise item whose read goes through a temporary of the body (row = (int) idx[i]; y[i][j] = W[row][j]):
+    the reads hoisted in front of the statements are only those whose index is made of loop indices and shape
+    arguments; W[row * d + j] has to stay where `row` is known."""
+    import caten_amd as ca
+    from caten_amd import _lib
+    print(f"case: rendered gather {ntok}x{d}", flush=True)
+    A = lambda id_, idx: {"op": "AREF", "id": id_, "index": idx}  # noqa: E731
+    add = lambda *a: {"op": "ADD", "args": list(a)}  # noqa: E731
+    mul = lambda *a: {"op": "MUL", "args": list(a)}  # noqa: E731
+    lt = lambda a, b: {"op": "<", "args": [a, b]}  # noqa: E731
+    glob = lambda id_, ty, nr, dt="float32": {"type": "DEFINE-GLOBAL", "id": id_, "dtype": dt, "pointer_p": nr > 0, "arg_type": ty, "nrank": nr}  # noqa: E731
+    item = {"name": "fused_gather", "blueprint": [
+        glob("val_y", "output", 2), glob("ntok", "shape", 0, "int64"), glob("d", "shape", 0, "int64"),
+        glob("val_w", "input", 2), glob("val_i", "input", 1),
+        {"type": "FOR", "idx": "_gid0", "upfrom": 0, "below": lt("_gid0", "ntok"), "by": 1},
+        {"type": "FOR", "idx": "_gid1", "upfrom": 0, "below": lt("_gid1", "d"), "by": 1},
+        {"type": "EXPR", "writes": [A("row", None)], "expr": {"op": "CAST", "dtype": "int64", "args": [A("val_i", "_gid0")]},
+         "declare_type": True, "dtype": "int64"},
+        {"type": "EXPR", "writes": [A("val_y", add(mul("d", "_gid0"), "_gid1"))], "expr": A("val_w", add(mul("d", "row"), "_gid1")), "dtype": "float32"},
+        {"type": "ENDFOR", "idx": "_gid1"},
+        {"type": "ENDFOR", "idx": "_gid0"},
+    ]}
+    src = ca.HipRenderer().render_kernel(item)
+    assert "_e < 4" in src and "_h0[_e] = val_i[_gid0];" in src  # the index array is read ahead ...
+    assert "] = val_w[" not in src.replace("val_y[_t] = val_w[", "") and "val_y[_t] = val_w[((d*row)+_gid1)];" in src  # ... the table is not
+    rng = np.random.default_rng(ntok)
+    vocab = 37
+    w = rng.normal(0, 1, (vocab, d)).astype(np.float32)
+    idx = rng.integers(0, vocab, ntok).astype(np.float32)
+    lib = _lib.load()
+    _lib.check(lib.cthip_set_option(b"render_routes", 0))
+    try:
+        (got,), prog = _run_item(ca, item, [np.zeros((ntok, d), np.float32), ntok, d, w, idx])
+        assert prog.last_route == "rendered"
+    finally:
+        _lib.check(lib.cthip_set_option(b"render_routes", 1))
+    assert np.array_equal(got, w[idx.astype(np.int64)])

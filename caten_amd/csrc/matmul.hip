@@ -2,12 +2,13 @@
 // fused per source/test-suite/test-scheduler.lisp:140-163) and Linear over m > 1 rows (prefill,
 // source/nn/linear.lisp:3-17) with the weights still packed (dequantised while they are staged).
 //
-// One 256-thread workgroup (4 wavefronts, 2x2) owns a 64x64 tile of C; each wavefront accumulates a
-// 32x32 sub-tile in 16 accumulator registers, with v_mfma_f32_32x32x2_f32 (k_gemm_f32, fp32 operands)
-// or v_mfma_f32_32x32x16_bf16 (k_gemm_split, operands split into bf16 terms, fp32 accumulation).  Operands are
-// staged through two LDS buffers with three K-steps of global loads in flight; 1024x1024 outputs give 256
-// workgroups = one per compute unit.  Quantised weights take k_gemm_qpc: 64x128 tiles, 512 threads, half of
-// them staging and half multiplying.  Finished tiles leave through LDS as whole rows (store_tile).
+// A workgroup owns a 64x64 tile of C; four of its wavefronts (2x2) accumulate a 32x32 sub-tile each in 16
+// accumulator registers, with v_mfma_f32_32x32x2_f32 (k_gemm_f32pc / k_gemm_f32, fp32 operands) or
+// v_mfma_f32_32x32x16_bf16 (k_gemm_split, operands split into bf16 terms, fp32 accumulation), while eight more
+// stage the operands (k_gemm_f32, packed weights with fp32 operands, is the one kernel whose four wavefronts do
+// both).  Operands go through LDS buffers with three K-steps of global loads in flight; 1024x1024 outputs give
+// 256 workgroups = one per compute unit.  Quantised weights take k_gemm_qpc: 64x128 tiles, four multiplying and
+// eight staging wavefronts.  Finished tiles leave through LDS as whole rows (store_tile).
 #include <hip/hip_bf16.h>
 
 #include "common.h"
@@ -53,7 +54,7 @@ struct GemmArgs {
 // products above 2^-24: fp32-grade results at a sixth of the bf16 rate, which is still 2.6 times the
 // fp32-operand MFMA peak.
 //
-// One 256-thread workgroup (2x2 wavefronts) owns a 64x64 tile of C and walks K in steps of 64.  The
+// A workgroup (2x2 multiplying wavefronts + eight staging ones) owns a 64x64 tile of C and walks K in steps of 64.  The
 // fp32 (or packed) operands of a step are converted ONCE per workgroup on their way into LDS, which
 // holds them k-contiguous per row in bf16, 16-byte chunks swizzled by row so that neither the operand
 // reads nor the staging writes collide on banks.  Two LDS buffers and three register sets keep the
@@ -106,10 +107,13 @@ struct ARegs {  // one K-step of A held by a thread: rows ar + 16 i
   float4 v0, v1, v2, v3;
 };
 
+// (a native vector type: copies of HIP's uint4 struct between address spaces can become memcpy calls, and register
+// sets written that way stay in scratch memory)
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
 template <int BMODE>
 struct BRegs {  // one K-step of B held by a thread between its request and its conversion
   static constexpr int NV = (BMODE == W_ROWMAJOR || BMODE == W_F32) ? 4 : (BMODE == W_F16 ? 2 : 1);
-  uint4 v[NV];
+  v4u v[NV];
 };
 
 // LDS rows are 64 bf16 = eight 16-byte chunks; chunk c of row r is stored at position c ^ swz(r), which
@@ -179,8 +183,7 @@ __device__ __forceinline__ void store_tile(const GemmArgs &a, const float *Cs, i
 }
 
 template <int BMODE, int NS, bool AL>
-__global__ __launch_bounds__(NS == 1 ? 256 : 768) void k_gemm_split(GemmArgs a) {
-  constexpr bool ROLES = NS != 1;  // one bf16 term per operand: too little to multiply per step to pay for the roles
+__global__ __launch_bounds__(768) void k_gemm_split(GemmArgs a) {
   constexpr int BM = 64, BN = 64, BK = 64, LDK = BK, NP = (NS == 1) ? 1 : (NS == 3) ? 2 : 3;
   constexpr int NSET = 3;  // register sets = K-steps of global loads in flight
   constexpr int kOpBytes = 2 * NP * BM * LDK * 2, kCBytes = BM * (BN + 4) * 4;
@@ -189,13 +192,12 @@ __global__ __launch_bounds__(NS == 1 ? 256 : 768) void k_gemm_split(GemmArgs a) 
   typedef unsigned short(*OpT)[NP][BM][LDK];
   OpT As = (OpT)smem, Bs = (OpT)(smem + kOpBytes);
   float *Cs = (float *)smem;
-  // ROLES: twelve wavefronts in three roles, one of each per SIMD: 0..3 multiply the current step out of one LDS
+  // Twelve wavefronts in three roles, one of each per SIMD: 0..3 multiply the current step out of one LDS
   // buffer, 4..7 stage the next step's A into the other (and request the step three further on), 8..11 do the same
   // for B.  Each role runs its own loop (same number of barriers on every path), so a stager's waits count the
   // younger requests of ITS loop and the conversions run under the other wavefronts' matrix instructions.
-  // Otherwise four wavefronts that each stage, request and multiply in turn.
   const int ltid = threadIdx.x, lane = ltid & 63;
-  const int role = ROLES ? __builtin_amdgcn_readfirstlane(ltid) >> 8 : 0;  // uniform over a wavefront, and known to be
+  const int role = __builtin_amdgcn_readfirstlane(ltid) >> 8;  // uniform over a wavefront, and known to be
   const int tid = ltid & 255;                                  // index within the role
   const int wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
   const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
@@ -233,7 +235,7 @@ __global__ __launch_bounds__(NS == 1 ? 256 : 768) void k_gemm_split(GemmArgs a) 
       auto ld = [&](int j) __attribute__((always_inline)) {
         const int k = kbeg + k0 + 4 * bkq + j, n = n0 + 4 * bnq;
         const float4 v = load4<AL>(a.B + (int64_t)k * N + n, k < K ? clamp04(N - n) : 0);
-        return make_uint4(__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z), __float_as_uint(v.w));
+        return v4u{__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z), __float_as_uint(v.w)};
       };
       // constant indices only: the sets must stay in registers
       rb.v[0] = ld(0);
@@ -246,14 +248,14 @@ __global__ __launch_bounds__(NS == 1 ? 256 : 768) void k_gemm_split(GemmArgs a) 
       const bool ok = n < N && k < K;
       const int64_t e = (int64_t)n * ldk + k;  // element index of the chunk
       if (BMODE == W_F32) {
-        const uint4 *src = ok ? (const uint4 *)((const float *)a.wq + e) : (const uint4 *)g_zeros;
+        const v4u *src = ok ? (const v4u *)((const float *)a.wq + e) : (const v4u *)g_zeros;
         const int st = ok ? 1 : 0;  // the zeros are 32 bytes long
         rb.v[0] = src[0];
         rb.v[BRegs<BMODE>::NV > 1 ? 1 : 0] = src[st];
         rb.v[BRegs<BMODE>::NV > 2 ? 2 : 0] = src[2 * st];
         rb.v[BRegs<BMODE>::NV > 3 ? 3 : 0] = src[3 * st];
       } else if (BMODE == W_F16) {
-        const uint4 *src = ok ? (const uint4 *)((const unsigned short *)a.wq + e) : (const uint4 *)g_zeros;
+        const v4u *src = ok ? (const v4u *)((const unsigned short *)a.wq + e) : (const v4u *)g_zeros;
         rb.v[0] = src[0];
         rb.v[BRegs<BMODE>::NV > 1 ? 1 : 0] = src[1];
       }
@@ -282,7 +284,7 @@ __global__ __launch_bounds__(NS == 1 ? 256 : 768) void k_gemm_split(GemmArgs a) 
         for (int p = 0; p < NP; p++)
           *(uint2 *)&Bs[buf][p][4 * bnq + i][8 * ((bkq >> 1) ^ swz(4 * bnq + i)) + 4 * (bkq & 1)] = pl[p];
       };
-      const uint4 q0 = rb.v[0], q1 = rb.v[BRegs<BMODE>::NV > 1 ? 1 : 0], q2 = rb.v[BRegs<BMODE>::NV > 2 ? 2 : 0], q3 = rb.v[BRegs<BMODE>::NV > 3 ? 3 : 0];
+      const v4u q0 = rb.v[0], q1 = rb.v[BRegs<BMODE>::NV > 1 ? 1 : 0], q2 = rb.v[BRegs<BMODE>::NV > 2 ? 2 : 0], q3 = rb.v[BRegs<BMODE>::NV > 3 ? 3 : 0];
       put(0, q0.x, q1.x, q2.x, q3.x);
       put(1, q0.y, q1.y, q2.y, q3.y);
       put(2, q0.z, q1.z, q2.z, q3.z);
@@ -292,7 +294,7 @@ __global__ __launch_bounds__(NS == 1 ? 256 : 768) void k_gemm_split(GemmArgs a) 
       if (BMODE == W_F32) {
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-          const uint4 q = rb.v[j];
+          const v4u q = rb.v[j];
           x[4 * j + 0] = __uint_as_float(q.x);
           x[4 * j + 1] = __uint_as_float(q.y);
           x[4 * j + 2] = __uint_as_float(q.z);
@@ -301,7 +303,7 @@ __global__ __launch_bounds__(NS == 1 ? 256 : 768) void k_gemm_split(GemmArgs a) 
       } else if (BMODE == W_F16) {
 #pragma unroll
         for (int j = 0; j < 2; j++) {
-          const uint4 q = rb.v[BRegs<BMODE>::NV > 1 ? j : 0];
+          const v4u q = rb.v[BRegs<BMODE>::NV > 1 ? j : 0];
           const unsigned dw[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
           for (int t = 0; t < 4; t++) {
@@ -352,37 +354,7 @@ __global__ __launch_bounds__(NS == 1 ? 256 : 768) void k_gemm_split(GemmArgs a) 
   // No conditions inside a staging step (past the last one the requests read zeros and stage them) and no exit
   // inside the loops: the waits before a set is staged then count on a known number of younger requests.
   static_assert(NSET == 3, "the loops below are unrolled by hand over the register sets");
-  if (nsteps > 0 && !ROLES) {
-    ARegs ra0, ra1, ra2;  // separate objects with named members: every set stays in registers
-    BRegs<BMODE> rb0, rb1, rb2;
-    auto step = [&](int i, ARegs &ran, BRegs<BMODE> &rbn) __attribute__((always_inline)) {
-      stage_a(ran, (i + 1) & 1);
-      stage_b(rbn, (i + 1) & 1);
-      fetch_a((i + 1 + NSET) * BK, ran);
-      fetch_b((i + 1 + NSET) * BK, rbn);
-      mma(i & 1);
-      __syncthreads();
-    };
-    fetch_a(0, ra0);
-    fetch_b(0, rb0);
-    fetch_a(BK, ra1);
-    fetch_b(BK, rb1);
-    fetch_a(2 * BK, ra2);
-    fetch_b(2 * BK, rb2);
-    stage_a(ra0, 0);
-    stage_b(rb0, 0);
-    fetch_a(3 * BK, ra0);
-    fetch_b(3 * BK, rb0);
-    __syncthreads();
-    int i = 0;
-    for (; i + NSET <= nsteps; i += NSET) {
-      step(i, ra1, rb1);
-      step(i + 1, ra2, rb2);
-      step(i + 2, ra0, rb0);
-    }
-    if (i < nsteps) step(i, ra1, rb1);
-    if (i + 1 < nsteps) step(i + 1, ra2, rb2);
-  } else if (nsteps > 0) {  // K = 0 comes without operands
+  if (nsteps > 0) {  // K = 0 comes without operands
     if (role == 0) {
       __syncthreads();
       for (int i = 0; i < nsteps; i++) {
@@ -441,7 +413,7 @@ __global__ __launch_bounds__(NS == 1 ? 256 : 768) void k_gemm_split(GemmArgs a) 
       Cs[(32 * wm + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * (BN + 4) + 32 * wn + (lane & 31)] = acc[r];
   }
   __syncthreads();
-  store_tile<BM, BN, ROLES ? 768 : 256>(a, Cs, m0, n0, ltid);
+  store_tile<BM, BN, 768>(a, Cs, m0, n0, ltid);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1247,7 +1219,7 @@ int launch_gemm(GemmArgs a, int bmode, int precision, float *static_ws, size_t s
 #define SPLIT3(MODE, AL)                                                                                      \
   if (precision == GEMM_BF16X6) hipLaunchKernelGGL((k_gemm_split<MODE, 6, AL>), grid, dim3(768), 0, st, a);      \
   else if (precision == GEMM_BF16X3) hipLaunchKernelGGL((k_gemm_split<MODE, 3, AL>), grid, dim3(768), 0, st, a); \
-  else hipLaunchKernelGGL((k_gemm_split<MODE, 1, AL>), grid, dim3(256), 0, st, a)
+  else hipLaunchKernelGGL((k_gemm_split<MODE, 1, AL>), grid, dim3(768), 0, st, a)
 #define SPLIT(MODE)      \
   case MODE:             \
     if (al) {            \

@@ -367,6 +367,21 @@ def test_unary(ops, oracle):
     assert ops.gelu(np.zeros(0, np.float32)).shape == (0,)
 
 
+@pytest.mark.parametrize("n", [1, 1023, 1024, 1025, 5000])
+def test_unary_on_pointers_that_are_not_16_byte_aligned(ops, oracle, n):
+    """Arrays that start 4 bytes into an allocation take the element-wise form of the kernel (whole blocks of 1024
+    and a tail) instead of the 128-bit one."""
+    from caten_amd import _lib
+    from caten_amd.ops import DeviceArray
+    print(f"case: unaligned unary n={n}", flush=True)
+    x = np.linspace(-4, 4, n + 1).astype(np.float32)
+    dx, dy = DeviceArray.from_numpy(x), DeviceArray((n + 1,), np.float32)
+    _lib.check(_lib.load().cthip_unary(_lib.ACT_GELU, dy.ptr + 4, dx.ptr + 4, n))
+    got = dy.numpy()
+    assert got[0] == 0.0  # the element in front of the output stays as allocated
+    close(got[1:], oracle.gelu_tanh(x[1:]), 1e-5, 1e-6)
+
+
 def test_embedding_and_argmax(ops, oracle):
     rng = np.random.default_rng(41)
     W = rng.normal(size=(523, 48)).astype(np.float32)

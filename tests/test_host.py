@@ -361,3 +361,30 @@ def test_conv_pool_and_backward_items_render():
     assert "_negative_infinity" in pool and "ct_max(m," in pool
     bwd = r.render_kernel(bp.linear_relu_backward())
     assert "ct_wave_add_f(acc)" in bwd and "_gid1+=64" in bwd
+
+
+def test_elementwise_and_row_items_hold_their_reads_in_registers():
+    """What the renderer does for memory parallelism, checked on the emitted source and compiled for gfx950:
+    element-wise items take four elements per thread with the reads issued first and flat operands addressed by
+    the flat position; row items load the row's input elements once, in front of the first loop over the row."""
+    from caten_amd import HipRenderer, blueprints as bp
+    r = HipRenderer()
+    g = bp.gelu_tanh()
+    src = r.render_kernel(g)
+    assert src.count("_e < 4") == 8  # (32-bit, 64-bit) x (whole block, last block) x (reads, statements)
+    assert "_h0[_e] = val_x[_t];" in src and "val_y[_t] = " in src and "val_x[((n*_gid0)+_gid1)]" not in src
+    assert "blockIdx.x * 1024 + 1024 <= _total" in src
+    gs = bp.gelu_tanh("fused_gelu_static", 64, 768)
+    src = r.render_kernel(gs)
+    assert "_h0[_e] = val_x[_t];" in src and "% (unsigned)(768)" in src  # a static bound is divided by the compiler
+    ln = bp.layernorm_rows("ln_static", True, 1e-5, 64, 768)
+    src = r.render_kernel(ln)
+    # three arrays held as [passes][4] quads; the three loops over the row read no global memory but the store
+    for k, name in enumerate(("val_x", "val_g", "val_b")):
+        assert src.count(f"_h{k}[_gid1_i][_gid1_k] = {name}[") == 1 and src.count(f"{name}[") == 1
+    sd = bp.softmax_rows()
+    src = r.render_kernel(sd)
+    assert src.count("_h0[_gid1_i] = val_x[((n*_gid0)+_gid1)];") == 6 and src.count("if (_gid1_ok)") == 0
+    assert src.count("m = _gid1_ok ? _w : m;") == 6 and src.count("s = _gid1_ok ? _w : s;") == 6
+    r.compile_kernel([g, gs, ln, sd])
+    assert r.code_object[:4] == b"\x7fELF"

@@ -1223,6 +1223,7 @@ struct KernelRenderer {
                           const std::string &dims, const std::string &slot, int per_thread, std::string &out, const std::string &ind) {
       std::vector<std::pair<std::string, std::string>> refs;  // rendered reference, element type
       std::function<void(const Sx &)> walk = [&](const Sx &e) {
+        if (e.call("where")) return;  // an arm of a `where` may be what keeps an index inside its array: not hoisted
         if (e.call("aref") && e.n() >= 3 && !e.v[2].is_sym("nil")) {
           const int g = arg_pos(it, e.v[1].s);
           if (g >= 0 && it.globals[g].pointer && it.globals[g].type == "input" && uses(e.v[2], idx) && plain_index(e.v[2])) {

@@ -803,3 +803,52 @@ def test_rendered_gather_keeps_its_indexed_read_behind_the_index(ntok, d):
     finally:
         _lib.check(lib.cthip_set_option(b"render_routes", 1))
     assert np.array_equal(got, w[idx.astype(np.int64)])
+
+
+@pytest.mark.parametrize("rows,n", [(3, 70), (5, 256), (2, 700)])
+@pytest.mark.parametrize("static", [False, True])
+def test_rendered_row_with_a_guarded_neighbour_read(rows, n, static):
+    """s = sum_j x[j]; y[j] = s + (0 < j ? x[j - 1] : 0).  The read of the left neighbour is only valid where the
+    `where` selects it (for j = 0 it lies in front of the row, for row 0 in front of the array): it has to stay
+    inside the conditional, while x[j] itself is held in registers."""
+    import caten_amd as ca
+    from caten_amd import _lib
+    print(f"case: rendered guarded neighbour {rows}x{n} static={static}", flush=True)
+    A = lambda id_, idx: {"op": "AREF", "id": id_, "index": idx}  # noqa: E731
+    add = lambda *a: {"op": "ADD", "args": list(a)}  # noqa: E731
+    mul = lambda *a: {"op": "MUL", "args": list(a)}  # noqa: E731
+    lt = lambda a, b: {"op": "<", "args": [a, b]}  # noqa: E731
+    R, N = (rows, n) if static else ("rows", "n")
+    idx = add(mul(N, "_gid0"), "_gid1")
+    left = {"op": "WHERE", "args": [lt(0, "_gid1"), A("val_x", add(idx, -1)), 0.0]}
+    glob = lambda id_, ty, nr, dt="float32": {"type": "DEFINE-GLOBAL", "id": id_, "dtype": dt, "pointer_p": nr > 0, "arg_type": ty, "nrank": nr}  # noqa: E731
+    shape = [] if static else [glob("rows", "shape", 0, "int64"), glob("n", "shape", 0, "int64")]
+    loop = {"type": "FOR", "idx": "_gid1", "upfrom": 0, "below": lt("_gid1", N), "by": 1}
+    item = {"name": "fused_left_neighbour", "blueprint": [glob("val_y", "output", 2)] + shape + [
+        glob("val_x", "input", 2),
+        {"type": "FOR", "idx": "_gid0", "upfrom": 0, "below": lt("_gid0", R), "by": 1},
+        {"type": "EXPR", "writes": [A("s", None)], "expr": 0.0, "declare_type": True, "dtype": "float32"},
+        dict(loop),
+        {"type": "EXPR", "writes": [A("s", None)], "expr": add("s", A("val_x", idx)), "dtype": "float32", "reduction": True},
+        {"type": "ENDFOR", "idx": "_gid1"},
+        dict(loop),
+        {"type": "EXPR", "writes": [A("val_y", idx)], "expr": add("s", left), "dtype": "float32"},
+        {"type": "ENDFOR", "idx": "_gid1"},
+        {"type": "ENDFOR", "idx": "_gid0"},
+    ]}
+    src = ca.HipRenderer().render_kernel(item)
+    assert "] = val_x[((" in src  # the row itself is held ...
+    assert "+-1)]" in src and "] = val_x[(((" not in src  # ... its left neighbour is read where the `where` selects it
+    rng = np.random.default_rng(n)
+    x = rng.normal(0, 1, (rows, n)).astype(np.float32)
+    lib = _lib.load()
+    _lib.check(lib.cthip_set_option(b"render_routes", 0))
+    try:
+        args = [np.zeros((rows, n), np.float32)] + ([] if static else [rows, n]) + [x]
+        (got,), prog = _run_item(ca, item, args)
+        assert prog.last_route == "rendered"
+    finally:
+        _lib.check(lib.cthip_set_option(b"render_routes", 1))
+    leftv = np.concatenate([np.zeros((rows, 1), np.float32), x[:, :-1]], axis=1)
+    want = x.astype(np.float64).sum(-1, keepdims=True) + leftv
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-4)

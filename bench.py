@@ -190,6 +190,20 @@ def main():
     lm_warm = time_lm_head(wms[:1], 200)
     lm_cold = time_lm_head(wms, 25 * len(wms))
     lm_cold["copies"] = len(wms)
+    # the streaming rate this box reaches: a 256 MiB device-to-device copy (read + written: twice that through HBM)
+    ncopy = 256 << 20
+    ca, cb = ops.DeviceArray((ncopy,), np.uint8), ops.DeviceArray((ncopy,), np.uint8)
+    for _ in range(2):
+        _lib.check(lib.cthip_d2d(cb.ptr, ca.ptr, ncopy))
+    _lib.check(lib.cthip_sync())
+    _lib.check(lib.cthip_timer_start())
+    for _ in range(10):
+        _lib.check(lib.cthip_d2d(cb.ptr, ca.ptr, ncopy))
+    _lib.check(lib.cthip_timer_stop(C.byref(ms)))
+    copy_gbs = 2.0 * ncopy / (ms.value * 1e-3 / 10) / 1e9
+    lm_cold["frac_of_copy"] = lm_cold["achieved"] / copy_gbs
+    ca.free()
+    cb.free()
     traffic = profile_traffic(args.model, args.kind)
 
     res = {
@@ -206,6 +220,8 @@ def main():
         # the whole decode step: every launch of one token, HIP events on the library's stream around K steps
         "roofline": {"bound": "hbm", "achieved": step_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": step_gbs / HBM_PEAK_GBS, "traffic": traffic,
+                     "measured_copy": {"achieved": copy_gbs, "unit": "GB/s", "frac": copy_gbs / HBM_PEAK_GBS,
+                                       "what": "256 MiB device-to-device copy on the library's stream, bytes read + written"},
                      "kernel": "one decode step = one replay of the step's launches (the dequant-in-register Linear "
                                "kernels, attention, argmax), packed weights + norms / biases + embedding rows + KV rows",
                      "bytes_per_launch": step_bytes, "us_per_launch": step_us,

@@ -135,6 +135,18 @@ def main():
     rr.compile_kernel([ig, igs])
     items.append(("GELU(tanh) (64,1024,768), RENDERED from its blueprint, dynamic shape", lambda: ig["compiled_object"](None, by, rows, d, bx)))
     items.append(("GELU(tanh) (64,1024,768), RENDERED from its blueprint, static shape", lambda: igs["compiled_object"](None, by, bx)))
+    # LayerNorm -> softmax as ONE rendered item (five loops over the row)
+    bg = HipBuffer(shape=[d], stride=[1], dtype="float32", nrank=1, value=g.ptr)
+    bb = HipBuffer(shape=[d], stride=[1], dtype="float32", nrank=1, value=b.ptr)
+    il = blueprints.layernorm_softmax_rows()
+    ils = blueprints.layernorm_softmax_rows("fused_layernorm_softmax_static", 1e-5, rows, d)
+    rr.render_kernel(il)
+    rr.render_kernel(ils)
+    rr.compile_kernel([il, ils])
+    items.append(("LayerNorm->softmax (64,1024,768), RENDERED from its blueprint, dynamic shape",
+                  lambda: il["compiled_object"](None, by, rows, d, bx, bg, bb)))
+    items.append(("LayerNorm->softmax (64,1024,768), RENDERED from its blueprint, static shape",
+                  lambda: ils["compiled_object"](None, by, bx, bg, bb)))
     for name, fn in items:
         us = _time(lib, fn)
         key = [k for k in want if name.startswith(k)]

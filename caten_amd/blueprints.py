@@ -124,6 +124,41 @@ def layernorm_rows(name: str = "fused_layernorm", affine: bool = True, eps: floa
     ]}
 
 
+def layernorm_softmax_rows(name: str = "fused_layernorm_softmax", eps: float = 1e-5, rows: int | None = None,
+                           n: int | None = None) -> dict:
+    """softmax(LayerNorm(x) * gamma + beta) over the last axis of (rows, n) as ONE kernel with five loops over the
+    row: mean, biased variance, maximum of the normalised row, sum of exp2, normalise (nn/normalization.lisp:39-58
+    followed by nn/activations.lisp:59-62,107-119 in one Schedule-Item).  Arguments: val_y, [rows, n,] val_x, val_g,
+    val_b."""
+    static = rows is not None and n is not None
+    R, N = (rows, n) if static else ("rows", "n")
+    idx = _add(_mul(N, "_gid0"), "_gid1")
+    xi = _A("val_x", idx)
+    nf = {"op": "CAST", "dtype": "float32", "args": [N]} if not static else float(N)
+    loop = {"type": "FOR", "idx": "_gid1", "upfrom": 0, "below": _lt("_gid1", N), "by": 1}
+    end = {"type": "ENDFOR", "idx": "_gid1"}
+    shapes = [] if static else [_glob("rows", "shape", 0, "int64"), _glob("n", "shape", 0, "int64")]
+    centred = _add(xi, _neg("u"))
+    ln = _add(_mul(_mul(centred, "r"), _A("val_g", "_gid1")), _A("val_b", "_gid1"))
+    ex = {"op": "EXP2", "args": [_mul(_add(ln, _neg("m")), 1.442695)]}
+    red = lambda name, expr: {"type": "EXPR", "writes": [_A(name, None)], "expr": expr, "dtype": "float32", "reduction": True}  # noqa: E731
+    decl = lambda name, expr: {"type": "EXPR", "writes": [_A(name, None)], "expr": expr, "declare_type": True, "dtype": "float32"}  # noqa: E731
+    return {"name": name, "blueprint": [
+        _glob("val_y", "output", 2), *shapes, _glob("val_x", "input", 2), _glob("val_g", "input", 1), _glob("val_b", "input", 1),
+        {"type": "FOR", "idx": "_gid0", "upfrom": 0, "below": _lt("_gid0", R), "by": 1},
+        decl("s", 0.0), dict(loop), red("s", _add("s", xi)), dict(end),
+        decl("u", _mul("s", {"op": "RECIP", "args": [nf]})),
+        decl("q", 0.0), dict(loop), red("q", _add("q", _mul(centred, centred))), dict(end),
+        decl("r", _rstd("q", N, eps)),
+        decl("m", float("-inf")), dict(loop), red("m", {"op": "MAX", "args": ["m", ln]}), dict(end),
+        decl("e", 0.0), dict(loop), red("e", _add("e", ex)), dict(end),
+        dict(loop),
+        {"type": "EXPR", "writes": [_A("val_y", idx)], "expr": _mul(ex, {"op": "RECIP", "args": ["e"]}), "dtype": "float32"},
+        dict(end),
+        {"type": "ENDFOR", "idx": "_gid0"},
+    ]}
+
+
 def rmsnorm_rows(name: str = "fused_rmsnorm", weight: bool = True, eps: float = 1e-5, rows: int | None = None,
                  n: int | None = None) -> dict:
     """RMSNorm over the last axis of (rows, n) (nn/normalization.lisp:78-92): x / sqrt(mean(x^2) + eps) [* w].

@@ -852,3 +852,22 @@ def test_rendered_row_with_a_guarded_neighbour_read(rows, n, static):
     leftv = np.concatenate([np.zeros((rows, 1), np.float32), x[:, :-1]], axis=1)
     want = x.astype(np.float64).sum(-1, keepdims=True) + leftv
     assert np.allclose(got, want, rtol=1e-5, atol=1e-4)
+
+
+@pytest.mark.parametrize("rows,n,static", [(7, 768, True), (7, 768, False), (5, 77, True), (5, 77, False), (3, 1000, False), (2, 2500, False)])
+def test_rendered_layernorm_softmax_in_one_item(oracle, rows, n, static):
+    """LayerNorm -> softmax fused into one Schedule-Item (five loops over the row, three input arrays held in registers)
+    against the oracle's LayerNorm followed by its softmax."""
+    import caten_amd as ca
+    from caten_amd import blueprints as bp
+    print(f"case: rendered layernorm->softmax {rows}x{n} static={static}", flush=True)
+    rng = np.random.default_rng(n + rows)
+    x = rng.normal(0, 2, (rows, n)).astype(np.float32)
+    g = rng.normal(1, 0.1, n).astype(np.float32)
+    b = rng.normal(0, 0.1, n).astype(np.float32)
+    item = bp.layernorm_softmax_rows("ln_sm", 1e-5, rows if static else None, n if static else None)
+    args = [np.zeros((rows, n), np.float32)] + ([] if static else [rows, n]) + [x, g, b]
+    (got,), prog = _run_item(ca, item, args)
+    assert prog.last_route == "rendered"  # no hand-written kernel is recognised for the pair
+    want = oracle.softmax(oracle.layernorm(x, g, b, 1e-5))
+    assert np.allclose(got, want, atol=1e-5, rtol=1e-4)

@@ -67,7 +67,35 @@ def cpu_baseline(cfg, weights, prompt, budget_s, kind, llama):
             break
     return {"value": steps / el, "unit": "tokens/s", "cores": 1, "kind": "port",
             "sample": f"{steps} decode steps after a {len(prompt)}-token prompt, fp32 dequantised weights, "
-                      f"gcc -O3 single thread (what BACKEND=CLANG runs at OMP=0), {el:.1f} s"}
+                      f"gcc -O3 single thread (what BACKEND=CLANG runs at OMP=0), {el:.1f} s",
+            "items": cpu_baseline_items()}
+
+
+def cpu_baseline_items():
+    """The same port on bounded samples of the two single-item configurations that bench_items.py times on the GPU:
+    relu(matmul) at 1024^3 (256 of the 1024 output rows) and the row ops of (64,1024,768) (half of the 65536 rows)."""
+    import oracle
+    rng = np.random.default_rng(0)
+    out = {}
+    A = rng.uniform(-1, 1, (256, 1024)).astype(np.float32)
+    B = rng.uniform(-1, 1, (1024, 1024)).astype(np.float32)
+    t0 = time.perf_counter()
+    oracle.matmul(A, B, relu=True)
+    el = time.perf_counter() - t0
+    out["relu(matmul) 1024^3"] = {"value": 2.0 * 256 * 1024 * 1024 / el / 1e9, "unit": "GFLOP/s", "sample": f"256 of 1024 output rows, {el:.2f} s"}
+    rows, d = 32768, 768
+    x = rng.standard_normal((rows, d), dtype=np.float32)
+    g, b = rng.normal(1, 0.02, d).astype(np.float32), rng.normal(0, 0.02, d).astype(np.float32)
+    t0 = time.perf_counter()
+    oracle.softmax(oracle.layernorm(x, g, b, 1e-5))
+    el = time.perf_counter() - t0
+    out["LayerNorm->softmax (64,1024,768)"] = {"value": 2.0 * rows * d * 4 / el / 1e9, "unit": "GB/s of the fused item's bytes",
+                                               "sample": f"{rows} of 65536 rows, two kernels as the reference runs them, {el:.2f} s"}
+    t0 = time.perf_counter()
+    oracle.gelu_tanh(x)
+    el = time.perf_counter() - t0
+    out["GELU(tanh) (64,1024,768)"] = {"value": 2.0 * rows * d * 4 / el / 1e9, "unit": "GB/s", "sample": f"{rows} of 65536 rows, {el:.2f} s"}
+    return out
 
 
 def main():

@@ -350,3 +350,251 @@ def linear_relu_backward(name: str = "fused_relu_bias_backward") -> dict:
         {"type": "EXPR", "writes": [_A("val_db", "_gid0")], "expr": "acc", "dtype": "float32"},
         {"type": "ENDFOR", "idx": "_gid0"},
     ]}
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# The Schedule-Items of one `forward` of the GPT-2 graph of apps/gpt2/gpt2.lisp:95 -- (caten (forward model (make-tensor
+# `(1 s) :from 'x) (iconst 'n))) over the Transformer of external/llm/layers.lisp:73-90 -- with the sequence length `s`
+# and the start position `n` symbolic and every model dimension static, the way that call compiles them.  The
+# partition into items follows the reference's kernel-count tests (source/test-suite/test-scheduler.lisp:28-45,140-163,
+# source/test-suite/external/test-llm.lisp:303-328, source/test-suite/test-iseq-lowerer.lisp:3-7): one kernel per
+# Embedding, LayerNorm and softmax; a Linear fuses with the element-wise work behind it (bias, GELU, the residual
+# add); attention is c_attn, scores (+ scale + mask), softmax, P.V, the head-merging copy and c_proj.  Argument order:
+# outputs, then the dynamic shapes in use, then inputs (source/codegen/rewriting-rules.lisp:207-231).
+def _shape(*names):
+    return [_glob(n, "shape", 0, "int64") for n in names]
+
+
+def _for(idx, below):
+    return {"type": "FOR", "idx": idx, "upfrom": 0, "below": _lt(idx, below), "by": 1}
+
+
+def _end(idx):
+    return {"type": "ENDFOR", "idx": idx}
+
+
+def _decl(name, value):
+    return {"type": "EXPR", "writes": [_A(name, None)], "expr": value, "declare_type": True, "dtype": "float32"}
+
+
+def _red(name, expr):
+    return {"type": "EXPR", "writes": [_A(name, None)], "expr": expr, "dtype": "float32", "reduction": True}
+
+
+def _store(id_, idx, expr, dtype="float32"):
+    return {"type": "EXPR", "writes": [_A(id_, idx)], "expr": expr, "dtype": dtype}
+
+
+def _eq(a, b):
+    """`==` as the reference spells it: not(a != b) (source/api/function.lisp)"""
+    return {"op": "NOT", "args": [{"op": "!=", "args": [a, b]}]}
+
+
+def _f32(e):
+    return {"op": "CAST", "dtype": "float32", "args": [e]}
+
+
+def gpt2_embed_tokens(vocab: int, dim: int, name: str = "fused_embedding_wte") -> dict:
+    """wte(tokens) (nn/embedding.lisp:13-25): out[t, d] = sum_v where(v == tok[t], W[v, d], 0).
+    Arguments: val_emb, s, val_tok, val_wte."""
+    return {"name": name, "blueprint": [
+        _glob("val_emb", "output", 2), *_shape("s"), _glob("val_tok", "input", 2), _glob("val_wte", "input", 2),
+        _for("_gid0", "s"), _for("_gid1", dim), _decl("acc", 0.0), _for("_gid2", vocab),
+        _red("acc", _add("acc", {"op": "WHERE", "args": [_eq(_f32("_gid2"), _A("val_tok", "_gid0")),
+                                                         _A("val_wte", _add(_mul(dim, "_gid2"), "_gid1")), 0.0]})),
+        _end("_gid2"), _store("val_emb", _add(_mul(dim, "_gid0"), "_gid1"), "acc"), _end("_gid1"), _end("_gid0"),
+    ]}
+
+
+def gpt2_embed_positions_add(max_pos: int, dim: int, name: str = "fused_embedding_wpe_add") -> dict:
+    """hi = token-emb + wpe(cast(start-pos + index-components)) (layers.lisp:80-82): the one-hot sum over the position
+    table compared with n + t, the token embedding added in the store.  Arguments: val_hi, s, n, val_emb, val_wpe."""
+    return {"name": name, "blueprint": [
+        _glob("val_hi", "output", 2), *_shape("s", "n"), _glob("val_emb", "input", 2), _glob("val_wpe", "input", 2),
+        _for("_gid0", "s"), _for("_gid1", dim), _decl("acc", 0.0), _for("_gid2", max_pos),
+        _red("acc", _add("acc", {"op": "WHERE", "args": [_eq(_f32("_gid2"), _f32(_add("n", "_gid0"))),
+                                                         _A("val_wpe", _add(_mul(dim, "_gid2"), "_gid1")), 0.0]})),
+        _end("_gid2"),
+        _store("val_hi", _add(_mul(dim, "_gid0"), "_gid1"), _add(_A("val_emb", _add(_mul(dim, "_gid0"), "_gid1")), "acc")),
+        _end("_gid1"), _end("_gid0"),
+    ]}
+
+
+def gpt2_causal_mask(name: str = "fused_triu_mask") -> dict:
+    """mask = triu(full((1 1 s n+s), -inf), diagonal = 1 + n) (layers.lisp:83; TriuNode, api/high-level-ops.lisp:278-291:
+    where(i <= j - k, x, 0), `<=` spelled not(j - k < i)).  Arguments: val_mask, s, n."""
+    t = _add("n", "s")
+    keep = {"op": "NOT", "args": [_lt(_add("_gid1", _neg(_add(1, "n"))), "_gid0")]}
+    return {"name": name, "blueprint": [
+        _glob("val_mask", "output", 4), *_shape("s", "n"),
+        _for("_gid0", "s"), _for("_gid1", t),
+        _store("val_mask", _add(_mul(t, "_gid0"), "_gid1"), {"op": "WHERE", "args": [keep, float("-inf"), 0.0]}),
+        _end("_gid1"), _end("_gid0"),
+    ]}
+
+
+def gpt2_layernorm(dim: int, eps: float = 1e-5, name: str = "fused_layernorm") -> dict:
+    """LayerNorm over rows of a static width (nn/normalization.lisp:39-58), 1 / n folded to a single-float constant as
+    the simplifier leaves it for a static shape.  Arguments: val_y, s, val_x, val_g, val_b."""
+    import numpy as np
+    inv = float(np.float32(1.0) / np.float32(dim))
+    idx = _add(_mul(dim, "_gid0"), "_gid1")
+    xi = _A("val_x", idx)
+    centred = _add(xi, _neg("u"))
+    rstd = {"op": "RECIP", "args": [{"op": "SQRT", "args": [_add(_mul("q", inv), eps)]}]}
+    return {"name": name, "blueprint": [
+        _glob("val_y", "output", 3), *_shape("s"), _glob("val_x", "input", 3), _glob("val_g", "input", 1), _glob("val_b", "input", 1),
+        _for("_gid0", "s"),
+        _decl("sm", 0.0), _for("_gid1", dim), _red("sm", _add("sm", xi)), _end("_gid1"),
+        _decl("u", _mul("sm", inv)),
+        _decl("q", 0.0), _for("_gid1", dim), _red("q", _add("q", _mul(centred, centred))), _end("_gid1"),
+        _decl("r", rstd),
+        _for("_gid1", dim),
+        _store("val_y", idx, _add(_mul(_mul(centred, "r"), _A("val_g", "_gid1")), _A("val_b", "_gid1"))),
+        _end("_gid1"), _end("_gid0"),
+    ]}
+
+
+def _gelu_of(x):
+    """GeLU :tanh decomposed as the reference does (nn/activations.lisp:202-215; tanh and sigmoid through exp2)"""
+    u = _mul(0.7978845608, _add(x, _mul(0.044715, _mul(x, _mul(x, x)))))
+    sig = {"op": "RECIP", "args": [_add(1.0, {"op": "EXP2", "args": [_mul(_mul(2.0, u), -1.4426950408889634)]})]}
+    return _mul(_mul(0.5, x), _add(1.0, _add(_mul(2.0, sig), -1.0)))
+
+
+def gpt2_linear(n_out: int, n_in: int, bias: bool = True, gelu: bool = False, residual: bool = False,
+                name: str = "fused_linear") -> dict:
+    """Linear over s rows (nn/linear.lisp:3-17: x @ W^T through a transposed view of W (n_out, n_in)) fused with what
+    follows it: + bias[j], GELU (c_fc, layers.lisp:53-59), + residual[t, j] (the !add of TransformerBlock, layers.lisp:69-71).
+    Arguments: val_y, s, val_x, val_w [, val_b] [, val_r]."""
+    e = "acc"
+    if bias:
+        e = _add("acc", _A("val_b", "_gid1"))
+    if gelu:
+        e = _gelu_of(e)
+    if residual:
+        e = _add(_A("val_r", _add(_mul(n_out, "_gid0"), "_gid1")), e)
+    return {"name": name, "blueprint": [
+        _glob("val_y", "output", 3), *_shape("s"), _glob("val_x", "input", 3), _glob("val_w", "input", 2),
+        *([_glob("val_b", "input", 1)] if bias else []), *([_glob("val_r", "input", 3)] if residual else []),
+        _for("_gid0", "s"), _for("_gid1", n_out), _decl("acc", 0.0), _for("_gid2", n_in),
+        _red("acc", _add("acc", _mul(_A("val_x", _add(_mul(n_in, "_gid0"), "_gid2")), _A("val_w", _add(_mul(n_in, "_gid1"), "_gid2"))))),
+        _end("_gid2"), _store("val_y", _add(_mul(n_out, "_gid0"), "_gid1"), e), _end("_gid1"), _end("_gid0"),
+    ]}
+
+
+def gpt2_cache_assign(dim: int, part: int, name: str = "fused_assign_cache") -> dict:
+    """!assign of the new key (part 1) / value (part 2) rows into the cache view [n, n+s) (merge-kv-cache,
+    layers.lisp:19-33): cache[(n + t), c] = qkv[t, part * dim + c]; heads and head-dim are contiguous on both sides and
+    collapse into one loop.  The cache is written in place.  Arguments: val_cache, s, n, val_qkv."""
+    return {"name": name, "blueprint": [
+        _glob("val_cache", "output", 4), *_shape("s", "n"), _glob("val_qkv", "input", 3),
+        _for("_gid0", "s"), _for("_gid1", dim),
+        _store("val_cache", _add(_mul(dim, _add("n", "_gid0")), "_gid1"), _A("val_qkv", _add(_mul(3 * dim, "_gid0"), _add(part * dim, "_gid1")))),
+        _end("_gid1"), _end("_gid0"),
+    ]}
+
+
+def gpt2_attention_scores(n_heads: int, head_dim: int, name: str = "fused_attention_scores") -> dict:
+    """scores = q . k^T / sqrt(head-dim) + mask (scaled-dot-product-attention, layers.lisp:3-5) over the cache view
+    [0, n+s): q is read out of the fused qkv rows, k out of the (max_len, heads, head_dim) cache, both through their
+    transposed views; the division is a multiplication by the folded constant.  Batched nest of four loops as in
+    source/test-suite/test-scheduler.lisp:126-138.  Arguments: val_sc, s, n, val_qkv, val_k, val_mask."""
+    dim = n_heads * head_dim
+    t = _add("n", "s")
+    return {"name": name, "blueprint": [
+        _glob("val_sc", "output", 4), *_shape("s", "n"), _glob("val_qkv", "input", 3), _glob("val_k", "input", 4), _glob("val_mask", "input", 4),
+        _for("_gid0", n_heads), _for("_gid1", "s"), _for("_gid2", t), _decl("acc", 0.0), _for("_gid3", head_dim),
+        _red("acc", _add("acc", _mul(_A("val_qkv", _add(_add(_mul(3 * dim, "_gid1"), _mul(head_dim, "_gid0")), "_gid3")),
+                                     _A("val_k", _add(_add(_mul(dim, "_gid2"), _mul(head_dim, "_gid0")), "_gid3"))))),
+        _end("_gid3"),
+        _store("val_sc", _add(_add(_mul(_mul("s", t), "_gid0"), _mul(t, "_gid1")), "_gid2"),
+               _add(_mul("acc", float(1.0 / head_dim ** 0.5)), _A("val_mask", _add(_mul(t, "_gid1"), "_gid2")))),
+        _end("_gid2"), _end("_gid1"), _end("_gid0"),
+    ]}
+
+
+def gpt2_softmax_rows(n_heads: int, name: str = "fused_softmax") -> dict:
+    """softmax over the last axis of (1, heads, s, n+s): heads and rows collapse into one loop of heads * s rows of
+    n + s (nn/activations.lisp:59-62,107-119).  Arguments: val_y, s, n, val_x."""
+    t = _add("n", "s")
+    idx = _add(_mul(t, "_gid0"), "_gid1")
+    ex = {"op": "EXP2", "args": [_mul(_add(_A("val_x", idx), _neg("m")), 1.4426950408889634)]}
+    return {"name": name, "blueprint": [
+        _glob("val_y", "output", 4), *_shape("s", "n"), _glob("val_x", "input", 4),
+        _for("_gid0", _mul(n_heads, "s")),
+        _decl("m", float("-inf")), _for("_gid1", t), _red("m", {"op": "MAX", "args": ["m", _A("val_x", idx)]}), _end("_gid1"),
+        _decl("e", 0.0), _for("_gid1", t), _red("e", _add("e", ex)), _end("_gid1"),
+        _for("_gid1", t), _store("val_y", idx, _mul(ex, {"op": "RECIP", "args": ["e"]})), _end("_gid1"),
+        _end("_gid0"),
+    ]}
+
+
+def gpt2_attention_values(n_heads: int, head_dim: int, name: str = "fused_attention_values") -> dict:
+    """out = probs . v over the cache view [0, n+s) (layers.lisp:3-5): v read in place out of the (max_len, heads,
+    head_dim) cache.  Arguments: val_o, s, n, val_p, val_v."""
+    dim = n_heads * head_dim
+    t = _add("n", "s")
+    return {"name": name, "blueprint": [
+        _glob("val_o", "output", 4), *_shape("s", "n"), _glob("val_p", "input", 4), _glob("val_v", "input", 4),
+        _for("_gid0", n_heads), _for("_gid1", "s"), _for("_gid2", head_dim), _decl("acc", 0.0), _for("_gid3", t),
+        _red("acc", _add("acc", _mul(_A("val_p", _add(_add(_mul(_mul("s", t), "_gid0"), _mul(t, "_gid1")), "_gid3")),
+                                     _A("val_v", _add(_add(_mul(dim, "_gid3"), _mul(head_dim, "_gid0")), "_gid2"))))),
+        _end("_gid3"),
+        _store("val_o", _add(_add(_mul(_mul(head_dim, "s"), "_gid0"), _mul(head_dim, "_gid1")), "_gid2"), "acc"),
+        _end("_gid2"), _end("_gid1"), _end("_gid0"),
+    ]}
+
+
+def gpt2_merge_heads(n_heads: int, head_dim: int, name: str = "fused_merge_heads") -> dict:
+    """(!reshape (!permute attn-output 0 2 1 3) ...) (layers.lisp:46-49): the contiguous copy that puts the heads of a
+    row side by side.  Arguments: val_y, s, val_o."""
+    dim = n_heads * head_dim
+    return {"name": name, "blueprint": [
+        _glob("val_y", "output", 3), *_shape("s"), _glob("val_o", "input", 4),
+        _for("_gid0", "s"), _for("_gid1", n_heads), _for("_gid2", head_dim),
+        _store("val_y", _add(_add(_mul(dim, "_gid0"), _mul(head_dim, "_gid1")), "_gid2"),
+               _A("val_o", _add(_add(_mul(_mul(head_dim, "s"), "_gid1"), _mul(head_dim, "_gid0")), "_gid2"))),
+        _end("_gid2"), _end("_gid1"), _end("_gid0"),
+    ]}
+
+
+def gpt2_argmax_last(vocab: int, name: str = "fused_argmax_last") -> dict:
+    """(!argmax (!view logits t -1 t)) (layers.lisp:90; ArgMaxNode, api/high-level-ops.lisp:314-325) over the LAST row of
+    the (1, s, vocab) logits: the view shows up as the offset vocab * (s - 1).  Arguments: val_out (int64), s, val_x."""
+    x = _A("val_x", _add(_mul(vocab, _add("s", -1)), _add(_mul(vocab, "_gid0"), "_gid1")))
+    rev = _f32(_add(_add(vocab, _neg(1)), _mul("_gid1", -1)))
+    return {"name": name, "blueprint": [
+        _glob("val_out", "output", 2, "int64"), *_shape("s"), _glob("val_x", "input", 3),
+        _for("_gid0", 1),
+        _decl("m", float("-inf")), _for("_gid1", vocab), _red("m", {"op": "MAX", "args": ["m", x]}), _end("_gid1"),
+        _decl("g", 0.0), _for("_gid1", vocab),
+        _red("g", {"op": "MAX", "args": ["g", {"op": "WHERE", "args": [_eq(x, "m"), rev, 0.0]}]}), _end("_gid1"),
+        _store("val_out", "_gid0", {"op": "CAST", "dtype": "int64", "args": [_add(_add(vocab, _neg("g")), _neg(1))]}, "int64"),
+        _end("_gid0"),
+    ]}
+
+
+def gpt2_step_items(cfg: dict) -> dict:
+    """Every distinct Schedule-Item of one GPT-2 `forward` for the shape `cfg` (the schedule cache gives the twelve
+    layers one set of kernels, source/codegen/jit.lisp:361-372)."""
+    D, H, F, V, L = cfg["dim"], cfg["n_heads"], cfg["ffn"], cfg["vocab"], cfg["max_seq"]
+    Dh = D // H
+    return {
+        "embed_tokens": gpt2_embed_tokens(V, D),
+        "embed_positions": gpt2_embed_positions_add(L, D),
+        "mask": gpt2_causal_mask(),
+        "layernorm": gpt2_layernorm(D, cfg.get("eps", 1e-5)),
+        "c_attn": gpt2_linear(3 * D, D, bias=True, name="fused_linear_c_attn"),
+        "assign_k": gpt2_cache_assign(D, 1, name="fused_assign_k"),
+        "assign_v": gpt2_cache_assign(D, 2, name="fused_assign_v"),
+        "scores": gpt2_attention_scores(H, Dh),
+        "softmax": gpt2_softmax_rows(H),
+        "values": gpt2_attention_values(H, Dh),
+        "merge_heads": gpt2_merge_heads(H, Dh),
+        "attn_proj": gpt2_linear(D, D, bias=True, residual=True, name="fused_linear_attn_proj"),
+        "c_fc": gpt2_linear(F, D, bias=True, gelu=True, name="fused_linear_c_fc_gelu"),
+        "mlp_proj": gpt2_linear(D, F, bias=True, residual=True, name="fused_linear_mlp_proj"),
+        "lm_head": gpt2_linear(V, D, bias=False, name="fused_linear_lm_head"),
+        "argmax": gpt2_argmax_last(V),
+    }

@@ -73,6 +73,25 @@ struct WMat {
 // gfx950: 256 MB of Infinity Cache in front of HBM
 static const int64_t kInfinityCacheBytes = 256ll << 20;
 
+// ---- batched, strided small matmul (bmm.hip) ----
+// element offset of an operand = base + sum_q batch_q * sb[q] + i * si + j * sj + k * sk (strides in elements;
+// an index the operand does not depend on has stride 0)
+struct BmmOperand {
+  int64_t base, sb[3], si, sj, sk;
+};
+struct BmmArgs {
+  float *C;
+  const float *A, *B;
+  const float *pre0, *pre1, *post;  // optional addends: before the activation (bias, mask) / after it (residual)
+  BmmOperand c, a, b, p0, p1, r;
+  int nb[3];                        // batch extents (1 where unused)
+  int M, N, K;
+  float alpha;
+  int act;
+};
+int bmm_variant(const BmmArgs &a);  // 0 = neither layout fits
+int launch_bmm(const BmmArgs &a);
+
 // Arguments of one fused Linear launch:
 //   y = act(prologue(x) . W^T + bias) + residual
 // Output rows >= split1 / split2 are routed to y1 / y2 (fused-qkv rows going straight

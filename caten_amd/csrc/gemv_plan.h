@@ -160,4 +160,28 @@ inline GemvPlan gemv_plan(const GemvPlanIn &in) {
   return p;
 }
 
+// How the split-K reduction + norm pass (rowops.hip) lays a row out: `wide` = four wavefronts per row instead of
+// one; `vpl` = the float4-per-lane count of the kernel instantiation chosen (one of 1,2,3,4,6,8 narrow / 1,2,4,8
+// wide); `nz` = the share bucket.  ok is false when no instantiation covers the row.
+struct ReduceNormPlan {
+  bool ok, wide;
+  int vpl, nz;
+};
+inline ReduceNormPlan reduce_norm_plan(int n, int nparts, long long rows) {
+  ReduceNormPlan p = {false, false, 0, 0};
+  if (n < 4 || n % 4 || n > 8192 || nparts < 1 || nparts > 16) return p;
+  p.nz = nparts <= 2 ? 2 : nparts <= 4 ? 4 : nparts <= 8 ? 8 : 16;
+  const int v1 = (n / 4 + 63) / 64, v4 = (n / 4 + 255) / 256;
+  // the shares of a row are all requested at once: VPL x NZ float4 per lane have to stay in registers
+  const bool narrow_fits = v1 * p.nz <= 32 && v1 <= 8, wide_fits = v4 * p.nz <= 32 && v4 <= 8;
+  if (!narrow_fits && !wide_fits) return p;
+  // four wavefronts per row where one cannot hold the row's shares, and for a prompt's few rows of some width: the
+  // pass is a single memory round trip, and four times the threads ask for it four times as wide
+  p.wide = !narrow_fits || (wide_fits && rows <= 2048 && n >= 512);
+  if (p.wide) p.vpl = v4 <= 1 ? 1 : v4 <= 2 ? 2 : v4 <= 4 ? 4 : 8;
+  else p.vpl = v1 <= 4 ? v1 : v1 <= 6 ? 6 : 8;
+  p.ok = true;
+  return p;
+}
+
 }  // namespace cthip

@@ -1308,9 +1308,10 @@ int launch_linear_gemm(float *y, const WMat *w, const float *x, int m, const flo
   return launch_gemm(a, B_WMAT, precision, nullptr, 0, defer);
 }
 
-// A matmul-shaped Schedule-Item routed here by the renderer: C (M,N) = act(A (M,K) . B + bias), B either (K,N)
+// A matmul-shaped Schedule-Item routed here by the renderer: C (M,N) = act(A (M,K) . B + bias) + residual, B either (K,N)
 // row-major or (N,K) rows read through a transposed view (Linear, source/nn/linear.lisp:3-17); fp32-grade operands.
-int matmul_routed(float *C, const float *A, const float *B, int M, int N, int K, int act, const float *bias, bool b_is_nk) {
+int matmul_routed(float *C, const float *A, const float *B, int M, int N, int K, int act, const float *bias, const float *residual,
+                  bool b_is_nk) {
   if (b_is_nk && M < 8) {  // a few rows of a Linear: the single-row kernels stream the weights once per row
     WMat w = {};
     w.type = CTHIP_F32;
@@ -1322,6 +1323,7 @@ int matmul_routed(float *C, const float *A, const float *B, int M, int N, int K,
     g.y = C;
     g.x = A;
     g.bias = bias;
+    g.residual = residual;
     g.act = act;
     g.x_stride = K;
     g.y_stride = N;
@@ -1331,6 +1333,7 @@ int matmul_routed(float *C, const float *A, const float *B, int M, int N, int K,
   a.C = C;
   a.A = A;
   a.bias = bias;
+  a.residual = residual;
   a.M = M;
   a.N = N;
   a.K = K;

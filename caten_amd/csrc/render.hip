@@ -501,6 +501,31 @@ static bool affine_of(const Sx &index, const std::string idx[3], int nidx, std::
   return v == v0 + 2 * out.c[0] + (nidx > 1 ? 3 * out.c[1] : 0) + (nidx > 2 ? 5 * out.c[2] : 0);
 }
 
+// the same over any number of indices
+struct AffineN {
+  long long base = 0;
+  std::vector<long long> c;
+};
+static bool affine_n(const Sx &index, const std::vector<std::string> &idx, std::map<std::string, long long> env, AffineN &out) {
+  const int n = (int)idx.size();
+  auto at = [&](int unit, bool check, long long &v) {
+    for (int k = 0; k < n; k++) env[idx[k]] = check ? 2 + 3 * k : (k == unit ? 1 : 0);
+    return eval_int(index, env, v);
+  };
+  long long v0, v;
+  if (!at(-1, false, v0)) return false;
+  out.base = v0;
+  out.c.assign(n, 0);
+  for (int k = 0; k < n; k++) {
+    if (!at(k, false, v)) return false;
+    out.c[k] = v - v0;
+  }
+  if (!at(-1, true, v)) return false;
+  long long want = v0;
+  for (int k = 0; k < n; k++) want += (2 + 3 * k) * out.c[k];
+  return v == want;
+}
+
 enum RouteKind { R_NONE = 0, R_MATMUL, R_EMBEDDING, R_ARGMAX, R_SOFTMAX, R_LAYERNORM, R_RMSNORM };
 struct Route {
   RouteKind kind = R_NONE;
@@ -510,6 +535,15 @@ struct Route {
   Sx bound[3];                              // their upper bounds
   int act = CTHIP_ACT_NONE;
   double eps = 0.0;                         // LayerNorm / RMSNorm: read off the item by evaluation
+  // matmul: the parallel loops outermost first (batch..., row i, column j), then the reduction index k
+  std::vector<std::string> lidx;
+  std::vector<Sx> lbound;
+  // matmul epilogue act(alpha * acc + pre...) + post...: up to two more operands, each added before or after the
+  // activation; embedding: the addend of `acc + other[..]`
+  int extra[2] = {-1, -1};
+  Sx extra_idx[2];
+  bool extra_post[2] = {false, false};
+  double alpha = 1.0;
 };
 
 struct Program {
@@ -550,45 +584,183 @@ static bool is_global_aref(const Item &it, const Sx &e, int &pos) {
   return pos >= 0 && it.globals[pos].pointer && it.globals[pos].dtype == "float32";
 }
 
-// for i < M: for j < N: { acc = 0; for k < K: acc += A[..] * B[..]; out[..] = epilogue(acc) }
+// ---- recognition by VALUE ----
+// The scalar statements between the loops (mean = s / n, rstd = 1 / sqrt(q / n + eps)) and the per-element
+// expressions come in whatever spelling the simplifier left (recip of a cast, a folded constant, operands in any
+// order), so they are recognised by VALUE: evaluated on probe numbers and compared with what the norm computes.
+struct Probe {
+  const Item *it = nullptr;
+  std::map<std::string, double> scalars;  // temporaries and by-value arguments
+  std::map<int, double> arrays;           // argument position of a global array -> what any element of it reads as
+  std::map<int, Sx> index;                // the index expression each array was read with
+};
+static bool sx_equal(const Sx &a, const Sx &b) {
+  if (a.kind != b.kind) return false;
+  if (a.kind == Sx::LIST) {
+    if (a.n() != b.n()) return false;
+    for (size_t k = 0; k < a.n(); k++)
+      if (!sx_equal(a.v[k], b.v[k])) return false;
+    return true;
+  }
+  return a.s == b.s && a.i == b.i && a.f == b.f;
+}
+static bool probe(const Sx &e, Probe &p, double &out) {
+  if (e.kind == Sx::INT) { out = (double)e.i; return true; }
+  if (e.kind == Sx::FLT) { out = e.f; return true; }
+  if (e.kind == Sx::SYM) {
+    auto f = p.scalars.find(e.s);
+    if (f == p.scalars.end()) return false;
+    out = f->second;
+    return true;
+  }
+  if (e.kind != Sx::LIST || e.v.empty() || e.v[0].kind != Sx::SYM) return false;
+  const std::string &op = e.v[0].s;
+  if (op == "aref") {
+    if (is_scalar_ref(e)) {
+      auto f = p.scalars.find(ref_name(e));
+      if (f == p.scalars.end()) return false;
+      out = f->second;
+      return true;
+    }
+    int pos;
+    if (!is_global_aref(*p.it, e, pos)) return false;
+    auto f = p.arrays.find(pos);
+    if (f == p.arrays.end()) return false;
+    auto seen = p.index.find(pos);
+    if (seen == p.index.end()) p.index[pos] = e.v[2];
+    else if (!sx_equal(seen->second, e.v[2])) return false;  // one element of each array per iteration
+    out = f->second;
+    return true;
+  }
+  if (op == "const") return e.n() >= 2 && probe(e.v[1], p, out);
+  if (op == "cast") {
+    if (e.n() < 3 || e.v[1].kind != Sx::SYM || e.v[1].s.rfind("float", 0) != 0) return false;
+    return probe(e.v[e.n() - 1], p, out);
+  }
+  std::vector<double> a;
+  for (size_t k = 1; k < e.n(); k++) {
+    double v;
+    if (!probe(e.v[k], p, v)) return false;
+    a.push_back(v);
+  }
+  if (a.empty()) return false;
+  if (op == "add") { out = 0; for (double v : a) out += v; return true; }
+  if (op == "mul") { out = 1; for (double v : a) out *= v; return true; }
+  if (op == "neg" && a.size() == 1) { out = -a[0]; return true; }
+  if (op == "recip" && a.size() == 1 && a[0] != 0) { out = 1.0 / a[0]; return true; }
+  if (op == "sqrt" && a.size() == 1 && a[0] >= 0) { out = sqrt(a[0]); return true; }
+  if (op == "max" && a.size() == 2) { out = a[0] > a[1] ? a[0] : a[1]; return true; }
+  if (op == "exp2" && a.size() == 1) { out = exp2(a[0]); return true; }
+  return false;
+}
+// (1e-6: a shape that is static lets the simplifier fold 1 / n into a single-float constant, 3e-8 off)
+static bool near(double a, double b) { return fabs(a - b) <= 1e-6 * (1.0 + fabs(b)); }
+static void global_arefs(const Item &it, const Sx &e, std::vector<int> &out) {
+  int pos;
+  if (e.call("aref")) {
+    if (is_global_aref(it, e, pos) && std::find(out.begin(), out.end(), pos) == out.end()) out.push_back(pos);
+    return;
+  }
+  if (e.kind == Sx::LIST)
+    for (const Sx &c : e.v) global_arefs(it, c, out);
+}
+
+// what the activations of the hand-written kernels compute, in double (Caten's decompositions: tanh(y) = 2 sigmoid(2y) - 1,
+// sigmoid(z) = recip(1 + exp2(-z / ln 2)); nn/activations.lisp:3-7,180-215, api/high-level-ops.lisp:112-117)
+static double act_value(int act, double x) {
+  switch (act) {
+    case CTHIP_ACT_RELU: return x > 0 ? x : 0.0;
+    case CTHIP_ACT_GELU: return 0.5 * x * (1.0 + tanh(0.7978845608028654 * (x + 0.044715 * x * x * x)));
+    case CTHIP_ACT_SILU: return x / (1.0 + exp(-x));
+    case CTHIP_ACT_SIGMOID: return 1.0 / (1.0 + exp(-x));
+    case CTHIP_ACT_TANH: return tanh(x);
+    default: return x;
+  }
+}
+
+// The statement that stores a matmul's result, recognised by VALUE: with the accumulator and the (up to two) other
+// arrays it reads set to probe numbers it has to give act(alpha * acc + pre...) + post... for one of the kernels'
+// activations and one assignment of the arrays to "before" / "after" the activation.  Without an activation any
+// factor alpha is accepted (attention's scores * recip(sqrt(head-dim)), external/llm/layers.lisp:3-5), with one
+// alpha is 1 (GELU after c_fc, ReLU: source/test-suite/test-scheduler.lisp:140-163).
+static bool probe_matmul_epilogue(const Item &it, const Sx &rhs, const std::string &acc, Route &r) {
+  std::vector<int> arrs;
+  global_arefs(it, rhs, arrs);
+  if (arrs.size() > 2) return false;
+  for (int a : arrs)
+    if (a == r.out) return false;
+  Probe p;
+  p.it = &it;
+  auto f = [&](double a, double e0, double e1, double &out) {
+    p.arrays.clear();
+    p.index.clear();
+    p.scalars[acc] = a;
+    if (arrs.size() > 0) p.arrays[arrs[0]] = e0;
+    if (arrs.size() > 1) p.arrays[arrs[1]] = e1;
+    return probe(rhs, p, out);
+  };
+  auto loose = [](double a, double b) { return fabs(a - b) <= 1e-5 * (1.0 + fabs(b)); };  // float-rounded GELU constants
+  const double pts[4][3] = {{0.7, 0.3, -0.2}, {-1.3, 0.5, 1.1}, {2.1, -0.4, 0.6}, {-0.15, -0.05, 0.1}};
+  double v0, v1;
+  if (!f(0.0, 0.0, 0.0, v0) || !f(1.0, 0.0, 0.0, v1)) return false;
+  const int acts[6] = {CTHIP_ACT_NONE, CTHIP_ACT_RELU, CTHIP_ACT_GELU, CTHIP_ACT_SILU, CTHIP_ACT_SIGMOID, CTHIP_ACT_TANH};
+  for (int act : acts) {
+    const double alpha = act == CTHIP_ACT_NONE ? v1 - v0 : 1.0;
+    if (act == CTHIP_ACT_NONE && (v0 != 0.0 || alpha == 0.0 || !std::isfinite(alpha))) continue;
+    for (int roles = 0; roles < (act == CTHIP_ACT_NONE ? 1 : 1 << arrs.size()); roles++) {
+      bool ok = true;
+      for (int q = 0; q < 4 && ok; q++) {
+        double got;
+        if (!f(pts[q][0], pts[q][1], pts[q][2], got)) return false;
+        double pre = alpha * pts[q][0], post = 0.0;
+        for (size_t k = 0; k < arrs.size(); k++) ((roles >> k) & 1 ? post : pre) += pts[q][1 + k];
+        ok = loose(got, act_value(act, pre) + post);
+      }
+      if (!ok) continue;
+      r.act = act;
+      r.alpha = alpha;
+      for (size_t k = 0; k < arrs.size(); k++) {
+        r.extra[k] = arrs[k];
+        r.extra_idx[k] = p.index[arrs[k]];
+        r.extra_post[k] = (roles >> k) & 1;
+      }
+      return true;
+    }
+  }
+  return false;
+}
+
+// for (batch...): for i < M: for j < N: { acc = 0; for k < K: acc += A[..] * B[..]; out[..] = epilogue(acc) }
+// -- the nest of (caten (!matmul a b)), with up to three batch loops in front (source/test-suite/test-scheduler.lisp:126-138)
 static bool match_matmul(const Item &it, Route &r) {
   const std::vector<BpNode> &b = it.body;
-  if (b.size() != 9) return false;
-  if (b[0].t != BpNode::FOR || b[1].t != BpNode::FOR || b[2].t != BpNode::EXPR || b[3].t != BpNode::FOR || b[4].t != BpNode::EXPR ||
-      b[5].t != BpNode::ENDFOR || b[6].t != BpNode::EXPR || b[7].t != BpNode::ENDFOR || b[8].t != BpNode::ENDFOR)
+  const int n = (int)b.size();
+  if (n < 9 || (n - 5) % 2) return false;
+  const int P = (n - 5) / 2;  // parallel loops
+  if (P < 2 || P > 5) return false;
+  for (int q = 0; q < P; q++)
+    if (b[q].t != BpNode::FOR || b[n - 1 - q].t != BpNode::ENDFOR) return false;
+  if (b[P].t != BpNode::EXPR || b[P + 1].t != BpNode::FOR || b[P + 2].t != BpNode::EXPR || b[P + 3].t != BpNode::ENDFOR || b[P + 4].t != BpNode::EXPR)
     return false;
-  const int fors[3] = {0, 1, 3};
-  for (int q = 0; q < 3; q++) {
-    const Sx *ub = upper_bound(b[fors[q]]);
-    if (!ub || !is_zero(b[fors[q]].upfrom)) return false;
-    r.idx[q] = b[fors[q]].idx;
-    r.bound[q] = *ub;
+  for (int q = 0; q <= P; q++) {
+    const BpNode &f = b[q < P ? q : P + 1];
+    const Sx *ub = upper_bound(f);
+    if (!ub || !is_zero(f.upfrom)) return false;
+    r.lidx.push_back(f.idx);
+    r.lbound.push_back(*ub);
   }
-  if (!b[2].declare || b[2].writes.size() != 1 || !is_scalar_ref(b[2].writes[0]) || !is_zero(b[2].rhs) || b[2].dtype != "float32") return false;
-  const std::string acc = ref_name(b[2].writes[0]);
+  const BpNode &decl = b[P], &red = b[P + 2], &st = b[P + 4];
+  if (!decl.declare || decl.writes.size() != 1 || !is_scalar_ref(decl.writes[0]) || !is_zero(decl.rhs) || decl.dtype != "float32") return false;
+  const std::string acc = ref_name(decl.writes[0]);
   Sx term;
-  if (!reduction_term(b[4], acc, "add", term) || !term.call("mul") || term.n() != 3) return false;
+  if (!reduction_term(red, acc, "add", term) || !term.call("mul") || term.n() != 3) return false;
   if (!is_global_aref(it, term.v[1], r.a) || !is_global_aref(it, term.v[2], r.b)) return false;
   r.a_idx = term.v[1].v[2];
   r.b_idx = term.v[2].v[2];
-  // the epilogue: acc, max(acc + bias, 0), acc + bias, max(acc, 0)
-  if (b[6].writes.size() != 1 || !is_global_aref(it, b[6].writes[0], r.out) || it.globals[r.out].type != "output") return false;
-  r.out_idx = b[6].writes[0].v[2];
-  Sx e = b[6].rhs;
-  r.act = CTHIP_ACT_NONE;
-  if (e.call("max") && e.n() == 3 && (is_zero(e.v[2]) || is_zero(e.v[1]))) {
-    const Sx inner = is_zero(e.v[2]) ? e.v[1] : e.v[2];  // (a copy: e's own element cannot be assigned to e)
-    e = inner;
-    r.act = CTHIP_ACT_RELU;
-  }
-  if (e.call("add") && e.n() == 3) {
-    const int ai = is_ref_to(e.v[1], acc) ? 1 : is_ref_to(e.v[2], acc) ? 2 : 0;
-    if (!ai || !is_global_aref(it, e.v[3 - ai], r.bias)) return false;
-    r.bias_idx = e.v[3 - ai].v[2];
-  } else if (!is_ref_to(e, acc)) {
-    return false;
-  }
+  if (st.writes.size() != 1 || !is_global_aref(it, st.writes[0], r.out) || it.globals[r.out].type != "output") return false;
+  r.out_idx = st.writes[0].v[2];
   if (r.out == r.a || r.out == r.b) return false;
+  if (!probe_matmul_epilogue(it, st.rhs, acc, r)) return false;
   r.kind = R_MATMUL;
   return true;
 }
@@ -622,13 +794,33 @@ static bool match_embedding(const Item &it, Route &r) {
   int dummy;
   if (uses(x, r.idx[2]) && !is_global_aref(it, x, dummy)) vside = &x, tside = &y;
   else if (uses(y, r.idx[2]) && !is_global_aref(it, y, dummy)) vside = &y, tside = &x;
-  if (!vside || !is_global_aref(it, *tside, r.b) || uses(tside->v[2], r.idx[2]) || uses(tside->v[2], r.idx[1])) return false;
-  r.b_idx = tside->v[2];
+  if (!vside) return false;
+  if (is_global_aref(it, *tside, r.b)) {
+    if (uses(tside->v[2], r.idx[2]) || uses(tside->v[2], r.idx[1])) return false;
+    r.b_idx = tside->v[2];
+  } else {
+    // the row is an EXPRESSION of the token position, not a stored index: wpe(start-pos + arange(seq-len)) of
+    // Transformer (external/llm/layers.lisp:81); which rows it names is worked out at launch
+    if (uses(*tside, r.idx[2]) || uses(*tside, r.idx[1]) || !uses(*tside, r.idx[0])) return false;
+    std::vector<int> none;
+    global_arefs(it, *tside, none);
+    if (!none.empty()) return false;
+    r.b = -1;
+    r.b_idx = *tside;
+  }
   r.bias_idx = *vside;
   if (!is_global_aref(it, term.v[2], r.a)) return false;
   r.a_idx = term.v[2].v[2];
-  if (b[6].writes.size() != 1 || !is_global_aref(it, b[6].writes[0], r.out) || !is_ref_to(b[6].rhs, acc)) return false;
+  if (b[6].writes.size() != 1 || !is_global_aref(it, b[6].writes[0], r.out)) return false;
   r.out_idx = b[6].writes[0].v[2];
+  // the stored value: acc, or acc + other[..] (the sum of two embeddings, layers.lisp:82)
+  const Sx &e = b[6].rhs;
+  if (!is_ref_to(e, acc)) {
+    if (!e.call("add") || e.n() != 3) return false;
+    const int ai = is_ref_to(e.v[1], acc) ? 1 : is_ref_to(e.v[2], acc) ? 2 : 0;
+    if (!ai || !is_global_aref(it, e.v[3 - ai], r.extra[0]) || r.extra[0] == r.out) return false;
+    r.extra_idx[0] = e.v[3 - ai].v[2];
+  }
   r.kind = R_EMBEDDING;
   return true;
 }
@@ -720,13 +912,13 @@ static bool match_softmax(const Item &it, Route &r) {
   const std::string s = ref_name(b[5].writes[0]);
   Sx t2, xi;
   int xp = -1;
-  if (!reduction_term(b[7], s, "add", t2) || !is_exp_of_shifted(it, t2, m, xp, xi) || xp != r.a) return false;
+  if (!reduction_term(b[7], s, "add", t2) || !is_exp_of_shifted(it, t2, m, xp, xi) || xp != r.a || !sx_equal(xi, r.a_idx)) return false;
   const Sx &e = b[10].rhs;
   if (!e.call("mul") || e.n() != 3) return false;
   const Sx *ex = nullptr, *rc = nullptr;
   if (e.v[2].call("recip")) ex = &e.v[1], rc = &e.v[2];
   else if (e.v[1].call("recip")) ex = &e.v[2], rc = &e.v[1];
-  if (!ex || rc->n() != 2 || !is_ref_to(rc->v[1], s) || !is_exp_of_shifted(it, *ex, m, xp, xi) || xp != r.a) return false;
+  if (!ex || rc->n() != 2 || !is_ref_to(rc->v[1], s) || !is_exp_of_shifted(it, *ex, m, xp, xi) || xp != r.a || !sx_equal(xi, r.a_idx)) return false;
   if (b[10].writes.size() != 1 || !is_global_aref(it, b[10].writes[0], r.out) || r.out == r.a) return false;
   r.out_idx = b[10].writes[0].v[2];
   r.kind = R_SOFTMAX;
@@ -734,82 +926,6 @@ static bool match_softmax(const Item &it, Route &r) {
 }
 
 // ---- LayerNorm / RMSNorm rows (source/nn/normalization.lisp:39-58,78-92) ----
-// The scalar statements between the loops (mean = s / n, rstd = 1 / sqrt(q / n + eps)) and the per-element
-// expressions come in whatever spelling the simplifier left (recip of a cast, a folded constant, operands in any
-// order), so they are recognised by VALUE: evaluated on probe numbers and compared with what the norm computes.
-struct Probe {
-  const Item *it = nullptr;
-  std::map<std::string, double> scalars;  // temporaries and by-value arguments
-  std::map<int, double> arrays;           // argument position of a global array -> what any element of it reads as
-  std::map<int, Sx> index;                // the index expression each array was read with
-};
-static bool sx_equal(const Sx &a, const Sx &b) {
-  if (a.kind != b.kind) return false;
-  if (a.kind == Sx::LIST) {
-    if (a.n() != b.n()) return false;
-    for (size_t k = 0; k < a.n(); k++)
-      if (!sx_equal(a.v[k], b.v[k])) return false;
-    return true;
-  }
-  return a.s == b.s && a.i == b.i && a.f == b.f;
-}
-static bool probe(const Sx &e, Probe &p, double &out) {
-  if (e.kind == Sx::INT) { out = (double)e.i; return true; }
-  if (e.kind == Sx::FLT) { out = e.f; return true; }
-  if (e.kind == Sx::SYM) {
-    auto f = p.scalars.find(e.s);
-    if (f == p.scalars.end()) return false;
-    out = f->second;
-    return true;
-  }
-  if (e.kind != Sx::LIST || e.v.empty() || e.v[0].kind != Sx::SYM) return false;
-  const std::string &op = e.v[0].s;
-  if (op == "aref") {
-    if (is_scalar_ref(e)) {
-      auto f = p.scalars.find(ref_name(e));
-      if (f == p.scalars.end()) return false;
-      out = f->second;
-      return true;
-    }
-    int pos;
-    if (!is_global_aref(*p.it, e, pos)) return false;
-    auto f = p.arrays.find(pos);
-    if (f == p.arrays.end()) return false;
-    auto seen = p.index.find(pos);
-    if (seen == p.index.end()) p.index[pos] = e.v[2];
-    else if (!sx_equal(seen->second, e.v[2])) return false;  // one element of each array per iteration
-    out = f->second;
-    return true;
-  }
-  if (op == "const") return e.n() >= 2 && probe(e.v[1], p, out);
-  if (op == "cast") {
-    if (e.n() < 3 || e.v[1].kind != Sx::SYM || e.v[1].s.rfind("float", 0) != 0) return false;
-    return probe(e.v[e.n() - 1], p, out);
-  }
-  std::vector<double> a;
-  for (size_t k = 1; k < e.n(); k++) {
-    double v;
-    if (!probe(e.v[k], p, v)) return false;
-    a.push_back(v);
-  }
-  if (a.empty()) return false;
-  if (op == "add") { out = 0; for (double v : a) out += v; return true; }
-  if (op == "mul") { out = 1; for (double v : a) out *= v; return true; }
-  if (op == "neg" && a.size() == 1) { out = -a[0]; return true; }
-  if (op == "recip" && a.size() == 1 && a[0] != 0) { out = 1.0 / a[0]; return true; }
-  if (op == "sqrt" && a.size() == 1 && a[0] >= 0) { out = sqrt(a[0]); return true; }
-  return false;
-}
-static bool near(double a, double b) { return fabs(a - b) <= 1e-9 * (1.0 + fabs(b)); }
-static void global_arefs(const Item &it, const Sx &e, std::vector<int> &out) {
-  int pos;
-  if (e.call("aref")) {
-    if (is_global_aref(it, e, pos) && std::find(out.begin(), out.end(), pos) == out.end()) out.push_back(pos);
-    return;
-  }
-  if (e.kind == Sx::LIST)
-    for (const Sx &c : e.v) global_arefs(it, c, out);
-}
 // the row length as the probes see it: a literal bound is itself, a symbolic one is bound to 7
 static bool probe_row_length(const Sx &bound, Probe &p, double &n) {
   if (const_value(bound, n)) return n >= 1;
@@ -856,7 +972,7 @@ static bool probe_affine_store(const Item &it, const BpNode &st, Probe &p, Route
     r.b = gpos, r.bias = bpos;
     if (gpos >= 0) r.b_idx = p.index[gpos];
     if (bpos >= 0) r.bias_idx = p.index[bpos];
-    r.a_idx = p.index.count(r.a) ? p.index[r.a] : r.a_idx;
+    if (p.index.count(r.a) && !sx_equal(p.index[r.a], r.a_idx)) return false;  // a shifted / strided view of x: not this norm
     return true;
   };
   if (extra.empty()) return fits(-1, -1);
@@ -1561,33 +1677,104 @@ struct KernelRenderer {
 };
 
 // entry points of the hand-written kernels the routes use (matmul.hip, linear.hip, rowops.hip)
-int matmul_routed(float *C, const float *A, const float *B, int M, int N, int K, int act, const float *bias, bool b_is_nk);
+int matmul_routed(float *C, const float *A, const float *B, int M, int N, int K, int act, const float *bias, const float *residual,
+                  bool b_is_nk);
+int launch_embedding(float *out, const float *W, const float *idx_f, const int *idx_i, int ntok, int vocab, int dim,
+                     const float *W2, const int *pos, int max_pos);
+int launch_embedding_rows(float *out, const float *W, long long first, long long step, int ntok, int vocab, int dim, const float *addend);
 
 static bool launch_route(Program &pg, void **args, const std::map<std::string, long long> &env, int &rc) {
   Route &r = pg.route;
   rc = 0;
   auto ptr = [&](int pos) { return *(void **)args[pos]; };
   auto bound = [&](int q, long long &v) { return eval_int(r.bound[q], env, v) && v >= 0 && v <= 0x7fffffff; };
+  auto aligned = [](const float *p) { return ((uintptr_t)p % 16) == 0; };
   if (r.kind == R_MATMUL) {
-    long long M, N, K;
-    if (!bound(0, M) || !bound(1, N) || !bound(2, K)) return false;
-    Affine ao, aa, ab, abias;
-    if (!affine_of(r.out_idx, r.idx, 3, env, ao) || !affine_of(r.a_idx, r.idx, 3, env, aa) || !affine_of(r.b_idx, r.idx, 3, env, ab)) return false;
-    // C (M,N) row-major, A (M,K) row-major
-    if (ao.base || ao.c[0] != N || ao.c[1] != 1 || ao.c[2] != 0) return false;
-    if (aa.base || aa.c[0] != K || aa.c[1] != 0 || aa.c[2] != 1) return false;
-    bool b_nk;
-    if (ab.base == 0 && ab.c[0] == 0 && ab.c[1] == 1 && ab.c[2] == N) b_nk = false;       // B (K,N) row-major
-    else if (ab.base == 0 && ab.c[0] == 0 && ab.c[1] == K && ab.c[2] == 1) b_nk = true;   // W (N,K) read through a transposed view
-    else return false;
-    const float *bias = nullptr;
-    if (r.bias >= 0) {
-      if (!affine_of(r.bias_idx, r.idx, 3, env, abias) || abias.base || abias.c[0] || abias.c[1] != 1 || abias.c[2]) return false;
-      bias = (const float *)ptr(r.bias);
+    const int nl = (int)r.lidx.size(), P = nl - 1;  // loops: batch..., i, j, then k
+    std::vector<long long> ext(nl);
+    for (int q = 0; q < nl; q++)
+      if (!eval_int(r.lbound[q], env, ext[q]) || ext[q] < 0 || ext[q] > 0x7fffffff) return false;
+    const long long M = ext[P - 2], N = ext[P - 1], K = ext[P];
+    long long nbatch = 1;
+    for (int q = 0; q < P - 2; q++) nbatch *= ext[q];
+    AffineN ao, aa, ab, ae[2];
+    if (!affine_n(r.out_idx, r.lidx, env, ao) || !affine_n(r.a_idx, r.lidx, env, aa) || !affine_n(r.b_idx, r.lidx, env, ab)) return false;
+    const int ii = P - 2, jj = P - 1, kk = P;
+    if (ao.c[kk] || aa.c[jj] || ab.c[ii]) return false;  // the result does not move with k, A not with j, B not with i
+    int nextra = 0;
+    for (int q = 0; q < 2; q++)
+      if (r.extra[q] >= 0) {
+        if (!affine_n(r.extra_idx[q], r.lidx, env, ae[q]) || ae[q].c[kk]) return false;
+        nextra++;
+      }
+    if (M == 0 || N == 0 || nbatch == 0) return true;
+    if (ao.base < 0 || aa.base < 0 || ab.base < 0) return false;
+    float *C = (float *)ptr(r.out) + ao.base;
+    const float *A = (const float *)ptr(r.a) + aa.base, *B = (const float *)ptr(r.b) + ab.base;
+    // (1) one dense row-major product: the MFMA GEMM, or the single-row kernels for a few rows of a Linear
+    bool b_nk = false;
+    bool dense = nbatch == 1 && r.alpha == 1.0 && ao.c[ii] == N && ao.c[jj] == 1 && aa.c[ii] == K && aa.c[kk] == 1 && aligned(C) && aligned(A) && aligned(B);
+    if (dense) {
+      if (ab.c[jj] == 1 && ab.c[kk] == N) b_nk = false;       // B (K,N) row-major
+      else if (ab.c[jj] == K && ab.c[kk] == 1) b_nk = true;   // W (N,K) read through a transposed view
+      else dense = false;
     }
-    if (M == 0 || N == 0) return true;
-    rc = matmul_routed((float *)ptr(r.out), (const float *)ptr(r.a), (const float *)ptr(r.b), (int)M, (int)N, (int)K, r.act, bias, b_nk);
-    pg.last_route = b_nk ? "cthip_linear" : "cthip_matmul";
+    const float *bias = nullptr, *resid = nullptr;
+    for (int q = 0; q < 2 && dense; q++) {
+      if (r.extra[q] < 0) continue;
+      if (ae[q].base < 0) return false;
+      const float *e = (const float *)ptr(r.extra[q]) + ae[q].base;
+      const bool by_col = ae[q].c[ii] == 0 && ae[q].c[jj] == 1, full = ae[q].c[ii] == N && ae[q].c[jj] == 1;
+      // without an activation "before" and "after" are the same thing
+      const bool may_pre = !r.extra_post[q] || r.act == CTHIP_ACT_NONE, may_post = r.extra_post[q] || r.act == CTHIP_ACT_NONE;
+      if (by_col && may_pre && !bias && aligned(e)) bias = e;
+      else if (full && may_post && !resid && aligned(e)) resid = e;
+      else dense = false;
+    }
+    if (dense) {
+      rc = matmul_routed(C, A, B, (int)M, (int)N, (int)K, r.act, bias, resid, b_nk);
+      pg.last_route = b_nk ? "cthip_linear" : "cthip_matmul";
+      return true;
+    }
+    // (2) batched / strided / scaled: the attention items over the cache view, chunked operands
+    if (P - 2 > 3) return false;
+    BmmArgs g = {};
+    g.C = (float *)ptr(r.out);
+    g.A = (const float *)ptr(r.a);
+    g.B = (const float *)ptr(r.b);
+    auto fill = [&](BmmOperand &o, const AffineN &f) {
+      o.base = f.base;
+      for (int q = 0; q < 3; q++) o.sb[q] = q < P - 2 ? f.c[q] : 0;
+      o.si = f.c[ii];
+      o.sj = f.c[jj];
+      o.sk = f.c[kk];
+    };
+    fill(g.c, ao);
+    fill(g.a, aa);
+    fill(g.b, ab);
+    for (int q = 0; q < 3; q++) g.nb[q] = q < P - 2 ? (int)ext[q] : 1;
+    g.M = (int)M, g.N = (int)N, g.K = (int)K;
+    g.alpha = (float)r.alpha;
+    g.act = r.act;
+    for (int q = 0; q < 2; q++) {
+      if (r.extra[q] < 0) continue;
+      if (ae[q].base < 0) return false;
+      const float *e = (const float *)ptr(r.extra[q]);
+      if (r.extra_post[q]) {
+        if (g.post) return false;
+        g.post = e;
+        fill(g.r, ae[q]);
+      } else if (!g.pre0) {
+        g.pre0 = e;
+        fill(g.p0, ae[q]);
+      } else {
+        g.pre1 = e;
+        fill(g.p1, ae[q]);
+      }
+    }
+    if (K == 0 || !bmm_variant(g)) return false;
+    rc = launch_bmm(g);
+    pg.last_route = "cthip_bmm";
     return true;
   }
   if (r.kind == R_EMBEDDING) {
@@ -1597,9 +1784,24 @@ static bool launch_route(Program &pg, void **args, const std::map<std::string, l
     if (!affine_of(r.out_idx, r.idx, 3, env, ao) || !affine_of(r.a_idx, r.idx, 3, env, aw) || !affine_of(r.b_idx, r.idx, 3, env, ai)) return false;
     if (ao.base || ao.c[0] != D || ao.c[1] != 1 || ao.c[2]) return false;  // out (T, D)
     if (aw.base || aw.c[0] || aw.c[1] != 1 || aw.c[2] != D) return false;  // W (V, D)
-    if (ai.base || ai.c[0] != 1 || ai.c[1] || ai.c[2]) return false;       // idx (T)
     Affine av;
     if (!affine_of(r.bias_idx, r.idx, 3, env, av) || av.base || av.c[0] || av.c[1] || av.c[2] != 1) return false;  // compared with v itself
+    const float *addend = nullptr;
+    if (r.extra[0] >= 0) {  // + other[t, d]
+      Affine ae;
+      if (!affine_of(r.extra_idx[0], r.idx, 3, env, ae) || ae.base || ae.c[0] != D || ae.c[1] != 1 || ae.c[2]) return false;
+      addend = (const float *)ptr(r.extra[0]);
+    }
+    if (r.b < 0) {
+      // rows first, first + step, ...: token position t selects row (first + step * t)
+      if (ai.c[1] || ai.c[2]) return false;
+      if (T == 0 || D == 0) return true;
+      rc = launch_embedding_rows((float *)ptr(r.out), (const float *)ptr(r.a), ai.base, ai.c[0], (int)T, (int)V, (int)D, addend);
+      pg.last_route = "cthip_embedding";
+      return true;
+    }
+    if (addend) return false;
+    if (ai.base || ai.c[0] != 1 || ai.c[1] || ai.c[2]) return false;       // idx (T)
     if (T == 0 || D == 0) return true;
     rc = cthip_embedding((float *)ptr(r.out), (const float *)ptr(r.a), (const float *)ptr(r.b), (int)T, (int)V, (int)D);
     pg.last_route = "cthip_embedding";
@@ -1609,7 +1811,8 @@ static bool launch_route(Program &pg, void **args, const std::map<std::string, l
     long long Rn, N;
     if (!bound(0, Rn) || !bound(1, N) || N < 1) return false;
     Affine ax, ao;
-    if (!affine_of(r.a_idx, r.idx, 2, env, ax) || ax.base || ax.c[0] != N || ax.c[1] != 1) return false;
+    // (a base offset = a view from some row on: the last position's logits, external/llm/layers.lisp:90)
+    if (!affine_of(r.a_idx, r.idx, 2, env, ax) || ax.base < 0 || (ax.c[0] != N && Rn > 1) || ax.c[1] != 1) return false;
     const std::string oi[3] = {r.idx[0], "", ""};
     if (!affine_of(r.out_idx, oi, 1, env, ao) || ao.base || (ao.c[0] != 1 && Rn > 1)) return false;
     // kept value (N - 1) - i and result N - g - 1, whatever their spelling
@@ -1626,7 +1829,7 @@ static bool launch_route(Program &pg, void **args, const std::map<std::string, l
       if (!eval_int(r.bias_idx, e2, v) || v != N - g - 1) return false;
     }
     if (Rn == 0) return true;
-    rc = cthip_argmax((int64_t *)ptr(r.out), (const float *)ptr(r.a), Rn, (int)N);
+    rc = cthip_argmax((int64_t *)ptr(r.out), (const float *)ptr(r.a) + ax.base, Rn, (int)N);
     pg.last_route = "cthip_argmax";
     return true;
   }

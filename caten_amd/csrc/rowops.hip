@@ -9,6 +9,7 @@
 // the row through L2.
 #include <type_traits>
 #include "common.h"
+#include "gemv_plan.h"
 
 namespace cthip {
 
@@ -278,14 +279,7 @@ __global__ __launch_bounds__(256) void k_reduce_norm_wide(ReduceNormArgs a) {
   }
 }
 
-static int reduce_norm_bucket(int nparts) { return nparts <= 2 ? 2 : nparts <= 4 ? 4 : nparts <= 8 ? 8 : 16; }
-bool reduce_norm_supported(int n, int nparts) {
-  if (n % 4 || n > 8192 || nparts < 1 || nparts > 16) return false;
-  // the shares of a row are all requested at once: VPL x NZ float4 per lane have to stay in registers; one
-  // wavefront per row where that fits, four otherwise
-  const int nz = reduce_norm_bucket(nparts);
-  return ((n / 4 + 63) / 64) * nz <= 32 || ((n / 4 + 255) / 256) * nz <= 32;
-}
+bool reduce_norm_supported(int n, int nparts) { return reduce_norm_plan(n, nparts, 1).ok || reduce_norm_plan(n, nparts, 1 << 20).ok; }
 
 int launch_reduce_norm(float *y, float *xout, const float *parts, int nparts, int64_t part_stride, const float *bias,
                        const float *resid, const float *g, const float *b, float eps, int64_t rows, int n, bool rms) {
@@ -293,10 +287,9 @@ int launch_reduce_norm(float *y, float *xout, const float *parts, int nparts, in
   if (!reduce_norm_supported(n, nparts)) return fail(CTHIP_E_BAD_ARG, "reduce + norm: rows of %d with %d shares", n, nparts);
   ReduceNormArgs a = {y, xout, parts, nparts, part_stride, bias, resid, g, b, eps, rows, n};
   hipStream_t st = state().stream;
-  // four wavefronts per row where one cannot hold the row's shares, and for a prompt's few rows of some width: the
-  // pass is a single memory round trip, and four times the threads ask for it four times as wide
-  if (((n / 4 + 63) / 64) * reduce_norm_bucket(nparts) > 32 || (rows <= 2048 && n >= 512)) {
-    const int vplw = (n / 4 + 255) / 256;
+  const ReduceNormPlan pl = reduce_norm_plan(n, nparts, rows);
+  if (pl.wide) {
+    const int vplw = pl.vpl;
     dim3 gridw((unsigned)rows), blockw(256);
 #define RW3(MODE, V, Z) hipLaunchKernelGGL((k_reduce_norm_wide<MODE, V, Z>), gridw, blockw, 0, st, a)
 #define RW2(MODE, V)                       \
@@ -316,7 +309,7 @@ int launch_reduce_norm(float *y, float *xout, const float *parts, int nparts, in
     CTHIP_LAUNCH_CHECK();
     return 0;
   }
-  const int vpl = (n / 4 + 63) / 64;
+  const int vpl = pl.vpl;
   // a row per wavefront; few rows (a prompt) go one to a workgroup so that they spread over the compute units
   const int wpb = rows <= 4096 ? 1 : 4;
   dim3 grid((unsigned)((rows + wpb - 1) / wpb)), block(64 * wpb);
@@ -477,6 +470,21 @@ __global__ __launch_bounds__(256) void k_embedding(float *__restrict__ out, cons
     // an index no vocabulary row equals selects nothing in the reference's one-hot sum: 0
     float v = hit ? W[(int64_t)id * dim + d] : 0.0f;
     if (W2) v += phit ? W2[(int64_t)p * dim + d] : 0.0f;
+    out[(int64_t)t * dim + d] = v;
+  }
+}
+
+// out[t,:] = W[first + step * t,:] (+ addend[t,:]): an Embedding whose indices are an arithmetic progression, as the
+// position table of Transformer is read (wpe(start-pos + arange(seq-len)), external/llm/layers.lisp:81-82).  A row
+// the table does not have selects nothing in the one-hot sum: 0.
+__global__ __launch_bounds__(256) void k_embedding_rows(float *__restrict__ out, const float *__restrict__ W, long long first,
+                                                        long long step, int vocab, int dim, const float *__restrict__ addend) {
+  const int t = blockIdx.x;
+  const long long row = first + step * t;
+  const bool hit = row >= 0 && row < vocab;
+  for (int d = threadIdx.x; d < dim; d += blockDim.x) {
+    float v = hit ? W[row * dim + d] : 0.0f;
+    if (addend) v += addend[(int64_t)t * dim + d];
     out[(int64_t)t * dim + d] = v;
   }
 }
@@ -1306,6 +1314,13 @@ int launch_embedding(float *out, const float *W, const float *idx_f, const int *
   if (ntok == 0) return 0;
   hipLaunchKernelGGL(k_embedding, dim3(ntok), dim3(256), 0, state().stream, out, W, idx_f, idx_i, vocab, dim, W2, pos,
                      max_pos);
+  CTHIP_LAUNCH_CHECK();
+  return 0;
+}
+
+int launch_embedding_rows(float *out, const float *W, long long first, long long step, int ntok, int vocab, int dim, const float *addend) {
+  if (ntok == 0) return 0;
+  hipLaunchKernelGGL(k_embedding_rows, dim3(ntok), dim3(256), 0, state().stream, out, W, first, step, vocab, dim, addend);
   CTHIP_LAUNCH_CHECK();
   return 0;
 }

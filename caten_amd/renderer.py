@@ -111,8 +111,24 @@ def sexp(e) -> str:
     return "(" + " ".join([op.lower()] + [sexp(a) for a in e.get("args", [])]) + ")"
 
 
+def item_from_sexp(text: str) -> dict:
+    """A Schedule-Item that already IS interchange text (what a Lisp process prints, a golden fixture): the text is
+    handed to the library as it is; only the argument list is read off it here, for marshalling."""
+    import re
+    body = "\n".join(ln for ln in text.splitlines() if not ln.lstrip().startswith(";"))
+    m = re.search(r"\(\s*item\s+([^\s()]+)", body, re.I)
+    if not m:
+        raise ValueError("item_from_sexp: expected (item NAME node...)")
+    globs = [{"type": "DEFINE-GLOBAL", "id": g[0].lower(), "dtype": g[1].lower(), "pointer_p": g[2].lower() == "t",
+              "arg_type": g[3].lower(), "nrank": int(g[4])}
+             for g in re.findall(r"\(\s*define-global\s+(\S+)\s+(\S+)\s+(\S+)\s+(\S+)\s+(\d+)\s*\)", body, re.I)]
+    return {"name": m.group(1).lower(), "blueprint": globs, "sexp": text}
+
+
 def item_sexp(item: dict) -> str:
     """A Schedule-Item as the text cthip_program_create reads."""
+    if item.get("sexp") is not None:
+        return item["sexp"]
     out = [f"(item {item['name'].lower()}"]
     for n in item["blueprint"]:
         t = n["type"]

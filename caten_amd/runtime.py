@@ -216,6 +216,50 @@ class GraphRuntime:
         """runtime-invoke-jit-kernel (runner.lisp:20-21; Metal passes the node too, metal.lisp:285-286)"""
         info.caller(node, *args)
 
+    # scalar arithmetic of the VM (runtime.lisp:396-449): dynamic shapes and strides are computed by :Add / :Mul /
+    # :Neg / :Idiv / :Mod / :Max / :Load nodes over rank-0 values; arrays go through JIT kernels on this backend
+    def _scalar_op(self, node: Node, args, fn):
+        vals = [self._num(a) for a in args]
+        if any(isinstance(a, AbstractBuffer) and a.nrank > 0 for a in args):
+            raise NotImplementedError(f"realize-node :{node.type} over arrays is not a VM operation on this backend "
+                                      f"(it is part of a JIT kernel)")
+        out = fn(*vals)
+        first = args[0]
+        if isinstance(first, AbstractBuffer):
+            b = first.copy()
+            b.value = out
+            return b
+        return out
+
+    def realize_add(self, node: Node, args):
+        return self._scalar_op(node, args, lambda *v: sum(v[1:], v[0]))
+
+    def realize_mul(self, node: Node, args):
+        def mul(*v):
+            out = v[0]
+            for x in v[1:]:
+                out = out * x
+            return out
+        return self._scalar_op(node, args, mul)
+
+    def realize_neg(self, node: Node, args):
+        return self._scalar_op(node, args, lambda x: -x)
+
+    def realize_idiv(self, node: Node, args):
+        return self._scalar_op(node, args, lambda a, b: a // b)
+
+    def realize_mod(self, node: Node, args):
+        return self._scalar_op(node, args, lambda a, b: a % b)
+
+    def realize_max(self, node: Node, args):
+        return self._scalar_op(node, args, max)
+
+    def realize_load(self, node: Node, args):
+        """:Load (runtime.lisp:396-405) of a rank-0 target: the node's :value, a number or a variable name"""
+        val = node.attrs["value"]
+        val = self._num(self.getvar(val)) if isinstance(val, str) else val
+        return self._scalar_op(node, args, lambda _t: val)
+
     def realize_pause_backward(self, node: Node, args):
         return tuple(args) if len(args) != 1 else args[0]
 

@@ -117,8 +117,16 @@ int cthip_launch(void *fn, const unsigned grid[3], const unsigned block[3], unsi
  *                     layout at every launch and falls back to its rendered kernel when it does not fit.
  * cthip_program_route: "rendered", or the shape recognised at creation ("matmul", "embedding", "argmax",
  * "softmax", "layernorm", "rmsnorm"); cthip_program_last_route: what the last launch ran ("rendered",
- * "cthip_matmul", "cthip_linear", "cthip_embedding", "cthip_argmax", "cthip_softmax", "cthip_layernorm",
- * "cthip_rmsnorm").  Strings stay valid until the program is destroyed.
+ * "cthip_matmul", "cthip_linear", "cthip_bmm", "cthip_embedding", "cthip_argmax", "cthip_softmax",
+ * "cthip_layernorm", "cthip_rmsnorm").  Strings stay valid until the program is destroyed.
+ * The matmul shape is the nest of (caten (!matmul a b)) behind up to three batch loops
+ * (source/test-suite/test-scheduler.lisp:117-138), its result stored as act(alpha * acc + pre...) + post... --
+ * recognised by the VALUE of the store statement, whatever its spelling: bias, GELU / ReLU / SiLU, residual add
+ * (test-scheduler.lisp:140-163; external/llm/layers.lisp:53-71), attention's scale and mask (layers.lisp:3-5).
+ * One dense row-major product runs the MFMA GEMM (fewer than eight rows of a Linear: the single-row kernels);
+ * batched, strided or offset operands -- q out of the fused qkv rows, k / v in place out of the cache view --
+ * the batched kernel ("cthip_bmm"); operands that fit neither, the rendered kernel.  The embedding shape covers
+ * indices that are an expression of the position (wpe(start-pos + arange), layers.lisp:81) and an added array.
  * Option "render_routes" 0 makes every program run its rendered kernel. */
 const char *cthip_render_header(void);
 int cthip_program_create(void **program, const char *blueprint);

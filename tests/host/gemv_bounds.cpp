@@ -196,7 +196,24 @@ static void walk(const Case &c) {
       }
 }
 
+// the split-K reduction + norm pass: whatever (row length, shares, rows) the launcher accepts, the instantiation it
+// picks covers the whole row (lanes x float4 per lane x 4 floats) and keeps its shares within the register budget
+static void check_reduce_norm_plans() {
+  for (int n = 4; n <= 8192; n += 4)
+    for (int nparts = 1; nparts <= 16; nparts++)
+      for (long long rows : {1ll, 512ll, 2048ll, 2049ll, 4096ll, 100000ll}) {
+        const ReduceNormPlan p = reduce_norm_plan(n, nparts, rows);
+        if (!p.ok) continue;
+        g_checked++;
+        const int lanes = p.wide ? 256 : 64;
+        const bool inst = p.wide ? (p.vpl == 1 || p.vpl == 2 || p.vpl == 4 || p.vpl == 8) : (p.vpl >= 1 && p.vpl <= 8 && p.vpl != 5 && p.vpl != 7);
+        if (lanes * p.vpl * 4 < n || !inst || p.vpl * p.nz > 64 || p.nz < nparts)
+          if (g_violations++ < 40) printf("VIOLATION reduce + norm: n %d shares %d rows %lld -> wide %d vpl %d nz %d\n", n, nparts, rows, p.wide, p.vpl, p.nz);
+      }
+}
+
 int main(int argc, char **argv) {
+  check_reduce_norm_plans();
   // default: a few seconds (every shape, the flag combinations thinned out on the large ones); "full": everything
   const bool full = argc > 1 && !strcmp(argv[1], "full");
   const int types[] = {CTHIP_Q8_0, CTHIP_Q4_0, CTHIP_F32, CTHIP_F16};

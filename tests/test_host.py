@@ -388,3 +388,105 @@ def test_elementwise_and_row_items_hold_their_reads_in_registers():
     assert src.count("m = _gid1_ok ? _w : m;") == 6 and src.count("s = _gid1_ok ? _w : s;") == 6
     r.compile_kernel([g, gs, ln, sd])
     assert r.code_object[:4] == b"\x7fELF"
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# The Schedule-Items of a GPT-2 `forward` (tests/golden/blueprints/): interchange text pinned as fixtures
+GOLDEN_BP = os.path.join(ROOT, "tests", "golden", "blueprints")
+GPT2_ITEM_ROUTES = {
+    "embed_tokens": "embedding", "embed_positions": "embedding", "mask": "rendered", "layernorm": "layernorm",
+    "c_attn": "matmul", "assign_k": "rendered", "assign_v": "rendered", "scores": "matmul", "softmax": "softmax",
+    "values": "matmul", "merge_heads": "rendered", "attn_proj": "matmul", "c_fc": "matmul", "mlp_proj": "matmul",
+    "lm_head": "matmul", "argmax": "argmax"}
+
+
+def _create(text: bytes):
+    from caten_amd import _lib
+    lib = _lib.load()
+    prog = ctypes.c_void_p()
+    rc = lib.cthip_program_create(ctypes.byref(prog), text)
+    assert rc == 0, lib.cthip_last_error().decode()
+    route, src = lib.cthip_program_route(prog).decode(), lib.cthip_program_source(prog).decode()
+    lib.cthip_program_destroy(prog)
+    return route, src
+
+
+def test_gpt2_step_items_print_as_their_golden_text_and_route():
+    """every distinct item of the decode step (external/llm/layers.lisp:3-90): the printer's text is the committed
+    fixture, the library reads it, and each Linear / attention / norm / embedding / argmax item has a hand-written
+    kernel behind it"""
+    from caten_amd import blueprints as bp, synth
+    from caten_amd.renderer import item_sexp
+    items = bp.gpt2_step_items(synth.GPT2_CONFIGS["gpt2"])
+    assert set(items) == set(GPT2_ITEM_ROUTES)
+    for key, item in items.items():
+        with open(os.path.join(GOLDEN_BP, f"gpt2_{key}.sexp")) as f:
+            golden = f.read()
+        assert item_sexp(item) == golden, f"{key}: the printed blueprint differs from tests/golden/blueprints/gpt2_{key}.sexp"
+        route, src = _create(golden.encode())
+        assert route == GPT2_ITEM_ROUTES[key], (key, route)
+        assert 'extern "C" __global__' in src
+
+
+def test_blueprints_in_a_lisp_printers_spelling_are_read_the_same():
+    """upper-case symbols, exponent markers (0.0f0, 1.0e-5, ...d0), single-float folded constants (1/768 =
+    0.0013020834, 3e-8 off), commutative operands in another order; and the one rendered matmul the reference's own
+    tests hold, with its index expressions verbatim (source/test-suite/test-scheduler.lisp:117-138)"""
+    for name, want in (("lisp_spelling_layernorm", "layernorm"), ("lisp_spelling_linear_gelu", "matmul"),
+                       ("reference_chunk_matmul", "matmul")):
+        with open(os.path.join(GOLDEN_BP, name + ".sexp"), "rb") as f:
+            route, _ = _create(f.read())
+        assert route == want, (name, route)
+
+
+def test_near_misses_of_the_decode_step_items_stay_rendered():
+    from caten_amd import HipRenderer, blueprints as bp
+    import copy
+    r = HipRenderer()
+
+    def route(item):
+        r.render_kernel(item)
+        return item["route"]
+    A = lambda id_, idx: {"op": "AREF", "id": id_, "index": idx}  # noqa: E731
+    # Linear + GELU with another constant inside the tanh: not the kernels' GELU
+    it = bp.gpt2_linear(32, 16, bias=True, gelu=True)
+    text = repr(it).replace("0.7978845608", "0.81")
+    assert route(eval(text, {"inf": float("inf")})) == "rendered"
+    assert route(bp.gpt2_linear(32, 16, bias=True, gelu=True)) == "matmul"
+    # an epilogue that squares the accumulator, one that reads three more arrays, one that reads the output
+    sq = bp.gpt2_linear(32, 16, bias=False)
+    sq["blueprint"][-3]["expr"] = {"op": "MUL", "args": ["acc", "acc"]}
+    assert route(sq) == "rendered"
+    three = bp.gpt2_linear(32, 16, bias=True, residual=True)
+    three["blueprint"].insert(1, {"type": "DEFINE-GLOBAL", "id": "val_z", "dtype": "float32", "pointer_p": True, "arg_type": "input", "nrank": 1})
+    three["blueprint"][-3]["expr"] = {"op": "ADD", "args": [three["blueprint"][-3]["expr"], A("val_z", "_gid1")]}
+    assert route(three) == "rendered"
+    own = bp.gpt2_linear(32, 16, bias=False)
+    own["blueprint"][-3]["expr"] = {"op": "ADD", "args": ["acc", A("val_y", {"op": "ADD", "args": [{"op": "MUL", "args": [32, "_gid0"]}, "_gid1"]})]}
+    assert route(own) == "rendered"
+    # the bias added AFTER the GELU is still a matmul item (the router decides at launch which kernel can apply it)
+    post = bp.gpt2_linear(32, 16, bias=False, gelu=True)
+    post["blueprint"].insert(4, {"type": "DEFINE-GLOBAL", "id": "val_b", "dtype": "float32", "pointer_p": True, "arg_type": "input", "nrank": 1})
+    post["blueprint"][-3]["expr"] = {"op": "ADD", "args": [post["blueprint"][-3]["expr"], A("val_b", "_gid1")]}
+    assert route(post) == "matmul"
+    # softmax whose second loop reads the row shifted by one element; LayerNorm whose store loop does
+    sm = bp.gpt2_softmax_rows(4)
+    shifted = copy.deepcopy(sm)
+    red = [n for n in shifted["blueprint"] if n.get("reduction") and n["writes"][0]["id"] == "e"][0]
+    aref = red["expr"]["args"][1]["args"][0]["args"][0]["args"][0]
+    assert aref["op"] == "AREF"
+    aref["index"] = {"op": "ADD", "args": [aref["index"], 1]}
+    assert route(sm) == "softmax" and route(shifted) == "rendered"
+    ln = bp.gpt2_layernorm(64)
+    shifted = copy.deepcopy(ln)
+    st = shifted["blueprint"][-3]
+    assert st["writes"][0]["id"] == "val_y"
+    centred = st["expr"]["args"][0]["args"][0]["args"][0]  # (x - u): the blueprint shares one aref object between its loops
+    xa = centred["args"][0]
+    assert xa["op"] == "AREF" and xa["id"] == "val_x"
+    st["expr"]["args"][0]["args"][0]["args"][0] = {"op": "ADD", "args": [A("val_x", {"op": "ADD", "args": [xa["index"], 1]}), centred["args"][1]]}
+    assert route(ln) == "layernorm" and route(shifted) == "rendered"
+    # the position embedding compared with something that also depends on the column: not a row gather
+    pe = bp.gpt2_embed_positions_add(64, 32)
+    bad = eval(repr(pe).replace("{'op': 'ADD', 'args': ['n', '_gid0']}", "{'op': 'ADD', 'args': ['n', '_gid1']}"), {"inf": float("inf")})
+    assert route(pe) == "embedding" and route(bad) == "rendered"

@@ -41,7 +41,9 @@ def _time(lib, fn, reps=50, warm=5):
     return ms.value * 1e3 / reps  # us
 
 
-def main():
+def measure(rendered_items: bool = True):
+    """Every figure as a dict.  `rendered_items` False leaves out the blueprint-rendered variants of the row ops (and
+    their hipRTC compilation) and times the hand-written items only."""
     lib = _lib.init(0)
     rng = np.random.default_rng(0)
     out = []
@@ -93,33 +95,6 @@ def main():
         ("LayerNorm (64,1024,768)", lambda: _lib.check(lib.cthip_layernorm(y.ptr, x.ptr, g.ptr, b.ptr, 1e-5, rows, d))),
         ("softmax (64,1024,768)", lambda: _lib.check(lib.cthip_softmax(y.ptr, x.ptr, rows, d))),
     ]
-    # the same softmax as a RENDERED kernel: blueprint -> HIP source (one wavefront per row) -> hipRTC
-    from caten_amd import blueprints
-    from caten_amd.renderer import HipRenderer
-    from caten_amd.buffer import HipBuffer
-
-    it = blueprints.softmax_rows()  # dynamic shape: rows and n are arguments
-    its = blueprints.softmax_rows("fused_softmax_static", rows, d)  # static shape: the bounds are literals
-    rr = HipRenderer()
-    rr.render_kernel(it)
-    rr.render_kernel(its)
-    rr.compile_kernel([it, its])
-    # buffers over the same device arrays the hand-written items use
-    bx = HipBuffer(shape=[rows, d], stride=[d, 1], dtype="float32", nrank=2, value=x.ptr)
-    by = HipBuffer(shape=[rows, d], stride=[d, 1], dtype="float32", nrank=2, value=y.ptr)
-    items.append(("softmax (64,1024,768), its blueprint through the program interface (routed to the row kernel), dynamic shape",
-                  lambda: it["compiled_object"](None, by, rows, d, bx)))
-
-    def rendered(item, *args):
-        def run():
-            _lib.check(lib.cthip_set_option(b"render_routes", 0))
-            try:
-                item["compiled_object"](None, *args)
-            finally:
-                _lib.check(lib.cthip_set_option(b"render_routes", 1))
-        return run
-    items.append(("softmax (64,1024,768), RENDERED from its blueprint, dynamic shape", rendered(it, by, rows, d, bx)))
-    items.append(("softmax (64,1024,768), RENDERED from its blueprint, static shape", rendered(its, by, bx)))
     # the streaming ceiling of this box: a device-to-device copy of the same array (the same bytes read and written)
     copy_us = _time(lib, lambda: _lib.check(lib.cthip_d2d(y.ptr, x.ptr, rows * d * 4)))
     if not np.array_equal(y.numpy()[rs], xh[rs]):
@@ -127,26 +102,54 @@ def main():
     copy_gbs = nbytes / (copy_us * 1e-6) / 1e9
     out.append({"item": "device-to-device copy (64,1024,768): the measured streaming ceiling", "us": copy_us, "achieved": copy_gbs,
                 "unit": "GB/s", "peak": 8000.0, "frac": copy_gbs / 8000.0, "bytes": nbytes})
-    # GELU(tanh) as a RENDERED element-wise kernel (there is no route for it: this is what an item of that shape runs)
-    ig = blueprints.gelu_tanh()
-    igs = blueprints.gelu_tanh("fused_gelu_static", rows, d)
-    rr.render_kernel(ig)
-    rr.render_kernel(igs)
-    rr.compile_kernel([ig, igs])
-    items.append(("GELU(tanh) (64,1024,768), RENDERED from its blueprint, dynamic shape", lambda: ig["compiled_object"](None, by, rows, d, bx)))
-    items.append(("GELU(tanh) (64,1024,768), RENDERED from its blueprint, static shape", lambda: igs["compiled_object"](None, by, bx)))
-    # LayerNorm -> softmax as ONE rendered item (five loops over the row)
-    bg = HipBuffer(shape=[d], stride=[1], dtype="float32", nrank=1, value=g.ptr)
-    bb = HipBuffer(shape=[d], stride=[1], dtype="float32", nrank=1, value=b.ptr)
-    il = blueprints.layernorm_softmax_rows()
-    ils = blueprints.layernorm_softmax_rows("fused_layernorm_softmax_static", 1e-5, rows, d)
-    rr.render_kernel(il)
-    rr.render_kernel(ils)
-    rr.compile_kernel([il, ils])
-    items.append(("LayerNorm->softmax (64,1024,768), RENDERED from its blueprint, dynamic shape",
-                  lambda: il["compiled_object"](None, by, rows, d, bx, bg, bb)))
-    items.append(("LayerNorm->softmax (64,1024,768), RENDERED from its blueprint, static shape",
-                  lambda: ils["compiled_object"](None, by, bx, bg, bb)))
+    if rendered_items:
+        # the same softmax as a RENDERED kernel: blueprint -> HIP source (one wavefront per row) -> hipRTC
+        from caten_amd import blueprints
+        from caten_amd.renderer import HipRenderer
+        from caten_amd.buffer import HipBuffer
+
+        it = blueprints.softmax_rows()  # dynamic shape: rows and n are arguments
+        its = blueprints.softmax_rows("fused_softmax_static", rows, d)  # static shape: the bounds are literals
+        rr = HipRenderer()
+        rr.render_kernel(it)
+        rr.render_kernel(its)
+        rr.compile_kernel([it, its])
+        # buffers over the same device arrays the hand-written items use
+        bx = HipBuffer(shape=[rows, d], stride=[d, 1], dtype="float32", nrank=2, value=x.ptr)
+        by = HipBuffer(shape=[rows, d], stride=[d, 1], dtype="float32", nrank=2, value=y.ptr)
+        items.append(("softmax (64,1024,768), its blueprint through the program interface (routed to the row kernel), dynamic shape",
+                      lambda: it["compiled_object"](None, by, rows, d, bx)))
+
+        def rendered(item, *args):
+            def run():
+                _lib.check(lib.cthip_set_option(b"render_routes", 0))
+                try:
+                    item["compiled_object"](None, *args)
+                finally:
+                    _lib.check(lib.cthip_set_option(b"render_routes", 1))
+            return run
+        items.append(("softmax (64,1024,768), RENDERED from its blueprint, dynamic shape", rendered(it, by, rows, d, bx)))
+        items.append(("softmax (64,1024,768), RENDERED from its blueprint, static shape", rendered(its, by, bx)))
+        # GELU(tanh) as a RENDERED element-wise kernel (there is no route for it: this is what an item of that shape runs)
+        ig = blueprints.gelu_tanh()
+        igs = blueprints.gelu_tanh("fused_gelu_static", rows, d)
+        rr.render_kernel(ig)
+        rr.render_kernel(igs)
+        rr.compile_kernel([ig, igs])
+        items.append(("GELU(tanh) (64,1024,768), RENDERED from its blueprint, dynamic shape", lambda: ig["compiled_object"](None, by, rows, d, bx)))
+        items.append(("GELU(tanh) (64,1024,768), RENDERED from its blueprint, static shape", lambda: igs["compiled_object"](None, by, bx)))
+        # LayerNorm -> softmax as ONE rendered item (five loops over the row)
+        bg = HipBuffer(shape=[d], stride=[1], dtype="float32", nrank=1, value=g.ptr)
+        bb = HipBuffer(shape=[d], stride=[1], dtype="float32", nrank=1, value=b.ptr)
+        il = blueprints.layernorm_softmax_rows()
+        ils = blueprints.layernorm_softmax_rows("fused_layernorm_softmax_static", 1e-5, rows, d)
+        rr.render_kernel(il)
+        rr.render_kernel(ils)
+        rr.compile_kernel([il, ils])
+        items.append(("LayerNorm->softmax (64,1024,768), RENDERED from its blueprint, dynamic shape",
+                      lambda: il["compiled_object"](None, by, rows, d, bx, bg, bb)))
+        items.append(("LayerNorm->softmax (64,1024,768), RENDERED from its blueprint, static shape",
+                      lambda: ils["compiled_object"](None, by, bx, bg, bb)))
     for name, fn in items:
         us = _time(lib, fn)
         key = [k for k in want if name.startswith(k)]
@@ -154,7 +157,13 @@ def main():
         gbs = nbytes / (us * 1e-6) / 1e9
         out.append({"item": name, "us": us, "achieved": gbs, "unit": "GB/s", "peak": 8000.0, "frac": gbs / 8000.0,
                     "frac_of_copy": gbs / copy_gbs, "bytes": nbytes})
-    for o in out:
+    for a in (A, B, Cm, x, y, g, b):
+        a.free()
+    return out
+
+
+def main():
+    for o in measure():
         print(json.dumps(o))
 
 

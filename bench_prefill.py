@@ -21,10 +21,11 @@ sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 from caten_amd import _lib, llm, synth  # noqa: E402
 
 
-def main(model="gpt2", kind="q8_0", s=512):
+def measure(model="gpt2", kind="q8_0", s=512, modes=(0, 3, 2, 1), weights=None, reps=5):
+    """one dict per operand format in `modes` (the first one is the reference the others' logits are checked against)"""
     llama = model in synth.LLAMA_CONFIGS
     cfg = synth.LLAMA_CONFIGS[model] if llama else synth.GPT2_CONFIGS[model]
-    w = synth.llama_weights(cfg, seed=0) if llama else synth.gpt2_weights(cfg, seed=0)
+    w = weights if weights is not None else (synth.llama_weights(cfg, seed=0) if llama else synth.gpt2_weights(cfg, seed=0))
     prompt = [float(t) for t in synth.prompt(cfg["vocab"], s, seed=0)]
     lib = _lib.init(0)
     m = llm.make_llama(cfg, llm.llama_state_dict(w, kind)) if llama else llm.make_gpt2(cfg, llm.gpt2_state_dict(w, kind))
@@ -37,7 +38,10 @@ def main(model="gpt2", kind="q8_0", s=512):
     att_flop = 2.0 * 2.0 * L * cfg["n_heads"] * (D // cfg["n_heads"]) * s * (s + 1) / 2
     names = {0: "fp32", 3: "3-term split bf16 (6 MFMAs per product)", 2: "2-term split bf16 (3 MFMAs per product)", 1: "bf16"}
     ref_tok = ref_logits = None
-    for mode, peak in ((0, 157.3), (3, 2500.0), (2, 2500.0), (1, 2500.0)):
+    peaks = {0: 157.3, 3: 2500.0, 2: 2500.0, 1: 2500.0}
+    out = []
+    for mode in modes:
+        peak = peaks[mode]
         _lib.check(lib.cthip_set_option(b"gemm_precision", mode))
         tok, logits = m.forward(prompt, s, 0, return_logits=True)
         if ref_logits is None:
@@ -53,17 +57,23 @@ def main(model="gpt2", kind="q8_0", s=512):
                 raise SystemExit(f"bench_prefill: {names[mode]}: {int(bad.sum())} logits differ from the fp32-operand run "
                                  f"(token {tok} vs {ref_tok}); no figure is reported for a wrong result")
         ts = []
-        for _ in range(5):
+        for _ in range(reps):
             t0 = time.perf_counter()
             m.forward(prompt, s, 0)
             ts.append(time.perf_counter() - t0)
         t = min(ts)
-        print(json.dumps({"item": f"prefill {s} tokens {model} {kind} ({names[mode]} MFMA operands)",
-                          "ms": t * 1e3, "tokens_per_s": s / t, "linear_TFLOPs": lin_flop / t / 1e12,
-                          "peak_TFLOPs": peak, "frac": lin_flop / t / 1e12 / peak,
-                          "linear_GFLOP": lin_flop / 1e9, "attention_GFLOP": att_flop / 1e9}))
+        out.append({"item": f"prefill {s} tokens {model} {kind} ({names[mode]} MFMA operands)", "gemm_precision": mode,
+                    "ms": t * 1e3, "tokens_per_s": s / t, "linear_TFLOPs": lin_flop / t / 1e12,
+                    "peak_TFLOPs": peak, "frac": lin_flop / t / 1e12 / peak,
+                    "linear_GFLOP": lin_flop / 1e9, "attention_GFLOP": att_flop / 1e9})
     _lib.check(lib.cthip_set_option(b"gemm_precision", 2))
     m.close()
+    return out
+
+
+def main(model="gpt2", kind="q8_0", s=512):
+    for o in measure(model, kind, s):
+        print(json.dumps(o))
 
 
 if __name__ == "__main__":

@@ -71,16 +71,23 @@ def gpt2_state_dict(weights: dict, linear_kind: str = "f32") -> Dict[str, Tensor
     return sd
 
 
-def llama_state_dict(weights: dict, linear_kind: str = "f32") -> Dict[str, Tensor]:
-    sd = {"tok_embeddings.weight": Tensor.from_f32(weights["tok_emb"]), "norm.weight": Tensor.from_f32(weights["norm_w"]),
-          "output.weight": Tensor.from_f32(weights["lm_head"], linear_kind)}
+def llama_state_dict(weights: dict, linear_kind: str = "f32", threads: int = 1) -> Dict[str, Tensor]:
+    """`threads` > 1 quantises the tensors on a thread pool (NumPy releases the interpreter lock inside its loops)."""
     names = {"attn_norm": "attention_norm.weight", "ffn_norm": "ffn_norm.weight", "wq": "attention.wq.weight",
              "wk": "attention.wk.weight", "wv": "attention.wv.weight", "wo": "attention.wo.weight",
              "w_gate": "feed_forward.w1.weight", "w_down": "feed_forward.w2.weight", "w_up": "feed_forward.w3.weight"}
+    jobs = [("tok_embeddings.weight", weights["tok_emb"], "f32"), ("norm.weight", weights["norm_w"], "f32"),
+            ("output.weight", weights["lm_head"], linear_kind)]
     for src, dst in names.items():
         for l, a in enumerate(weights[src]):
-            sd[f"layers.{l}.{dst}"] = Tensor.from_f32(a, linear_kind if src.startswith("w") else "f32")
-    return sd
+            jobs.append((f"layers.{l}.{dst}", a, linear_kind if src.startswith("w") else "f32"))
+    if threads > 1:
+        from concurrent.futures import ThreadPoolExecutor
+        with ThreadPoolExecutor(threads) as pool:
+            tensors = list(pool.map(lambda j: Tensor.from_f32(j[1], j[2]), jobs))
+    else:
+        tensors = [Tensor.from_f32(a, kind) for _, a, kind in jobs]
+    return {key: t for (key, _, _), t in zip(jobs, tensors)}
 
 
 class Transformer:

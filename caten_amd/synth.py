@@ -52,10 +52,37 @@ GPT2_LINEAR_KEYS = ("attn_w", "proj_w", "fc_w", "fc2_w")  # + "lm_head"
 LLAMA_LINEAR_KEYS = ("wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down")  # + "lm_head"
 
 
-def llama_weights(cfg: dict, seed: int = 0) -> dict:
-    rng = np.random.default_rng(seed)
+def llama_weights(cfg: dict, seed: int = 0, threads: int = 1) -> dict:
+    """Random-init fp32 weights ~N(0,0.02), norm weights ~N(1,0.02).  `threads` > 1 draws every tensor from a
+    generator of its own (seeded by (seed, tensor number)) on a thread pool: other values than the serial stream
+    gives, the same distribution, and a 1.1 B-parameter model in seconds instead of a minute."""
     D, F, V, L = cfg["dim"], cfg["ffn"], cfg["vocab"], cfg["n_layers"]
     KD = D // cfg["n_heads"] * cfg["n_kv_heads"]
+    if threads > 1:
+        from concurrent.futures import ThreadPoolExecutor
+        per_layer = {"attn_norm": ((D,), 1.0), "ffn_norm": ((D,), 1.0), "wq": ((D, D), 0.0), "wk": ((KD, D), 0.0),
+                     "wv": ((KD, D), 0.0), "wo": ((D, D), 0.0), "w_gate": ((F, D), 0.0), "w_up": ((F, D), 0.0),
+                     "w_down": ((D, F), 0.0)}
+        jobs = [("tok_emb", None, (V, D), 0.0), ("norm_w", None, (D,), 1.0), ("lm_head", None, (V, D), 0.0)]
+        jobs += [(k, l, sh, mean) for l in range(L) for k, (sh, mean) in per_layer.items()]
+
+        def draw(i):
+            _, _, shape, mean = jobs[i]
+            a = np.random.default_rng([seed, i]).standard_normal(shape, dtype=np.float32)
+            a *= np.float32(0.02)
+            if mean:
+                a += np.float32(mean)
+            return a
+        with ThreadPoolExecutor(threads) as pool:
+            arrs = list(pool.map(draw, range(len(jobs))))
+        w = {k: [None] * L for k in per_layer}
+        for (k, l, _, _), a in zip(jobs, arrs):
+            if l is None:
+                w[k] = a
+            else:
+                w[k][l] = a
+        return w
+    rng = np.random.default_rng(seed)
 
     def n(*shape, mean=0.0):
         return (mean + 0.02 * rng.standard_normal(shape, dtype=np.float32)).astype(np.float32)

@@ -27,6 +27,9 @@ struct State {
   int prefill_gemm = 1;   // option "prefill_gemm": 0 = prompts are fed row by row through the decode step
   int decode_fused = 1;   // option "decode_fused": 0 = five launches per layer instead of three
   int render_routes = 1;  // option "render_routes": 0 = every program runs its rendered kernel, none a hand-written one
+  // option "decode_skip": launches of the three-launch decode step that are left out, for knock-out timing (bits: 1 qkv,
+  // 2 attention + projection, 4 MLP, 8 the sum in front of lm_head, 16 lm_head + argmax); tokens are meaningless then
+  int decode_skip = 0;
 };
 State &state();
 // cthip_alloc without the zero fill, for temporaries that are fully written before they are read

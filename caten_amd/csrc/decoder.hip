@@ -430,6 +430,7 @@ static int queue_step(Decoder *d, bool with_head, bool embed) {
     // four workgroups per head repeat the head's attention and share its slab of the projection: what one
     // compute unit must fetch bounds a launch (GPT-2 small: 182 -> 173 us / step; six or twelve: no further gain)
     const int replicas = 4;
+    const int skip = state().decode_skip;  // knock-out timing only
     for (int l = 0; l < c.n_layers; l++) {
       Layer &L = d->layers[l];
       DecQkvArgs qa = {};
@@ -449,7 +450,7 @@ static int queue_step(Decoder *d, bool with_head, bool embed) {
       qa.vc = L.v_cache;
       qa.pos = pos;
       qa.rows = 3 * D;
-      TRY(launch_dec_qkv(qa, L.attn->type, l > 0));
+      if (!(skip & 1)) TRY(launch_dec_qkv(qa, L.attn->type, l > 0));
       DecAttnArgs aa = {};
       aa.q = d->q;
       aa.kc = L.k_cache;
@@ -460,7 +461,7 @@ static int queue_step(Decoder *d, bool with_head, bool embed) {
       aa.part = d->patt;
       aa.zero = d->pmlp;
       aa.zero_n16 = (int64_t)kDecXcds * D * 8 / 16;
-      TRY(launch_dec_attn_proj(aa, L.attn->type, c.n_heads, D, replicas));
+      if (!(skip & 2)) TRY(launch_dec_attn_proj(aa, L.attn->type, c.n_heads, D, replicas));
       DecMlpArgs ma = {};
       ma.st.base = d->x2;
       ma.st.bias = L.proj_b;
@@ -476,15 +477,15 @@ static int queue_step(Decoder *d, bool with_head, bool embed) {
       ma.pq = L.fc2_sq;
       ma.pd = (const unsigned short *)L.fc2_sd;
       ma.accum = d->pmlp;
-      TRY(launch_dec_mlp(ma, L.attn->type, F, c.n_heads));
+      if (!(skip & 4)) TRY(launch_dec_mlp(ma, L.attn->type, F, c.n_heads));
     }
     DecStage fin = {};
     fin.base = d->x;
     fin.bias = d->layers[c.n_layers - 1].fc2_b;
     fin.iparts = d->pmlp;
     fin.D = D;
-    TRY(launch_dec_sum(fin, d->x));
-    if (with_head) TRY(queue_head(d));
+    if (!(skip & 8)) TRY(launch_dec_sum(fin, d->x));
+    if (with_head && !(skip & 16)) TRY(queue_head(d));
     return 0;
   }
   if (d->fused_gqa) {

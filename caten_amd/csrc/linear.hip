@@ -673,6 +673,11 @@ int cthip_set_option(const char *name, int value) {
     else state().decode_fused = value;
     return 0;
   }
+  if (!strcmp(name, "decode_skip")) {
+    if (value < 0 || value > 31) return fail(CTHIP_E_BAD_ARG, "cthip_set_option: decode_skip is a mask of 5 bits");
+    state().decode_skip = value;
+    return 0;
+  }
   if (!strcmp(name, "gemm_bf16")) {  // 1 = operands rounded to bf16, 0 = back to the default
     state().gemm_precision = value ? GEMM_BF16 : GEMM_BF16X3;
     return 0;

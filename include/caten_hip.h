@@ -208,7 +208,10 @@ int cthip_linear(float *y, const void *wmat, const float *x, int m, const float 
  * "gemv_stream_weights": whether the single-row Linear kernels request the weights with the non-temporal
  *   hint: -1 (default) = per matrix -- a matrix larger than the 256 MB Infinity Cache, and every matrix of a
  *   decoder session whose weights together exceed three quarters of it; 0 = never; 1 = always.  Results do
- *   not depend on it.  A decoder session picks its kernels when it first runs. */
+ *   not depend on it.  A decoder session picks its kernels when it first runs.
+ * "decode_skip": knock-out timing of the three-launch decode step -- a mask of launches a session created
+ *   afterwards leaves out (1 qkv, 2 attention + projection, 4 MLP, 8 the sum in front of lm_head,
+ *   16 lm_head + argmax).  Tokens and logits of such a session are meaningless; 0 (default) = none. */
 int cthip_set_option(const char *name, int value);
 
 /* !relu(!matmul A B) (api/high-level-ops.lisp:76-99; fused per test-scheduler.lisp:140-163):

@@ -89,6 +89,8 @@ PROTOTYPES = {
     "cthip_argmax": (_i, [_vp, _vp, _i64, _i]),
     "cthip_rope": (_i, [_vp, _vp, _i, _i, _i, _i, _f, _i]),
     "cthip_sdpa_cached": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i]),
+    "cthip_kv_append_q8": (_i, [_vp, _vp, _vp, _i, _i, _i]),
+    "cthip_sdpa_cached_q8": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
     "cthip_decoder_create": (_i, [_vpp, C.POINTER(DecoderConfig)]),
     "cthip_decoder_destroy": (_i, [_vp]),
     "cthip_decoder_load": (_i, [_vp, C.c_char_p, _i, _vp, _i64, _i64]),
@@ -98,6 +100,7 @@ PROTOTYPES = {
     "cthip_decoder_generate_until": (_i, [_vp, _i, _i64, _vp, C.POINTER(_i)]),
     "cthip_decoder_position": (_i, [_vp]),
     "cthip_decoder_step_bytes": (_i64, [_vp, _i]),
+    "cthip_decoder_layer_launches": (_i, [_vp]),
     "cthip_decoder_peek": (_i, [_vp, C.c_char_p, _vpp, C.POINTER(_i64)]),
     "cthip_gguf_open": (_i, [_vpp, C.c_char_p]),
     "cthip_gguf_close": (_i, [_vp]),

@@ -30,6 +30,7 @@ struct State {
   // option "decode_skip": launches of the three-launch decode step that are left out, for knock-out timing (bits: 1 qkv,
   // 2 attention + projection, 4 MLP, 8 the sum in front of lm_head, 16 lm_head + argmax); tokens are meaningless then
   int decode_skip = 0;
+  int kv_cache = 0;  // option "kv_cache": 1 = sessions created afterwards keep their KV cache as Q8_0 rows (kvq.hip)
 };
 State &state();
 // cthip_alloc without the zero fill, for temporaries that are fully written before they are read
@@ -94,6 +95,12 @@ struct BmmArgs {
 };
 int bmm_variant(const BmmArgs &a);  // 0 = neither layout fits
 int launch_bmm(const BmmArgs &a);
+
+// ---- KV cache as Q8_0 rows (kvq.hip): quant plane int8[max_len][KD], scale plane fp16[max_len][KD/32] ----
+int launch_kvq_append(void *q, void *d, const float *src, int64_t src_stride, int s, int row0, const int *pos, int KD);
+int launch_kvq_dequant(float *dst, const void *q, const void *d, int rows, int KD);
+int launch_attn_q8(float *out, const float *q, const void *kq, const void *kd, const void *vq, const void *vd, int start_pos,
+                   const int *pos, int H, int Hkv, int Dh);
 
 // Arguments of one fused Linear launch:
 //   y = act(prologue(x) . W^T + bias) + residual

@@ -470,6 +470,19 @@ __global__ void k_xcd_probe(int *out) {
   }
 }
 
+// The accumulators of the column Linears are updated by DIFFERENT workgroups of an XCD with atomics that carry no
+// device-scope bits.  That the additions of all compute units of an XCD meet (in its L2) is a property of the part,
+// not a promise of the memory model, so it is checked before a session relies on it: every thread adds a known
+// fixed-point value to a cell of its XCD's row that way (acc) and the same value with a device-scope atomic (ref);
+// the two arrays must be identical after the kernel.  64 cells per XCD, thousands of workgroups on all compute units.
+__global__ __launch_bounds__(256) void k_xcd_atomics_probe(long long *acc, long long *ref) {
+  const int x = xcd_id();
+  const int cell = x * 64 + (threadIdx.x & 63);
+  const long long v = to_fix(0.125f * (float)(1 + (blockIdx.x % 7)) + 0.001f * (float)(threadIdx.x >> 6));
+  __hip_atomic_fetch_add(acc + cell, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  __hip_atomic_fetch_add(ref + cell, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // ------------------------------------------------------------------ host side
 static int type_xpc(int type) { return type == CTHIP_Q8_0 ? 16 : type == CTHIP_F16 ? 8 : type == CTHIP_F32 ? 4 : 0; }
 
@@ -483,16 +496,38 @@ bool dec_fused_supported(int type_attn, int type_proj, int type_fc, int type_fc2
   return true;
 }
 
+// max_id: the largest XCD id seen; *max_id = -1 when the per-XCD atomics did not add up (see k_xcd_atomics_probe)
 int dec_xcd_probe(int *max_id) {
+  static int cached = -2;  // the answer is a property of the device: asked once per process
+  if (cached != -2) {
+    *max_id = cached;
+    return 0;
+  }
   int *dev = nullptr;
-  int rc = cthip_alloc((void **)&dev, 256);
+  const size_t cells = (size_t)kDecXcds * 64;
+  int rc = cthip_alloc((void **)&dev, 256 + 2 * cells * sizeof(long long));  // zero-filled
   if (rc) return rc;
+  long long *acc = (long long *)((char *)dev + 256), *ref = acc + cells;
   hipLaunchKernelGGL(k_xcd_probe, dim3(4096), dim3(64), 0, state().stream, dev);
   hipError_t e = hipGetLastError();
+  if (e == hipSuccess) {
+    hipLaunchKernelGGL(k_xcd_atomics_probe, dim3(4096), dim3(256), 0, state().stream, acc, ref);
+    e = hipGetLastError();
+  }
+  long long host[2 * kDecXcds * 64];
   if (e == hipSuccess) rc = cthip_d2h(max_id, dev, sizeof(int));
+  if (e == hipSuccess && !rc) rc = cthip_d2h(host, acc, sizeof(host));
   cthip_free(dev);
   if (e != hipSuccess) return fail((int)e, "decoder: XCD probe -> %s", hipGetErrorString(e));
-  return rc;
+  if (rc) return rc;
+  long long total = 0;
+  for (size_t k = 0; k < cells; k++) {
+    if (host[k] != host[cells + k]) *max_id = -1;
+    total += host[cells + k] != 0;
+  }
+  if (total == 0) *max_id = -1;  // nothing was added at all
+  cached = *max_id;
+  return 0;
 }
 
 // group_cols columns per group; scales (Q8_0): groups_per_scale groups share the 32-column block of a scale

@@ -62,6 +62,8 @@ struct Layer {
   // Llama: attn = wq|wk|wv, proj = wo, fc = gate|up, fc2 = down, ln1_g/ln2_g = rms weights
   bool fc_pairs = false;  // gate / up rows interleaved, SwiGLU in the gate|up launch
   float *k_cache = nullptr, *v_cache = nullptr;
+  // option kv_cache 1: the cache as Q8_0 rows instead (quant and scale planes; k_cache / v_cache stay null)
+  void *kq = nullptr, *kdq = nullptr, *vq = nullptr, *vdq = nullptr;
   // three-launch decode layer: attn.c_proj by head and mlp.c_proj by 16-column slab (quant / scale planes)
   void *proj_hq = nullptr, *proj_hd = nullptr, *fc2_sq = nullptr, *fc2_sd = nullptr;
 };
@@ -99,6 +101,9 @@ struct Decoder {
   // grouped-query layers (decode_gqa.hip): the attention projection has an accumulator set of its own
   bool fused_gqa = false;
   long long *pattn = nullptr;
+  // KV cache kept as Q8_0 rows (kvq.hip); peek_f32: fp32 copy of one layer's cache for cthip_decoder_peek
+  bool kvq = false;
+  float *peek_f32 = nullptr;
   hipGraphExec_t g_step = nullptr, g_body = nullptr, g_multi = nullptr;
   int64_t weight_bytes = 0, vector_bytes = 0;
   std::vector<void *> owned;  // device blocks to free
@@ -296,10 +301,20 @@ static int finalize(Decoder *d) {
   d->vector_bytes -= 4 * (int64_t)V * D;
   if (c.arch == CTHIP_ARCH_GPT2) d->vector_bytes -= 4 * (int64_t)c.max_seq * D;
 
+  d->kvq = state().kv_cache == 1;
+  if (d->kvq && KD % 32) return fail(CTHIP_E_UNSUPPORTED, "decoder: a Q8_0 KV cache needs rows of whole 32-element blocks, not %d", KD);
   for (int l = 0; l < c.n_layers; l++) {
+    Layer &L = d->layers[l];
+    if (d->kvq) {  // zero quants and zero scales: rows of zeros, as the fp32 cache starts
+      TRY(dev_alloc(d, &L.kq, (size_t)c.max_seq * KD));
+      TRY(dev_alloc(d, &L.vq, (size_t)c.max_seq * KD));
+      TRY(dev_alloc(d, &L.kdq, sizeof(unsigned short) * (size_t)c.max_seq * (KD / 32)));
+      TRY(dev_alloc(d, &L.vdq, sizeof(unsigned short) * (size_t)c.max_seq * (KD / 32)));
+      continue;
+    }
     // merge-kv-cache creates (B, max_len, H, Dh) zeros once (layers.lisp:25-26)
-    TRY(dev_alloc(d, (void **)&d->layers[l].k_cache, sizeof(float) * (size_t)c.max_seq * KD));
-    TRY(dev_alloc(d, (void **)&d->layers[l].v_cache, sizeof(float) * (size_t)c.max_seq * KD));
+    TRY(dev_alloc(d, (void **)&L.k_cache, sizeof(float) * (size_t)c.max_seq * KD));
+    TRY(dev_alloc(d, (void **)&L.v_cache, sizeof(float) * (size_t)c.max_seq * KD));
   }
   const int hdim = c.arch == CTHIP_ARCH_GPT2 ? F : 2 * F;
   TRY(dev_alloc(d, (void **)&d->x, sizeof(float) * D));
@@ -333,7 +348,7 @@ static int finalize(Decoder *d) {
     for (WMat *w : ws)
       if (w) w->stream = total > kInfinityCacheBytes / 4 * 3;
   }
-  if (c.arch == CTHIP_ARCH_GPT2 && state().decode_fused &&
+  if (c.arch == CTHIP_ARCH_GPT2 && state().decode_fused && !d->kvq &&
       dec_fused_supported(d->layers[0].attn->type, d->layers[0].proj->type, d->layers[0].fc->type,
                           d->layers[0].fc2->type, D, c.n_heads, F)) {
     // the per-XCD accumulators assume what gfx950 has: XCD ids 0..7
@@ -358,7 +373,7 @@ static int finalize(Decoder *d) {
       TRY(dev_alloc(d, (void **)&d->pmlp, sizeof(long long) * (size_t)kDecXcds * D));
     }
   }
-  if (c.arch == CTHIP_ARCH_LLAMA && state().decode_fused &&
+  if (c.arch == CTHIP_ARCH_LLAMA && state().decode_fused && !d->kvq &&
       gqa_fused_supported(d->layers[0].attn->type, d->layers[0].proj->type, d->layers[0].fc->type, d->layers[0].fc2->type,
                           D, c.n_heads, c.n_kv_heads, F)) {
     int max_id = -1;
@@ -573,7 +588,7 @@ static int queue_step(Decoder *d, bool with_head, bool embed) {
     a.split2 = D + KD;
     a.x_stride = D;
     a.y_stride = D;
-    if (gpt2) {
+    if (gpt2 && !d->kvq) {
       a.y1 = L.k_cache;
       a.y2 = L.v_cache;
       a.pos = pos;
@@ -585,7 +600,17 @@ static int queue_step(Decoder *d, bool with_head, bool embed) {
       a.pos_stride = 0;
     }
     TRY(launch_gemv(L.attn, a, 1));
-    if (!gpt2) {
+    if (d->kvq) {
+      // the new row is in kv_tmp (k then v): rotate q and k where the model rotates, quantise the row into the
+      // cache at `pos`, attend over the Q8_0 rows
+      if (!gpt2) {
+        TRY(launch_rope(d->q, d->q, 1, 1, c.n_heads, Dh, c.rope_base, 0, pos));
+        TRY(launch_rope(d->kv_tmp, d->kv_tmp, 1, 1, c.n_kv_heads, Dh, c.rope_base, 0, pos));
+      }
+      TRY(launch_kvq_append(L.kq, L.kdq, d->kv_tmp, KD, 1, 0, pos, KD));
+      TRY(launch_kvq_append(L.vq, L.vdq, d->kv_tmp + KD, KD, 1, 0, pos, KD));
+      TRY(launch_attn_q8(d->att, d->q, L.kq, L.kdq, L.vq, L.vdq, 0, pos, c.n_heads, c.n_kv_heads, Dh));
+    } else if (!gpt2) {
       // q and the new key are rotated inside the attention launch, which also appends k / v at `pos`
       TRY(launch_attn_rope_append(d->att, d->q, L.k_cache, L.v_cache, d->kv_tmp, pos, c.n_heads, c.n_kv_heads, Dh,
                                   c.rope_base));
@@ -676,7 +701,7 @@ static int prefill(Decoder *d, const int *ids, int s, int n) {
   const int QW = D + 2 * KD, HW = gpt2 ? F : 2 * F;
   const int prec = state().gemm_precision;
   int rc = 0;
-  float *X = nullptr, *XN = nullptr, *QKV = nullptr, *Q = nullptr, *ATT = nullptr, *Hb = nullptr, *G = nullptr;
+  float *X = nullptr, *XN = nullptr, *QKV = nullptr, *Q = nullptr, *ATT = nullptr, *Hb = nullptr, *G = nullptr, *KF = nullptr, *VF = nullptr;
   int *ids_dev = nullptr;
   std::vector<void *> tmp;
   auto alloc = [&](void **p, size_t bytes) {
@@ -695,6 +720,10 @@ static int prefill(Decoder *d, const int *ids, int s, int n) {
   TRY(alloc((void **)&ATT, sizeof(float) * (size_t)s * D));
   TRY(alloc((void **)&Hb, sizeof(float) * (size_t)s * HW));
   if (!gpt2) TRY(alloc((void **)&G, sizeof(float) * (size_t)s * F));
+  if (d->kvq) {
+    TRY(alloc((void **)&KF, sizeof(float) * (size_t)(n + s) * KD));
+    TRY(alloc((void **)&VF, sizeof(float) * (size_t)(n + s) * KD));
+  }
   TRY(alloc((void **)&ids_dev, sizeof(int) * (size_t)s));
   TRY(cthip_h2d(ids_dev, ids, sizeof(int) * (size_t)s));
   {
@@ -730,6 +759,17 @@ static int prefill(Decoder *d, const int *ids, int s, int n) {
     TRY(norm(XN, X, d->layers[0].ln1_g, d->layers[0].ln1_b));
     for (int l = 0; l < c.n_layers; l++) {
       Layer &L = d->layers[l];
+      if (d->kvq) {
+        // attention of a prompt batch runs on fp32 rows: the cached rows [0, n) are widened into a temporary, the
+        // batch's rows [n, n + s) join them (rotated where the model rotates) and are quantised into the cache
+        TRY(launch_kvq_dequant(KF, L.kq, L.kdq, n, KD));
+        TRY(launch_kvq_dequant(VF, L.vq, L.vdq, n, KD));
+        TRY(launch_linear_gemm(QKV, L.attn, XN, s, L.attn_b, nullptr, CTHIP_ACT_NONE, prec));
+        TRY(launch_qkv_split(Q, KF, VF, QKV, s, n, c.n_heads, c.n_kv_heads, Dh, gpt2 ? 0.0f : c.rope_base));
+        TRY(launch_kvq_append(L.kq, L.kdq, KF + (int64_t)n * KD, KD, s, n, nullptr, KD));
+        TRY(launch_kvq_append(L.vq, L.vdq, VF + (int64_t)n * KD, KD, s, n, nullptr, KD));
+        TRY(launch_attn(ATT, Q, KF, VF, s, n, nullptr, n + s, c.n_heads, c.n_kv_heads, Dh));
+      } else {
       if (gpt2 && D % 128 == 0 && KD % 128 == 0) {
         // no rotation: the thirds of the fused projection go straight to the query rows and the cache rows
         const GemmRoute rt = {{Q, L.k_cache + (int64_t)n * KD, L.v_cache + (int64_t)n * KD}, {0, D, D + KD}, {D, KD, KD}};
@@ -739,6 +779,7 @@ static int prefill(Decoder *d, const int *ids, int s, int n) {
         TRY(launch_qkv_split(Q, L.k_cache, L.v_cache, QKV, s, n, c.n_heads, c.n_kv_heads, Dh, gpt2 ? 0.0f : c.rope_base));
       }
       TRY(launch_attn(ATT, Q, L.k_cache, L.v_cache, s, n, nullptr, n + s, c.n_heads, c.n_kv_heads, Dh));
+      }
       TRY(linear_residual_norm(L.proj, ATT, L.proj_b, L.ln2_g, L.ln2_b));
       const float *hin = Hb;
       if (!gpt2 && L.fc_pairs && (2 * F) % 4 == 0) {  // SwiGLU in the epilogue of the gate|up launch
@@ -966,14 +1007,26 @@ int cthip_decoder_generate_until(void *dec, int max_steps, int64_t eos_token, in
 
 int cthip_decoder_position(const void *dec) { return dec ? ((const Decoder *)dec)->position : -1; }
 
+int cthip_decoder_layer_launches(void *dec) {
+  CTHIP_REQUIRE_INIT();
+  CTHIP_ARG(dec != nullptr);
+  Decoder *d = (Decoder *)dec;
+  int rc = finalize(d);
+  if (rc) return -1;
+  if (d->fused || d->fused_gqa) return 3;
+  if (d->kvq) return d->cfg.arch == CTHIP_ARCH_GPT2 ? 7 : 9;  // + two appends (+ two rotations) around the attention launch
+  return 5;
+}
+
 int64_t cthip_decoder_step_bytes(const void *dec, int t) {
   const Decoder *d = (const Decoder *)dec;
   if (!d || !d->finalized) return -1;
   const cthip_decoder_config &c = d->cfg;
   const int64_t KD = kv_dim(c);
   int64_t emb = 4LL * c.dim * (c.arch == CTHIP_ARCH_GPT2 ? 2 : 1);
-  int64_t kv_read = 2LL * c.n_layers * t * KD * 4;
-  int64_t kv_write = 2LL * c.n_layers * KD * 4;
+  // per element of a cache row: 4 bytes, or 1 + 2 / 32 as Q8_0
+  int64_t kv_read = d->kvq ? 2LL * c.n_layers * t * (KD + KD / 32 * 2) : 2LL * c.n_layers * t * KD * 4;
+  int64_t kv_write = d->kvq ? 2LL * c.n_layers * (KD + KD / 32 * 2) : 2LL * c.n_layers * KD * 4;
   return d->weight_bytes + d->vector_bytes + emb + kv_read + kv_write;
 }
 
@@ -993,12 +1046,26 @@ int cthip_decoder_peek(void *dec, const char *what, void **ptr, int64_t *n_float
   } else if (!strcmp(what, "x")) {
     p = d->x;
     n = c.dim;
-  } else if (sscanf(what, "k_cache.%d", &l) == 1 && l >= 0 && l < c.n_layers) {
-    p = d->layers[l].k_cache;
+  } else if ((sscanf(what, "k_cache.%d", &l) == 1 || sscanf(what, "v_cache.%d", &l) == 1) && l >= 0 && l < c.n_layers) {
+    const bool key = what[0] == 'k';
     n = (int64_t)c.max_seq * kv_dim(c);
-  } else if (sscanf(what, "v_cache.%d", &l) == 1 && l >= 0 && l < c.n_layers) {
-    p = d->layers[l].v_cache;
-    n = (int64_t)c.max_seq * kv_dim(c);
+    if (d->kvq) {
+      // Q8_0 rows: what the caller gets is their fp32 value, in a buffer that the next peek overwrites
+      if (!d->peek_f32 && (rc = dev_alloc(d, (void **)&d->peek_f32, sizeof(float) * (size_t)n))) return rc;
+      const Layer &L = d->layers[l];
+      if ((rc = launch_kvq_dequant(d->peek_f32, key ? L.kq : L.vq, key ? L.kdq : L.vdq, c.max_seq, kv_dim(c)))) return rc;
+      p = d->peek_f32;
+    } else {
+      p = key ? d->layers[l].k_cache : d->layers[l].v_cache;
+    }
+  } else if ((sscanf(what, "k_cache_q8.%d", &l) == 1 || sscanf(what, "v_cache_q8.%d", &l) == 1) && d->kvq && l >= 0 && l < c.n_layers) {
+    // the quant plane itself, int8[max_seq][KD]; n counts its bytes in units of four
+    p = what[0] == 'k' ? d->layers[l].kq : d->layers[l].vq;
+    n = (int64_t)c.max_seq * kv_dim(c) / 4;
+  } else if ((sscanf(what, "k_cache_d.%d", &l) == 1 || sscanf(what, "v_cache_d.%d", &l) == 1) && d->kvq && l >= 0 && l < c.n_layers) {
+    // the scale plane, fp16[max_seq][KD / 32]; n counts its bytes in units of four
+    p = what[0] == 'k' ? d->layers[l].kdq : d->layers[l].vdq;
+    n = (int64_t)c.max_seq * (kv_dim(c) / 32) / 2;
   } else {
     return fail(CTHIP_E_BAD_ARG, "cthip_decoder_peek: unknown buffer '%s'", what);
   }

@@ -209,6 +209,11 @@ int cthip_linear(float *y, const void *wmat, const float *x, int m, const float 
  *   hint: -1 (default) = per matrix -- a matrix larger than the 256 MB Infinity Cache, and every matrix of a
  *   decoder session whose weights together exceed three quarters of it; 0 = never; 1 = always.  Results do
  *   not depend on it.  A decoder session picks its kernels when it first runs.
+ * "kv_cache": how decoder sessions created afterwards keep their KV cache: 0 (default) = fp32 rows, the
+ *   reference's dense cache (external/llm/layers.lisp:19-33); 1 = GGUF-Q8_0 rows (blocks of 32 int8 and one fp16
+ *   scale per cache row, quantised once when the row is appended): 3.76x fewer cache bytes held and read per
+ *   step.  Such a session runs one launch per Linear; logits stay within rtol 2e-2 / atol 2e-2 of the fp32
+ *   cache's on the tested models (the band of 8-bit keys and values, not of the fp32 arithmetic around them).
  * "decode_skip": knock-out timing of the three-launch decode step -- a mask of launches a session created
  *   afterwards leaves out (1 qkv, 2 attention + projection, 4 MLP, 8 the sum in front of lm_head,
  *   16 lm_head + argmax).  Tokens and logits of such a session are meaningless; 0 (default) = none. */
@@ -257,6 +262,16 @@ int cthip_rope(float *out, const float *x, int B, int S, int H, int Dh, float ba
  * "gemm_precision" is 0. */
 int cthip_sdpa_cached(float *out, const float *q, const float *k_cache, const float *v_cache,
                       int S, int start_pos, int H, int Hkv, int Dh);
+/* The same cache as GGUF-Q8_0 rows (the reference's cache is dense fp32, layers.lisp:19-33; its Q8_0 block is
+ * external/gguf/dequantize.lisp:40-53): a quant plane int8[max_len][kv_dim] and a scale plane fp16[max_len][kv_dim/32].
+ * cthip_kv_append_q8 quantises `s` fp32 rows (s, kv_dim) into cache rows row0 .. row0+s-1 (per block of 32:
+ * d = absmax / 127 stored as fp16, q = x / d rounded half away from zero -- ggml's reference row quantiser).
+ * cthip_sdpa_cached_q8 attends ONE query row (H, Dh) over cache rows 0 .. T-1 (the decode step; every key is
+ * visible to the last position), out (H, Dh): the products run on the integers, a block's scale is applied to
+ * its partial sum. */
+int cthip_kv_append_q8(void *q_plane, void *d_plane, const float *rows, int s, int row0, int kv_dim);
+int cthip_sdpa_cached_q8(float *out, const float *q, const void *k_q, const void *k_d, const void *v_q, const void *v_d, int T,
+                         int H, int Hkv, int Dh);
 
 /* ================================================================== */
 /* Decoder session: Transformer (external/llm/layers.lisp:73-90) and   */
@@ -303,9 +318,18 @@ int cthip_decoder_generate(void *dec, int steps, int64_t *tokens_out);
 int cthip_decoder_generate_until(void *dec, int max_steps, int64_t eos_token, int64_t *tokens_out, int *n_generated);
 /* Current position (tokens in the KV cache). */
 int cthip_decoder_position(const void *dec);
-/* Bytes of HBM one decode step must read at position t (weights + norms/biases + KV rows). */
+/* Bytes of HBM one decode step must read at position t (weights + norms/biases + KV rows at their stored
+ * size: 4 bytes per element, 1.0625 with option "kv_cache" 1). */
 int64_t cthip_decoder_step_bytes(const void *dec, int t);
-/* Device pointers into the session, for parity tests: "k_cache.<l>", "v_cache.<l>", "logits", "x". */
+/* Launches per layer of one decode step of this session: 3 (attention + projection and the whole MLP merged,
+ * per-XCD accumulators -- taken only when the device passed the load-time checks that XCD ids are 0..7 and that
+ * atomics of different workgroups of an XCD meet in its L2), 5 (one launch per Linear + attention), more with a
+ * Q8_0 KV cache (the append and, for RoPE models, the rotations are launches of their own).  -1 on error. */
+int cthip_decoder_layer_launches(void *dec);
+/* Device pointers into the session, for parity tests: "k_cache.<l>", "v_cache.<l>" (fp32 rows; with a Q8_0
+ * cache their dequantised values, in a buffer the next peek overwrites), "logits", "x"; with a Q8_0 cache also
+ * the planes themselves, "k_cache_q8.<l>" / "v_cache_q8.<l>" (int8[max_seq][kv_dim]) and "k_cache_d.<l>" /
+ * "v_cache_d.<l>" (fp16[max_seq][kv_dim / 32]), n_floats counting their bytes in units of four. */
 int cthip_decoder_peek(void *dec, const char *what, void **ptr, int64_t *n_floats);
 
 /* ================================================================== */

@@ -76,6 +76,24 @@
 (defun buffer-nbytes (buffer)
   (* (buffer-storage-size buffer) (dtype/size-of (buffer-dtype buffer))))
 
+;; What a rank > 0 HipBuffer keeps in its `value` slot is not the raw device pointer but a BLOCK: the pointer plus a
+;; flag that the storage is still allocated.  copy-buffer (source/runtime/buffer.lisp:60-68) copies slots, so a :View's
+;; buffer, every other copy and the buffer that opened the storage all hold the SAME block object.  Device storage has
+;; to go back to the allocator exactly once and must never be touched afterwards -- the caching allocator hands a freed
+;; address to the next open-buffer -- so: the first close-buffer through any of them frees the block and marks it dead;
+;; later closes (free-runtime closes every buffer of the variable table, runtime.lisp:76-81) find it dead and do
+;; nothing; and a stale view of a closed pool signals an error instead of reading or freeing somebody else's memory.
+(defstruct (hip-block (:constructor make-hip-block (pointer))) pointer (alive t))
+
+(defun device-pointer (buffer)
+  "The device address of a rank > 0 HipBuffer whose storage is still open."
+  (let ((blk (buffer-value buffer)))
+    (unless (hip-block-p blk)
+      (error "Caten[HIP]: ~a holds no device storage (open-buffer it first)" buffer))
+    (unless (hip-block-alive blk)
+      (error "Caten[HIP]: the storage of ~a has been closed" buffer))
+    (hip-block-pointer blk)))
+
 (defmethod open-buffer ((runtime HipRuntime) (buffer HipBuffer))
   ;; rank-0 buffers stay Lisp numbers, as in every other backend (metal.lisp:114-121);
   ;; cthip_alloc returns zeroed storage from a caching allocator
@@ -84,49 +102,42 @@
             (if (eql (buffer-dtype buffer) :bool) nil (coerce 0 (dtype->lisp (buffer-dtype buffer)))))
       (with-foreign-object (out :pointer)
         (check (%alloc out (buffer-nbytes buffer)))
-        (setf (gethash (pointer-address (mem-ref out :pointer)) *opened*) t)
-        (setf (buffer-value buffer) (mem-ref out :pointer)))))
-
-;; copy-buffer (source/runtime/buffer.lisp:60-68) shares the storage between a :View's buffer and its base, and
-;; free-runtime closes every buffer of the variable table (runtime.lisp:76-81).  Device storage must go back
-;; exactly once, so the pointers this backend opened are kept in a table: the first close of a pointer frees it,
-;; later closes (of views and copies, or of the same buffer again) only forget it.
-(defvar *opened* (make-hash-table :test #'eql) "device address -> t for every block open-buffer / copy-buffer-value took")
+        (setf (buffer-value buffer) (make-hip-block (mem-ref out :pointer))))))
 
 (defmethod close-buffer ((runtime HipRuntime) (buffer HipBuffer))
-  (when (pointerp (buffer-value buffer))
-    (let ((address (pointer-address (buffer-value buffer))))
-      (when (gethash address *opened*)
-        (remhash address *opened*)
-        (check (%free (buffer-value buffer)))))
-    (setf (buffer-value buffer) nil)))
+  (let ((blk (buffer-value buffer)))
+    (when (hip-block-p blk)
+      (when (hip-block-alive blk)
+        (setf (hip-block-alive blk) nil) ; every buffer sharing the block sees it closed from here on
+        (check (%free (hip-block-pointer blk))))
+      (setf (buffer-value buffer) nil))))
 
 (defmethod transfer-from-array ((runtime HipRuntime) (buffer HipBuffer) array)
   ;; the array is pinned only for the duration of the call; cthip_h2d stages it
   (with-pointer-to-vector-data (src array)
-    (check (%h2d (buffer-value buffer) src (buffer-nbytes buffer)))))
+    (check (%h2d (device-pointer buffer) src (buffer-nbytes buffer)))))
 
 (defmethod transfer-into-array ((buffer HipBuffer))
-  (when (numberp (buffer-value buffer))
+  (unless (hip-block-p (buffer-value buffer)) ; rank 0: the Lisp number / boolean itself
     (return-from transfer-into-array (buffer-value buffer)))
   (let ((placeholder (make-array (buffer-storage-size buffer) :element-type (dtype->lisp (buffer-dtype buffer)))))
     (with-pointer-to-vector-data (dst placeholder)
-      (check (%d2h dst (buffer-value buffer) (buffer-nbytes buffer)))) ; synchronises the stream
+      (check (%d2h dst (device-pointer buffer) (buffer-nbytes buffer)))) ; synchronises the stream
     placeholder))
 
 (defmethod copy-buffer-value ((runtime HipRuntime) (buffer HipBuffer))
-  (if (pointerp (buffer-value buffer))
+  ;; new storage with the same bytes: a block of its own, owned by whichever buffer the caller stores it in
+  (if (hip-block-p (buffer-value buffer))
       (with-foreign-object (out :pointer)
         (check (%alloc out (buffer-nbytes buffer)))
-        (check (%d2d (mem-ref out :pointer) (buffer-value buffer) (buffer-nbytes buffer)))
-        (setf (gethash (pointer-address (mem-ref out :pointer)) *opened*) t)
-        (mem-ref out :pointer))
+        (check (%d2d (mem-ref out :pointer) (device-pointer buffer) (buffer-nbytes buffer)))
+        (make-hip-block (mem-ref out :pointer)))
       (buffer-value buffer)))
 
 (defmethod bref ((buffer HipBuffer) idx)
   (let ((type (->cffi-dtype (buffer-dtype buffer))))
     (with-foreign-object (tmp type)
-      (check (%d2h tmp (inc-pointer (buffer-value buffer) (* idx (dtype/size-of (buffer-dtype buffer))))
+      (check (%d2h tmp (inc-pointer (device-pointer buffer) (* idx (dtype/size-of (buffer-dtype buffer))))
                    (dtype/size-of (buffer-dtype buffer))))
       (mem-ref tmp type))))
 
@@ -249,13 +260,13 @@
   "Weights loaded from GGUF are LispBuffers whatever BACKEND is (external/gguf/tensor-info.lisp:104-120)
 and enter through :Allocate :from untouched (source/runtime/runtime.lisp:228-243): upload once, cache."
   (cond
-    ((typep buf 'HipBuffer) (buffer-value buf))
+    ((typep buf 'HipBuffer) (device-pointer buf))
     ((and (buffer-p buf) (arrayp (buffer-value buf)))
      (or (gethash buf (hp-uploads hp))
          (let ((dev (make-buffer (buffer-shape buf) (buffer-stride buf) (buffer-dtype buf) (buffer-views buf) :device 'HipBuffer)))
            (open-buffer runtime dev)
            (transfer-from-array runtime dev (buffer-value buf))
-           (setf (gethash buf (hp-uploads hp)) (buffer-value dev)))))
+           (setf (gethash buf (hp-uploads hp)) (device-pointer dev)))))
     (t (error "Caten[HIP]: ~a is neither a device buffer nor a host array" buf))))
 
 (defmethod invoke ((hp Hip-Program) runtime node &rest buffers)
@@ -360,8 +371,8 @@ external/gguf/tensor-info.lisp:104-120, before it would dequantise them)."
   "A LayerNorm in front of this Linear is carried through the product from now on (cthip_wmat_fold_layernorm): later
 :QLinear nodes with prologue :layernorm and these same gamma / beta / bias buffers need the row statistics only in
 their epilogue."
-  (check (%wmat-fold-layernorm (packed-weight-handle weight) (buffer-value gamma) (buffer-value beta)
-                               (if bias (buffer-value bias) (null-pointer)))))
+  (check (%wmat-fold-layernorm (packed-weight-handle weight) (device-pointer gamma) (device-pointer beta)
+                               (if bias (device-pointer bias) (null-pointer)))))
 
 (defmethod realize-node ((id (eql :QLinear)) (runtime HipRuntime) node args)
   (let* ((y (first args))
@@ -374,8 +385,8 @@ their epilogue."
          (norm-b (when (and (getattr node :has-norm) rest) (pop rest)))
          (m (/ (buffer-storage-size x) (* (packed-weight-cols (buffer-value w))
                                           (if (eql (getattr node :prologue) :swiglu) 2 1)))))
-    (flet ((ptr (b) (if b (buffer-value b) (null-pointer))))
-      (check (%linear (buffer-value y) (packed-weight-handle (buffer-value w)) (buffer-value x) m
+    (flet ((ptr (b) (if b (device-pointer b) (null-pointer))))
+      (check (%linear (device-pointer y) (packed-weight-handle (buffer-value w)) (device-pointer x) m
                       (ptr bias) (ptr residual) (getf +acts+ (getattr node :act)) (getf +prologues+ (getattr node :prologue))
                       (ptr norm-g) (ptr norm-b) (getattr node :eps))))
     y))

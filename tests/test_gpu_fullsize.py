@@ -85,6 +85,15 @@ def test_gpt2_small_fp32_full_size_matches_oracle(oracle):
     model = llm.make_gpt2(cfg, sd)
     long_run = llm.gpt2_generate(model, prompt, 100, on_device=True)
     assert long_run[:steps] == want_tokens
+    # depth: the cache now holds 115 rows written by the device-resident loop.  One more forward, of the 100th token at
+    # position 115: its logits against the independent fp64 decoder run over the whole 116-token history.
+    import torch
+    from tests.test_oracle_decoders import torch_gpt2_logits
+    tok, late = model.forward([float(long_run[-1])], 1, len(prompt) + 99, return_logits=True)
+    with torch.no_grad():
+        ref = torch_gpt2_logits(cfg, w, list(prompt) + long_run)[-1].numpy()
+    close(late, ref)
+    assert tok == int(np.argmax(ref))
     model.close()
     model = llm.make_gpt2(cfg, sd)
     assert llm.gpt2_generate(model, prompt, 100, on_device=False) == long_run
@@ -126,6 +135,12 @@ def test_gpt2_small_q8_0_prefill_512_matches_fp64_decoder(oracle):
             want = int(torch.argmax(torch_gpt2_logits(cfg, wd, toks)[-1]))
         assert t == want
         toks.append(t)
+    # depth: the logits of the forward at position 514 (512 prompt rows from the batch, two from the decode step)
+    tok3, late = model.forward([float(toks[-1])], 1, len(toks) - 1, return_logits=True)
+    with torch.no_grad():
+        ref = torch_gpt2_logits(cfg, wd, toks)[-1].numpy()
+    close(late, ref)
+    assert tok3 == int(np.argmax(ref))
     model.close()
 
 
@@ -151,13 +166,20 @@ def test_llama_1b_q4_0_full_size(oracle):
     assert tok == int(np.argmax(ref))
     close(logits, ref)
     on_device = [tok] + model.generate_on_device(127)
+    # depth: the cache holds 255 rows, 127 of them written by the device-resident loop.  The forward of the 128th token
+    # at position 255: its logits against the independent fp64 decoder over the whole 256-token history.
+    tok_late, late = model.forward([float(on_device[-1])], 1, 255, return_logits=True)
     model.close()
     toks = list(prompt)
-    for t in on_device[:3]:
+    for t in on_device[:2]:
         with torch.no_grad():
             want = int(torch.argmax(torch_llama_logits(cfg, wd, toks)[-1]))
         assert t == want
         toks.append(t)
+    with torch.no_grad():
+        ref = torch_llama_logits(cfg, wd, list(prompt) + on_device)[-1].numpy()
+    close(late, ref)
+    assert tok_late == int(np.argmax(ref))
     del wd
     model = llm.make_llama(cfg, sd)
     assert llm.gpt2_generate(model, prompt, 128, on_device=False) == on_device

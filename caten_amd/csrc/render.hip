@@ -556,6 +556,11 @@ struct Program {
   Sx grid_global[3], grid_local[3];
   Route route;
   hipFunction_t fn = nullptr;
+  // what the matmul route derived from the shape arguments at the last launch: the layers of a model share one program
+  // and launch it with the same shapes, so the index expressions are evaluated once per set of values
+  std::vector<long long> memo_key, memo_ext;
+  bool memo_ok = false;
+  AffineN memo_aff[5];
 };
 
 static int arg_pos(const Item &it, const std::string &id) {
@@ -1691,22 +1696,31 @@ static bool launch_route(Program &pg, void **args, const std::map<std::string, l
   auto aligned = [](const float *p) { return ((uintptr_t)p % 16) == 0; };
   if (r.kind == R_MATMUL) {
     const int nl = (int)r.lidx.size(), P = nl - 1;  // loops: batch..., i, j, then k
-    std::vector<long long> ext(nl);
-    for (int q = 0; q < nl; q++)
-      if (!eval_int(r.lbound[q], env, ext[q]) || ext[q] < 0 || ext[q] > 0x7fffffff) return false;
+    const int ii = P - 2, jj = P - 1, kk = P;
+    std::vector<long long> key;
+    key.reserve(env.size());
+    for (const auto &kv : env) key.push_back(kv.second);
+    if (!pg.memo_ok || key != pg.memo_key) {
+      pg.memo_ok = false;
+      pg.memo_key = key;
+      pg.memo_ext.assign(nl, 0);
+      for (int q = 0; q < nl; q++)
+        if (!eval_int(r.lbound[q], env, pg.memo_ext[q]) || pg.memo_ext[q] < 0 || pg.memo_ext[q] > 0x7fffffff) return false;
+      if (!affine_n(r.out_idx, r.lidx, env, pg.memo_aff[0]) || !affine_n(r.a_idx, r.lidx, env, pg.memo_aff[1]) ||
+          !affine_n(r.b_idx, r.lidx, env, pg.memo_aff[2]))
+        return false;
+      // the result does not move with k, A not with j, B not with i
+      if (pg.memo_aff[0].c[kk] || pg.memo_aff[1].c[jj] || pg.memo_aff[2].c[ii]) return false;
+      for (int q = 0; q < 2; q++)
+        if (r.extra[q] >= 0 && (!affine_n(r.extra_idx[q], r.lidx, env, pg.memo_aff[3 + q]) || pg.memo_aff[3 + q].c[kk])) return false;
+      pg.memo_ok = true;
+    }
+    const std::vector<long long> &ext = pg.memo_ext;
     const long long M = ext[P - 2], N = ext[P - 1], K = ext[P];
     long long nbatch = 1;
     for (int q = 0; q < P - 2; q++) nbatch *= ext[q];
-    AffineN ao, aa, ab, ae[2];
-    if (!affine_n(r.out_idx, r.lidx, env, ao) || !affine_n(r.a_idx, r.lidx, env, aa) || !affine_n(r.b_idx, r.lidx, env, ab)) return false;
-    const int ii = P - 2, jj = P - 1, kk = P;
-    if (ao.c[kk] || aa.c[jj] || ab.c[ii]) return false;  // the result does not move with k, A not with j, B not with i
-    int nextra = 0;
-    for (int q = 0; q < 2; q++)
-      if (r.extra[q] >= 0) {
-        if (!affine_n(r.extra_idx[q], r.lidx, env, ae[q]) || ae[q].c[kk]) return false;
-        nextra++;
-      }
+    const AffineN &ao = pg.memo_aff[0], &aa = pg.memo_aff[1], &ab = pg.memo_aff[2];
+    const AffineN *ae = pg.memo_aff + 3;
     if (M == 0 || N == 0 || nbatch == 0) return true;
     if (ao.base < 0 || aa.base < 0 || ab.base < 0) return false;
     float *C = (float *)ptr(r.out) + ao.base;

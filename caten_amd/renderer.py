@@ -255,43 +255,59 @@ class HipProgram:
 
     def __init__(self, name: str, program, defglobals: List[dict], renderer: HipRenderer):
         self.name, self.program, self.defglobals, self.renderer = name, program, defglobals, renderer
+        # the argument block is built once: one ctypes cell per DEFINE-GLOBAL (a pointer or a by-value scalar of the
+        # declared dtype) and the array of their addresses cthip_program_launch takes; a call only stores values
+        self._cells = [C.c_void_p() if g["pointer_p"] else CTYPES[g["dtype"]]() for g in defglobals]
+        self._argv = (C.c_void_p * len(self._cells))(*[C.addressof(c) for c in self._cells])
+        self._pointer = [bool(g["pointer_p"]) for g in defglobals]
+        self._launch = _lib.load().cthip_program_launch
 
     @property
     def last_route(self) -> str:
         return _lib.load().cthip_program_last_route(self.program).decode()
 
     def __call__(self, node, *args):
-        lib = _lib.load()
-        if len(args) != len(self.defglobals):
+        if len(args) != len(self._cells):
             raise AssertionError(f"HIP: {self.name} takes {len(self.defglobals)} arguments, got {len(args)}")
-        boxed, cells = [], []
-        for a, g in zip(args, self.defglobals):
-            if g["pointer_p"]:
+        boxed = None
+        for k, a in enumerate(args):
+            if self._pointer[k]:
                 if isinstance(a, AbstractBuffer) and a.nrank > 0:
-                    if not isinstance(a.value, int):
-                        raise TypeError(f"HIP: please transfer the buffer {g['id']} to the device first")
-                    boxed.append(C.c_void_p(a.value))
-                elif isinstance(a, AbstractBuffer) or isinstance(a, (bool, int, float, np.number)):
+                    v = a.value
+                    if not isinstance(v, int):
+                        raise TypeError(f"HIP: please transfer the buffer {self.defglobals[k]['id']} to the device first")
+                    self._cells[k].value = v
+                elif isinstance(a, (AbstractBuffer, bool, int, float, np.number)):
                     # a rank-0 value passed by pointer: a one-element device cell holding the number
-                    v = a.value if isinstance(a, AbstractBuffer) else a
-                    host = CTYPES[g["dtype"]](v)
-                    cell = C.c_void_p()
-                    _lib.check(lib.cthip_alloc(C.byref(cell), 8))
-                    _lib.check(lib.cthip_h2d(cell, C.byref(host), C.sizeof(host)))
-                    cells.append((cell, host, a))
-                    boxed.append(C.c_void_p(cell.value))
+                    boxed = self._box(k, a, boxed)
                 else:
-                    raise TypeError(f"HIP: argument {g['id']} must be a device buffer")
+                    raise TypeError(f"HIP: argument {self.defglobals[k]['id']} must be a device buffer")
             else:
-                v = a.value if isinstance(a, AbstractBuffer) else a
-                boxed.append(CTYPES[g["dtype"]](v))
-        argv = (C.c_void_p * len(boxed))(*[C.cast(C.pointer(b), C.c_void_p) for b in boxed])
+                self._cells[k].value = a.value if isinstance(a, AbstractBuffer) else a
+        if boxed is None:
+            rc = self._launch(self.program, self._argv, len(self._cells))
+            if rc != 0:
+                _lib.check(rc)
+            return
+        lib = _lib.load()
         try:
-            _lib.check(lib.cthip_program_launch(self.program, argv, len(boxed)))
-            for cell, host, a in cells:  # write the scalars back (synchronises, as the CLANG call does)
+            _lib.check(self._launch(self.program, self._argv, len(self._cells)))
+            for cell, host, a in boxed:  # write the scalars back (synchronises, as the CLANG call does)
                 _lib.check(lib.cthip_d2h(C.byref(host), cell, C.sizeof(host)))
                 if isinstance(a, AbstractBuffer):
                     a.value = host.value
         finally:
-            for cell, _h, _a in cells:
+            for cell, _h, _a in boxed:
                 lib.cthip_free(cell)
+
+    def _box(self, k, a, boxed):
+        lib = _lib.load()
+        v = a.value if isinstance(a, AbstractBuffer) else a
+        host = CTYPES[self.defglobals[k]["dtype"]](v)
+        cell = C.c_void_p()
+        _lib.check(lib.cthip_alloc(C.byref(cell), 8))
+        _lib.check(lib.cthip_h2d(cell, C.byref(host), C.sizeof(host)))
+        self._cells[k].value = cell.value
+        boxed = boxed or []
+        boxed.append((cell, host, a))
+        return boxed

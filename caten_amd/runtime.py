@@ -83,6 +83,7 @@ class GraphRuntime:
         self.profile = os.environ.get("PROFILE", "0") == "1"
         self.times = {"kernel": 0.0, "vm": 0.0, "allocate": 0.0}
         self._casts: List[AbstractBuffer] = []  # storage opened by :View nodes that cast a scalar to an array
+        self._methods: Dict[str, Callable] = {}  # node type -> its realize-node method
 
     # runtime-setvar / runtime-getvar (runtime.lisp:66-74)
     def setvar(self, var, value):
@@ -98,21 +99,26 @@ class GraphRuntime:
     def step(self) -> bool:
         """runtime-step (runtime.lisp:106-132)"""
         node = self.graph[self.pc]
-        t1 = time.perf_counter()
+        t1 = time.perf_counter() if self.profile else 0.0
+        variables = self.variables
         try:
-            args = [a if isinstance(a, (int, float)) and not isinstance(a, bool) else self.getvar(a)
+            args = [a if type(a) is int or type(a) is float else (variables[a] if a in variables else self.getvar(a))
                     for a in node.reads]
             out = self.realize_node(node, args)
         except Exception as e:  # wrapped like handler-bind ... runtime-error
             raise RuntimeError_(self, e) from e
         if self.profile and node.type != "JIT_KERNEL":
             self.times["allocate" if node.type == "Allocate" else "vm"] += time.perf_counter() - t1
-        if not isinstance(out, tuple):
-            out = (out,)
-        if node.writes and len(out) != len(node.writes):
-            raise RuntimeError_(self, AssertionError("Runtime: the number of outputs does not match the number of writes."))
-        for place, value in zip(node.writes, out):
-            self.setvar(place, value)
+        writes = node.writes
+        if len(writes) == 1 and not isinstance(out, tuple):
+            self.setvar(writes[0], out)
+        else:
+            if not isinstance(out, tuple):
+                out = (out,)
+            if writes and len(out) != len(writes):
+                raise RuntimeError_(self, AssertionError("Runtime: the number of outputs does not match the number of writes."))
+            for place, value in zip(writes, out):
+                self.setvar(place, value)
         self.pc += 1
         return True
 
@@ -144,9 +150,12 @@ class GraphRuntime:
 
     # ---- realize-node ----
     def realize_node(self, node: Node, args):
-        fn = getattr(self, "realize_" + node.type.lower().replace("/", "_").replace("-", "_"), None)
+        fn = self._methods.get(node.type)
         if fn is None:
-            raise NotImplementedError(f"realize-node: no method for node type :{node.type} on {type(self).__name__}")
+            fn = getattr(self, "realize_" + node.type.lower().replace("/", "_").replace("-", "_"), None)
+            if fn is None:
+                raise NotImplementedError(f"realize-node: no method for node type :{node.type} on {type(self).__name__}")
+            self._methods[node.type] = fn
         return fn(node, args)
 
     def _num(self, x):

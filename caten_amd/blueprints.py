@@ -598,3 +598,47 @@ def gpt2_step_items(cfg: dict) -> dict:
         "lm_head": gpt2_linear(V, D, bias=False, name="fused_linear_lm_head"),
         "argmax": gpt2_argmax_last(V),
     }
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Items of RoPE / SwiGLU blocks (nn/positional-encoding.lisp:3-64, nn/activations.lisp:180-189).  The reference has no
+# model that uses them in a decoder (its Transformer is GPT-2 shaped), so only the element-wise items exist here;
+# both run as rendered kernels.
+def rope_rows(n_heads: int, head_dim: int, base: float = 10000.0, name: str = "fused_rope") -> dict:
+    """`(!rope x dim)` over (1, s, heads, head_dim) with the tables computed in place, as the module builds them
+    (positional-encoding.lisp:23-48): theta_i = exp(-(2i / head_dim) * log(base)) with exp(x) = exp2(x / ln 2) and
+    log(x) = log2(x) * ln 2 (api/function.lisp:432-448), cos(a) = sin(a + pi/2) (api/high-level-ops.lisp:119-122);
+    the two rotated halves are written into the even / odd elements of the output (the `!concatenate` of two
+    strided views).  Positions are 0..s-1: the module takes no start position.  Arguments: val_y, s, val_x."""
+    import math
+    half = head_dim // 2
+    i_f = _f32("_gid2")
+    log_base = _mul({"op": "LOG2", "args": [float(base)]}, 0.6931471805599453)
+    theta = {"op": "EXP2", "args": [_mul(_neg(_mul(_mul(_mul(2.0, i_f), {"op": "RECIP", "args": [float(head_dim)]}), log_base)), 1.4426950408889634)]}
+    ang = _mul(_f32("_gid0"), theta)
+    sin = {"op": "SIN", "args": [ang]}
+    cos = {"op": "SIN", "args": [_add(ang, math.pi / 2)]}
+    row = _add(_mul(n_heads * head_dim, "_gid0"), _mul(head_dim, "_gid1"))
+    e0, e1 = _add(row, _mul(2, "_gid2")), _add(row, _add(_mul(2, "_gid2"), 1))
+    x0, x1 = _A("val_x", e0), _A("val_x", e1)
+    return {"name": name, "blueprint": [
+        _glob("val_y", "output", 4), *_shape("s"), _glob("val_x", "input", 4),
+        _for("_gid0", "s"), _for("_gid1", n_heads), _for("_gid2", half),
+        _store("val_y", e0, _add(_mul(x0, cos), _neg(_mul(x1, sin)))),
+        _store("val_y", e1, _add(_mul(x0, sin), _mul(x1, cos))),
+        _end("_gid2"), _end("_gid1"), _end("_gid0"),
+    ]}
+
+
+def swiglu_rows(width: int, name: str = "fused_swiglu") -> dict:
+    """silu(gate) * up over (s, width) (SiLU, nn/activations.lisp:180-189: x * sigmoid(x), sigmoid through exp2).
+    Arguments: val_y, s, val_g, val_u."""
+    idx = _add(_mul(width, "_gid0"), "_gid1")
+    g = _A("val_g", idx)
+    sig = {"op": "RECIP", "args": [_add(1.0, {"op": "EXP2", "args": [_mul(g, -1.4426950408889634)]})]}
+    return {"name": name, "blueprint": [
+        _glob("val_y", "output", 2), *_shape("s"), _glob("val_g", "input", 2), _glob("val_u", "input", 2),
+        _for("_gid0", "s"), _for("_gid1", width),
+        _store("val_y", idx, _mul(_mul(g, sig), _A("val_u", idx))),
+        _end("_gid1"), _end("_gid0"),
+    ]}

@@ -1,4 +1,4 @@
-"""Writes tests/golden/blueprints/gpt2_*.sexp: the interchange text of every Schedule-Item of one GPT-2-small `forward`
+"""Writes tests/golden/blueprints/gpt2_*.sexp (and rope_32x64.sexp, swiglu_5632.sexp): the interchange text of every Schedule-Item of one GPT-2-small `forward`
 (caten_amd.blueprints.gpt2_step_items), exactly what the Python mirror's printer hands cthip_program_create.  The
 fixtures pin that text: tests/test_host.py fails when the printer, the blueprints or the library's reading of them drift.
 Run from the repository root:  python tests/golden/make_blueprints.py"""
@@ -18,3 +18,8 @@ if __name__ == "__main__":
         with open(os.path.join(out, f"gpt2_{key}.sexp"), "w") as f:
             f.write(item_sexp(item))
         print("wrote", key)
+    # the element-wise items of RoPE / SwiGLU blocks (Llama-1.1B shape: 32 heads of 64, FFN 5632)
+    for fname, item in (("rope_32x64", blueprints.rope_rows(32, 64)), ("swiglu_5632", blueprints.swiglu_rows(5632))):
+        with open(os.path.join(out, fname + ".sexp"), "w") as f:
+            f.write(item_sexp(item))
+        print("wrote", fname)

@@ -202,3 +202,26 @@ def test_linear_items_with_their_epilogues_vs_oracle(oracle):
             close_buffer(None, q)
     close_buffer(None, d_w)
     close_buffer(None, d_b)
+
+
+def test_rope_and_swiglu_items_vs_oracle(oracle):
+    """the element-wise items of RoPE / SwiGLU blocks as rendered kernels: `(!rope x dim)` at the reference's own bar
+    (atol 1e-5 rtol 5e-4, source/test-suite/nn/test-rope.lisp:38-66) against the oracle (pinned by the torchtune
+    formula), silu(gate) * up at 1e-6 (test-activations.lisp:153-162)"""
+    from caten_amd import blueprints as bp
+    from caten_amd.buffer import close_buffer
+    H, Dh, F = 8, 64, 1536
+    k_rope, k_glu = _run_items([bp.rope_rows(H, Dh), bp.swiglu_rows(F)])
+    rng = np.random.default_rng(12)
+    for s in (1, 10, 77):
+        x = rng.standard_normal((1, s, H, Dh)).astype(np.float32)
+        d_x, d_y = _dev(x), _dev(np.zeros_like(x))
+        k_rope(None, d_y, s, d_x)
+        assert np.allclose(_host(d_y, x.shape), oracle.rope(x, 10000.0, 0), rtol=5e-4, atol=1e-5)
+        gate, up = rng.standard_normal((s, F)).astype(np.float32) * 3, rng.standard_normal((s, F)).astype(np.float32)
+        d_g, d_u, d_o = _dev(gate), _dev(up), _dev(np.zeros_like(up))
+        k_glu(None, d_o, s, d_g, d_u)
+        assert np.allclose(_host(d_o, up.shape), oracle.silu(gate) * up, rtol=1e-6, atol=1e-6)
+        assert k_rope.last_route == "rendered" and k_glu.last_route == "rendered"
+        for b in (d_x, d_y, d_g, d_u, d_o):
+            close_buffer(None, b)

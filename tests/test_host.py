@@ -428,6 +428,19 @@ def test_gpt2_step_items_print_as_their_golden_text_and_route():
         assert 'extern "C" __global__' in src
 
 
+def test_rope_and_swiglu_items_print_as_their_golden_text():
+    """RoPE with its tables computed in place (nn/positional-encoding.lisp:23-48) and silu(gate) * up
+    (nn/activations.lisp:180-189): element-wise items, rendered"""
+    from caten_amd import blueprints as bp
+    from caten_amd.renderer import item_sexp
+    for fname, item in (("rope_32x64", bp.rope_rows(32, 64)), ("swiglu_5632", bp.swiglu_rows(5632))):
+        with open(os.path.join(GOLDEN_BP, fname + ".sexp")) as f:
+            golden = f.read()
+        assert item_sexp(item) == golden, fname
+        route, src = _create(golden.encode())
+        assert route == "rendered" and 'extern "C" __global__' in src
+
+
 def test_blueprints_in_a_lisp_printers_spelling_are_read_the_same():
     """upper-case symbols, exponent markers (0.0f0, 1.0e-5, ...d0), single-float folded constants (1/768 =
     0.0013020834, 3e-8 off), commutative operands in another order; and the one rendered matmul the reference's own

@@ -26,6 +26,7 @@ struct State {
   int decoder_graph = 1;  // option "decoder_graph": 0 = the step's launches are issued one by one (kernel tracing)
   int prefill_gemm = 1;   // option "prefill_gemm": 0 = prompts are fed row by row through the decode step
   int decode_fused = 1;   // option "decode_fused": 0 = five launches per layer instead of three
+  int decode_flow = 0;    // option "decode_flow": 1 = GPT-2 / Q8_0 sessions run all layers of a step as one launch (decode_flow.hip)
   int render_routes = 1;  // option "render_routes": 0 = every program runs its rendered kernel, none a hand-written one
   // option "decode_skip": launches of the three-launch decode step that are left out, for knock-out timing (bits: 1 qkv,
   // 2 attention + projection, 4 MLP, 8 the sum in front of lm_head, 16 lm_head + argmax); tokens are meaningless then

@@ -71,6 +71,60 @@ struct DecMlpArgs {
   long long *accum;          // [kDecXcds][D]
 };
 
+#ifdef CTHIP_DECODE_DEVICE_HELPERS
+// Weight formats of the fused launches: a 16-byte chunk holds XPC weights (Q8_0: 16 int8, fp16: 8, fp32: 4); only
+// Q8_0 has a scale plane (one fp16 per 32 weights).
+template <int TYPE>
+struct DecFmt {
+  static constexpr int XPC = Fmt<TYPE>::XPC;
+  static constexpr bool QUANT = TYPE == CTHIP_Q8_0;
+};
+
+// XPC consecutive floats of a vector in LDS
+template <int XPC>
+__device__ __forceinline__ void lds_floats(const float *p, float *xr) {
+#pragma unroll
+  for (int t = 0; t < XPC / 4; t++) {
+    const float4 v = *(const float4 *)(p + 4 * t);
+    xr[4 * t + 0] = v.x;
+    xr[4 * t + 1] = v.y;
+    xr[4 * t + 2] = v.z;
+    xr[4 * t + 3] = v.w;
+  }
+}
+
+// One row of D = 256 * KC weights against the staged vector: 16 lanes per row, lane l owns chunks l + 16 j.  Two
+// running sums: a chain of dependent FMAs issues at half rate when the SIMD holds one wavefront.
+template <int TYPE, int KC>
+__device__ __forceinline__ float dec_row_dot(const uint4 *w, const unsigned *sc, const float *xs, int l) {
+  constexpr int XPC = DecFmt<TYPE>::XPC, NCL = KC * 16 / XPC;
+  float acc[2] = {0.0f, 0.0f};
+#pragma unroll
+  for (int j = 0; j < NCL; j++) {
+    const int c = l + 16 * j;
+    float xr[XPC];
+    lds_floats<XPC>(xs + c * XPC, xr);
+    acc[j & 1] += chunk_dot<TYPE>(w[j], DecFmt<TYPE>::QUANT ? half_bits_to_float((unsigned short)sc[j]) : 1.0f, xr, 0.0f);
+  }
+  return row16_sum(acc[0] + acc[1]);
+}
+
+// requests of one row's chunks (and block scales) for dec_row_dot
+template <int TYPE, int KC>
+__device__ __forceinline__ void dec_row_request(const void *wq, const unsigned short *wd, int64_t row, int l, uint4 *w, unsigned *sc) {
+  constexpr int XPC = DecFmt<TYPE>::XPC, NCL = KC * 16 / XPC;
+  const uint4 *qp = (const uint4 *)wq + row * (16 * NCL);
+#pragma unroll
+  for (int j = 0; j < NCL; j++) {
+    const int c = l + 16 * j;
+    w[j] = qp[c];
+    if (DecFmt<TYPE>::QUANT) sc[j] = wd[row * (8 * KC) + ((c * XPC) >> 5)];
+    else sc[j] = 0;
+  }
+}
+
+#endif  // CTHIP_DECODE_DEVICE_HELPERS
+
 bool dec_fused_supported(int type_attn, int type_proj, int type_fc, int type_fc2, int D, int H, int F);
 int dec_xcd_probe(int *max_id);
 int dec_relay_heads(const WMat *w, int DH, void **pq, void **pd);
@@ -79,6 +133,51 @@ int launch_dec_qkv(const DecQkvArgs &a, int type, bool from_accum);
 int launch_dec_attn_proj(const DecAttnArgs &a, int type, int H, int D, int replicas);
 int launch_dec_mlp(const DecMlpArgs &a, int type, int F, int H);
 int launch_dec_sum(const DecStage &s, float *out);
+
+}  // namespace cthip
+
+// ---- all layers of a step as one launch of role-specialised workgroups (decode_flow.hip) ----
+namespace cthip {
+
+struct FlowLayer {
+  const void *attn_q;             // c_attn quant plane int8 [3D][D]
+  const unsigned short *attn_d;   // ... scale plane fp16 [3D][D/32]
+  const float *attn_s, *attn_c;   // LayerNorm1 folded through c_attn: W.gamma, W.beta + bias
+  const void *proj_q;             // attn.c_proj int8 [D][D]
+  const unsigned short *proj_d;   // fp16 [D][D/32]
+  const float *proj_b;
+  const void *fc_q;               // c_fc int8 [F][D]
+  const unsigned short *fc_d;     // fp16 [F][D/32]
+  const float *fc_s, *fc_c;       // LayerNorm2 folded through c_fc
+  const void *fc2_sq;             // mlp.c_proj by 32-column slab: int8 [F/32][D][32]
+  const unsigned short *fc2_sd;   // fp16 [F/32][D]
+  const float *fc2_b;
+  const float *ln1_g, *ln2_g;
+  float *kc, *vc;                 // K / V cache (max_seq, D)
+};
+
+struct FlowArgs {
+  const FlowLayer *layers;        // device array, n_layers entries
+  int n_layers, D, H, F, NM;      // NM = F / 32
+  float eps;
+  // tagged elements (value in the low, tag in the high 32 bits), one buffer per (layer, phase)
+  // (X, O and XP are broadcast to many workgroups and kept in several copies: [copies][n_layers][D])
+  unsigned long long *X;          // [n_layers][D]       a layer's input (layer 0 reads x0 instead)
+  unsigned long long *QKV;        // [n_layers][3D]
+  unsigned long long *O;          // [n_layers][D]       the heads' attention outputs
+  unsigned long long *XP;         // [n_layers][D]       x' = x + attention
+  unsigned long long *PM;         // [n_layers][NM][D]   the MLP workgroups' shares of mlp.c_proj
+  const float *x0;                // the step's input row (fp32, written by an earlier launch)
+  float *x_out;                   // the residual vector after the last layer, for lm_head
+  const int *tokpos;              // [1] = position
+  int *state;                     // [0] = epoch of the next step's tags, [1] = a waiter gave up
+  long long *trace;               // null, or [workgroups][n_layers][4] clock stamps of the last step (option decode_flow 2)
+};
+
+bool dec_flow_supported(int type_attn, int type_proj, int type_fc, int type_fc2, int D, int H, int F, int n_layers);
+int dec_flow_grid(int D, int H, int F);
+void dec_flow_copies(int *x, int *o, int *xp);  // copies kept of the buffers X, O, XP
+int launch_dec_flow(const FlowArgs &a);
 
 }  // namespace cthip
 

@@ -25,6 +25,7 @@
 
 #include "common.h"
 #include "gemv_kernels.h"
+#define CTHIP_DECODE_DEVICE_HELPERS
 #include "decode_fused.h"
 
 namespace cthip {
@@ -128,57 +129,6 @@ __device__ __forceinline__ void dec_stage_finish(const DecStage &s, DecStageRegs
     m2 += red[16 + w] + red[w] * dw * dw;
   }
   rstd = 1.0f / sqrtf(fmaxf(m2 * inv_n, 0.0f) + s.eps);
-}
-
-// Weight formats of the fused launches: a 16-byte chunk holds XPC weights (Q8_0: 16 int8, fp16: 8, fp32: 4); only
-// Q8_0 has a scale plane (one fp16 per 32 weights).
-template <int TYPE>
-struct DecFmt {
-  static constexpr int XPC = Fmt<TYPE>::XPC;
-  static constexpr bool QUANT = TYPE == CTHIP_Q8_0;
-};
-
-// XPC consecutive floats of a vector in LDS
-template <int XPC>
-__device__ __forceinline__ void lds_floats(const float *p, float *xr) {
-#pragma unroll
-  for (int t = 0; t < XPC / 4; t++) {
-    const float4 v = *(const float4 *)(p + 4 * t);
-    xr[4 * t + 0] = v.x;
-    xr[4 * t + 1] = v.y;
-    xr[4 * t + 2] = v.z;
-    xr[4 * t + 3] = v.w;
-  }
-}
-
-// One row of D = 256 * KC weights against the staged vector: 16 lanes per row, lane l owns chunks l + 16 j.  Two
-// running sums: a chain of dependent FMAs issues at half rate when the SIMD holds one wavefront.
-template <int TYPE, int KC>
-__device__ __forceinline__ float dec_row_dot(const uint4 *w, const unsigned *sc, const float *xs, int l) {
-  constexpr int XPC = DecFmt<TYPE>::XPC, NCL = KC * 16 / XPC;
-  float acc[2] = {0.0f, 0.0f};
-#pragma unroll
-  for (int j = 0; j < NCL; j++) {
-    const int c = l + 16 * j;
-    float xr[XPC];
-    lds_floats<XPC>(xs + c * XPC, xr);
-    acc[j & 1] += chunk_dot<TYPE>(w[j], DecFmt<TYPE>::QUANT ? half_bits_to_float((unsigned short)sc[j]) : 1.0f, xr, 0.0f);
-  }
-  return row16_sum(acc[0] + acc[1]);
-}
-
-// requests of one row's chunks (and block scales) for dec_row_dot
-template <int TYPE, int KC>
-__device__ __forceinline__ void dec_row_request(const void *wq, const unsigned short *wd, int64_t row, int l, uint4 *w, unsigned *sc) {
-  constexpr int XPC = DecFmt<TYPE>::XPC, NCL = KC * 16 / XPC;
-  const uint4 *qp = (const uint4 *)wq + row * (16 * NCL);
-#pragma unroll
-  for (int j = 0; j < NCL; j++) {
-    const int c = l + 16 * j;
-    w[j] = qp[c];
-    if (DecFmt<TYPE>::QUANT) sc[j] = wd[row * (8 * KC) + ((c * XPC) >> 5)];
-    else sc[j] = 0;
-  }
 }
 
 // ---- launch 1: LayerNorm1 folded through c_attn; 16 rows per workgroup ----

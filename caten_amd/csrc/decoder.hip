@@ -98,6 +98,9 @@ struct Decoder {
   bool fused = false;
   float *x2 = nullptr, *patt = nullptr;
   long long *pmlp = nullptr;
+  // all layers of a step as one launch (decode_flow.hip): the tagged hand-over buffers and the launch's arguments
+  bool flow = false;
+  FlowArgs flow_args = {};
   // grouped-query layers (decode_gqa.hip): the attention projection has an accumulator set of its own
   bool fused_gqa = false;
   long long *pattn = nullptr;
@@ -348,7 +351,73 @@ static int finalize(Decoder *d) {
     for (WMat *w : ws)
       if (w) w->stream = total > kInfinityCacheBytes / 4 * 3;
   }
-  if (c.arch == CTHIP_ARCH_GPT2 && state().decode_fused && !d->kvq &&
+  if (c.arch == CTHIP_ARCH_GPT2 && state().decode_flow && !d->kvq) {
+    bool ok = true;
+    for (int l = 0; l < c.n_layers && ok; l++) {
+      Layer &L = d->layers[l];
+      ok = dec_flow_supported(L.attn->type, L.proj->type, L.fc->type, L.fc2->type, D, c.n_heads, F, c.n_layers);
+    }
+    if (ok) {
+      const int H = c.n_heads, NM = F / 32, NL = c.n_layers;
+      std::vector<FlowLayer> fl(NL);
+      for (int l = 0; l < NL; l++) {
+        Layer &L = d->layers[l];
+        TRY(dec_relay_heads(L.fc2, 32, &L.fc2_sq, &L.fc2_sd));  // 32-column slabs: one per MLP workgroup
+        d->owned.insert(d->owned.end(), {L.fc2_sq, L.fc2_sd});
+        FlowLayer &f = fl[l];
+        f.attn_q = L.attn->q;
+        f.attn_d = (const unsigned short *)L.attn->d;
+        f.attn_s = L.attn_s;
+        f.attn_c = L.attn_c;
+        f.proj_q = L.proj->q;
+        f.proj_d = (const unsigned short *)L.proj->d;
+        f.proj_b = L.proj_b;
+        f.fc_q = L.fc->q;
+        f.fc_d = (const unsigned short *)L.fc->d;
+        f.fc_s = L.fc_s;
+        f.fc_c = L.fc_c;
+        f.fc2_sq = L.fc2_sq;
+        f.fc2_sd = (const unsigned short *)L.fc2_sd;
+        f.fc2_b = L.fc2_b;
+        f.ln1_g = L.ln1_g;
+        f.ln2_g = L.ln2_g;
+        f.kc = L.k_cache;
+        f.vc = L.v_cache;
+      }
+      FlowArgs &fa = d->flow_args;
+      FlowLayer *dl = nullptr;
+      TRY(dev_alloc(d, (void **)&dl, sizeof(FlowLayer) * NL));
+      TRY(cthip_h2d(dl, fl.data(), sizeof(FlowLayer) * NL));
+      fa.layers = dl;
+      fa.n_layers = NL;
+      fa.D = D;
+      fa.H = H;
+      fa.F = F;
+      fa.NM = NM;
+      fa.eps = c.eps;
+      // zero-filled: no element carries a tag of any step (epochs start at 1)
+      int cx, co, cxp;
+      dec_flow_copies(&cx, &co, &cxp);
+      const size_t per_layer = (size_t)D * (cx + 3 + co + cxp + NM);
+      unsigned long long *ll = nullptr;
+      TRY(dev_alloc(d, (void **)&ll, 8 * per_layer * NL));
+      fa.X = ll;
+      fa.QKV = fa.X + (size_t)cx * NL * D;
+      fa.O = fa.QKV + (size_t)NL * 3 * D;
+      fa.XP = fa.O + (size_t)co * NL * D;
+      fa.PM = fa.XP + (size_t)cxp * NL * D;
+      fa.x0 = d->x;
+      fa.x_out = d->x;
+      fa.tokpos = d->tokpos;
+      TRY(dev_alloc(d, (void **)&fa.state, 256));
+      if (state().decode_flow == 2)
+        TRY(dev_alloc(d, (void **)&fa.trace, sizeof(long long) * 4 * (size_t)NL * dec_flow_grid(D, H, F)));
+      const int st0[2] = {1, 0};
+      TRY(cthip_h2d(fa.state, st0, sizeof(st0)));
+      d->flow = true;
+    }
+  }
+  if (c.arch == CTHIP_ARCH_GPT2 && state().decode_fused && !d->kvq && !d->flow &&
       dec_fused_supported(d->layers[0].attn->type, d->layers[0].proj->type, d->layers[0].fc->type,
                           d->layers[0].fc2->type, D, c.n_heads, F)) {
     // the per-XCD accumulators assume what gfx950 has: XCD ids 0..7
@@ -439,6 +508,11 @@ static int queue_step(Decoder *d, bool with_head, bool embed) {
   const bool gpt2 = c.arch == CTHIP_ARCH_GPT2;
   // embed = false: the previous step's head has already gathered this step's input (queue_head)
   if (embed) TRY(launch_embedding(d->x, d->wte, nullptr, tok, 1, V, D, gpt2 ? d->wpe : nullptr, pos, c.max_seq));
+  if (d->flow) {
+    TRY(launch_dec_flow(d->flow_args));
+    if (with_head) TRY(queue_head(d));
+    return 0;
+  }
   if (d->fused) {
     // Three launches per layer.  The residual stream alternates between d->x and d->x2 as "base + bias +
     // partials": each launch adds up what its predecessor left and block 0 stores the sum for the launch after.
@@ -810,6 +884,20 @@ done:
   return rc;
 }
 
+// After a synchronising copy: did a workgroup of the one-launch step give up waiting?  The step's results are void
+// then; the epoch moves on so that no tag of the failed step can match later.
+static int flow_check(Decoder *d) {
+  if (!d->flow) return 0;
+  int st[2] = {0, 0};
+  int rc = cthip_d2h(st, d->flow_args.state, sizeof(st));
+  if (rc || !st[1]) return rc;
+  const int next[2] = {st[0] + 2, 0};
+  if ((rc = cthip_h2d(d->flow_args.state, next, sizeof(next)))) return rc;
+  return fail(CTHIP_E_STATE, "decoder: a workgroup of the one-launch decode step waited for its input beyond the poll limit; "
+                             "the step's results are void (are all %d workgroups resident at once?)",
+              dec_flow_grid(d->cfg.dim, d->cfg.n_heads, d->cfg.ffn));
+}
+
 static int run_step(Decoder *d, bool with_head) {
   if (d->use_graph) {
     CTHIP_CHECK(hipGraphLaunch(with_head ? d->g_step : d->g_body, state().stream));
@@ -942,6 +1030,7 @@ int cthip_decoder_forward(void *dec, const float *tokens, int s, int n, int64_t 
   }
   if (logits_out && (rc = cthip_d2h(logits_out, d->logits, sizeof(float) * (size_t)c.vocab))) return rc;
   if ((rc = cthip_d2h(token, d->token64, sizeof(int64_t)))) return rc;
+  if ((rc = flow_check(d))) return rc;
   d->position = n + s;
   d->primed = true;
   return 0;
@@ -983,6 +1072,7 @@ static int generate_impl(Decoder *d, int steps, int eos, int64_t *tokens_out, in
     if ((rc = run_step(d, true))) return rc;
   int n = 0;
   if ((rc = cthip_d2h(&n, d->hist_n, sizeof(int)))) return rc;  // synchronises
+  if ((rc = flow_check(d))) return rc;
   if (n < 0 || n > steps) return fail(CTHIP_E_STATE, "cthip_decoder_generate: the device reports %d tokens for %d steps", n, steps);
   if (n && (rc = cthip_d2h(tokens_out, d->history, sizeof(int64_t) * (size_t)n))) return rc;
   d->position += n;
@@ -1013,6 +1103,7 @@ int cthip_decoder_layer_launches(void *dec) {
   Decoder *d = (Decoder *)dec;
   int rc = finalize(d);
   if (rc) return -1;
+  if (d->flow) return 1;  // all layers are ONE launch
   if (d->fused || d->fused_gqa) return 3;
   if (d->kvq) return d->cfg.arch == CTHIP_ARCH_GPT2 ? 7 : 9;  // + two appends (+ two rotations) around the attention launch
   return 5;
@@ -1046,6 +1137,10 @@ int cthip_decoder_peek(void *dec, const char *what, void **ptr, int64_t *n_float
   } else if (!strcmp(what, "x")) {
     p = d->x;
     n = c.dim;
+  } else if (!strcmp(what, "flow_trace") && d->flow && d->flow_args.trace) {
+    // int64 clock stamps [workgroups][n_layers][4]; n counts their bytes in units of four
+    p = d->flow_args.trace;
+    n = (int64_t)dec_flow_grid(c.dim, c.n_heads, c.ffn) * c.n_layers * 4 * 2;
   } else if ((sscanf(what, "k_cache.%d", &l) == 1 || sscanf(what, "v_cache.%d", &l) == 1) && l >= 0 && l < c.n_layers) {
     const bool key = what[0] == 'k';
     n = (int64_t)c.max_seq * kv_dim(c);

@@ -673,6 +673,11 @@ int cthip_set_option(const char *name, int value) {
     else state().decode_fused = value;
     return 0;
   }
+  if (!strcmp(name, "decode_flow")) {
+    if (value < 0 || value > 2) return fail(CTHIP_E_BAD_ARG, "cthip_set_option: decode_flow is 0, 1 or 2 (1 with a timeline of the last step)");
+    state().decode_flow = value;
+    return 0;
+  }
   if (!strcmp(name, "kv_cache")) {
     if (value != 0 && value != 1) return fail(CTHIP_E_BAD_ARG, "cthip_set_option: kv_cache is 0 (fp32 rows) or 1 (Q8_0 rows)");
     state().kv_cache = value;

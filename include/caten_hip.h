@@ -216,7 +216,14 @@ int cthip_linear(float *y, const void *wmat, const float *x, int m, const float 
  *   cache's on the tested models (the band of 8-bit keys and values, not of the fp32 arithmetic around them).
  * "decode_skip": knock-out timing of the three-launch decode step -- a mask of launches a session created
  *   afterwards leaves out (1 qkv, 2 attention + projection, 4 MLP, 8 the sum in front of lm_head,
- *   16 lm_head + argmax).  Tokens and logits of such a session are meaningless; 0 (default) = none. */
+ *   16 lm_head + argmax).  Tokens and logits of such a session are meaningless; 0 (default) = none.
+ * "decode_flow": 1 = GPT-2 shaped Q8_0 sessions (d 256 / 4 heads or d 768 / 12 heads, fp32 cache) created
+ *   afterwards run all layers of a decode step as ONE launch of role-specialised workgroups that hand their
+ *   results over through tagged device memory (csrc/decode_flow.hip) -- an experiment kept for its measurements:
+ *   same tokens, logits inside the fp32 band, and SLOWER than the three launches per layer it replaces.
+ *   2 = the same, and every workgroup keeps clock stamps of its last step (cthip_decoder_peek "flow_trace").
+ *   It needs every one of its workgroups resident at once; a step whose bounded waits run out fails with
+ *   CTHIP_E_STATE instead of hanging.  0 (default) = off. */
 int cthip_set_option(const char *name, int value);
 
 /* !relu(!matmul A B) (api/high-level-ops.lisp:76-99; fused per test-scheduler.lisp:140-163):

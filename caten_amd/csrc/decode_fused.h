@@ -72,13 +72,27 @@ struct DecMlpArgs {
 };
 
 #ifdef CTHIP_DECODE_DEVICE_HELPERS
-// Weight formats of the fused launches: a 16-byte chunk holds XPC weights (Q8_0: 16 int8, fp16: 8, fp32: 4); only
-// Q8_0 has a scale plane (one fp16 per 32 weights).
+// Weight formats of the fused launches: a 16-byte chunk holds XPC weights (Q8_0: 16 int8, Q4_0: 32 nibbles = one
+// block, fp16: 8, fp32: 4); the quantised formats have a scale plane (one fp16 per 32 weights).  LPR lanes share a
+// row: 16, or 8 where a chunk is a whole block of 32 (a row of D = 256 KC columns is then 8 KC chunks).  Rows whose
+// chunks are 128 bytes of the staged vector apart are read from LDS with the 16-byte slot index xor-ed by the
+// block index (SWZ), or every lane of a row group would hit the same banks.
 template <int TYPE>
 struct DecFmt {
   static constexpr int XPC = Fmt<TYPE>::XPC;
-  static constexpr bool QUANT = TYPE == CTHIP_Q8_0;
+  static constexpr bool QUANT = TYPE == CTHIP_Q8_0 || TYPE == CTHIP_Q4_0;
+  static constexpr int LPR = XPC >= 32 ? 8 : 16;
+  static constexpr bool SWZ = XPC >= 32;
+  static constexpr int RPW = 64 / LPR;  // rows per wavefront
 };
+
+// float4 slot of the i4-th float4 of a staged vector
+template <bool SWZ>
+__device__ __forceinline__ int dec_slot(int i4) {
+  if (!SWZ) return i4;
+  const int blk = i4 >> 3;
+  return (blk << 3) | ((i4 ^ blk) & 7);
+}
 
 // XPC consecutive floats of a vector in LDS
 template <int XPC>
@@ -93,30 +107,62 @@ __device__ __forceinline__ void lds_floats(const float *p, float *xr) {
   }
 }
 
-// One row of D = 256 * KC weights against the staged vector: 16 lanes per row, lane l owns chunks l + 16 j.  Two
+// chunk c of a staged vector (swizzled where the format says so); returns the sum of its floats where the format
+// needs it (Q4_0 stores n + 8), else 0
+template <int TYPE>
+__device__ __forceinline__ float dec_chunk_floats(const float *xs, int c, float *xr) {
+  constexpr int XPC = DecFmt<TYPE>::XPC;
+  if (!DecFmt<TYPE>::SWZ) {
+    lds_floats<XPC>(xs + c * XPC, xr);
+    return 0.0f;
+  }
+  float part[8];
+#pragma unroll
+  for (int k = 0; k < 8; k++) {
+    const float4 v = ((const float4 *)xs)[(c << 3) | ((k ^ c) & 7)];
+    xr[4 * k + 0] = v.x;
+    xr[4 * k + 1] = v.y;
+    xr[4 * k + 2] = v.z;
+    xr[4 * k + 3] = v.w;
+    part[k] = (v.x + v.y) + (v.z + v.w);
+  }
+  return ((part[0] + part[1]) + (part[2] + part[3])) + ((part[4] + part[5]) + (part[6] + part[7]));
+}
+
+// sum over the LPR lanes of a row
+template <int LPR>
+__device__ __forceinline__ float dec_row_sum(float v) {
+  v += dpp_f<0xB1>(v);   // quad_perm [1,0,3,2]
+  v += dpp_f<0x4E>(v);   // quad_perm [2,3,0,1]
+  v += dpp_f<0x141>(v);  // row_half_mirror
+  if (LPR == 16) v += dpp_f<0x140>(v);  // row_mirror
+  return v;
+}
+
+// One row of D = 256 * KC weights against the staged vector: LPR lanes per row, lane l owns chunks l + LPR j.  Two
 // running sums: a chain of dependent FMAs issues at half rate when the SIMD holds one wavefront.
 template <int TYPE, int KC>
 __device__ __forceinline__ float dec_row_dot(const uint4 *w, const unsigned *sc, const float *xs, int l) {
-  constexpr int XPC = DecFmt<TYPE>::XPC, NCL = KC * 16 / XPC;
+  constexpr int XPC = DecFmt<TYPE>::XPC, LPR = DecFmt<TYPE>::LPR, NCL = KC * 256 / XPC / LPR;
   float acc[2] = {0.0f, 0.0f};
 #pragma unroll
   for (int j = 0; j < NCL; j++) {
-    const int c = l + 16 * j;
+    const int c = l + LPR * j;
     float xr[XPC];
-    lds_floats<XPC>(xs + c * XPC, xr);
-    acc[j & 1] += chunk_dot<TYPE>(w[j], DecFmt<TYPE>::QUANT ? half_bits_to_float((unsigned short)sc[j]) : 1.0f, xr, 0.0f);
+    const float xsum = dec_chunk_floats<TYPE>(xs, c, xr);
+    acc[j & 1] += chunk_dot<TYPE>(w[j], DecFmt<TYPE>::QUANT ? half_bits_to_float((unsigned short)sc[j]) : 1.0f, xr, xsum);
   }
-  return row16_sum(acc[0] + acc[1]);
+  return dec_row_sum<LPR>(acc[0] + acc[1]);
 }
 
 // requests of one row's chunks (and block scales) for dec_row_dot
 template <int TYPE, int KC>
 __device__ __forceinline__ void dec_row_request(const void *wq, const unsigned short *wd, int64_t row, int l, uint4 *w, unsigned *sc) {
-  constexpr int XPC = DecFmt<TYPE>::XPC, NCL = KC * 16 / XPC;
-  const uint4 *qp = (const uint4 *)wq + row * (16 * NCL);
+  constexpr int XPC = DecFmt<TYPE>::XPC, LPR = DecFmt<TYPE>::LPR, NCL = KC * 256 / XPC / LPR;
+  const uint4 *qp = (const uint4 *)wq + row * (LPR * NCL);
 #pragma unroll
   for (int j = 0; j < NCL; j++) {
-    const int c = l + 16 * j;
+    const int c = l + LPR * j;
     w[j] = qp[c];
     if (DecFmt<TYPE>::QUANT) sc[j] = wd[row * (8 * KC) + ((c * XPC) >> 5)];
     else sc[j] = 0;
@@ -128,7 +174,7 @@ __device__ __forceinline__ void dec_row_request(const void *wq, const unsigned s
 bool dec_fused_supported(int type_attn, int type_proj, int type_fc, int type_fc2, int D, int H, int F);
 int dec_xcd_probe(int *max_id);
 int dec_relay_heads(const WMat *w, int DH, void **pq, void **pd);
-int dec_relay_slabs(const WMat *w, void **pq, void **pd);
+int dec_relay_slabs(const WMat *w, void **pq, void **pd);  // slabs of 16 columns (a whole block of 32 for Q4_0)
 int launch_dec_qkv(const DecQkvArgs &a, int type, bool from_accum);
 int launch_dec_attn_proj(const DecAttnArgs &a, int type, int H, int D, int replicas);
 int launch_dec_mlp(const DecMlpArgs &a, int type, int F, int H);

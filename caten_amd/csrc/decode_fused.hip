@@ -1,12 +1,13 @@
 // Three launches per layer for one decode row of a GPT-2 shaped Transformer (external/llm/layers.lisp:35-71)
-// with Q8_0, fp32 or fp16 weights (template argument TYPE), instead of five.  A decode step is bound by the number of DEPENDENT launches, not by
+// with Q8_0, Q4_0, fp32 or fp16 weights (template argument TYPE), instead of five.  A decode step is bound by the number of DEPENDENT launches, not by
 // bytes, so two pairs of consecutive Linears are merged around the vector that sits between them:
 //
 //   k_dec_qkv        x -> LayerNorm1 -> c_attn (+bias): q to a buffer, k / v rows into the cache at `pos`
 //   k_dec_attn_proj  four workgroups per head: attention over cache rows 0..pos, then a quarter of the rows of
 //                    that head's 64 columns of attn.c_proj applied to its 64 outputs -> one partial vector per head
-//   k_dec_mlp        one workgroup per 16 hidden units: LayerNorm2 -> those rows of c_fc (+bias, GELU) ->
-//                    their 16 columns of mlp.c_proj -> partial vector, added into one accumulator per XCD
+//   k_dec_mlp        one workgroup per 16 hidden units (32 with Q4_0 weights, whose blocks are 32 wide): LayerNorm2
+//                    -> those rows of c_fc (+bias, GELU) -> their columns of mlp.c_proj -> partial vector, added
+//                    into one accumulator per XCD
 //
 // A Linear whose INPUT is split over workgroups produces one partial output vector per workgroup; the
 // consumer of the vector adds the partials while it stages its input, so the residual stream travels as
@@ -71,7 +72,7 @@ __device__ __forceinline__ void dec_stage_request(const DecStage &s, DecStageReg
 
 // Adds the answers up, writes gamma * x to LDS and returns the LayerNorm statistics of x; block 0 also stores x to
 // s.xout.  red holds 24 floats.  blockDim.x == 256.
-template <int MODE, int NP>
+template <bool SWZ, int MODE, int NP>
 __device__ __forceinline__ void dec_stage_finish(const DecStage &s, DecStageRegs<MODE, NP> &r, float *xs, float *red,
                                                  float &mu, float &rstd) {
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
@@ -108,7 +109,7 @@ __device__ __forceinline__ void dec_stage_finish(const DecStage &s, DecStageRegs
   const float dm = mean_t - mean_w;
   const float m2_w = wave_sum(m2_t + cnt * dm * dm);
   if (active) {
-    ((float4 *)xs)[i] = make_float4(v.x * g.x, v.y * g.y, v.z * g.z, v.w * g.w);
+    ((float4 *)xs)[dec_slot<SWZ>(i)] = make_float4(v.x * g.x, v.y * g.y, v.z * g.z, v.w * g.w);
     if (blockIdx.x == 0 && s.xout) ((float4 *)s.xout)[i] = v;
   }
   if (lane == 0) {
@@ -131,29 +132,30 @@ __device__ __forceinline__ void dec_stage_finish(const DecStage &s, DecStageRegs
   rstd = 1.0f / sqrtf(fmaxf(m2 * inv_n, 0.0f) + s.eps);
 }
 
-// ---- launch 1: LayerNorm1 folded through c_attn; 16 rows per workgroup ----
+// ---- launch 1: LayerNorm1 folded through c_attn; 16 rows per workgroup (32 with 8 lanes a row) ----
 template <int TYPE, int KC, int MODE, int NP>
 __global__ __launch_bounds__(256) void k_dec_qkv(DecQkvArgs a) {
+  typedef DecFmt<TYPE> F;
   __shared__ __align__(16) float xs[256 * KC];
   __shared__ float red[24];
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
-  const int g = lane >> 4, l = lane & 15;
+  const int g = lane / F::LPR, l = lane % F::LPR;
   const int D = a.st.D;
-  int row = blockIdx.x * 16 + wv * 4 + g;
+  int row = blockIdx.x * (4 * F::RPW) + wv * F::RPW + g;
   const bool row_ok = row < a.rows;
   row = row_ok ? row : a.rows - 1;
   DecStageRegs<MODE, NP> sr;
   dec_stage_request(a.st, sr);
   const int posv = a.pos[0];
   __builtin_amdgcn_sched_barrier(0);
-  constexpr int NCL = KC * 16 / DecFmt<TYPE>::XPC;
+  constexpr int NCL = KC * 256 / F::XPC / F::LPR;
   uint4 w[NCL];
   unsigned sc[NCL];
   dec_row_request<TYPE, KC>(a.wq, a.wd, row, l, w, sc);
   const float fs = a.fold_s[row], fc = a.fold_c[row];
   __builtin_amdgcn_sched_barrier(0);
   float mu, rstd;
-  dec_stage_finish(a.st, sr, xs, red, mu, rstd);
+  dec_stage_finish<F::SWZ>(a.st, sr, xs, red, mu, rstd);
   const float acc = dec_row_dot<TYPE, KC>(w, sc, xs, l);
   if (l == 0 && row_ok) {
     // rstd * (W.(gamma x) - mu * W.gamma) + (W.beta + bias)  =  W.LayerNorm(x) + bias
@@ -297,9 +299,14 @@ void k_dec_attn_proj(DecAttnArgs a) {
   // partial projection: row r of the slab times the head's outputs; CPR lanes share a row
   float xr[XPC];
   lds_floats<XPC>(oh + pc * XPC, xr);
+  float xsum = 0.0f;
+  if (TYPE == CTHIP_Q4_0) {
+#pragma unroll
+    for (int t = 0; t < XPC; t++) xsum += xr[t];
+  }
 #pragma unroll
   for (int j = 0; j < JR; j++) {
-    float s = chunk_dot<TYPE>(pw[j], DecFmt<TYPE>::QUANT ? half_bits_to_float((unsigned short)ps[j]) : 1.0f, xr, 0.0f);
+    float s = chunk_dot<TYPE>(pw[j], DecFmt<TYPE>::QUANT ? half_bits_to_float((unsigned short)ps[j]) : 1.0f, xr, xsum);
     if (CPR >= 2) s += dpp_f<0xB1>(s);    // quad_perm [1,0,3,2]
     if (CPR >= 4) s += dpp_f<0x4E>(s);    // quad_perm [2,3,0,1]
     if (CPR >= 8) s += dpp_f<0x141>(s);   // row_half_mirror
@@ -309,26 +316,29 @@ void k_dec_attn_proj(DecAttnArgs a) {
   }
 }
 
-// ---- launch 3: LayerNorm2 folded through 16 rows of c_fc, GELU, their 16 columns of mlp.c_proj ----
+// ---- launch 3: LayerNorm2 folded through RPB rows of c_fc, GELU, their RPB columns of mlp.c_proj ----
+// RPB = 16 hidden units per workgroup, 32 where a row takes 8 lanes (Q4_0: the slab is then one block per row)
 template <int TYPE, int KC, int NP>
 __global__ __launch_bounds__(256) void k_dec_mlp(DecMlpArgs a) {
+  typedef DecFmt<TYPE> F;
+  constexpr int RPB = 4 * F::RPW;
   __shared__ __align__(16) float xs[256 * KC];
   __shared__ float red[24];
-  __shared__ __align__(16) float hs[16];
+  __shared__ __align__(16) float hs[RPB];
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
-  const int g = lane >> 4, l = lane & 15;
+  const int g = lane / F::LPR, l = lane % F::LPR;
   const int D = a.st.D;
   const int slab = blockIdx.x;
-  const int row = slab * 16 + wv * 4 + g;  // < F: the launcher requires F % 16 == 0
+  const int row = slab * RPB + wv * F::RPW + g;  // < F: the launcher requires F % RPB == 0
   DecStageRegs<1, NP> sr;
   dec_stage_request(a.st, sr);
   __builtin_amdgcn_sched_barrier(0);
-  constexpr int XPC = DecFmt<TYPE>::XPC, NCL = KC * 16 / XPC, SCH = 16 / XPC;
+  constexpr int XPC = F::XPC, NCL = KC * 256 / XPC / F::LPR, SCH = RPB / XPC;
   uint4 w[NCL];
   unsigned sc[NCL];
   dec_row_request<TYPE, KC>(a.wq, a.wd, row, l, w, sc);
   const float fs = a.fold_s[row], fc = a.fold_c[row];
-  // this slab's 16 columns (SCH chunks) of the second Linear: row r = tid + 256 j (D = 256 * KC)
+  // this slab's RPB columns (SCH chunks) of the second Linear: row r = tid + 256 j (D = 256 * KC)
   uint4 pw[KC][SCH];
   unsigned ps[KC];
 #pragma unroll
@@ -336,22 +346,24 @@ __global__ __launch_bounds__(256) void k_dec_mlp(DecMlpArgs a) {
     const int r = tid + 256 * j;
 #pragma unroll
     for (int k = 0; k < SCH; k++) pw[j][k] = ((const uint4 *)a.pq)[((int64_t)slab * D + r) * SCH + k];
-    ps[j] = DecFmt<TYPE>::QUANT ? a.pd[(int64_t)(slab >> 1) * D + r] : 0;
+    // one scale per 32 columns: two slabs of 16 share it, a slab of 32 has its own
+    ps[j] = F::QUANT ? a.pd[(int64_t)(RPB == 16 ? slab >> 1 : slab) * D + r] : 0;
   }
   __builtin_amdgcn_sched_barrier(0);
   float mu, rstd;
-  dec_stage_finish(a.st, sr, xs, red, mu, rstd);
+  dec_stage_finish<F::SWZ>(a.st, sr, xs, red, mu, rstd);
   const float acc = dec_row_dot<TYPE, KC>(w, sc, xs, l);
-  if (l == 0) hs[wv * 4 + g] = ct_gelu(rstd * (acc - mu * fs) + fc);
+  if (l == 0) hs[wv * F::RPW + g] = ct_gelu(rstd * (acc - mu * fs) + fc);
   __syncthreads();
-  float hr[16];
+  float hr[RPB], hsum = 0.0f;
 #pragma unroll
-  for (int t = 0; t < 4; t++) {
+  for (int t = 0; t < RPB / 4; t++) {
     const float4 v = *(const float4 *)(hs + 4 * t);
     hr[4 * t + 0] = v.x;
     hr[4 * t + 1] = v.y;
     hr[4 * t + 2] = v.z;
     hr[4 * t + 3] = v.w;
+    if (TYPE == CTHIP_Q4_0) hsum += (v.x + v.y) + (v.z + v.w);
   }
   long long *accum = a.accum + (int64_t)xcd_id() * D;
 #pragma unroll
@@ -359,7 +371,7 @@ __global__ __launch_bounds__(256) void k_dec_mlp(DecMlpArgs a) {
     float s = 0.0f;
 #pragma unroll
     for (int k = 0; k < SCH; k++)
-      s += chunk_dot<TYPE>(pw[j][k], DecFmt<TYPE>::QUANT ? half_bits_to_float((unsigned short)ps[j]) : 1.0f, hr + XPC * k, 0.0f);
+      s += chunk_dot<TYPE>(pw[j][k], F::QUANT ? half_bits_to_float((unsigned short)ps[j]) : 1.0f, hr + XPC * k, hsum);
     // no device-scope bits: the addition happens in this XCD's L2.  (One device-wide accumulator instead of
     // one per XCD costs the 192 workgroups more in contention than the seven arrays cost the reader.)
     __hip_atomic_fetch_add(accum + tid + 256 * j, to_fix(s), __ATOMIC_RELAXED,
@@ -434,11 +446,13 @@ __global__ __launch_bounds__(256) void k_xcd_atomics_probe(long long *acc, long 
 }
 
 // ------------------------------------------------------------------ host side
-static int type_xpc(int type) { return type == CTHIP_Q8_0 ? 16 : type == CTHIP_F16 ? 8 : type == CTHIP_F32 ? 4 : 0; }
+static int type_xpc(int type) { return type == CTHIP_Q8_0 ? 16 : type == CTHIP_Q4_0 ? 32 : type == CTHIP_F16 ? 8 : type == CTHIP_F32 ? 4 : 0; }
+// rows of a 256-thread workgroup: 16 lanes a row, 8 where a chunk is a block of 32
+static int type_rpb(int type) { return type == CTHIP_Q4_0 ? 32 : 16; }
 
 bool dec_fused_supported(int type_attn, int type_proj, int type_fc, int type_fc2, int D, int H, int F) {
   if (type_attn != type_proj || type_attn != type_fc || type_attn != type_fc2) return false;
-  if (type_attn != CTHIP_Q8_0 && type_attn != CTHIP_F32 && type_attn != CTHIP_F16) return false;
+  if (type_attn != CTHIP_Q8_0 && type_attn != CTHIP_Q4_0 && type_attn != CTHIP_F32 && type_attn != CTHIP_F16) return false;
   if (D % 256 || D < 256 || D > 1024) return false;
   if (H <= 0 || D % H || D / H != 64) return false;
   if (H != 4 && H != 8 && H != 12 && H != 16) return false;
@@ -494,7 +508,7 @@ static int relay(const WMat *w, int group_cols, void **pq, void **pd) {
   hipLaunchKernelGGL(k_relay_chunks, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, state().stream, (const uint4 *)w->q,
                      (uint4 *)*pq, rows, cpr, cpg);
   CTHIP_LAUNCH_CHECK();
-  if (w->type == CTHIP_Q8_0) {
+  if (w->type == CTHIP_Q8_0 || w->type == CTHIP_Q4_0) {
     const int spr = (int)(w->cols / 32), spg = group_cols >= 32 ? group_cols / 32 : 1;
     if ((rc = cthip_alloc(pd, (size_t)rows * spr * 2))) return rc;
     const int64_t ns = (int64_t)rows * spr;
@@ -506,11 +520,12 @@ static int relay(const WMat *w, int group_cols, void **pq, void **pd) {
 }
 
 int dec_relay_heads(const WMat *w, int DH, void **pq, void **pd) { return relay(w, DH, pq, pd); }
-int dec_relay_slabs(const WMat *w, void **pq, void **pd) { return relay(w, 16, pq, pd); }
+int dec_relay_slabs(const WMat *w, void **pq, void **pd) { return relay(w, type_rpb(w->type), pq, pd); }
 
 #define DEC_TYPES(GO_T)                 \
   switch (type) {                       \
     case CTHIP_Q8_0: GO_T(CTHIP_Q8_0); break; \
+    case CTHIP_Q4_0: GO_T(CTHIP_Q4_0); break; \
     case CTHIP_F32: GO_T(CTHIP_F32); break;   \
     case CTHIP_F16: GO_T(CTHIP_F16); break;   \
     default: return fail(CTHIP_E_BAD_ARG, "decoder: the three-launch layer has no kernels for weight type %d", type); \
@@ -519,7 +534,8 @@ int dec_relay_slabs(const WMat *w, void **pq, void **pd) { return relay(w, 16, p
 int launch_dec_qkv(const DecQkvArgs &a, int type, bool from_accum) {
   const int D = a.st.D, KC = D / 256;
   if (D % 256 || KC < 1 || KC > 4 || a.rows != 3 * D) return fail(CTHIP_E_BAD_ARG, "decoder: fused qkv launch with D = %d, rows = %d", D, a.rows);
-  dim3 grid((a.rows + 15) / 16), block(256);
+  const int rpb = type_rpb(type);
+  dim3 grid((a.rows + rpb - 1) / rpb), block(256);
   hipStream_t st = state().stream;
 #define GO(T, KC_)                                                                                  \
   case KC_:                                                                                         \
@@ -565,8 +581,9 @@ int launch_dec_attn_proj(const DecAttnArgs &a, int type, int H, int D, int repli
 int launch_dec_mlp(const DecMlpArgs &a, int type, int F, int H) {
   const int D = a.st.D, KC = D / 256;
   if (D % 256 || KC < 1 || KC > 4 || F % 32) return fail(CTHIP_E_BAD_ARG, "decoder: fused MLP launch with D = %d, F = %d", D, F);
+  const int rpb = type_rpb(type);
   if (H != 4 && H != 8 && H != 12 && H != 16) return fail(CTHIP_E_BAD_ARG, "decoder: fused MLP launch with %d heads", H);
-  dim3 grid(F / 16), block(256);
+  dim3 grid(F / rpb), block(256);
   hipStream_t st = state().stream;
 #define GO2(T, KC_, NP_) hipLaunchKernelGGL((k_dec_mlp<T, KC_, NP_>), grid, block, 0, st, a)
 #define GO(T, KC_)                     \

@@ -35,7 +35,7 @@ def _dequantised(oracle, weights, keys, kind):
 
 
 @pytest.mark.parametrize("name,kind", [("gpt2-tiny", "f32"), ("gpt2-tiny", "q8_0"), ("gpt2-tiny", "q4_0"),
-                                       ("gpt2-tiny", "f16"), ("gpt2-mini", "q8_0")])
+                                       ("gpt2-tiny", "f16"), ("gpt2-mini", "q8_0"), ("gpt2-mini", "q4_0")])
 def test_gpt2_generate_matches_oracle(oracle, name, kind):
     print(f"case: gpt2 decode {name} {kind}", flush=True)
     from caten_amd import synth, llm
@@ -47,6 +47,7 @@ def test_gpt2_generate_matches_oracle(oracle, name, kind):
     want_tokens, want_logits = ref.generate(prompt, steps, onehot=(name == "gpt2-tiny"), keep_logits=True)
 
     model = llm.make_gpt2(cfg, llm.gpt2_state_dict(w, kind))
+    assert model.lib.cthip_decoder_layer_launches(model.handle) == 3  # every weight format runs the three-launch layer
     got_tokens, got_logits = llm.gpt2_generate(model, prompt, steps, on_device=False, keep_logits=True)
     assert got_tokens == want_tokens
     for g, r in zip(got_logits, want_logits):
@@ -135,7 +136,8 @@ def test_streamed_weights_decode_identical(arch):
 
 
 @pytest.mark.parametrize("name,plen,kind", [("gpt2-tiny", 5, "q8_0"), ("gpt2-mini", 40, "q8_0"), ("gpt2-tiny", 5, "f32"),
-                                            ("gpt2-mini", 40, "f32"), ("gpt2-tiny", 5, "f16"), ("gpt2-mini", 40, "f16")])
+                                            ("gpt2-mini", 40, "f32"), ("gpt2-tiny", 5, "f16"), ("gpt2-mini", 40, "f16"),
+                                            ("gpt2-tiny", 5, "q4_0"), ("gpt2-mini", 40, "q4_0")])
 def test_three_launch_layer_equals_five_launch_layer(name, plen, kind):
     """The decode layer as three launches (attention + its projection, and the whole MLP, one launch each, partial
     vectors added up by the consumer) and as five launches (one per Linear) are the same function: identical greedy

@@ -217,33 +217,41 @@ def decode_config(lib, name, model_name, kind, weights, prompt, steps, warmup, c
 
 
 def byoc_decode(cfg, weights, prompt, steps, want_tokens):
-    """the plug-in path: the compiled graph's node list walked by the VM, every item through cthip_program_launch"""
+    """the plug-in path: the compiled graph's node list, every item through cthip_program_launch; walked inside the
+    library (one call per forward), and -- fewer steps, for comparison -- node by node on the host"""
     from caten_amd import graphs
     from caten_amd.buffer import transfer_into_array
-    g = graphs.GPT2Graph(cfg, weights)
-    toks = [int(t) for t in prompt]
-    tok = int(np.asarray(transfer_into_array(g.forward(toks, 0))).ravel()[0])
-    got, n = [tok], len(toks)
-    for _ in range(3):  # warm-up steps (pools of the step's shapes, uploads)
-        tok = int(np.asarray(transfer_into_array(g.forward([tok], n))).ravel()[0])
-        got.append(tok)
-        n += 1
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        tok = int(np.asarray(transfer_into_array(g.forward([tok], n))).ravel()[0])
-        got.append(tok)
-        n += 1
-    wall = time.perf_counter() - t0
-    routes = g.routes()
-    launches = g.n_kernels
-    g.close()
-    k = min(len(got), len(want_tokens))
-    if want_tokens and got[:k] != want_tokens[:k]:
-        raise SystemExit(f"bench: plug-in path: tokens {got[:k]} differ from the CPU port's {want_tokens[:k]}")
+
+    def run(native, nsteps):
+        g = graphs.GPT2Graph(cfg, weights, native=native)
+        toks = [int(t) for t in prompt]
+        tok = int(np.asarray(transfer_into_array(g.forward(toks, 0))).ravel()[0])
+        got, n = [tok], len(toks)
+        for _ in range(3):  # warm-up steps (pools of the step's shapes, uploads)
+            tok = int(np.asarray(transfer_into_array(g.forward([tok], n))).ravel()[0])
+            got.append(tok)
+            n += 1
+        t0 = time.perf_counter()
+        for _ in range(nsteps):
+            tok = int(np.asarray(transfer_into_array(g.forward([tok], n))).ravel()[0])
+            got.append(tok)
+            n += 1
+        wall = time.perf_counter() - t0
+        routes, launches = g.routes(), g.n_kernels
+        g.close()
+        k = min(len(got), len(want_tokens))
+        if want_tokens and got[:k] != want_tokens[:k]:
+            raise SystemExit(f"bench: plug-in path: tokens {got[:k]} differ from the CPU port's {want_tokens[:k]}")
+        return wall, routes, launches, k
+
+    wall, routes, launches, k = run(True, steps)
+    host_wall = run(False, max(5, steps // 5))[0] / max(5, steps // 5)
     return {"value": steps / wall, "unit": "tokens/s", "ms_per_step": wall * 1e3 / steps, "steps": steps,
             "launches_per_step": launches, "weights": "fp32 (what gguf->state-dict hands a Caten graph whatever the file's type)",
-            "what": "GPT-2-small graph as Allocate / scalar / JIT_KERNEL nodes walked by the VM mirror; one cthip_program_launch per "
-                    "Schedule-Item, token returned to the host after every forward (the reference's gpt2-generate loop)",
+            "what": "GPT-2-small graph as Allocate / scalar / JIT_KERNEL nodes, walked inside the library (cthip_vm_run, one call "
+                    "per forward); one cthip_program_launch per Schedule-Item, token returned to the host after every forward "
+                    "(the reference's gpt2-generate loop)",
+            "ms_per_step_walked_on_the_host": host_wall * 1e3,
             "hand_written_items": sorted(k for k, v in routes.items() if v != "rendered"),
             "rendered_items": sorted(k for k, v in routes.items() if v == "rendered"),
             "checked": f"{k} greedy tokens equal the CPU port's" if want_tokens else "unchecked (no CPU leg)"}

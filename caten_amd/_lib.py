@@ -68,6 +68,18 @@ PROTOTYPES = {
     "cthip_program_last_route": (C.c_char_p, [_vp]),
     "cthip_program_bind": (_i, [_vp, _vp]),
     "cthip_program_launch": (_i, [_vp, C.POINTER(C.c_void_p), _i]),
+    "cthip_vm_create": (_i, [_vpp, _i]),
+    "cthip_vm_destroy": (_i, [_vp]),
+    "cthip_vm_add_scalar": (_i, [_vp, _i, _i, _i, C.POINTER(_i), C.POINTER(C.c_longlong), C.POINTER(C.c_double)]),
+    "cthip_vm_add_allocate": (_i, [_vp, _i, _i, _i, C.POINTER(_i), C.POINTER(C.c_longlong)]),
+    "cthip_vm_add_kernel": (_i, [_vp, _vp, _i, C.POINTER(_i), C.POINTER(C.c_longlong), C.POINTER(C.c_double), C.POINTER(_i),
+                                 _i, C.POINTER(_i), C.POINTER(_i)]),
+    "cthip_vm_set_int": (_i, [_vp, _i, C.c_longlong]),
+    "cthip_vm_set_float": (_i, [_vp, _i, C.c_double]),
+    "cthip_vm_set_buffer": (_i, [_vp, _i, _vp]),
+    "cthip_vm_run": (_i, [_vp]),
+    "cthip_vm_get": (_i, [_vp, _i, C.POINTER(_i), C.POINTER(C.c_longlong), C.POINTER(C.c_double), _vpp]),
+    "cthip_vm_launches": (C.c_longlong, [_vp]),
     "cthip_timer_start": (_i, []),
     "cthip_timer_stop": (_i, [C.POINTER(_f)]),
     "cthip_dequant": (_i, [_i, _vp, _i64, _vp]),

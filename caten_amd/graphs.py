@@ -35,7 +35,7 @@ def _row_major(shape):
 class GPT2Graph:
     """make-gpt2's compiled model (apps/gpt2/gpt2.lisp:82-95) behind `forward(x, s, n)`."""
 
-    def __init__(self, cfg: dict, weights: dict, device: int = 0):
+    def __init__(self, cfg: dict, weights: dict, device: int = 0, native: bool = True):
         self.cfg = dict(cfg)
         D, H, F, V, L, NL = cfg["dim"], cfg["n_heads"], cfg["ffn"], cfg["vocab"], cfg["max_seq"], cfg["n_layers"]
         Dh = D // H
@@ -107,7 +107,7 @@ class GPT2Graph:
         kernel("lm_head", ["logits"], [alloc("logits", ["s", V]), "s", "lnf", param("lm_head", weights["lm_head"])])
         kernel("argmax", ["out"], [alloc("out", [1, 1], "int64"), "s", "logits"])
         self.params = params
-        self.vm = HipRuntime(g, fw_outputs=["out"], renderer=self.renderer, device=device)
+        self.vm = HipRuntime(g, fw_outputs=["out"], renderer=self.renderer, device=device, native=native)
         self.n_kernels = sum(1 for n in g if n.type == "JIT_KERNEL")
 
     def forward(self, tokens, n: int):

@@ -278,10 +278,38 @@ class HipRuntime(GraphRuntime):
     (cf. MetalRuntime's initialize-instance :after, source/byoc/metal.lisp:106-112)."""
     buffer_type = HipBuffer
 
-    def __init__(self, graph=(), fw_outputs=(), variables=None, renderer=None, device: int = 0):
+    def __init__(self, graph=(), fw_outputs=(), variables=None, renderer=None, device: int = 0, native: bool = True):
         super().__init__(list(graph), fw_outputs, variables, renderer)
         self.lib = _lib.init(device)
         self._uploaded: Dict[int, HipBuffer] = {}
+        # native: hand the node list to the library at the first forward and walk it there (NativeWalk); lists
+        # with node kinds that walk does not know, and PROFILE=1 runs, are walked here
+        self.native = native
+        self._walk: Optional[NativeWalk] = None
+
+    def forward(self, *params):
+        if self.native and not self.profile and self._walk is None:
+            try:
+                self._walk = NativeWalk(self)
+            except Exception:
+                # a list the library does not walk -- or a malformed one, which the walk here reports at its node,
+                # wrapped like the reference's runtime-error
+                self.native = False
+        if self._walk is not None:
+            try:
+                return self._walk.forward(params)
+            except _lib.HipError as e:
+                raise RuntimeError_(self, e) from e
+        return super().forward(*params)
+
+    def getvar(self, var):
+        # after a forward walked by the library the variable table lives there
+        if self._walk is not None and var in self._walk.slots:
+            try:
+                return self._walk._output(var)
+            except KeyError:
+                pass
+        return super().getvar(var)
 
     def adopt(self, buf: AbstractBuffer) -> AbstractBuffer:
         """Weights loaded from GGUF are host buffers whatever the backend
@@ -309,10 +337,174 @@ class HipRuntime(GraphRuntime):
         _lib.check(self.lib.cthip_sync())
 
     def free(self):
+        if self._walk is not None:
+            self._walk.close()
+            self._walk = None
         super().free()
         for b in self._uploaded.values():
             close_buffer(self, b)
         self._uploaded.clear()
+
+
+class NativeWalk:
+    """The node list of a HipRuntime handed to the library once, so that a forward is one call (cthip_vm_run) instead
+    of one host step per node: the walk of runtime-forward (runtime.lisp:106-145) over `:Allocate`, the scalar nodes
+    and `:JIT_KERNEL`.  Raises NotImplementedError for a list that holds anything else (views, custom ops, kernels
+    with boxed rank-0 outputs); the runtime then keeps walking it here."""
+
+    SCALAR_OPS = {"Add": 0, "Mul": 1, "Neg": 2, "Idiv": 3, "Mod": 4, "Max": 5}
+    DTYPE_CODES = {"bool": 1, "float64": 2, "float32": 3, "uint64": 4, "int64": 5, "uint32": 6, "int32": 7,
+                   "uint16": 8, "int16": 9, "uint8": 10, "int8": 11}
+
+    def __init__(self, rt: "HipRuntime"):
+        from .renderer import HipProgram
+        self.rt, self.lib = rt, rt.lib
+        self.slots: Dict[Any, int] = {}
+        self.inputs: Dict[Any, int] = {}        # symbol bound by forward(...) -> slot of the `:Allocate :from` that reads it
+        self.meta: Dict[int, tuple] = {}        # slot -> (dtype, shape operands) of the :Allocate that opened it
+        for n in rt.graph:
+            for name in list(n.writes) + [r for r in n.reads if isinstance(r, str)]:
+                self.slots.setdefault(name, len(self.slots))
+            frm = n.attrs.get("from") if n.type == "Allocate" else None
+            if isinstance(frm, str):
+                self.slots.setdefault(frm, len(self.slots))
+        self.vm = C.c_void_p()
+        _lib.check(self.lib.cthip_vm_create(C.byref(self.vm), max(1, len(self.slots))))
+        self._holders: Dict[int, HipBuffer] = {}
+        try:
+            for n in rt.graph:
+                self._add(n, HipProgram)
+        except Exception:
+            self.close()
+            raise
+
+    def _operands(self, reads):
+        k = (C.c_int * len(reads))()
+        iv = (C.c_longlong * len(reads))()
+        fv = (C.c_double * len(reads))()
+        for j, r in enumerate(reads):
+            if isinstance(r, str):
+                k[j], iv[j] = 2, self.slots[r]
+            elif isinstance(r, (bool, int, np.integer)):
+                k[j], iv[j] = 0, int(r)
+            elif isinstance(r, (float, np.floating)):
+                k[j], fv[j] = 1, float(r)
+            else:
+                raise NotImplementedError(f"native walk: operand {r!r}")
+        return k, iv, fv
+
+    def _add(self, n: Node, HipProgram):
+        lib = self.lib
+        if n.type == "Allocate":
+            out = self.slots[n.writes[0]]
+            frm = n.attrs.get("from")
+            if frm is not None:
+                if isinstance(frm, AbstractBuffer):  # a parameter: uploaded once, bound for good
+                    dev = self.rt.adopt(frm)
+                    if dev.nrank == 0:
+                        raise NotImplementedError("native walk: a rank-0 parameter")
+                    _lib.check(lib.cthip_vm_set_buffer(self.vm, out, dev.value))
+                else:
+                    self.inputs[frm] = out
+                return
+            nrank = n.attrs["nrank"]
+            if nrank == 0:
+                raise NotImplementedError("native walk: a rank-0 :Allocate")
+            k, iv, _ = self._operands(n.reads[:nrank])
+            _lib.check(lib.cthip_vm_add_allocate(self.vm, out, np.dtype(DTYPES[n.attrs["dtype"]]).itemsize, nrank, k, iv))
+            self.meta[out] = (n.attrs["dtype"], list(n.reads[:nrank]))
+        elif n.type in self.SCALAR_OPS:
+            k, iv, fv = self._operands(n.reads)
+            _lib.check(lib.cthip_vm_add_scalar(self.vm, self.SCALAR_OPS[n.type], self.slots[n.writes[0]], len(n.reads), k, iv, fv))
+        elif n.type == "JIT_KERNEL":
+            info: CompiledKernel = n.attrs["kernel_info"]
+            prog = info.caller
+            if not isinstance(prog, HipProgram):
+                raise NotImplementedError("native walk: a kernel whose caller is not a HipProgram")
+            codes = (C.c_int * len(n.reads))()
+            for j, (g, r) in enumerate(zip(prog.defglobals, n.reads)):
+                if g["pointer_p"]:
+                    if not isinstance(r, str):
+                        raise NotImplementedError("native walk: a number passed by pointer")
+                    codes[j] = 0
+                else:
+                    codes[j] = self.DTYPE_CODES[g["dtype"]]
+            if len(prog.defglobals) != len(n.reads):
+                raise AssertionError(f"HIP: {prog.name} takes {len(prog.defglobals)} arguments, got {len(n.reads)}")
+            k, iv, fv = self._operands(n.reads)
+            pos = (C.c_int * len(info.out_positions))(*info.out_positions)
+            outs = (C.c_int * len(n.writes))(*[self.slots[w] for w in n.writes])
+            if len(info.out_positions) != len(n.writes):
+                raise AssertionError("Runtime: the number of outputs does not match the number of writes.")
+            _lib.check(lib.cthip_vm_add_kernel(self.vm, prog.program, len(n.reads), k, iv, fv, codes, len(n.writes), pos, outs))
+            for w, p_ in zip(n.writes, info.out_positions):  # the written name is the same storage as the argument
+                src = n.reads[p_]
+                if isinstance(src, str) and self.slots[src] in self.meta:
+                    self.meta[self.slots[w]] = self.meta[self.slots[src]]
+        else:
+            raise NotImplementedError(f"native walk: node type :{n.type}")
+
+    def forward(self, params):
+        lib, rt = self.lib, self.rt
+        for name, v in params:
+            rt.setvar(name, v)
+            slot = self.inputs.get(name, self.slots.get(name))
+            if slot is None:
+                continue
+            if isinstance(v, AbstractBuffer) and v.nrank > 0:
+                _lib.check(lib.cthip_vm_set_buffer(self.vm, slot, rt.adopt(v).value))
+                continue
+            x = v.value if isinstance(v, AbstractBuffer) else v
+            if isinstance(x, (bool, int, np.integer)):
+                _lib.check(lib.cthip_vm_set_int(self.vm, slot, int(x)))
+            else:
+                _lib.check(lib.cthip_vm_set_float(self.vm, slot, float(x)))
+        rc = lib.cthip_vm_run(self.vm)
+        if rc != 0:
+            _lib.check(rc)
+        outs = tuple(self._output(o) for o in rt.fw_outputs)
+        for name, b in zip(rt.fw_outputs, outs):
+            rt.variables[name] = b
+        return outs[0] if len(outs) == 1 else outs
+
+    def _value(self, slot):
+        kind, iv, fv, ptr = C.c_int(), C.c_longlong(), C.c_double(), C.c_void_p()
+        _lib.check(self.lib.cthip_vm_get(self.vm, slot, C.byref(kind), C.byref(iv), C.byref(fv), C.byref(ptr)))
+        return kind.value, iv.value, fv.value, ptr.value
+
+    def _output(self, name):
+        slot = self.slots[name]
+        kind, iv, fv, ptr = self._value(slot)
+        if kind == 1:
+            return iv
+        if kind == 2:
+            return fv
+        if kind != 3 or slot not in self.meta:
+            raise KeyError(f"Runtime: the variable {name} is not defined in the graph.")
+        dtype, shape_ops = self.meta[slot]
+        shape = [int(self._value(self.slots[s])[1]) if isinstance(s, str) else int(s) for s in shape_ops]
+        stride, acc = [], 1
+        for s in reversed(shape):
+            stride.append(acc)
+            acc *= s
+        # the storage belongs to the walk's pool: the holder is never closed here, the result is a copy of it
+        holder = self._holders.get(slot)
+        if holder is None or holder.value != ptr or holder.shape != shape:
+            holder = make_buffer(shape, list(reversed(stride)), dtype, None, value=ptr, device=HipBuffer)
+            self._holders[slot] = holder
+        return holder.copy()
+
+    @property
+    def launches(self) -> int:
+        return int(self.lib.cthip_vm_launches(self.vm))
+
+    def close(self):
+        if self.vm:
+            self.lib.cthip_vm_destroy(self.vm)
+            self.vm = C.c_void_p()
+        for h in self._holders.values():
+            h._value = None
+        self._holders.clear()
 
 
 class HipAutoScheduler:

@@ -138,6 +138,47 @@ const char *cthip_program_last_route(const void *program);
 int cthip_program_bind(void *program, void *module);
 int cthip_program_launch(void *program, void **args, int nargs);
 
+/* ---- the walk of a compiled node list behind one call per forward ----
+ * runtime-forward / runtime-step (source/runtime/runtime.lisp:106-145) over the three node kinds a compiled model
+ * consists of: `:Allocate` (runtime.lisp:228-259: a pool per node, the same shape gets the same storage back with
+ * its contents, another shape a new zero-filled one), the scalar nodes that compute dynamic shapes
+ * (`:Add :Mul :Neg :Idiv :Mod :Max`, runtime.lisp:396-449; integer division and modulo round toward minus
+ * infinity) and `:JIT_KERNEL` (source/codegen/runner.lisp:20-32: launch, then writes[k] = args[out-positions[k]]).
+ * For hosts whose own walk costs more per node than a launch: the list is handed over once, variables as slot
+ * numbers, callers as programs; a forward binds the inputs and calls cthip_vm_run.  Node kinds beyond these
+ * (views, custom ops) stay with the host's walk.
+ *   operands: kinds[k] 0 = the integer ivals[k], 1 = the float fvals[k], 2 = slot ivals[k]
+ *   dtypes[k] of a kernel argument: CTHIP_VM_PTR = the slot's device pointer, else the by-value scalar type the
+ *     number is cast to (coerce-dtyped-buffer, source/codegen/helpers.lisp:118-125)
+ * Parameters and inputs bound with cthip_vm_set_buffer (`:Allocate :from`, runtime.lisp:228-243) are never freed
+ * here; buffers the walk opened are freed by cthip_vm_destroy.  cthip_vm_get: kind 0 = unset, 1 = integer,
+ * 2 = float, 3 = device buffer.  A failing node stops the walk; the message names its index. */
+#define CTHIP_VM_PTR 0
+#define CTHIP_VM_BOOL 1
+#define CTHIP_VM_F64 2
+#define CTHIP_VM_F32 3
+#define CTHIP_VM_U64 4
+#define CTHIP_VM_I64 5
+#define CTHIP_VM_U32 6
+#define CTHIP_VM_I32 7
+#define CTHIP_VM_U16 8
+#define CTHIP_VM_I16 9
+#define CTHIP_VM_U8 10
+#define CTHIP_VM_I8 11
+int cthip_vm_create(void **vm, int n_slots);
+int cthip_vm_destroy(void *vm);
+/* op: 0 Add, 1 Mul, 2 Neg, 3 Idiv, 4 Mod, 5 Max; the result is an integer when every operand is */
+int cthip_vm_add_scalar(void *vm, int op, int out, int n_in, const int *kinds, const long long *ivals, const double *fvals);
+int cthip_vm_add_allocate(void *vm, int out, int elem_bytes, int nrank, const int *kinds, const long long *ivals);
+int cthip_vm_add_kernel(void *vm, void *program, int nargs, const int *kinds, const long long *ivals, const double *fvals,
+                        const int *dtypes, int n_out, const int *out_positions, const int *out_slots);
+int cthip_vm_set_int(void *vm, int slot, long long value);
+int cthip_vm_set_float(void *vm, int slot, double value);
+int cthip_vm_set_buffer(void *vm, int slot, void *device_ptr);
+int cthip_vm_run(void *vm);
+int cthip_vm_get(const void *vm, int slot, int *kind, long long *ivalue, double *fvalue, void **device_ptr);
+long long cthip_vm_launches(const void *vm);  /* kernels launched so far */
+
 /* Event timing on the library's stream (PROFILE=1 in the reference times each
  * JIT kernel on the host clock, source/codegen/runner.lisp:7-31). */
 int cthip_timer_start(void);

@@ -15,15 +15,19 @@ HAND_WRITTEN = {"embed_tokens": "cthip_embedding", "embed_positions": "cthip_emb
 RENDERED = ("mask", "assign_k", "assign_v", "merge_heads")  # element-wise generators and copies
 
 
-def _run(oracle, name, prompt_len, steps, seed=0):
+def _run(oracle, name, prompt_len, steps, seed=0, native=True):
     from caten_amd import synth, graphs
     cfg = synth.GPT2_CONFIGS[name]
     w = synth.gpt2_weights(cfg, seed=seed)
     prompt = synth.prompt(cfg["vocab"], prompt_len, seed=seed)
-    model = graphs.GPT2Graph(cfg, w)
+    model = graphs.GPT2Graph(cfg, w, native=native)
     from caten_amd.buffer import transfer_into_array
     try:
         got = model.generate(prompt, steps)
+        # native: the node list is walked by the library, one call per forward; else node by node on the host
+        assert (model.vm._walk is not None) == native
+        if native:
+            assert model.vm._walk.launches == steps * model.n_kernels
         routes = model.routes()
         n_kernels = model.n_kernels
         logits = np.asarray(transfer_into_array(model.vm.getvar("logits"))).reshape(-1, cfg["vocab"])[-1]
@@ -35,8 +39,9 @@ def _run(oracle, name, prompt_len, steps, seed=0):
     return got, want, routes, n_kernels, cfg
 
 
-def test_gpt2_tiny_forward_through_the_vm_matches_oracle(oracle):
-    got, want, routes, n_kernels, cfg = _run(oracle, "gpt2-tiny", 8, 12)
+@pytest.mark.parametrize("native", [True, False])
+def test_gpt2_tiny_forward_through_the_vm_matches_oracle(oracle, native):
+    got, want, routes, n_kernels, cfg = _run(oracle, "gpt2-tiny", 8, 12, native=native)
     assert got == want, f"plug-in path {got} vs oracle {want}"
     assert n_kernels == 6 + 12 * cfg["n_layers"]  # embeddings, mask, ln_f, lm_head, argmax + 12 items per block
     for k, entry in HAND_WRITTEN.items():
@@ -45,10 +50,11 @@ def test_gpt2_tiny_forward_through_the_vm_matches_oracle(oracle):
         assert routes[k] == "rendered", (k, routes[k])
 
 
-def test_gpt2_tiny_single_token_prompt_and_ragged_lengths(oracle):
+@pytest.mark.parametrize("native", [True, False])
+def test_gpt2_tiny_single_token_prompt_and_ragged_lengths(oracle, native):
     # s = 1 from the first call on (every Linear a single-row launch), then a 5-token prompt (fewer than 8 rows)
     for plen in (1, 5):
-        got, want, routes, _, _ = _run(oracle, "gpt2-tiny", plen, 9, seed=plen)
+        got, want, routes, _, _ = _run(oracle, "gpt2-tiny", plen, 9, seed=plen, native=native)
         assert got == want, (plen, got, want)
 
 
@@ -225,3 +231,70 @@ def test_rope_and_swiglu_items_vs_oracle(oracle):
         assert k_rope.last_route == "rendered" and k_glu.last_route == "rendered"
         for b in (d_x, d_y, d_g, d_u, d_o):
             close_buffer(None, b)
+
+
+def test_the_librarys_walk_of_scalar_nodes_equals_the_hosts():
+    """:Add :Mul :Neg :Idiv :Mod :Max over numbers (runtime.lisp:396-449): the walk inside the library gives what the
+    host's walk gives, also for negative operands of the integer division and for mixed integers and floats"""
+    from caten_amd.runtime import HipRuntime, Node
+    g = [Node("Add", ["a"], ["n", "s", 3]), Node("Mul", ["b"], ["a", "s", 2]), Node("Neg", ["c"], ["b"]),
+         Node("Idiv", ["d"], ["c", 7]), Node("Mod", ["e"], ["c", 7]), Node("Max", ["f"], ["d", "e", -100]),
+         Node("Mod", ["g"], ["a", -5]), Node("Idiv", ["h"], ["a", -5]), Node("Mul", ["i"], ["a", 0.5]),
+         Node("Idiv", ["j"], ["i", 2]), Node("Mod", ["k"], ["c", 2.5])]
+    outs = [n.writes[0] for n in g]
+    for n, s in ((0, 1), (5, 3), (17, 16), (1023, 1)):
+        res = []
+        for native in (True, False):
+            rt = HipRuntime(g, fw_outputs=outs, native=native)
+            res.append(rt.forward(("n", n), ("s", s)))
+            assert (rt._walk is not None) == native
+            rt.free()
+        assert res[0] == res[1], (n, s, res)
+        assert all(type(a) is type(b) for a, b in zip(*res)), res
+
+
+def test_a_list_with_other_node_kinds_stays_with_the_hosts_walk():
+    """a :View is not one of the three node kinds the library walks: the runtime keeps the list and walks it itself"""
+    from caten_amd.runtime import HipRuntime, Node
+    from caten_amd.buffer import transfer_into_array
+    g = [Node("Allocate", ["x"], [4, 6, 6, 1], {"nrank": 2, "dtype": "float32"}),
+         Node("View", ["v"], ["x", 2, 6, 0, 0, 2, 6, 1, 1, 6, 1], {"nrank": 2, "broadcast": [False, False]})]
+    rt = HipRuntime(g, fw_outputs=["v"])
+    v = rt.forward()
+    assert rt._walk is None and rt.native is False
+    assert v.shape == [2, 6] and np.array_equal(transfer_into_array(v), np.zeros(12, np.float32))
+    rt.free()
+
+
+def test_pools_of_the_librarys_walk_keep_and_clear_storage_like_the_hosts():
+    """a buffer whose shape is unchanged comes back with its contents (the KV cache lives on that); one whose shape
+    changed is zero-filled again, whether its storage was kept or not (runtime.lisp:248-259)"""
+    from caten_amd import blueprints, renderer
+    from caten_amd.runtime import HipRuntime, Node, CompiledKernel
+    from caten_amd.buffer import transfer_into_array
+    # y[i] = y[i] + 1 over n elements: what is read is what the pool handed out
+    item = {"name": "fused_increment", "blueprint": [
+        {"type": "DEFINE-GLOBAL", "id": "y", "dtype": "float32", "pointer_p": True, "arg_type": "output", "nrank": 1},
+        {"type": "DEFINE-GLOBAL", "id": "n", "dtype": "int64", "pointer_p": False, "arg_type": "shape", "nrank": 0},
+        {"type": "FOR", "idx": "_gid0", "upfrom": 0, "below": {"op": "<", "args": ["_gid0", "n"]}, "by": 1, "scope": "local"},
+        {"type": "EXPR", "writes": [{"op": "AREF", "id": "y", "index": "_gid0"}],
+         "expr": {"op": "ADD", "args": [{"op": "AREF", "id": "y", "index": "_gid0"}, 1.0]}, "dtype": "float32"},
+        {"type": "ENDFOR", "idx": "_gid0"}]}
+    r = renderer.HipRenderer()
+    r.render_kernel(item)
+    r.compile_kernel([item])
+    info = CompiledKernel(item["name"], item["compiled_object"], out_positions=(0,))
+    for native in (True, False):
+        g = [Node("Allocate", ["y"], ["n", 1], {"nrank": 1, "dtype": "float32"}),
+             Node("JIT_KERNEL", ["y"], ["y", "n"], {"kernel_info": info, "dtypes": ["float32", "int64"]})]
+        rt = HipRuntime(g, fw_outputs=["y"], renderer=r, native=native)
+        seen = []
+        for n in (8, 8, 8, 5, 12, 12, 300, 8):
+            seen.append((n, np.asarray(transfer_into_array(rt.forward(("n", n)))).tolist()))
+        rt.free()
+        want, cur, last = [], 0, None
+        for n in (8, 8, 8, 5, 12, 12, 300, 8):
+            cur = cur + 1 if n == last else 1
+            last = n
+            want.append((n, [float(cur)] * n))
+        assert seen == want, (native, seen)

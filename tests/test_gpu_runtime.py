@@ -73,7 +73,7 @@ def test_caching_allocator_reuses_blocks(rt):
     _lib.check(lib.cthip_free(p))
 
 
-def _relu_matmul_graph(ca, M, N, K):
+def _relu_matmul_graph(ca, M, N, K, native=True):
     """The VM graph `jit` would hand the runtime for (caten (!relu (!matmul a b))) with symbolic sizes."""
     from tests.test_host import _matmul_item
     r = ca.HipRenderer()
@@ -88,13 +88,15 @@ def _relu_matmul_graph(ca, M, N, K):
         ca.Node("JIT_KERNEL", ["out2"], ["out", "m", "n", "kk", "a", "b"],
                 {"kernel_info": info, "dtypes": ["float32", "int64", "int64", "int64", "float32", "float32"]}),
     ]
-    return ca.HipRuntime(graph, fw_outputs=["out2"], renderer=r)
+    return ca.HipRuntime(graph, fw_outputs=["out2"], renderer=r, native=native)
 
 
-def test_vm_runs_a_rendered_kernel_with_dynamic_shapes(oracle):
+@pytest.mark.parametrize("native", [True, False])
+def test_vm_runs_a_rendered_kernel_with_dynamic_shapes(oracle, native):
+    """native: the node list is walked inside the library (one call per forward); else node by node on the host"""
     import caten_amd as ca
     from caten_amd.buffer import AbstractBuffer, make_buffer, transfer_into_array
-    vm = _relu_matmul_graph(ca, 0, 0, 0)
+    vm = _relu_matmul_graph(ca, 0, 0, 0, native=native)
     rng = np.random.default_rng(0)
     pools = []
     for (M, N, K) in ((33, 20, 17), (33, 20, 17), (64, 64, 64), (5, 300, 9)):
@@ -107,7 +109,9 @@ def test_vm_runs_a_rendered_kernel_with_dynamic_shapes(oracle):
         got = transfer_into_array(out).reshape(M, N)
         want = oracle.matmul(A, B, relu=True)
         assert np.max(np.abs(got - want)) < 1e-4
-        pools.append(vm.graph[2].attrs["pool"].value)
+        assert (vm._walk is not None) == native
+        pools.append(out.value if native else vm.graph[2].attrs["pool"].value)
+        assert out.value == pools[-1]
     assert pools[0] == pools[1]  # equal shape -> the :Allocate pool is reused (runtime.lisp:248-252)
     vm.free()
 

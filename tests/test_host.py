@@ -452,6 +452,18 @@ def test_blueprints_in_a_lisp_printers_spelling_are_read_the_same():
         assert route == want, (name, route)
 
 
+def test_the_references_own_rendered_item_renders_to_the_same_statement():
+    """the one Schedule-Item whose blueprint AND rendered C the reference prints side by side
+    (docs/end-to-end-example.lisp:225-250): `val_6[0] = sin(sin((1.0+1.5707964)));` -- the HIP text is that statement
+    with single-precision spellings"""
+    with open(os.path.join(GOLDEN_BP, "reference_sincos_item.sexp"), "rb") as f:
+        route, src = _create(f.read())
+    assert route == "rendered"
+    body = [ln.strip() for ln in src.splitlines() if ln.strip().startswith("val_6[0]")]
+    assert body == ["val_6[0] = sinf(sinf((1.0f+1.5707964f)));"], src
+    assert "fused_sin_sin_add_load_load6914144(float* val_6)" in src  # the reference's signature, verbatim
+
+
 def test_near_misses_of_the_decode_step_items_stay_rendered():
     from caten_amd import HipRenderer, blueprints as bp
     import copy

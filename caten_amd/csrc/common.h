@@ -254,6 +254,15 @@ __device__ __forceinline__ float wave_max(float v) {
   v = row16_max(v);
   return fmaxf(fmaxf(lane_bcast(v, 0), lane_bcast(v, 16)), fmaxf(lane_bcast(v, 32), lane_bcast(v, 48)));
 }
+// The four aligned groups of 16 lanes of a wavefront hold one value each (the same in every lane of a group): their
+// maximum / sum, in every lane.  Four lane reads on the scalar unit; a butterfly of __shfl_xor is two trips through
+// the LDS crossbar.  (All 64 lanes must be active.)
+__device__ __forceinline__ float groups16_max(float v) {
+  return fmaxf(fmaxf(lane_bcast(v, 0), lane_bcast(v, 16)), fmaxf(lane_bcast(v, 32), lane_bcast(v, 48)));
+}
+__device__ __forceinline__ float groups16_sum(float v) {
+  return (lane_bcast(v, 0) + lane_bcast(v, 16)) + (lane_bcast(v, 32) + lane_bcast(v, 48));
+}
 // sum over aligned groups of G lanes (G = 16, 32, 64); every lane gets the group's sum
 template <int G>
 __device__ __forceinline__ float group_sum(float v) {

@@ -245,14 +245,12 @@ __device__ __forceinline__ void flow_role_a(const FlowArgs &a, int h, float *sme
           d = fmaf(q4.y, kk.y, d);
           d = fmaf(q4.z, kk.z, d);
           d = fmaf(q4.w, kk.w, d);
-#pragma unroll
-          for (int o = LPK / 2; o > 0; o >>= 1) d += __shfl_xor(d, o, 64);
+          d = row16_sum(d);  // LPK == 16: the key's lanes are one row of the data-parallel primitives
           sk[u] = jk < T ? d * scale : -INFINITY;
           tmax = fmaxf(tmax, sk[u]);
         }
       }
-#pragma unroll
-      for (int o = LPK; o < 64; o <<= 1) tmax = fmaxf(tmax, __shfl_xor(tmax, o, 64));
+      tmax = groups16_max(tmax);
       const float m_new = fmaxf(m, tmax);   // finite: key t0 + 4 wv of step 0 exists
       const float corr = ct_exp(m - m_new);  // 0 on its first tile (m = -inf)
       float psum = 0.0f;
@@ -271,8 +269,7 @@ __device__ __forceinline__ void flow_role_a(const FlowArgs &a, int h, float *sme
           acc[3] = fmaf(p, vv.w, acc[3]);
         }
       }
-#pragma unroll
-      for (int o = LPK; o < 64; o <<= 1) psum += __shfl_xor(psum, o, 64);
+      psum = groups16_sum(psum);
       lsum = lsum * corr + psum;
       m = m_new;
     }

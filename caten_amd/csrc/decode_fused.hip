@@ -233,14 +233,23 @@ void k_dec_attn_proj(DecAttnArgs a) {
       d = fmaf(q4.y, kr[u].y, d);
       d = fmaf(q4.z, kr[u].z, d);
       d = fmaf(q4.w, kr[u].w, d);
+      // over the key's 16 lanes: data-parallel-primitive adds, no trip through the LDS crossbar
+      if (LPK == 16) {
+        d = row16_sum(d);
+      } else {
 #pragma unroll
-      for (int o = LPK / 2; o > 0; o >>= 1) d += __shfl_xor(d, o, 64);
+        for (int o = LPK / 2; o > 0; o >>= 1) d += __shfl_xor(d, o, 64);
+      }
       const bool ok = (t0 + (wv * NP + u) * KPW + g) < T;
       sc[u] = ok ? d * scale : -INFINITY;
       tmax = fmaxf(tmax, sc[u]);
     }
+    if (LPK == 16) {
+      tmax = groups16_max(tmax);
+    } else {
 #pragma unroll
-    for (int o = LPK; o < 64; o <<= 1) tmax = fmaxf(tmax, __shfl_xor(tmax, o, 64));
+      for (int o = LPK; o < 64; o <<= 1) tmax = fmaxf(tmax, __shfl_xor(tmax, o, 64));
+    }
     const float m_new = fmaxf(m, tmax);
     const float corr = ct_exp(m - m_new);
     float psum = 0.0f;
@@ -255,8 +264,12 @@ void k_dec_attn_proj(DecAttnArgs a) {
       acc[2] = fmaf(p, vr[u].z, acc[2]);
       acc[3] = fmaf(p, vr[u].w, acc[3]);
     }
+    if (LPK == 16) {
+      psum = groups16_sum(psum);
+    } else {
 #pragma unroll
-    for (int o = LPK; o < 64; o <<= 1) psum += __shfl_xor(psum, o, 64);
+      for (int o = LPK; o < 64; o <<= 1) psum += __shfl_xor(psum, o, 64);
+    }
     lsum = lsum * corr + psum;
     m = m_new;
   };

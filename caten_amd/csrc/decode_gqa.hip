@@ -250,8 +250,7 @@ void k_gqa_attn_proj(GqaAttnArgs a) {
       sc[u] = ok ? d * scale : -INFINITY;
       tmax = fmaxf(tmax, sc[u]);
     }
-#pragma unroll
-    for (int o = LPK; o < 64; o <<= 1) tmax = fmaxf(tmax, __shfl_xor(tmax, o, 64));
+    tmax = groups16_max(tmax);  // LPK == 16: one value per group of 16 lanes
     const float m_new = fmaxf(m, tmax);
     const float corr = ct_exp(m - m_new);
     float psum = 0.0f;
@@ -266,8 +265,7 @@ void k_gqa_attn_proj(GqaAttnArgs a) {
       acc[2] = fmaf(p, vr[u].z, acc[2]);
       acc[3] = fmaf(p, vr[u].w, acc[3]);
     }
-#pragma unroll
-    for (int o = LPK; o < 64; o <<= 1) psum += __shfl_xor(psum, o, 64);
+    psum = groups16_sum(psum);
     lsum = lsum * corr + psum;
     m = m_new;
   };

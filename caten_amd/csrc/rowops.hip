@@ -695,14 +695,22 @@ void k_attn_cached(float *__restrict__ out, const float *__restrict__ q,
       d = fmaf(q4.y, kr[u].y, d);
       d = fmaf(q4.z, kr[u].z, d);
       d = fmaf(q4.w, kr[u].w, d);
+      if (LPK == 16) {  // the key's lanes are one row of the data-parallel primitives: no trip through the LDS crossbar
+        d = row16_sum(d);
+      } else {
 #pragma unroll
-      for (int o = LPK / 2; o > 0; o >>= 1) d += __shfl_xor(d, o, 64);
+        for (int o = LPK / 2; o > 0; o >>= 1) d += __shfl_xor(d, o, 64);
+      }
       const bool ok = (t0 + (wv * NP + u) * KPW + g) < T;
       sc[u] = ok ? d * scale : -INFINITY;
       tmax = fmaxf(tmax, sc[u]);
     }
+    if (LPK == 16) {
+      tmax = groups16_max(tmax);
+    } else {
 #pragma unroll
-    for (int o = LPK; o < 64; o <<= 1) tmax = fmaxf(tmax, __shfl_xor(tmax, o, 64));
+      for (int o = LPK; o < 64; o <<= 1) tmax = fmaxf(tmax, __shfl_xor(tmax, o, 64));
+    }
     const float m_new = fmaxf(m, tmax);   // finite: this wavefront has at least one key here
     const float corr = ct_exp(m - m_new);  // 0 on its first tile (m = -inf)
     float ps = 0.0f;
@@ -717,8 +725,12 @@ void k_attn_cached(float *__restrict__ out, const float *__restrict__ q,
       acc[2] = fmaf(p, vr[u].z, acc[2]);
       acc[3] = fmaf(p, vr[u].w, acc[3]);
     }
+    if (LPK == 16) {  // every lane of a key holds the same p
+      ps = groups16_sum(ps);
+    } else {
 #pragma unroll
-    for (int o = LPK; o < 64; o <<= 1) ps += __shfl_xor(ps, o, 64);  // every lane of a key holds the same p
+      for (int o = LPK; o < 64; o <<= 1) ps += __shfl_xor(ps, o, 64);
+    }
     l = l * corr + ps;
     m = m_new;
   };

@@ -103,6 +103,9 @@ PROTOTYPES = {
     "cthip_sdpa_cached": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i]),
     "cthip_kv_append_q8": (_i, [_vp, _vp, _vp, _i, _i, _i]),
     "cthip_sdpa_cached_q8": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
+    "cthip_kv_page_rows": (_i, []),
+    "cthip_kv_append_paged": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i]),
+    "cthip_sdpa_cached_paged": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i]),
     "cthip_decoder_create": (_i, [_vpp, C.POINTER(DecoderConfig)]),
     "cthip_decoder_destroy": (_i, [_vp]),
     "cthip_decoder_load": (_i, [_vp, C.c_char_p, _i, _vp, _i64, _i64]),

@@ -31,7 +31,9 @@ struct State {
   // option "decode_skip": launches of the three-launch decode step that are left out, for knock-out timing (bits: 1 qkv,
   // 2 attention + projection, 4 MLP, 8 the sum in front of lm_head, 16 lm_head + argmax); tokens are meaningless then
   int decode_skip = 0;
-  int kv_cache = 0;  // option "kv_cache": 1 = sessions created afterwards keep their KV cache as Q8_0 rows (kvq.hip)
+  // option "kv_cache": how sessions created afterwards keep their KV cache: 1 = as Q8_0 rows (kvq.hip), 2 = fp32 rows in
+  // pages opened as the position reaches them (kvp.hip)
+  int kv_cache = 0;
 };
 State &state();
 // cthip_alloc without the zero fill, for temporaries that are fully written before they are read
@@ -98,6 +100,13 @@ int bmm_variant(const BmmArgs &a);  // 0 = neither layout fits
 int launch_bmm(const BmmArgs &a);
 
 // ---- KV cache as Q8_0 rows (kvq.hip): quant plane int8[max_len][KD], scale plane fp16[max_len][KD/32] ----
+// the KV cache in pages (kvp.hip): rows per page; row r of a layer lives at pages[r / kKvPageRows] + (r % kKvPageRows) * KD
+constexpr int kKvPageRows = 64;
+int launch_kvp_append(float *const *kpages, float *const *vpages, const float *ksrc, const float *vsrc, int64_t src_stride, int s,
+                      int row0, const int *pos, int KD);
+int launch_kvp_gather(float *dst, const float *const *pages, int rows, int KD);
+int launch_attn_paged(float *out, const float *q, const float *const *kpages, const float *const *vpages, int start_pos,
+                      const int *pos, int H, int Hkv, int Dh);
 int launch_kvq_append(void *q, void *d, const float *src, int64_t src_stride, int s, int row0, const int *pos, int KD);
 int launch_kvq_dequant(float *dst, const void *q, const void *d, int rows, int KD);
 int launch_attn_q8(float *out, const float *q, const void *kq, const void *kd, const void *vq, const void *vd, int start_pos,

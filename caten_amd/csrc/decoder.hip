@@ -64,6 +64,9 @@ struct Layer {
   float *k_cache = nullptr, *v_cache = nullptr;
   // option kv_cache 1: the cache as Q8_0 rows instead (quant and scale planes; k_cache / v_cache stay null)
   void *kq = nullptr, *kdq = nullptr, *vq = nullptr, *vdq = nullptr;
+  // option kv_cache 2: the cache in pages (kvp.hip): device tables of page pointers and the host's copy of them
+  float **k_pages = nullptr, **v_pages = nullptr;
+  std::vector<float *> k_page_host, v_page_host;
   // three-launch decode layer: attn.c_proj by head and mlp.c_proj by 16-column slab (quant / scale planes)
   void *proj_hq = nullptr, *proj_hd = nullptr, *fc2_sq = nullptr, *fc2_sd = nullptr;
 };
@@ -107,6 +110,8 @@ struct Decoder {
   // KV cache kept as Q8_0 rows (kvq.hip); peek_f32: fp32 copy of one layer's cache for cthip_decoder_peek
   bool kvq = false;
   float *peek_f32 = nullptr;
+  // KV cache in pages (kvp.hip)
+  bool kvp = false;
   hipGraphExec_t g_step = nullptr, g_body = nullptr, g_multi = nullptr;
   int64_t weight_bytes = 0, vector_bytes = 0;
   std::vector<void *> owned;  // device blocks to free
@@ -214,6 +219,31 @@ static int to_wmat(Decoder *d, const std::vector<std::string> &keys, int64_t wan
   return 0;
 }
 
+// Paged cache: opens the pages that rows [0, rows) need and extends the layers' tables.  Called by the host before it
+// queues work that reaches those rows; the tables' addresses stay what the captured graphs hold.
+static int ensure_pages(Decoder *d, int rows) {
+  if (!d->kvp) return 0;
+  const cthip_decoder_config &c = d->cfg;
+  const size_t want = (size_t)(rows + kKvPageRows - 1) / kKvPageRows;
+  const size_t bytes = sizeof(float) * (size_t)kKvPageRows * kv_dim(c);
+  for (Layer &L : d->layers) {
+    const size_t have = L.k_page_host.size();
+    if (have >= want) continue;
+    for (size_t p = have; p < want; p++) {
+      float *k = nullptr, *v = nullptr;
+      int rc;
+      if ((rc = dev_alloc(d, (void **)&k, bytes))) return rc;  // zero-filled, as the dense cache starts
+      if ((rc = dev_alloc(d, (void **)&v, bytes))) return rc;
+      L.k_page_host.push_back(k);
+      L.v_page_host.push_back(v);
+    }
+    int rc;
+    if ((rc = cthip_h2d(L.k_pages + have, L.k_page_host.data() + have, sizeof(float *) * (want - have)))) return rc;
+    if ((rc = cthip_h2d(L.v_pages + have, L.v_page_host.data() + have, sizeof(float *) * (want - have)))) return rc;
+  }
+  return 0;
+}
+
 static int queue_step(Decoder *d, bool with_head, bool embed = true);
 static int queue_head(Decoder *d);
 
@@ -305,9 +335,17 @@ static int finalize(Decoder *d) {
   if (c.arch == CTHIP_ARCH_GPT2) d->vector_bytes -= 4 * (int64_t)c.max_seq * D;
 
   d->kvq = state().kv_cache == 1;
+  d->kvp = state().kv_cache == 2;
   if (d->kvq && KD % 32) return fail(CTHIP_E_UNSUPPORTED, "decoder: a Q8_0 KV cache needs rows of whole 32-element blocks, not %d", KD);
+  if (d->kvp && KD % 4) return fail(CTHIP_E_UNSUPPORTED, "decoder: a paged KV cache needs rows of a multiple of four floats, not %d", KD);
   for (int l = 0; l < c.n_layers; l++) {
     Layer &L = d->layers[l];
+    if (d->kvp) {  // tables of page pointers, all null: pages are opened as positions are reached (ensure_pages)
+      const size_t np = (size_t)(c.max_seq + kKvPageRows - 1) / kKvPageRows;
+      TRY(dev_alloc(d, (void **)&L.k_pages, sizeof(float *) * np));
+      TRY(dev_alloc(d, (void **)&L.v_pages, sizeof(float *) * np));
+      continue;
+    }
     if (d->kvq) {  // zero quants and zero scales: rows of zeros, as the fp32 cache starts
       TRY(dev_alloc(d, &L.kq, (size_t)c.max_seq * KD));
       TRY(dev_alloc(d, &L.vq, (size_t)c.max_seq * KD));
@@ -351,7 +389,7 @@ static int finalize(Decoder *d) {
     for (WMat *w : ws)
       if (w) w->stream = total > kInfinityCacheBytes / 4 * 3;
   }
-  if (c.arch == CTHIP_ARCH_GPT2 && state().decode_flow && !d->kvq) {
+  if (c.arch == CTHIP_ARCH_GPT2 && state().decode_flow && !d->kvq && !d->kvp) {
     bool ok = true;
     for (int l = 0; l < c.n_layers && ok; l++) {
       Layer &L = d->layers[l];
@@ -417,7 +455,7 @@ static int finalize(Decoder *d) {
       d->flow = true;
     }
   }
-  if (c.arch == CTHIP_ARCH_GPT2 && state().decode_fused && !d->kvq && !d->flow &&
+  if (c.arch == CTHIP_ARCH_GPT2 && state().decode_fused && !d->kvq && !d->kvp && !d->flow &&
       dec_fused_supported(d->layers[0].attn->type, d->layers[0].proj->type, d->layers[0].fc->type,
                           d->layers[0].fc2->type, D, c.n_heads, F)) {
     // the per-XCD accumulators assume what gfx950 has: XCD ids 0..7
@@ -442,7 +480,7 @@ static int finalize(Decoder *d) {
       TRY(dev_alloc(d, (void **)&d->pmlp, sizeof(long long) * (size_t)kDecXcds * D));
     }
   }
-  if (c.arch == CTHIP_ARCH_LLAMA && state().decode_fused && !d->kvq &&
+  if (c.arch == CTHIP_ARCH_LLAMA && state().decode_fused && !d->kvq && !d->kvp &&
       gqa_fused_supported(d->layers[0].attn->type, d->layers[0].proj->type, d->layers[0].fc->type, d->layers[0].fc2->type,
                           D, c.n_heads, c.n_kv_heads, F)) {
     int max_id = -1;
@@ -662,7 +700,7 @@ static int queue_step(Decoder *d, bool with_head, bool embed) {
     a.split2 = D + KD;
     a.x_stride = D;
     a.y_stride = D;
-    if (gpt2 && !d->kvq) {
+    if (gpt2 && !d->kvq && !d->kvp) {
       a.y1 = L.k_cache;
       a.y2 = L.v_cache;
       a.pos = pos;
@@ -684,6 +722,15 @@ static int queue_step(Decoder *d, bool with_head, bool embed) {
       TRY(launch_kvq_append(L.kq, L.kdq, d->kv_tmp, KD, 1, 0, pos, KD));
       TRY(launch_kvq_append(L.vq, L.vdq, d->kv_tmp + KD, KD, 1, 0, pos, KD));
       TRY(launch_attn_q8(d->att, d->q, L.kq, L.kdq, L.vq, L.vdq, 0, pos, c.n_heads, c.n_kv_heads, Dh));
+    } else if (d->kvp) {
+      // the new row is in kv_tmp (k then v): rotate q and k where the model rotates, copy the row into its page,
+      // attend over the pages
+      if (!gpt2) {
+        TRY(launch_rope(d->q, d->q, 1, 1, c.n_heads, Dh, c.rope_base, 0, pos));
+        TRY(launch_rope(d->kv_tmp, d->kv_tmp, 1, 1, c.n_kv_heads, Dh, c.rope_base, 0, pos));
+      }
+      TRY(launch_kvp_append(L.k_pages, L.v_pages, d->kv_tmp, d->kv_tmp + KD, KD, 1, 0, pos, KD));
+      TRY(launch_attn_paged(d->att, d->q, L.k_pages, L.v_pages, 0, pos, c.n_heads, c.n_kv_heads, Dh));
     } else if (!gpt2) {
       // q and the new key are rotated inside the attention launch, which also appends k / v at `pos`
       TRY(launch_attn_rope_append(d->att, d->q, L.k_cache, L.v_cache, d->kv_tmp, pos, c.n_heads, c.n_kv_heads, Dh,
@@ -794,7 +841,7 @@ static int prefill(Decoder *d, const int *ids, int s, int n) {
   TRY(alloc((void **)&ATT, sizeof(float) * (size_t)s * D));
   TRY(alloc((void **)&Hb, sizeof(float) * (size_t)s * HW));
   if (!gpt2) TRY(alloc((void **)&G, sizeof(float) * (size_t)s * F));
-  if (d->kvq) {
+  if (d->kvq || d->kvp) {
     TRY(alloc((void **)&KF, sizeof(float) * (size_t)(n + s) * KD));
     TRY(alloc((void **)&VF, sizeof(float) * (size_t)(n + s) * KD));
   }
@@ -842,6 +889,15 @@ static int prefill(Decoder *d, const int *ids, int s, int n) {
         TRY(launch_qkv_split(Q, KF, VF, QKV, s, n, c.n_heads, c.n_kv_heads, Dh, gpt2 ? 0.0f : c.rope_base));
         TRY(launch_kvq_append(L.kq, L.kdq, KF + (int64_t)n * KD, KD, s, n, nullptr, KD));
         TRY(launch_kvq_append(L.vq, L.vdq, VF + (int64_t)n * KD, KD, s, n, nullptr, KD));
+        TRY(launch_attn(ATT, Q, KF, VF, s, n, nullptr, n + s, c.n_heads, c.n_kv_heads, Dh));
+      } else if (d->kvp) {
+        // attention of a prompt batch runs on dense rows: the cached rows [0, n) are gathered out of their pages, the
+        // batch's rows [n, n + s) join them (rotated where the model rotates) and are copied into their pages
+        TRY(launch_kvp_gather(KF, L.k_pages, n, KD));
+        TRY(launch_kvp_gather(VF, L.v_pages, n, KD));
+        TRY(launch_linear_gemm(QKV, L.attn, XN, s, L.attn_b, nullptr, CTHIP_ACT_NONE, prec));
+        TRY(launch_qkv_split(Q, KF, VF, QKV, s, n, c.n_heads, c.n_kv_heads, Dh, gpt2 ? 0.0f : c.rope_base));
+        TRY(launch_kvp_append(L.k_pages, L.v_pages, KF + (int64_t)n * KD, VF + (int64_t)n * KD, KD, s, n, nullptr, KD));
         TRY(launch_attn(ATT, Q, KF, VF, s, n, nullptr, n + s, c.n_heads, c.n_kv_heads, Dh));
       } else {
       if (gpt2 && D % 128 == 0 && KD % 128 == 0) {
@@ -1007,6 +1063,7 @@ int cthip_decoder_forward(void *dec, const float *tokens, int s, int n, int64_t 
                 n + s - 1, c.max_seq);
   int rc = finalize(d);
   if (rc) return rc;
+  if ((rc = ensure_pages(d, n + s))) return rc;
   int zero = 0;
   if ((rc = cthip_h2d(d->hist_n, &zero, sizeof(int)))) return rc;
   {
@@ -1046,6 +1103,7 @@ static int generate_impl(Decoder *d, int steps, int eos, int64_t *tokens_out, in
   if (n_generated) *n_generated = 0;
   if (steps == 0) return 0;
   int rc, zero = 0;
+  if ((rc = ensure_pages(d, d->position + steps))) return rc;
   if ((rc = cthip_h2d(d->hist_n, &zero, sizeof(int)))) return rc;
   const int ctrl[2] = {eos, 0};
   if ((rc = cthip_h2d(d->ctrl, ctrl, sizeof(ctrl)))) return rc;
@@ -1105,6 +1163,7 @@ int cthip_decoder_layer_launches(void *dec) {
   if (rc) return -1;
   if (d->flow) return 1;  // all layers are ONE launch
   if (d->fused || d->fused_gqa) return 3;
+  if (d->kvp) return d->cfg.arch == CTHIP_ARCH_GPT2 ? 6 : 8;  // + one append (+ two rotations) around the attention launch
   if (d->kvq) return d->cfg.arch == CTHIP_ARCH_GPT2 ? 7 : 9;  // + two appends (+ two rotations) around the attention launch
   return 5;
 }
@@ -1144,7 +1203,14 @@ int cthip_decoder_peek(void *dec, const char *what, void **ptr, int64_t *n_float
   } else if ((sscanf(what, "k_cache.%d", &l) == 1 || sscanf(what, "v_cache.%d", &l) == 1) && l >= 0 && l < c.n_layers) {
     const bool key = what[0] == 'k';
     n = (int64_t)c.max_seq * kv_dim(c);
-    if (d->kvq) {
+    if (d->kvp) {
+      // pages: what the caller gets is the rows as one dense array (zeros where no page has been opened), in a buffer
+      // that the next peek overwrites
+      if (!d->peek_f32 && (rc = dev_alloc(d, (void **)&d->peek_f32, sizeof(float) * (size_t)n))) return rc;
+      const Layer &L = d->layers[l];
+      if ((rc = launch_kvp_gather(d->peek_f32, key ? L.k_pages : L.v_pages, c.max_seq, kv_dim(c)))) return rc;
+      p = d->peek_f32;
+    } else if (d->kvq) {
       // Q8_0 rows: what the caller gets is their fp32 value, in a buffer that the next peek overwrites
       if (!d->peek_f32 && (rc = dev_alloc(d, (void **)&d->peek_f32, sizeof(float) * (size_t)n))) return rc;
       const Layer &L = d->layers[l];

@@ -1,0 +1,223 @@
+// KV cache kept in pages (option "kv_cache" 2).  The reference allocates its cache densely and once, `(B, max_len, H,
+// Dh)` zeros (external/llm/layers.lisp:19-33), so a session holds max_len rows per layer whether it ever reaches them
+// or not.  Here a session can instead hold pages of kKvPageRows rows that are opened when the position first
+// reaches them: per layer a table of page pointers in device memory (`pages[row / 64] + (row % 64) * KD`), which the
+// host extends before it queues the steps that need the rows.  The table's address never changes, so captured graphs
+// stay valid while the cache grows.  Rows are fp32, as in the reference: results are those of the dense cache bit for
+// bit wherever the arithmetic is the same (the attention below adds in the order of k_attn_cached).
+#include <type_traits>
+
+#include "common.h"
+
+namespace cthip {
+
+__device__ __forceinline__ const float *kvp_row(const float *const *pages, int row, int KD) {
+  return pages[row / kKvPageRows] + (int64_t)(row % kKvPageRows) * KD;
+}
+
+// ---- append: fp32 rows -> cache rows [row0 + pos, row0 + pos + s) of the key pages and of the value pages ----
+__global__ __launch_bounds__(256) void k_kvp_append(float *const *__restrict__ kpages, float *const *__restrict__ vpages,
+                                                    const float *__restrict__ ksrc, const float *__restrict__ vsrc,
+                                                    int64_t src_stride, int s, int row0, const int *__restrict__ pos, int KD) {
+  const int n4 = KD / 4;
+  const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (e >= (int64_t)s * n4) return;
+  const int i = (int)(e / n4), c = (int)(e % n4);
+  const int row = row0 + (pos ? pos[0] : 0) + i;
+  float *kd = kpages[row / kKvPageRows] + (int64_t)(row % kKvPageRows) * KD;
+  float *vd = vpages[row / kKvPageRows] + (int64_t)(row % kKvPageRows) * KD;
+  ((float4 *)kd)[c] = ((const float4 *)(ksrc + (int64_t)i * src_stride))[c];
+  ((float4 *)vd)[c] = ((const float4 *)(vsrc + (int64_t)i * src_stride))[c];
+}
+
+// ---- rows [0, t) as one dense array (prompt batches attend over dense rows; rows of pages not opened yet are zero) ----
+__global__ __launch_bounds__(256) void k_kvp_gather(float *__restrict__ dst, const float *const *__restrict__ pages, int64_t n4, int KD) {
+  const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (e >= n4) return;
+  const int kd4 = KD / 4;
+  const int row = (int)(e / kd4), c = (int)(e % kd4);
+  const float *page = pages[row / kKvPageRows];
+  ((float4 *)dst)[e] = page ? ((const float4 *)(page + (int64_t)(row % kKvPageRows) * KD))[c] : make_float4(0.f, 0.f, 0.f, 0.f);
+}
+
+// ---- one query row per head over cache rows 0..T-1 (T = start_pos + pos + 1), GQA ----
+// The lane layout of k_attn_cached (rowops.hip): a key row of a head is read by DH/4 adjacent lanes as one float4
+// each, a wavefront holds KPT passes of K and V (all page pointers requested first, then all rows: two memory
+// round trips a tile instead of one), online softmax per wavefront, one meeting in LDS.
+template <int DH>
+__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)))
+void k_attn_cached_paged(float *__restrict__ out, const float *__restrict__ q, const float *const *__restrict__ kpages,
+                         const float *const *__restrict__ vpages, int start_pos, const int *__restrict__ pos, int H, int Hkv) {
+  constexpr int LPK = DH / 4, KPW = 64 / LPK, KPT = 4, NW = 16, TILE = NW * KPW * KPT;
+  __shared__ float part[NW][DH];
+  __shared__ float pm[NW], pl[NW];
+  const int h = blockIdx.x;
+  const int T = start_pos + (pos ? pos[0] : 0) + 1;
+  const int hk = h / (H / Hkv);
+  const int KD = Hkv * DH;
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int g = lane / LPK, c = lane % LPK;
+  const float4 q4 = *(const float4 *)(q + (int64_t)h * DH + 4 * c);
+  const float scale = 1.0f / sqrtf((float)DH);
+  float m = -INFINITY, l = 0.0f;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  auto tile = [&](auto np_tag, int t0) {
+    constexpr int NP = decltype(np_tag)::value;
+    const float *kpg[NP], *vpg[NP];
+    unsigned off[NP];
+#pragma unroll
+    for (int u = 0; u < NP; u++) {
+      const int j = t0 + (wv * NP + u) * KPW + g;
+      const int jj = min(j, T - 1);  // clamped: masked below, never a row that has no page yet
+      kpg[u] = kpages[jj / kKvPageRows];
+      vpg[u] = vpages[jj / kKvPageRows];
+      off[u] = (unsigned)(jj % kKvPageRows) * (unsigned)KD + (unsigned)(hk * DH + 4 * c);
+    }
+    float4 kr[NP], vr[NP];
+#pragma unroll
+    for (int u = 0; u < NP; u++) {
+      kr[u] = *(const float4 *)(kpg[u] + off[u]);
+      vr[u] = *(const float4 *)(vpg[u] + off[u]);
+    }
+    float sc[NP];
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < NP; u++) {
+      float d = q4.x * kr[u].x;
+      d = fmaf(q4.y, kr[u].y, d);
+      d = fmaf(q4.z, kr[u].z, d);
+      d = fmaf(q4.w, kr[u].w, d);
+      if (LPK == 16) {
+        d = row16_sum(d);
+      } else {
+#pragma unroll
+        for (int o = LPK / 2; o > 0; o >>= 1) d += __shfl_xor(d, o, 64);
+      }
+      const bool ok = (t0 + (wv * NP + u) * KPW + g) < T;
+      sc[u] = ok ? d * scale : -INFINITY;
+      tmax = fmaxf(tmax, sc[u]);
+    }
+    if (LPK == 16) {
+      tmax = groups16_max(tmax);
+    } else {
+#pragma unroll
+      for (int o = LPK; o < 64; o <<= 1) tmax = fmaxf(tmax, __shfl_xor(tmax, o, 64));
+    }
+    const float m_new = fmaxf(m, tmax);   // finite: this wavefront has at least one key here
+    const float corr = ct_exp(m - m_new);  // 0 on its first tile (m = -inf)
+    float ps = 0.0f;
+#pragma unroll
+    for (int k2 = 0; k2 < 4; k2++) acc[k2] *= corr;
+#pragma unroll
+    for (int u = 0; u < NP; u++) {
+      const float p = ct_exp(sc[u] - m_new);  // exp2(-inf) = 0 for masked keys
+      ps += p;
+      acc[0] = fmaf(p, vr[u].x, acc[0]);
+      acc[1] = fmaf(p, vr[u].y, acc[1]);
+      acc[2] = fmaf(p, vr[u].z, acc[2]);
+      acc[3] = fmaf(p, vr[u].w, acc[3]);
+    }
+    if (LPK == 16) {  // every lane of a key holds the same p
+      ps = groups16_sum(ps);
+    } else {
+#pragma unroll
+      for (int o = LPK; o < 64; o <<= 1) ps += __shfl_xor(ps, o, 64);
+    }
+    l = l * corr + ps;
+    m = m_new;
+  };
+  if (T <= TILE) {
+    if (wv * KPT * KPW < T) tile(std::integral_constant<int, KPT>(), 0);  // (uniform per wavefront)
+  } else {
+    for (int t0 = 0; t0 < T; t0 += 2 * TILE) {
+      if (t0 + wv * 2 * KPT * KPW >= T) break;  // nothing left for this wavefront (uniform)
+      tile(std::integral_constant<int, 2 * KPT>(), t0);
+    }
+  }
+#pragma unroll
+  for (int o = LPK; o < 64; o <<= 1) {
+#pragma unroll
+    for (int k2 = 0; k2 < 4; k2++) acc[k2] += __shfl_xor(acc[k2], o, 64);
+  }
+  if (lane < LPK) {
+#pragma unroll
+    for (int k2 = 0; k2 < 4; k2++) part[wv][4 * lane + k2] = acc[k2];
+  }
+  if (lane == 0) {
+    pm[wv] = m;
+    pl[wv] = l;
+  }
+  __syncthreads();
+  if (tid < DH) {
+    float M = pm[0];
+#pragma unroll
+    for (int w = 1; w < NW; w++) M = fmaxf(M, pm[w]);
+    float o = 0.0f, L = 0.0f;
+#pragma unroll
+    for (int w = 0; w < NW; w++) {
+      const float e = ct_exp(pm[w] - M);  // wavefronts without keys hold m = -inf: weight 0
+      o = fmaf(e, part[w][tid], o);
+      L = fmaf(e, pl[w], L);
+    }
+    out[(int64_t)h * DH + tid] = o / L;
+  }
+}
+
+int launch_kvp_append(float *const *kpages, float *const *vpages, const float *ksrc, const float *vsrc, int64_t src_stride, int s,
+                      int row0, const int *pos, int KD) {
+  if (s == 0) return 0;
+  if (KD % 4) return fail(CTHIP_E_BAD_ARG, "paged KV cache: rows of %d floats are not a multiple of four", KD);
+  const int64_t n = (int64_t)s * (KD / 4);
+  hipLaunchKernelGGL(k_kvp_append, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, state().stream, kpages, vpages, ksrc, vsrc,
+                     src_stride, s, row0, pos, KD);
+  CTHIP_LAUNCH_CHECK();
+  return 0;
+}
+
+int launch_kvp_gather(float *dst, const float *const *pages, int rows, int KD) {
+  if (rows == 0) return 0;
+  const int64_t n4 = (int64_t)rows * (KD / 4);
+  hipLaunchKernelGGL(k_kvp_gather, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, state().stream, dst, pages, n4, KD);
+  CTHIP_LAUNCH_CHECK();
+  return 0;
+}
+
+int launch_attn_paged(float *out, const float *q, const float *const *kpages, const float *const *vpages, int start_pos,
+                      const int *pos, int H, int Hkv, int Dh) {
+  dim3 grid(H), block(1024);
+  hipStream_t st = state().stream;
+  switch (Dh) {
+    case 32: hipLaunchKernelGGL((k_attn_cached_paged<32>), grid, block, 0, st, out, q, kpages, vpages, start_pos, pos, H, Hkv); break;
+    case 64: hipLaunchKernelGGL((k_attn_cached_paged<64>), grid, block, 0, st, out, q, kpages, vpages, start_pos, pos, H, Hkv); break;
+    case 128: hipLaunchKernelGGL((k_attn_cached_paged<128>), grid, block, 0, st, out, q, kpages, vpages, start_pos, pos, H, Hkv); break;
+    default: return fail(CTHIP_E_UNSUPPORTED, "attention: head_dim %d (supported: 32, 64, 128)", Dh);
+  }
+  CTHIP_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // namespace cthip
+
+using namespace cthip;
+
+extern "C" {
+
+int cthip_kv_page_rows(void) { return kKvPageRows; }
+
+int cthip_kv_append_paged(void *const *k_pages, void *const *v_pages, const float *k_rows, const float *v_rows, int s, int row0,
+                          int kv_dim) {
+  CTHIP_REQUIRE_INIT();
+  CTHIP_ARG(s >= 0 && row0 >= 0 && kv_dim > 0 && kv_dim % 4 == 0);
+  CTHIP_ARG(s == 0 || (k_pages && v_pages && k_rows && v_rows));
+  return launch_kvp_append((float *const *)k_pages, (float *const *)v_pages, k_rows, v_rows, kv_dim, s, row0, nullptr, kv_dim);
+}
+
+int cthip_sdpa_cached_paged(float *out, const float *q, const void *const *k_pages, const void *const *v_pages, int T, int H, int Hkv,
+                            int Dh) {
+  CTHIP_REQUIRE_INIT();
+  CTHIP_ARG(T >= 1 && H > 0 && Hkv > 0 && H % Hkv == 0);
+  CTHIP_ARG(out && q && k_pages && v_pages);
+  return launch_attn_paged(out, q, (const float *const *)k_pages, (const float *const *)v_pages, T - 1, nullptr, H, Hkv, Dh);
+}
+
+}  // extern "C"

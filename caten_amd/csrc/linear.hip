@@ -679,7 +679,7 @@ int cthip_set_option(const char *name, int value) {
     return 0;
   }
   if (!strcmp(name, "kv_cache")) {
-    if (value != 0 && value != 1) return fail(CTHIP_E_BAD_ARG, "cthip_set_option: kv_cache is 0 (fp32 rows) or 1 (Q8_0 rows)");
+    if (value < 0 || value > 2) return fail(CTHIP_E_BAD_ARG, "cthip_set_option: kv_cache is 0 (fp32 rows), 1 (Q8_0 rows) or 2 (fp32 rows in pages)");
     state().kv_cache = value;
     return 0;
   }

@@ -255,6 +255,9 @@ int cthip_linear(float *y, const void *wmat, const float *x, int m, const float 
  *   scale per cache row, quantised once when the row is appended): 3.76x fewer cache bytes held and read per
  *   step.  Such a session runs one launch per Linear; logits stay within rtol 2e-2 / atol 2e-2 of the fp32
  *   cache's on the tested models (the band of 8-bit keys and values, not of the fp32 arithmetic around them).
+ *   2 = fp32 rows in pages of cthip_kv_page_rows() rows per layer, opened when the position first reaches them
+ *   (a session then holds the rows it has used instead of max_seq rows); such a session runs one launch per
+ *   Linear; tokens and logits are those of the dense cache.
  * "decode_skip": knock-out timing of the three-launch decode step -- a mask of launches a session created
  *   afterwards leaves out (1 qkv, 2 attention + projection, 4 MLP, 8 the sum in front of lm_head,
  *   16 lm_head + argmax).  Tokens and logits of such a session are meaningless; 0 (default) = none.
@@ -320,6 +323,16 @@ int cthip_sdpa_cached(float *out, const float *q, const float *k_cache, const fl
 int cthip_kv_append_q8(void *q_plane, void *d_plane, const float *rows, int s, int row0, int kv_dim);
 int cthip_sdpa_cached_q8(float *out, const float *q, const void *k_q, const void *k_d, const void *v_q, const void *v_d, int T,
                          int H, int Hkv, int Dh);
+/* The same cache in pages (the reference allocates (B, max_len, H, Dh) once, layers.lisp:25-26): row r lives at
+ * pages[r / cthip_kv_page_rows()] + (r % cthip_kv_page_rows()) * kv_dim, `pages` a device array of device pointers
+ * that the owner extends as positions are reached.  cthip_kv_append_paged copies `s` fp32 key rows and value rows
+ * (s, kv_dim) into rows row0 .. row0+s-1 of the key pages and the value pages; cthip_sdpa_cached_paged attends ONE
+ * query row (H, Dh) over rows 0 .. T-1, out (H, Dh), with the arithmetic of cthip_sdpa_cached. */
+int cthip_kv_page_rows(void);
+int cthip_kv_append_paged(void *const *k_pages, void *const *v_pages, const float *k_rows, const float *v_rows, int s, int row0,
+                          int kv_dim);
+int cthip_sdpa_cached_paged(float *out, const float *q, const void *const *k_pages, const void *const *v_pages, int T, int H, int Hkv,
+                            int Dh);
 
 /* ================================================================== */
 /* Decoder session: Transformer (external/llm/layers.lisp:73-90) and   */

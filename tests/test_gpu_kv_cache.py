@@ -131,3 +131,107 @@ def test_three_launch_layer_is_what_supported_shapes_run():
     m = llm.make_llama(cfg, llm.llama_state_dict(synth.llama_weights(cfg, seed=1), "q4_0"))
     assert lib.cthip_decoder_layer_launches(m.handle) == 3
     m.close()
+
+
+@pytest.mark.parametrize("H,Hkv,Dh", [(4, 4, 64), (8, 2, 64), (4, 2, 32), (2, 1, 128)])
+def test_append_and_attention_over_paged_rows(oracle, H, Hkv, Dh):
+    """The cache in pages (option "kv_cache" 2; the reference allocates max_len rows at once, layers.lisp:25-26): rows
+    appended through the page table come back from it, and one query row over the pages gives, bit for bit, what
+    cthip_sdpa_cached gives over the same rows laid out densely -- and the oracle's attention inside rtol 1e-3 /
+    atol 1e-4."""
+    print(f"case: paged cache rows H {H} Hkv {Hkv} Dh {Dh}", flush=True)
+    import ctypes as C
+    from caten_amd import _lib
+    from caten_amd.ops import DeviceArray
+    lib = _lib.init()
+    P = lib.cthip_kv_page_rows()
+    assert P == 64
+    KD, L = Hkv * Dh, 600
+    npages = (L + P - 1) // P
+    rng = np.random.default_rng(H * 11 + Dh)
+    k = rng.standard_normal((L, KD)).astype(np.float32)
+    v = rng.standard_normal((L, KD)).astype(np.float32)
+    # pages in scrambled order, as an allocator hands them out
+    order = rng.permutation(npages)
+    kpool, vpool = DeviceArray((npages, P, KD), np.float32), DeviceArray((npages, P, KD), np.float32)
+    ktab = np.array([kpool.ptr + 4 * int(order[p]) * P * KD for p in range(npages)], np.uint64)
+    vtab = np.array([vpool.ptr + 4 * int(order[p]) * P * KD for p in range(npages)], np.uint64)
+    dkt, dvt = DeviceArray.from_numpy(ktab), DeviceArray.from_numpy(vtab)
+    dk, dv = DeviceArray.from_numpy(k), DeviceArray.from_numpy(v)
+    for row0, s in ((0, 17), (17, 1), (18, 1), (19, 45), (64, 1), (65, L - 65)):  # pieces that end on, and cross, page edges
+        _lib.check(lib.cthip_kv_append_paged(dkt.ptr, dvt.ptr, dk.ptr + 4 * row0 * KD, dv.ptr + 4 * row0 * KD, s, row0, KD))
+    got_k = kpool.numpy()[order].reshape(npages * P, KD)[:L]
+    got_v = vpool.numpy()[order].reshape(npages * P, KD)[:L]
+    assert np.array_equal(got_k, k) and np.array_equal(got_v, v)
+    out, ref = DeviceArray((H, Dh), np.float32), DeviceArray((H, Dh), np.float32)
+    for T in (1, 2, 63, 64, 65, 255, 256, 257, 600):
+        q = rng.standard_normal((1, H, Dh)).astype(np.float32)
+        dq_ = DeviceArray.from_numpy(q)
+        _lib.check(lib.cthip_sdpa_cached_paged(out.ptr, dq_.ptr, dkt.ptr, dvt.ptr, T, H, Hkv, Dh))
+        _lib.check(lib.cthip_sdpa_cached(ref.ptr, dq_.ptr, dk.ptr, dv.ptr, 1, T - 1, H, Hkv, Dh))
+        got = out.numpy()
+        assert np.array_equal(got, ref.numpy()), T
+        want = oracle.sdpa(q, k[:T].reshape(T, Hkv, Dh), v[:T].reshape(T, Hkv, Dh))[0]
+        assert np.allclose(got, want, rtol=1e-3, atol=1e-4), (T, float(np.max(np.abs(got - want))))
+
+
+@pytest.mark.parametrize("arch,plen", [("gpt2", 3), ("gpt2", 70), ("llama", 3), ("llama", 70)])
+def test_decoder_with_a_paged_cache_equals_the_dense_cache(arch, plen):
+    """A session whose cache lives in pages against one with the dense cache, both with one launch per Linear: a prompt
+    fed row by row or as one batch that crosses a page edge, then decode steps across another edge.  Same tokens; for
+    the GPT-2 shape the same logits and cache rows bit for bit (the arithmetic is the same); where the model rotates,
+    q and k are rotated by a launch of their own instead of inside the attention launch, so logits are compared inside
+    the fp32 band (rtol 1e-3 / atol 1e-4).  The paged session holds the rows it has reached, not max_seq rows."""
+    print(f"case: decoder with paged cache {arch} prompt {plen}", flush=True)
+    import ctypes as C
+    from caten_amd import _lib, synth, llm
+    lib = _lib.init()
+    if arch == "gpt2":
+        cfg = dict(synth.GPT2_CONFIGS["gpt2-tiny"], max_seq=1024)
+        sd = llm.gpt2_state_dict(synth.gpt2_weights(cfg, seed=23), "q8_0")
+        make = llm.make_gpt2
+    else:
+        cfg = dict(synth.LLAMA_CONFIGS["llama-tiny"], max_seq=1024)
+        sd = llm.llama_state_dict(synth.llama_weights(cfg, seed=23), "q4_0")
+        make = llm.make_llama
+    prompt = synth.prompt(cfg["vocab"], plen, seed=23)
+    kd = cfg["dim"] // cfg["n_heads"] * cfg.get("n_kv_heads", cfg["n_heads"])
+    steps = 70
+    runs = {}
+    live = C.c_size_t()
+    try:
+        _lib.check(lib.cthip_set_option(b"decode_fused", 0))
+        for mode in (0, 2):
+            _lib.check(lib.cthip_set_option(b"kv_cache", mode))
+            _lib.check(lib.cthip_cache_stats(C.byref(live), None, None))
+            before = live.value
+            m = make(cfg, sd)
+            toks, logs = llm.gpt2_generate(m, prompt, steps, on_device=False, keep_logits=True)
+            _lib.check(lib.cthip_cache_stats(C.byref(live), None, None))
+            held = live.value - before
+            n_rows = plen + steps - 1
+            k0 = m.peek("k_cache.0").reshape(cfg["max_seq"], kd).copy()
+            vl = m.peek(f"v_cache.{cfg['n_layers'] - 1}").reshape(cfg["max_seq"], kd).copy()
+            launches = lib.cthip_decoder_layer_launches(m.handle)
+            m.close()
+            m = make(cfg, sd)
+            assert llm.gpt2_generate(m, prompt, steps, on_device=True) == toks  # the device-resident loop, pages opened ahead
+            m.close()
+            runs[mode] = (toks, logs, k0, vl, launches, held, n_rows)
+    finally:
+        _lib.check(lib.cthip_set_option(b"kv_cache", 0))
+        _lib.check(lib.cthip_set_option(b"decode_fused", 1))
+    (t0, l0, k0, v0, n0, held0, n_rows), (t2, l2, k2, v2, n2, held2, _) = runs[0], runs[2]
+    assert t0 == t2
+    assert n0 == 5 and n2 == (6 if arch == "gpt2" else 8)
+    if arch == "gpt2":
+        assert all(np.array_equal(a, b) for a, b in zip(l0, l2))
+        assert np.array_equal(k0, k2) and np.array_equal(v0, v2)
+    else:
+        for a, b in zip(l0, l2):
+            assert np.allclose(b, a, rtol=1e-3, atol=1e-4), float(np.max(np.abs(a - b)))
+        assert np.allclose(k2[:n_rows], k0[:n_rows], rtol=1e-5, atol=1e-6) and np.array_equal(v0, v2)
+    assert not k2[n_rows:].any()  # rows never reached read as zeros, as the dense cache holds them
+    # the dense session holds max_seq rows per layer, the paged one three pages (139 or 72 rows reached)
+    dense_rows = 2 * cfg["n_layers"] * cfg["max_seq"] * kd * 4
+    assert held0 - held2 > dense_rows // 2, (held0, held2, dense_rows)

@@ -539,6 +539,77 @@ __global__ __launch_bounds__(1024) void k_argmax(int64_t *__restrict__ out, cons
   }
 }
 
+// A few long rows (the logits of a decode step: one row of 50 257): one block per row reads its row alone, a
+// memory round trip per 1024 elements.  Here kArgmaxParts blocks per row each reduce a contiguous part ...
+constexpr int kArgmaxParts = 64;
+__global__ __launch_bounds__(256) void k_argmax_parts(float *__restrict__ pv, int *__restrict__ pi, const float *__restrict__ x, int n) {
+  __shared__ float sm[4];
+  __shared__ int si[4];
+  const int row = blockIdx.x, part = blockIdx.y;
+  const int per = (n + kArgmaxParts - 1) / kArgmaxParts;
+  const int lo = part * per, hi = min(n, lo + per);
+  const float *__restrict__ xr = x + (int64_t)row * n;
+  float best = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int i = lo + threadIdx.x; i < hi; i += 256) {
+    const float v = xr[i];
+    if (v > best || (v == best && i < bi)) {
+      best = v;
+      bi = i;
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ob = __shfl_xor(best, o, 64);
+    const int oi = __shfl_xor(bi, o, 64);
+    if (ob > best || (ob == best && oi < bi)) {
+      best = ob;
+      bi = oi;
+    }
+  }
+  if ((threadIdx.x & 63) == 0) {
+    sm[threadIdx.x >> 6] = best;
+    si[threadIdx.x >> 6] = bi;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int k = 1; k < 4; k++)
+      if (sm[k] > best || (sm[k] == best && si[k] < bi)) {
+        best = sm[k];
+        bi = si[k];
+      }
+    pv[row * kArgmaxParts + part] = best;
+    pi[row * kArgmaxParts + part] = bi;
+  }
+}
+// ... and one wavefront per row settles the parts (lowest index among equal maxima, as k_argmax).
+__global__ __launch_bounds__(64) void k_argmax_settle(int64_t *__restrict__ out, const float *__restrict__ pv, const int *__restrict__ pi,
+                                                      int *__restrict__ tok_out, int *__restrict__ pos,
+                                                      int64_t *__restrict__ history, int *__restrict__ hist_n) {
+  const int row = blockIdx.x;
+  float best = pv[row * kArgmaxParts + threadIdx.x];
+  int bi = pi[row * kArgmaxParts + threadIdx.x];
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ob = __shfl_xor(best, o, 64);
+    const int oi = __shfl_xor(bi, o, 64);
+    if (ob > best || (ob == best && oi < bi)) {
+      best = ob;
+      bi = oi;
+    }
+  }
+  if (threadIdx.x == 0) {
+    if (bi == 0x7fffffff) bi = 0;  // all-NaN / empty row
+    out[row] = bi;
+    if (tok_out) *tok_out = bi;
+    if (history) {
+      history[*hist_n] = bi;
+      *hist_n = *hist_n + 1;
+    }
+    if (pos) *pos = *pos + 1;
+  }
+}
+
 // RoPE on (B,S,H,Dh), one thread per (pair)
 __global__ __launch_bounds__(256) void k_rope(float *__restrict__ out, const float *__restrict__ x, int64_t npairs,
                                               int S, int H, int Dh, float log2_base, int start_pos,
@@ -1340,6 +1411,22 @@ int launch_embedding_rows(float *out, const float *W, long long first, long long
 int launch_argmax(int64_t *out, const float *x, int64_t rows, int n, int *tok_out, int *pos, int64_t *history,
                   int *hist_n) {
   if (rows == 0) return 0;
+  static_assert(kArgmaxParts == 64, "k_argmax_settle reads one part per lane");
+  if (rows <= 16 && n >= 8192) {  // few long rows: parts of a row in parallel, then one wavefront per row
+    float *pv = nullptr;
+    int rc = alloc_scratch((void **)&pv, (size_t)rows * kArgmaxParts * 8);
+    if (rc) return rc;
+    int *pi = (int *)(pv + rows * kArgmaxParts);
+    hipLaunchKernelGGL(k_argmax_parts, dim3((unsigned)rows, kArgmaxParts), dim3(256), 0, state().stream, pv, pi, x, n);
+    hipError_t e = hipGetLastError();
+    if (e == hipSuccess) {
+      hipLaunchKernelGGL(k_argmax_settle, dim3((unsigned)rows), dim3(64), 0, state().stream, out, pv, pi, tok_out, pos, history, hist_n);
+      e = hipGetLastError();
+    }
+    rc = cthip_free(pv);  // stream-ordered: handed out again only to later work on this stream
+    if (e != hipSuccess) return fail((int)e, "argmax: launch -> %s", hipGetErrorString(e));
+    return rc;
+  }
   hipLaunchKernelGGL(k_argmax, dim3((unsigned)rows), dim3(1024), 0, state().stream, out, x, n, tok_out, pos, history,
                      hist_n);
   CTHIP_LAUNCH_CHECK();

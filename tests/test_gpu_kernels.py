@@ -395,6 +395,17 @@ def test_embedding_and_argmax(ops, oracle):
         assert ops.argmax(x) == oracle.argmax(x)
     x = rng.normal(size=(9, 50257)).astype(np.float32)
     assert np.array_equal(ops.argmax(x), np.array([oracle.argmax(r) for r in x]))
+    # few long rows are reduced in 64 parts per row, then settled: ties across parts, the maximum in the last, short
+    # part, rows of -inf and of NaN, and the sizes either side of where that path starts
+    for n in (8191, 8192, 8193, 50257, 50304):
+        x = rng.integers(0, 3, (3, n)).astype(np.float32)
+        x[1, :] = 0.0
+        x[1, n - 1] = 7.0
+        x[2, :] = -np.inf
+        assert np.array_equal(ops.argmax(x), np.array([oracle.argmax(r) for r in x])), n
+        assert ops.argmax(np.full(n, np.nan, np.float32)) == 0
+    x = rng.normal(size=(17, 9000)).astype(np.float32)  # more rows than that path takes
+    assert np.array_equal(ops.argmax(x), np.array([oracle.argmax(r) for r in x]))
     assert ops.argmax(np.arange(10, dtype=np.float32)) == 9  # test-ops.lisp:107-114
 
 

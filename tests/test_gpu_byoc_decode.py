@@ -298,3 +298,36 @@ def test_pools_of_the_librarys_walk_keep_and_clear_storage_like_the_hosts():
             last = n
             want.append((n, [float(cur)] * n))
         assert seen == want, (native, seen)
+
+
+def test_the_librarys_walk_reports_what_the_hosts_walk_reports():
+    """a forward that leaves a shape variable unset stops at the node that needs it, wrapped as the reference's
+    runtime-error (runtime.lisp:84-104) whichever side walks the list; the entry points refuse malformed nodes"""
+    import ctypes as C
+    from caten_amd import _lib
+    from caten_amd.runtime import HipRuntime, Node, RuntimeError_
+    g = [Node("Add", ["t"], ["n", "s"]), Node("Allocate", ["y"], ["t", 1], {"nrank": 1, "dtype": "float32"})]
+    for native in (True, False):
+        rt = HipRuntime(g, fw_outputs=["y"], native=native)
+        with pytest.raises(RuntimeError_) as e:
+            rt.forward(("n", 3))  # s is never bound
+        assert "Runtime-Error" in str(e.value)
+        if native:
+            assert "vm: node 0" in str(e.value)
+        y = rt.forward(("n", 3), ("s", 2))  # the runtime is usable afterwards
+        assert y.shape == [5]
+        rt.free()
+    lib = _lib.init()
+    vm = C.c_void_p()
+    _lib.check(lib.cthip_vm_create(C.byref(vm), 4))
+    kinds, iv, fv = (C.c_int * 2)(2, 0), (C.c_longlong * 2)(1, 7), (C.c_double * 2)()
+    assert lib.cthip_vm_add_scalar(vm, 9, 0, 2, kinds, iv, fv) == _lib.E_BAD_ARG          # no such operation
+    assert lib.cthip_vm_add_scalar(vm, 2, 0, 2, kinds, iv, fv) == _lib.E_BAD_ARG          # :Neg of two operands
+    bad = (C.c_longlong * 2)(99, 7)
+    assert lib.cthip_vm_add_scalar(vm, 0, 0, 2, kinds, bad, fv) == _lib.E_BAD_ARG         # a slot that does not exist
+    assert lib.cthip_vm_add_allocate(vm, 1, 4, 9, kinds, iv) == _lib.E_BAD_ARG            # rank 9
+    assert lib.cthip_vm_set_buffer(vm, 0, None) == _lib.E_BAD_ARG
+    _lib.check(lib.cthip_vm_add_scalar(vm, 3, 0, 2, kinds, (C.c_longlong * 2)(1, 0), fv))  # slot 1 // 0
+    _lib.check(lib.cthip_vm_set_int(vm, 1, 5))
+    assert lib.cthip_vm_run(vm) == _lib.E_STATE and b"division by zero" in lib.cthip_last_error()
+    _lib.check(lib.cthip_vm_destroy(vm))

@@ -33,6 +33,12 @@ def test_calls_fail_loudly_without_init():
     assert lib.cthip_alloc(ctypes.byref(p), 16) == -1
     assert b"cthip_init" in lib.cthip_last_error()
     assert lib.cthip_softmax(None, None, 1, 4) == -1
+    # the walk of a node list and the paged cache entry points need a device too
+    assert lib.cthip_vm_create(ctypes.byref(p), 4) == -1
+    assert lib.cthip_vm_run(None) == -1
+    assert lib.cthip_kv_append_paged(None, None, None, None, 0, 0, 64) == -1
+    assert lib.cthip_kv_page_rows() == 64  # a constant of the layout: no device needed
+    assert lib.cthip_vm_launches(None) == -1 and lib.cthip_vm_destroy(None) == 0
 
 
 def test_backend_registry():

@@ -49,6 +49,7 @@ struct DecQkvArgs {
   float *q, *kc, *vc;        // q (D), K / V cache (max_seq, D)
   const int *pos;
   int rows;                  // 3D
+  int kv_stride;             // floats between cache rows: D; 0 = kc / vc are one row (the new row goes to a buffer)
 };
 
 struct DecAttnArgs {
@@ -59,6 +60,20 @@ struct DecAttnArgs {
   float *part;               // out: fp32 [H][D], head h's share of the projection
   void *zero;                // cleared here: the MLP accumulators
   int64_t zero_n16;          // ... in 16-byte units
+};
+
+// the same launch over a cache kept as Q8_0 rows (kvq.hip): the step's new key / value row arrives as fp32 (k then v,
+// D floats each), is quantised here, joins the keys as the last row and is stored into the planes
+struct DecAttnQ8Args {
+  const float *q, *newkv;
+  signed char *kq, *vq;        // quant planes int8 [max_seq][D]
+  unsigned short *kd, *vd;     // scale planes fp16 [max_seq][D / 32]
+  const int *pos;
+  const void *pq;
+  const unsigned short *pd;
+  float *part;
+  void *zero;
+  int64_t zero_n16;
 };
 
 struct DecMlpArgs {
@@ -177,6 +192,7 @@ int dec_relay_heads(const WMat *w, int DH, void **pq, void **pd);
 int dec_relay_slabs(const WMat *w, void **pq, void **pd);  // slabs of 16 columns (a whole block of 32 for Q4_0)
 int launch_dec_qkv(const DecQkvArgs &a, int type, bool from_accum);
 int launch_dec_attn_proj(const DecAttnArgs &a, int type, int H, int D, int replicas);
+int launch_dec_attn_proj_q8(const DecAttnQ8Args &a, int type, int H, int D, int replicas);
 int launch_dec_mlp(const DecMlpArgs &a, int type, int F, int H);
 int launch_dec_sum(const DecStage &s, float *out);
 

@@ -161,8 +161,8 @@ __global__ __launch_bounds__(256) void k_dec_qkv(DecQkvArgs a) {
     // rstd * (W.(gamma x) - mu * W.gamma) + (W.beta + bias)  =  W.LayerNorm(x) + bias
     const float v = rstd * (acc - mu * fs) + fc;
     if (row < D) a.q[row] = v;
-    else if (row < 2 * D) a.kc[(int64_t)posv * D + (row - D)] = v;
-    else a.vc[(int64_t)posv * D + (row - 2 * D)] = v;
+    else if (row < 2 * D) a.kc[(int64_t)posv * a.kv_stride + (row - D)] = v;
+    else a.vc[(int64_t)posv * a.kv_stride + (row - 2 * D)] = v;
   }
 }
 
@@ -310,6 +310,224 @@ void k_dec_attn_proj(DecAttnArgs a) {
   }
   __syncthreads();
   // partial projection: row r of the slab times the head's outputs; CPR lanes share a row
+  float xr[XPC];
+  lds_floats<XPC>(oh + pc * XPC, xr);
+  float xsum = 0.0f;
+  if (TYPE == CTHIP_Q4_0) {
+#pragma unroll
+    for (int t = 0; t < XPC; t++) xsum += xr[t];
+  }
+#pragma unroll
+  for (int j = 0; j < JR; j++) {
+    float s = chunk_dot<TYPE>(pw[j], DecFmt<TYPE>::QUANT ? half_bits_to_float((unsigned short)ps[j]) : 1.0f, xr, xsum);
+    if (CPR >= 2) s += dpp_f<0xB1>(s);    // quad_perm [1,0,3,2]
+    if (CPR >= 4) s += dpp_f<0x4E>(s);    // quad_perm [2,3,0,1]
+    if (CPR >= 8) s += dpp_f<0x141>(s);   // row_half_mirror
+    if (CPR >= 16) s += dpp_f<0x140>(s);  // row_mirror
+    const int r = pr0 + RPP * j;
+    if (pc == 0 && r < rr) a.part[(int64_t)h * D + rbase + r] = s;
+  }
+}
+
+// ---- launch 2 over a cache of Q8_0 rows ----
+// The attention of k_attn_cached_q8 (kvq.hip) with sixteen wavefronts: a key row of a head is 64 int8 = 4 lanes x 16
+// bytes, a wavefront covers 16 keys a pass, the products run on the integers and a block's scale is applied to its
+// partial sum.  The step's new row is quantised here as k_kvq_append quantises it (per block of 32: d = absmax / 127
+// kept as fp16, q = x / d rounded half away from zero) by the one wavefront that owns key T - 1, after it has
+// requested its other keys; it uses the row in that form and, in the head's first workgroup, stores it into the
+// planes -- the session's two append launches and its attention launch in one.
+template <int TYPE, int JR>
+__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)))
+void k_dec_attn_proj_q8(DecAttnQ8Args a) {
+  constexpr int DH = 64, LPK = DH / 16, KPW = 64 / LPK, KPT = 2, NW = 16, TILE = NW * KPW * KPT;
+  constexpr int XPC = DecFmt<TYPE>::XPC;
+  constexpr int CPR = DH / XPC, RPP = 1024 / CPR;
+  __shared__ float part[NW][DH];
+  __shared__ float pm[NW], pl[NW];
+  __shared__ __align__(16) float oh[DH];
+  const int h = blockIdx.x, H = gridDim.x, D = H * DH, nb = D / 32;
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int g = lane / LPK, c = lane % LPK;
+  const int rr = D / (int)gridDim.y, rbase = (int)blockIdx.y * rr;
+  const int pc = tid % CPR, pr0 = tid / CPR;
+  uint4 pw[JR];
+  unsigned ps[JR];
+#pragma unroll
+  for (int j = 0; j < JR; j++) {
+    int r = pr0 + RPP * j;
+    r = rbase + (r < rr ? r : rr - 1);
+    pw[j] = ((const uint4 *)a.pq)[((int64_t)h * D + r) * CPR + pc];
+    ps[j] = DecFmt<TYPE>::QUANT ? a.pd[((int64_t)h * D + r) * (DH / 32) + ((pc * XPC) >> 5)] : 0;
+  }
+  const int T = a.pos[0] + 1;
+  const int col = h * DH + 16 * c;  // first of this lane's 16 elements inside a cache row
+  float qr[16];
+#pragma unroll
+  for (int e = 0; e < 4; e++) {
+    const float4 v = *(const float4 *)(a.q + col + 4 * e);
+    qr[4 * e] = v.x, qr[4 * e + 1] = v.y, qr[4 * e + 2] = v.z, qr[4 * e + 3] = v.w;
+  }
+  // this lane's 16 elements of a new row, quantised; lanes c and c ^ 1 share a block of 32
+  auto quantise = [&](const float *src, uint4 &qv, unsigned &dv) {
+    float x[16];
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      const float4 v = *(const float4 *)(src + col + 4 * e);
+      x[4 * e] = v.x, x[4 * e + 1] = v.y, x[4 * e + 2] = v.z, x[4 * e + 3] = v.w;
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 16; e++) amax = fmaxf(amax, fabsf(x[e]));
+    amax = fmaxf(amax, dpp_f<0xB1>(amax));  // quad_perm [1,0,3,2]: the block's other half
+    const float dd = amax / 127.0f;
+    const float inv = dd != 0.0f ? 1.0f / dd : 0.0f;
+    unsigned w[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int e = 0; e < 16; e++) {
+      const float t = x[e] * inv;
+      const int r = (int)(t + copysignf(0.5f, t));  // = copysign(floor(|t| + 0.5), t): the conversion truncates
+      w[e >> 2] |= ((unsigned)r & 255u) << (8 * (e & 3));
+    }
+    qv = make_uint4(w[0], w[1], w[2], w[3]);
+    dv = __builtin_bit_cast(unsigned short, (_Float16)dd);
+  };
+  {  // the accumulators of the MLP launch are cleared here: their last reader (this layer's k_dec_qkv) has finished
+    uint4 *z = (uint4 *)a.zero;
+    const uint4 zz = make_uint4(0u, 0u, 0u, 0u);
+    const int64_t nthr = (int64_t)H * gridDim.y * 1024;
+    for (int64_t k = ((int64_t)blockIdx.y * H + h) * 1024 + tid; k < a.zero_n16; k += nthr) z[k] = zz;
+  }
+  const float scale = 1.0f / sqrtf((float)DH);
+  float m = -INFINITY, l = 0.0f;
+  float acc[16];
+#pragma unroll
+  for (int e = 0; e < 16; e++) acc[e] = 0.0f;
+  auto widen = [](const uint4 w, float *f) {
+    const uint32_t dw[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+      const int v = (int)dw[t];
+      f[4 * t + 0] = (float)(int)(int8_t)v;
+      f[4 * t + 1] = (float)(int)(int8_t)(v >> 8);
+      f[4 * t + 2] = (float)(int)(int8_t)(v >> 16);
+      f[4 * t + 3] = (float)(v >> 24);
+    }
+  };
+  // One tile = NP key passes per wavefront, all requested together: wavefront wv owns keys t0 + (wv*NP + u)*KPW + g.
+  // (tiles of four passes for long contexts, as the fp32 launch has them, do not fit 128 registers here)
+  auto tile = [&](auto np_tag, int t0) {
+    constexpr int NP = decltype(np_tag)::value;
+    uint4 kr[NP], vr[NP];
+    unsigned ks[NP], vs[NP];
+    const int j0 = t0 + wv * NP * KPW;
+#pragma unroll
+    for (int u = 0; u < NP; u++) {
+      const int j = j0 + u * KPW + g;
+      const int jj = min(j, max(T - 2, 0));  // clamped: masked below; row T - 1 is not in the planes yet
+      kr[u] = *(const uint4 *)(a.kq + (int64_t)jj * D + col);
+      vr[u] = *(const uint4 *)(a.vq + (int64_t)jj * D + col);
+      ks[u] = a.kd[(int64_t)jj * nb + (col >> 5)];
+      vs[u] = a.vd[(int64_t)jj * nb + (col >> 5)];
+    }
+    if (T - 1 >= j0 && T - 1 < j0 + NP * KPW) {  // (uniform) this wavefront owns the new row
+      uint4 knq, vnq;
+      unsigned knd, vnd;
+      quantise(a.newkv, knq, knd);
+      quantise(a.newkv + D, vnq, vnd);
+#pragma unroll
+      for (int u = 0; u < NP; u++) {
+        if (j0 + u * KPW + g == T - 1) {
+          kr[u] = knq, vr[u] = vnq, ks[u] = knd, vs[u] = vnd;
+          if (blockIdx.y == 0) {  // the `!assign` into the cache row at pos
+            *(uint4 *)(a.kq + (int64_t)(T - 1) * D + col) = knq;
+            *(uint4 *)(a.vq + (int64_t)(T - 1) * D + col) = vnq;
+            if ((c & 1) == 0) {
+              a.kd[(int64_t)(T - 1) * nb + (col >> 5)] = (unsigned short)knd;
+              a.vd[(int64_t)(T - 1) * nb + (col >> 5)] = (unsigned short)vnd;
+            }
+          }
+        }
+      }
+    }
+    float sc[NP];
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < NP; u++) {
+      float kf[16];
+      widen(kr[u], kf);
+      float dsum = 0.0f;
+#pragma unroll
+      for (int e = 0; e < 16; e++) dsum = fmaf(qr[e], kf[e], dsum);
+      dsum *= half_bits_to_float((unsigned short)ks[u]);
+      dsum += dpp_f<0xB1>(dsum);  // over the key's four lanes
+      dsum += dpp_f<0x4E>(dsum);
+      const bool ok = (j0 + u * KPW + g) < T;
+      sc[u] = ok ? dsum * scale : -INFINITY;
+      tmax = fmaxf(tmax, sc[u]);
+    }
+    tmax = wave_max(tmax);
+    const float m_new = fmaxf(m, tmax);   // finite: this wavefront has at least one key here
+    const float corr = ct_exp(m - m_new);  // 0 on its first tile (m = -inf)
+    float psum = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 16; e++) acc[e] *= corr;
+#pragma unroll
+    for (int u = 0; u < NP; u++) {
+      const float p = ct_exp(sc[u] - m_new);  // exp2(-inf) = 0 for masked keys
+      psum += p;
+      float vf[16];
+      widen(vr[u], vf);
+      const float pv = p * half_bits_to_float((unsigned short)vs[u]);
+#pragma unroll
+      for (int e = 0; e < 16; e++) acc[e] = fmaf(pv, vf[e], acc[e]);
+    }
+    psum = wave_sum(psum) * 0.25f;  // every one of a key's four lanes holds the same p
+    l = l * corr + psum;
+    m = m_new;
+  };
+  int nact;  // wavefronts that hold keys
+  if (T <= TILE) {
+    nact = (T + KPT * KPW - 1) / (KPT * KPW);
+    if (wv < nact) tile(std::integral_constant<int, KPT>(), 0);  // (uniform per wavefront)
+  } else {
+    nact = NW;
+    for (int t0 = 0; t0 < T; t0 += TILE) {
+      if (t0 + wv * KPT * KPW >= T) break;  // nothing left for this wavefront (uniform)
+      tile(std::integral_constant<int, KPT>(), t0);
+    }
+  }
+  if (wv < nact) {
+    // the sum over the wavefront's 16 key groups, halving what is exchanged each time: a lane ends with one of its 16
+    // columns, number 8 b0 + 4 b1 + 2 b2 + b3 (b = bits of g)
+    float r8[8], r4[4], r2[2], r1;
+    const bool b0 = g & 1, b1 = g & 2, b2 = g & 4, b3 = g & 8;
+#pragma unroll
+    for (int i = 0; i < 8; i++) r8[i] = (b0 ? acc[i + 8] : acc[i]) + __shfl_xor(b0 ? acc[i] : acc[i + 8], 4, 64);
+#pragma unroll
+    for (int i = 0; i < 4; i++) r4[i] = (b1 ? r8[i + 4] : r8[i]) + __shfl_xor(b1 ? r8[i] : r8[i + 4], 8, 64);
+#pragma unroll
+    for (int i = 0; i < 2; i++) r2[i] = (b2 ? r4[i + 2] : r4[i]) + __shfl_xor(b2 ? r4[i] : r4[i + 2], 16, 64);
+    r1 = (b3 ? r2[1] : r2[0]) + __shfl_xor(b3 ? r2[0] : r2[1], 32, 64);
+    part[wv][16 * c + 8 * (int)b0 + 4 * (int)b1 + 2 * (int)b2 + (int)b3] = r1;
+    if (lane == 0) {
+      pm[wv] = m;
+      pl[wv] = l;
+    }
+  }
+  __syncthreads();
+  if (tid < DH) {
+    float M = pm[0];
+    for (int w = 1; w < nact; w++) M = fmaxf(M, pm[w]);
+    float o = 0.0f, L = 0.0f;
+    for (int w = 0; w < nact; w++) {
+      const float e = ct_exp(pm[w] - M);
+      o = fmaf(e, part[w][tid], o);
+      L = fmaf(e, pl[w], L);
+    }
+    oh[tid] = o / L;
+  }
+  __syncthreads();
+  // partial projection, as in k_dec_attn_proj
   float xr[XPC];
   lds_floats<XPC>(oh + pc * XPC, xr);
   float xsum = 0.0f;
@@ -584,6 +802,27 @@ int launch_dec_attn_proj(const DecAttnArgs &a, int type, int H, int D, int repli
     case 2: hipLaunchKernelGGL((k_dec_attn_proj<T, 64, 2>), grid, block, 0, st, a); break;   \
     case 3: hipLaunchKernelGGL((k_dec_attn_proj<T, 64, 3>), grid, block, 0, st, a); break;   \
     default: hipLaunchKernelGGL((k_dec_attn_proj<T, 64, 4>), grid, block, 0, st, a); break;  \
+  }
+  DEC_TYPES(GO_T)
+#undef GO_T
+  CTHIP_LAUNCH_CHECK();
+  return 0;
+}
+
+int launch_dec_attn_proj_q8(const DecAttnQ8Args &a, int type, int H, int D, int replicas) {
+  const int xpc = type_xpc(type);
+  if (D != H * 64 || D > 1024 || replicas < 1 || D % replicas || !xpc)
+    return fail(CTHIP_E_BAD_ARG, "decoder: fused attention launch with D = %d, H = %d, %d workgroups per head", D, H, replicas);
+  dim3 grid(H, replicas), block(1024);
+  hipStream_t st = state().stream;
+  const int rpp = 1024 / (64 / xpc), jr = (D / replicas + rpp - 1) / rpp;
+  if (jr > 4) return fail(CTHIP_E_BAD_ARG, "decoder: fused attention launch needs %d passes over its slab", jr);
+#define GO_T(T)                                                                                 \
+  switch (jr) {                                                                                 \
+    case 1: hipLaunchKernelGGL((k_dec_attn_proj_q8<T, 1>), grid, block, 0, st, a); break;       \
+    case 2: hipLaunchKernelGGL((k_dec_attn_proj_q8<T, 2>), grid, block, 0, st, a); break;       \
+    case 3: hipLaunchKernelGGL((k_dec_attn_proj_q8<T, 3>), grid, block, 0, st, a); break;       \
+    default: hipLaunchKernelGGL((k_dec_attn_proj_q8<T, 4>), grid, block, 0, st, a); break;      \
   }
   DEC_TYPES(GO_T)
 #undef GO_T

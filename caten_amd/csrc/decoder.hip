@@ -455,7 +455,8 @@ static int finalize(Decoder *d) {
       d->flow = true;
     }
   }
-  if (c.arch == CTHIP_ARCH_GPT2 && state().decode_fused && !d->kvq && !d->kvp && !d->flow &&
+  // (a cache of Q8_0 rows keeps the three launches: the attention launch has a variant over the planes)
+  if (c.arch == CTHIP_ARCH_GPT2 && state().decode_fused && !d->kvp && !d->flow &&
       dec_fused_supported(d->layers[0].attn->type, d->layers[0].proj->type, d->layers[0].fc->type,
                           d->layers[0].fc2->type, D, c.n_heads, F)) {
     // the per-XCD accumulators assume what gfx950 has: XCD ids 0..7
@@ -573,8 +574,9 @@ static int queue_step(Decoder *d, bool with_head, bool embed) {
       qa.fold_s = L.attn_s;
       qa.fold_c = L.attn_c;
       qa.q = d->q;
-      qa.kc = L.k_cache;
-      qa.vc = L.v_cache;
+      qa.kc = d->kvq ? d->kv_tmp : L.k_cache;  // Q8_0 rows: the new row is quantised by the attention launch
+      qa.vc = d->kvq ? d->kv_tmp + D : L.v_cache;
+      qa.kv_stride = d->kvq ? 0 : D;
       qa.pos = pos;
       qa.rows = 3 * D;
       if (!(skip & 1)) TRY(launch_dec_qkv(qa, L.attn->type, l > 0));
@@ -588,7 +590,22 @@ static int queue_step(Decoder *d, bool with_head, bool embed) {
       aa.part = d->patt;
       aa.zero = d->pmlp;
       aa.zero_n16 = (int64_t)kDecXcds * D * 8 / 16;
-      if (!(skip & 2)) TRY(launch_dec_attn_proj(aa, L.attn->type, c.n_heads, D, replicas));
+      if (d->kvq) {
+        DecAttnQ8Args a8 = {};
+        a8.q = d->q;
+        a8.newkv = d->kv_tmp;
+        a8.kq = (signed char *)L.kq;
+        a8.vq = (signed char *)L.vq;
+        a8.kd = (unsigned short *)L.kdq;
+        a8.vd = (unsigned short *)L.vdq;
+        a8.pos = pos;
+        a8.pq = aa.pq;
+        a8.pd = aa.pd;
+        a8.part = aa.part;
+        a8.zero = aa.zero;
+        a8.zero_n16 = aa.zero_n16;
+        if (!(skip & 2)) TRY(launch_dec_attn_proj_q8(a8, L.attn->type, c.n_heads, D, replicas));
+      } else if (!(skip & 2)) TRY(launch_dec_attn_proj(aa, L.attn->type, c.n_heads, D, replicas));
       DecMlpArgs ma = {};
       ma.st.base = d->x2;
       ma.st.bias = L.proj_b;
@@ -1162,7 +1179,7 @@ int cthip_decoder_layer_launches(void *dec) {
   int rc = finalize(d);
   if (rc) return -1;
   if (d->flow) return 1;  // all layers are ONE launch
-  if (d->fused || d->fused_gqa) return 3;
+  if (d->fused || d->fused_gqa) return 3;  // (GPT-2 shapes: also over a cache of Q8_0 rows)
   if (d->kvp) return d->cfg.arch == CTHIP_ARCH_GPT2 ? 6 : 8;  // + one append (+ two rotations) around the attention launch
   if (d->kvq) return d->cfg.arch == CTHIP_ARCH_GPT2 ? 7 : 9;  // + two appends (+ two rotations) around the attention launch
   return 5;

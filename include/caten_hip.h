@@ -253,7 +253,7 @@ int cthip_linear(float *y, const void *wmat, const float *x, int m, const float 
  * "kv_cache": how decoder sessions created afterwards keep their KV cache: 0 (default) = fp32 rows, the
  *   reference's dense cache (external/llm/layers.lisp:19-33); 1 = GGUF-Q8_0 rows (blocks of 32 int8 and one fp16
  *   scale per cache row, quantised once when the row is appended): 3.76x fewer cache bytes held and read per
- *   step.  Such a session runs one launch per Linear; logits stay within rtol 2e-2 / atol 2e-2 of the fp32
+ *   step.  Such a session runs one launch per Linear (GPT-2 shapes: three launches per layer); logits stay within rtol 2e-2 / atol 2e-2 of the fp32
  *   cache's on the tested models (the band of 8-bit keys and values, not of the fp32 arithmetic around them).
  *   2 = fp32 rows in pages of cthip_kv_page_rows() rows per layer, opened when the position first reaches them
  *   (a session then holds the rows it has used instead of max_seq rows); such a session runs one launch per

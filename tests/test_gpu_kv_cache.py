@@ -235,3 +235,74 @@ def test_decoder_with_a_paged_cache_equals_the_dense_cache(arch, plen):
     # the dense session holds max_seq rows per layer, the paged one three pages (139 or 72 rows reached)
     dense_rows = 2 * cfg["n_layers"] * cfg["max_seq"] * kd * 4
     assert held0 - held2 > dense_rows // 2, (held0, held2, dense_rows)
+
+
+@pytest.mark.parametrize("name,wtype,plen", [("gpt2-tiny", "q8_0", 3), ("gpt2-tiny", "q4_0", 20), ("gpt2-mini", "q8_0", 5),
+                                              ("gpt2-mini", "q8_0", 505)])
+def test_three_launch_layer_over_a_q8_0_cache(oracle, name, wtype, plen):
+    """GPT-2 shapes keep three launches per layer over Q8_0 cache rows: the attention launch quantises the step's new
+    row itself.  Bars: layer 0's planes are the oracle's quantisation of the rows the fp32-cache session of the same
+    three-launch layer wrote, bit for bit (decoded rows and batched prompt rows alike); logits inside the 8-bit band of
+    the seven-launch Q8_0 session; two runs bit-identical; the device-resident loop gives the same tokens.  The long
+    prompt makes the decode steps cross the 512 keys one pass of the launch covers."""
+    print(f"case: three-launch layer over q8_0 cache {name} {wtype} prompt {plen}", flush=True)
+    from caten_amd import _lib, synth, llm
+    lib = _lib.init()
+    cfg = dict(synth.GPT2_CONFIGS[name], n_layers=2)
+    if plen > 100:
+        cfg["max_seq"] = 640
+    sd = llm.gpt2_state_dict(synth.gpt2_weights(cfg, seed=31), wtype)
+    prompt = synth.prompt(cfg["vocab"], plen, seed=31)
+    kd, steps = cfg["dim"], 14
+    n_rows = plen + steps - 1
+    runs = []
+    try:
+        for kv, fused in ((1, 1), (1, 0), (0, 1), (1, 1)):
+            _lib.check(lib.cthip_set_option(b"kv_cache", kv))
+            _lib.check(lib.cthip_set_option(b"decode_fused", fused))
+            m = llm.make_gpt2(cfg, sd)
+            toks, logs = llm.gpt2_generate(m, prompt, steps, on_device=False, keep_logits=True)
+            launches = lib.cthip_decoder_layer_launches(m.handle)
+            rows = [m.peek(f"{n}.0").reshape(cfg["max_seq"], kd)[:n_rows].copy() for n in ("k_cache", "v_cache")]
+            planes = None
+            if kv:
+                planes = [(m.peek(f"{n}_cache_q8.0").view(np.int8).reshape(cfg["max_seq"], kd)[:n_rows].copy(),
+                           m.peek(f"{n}_cache_d.0").view(np.uint16).reshape(cfg["max_seq"], kd // 32)[:n_rows].copy())
+                          for n in ("k", "v")]
+            m.close()
+            if kv and fused:
+                m = llm.make_gpt2(cfg, sd)
+                assert llm.gpt2_generate(m, prompt, steps, on_device=True) == toks
+                m.close()
+            runs.append((toks, logs, launches, rows, planes))
+    finally:
+        _lib.check(lib.cthip_set_option(b"kv_cache", 0))
+        _lib.check(lib.cthip_set_option(b"decode_fused", 1))
+    a, b, f, a2 = runs
+    assert (a[2], b[2], f[2]) == (3, 7, 3)
+    assert a[0] == a2[0] and all(np.array_equal(x, y) for x, y in zip(a[1], a2[1]))
+    for (q, d), (q2, d2) in zip(a[4], a2[4]):
+        assert np.array_equal(q, q2) and np.array_equal(d, d2)
+
+    def agree(t0, t1):
+        n = 0
+        while n < steps and t0[n] == t1[n]:
+            n += 1
+        return n
+
+    # against the seven-launch session over the same kind of cache: a near-tie may turn the greedy choice
+    same = agree(a[0], b[0])
+    print("tokens", a[0], b[0], "agree for", same, flush=True)
+    assert same >= steps // 2
+    for x, y in zip(a[1][:same + 1], b[1][:same + 1]):
+        assert np.allclose(x, y, rtol=2e-2, atol=2e-2), float(np.max(np.abs(x - y)))
+    # against the fp32 cache of the same three launches: layer 0's rows depend on the tokens only
+    same = agree(a[0], f[0])
+    assert same >= steps // 2
+    rows = min(plen + same, n_rows)
+    for (q, d), r in zip(a[4], f[3]):
+        want_q, want_d = _planes(oracle, r[:rows])
+        assert np.array_equal(q[:rows], want_q) and np.array_equal(d[:rows], want_d)
+    for x, y in zip(a[1][:same + 1], f[1][:same + 1]):
+        assert np.allclose(x, y, rtol=2e-2, atol=2e-2), float(np.max(np.abs(x - y)))
+    assert not np.array_equal(a[1][-1], f[1][-1])  # the cache IS quantised

@@ -291,8 +291,12 @@ __device__ __forceinline__ float half_bits_to_float(unsigned short h) {
 __device__ __forceinline__ float ct_exp(float x) { return exp2f(x * 1.442695f); }
 __device__ __forceinline__ float ct_sigmoid(float x) { return 1.0f / (1.0f + exp2f(x * -1.442695f)); }
 __device__ __forceinline__ float ct_tanh(float y) { return 2.0f * ct_sigmoid(2.0f * y) - 1.0f; }
+// GELU(tanh): 0.5 x (1 + tanh(u)) = x sigmoid(2u), u = sqrt(2/pi) (x + 0.044715 x^3) -- the same function without the
+// cancellation in 1 + tanh(u) for negative x, as one exponential and one reciprocal (each within an ulp: the GEMM
+// epilogue of c_fc spends a fifth of its launch on this function when it divides and handles subnormal exponentials)
 __device__ __forceinline__ float ct_gelu(float x) {
-  return 0.5f * x * (1.0f + ct_tanh(0.7978846f * (x + 0.044715f * (x * x * x))));
+  const float u2 = -2.3022082f * (x * fmaf(0.044715f * x, x, 1.0f));  // -2 u log2(e)
+  return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(u2));
 }
 __device__ __forceinline__ float ct_silu(float x) { return x * ct_sigmoid(x); }
 __device__ __forceinline__ float apply_act(int act, float v) {

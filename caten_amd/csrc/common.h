@@ -143,6 +143,10 @@ struct GemvArgs {
   float eps;
   int rows, cols;
   int act, pro;
+  // A launch over a slice of the columns of a wider matrix (set by the launcher; 0 = the matrix is `cols` wide):
+  // 16-byte chunks and block scales between the starts of two rows, and where the `up` half of a SwiGLU input
+  // starts behind x (q, d and x then point at the slice's first column)
+  int ld_chunks, ld_scales, up_off;
   int64_t x_stride, y_stride;  // between the m input / output vectors (blockIdx.y)
   // fused greedy argmax over the output rows (m == 1 only); all null when unused.
   // am_val/am_idx hold one partial (best value, lowest row) per wavefront of the launch.

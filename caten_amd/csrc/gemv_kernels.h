@@ -140,7 +140,7 @@ __device__ __forceinline__ void coop_prologue(const GemvArgs &a, const float *__
   if (a.pro == CTHIP_PRO_SWIGLU) {
     for (int i = tid; i < n4; i += nthr) {
       float4 v = ((const float4 *)x)[i];
-      float4 u = ((const float4 *)(x + a.cols))[i];
+      float4 u = ((const float4 *)(x + (a.up_off ? a.up_off : a.cols)))[i];
       ((float4 *)xs)[i] = make_float4(ct_silu(v.x) * u.x, ct_silu(v.y) * u.y, ct_silu(v.z) * u.z, ct_silu(v.w) * u.w);
     }
     __syncthreads();
@@ -289,8 +289,8 @@ __device__ __forceinline__ void gemv_ring(const GemvArgs &a, float *xs_lds, floa
   const int m = blockIdx.y;
   const float *__restrict__ x = a.x + (int64_t)m * a.x_stride;
   const uint4 *__restrict__ qp = (const uint4 *)a.q;
-  const int64_t row_chunks = nchunks;
-  const int scales_per_row = a.cols >> 5;
+  const int64_t row_chunks = a.ld_chunks ? a.ld_chunks : nchunks;
+  const int scales_per_row = a.ld_scales ? a.ld_scales : a.cols >> 5;
   const int nrq = (a.rows + RPW - 1) / RPW;
   const float *zf = (const float *)g_gemv_zeros;
   const uint4 *z16 = (const uint4 *)g_gemv_zeros;
@@ -312,7 +312,7 @@ __device__ __forceinline__ void gemv_ring(const GemvArgs &a, float *xs_lds, floa
   float gr[QUANT ? 1 : KC][QUANT ? 1 : XPC];  // gamma of an unstaged folded norm (fp32 / fp16 weights)
   const float4 *x4 = (const float4 *)x;
   // the second operand of the staging: the gate's partner, gamma, or (unused) the vector again
-  const float4 *u4 = swiglu ? (const float4 *)(x + a.cols) : (layernorm || folded) && a.norm_g ? (const float4 *)a.norm_g : x4;
+  const float4 *u4 = swiglu ? (const float4 *)(x + (a.up_off ? a.up_off : a.cols)) : (layernorm || folded) && a.norm_g ? (const float4 *)a.norm_g : x4;
   const float4 *b4 = (direct && a.norm_b) ? (const float4 *)a.norm_b : x4;  // beta of a LayerNorm applied here
   if (early) {
 #pragma unroll
@@ -617,8 +617,8 @@ __global__ __launch_bounds__(256) void k_gemv(GemvArgs a) {
   const int m = blockIdx.y;
   const float *__restrict__ x = a.x + (int64_t)m * a.x_stride;
   const uint4 *__restrict__ qp = (const uint4 *)a.q;
-  const int64_t row_chunks = nchunks;  // 16-byte chunks per row in the quant plane
-  const int scales_per_row = a.cols >> 5;
+  const int64_t row_chunks = a.ld_chunks ? a.ld_chunks : nchunks;  // 16-byte chunks per row in the quant plane
+  const int scales_per_row = a.ld_scales ? a.ld_scales : a.cols >> 5;
   const int nrq = (a.rows + RPW - 1) / RPW;
 
   // LayerNorm / RMSNorm folded through the product instead of applied to the input first:

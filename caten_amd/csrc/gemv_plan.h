@@ -64,6 +64,29 @@ inline int gemv_pick_shape(int type, int cols) {
   return best;
 }
 
+// Rows wider than any register-resident variant (FFN down-projections of 7B-class models and up) are multiplied as
+// column slices of equal width, one launch each: slice 0 carries the epilogue, every later one adds its products to
+// what is there.  Returns the number of slices (0 = the width needs none, or cannot be cut on block boundaries into
+// widths that variants cover) and their width (the last slice has what is left).
+inline int gemv_slices(int type, long long cols, int *width) {
+  const int xpc = gemv_xpc(type);
+  const int unit = (type == CTHIP_Q8_0 || type == CTHIP_Q4_0) ? 32 : xpc;  // a slice starts on a block scale
+  if (cols <= 0 || cols > 0x7fffffff || cols % unit) return 0;
+  int maxc = 0;
+  for (const GemvShape &sh : gemv_shapes())
+    if (sh.type == type && sh.G * sh.KC * xpc > maxc) maxc = sh.G * sh.KC * xpc;
+  if (!maxc || cols <= maxc) return 0;
+  for (int n = (int)((cols + maxc - 1) / maxc); n <= 64; n++) {
+    const int wdt = (int)(((cols + n - 1) / n + unit - 1) / unit * unit);
+    const long long last = cols - (long long)wdt * (n - 1);
+    if (wdt <= maxc && last > 0 && gemv_pick_shape(type, wdt) >= 0 && gemv_pick_shape(type, (int)last) >= 0) {
+      *width = wdt;
+      return n;
+    }
+  }
+  return 0;
+}
+
 struct GemvPlanIn {
   int type, rows, cols, m;
   int pro;            // CTHIP_PRO_*

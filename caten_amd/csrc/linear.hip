@@ -344,7 +344,10 @@ int launch_prologue(float *out, const float *x, int cols, int pro, const float *
   return 0;
 }
 
-bool gemv_is_direct(const WMat *w) { return pick_variant(w->type, (int)w->cols) != nullptr; }
+bool gemv_is_direct(const WMat *w) {
+  int width = 0;
+  return pick_variant(w->type, (int)w->cols) != nullptr || gemv_slices(w->type, (long long)w->cols, &width) > 0;
+}
 int gemv_rows_per_wave(int type, int64_t cols) {
   const GemvVariant *v = cols <= 0x7fffffff ? pick_variant(type, (int)cols) : nullptr;
   return v ? 64 / v->G : 0;
@@ -365,19 +368,10 @@ int launch_swiglu_pairs(float *out, const float *in, int64_t n) {
   return 0;
 }
 
-// Queues one fused Linear on the stream. Used by cthip_linear and by the decoder.
-int launch_gemv(const WMat *w, GemvArgs a, int m) {
+// one launch of a register-resident variant over a.cols columns (a whole matrix, or a column slice of one)
+static int launch_variant(const GemvVariant *v, const WMat *w, GemvArgs a, int m) {
   State &s = state();
-  a.q = w->q;
-  a.d = (const unsigned short *)w->d;
-  a.rows = (int)w->rows;
-  a.cols = (int)w->cols;
-  if (a.split1 <= 0) a.split1 = a.split2 = a.rows;
-  if (a.am_val && m != 1) return fail(CTHIP_E_BAD_ARG, "gemv: the fused argmax needs m == 1");
-  const GemvVariant *v = pick_variant(w->type, a.cols);
-  if (a.pair_swiglu && (!v || v->G > 32 || (a.rows & 1) || a.am_val || a.residual || a.split1 != a.rows))
-    return fail(CTHIP_E_UNSUPPORTED, "gemv: the paired SwiGLU epilogue needs two rows per wavefront and plain outputs");
-  if (v) {
+  {
     const int vi = (int)(v - all_variants().data());
     static std::vector<int> occ_cache(all_variants().size(), 0);
     GemvPlanIn in = {};
@@ -422,6 +416,52 @@ int launch_gemv(const WMat *w, GemvArgs a, int m) {
     if (a.am_val) {
       hipLaunchKernelGGL(k_argmax_finish, dim3(1), dim3(256), 0, s.stream, a, p.nwaves);
       CTHIP_LAUNCH_CHECK();
+    }
+    return 0;
+  }
+}
+
+// Queues one fused Linear on the stream. Used by cthip_linear and by the decoder.
+int launch_gemv(const WMat *w, GemvArgs a, int m) {
+  State &s = state();
+  a.q = w->q;
+  a.d = (const unsigned short *)w->d;
+  a.rows = (int)w->rows;
+  a.cols = (int)w->cols;
+  a.ld_chunks = a.ld_scales = a.up_off = 0;
+  if (a.split1 <= 0) a.split1 = a.split2 = a.rows;
+  if (a.am_val && m != 1) return fail(CTHIP_E_BAD_ARG, "gemv: the fused argmax needs m == 1");
+  const GemvVariant *v = pick_variant(w->type, a.cols);
+  if (a.pair_swiglu && (!v || v->G > 32 || (a.rows & 1) || a.am_val || a.residual || a.split1 != a.rows))
+    return fail(CTHIP_E_UNSUPPORTED, "gemv: the paired SwiGLU epilogue needs two rows per wavefront and plain outputs");
+  if (v) return launch_variant(v, w, a, m);
+  // wider than any variant: column slices, when nothing in the launch needs the whole row at once (a norm of the
+  // input, an activation of the sum, an argmax) and the output is one plain vector per input row
+  int width = 0;
+  const int nsl = (a.pro == CTHIP_PRO_NONE || a.pro == CTHIP_PRO_SWIGLU) && a.act == CTHIP_ACT_NONE && !a.am_val &&
+                          !a.fold_s && a.split1 == a.rows && a.y
+                      ? gemv_slices(w->type, a.cols, &width)
+                      : 0;
+  if (nsl > 0) {
+    const int xpc = xpc_of(w->type), cols = a.cols;
+    for (int sl = 0; sl < nsl; sl++) {
+      const int c0 = sl * width;
+      GemvArgs b = a;
+      b.cols = sl + 1 < nsl ? width : cols - c0;
+      b.q = (const char *)w->q + (int64_t)(c0 / xpc) * 16;
+      b.d = w->d ? (const unsigned short *)w->d + (c0 >> 5) : nullptr;
+      b.x = a.x + c0;
+      b.ld_chunks = cols / xpc;
+      b.ld_scales = cols >> 5;
+      b.up_off = a.pro == CTHIP_PRO_SWIGLU ? cols : 0;
+      if (sl > 0) {  // adds to what the slices before it left (each output element is read and written by one lane)
+        b.bias = b.bias0 = nullptr;
+        b.residual = a.y;
+      }
+      const GemvVariant *vs = pick_variant(w->type, b.cols);
+      if (!vs) return fail(CTHIP_E_STATE, "gemv: no variant for a slice of %d columns", b.cols);
+      const int rc = launch_variant(vs, w, b, m);
+      if (rc) return rc;
     }
     return 0;
   }
@@ -567,7 +607,7 @@ int cthip_wmat_fold_layernorm(void *wmat, const float *gamma, const float *beta,
   CTHIP_REQUIRE_INIT();
   CTHIP_ARG(wmat != nullptr && gamma != nullptr && beta != nullptr);
   WMat *w = (WMat *)wmat;
-  if (!gemv_is_direct(w)) return fail(CTHIP_E_UNSUPPORTED, "cthip_wmat_fold_layernorm: no single-row kernel covers %lld columns", (long long)w->cols);
+  if (!pick_variant(w->type, (int)w->cols)) return fail(CTHIP_E_UNSUPPORTED, "cthip_wmat_fold_layernorm: no single-row kernel covers %lld columns", (long long)w->cols);
   int rc;
   if (!w->fold_s && (rc = cthip_alloc((void **)&w->fold_s, sizeof(float) * (size_t)w->rows))) return rc;
   if (!w->fold_c && (rc = cthip_alloc((void **)&w->fold_c, sizeof(float) * (size_t)w->rows))) return rc;

@@ -39,6 +39,7 @@ struct Case {
   int type, rows, cols, m, pro;
   bool fold, bias, bias0, residual, argmax, pair;
   int cus, occ;
+  int full_cols, col0;  // the launch covers columns [col0, col0 + cols) of a matrix full_cols wide (0 = the whole matrix)
 };
 
 static void walk(const Case &c) {
@@ -61,17 +62,21 @@ static void walk(const Case &c) {
   const bool swiglu = c.pro == CTHIP_PRO_SWIGLU, layernorm = c.pro == CTHIP_PRO_LAYERNORM;
   const bool folded = c.pro == CTHIP_PRO_RMSNORM || (layernorm && fold);
   const bool coop = p.stage;
-  const int in_cols = swiglu ? 2 * c.cols : c.cols;
+  // a column slice: the launcher's pointer offsets, row pitches and gate / up distance (launch_gemv in linear.hip)
+  const int full = c.full_cols ? c.full_cols : c.cols;
+  const long long q0 = 16ll * (c.col0 / XPC), d0 = 2ll * (c.col0 >> 5), x0 = 4ll * c.col0, upo = full;
+  const int in_cols = swiglu ? 2 * full : full;
   const long long x_stride = in_cols, out_rows = c.pair ? c.rows / 2 : c.rows, y_stride = out_rows;
-  const long long row_bytes = c.type == CTHIP_Q8_0 ? c.cols : c.type == CTHIP_Q4_0 ? c.cols / 2 : c.type == CTHIP_F16 ? 2ll * c.cols : 4ll * c.cols;
-  Region Q = {"quant plane", true, row_bytes * c.rows}, D = {"scale plane", QUANT, 2ll * (c.cols / 32) * c.rows};
+  const long long row_bytes = c.type == CTHIP_Q8_0 ? full : c.type == CTHIP_Q4_0 ? full / 2 : c.type == CTHIP_F16 ? 2ll * full : 4ll * full;
+  Region Q = {"quant plane", true, row_bytes * c.rows}, D = {"scale plane", QUANT, 2ll * (full / 32) * c.rows};
   Region X = {"x", true, 4 * x_stride * c.m}, NG = {"norm_g", c.pro == CTHIP_PRO_LAYERNORM || c.pro == CTHIP_PRO_RMSNORM, 4ll * c.cols};
   Region NB = {"norm_b", layernorm, 4ll * c.cols}, B = {"bias", bias, 4ll * c.rows}, R = {"residual", c.residual, 4 * y_stride * c.m};
   Region FS = {"fold_s", fold, 4ll * c.rows}, Y = {"y", true, 4 * y_stride * c.m}, AM = {"argmax partials", c.argmax, 4ll * 16384};
   Region LDS = {"LDS staging buffer", p.lds > 0, (long long)p.lds}, RED = {"red", true, 4 * 24};
   const int nchunks = c.cols / XPC, nrq = (c.rows + RPW - 1) / RPW, n4 = c.cols >> 2;
   const int nthr = (int)p.block, wpb = nthr >> 6, total_waves = (int)p.grid_x * wpb;
-  const int scales_per_row = c.cols >> 5;
+  const int scales_per_row = full >> 5;
+  const long long row_chunks = full / XPC;
   const bool ring = PD > 1;
   if (ring && nthr != 256) { g_violations++; printf("VIOLATION %s: the looping kernel is compiled for 256 threads, launched with %d\n", g_case.c_str(), nthr); }
   const bool epi_kernel = p.kernel == GEMV_K_LOOP_EPI, direct_kernel = p.kernel == GEMV_K_LOOP_DIRECT;
@@ -79,15 +84,15 @@ static void walk(const Case &c) {
     for (unsigned bx = 0; bx < p.grid_x; bx++)
       for (int tid = 0; tid < nthr; tid++) {
         const int lane = tid & 63, g = lane / G, l = lane % G, wave = (int)bx * wpb + (tid >> 6);
-        const long long xoff = 4 * x_stride * m;
+        const long long xoff = 4 * x_stride * m + x0;
         auto tile = [&](int rq, const char *what) {
           int row = rq * RPW + g;
           row = row < c.rows ? row : c.rows - 1;
           for (int j = 0; j < KC; j++) {
             const int cc = l + G * j;
             if (cc >= nchunks) continue;  // reads the zero block
-            touch(Q, ((long long)row * nchunks + cc) * 16, 16, what);
-            if (QUANT) touch(D, 2 * ((long long)row * scales_per_row + (c.type == CTHIP_Q8_0 ? (cc >> 1) : cc)), 2, what);
+            touch(Q, q0 + ((long long)row * row_chunks + cc) * 16, 16, what);
+            if (QUANT) touch(D, d0 + 2 * ((long long)row * scales_per_row + (c.type == CTHIP_Q8_0 ? (cc >> 1) : cc)), 2, what);
           }
           return row;
         };
@@ -128,7 +133,7 @@ static void walk(const Case &c) {
         };
         auto coop_prologue = [&](bool normalise) {
           if (!swiglu && !normalise) { for (int i = tid; i < n4; i += nthr) touch(X, xoff + 16ll * i, 16, "copy"), touch(LDS, 16ll * i, 16, "copy"); return; }
-          if (swiglu) { for (int i = tid; i < n4; i += nthr) touch(X, xoff + 16ll * i, 16, "gate"), touch(X, xoff + 4ll * c.cols + 16ll * i, 16, "up"), touch(LDS, 16ll * i, 16, "swiglu"); return; }
+          if (swiglu) { for (int i = tid; i < n4; i += nthr) touch(X, xoff + 16ll * i, 16, "gate"), touch(X, xoff + 4ll * upo + 16ll * i, 16, "up"), touch(LDS, 16ll * i, 16, "swiglu"); return; }
           for (int i = tid; i < n4; i += nthr) {
             touch(X, xoff + 16ll * i, 16, "norm input");
             touch(NG, 16ll * i, 16, "norm gamma");
@@ -164,7 +169,7 @@ static void walk(const Case &c) {
               int i = tid + k * 256;
               i = i < n4 ? i : n4 - 1;
               touch(X, xoff + 16ll * i, 16, "early input");
-              if (swiglu) touch(X, xoff + 4ll * c.cols + 16ll * i, 16, "early up");
+              if (swiglu) touch(X, xoff + 4ll * upo + 16ll * i, 16, "early up");
               else if ((layernorm || folded) && NG.present) touch(NG, 16ll * i, 16, "early gamma");
               if (direct_kernel && direct) touch(NB, 16ll * i, 16, "early beta");
             }
@@ -178,7 +183,7 @@ static void walk(const Case &c) {
           if (coop && !early) coop_prologue(true);
           if (early) {
             for (int i = tid; i < n4; i += 256) {
-              if (i >= tid + 4 * 256) { touch(X, xoff + 16ll * i, 16, "late input"); if (swiglu) touch(X, xoff + 4ll * c.cols + 16ll * i, 16, "late up"); else if (NG.present) touch(NG, 16ll * i, 16, "late gamma"); }
+              if (i >= tid + 4 * 256) { touch(X, xoff + 16ll * i, 16, "late input"); if (swiglu) touch(X, xoff + 4ll * upo + 16ll * i, 16, "late up"); else if (NG.present) touch(NG, 16ll * i, 16, "late gamma"); }
               touch(LDS, 16ll * i, 16, "stage");
             }
             touch(RED, 4 * (tid >> 6), 4, "red"), touch(RED, 4 * (8 + (tid >> 6)), 4, "red"), touch(RED, 4 * (16 + (tid >> 6)), 4, "red");
@@ -212,7 +217,59 @@ static void check_reduce_norm_plans() {
       }
 }
 
+// "shape TYPE ROWS COLS [TYPE ROWS COLS ...]": only these Linears (TYPE = the library's code: 0 fp32, 1 fp16, 2 Q4_0,
+// 8 Q8_0), with every prologue and the flag sets a decoder launches -- for a model size outside the table below
+static int walk_given_shapes(int argc, char **argv) {
+  for (int i = 2; i + 2 < argc; i += 3) {
+    const int type = atoi(argv[i]), rows = atoi(argv[i + 1]), cols = atoi(argv[i + 2]);
+    const int xpc = gemv_xpc(type);
+    if (rows <= 0 || cols <= 0 || xpc <= 0 || cols % xpc || ((type == CTHIP_Q8_0 || type == CTHIP_Q4_0) && cols % 32)) {
+      printf("gemv bounds: shape %d %d %d is not a Linear of the library\n", type, rows, cols);
+      return 2;
+    }
+    int width = 0;
+    const int nsl = gemv_pick_shape(type, cols) < 0 ? gemv_slices(type, cols, &width) : 0;
+    if (nsl > 0) {  // what launch_gemv queues for a row wider than any variant: no norm, no activation, no argmax
+      for (int pro : {(int)CTHIP_PRO_NONE, (int)CTHIP_PRO_SWIGLU})
+        for (int flags : {0, 2, 8, 10})
+          for (int mm : {1, 3})
+            for (int sl = 0; sl < nsl; sl++) {
+              Case c = {};
+              c.type = type; c.rows = rows; c.m = mm; c.pro = pro; c.cus = 256; c.occ = 2;
+              c.full_cols = cols; c.col0 = sl * width; c.cols = sl + 1 < nsl ? width : cols - c.col0;
+              c.bias = sl == 0 && (flags & 2);
+              c.residual = sl > 0 || (flags & 8);
+              walk(c);
+            }
+      continue;
+    }
+    for (int pro = 0; pro <= 3; pro++)
+      for (int flags : {0, 2, 8, 10, 11, 15, 17, 24}) {
+        Case c = {};
+        c.type = type; c.rows = rows; c.cols = cols; c.m = 1; c.pro = pro;
+        c.fold = (flags & 1) && pro == CTHIP_PRO_LAYERNORM;
+        if ((flags & 1) && pro != CTHIP_PRO_LAYERNORM) continue;
+        if ((flags & 4) && !c.fold) continue;
+        c.bias = (flags & 2) || c.fold;
+        c.bias0 = c.fold && (flags & 4);
+        c.residual = flags & 8;
+        c.argmax = flags & 16;
+        c.cus = 256; c.occ = 2;
+        walk(c);
+      }
+    if (rows % 2 == 0) {
+      Case c = {};
+      c.type = type; c.rows = rows; c.cols = cols; c.m = 1; c.pro = CTHIP_PRO_RMSNORM; c.pair = true; c.cus = 256; c.occ = 2;
+      const int sh = gemv_pick_shape(type, cols);
+      if (sh >= 0 && gemv_shapes()[sh].G <= 32) walk(c);
+    }
+  }
+  printf("gemv bounds: %lld launches, %lld accesses checked, %lld violations\n", g_launches, g_checked, g_violations);
+  return g_violations ? 1 : 0;
+}
+
 int main(int argc, char **argv) {
+  if (argc > 1 && !strcmp(argv[1], "shape")) return walk_given_shapes(argc, argv);
   check_reduce_norm_plans();
   // default: a few seconds (every shape, the flag combinations thinned out on the large ones); "full": everything
   const bool full = argc > 1 && !strcmp(argv[1], "full");

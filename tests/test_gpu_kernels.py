@@ -303,6 +303,38 @@ def test_gemv_fallback_shapes_with_prologue(ops, oracle):
     close(ops.linear(x, wm, prologue="layernorm", norm_g=g), oracle.linear(oracle.layernorm(x, g), wd))
 
 
+@pytest.mark.parametrize("kind,rows,cols,m", [("q4_0", 4096, 11008, 1), ("q8_0", 1000, 11008, 1), ("q4_0", 515, 28672, 1),
+                                              ("f32", 300, 12288, 1), ("f16", 300, 6400, 1), ("q8_0", 300, 8224, 3)])
+def test_gemv_rows_wider_than_any_variant_go_as_column_slices(ops, oracle, kind, rows, cols, m):
+    """FFN down-projections of 7B-class models and up (11008, 13824, 28672 input features) are wider than what a
+    lane group keeps in registers: the launcher cuts the columns into equal slices, slice 0 carries bias and
+    residual, the others add to it.  Every column gets a weight that a wrong slice offset or row pitch would miss;
+    SwiGLU reads `up` behind the whole gate half, not behind the slice."""
+    print(f"case: sliced gemv {kind} ({rows},{cols}) m {m}", flush=True)
+    from caten_amd.llm import Tensor
+    rng = np.random.default_rng(rows + cols)
+    w = rng.normal(0, 0.02, (rows, cols)).astype(np.float32)
+    w[:, ::97] += 0.05  # columns that stand out, spread over every slice
+    x = rng.normal(0.1, 1, (m, cols)).astype(np.float32)
+    b = rng.normal(0, 0.02, rows).astype(np.float32)
+    r = rng.normal(0, 1, (m, rows)).astype(np.float32)
+    t = Tensor.from_f32(w, kind)
+    wd = oracle.dequant(kind, t.raw, w.size).reshape(rows, cols)
+    wm = ops.WeightMatrix(kind, t.raw, rows, cols)
+    tol = dict(rtol=2e-4, atol=2e-4)
+    xs, rs = (x[0], r[0]) if m == 1 else (x, r)
+    close(ops.linear(xs, wm), oracle.linear(xs, wd), **tol)
+    close(ops.linear(xs, wm, bias=b, residual=rs), oracle.linear(xs, wd, b) + rs, **tol)
+    xu = rng.normal(0, 1, (m, 2 * cols)).astype(np.float32)
+    sw = (oracle.silu(xu[:, :cols]) * xu[:, cols:]).astype(np.float32)
+    xus, sws = (xu[0], sw[0]) if m == 1 else (xu, sw)
+    close(ops.linear(xus, wm, residual=rs, prologue="swiglu"), oracle.linear(sws, wd) + rs, **tol)
+    # what needs the whole row at once still goes through the wave-per-row kernel
+    g = rng.normal(1, 0.02, cols).astype(np.float32)
+    close(ops.linear(xs, wm, act="relu", prologue="rmsnorm", norm_g=g), oracle.relu(oracle.linear(oracle.rmsnorm(xs, g), wd)), **tol)
+    wm.free()
+
+
 def test_linear_batched_rows(ops, oracle):
     from caten_amd.llm import Tensor
     rng = np.random.default_rng(23)

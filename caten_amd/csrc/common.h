@@ -340,10 +340,19 @@ CTHIP_SBYTE(2)
 CTHIP_SBYTE(3)
 #undef CTHIP_SBYTE
 
-// RoPE of four consecutive elements of a head (positional-encoding.lisp:3-64) at position `at`
-__device__ __forceinline__ float4 rope4(float4 x, int c, int DH, float log2_base, int at) {
-  // lane c holds elements 4c..4c+3 = pairs 2c and 2c+1 of the head; same arithmetic as k_rope
-  float o[4] = {x.x, x.y, x.z, x.w};
+// RoPE of four consecutive elements of a head (positional-encoding.lisp:3-64) at position `at`: lane c holds elements
+// 4c..4c+3 = pairs 2c and 2c+1 of the head; same arithmetic as k_rope.  The angles' sines and cosines depend on
+// (c, at) only, so a launch that rotates a query and a key at the same place computes them once.
+// the rotation of one pair with its roundings pinned, so that every kernel that rotates gives the same bits
+__device__ __forceinline__ void rope_pair(float x0, float x1, float sn, float cs, float &o0, float &o1) {
+  o0 = __fmaf_rn(x0, cs, -__fmul_rn(x1, sn));
+  o1 = __fmaf_rn(x0, sn, __fmul_rn(x1, cs));
+}
+struct Rope4 {
+  float sn[2], cs[2];
+};
+__device__ __forceinline__ Rope4 rope4_angles(int c, int DH, float log2_base, int at) {
+  Rope4 r;
 #pragma unroll
   for (int t = 0; t < 2; t++) {
     const int i = 2 * c + t;
@@ -351,13 +360,18 @@ __device__ __forceinline__ float4 rope4(float4 x, int c, int DH, float log2_base
     const float logb = log2_base * 0.6931472f;
     const float theta = exp2f(-(expo * logb) * 1.442695f);
     const float ang = (float)at * theta;
-    float sn, cs;
-    sincosf(ang, &sn, &cs);
-    const float x0 = o[2 * t], x1 = o[2 * t + 1];
-    o[2 * t] = x0 * cs - x1 * sn;
-    o[2 * t + 1] = x0 * sn + x1 * cs;
+    sincosf(ang, &r.sn[t], &r.cs[t]);
   }
-  return make_float4(o[0], o[1], o[2], o[3]);
+  return r;
+}
+__device__ __forceinline__ float4 rope4_apply(float4 x, const Rope4 &r) {
+  float4 o;
+  rope_pair(x.x, x.y, r.sn[0], r.cs[0], o.x, o.y);
+  rope_pair(x.z, x.w, r.sn[1], r.cs[1], o.z, o.w);
+  return o;
+}
+__device__ __forceinline__ float4 rope4(float4 x, int c, int DH, float log2_base, int at) {
+  return rope4_apply(x, rope4_angles(c, DH, log2_base, at));
 }
 
 }  // namespace cthip

@@ -630,8 +630,7 @@ __global__ __launch_bounds__(256) void k_rope(float *__restrict__ out, const flo
   float sn, cs;
   sincosf(ang, &sn, &cs);
   const float x0 = x[2 * p], x1 = x[2 * p + 1];
-  out[2 * p] = x0 * cs - x1 * sn;
-  out[2 * p + 1] = x0 * sn + x1 * cs;
+  rope_pair(x0, x1, sn, cs, out[2 * p], out[2 * p + 1]);
 }
 
 // Llama-shaped decode: rotate the new key row (Hkv,Dh) at position pos[0] into the K cache and
@@ -653,8 +652,7 @@ __global__ __launch_bounds__(256) void k_rope_append(float *__restrict__ kc, flo
   const float x0 = kv[2 * p], x1 = kv[2 * p + 1];
   float *ko = kc + (int64_t)at * KD;
   float *vo = vc + (int64_t)at * KD;
-  ko[2 * p] = x0 * cs - x1 * sn;
-  ko[2 * p + 1] = x0 * sn + x1 * cs;
+  rope_pair(x0, x1, sn, cs, ko[2 * p], ko[2 * p + 1]);
   vo[2 * p] = kv[KD + 2 * p];
   vo[2 * p + 1] = kv[KD + 2 * p + 1];
 }
@@ -680,8 +678,7 @@ __global__ __launch_bounds__(256) void k_qkv_split(float *__restrict__ q, float 
       const float theta = exp2f(-(expo * (log2_base * 0.6931472f)) * 1.442695f);
       float sn, cs;
       sincosf((float)at * theta, &sn, &cs);
-      o0 = x0 * cs - x1 * sn;
-      o1 = x0 * sn + x1 * cs;
+      rope_pair(x0, x1, sn, cs, o0, o1);
     }
     float *dst = isq ? qo : ko;
     dst[2 * pp] = o0;
@@ -730,8 +727,9 @@ void k_attn_cached(float *__restrict__ out, const float *__restrict__ q,
   float4 kn = make_float4(0.f, 0.f, 0.f, 0.f), vn = kn;
   if (APPEND) {
     const int KD = Hkv * DH;
-    q4 = rope4(q4, c, DH, log2_base, T - 1);
-    kn = rope4(*(const float4 *)(newkv + hk * DH + 4 * c), c, DH, log2_base, T - 1);
+    const Rope4 ra = rope4_angles(c, DH, log2_base, T - 1);
+    q4 = rope4_apply(q4, ra);
+    kn = rope4_apply(*(const float4 *)(newkv + hk * DH + 4 * c), ra);
     vn = *(const float4 *)(newkv + KD + hk * DH + 4 * c);
     if (h % (H / Hkv) == 0 && tid < LPK) {
       ((float4 *)(kc + (int64_t)(T - 1) * KD + hk * DH))[c] = kn;

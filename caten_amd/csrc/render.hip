@@ -75,16 +75,22 @@ struct Parser {
       else break;
     }
   }
+  // Every later pass (rendering, probing, matching) recurses over the tree this builds, so the depth is bounded here:
+  // no item of a real graph nests anywhere near this deep, and text that does must not run the host out of stack.
+  static constexpr int kMaxDepth = 256;
+  int depth = 0;
   bool parse(Sx &out) {
     skip();
     if (!*p) return err = "unexpected end of text", false;
     if (*p == '(') {
+      if (depth >= kMaxDepth) return err = "lists nested deeper than 256", false;
       p++;
+      depth++;
       out = Sx();
       for (;;) {
         skip();
         if (!*p) return err = "unbalanced '('", false;
-        if (*p == ')') { p++; return true; }
+        if (*p == ')') { p++; depth--; return true; }
         Sx e;
         if (!parse(e)) return false;
         out.v.push_back(std::move(e));
@@ -202,6 +208,10 @@ static bool build_item(const Sx &top, Item &it, std::string &err) {
       b.upfrom = n.v[2];
       b.below = n.v[3];
       b.by = n.v[4];
+      // a loop that does not advance would never leave its kernel
+      if ((b.by.kind == Sx::INT && b.by.i < 1) || (b.by.kind == Sx::FLT && !(b.by.f >= 1.0)))
+        return err = "for: the step must be at least 1", false;
+      if (n.v[1].kind != Sx::SYM || n.v[1].s.empty()) return err = "for: the index must be a symbol", false;
       b.global_scope = n.n() > 5 && n.v[5].is_sym("global");
       it.body.push_back(b);
       depth++;
@@ -269,6 +279,7 @@ struct Rend {
     }
     // the shortest decimal that reads back as the same float, in positional notation (as Caten's ~f prints)
     const float fv = (float)v;
+    if (isinf(fv)) return fv > 0 ? "_infinity" : "_negative_infinity";  // a double past the float range
     int prec = 0;
     for (; prec <= 8; prec++) {
       snprintf(buf, sizeof(buf), "%.*e", prec, (double)fv);

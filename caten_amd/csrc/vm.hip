@@ -180,6 +180,8 @@ static int vm_allocate(Vm &vm, int idx, VmNode &n) {
     if (!vm_value(vm, n.in[(size_t)k], v) || v.kind != VM_INT || v.i < 0)
       return fail(CTHIP_E_STATE, "vm: node %d: axis %d of an :Allocate is not a non-negative integer that has been set", idx, k);
     shape[k] = v.i;
+    if (v.i && count > (1ll << 46) / v.i)  // (a wrapped product would open a small buffer for kernels that believe the shape)
+      return fail(CTHIP_E_BAD_ARG, "vm: node %d: an :Allocate of more than 2^46 elements", idx);
     count *= v.i;
   }
   bool same = n.pool != nullptr && (int)n.pool_shape.size() == nrank;

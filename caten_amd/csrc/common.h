@@ -22,6 +22,9 @@ struct State {
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   int gemm_precision = GEMM_BF16X3_DEFAULT;  // option "gemm_precision" (GEMM_*) of m > 1 Linear launches
   int gemv_stream = -1;  // option "gemv_stream_weights": -1 = per matrix (WMat::stream), 0 / 1 = never / always
+  // option "gemv_wide": which single-row launches take the wide-row kernel (input vector in LDS): 0 = none, 1 = rows
+  // no register-resident variant covers or only one that runs a single wavefront per SIMD, 2 = every launch it supports
+  int gemv_wide = 1;
   // decoder sessions read these when they first run
   int decoder_graph = 1;  // option "decoder_graph": 0 = the step's launches are issued one by one (kernel tracing)
   int prefill_gemm = 1;   // option "prefill_gemm": 0 = prompts are fed row by row through the decode step
@@ -171,6 +174,9 @@ struct GemvArgs {
 // most wavefronts any GEMV launch uses (sizes the am_val / am_idx scratch)
 constexpr int kGemvMaxWaves = 16384;
 int launch_gemv(const WMat *w, GemvArgs a, int m);
+// the same Linear by the wide-row kernel (gemv_wide.hip: input vector in LDS); a.q / a.d / a.rows / a.cols are set here
+bool gemv_wide_supported(const WMat *w, const GemvArgs &a);
+int launch_gemv_wide(const WMat *w, GemvArgs a, int m);
 int wmat_create_impl(WMat **out, int type, const void *raw, int64_t rows, int64_t cols);
 // true when a register-resident GEMV variant covers the matrix (no temporary is allocated at launch)
 bool gemv_is_direct(const WMat *w);

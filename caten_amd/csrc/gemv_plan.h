@@ -183,6 +183,43 @@ inline GemvPlan gemv_plan(const GemvPlanIn &in) {
   return p;
 }
 
+// The wide-row kernel (gemv_wide.hip): the input vector lives in LDS instead of in registers, so a row may be as
+// wide as LDS holds and the registers a lane needs do not grow with the width.  A round = 64 chunks (one per lane);
+// a tile = nc rounds of a pair of neighbouring rows, requested together; a row = tpr tiles.  lds counts floats: the staged vector, one
+// sum per chunk for 4-bit weights, 16 for the reduction of a norm's statistics.
+struct GemvWidePlan {
+  bool ok = false;
+  int nc = 0, tpr = 0, rw = 1;  // rw: rows a wavefront streams together (1 or 2)
+  unsigned grid = 0, block = 512;
+  size_t lds_floats = 0;
+};
+constexpr size_t kGemvWideMaxLdsBytes = 150 * 1024;
+inline GemvWidePlan gemv_wide_plan(int type, long long rows, long long cols, int compute_units) {
+  GemvWidePlan p;
+  if (type != CTHIP_Q8_0 && type != CTHIP_Q4_0) return p;
+  if (rows <= 0 || rows > 0x7fffffff || cols < 64 || cols % 32 || cols > 0x7fffffff) return p;
+  const int xpc = gemv_xpc(type);
+  const int nchunks = (int)(cols / xpc);
+  p.lds_floats = (size_t)cols + (type == CTHIP_Q4_0 ? (size_t)nchunks : 0) + 16;
+  if (p.lds_floats * 4 > kGemvWideMaxLdsBytes) return p;
+  const int rounds = (nchunks + 63) / 64;
+  // (six 16-byte requests of weights per lane and tile: 3, 2 or 1 rounds of two rows)
+  // (4-bit chunks are 32 inputs wide: with more than one round's inputs between LDS and the arithmetic the kernel
+  // does not fit the 128 registers that let four wavefronts share a SIMD)
+  p.nc = type == CTHIP_Q4_0 ? 1 : rounds % 3 == 0 ? 3 : rounds % 2 == 0 ? 2 : 1;
+  p.tpr = rounds / p.nc;
+  // two workgroups per compute unit where LDS holds two copies of the vector; never more wavefronts than rows
+  const long long per_cu = p.lds_floats * 4 * 2 <= kGemvWideMaxLdsBytes ? 2 : 1;
+  long long grid = (long long)compute_units * per_cu;
+  // rows go in pairs where the pairs still fill every wavefront slot of the launch
+  p.rw = (rows + 1) / 2 >= grid * 8 ? 2 : 1;
+  const long long need = ((rows + p.rw - 1) / p.rw + 7) / 8;
+  if (grid > need) grid = need;
+  p.grid = (unsigned)(grid < 1 ? 1 : grid);
+  p.ok = true;
+  return p;
+}
+
 // How the split-K reduction + norm pass (rowops.hip) lays a row out: `wide` = four wavefronts per row instead of
 // one; `vpl` = the float4-per-lane count of the kernel instantiation chosen (one of 1,2,3,4,6,8 narrow / 1,2,4,8
 // wide); `nz` = the share bucket.  ok is false when no instantiation covers the row.

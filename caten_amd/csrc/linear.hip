@@ -363,7 +363,8 @@ int launch_prologue(float *out, const float *x, int cols, int pro, const float *
 
 bool gemv_is_direct(const WMat *w) {
   int width = 0;
-  return pick_variant(w->type, (int)w->cols) != nullptr || gemv_slices(w->type, (long long)w->cols, &width) > 0;
+  return pick_variant(w->type, (int)w->cols) != nullptr || gemv_slices(w->type, (long long)w->cols, &width) > 0 ||
+         gemv_wide_plan(w->type, w->rows, w->cols, state().compute_units).ok;
 }
 int gemv_rows_per_wave(int type, int64_t cols) {
   const GemvVariant *v = cols <= 0x7fffffff ? pick_variant(type, (int)cols) : nullptr;
@@ -451,6 +452,15 @@ int launch_gemv(const WMat *w, GemvArgs a, int m) {
   const GemvVariant *v = pick_variant(w->type, a.cols);
   if (a.pair_swiglu && (!v || v->G > 32 || (a.rows & 1) || a.am_val || a.residual || a.split1 != a.rows))
     return fail(CTHIP_E_UNSUPPORTED, "gemv: the paired SwiGLU epilogue needs two rows per wavefront and plain outputs");
+  // The wide-row kernel takes the rows no variant covers, and those whose variant holds so much of the input vector
+  // per lane (128 floats: 4-bit rows past 6144 columns, 8-bit rows past 4096) that it needs more than 256 registers
+  // and runs one wavefront per SIMD (Llama-70B shape, 8192-wide 4-bit rows: 12.3 -> 11.8 ms per step; narrower
+  // rows are faster from registers: 7B / 13B shapes 1.83 / 2.96 ms against 2.02 / 3.29 with every launch here).
+  // (a wavefront here takes whole rows: with few rows it leaves compute units idle -- GPT-2 large's 1280 x 5120
+  // projection is slower here, GPT-2 XL's 1600 x 6400, whose variant needs 366 registers, faster)
+  const bool heavy = v && ((w->type == CTHIP_Q4_0 && v->KC >= 4 && a.rows >= 1024) ||
+                           (w->type == CTHIP_Q8_0 && (v->KC >= 8 ? a.rows >= 1024 : v->KC >= 6 && a.rows >= 4096)));
+  if (s.gemv_wide && (!v || heavy || s.gemv_wide >= 2) && gemv_wide_supported(w, a)) return launch_gemv_wide(w, a, m);
   if (v) return launch_variant(v, w, a, m);
   // wider than any variant: column slices, when nothing in the launch needs the whole row at once (a norm of the
   // input, an activation of the sum, an argmax) and the output is one plain vector per input row
@@ -724,6 +734,11 @@ int cthip_set_option(const char *name, int value) {
   if (!strcmp(name, "gemv_stream_weights")) {
     if (value < -1 || value > 1) return fail(CTHIP_E_BAD_ARG, "cthip_set_option: gemv_stream_weights is -1, 0 or 1");
     state().gemv_stream = value;
+    return 0;
+  }
+  if (!strcmp(name, "gemv_wide")) {
+    if (value < 0 || value > 2) return fail(CTHIP_E_BAD_ARG, "cthip_set_option: gemv_wide is 0, 1 or 2");
+    state().gemv_wide = value;
     return 0;
   }
   if (!strcmp(name, "decoder_graph") || !strcmp(name, "prefill_gemm") || !strcmp(name, "decode_fused") ||

@@ -250,6 +250,12 @@ int cthip_linear(float *y, const void *wmat, const float *x, int m, const float 
  *   hint: -1 (default) = per matrix -- a matrix larger than the 256 MB Infinity Cache, and every matrix of a
  *   decoder session whose weights together exceed three quarters of it; 0 = never; 1 = always.  Results do
  *   not depend on it.  A decoder session picks its kernels when it first runs.
+ * "gemv_wide": which single-row Linear launches take the wide-row kernel (input vector staged in LDS instead of
+ *   held in registers; Q8_0 / Q4_0 rows of up to 36 000 columns, no LayerNorm prologue, no fused argmax): 0 = none
+ *   (rows wider than the register-resident kernels cover go as column slices, one launch each), 1 (default) = the
+ *   rows no register-resident kernel covers and those whose register-resident kernel runs one wavefront per SIMD
+ *   (4-bit rows past 6144 columns, 8-bit rows past 4096), 2 = every launch it supports.  Results differ between the two kernel
+ *   families only in summation order.
  * "kv_cache": how decoder sessions created afterwards keep their KV cache: 0 (default) = fp32 rows, the
  *   reference's dense cache (external/llm/layers.lisp:19-33); 1 = GGUF-Q8_0 rows (blocks of 32 int8 and one fp16
  *   scale per cache row, quantised once when the row is appended): 3.76x fewer cache bytes held and read per

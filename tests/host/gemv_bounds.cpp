@@ -201,6 +201,94 @@ static void walk(const Case &c) {
       }
 }
 
+// The wide-row kernel (caten_amd/csrc/gemv_wide.hip: input vector in LDS, rows streamed as tiles of nc rounds): the
+// plan is the library's (gemv_wide_plan), the walk a transcription of k_gemv_wide's requests, LDS traffic and stores.
+static void walk_wide(int type, int rows, int cols, int m_rows, int pro, bool bias, bool residual, bool gamma, int cus) {
+  const GemvWidePlan p = gemv_wide_plan(type, rows, cols, cus);
+  char buf[200];
+  snprintf(buf, sizeof(buf), "wide type %d (%d,%d) m %d pro %d bias %d resid %d gamma %d cus %d", type, rows, cols, m_rows, pro, bias, residual, gamma, cus);
+  g_case = buf;
+  if (!p.ok) return;
+  g_launches++;
+  const bool Q4 = type == CTHIP_Q4_0, swiglu = pro == CTHIP_PRO_SWIGLU, rms = pro == CTHIP_PRO_RMSNORM;
+  const int XPC = gemv_xpc(type), F4 = XPC / 4, NC = p.nc, RW = p.rw, PD = 12 / (NC * RW), tpr = p.tpr;
+  const int nchunks = cols / XPC, n4 = cols >> 2, spr = cols >> 5;
+  const long long x_stride = swiglu ? 2ll * cols : cols, y_stride = rows;
+  Region Q = {"quant plane", true, (Q4 ? cols / 2 : (long long)cols) * rows}, D = {"scale plane", true, 2ll * spr * rows};
+  Region X = {"x", true, 4 * x_stride * m_rows}, NG = {"norm_g", rms && gamma, 4ll * cols}, B = {"bias", bias, 4ll * rows};
+  Region R = {"residual", residual, 4 * y_stride * m_rows}, Y = {"y", true, 4 * y_stride * m_rows};
+  Region LDS = {"LDS", true, 4ll * (long long)p.lds_floats};
+  const long long csum0 = 4ll * cols, red0 = csum0 + (Q4 ? 4ll * nchunks : 0);
+  if (p.lds_floats * 4 > kGemvWideMaxLdsBytes || p.block != 512 || NC * tpr * 64 < nchunks || 12 % (NC * RW) || (RW != 1 && RW != 2)) {
+    g_violations++;
+    printf("VIOLATION %s: plan nc %d tpr %d lds %zu block %u\n", g_case.c_str(), NC, tpr, p.lds_floats, p.block);
+    return;
+  }
+  auto slot = [&](int i) { return (i & ~(F4 - 1)) | ((i ^ (i / F4)) & (F4 - 1)); };
+  const int total_waves = (int)p.grid * 8;
+  for (int m = 0; m < m_rows; m++)
+    for (unsigned bx = 0; bx < p.grid; bx++)
+      for (int tid = 0; tid < 512; tid++) {
+        const int lane = tid & 63, wv = tid >> 6, wave = (int)bx * 8 + wv;
+        const long long xoff = 4 * x_stride * m;
+        const int npairs = (rows + RW - 1) / RW;
+        const int pairs_w = wave < npairs ? (npairs - wave + total_waves - 1) / total_waves : 0, nt = pairs_w * tpr;
+        int rq_pair = wave < npairs ? wave : npairs - 1, rq_grp = 0, rq_left = nt;
+        auto request = [&]() {
+          const int row0 = RW * rq_pair, row1 = row0 + RW - 1 < rows ? row0 + RW - 1 : rows - 1;
+          for (int k = 0; k < NC; k++) {
+            const int c = (rq_grp * NC + k) * 64 + lane;
+            if (c >= nchunks) continue;  // reads the zero block
+            for (int row : {row0, row1}) {
+              touch(Q, ((long long)row * nchunks + c) * 16, 16, "wide tile");
+              touch(D, 2 * ((long long)row * spr + (Q4 ? c : c >> 1)), 2, "wide scale");
+            }
+          }
+          const int er = (lane & 2) ? row1 : row0;
+          const bool want_r = lane & 1;
+          if (want_r ? residual : bias) touch(want_r ? R : B, want_r ? 4 * (y_stride * m + er) : 4ll * er, 4, "wide epilogue request");
+          else if (bias) touch(B, 4ll * er, 4, "wide epilogue request");
+          else if (residual) touch(R, 4 * (y_stride * m + er), 4, "wide epilogue request");
+          if (rq_left > 1) { rq_left--; if (++rq_grp == tpr) { rq_grp = 0; rq_pair += total_waves; } }
+        };
+        request();
+        for (int i = tid; i < n4; i += 512) {
+          touch(X, xoff + 16ll * i, 16, "wide input");
+          if (swiglu) touch(X, xoff + 4ll * cols + 16ll * i, 16, "wide up");
+          else if (rms && gamma) touch(NG, 16ll * i, 16, "wide gamma");
+          touch(LDS, 16ll * slot(i), 16, "wide stage");
+        }
+        if (rms) touch(LDS, red0 + 4 * wv, 4, "wide red");
+        if (Q4)
+          for (int c = tid; c < nchunks; c += 512) {
+            for (int t = 0; t < F4; t++) touch(LDS, 16ll * (F4 * c + (t ^ (c & (F4 - 1)))), 16, "wide chunk sum read");
+            touch(LDS, csum0 + 4ll * c, 4, "wide chunk sum");
+          }
+        for (int pp = 1; pp < PD; pp++) request();
+        int cs_pair = wave, cs_grp = 0;
+        auto consume = [&]() {
+          for (int k = 0; k < NC; k++) {
+            const int c = (cs_grp * NC + k) * 64 + lane, cl = c < nchunks ? c : nchunks - 1;
+            for (int t = 0; t < F4; t++) touch(LDS, 16ll * (F4 * cl + (t ^ (cl & (F4 - 1)))), 16, "wide x read");
+            if (Q4) touch(LDS, csum0 + 4ll * cl, 4, "wide chunk sum read");
+          }
+          if (++cs_grp == tpr) {
+            const int row0 = RW * cs_pair;
+            if (row0 >= rows) { g_violations++; printf("VIOLATION %s: stores row %d\n", g_case.c_str(), row0); }
+            if (lane == 0) touch(Y, 4 * (y_stride * m + row0), 4, "wide store");
+            if (RW > 1 && lane == 1 && row0 + 1 < rows) touch(Y, 4 * (y_stride * m + row0 + 1), 4, "wide store");
+            cs_grp = 0;
+            cs_pair += total_waves;
+          }
+        };
+        int t = 0;
+        for (; t + PD <= nt; t += PD)
+          for (int pp = 0; pp < PD; pp++) { consume(); request(); }
+        for (int pp = 0; pp < PD; pp++)
+          if (t + pp < nt) consume();
+      }
+}
+
 // the split-K reduction + norm pass: whatever (row length, shares, rows) the launcher accepts, the instantiation it
 // picks covers the whole row (lanes x float4 per lane x 4 floats) and keeps its shares within the register budget
 static void check_reduce_norm_plans() {
@@ -227,6 +315,13 @@ static int walk_given_shapes(int argc, char **argv) {
       printf("gemv bounds: shape %d %d %d is not a Linear of the library\n", type, rows, cols);
       return 2;
     }
+    for (int pro : {(int)CTHIP_PRO_NONE, (int)CTHIP_PRO_SWIGLU, (int)CTHIP_PRO_RMSNORM})
+      for (int flags = 0; flags < 4; flags++)
+        for (int mm : {1, 3}) {
+          if (mm == 3 && flags != 3) continue;
+          walk_wide(type, rows, cols, mm, pro, flags & 1, flags & 2, flags & 1, 256);
+        }
+    walk_wide(type, rows, cols, 1, CTHIP_PRO_NONE, true, true, false, 64);
     int width = 0;
     const int nsl = gemv_pick_shape(type, cols) < 0 ? gemv_slices(type, cols, &width) : 0;
     if (nsl > 0) {  // what launch_gemv queues for a row wider than any variant: no norm, no activation, no argmax
@@ -322,6 +417,12 @@ int main(int argc, char **argv) {
       }
     }
   }
+  // the wide-row kernel on widths around its tile sizes, and rows fewer / more than wavefronts
+  for (int type : {CTHIP_Q8_0, CTHIP_Q4_0})
+    for (int cols : {64, 96, 2048, 2080, 4096, 5504, 6144, 8192, 8224, 11008})
+      for (int rows : {1, 7, 513, 4100})
+        for (int pro : {(int)CTHIP_PRO_NONE, (int)CTHIP_PRO_SWIGLU, (int)CTHIP_PRO_RMSNORM})
+          walk_wide(type, rows, cols, rows < 100 ? 3 : 1, pro, rows & 1, cols & 64, true, 256);
   printf("gemv bounds: %lld launches, %lld accesses checked, %lld violations\n", g_launches, g_checked, g_violations);
   return g_violations ? 1 : 0;
 }

@@ -303,14 +303,25 @@ def test_gemv_fallback_shapes_with_prologue(ops, oracle):
     close(ops.linear(x, wm, prologue="layernorm", norm_g=g), oracle.linear(oracle.layernorm(x, g), wd))
 
 
+@pytest.mark.parametrize("wide", [0, 1])
 @pytest.mark.parametrize("kind,rows,cols,m", [("q4_0", 4096, 11008, 1), ("q8_0", 1000, 11008, 1), ("q4_0", 515, 28672, 1),
                                               ("f32", 300, 12288, 1), ("f16", 300, 6400, 1), ("q8_0", 300, 8224, 3)])
-def test_gemv_rows_wider_than_any_variant_go_as_column_slices(ops, oracle, kind, rows, cols, m):
+def test_gemv_rows_wider_than_any_variant(ops, oracle, kind, rows, cols, m, wide):
     """FFN down-projections of 7B-class models and up (11008, 13824, 28672 input features) are wider than what a
-    lane group keeps in registers: the launcher cuts the columns into equal slices, slice 0 carries bias and
-    residual, the others add to it.  Every column gets a weight that a wrong slice offset or row pitch would miss;
-    SwiGLU reads `up` behind the whole gate half, not behind the slice."""
-    print(f"case: sliced gemv {kind} ({rows},{cols}) m {m}", flush=True)
+    lane group keeps in registers.  Quantised rows that LDS holds take the wide-row kernel (option gemv_wide 1, the
+    default); otherwise (gemv_wide 0, fp32 / fp16 rows) the launcher cuts the columns into equal slices, slice 0
+    carries bias and residual, the others add to it.  Every column gets a weight that a wrong chunk index, slice
+    offset or row pitch would miss; SwiGLU reads `up` behind the whole gate half."""
+    print(f"case: wide gemv {kind} ({rows},{cols}) m {m} gemv_wide {wide}", flush=True)
+    from caten_amd import _lib
+    _lib.check(_lib.load().cthip_set_option(b"gemv_wide", wide))
+    try:
+        _wide_rows_case(ops, oracle, kind, rows, cols, m)
+    finally:
+        _lib.check(_lib.load().cthip_set_option(b"gemv_wide", 1))
+
+
+def _wide_rows_case(ops, oracle, kind, rows, cols, m):
     from caten_amd.llm import Tensor
     rng = np.random.default_rng(rows + cols)
     w = rng.normal(0, 0.02, (rows, cols)).astype(np.float32)
@@ -333,6 +344,46 @@ def test_gemv_rows_wider_than_any_variant_go_as_column_slices(ops, oracle, kind,
     g = rng.normal(1, 0.02, cols).astype(np.float32)
     close(ops.linear(xs, wm, act="relu", prologue="rmsnorm", norm_g=g), oracle.relu(oracle.linear(oracle.rmsnorm(xs, g), wd)), **tol)
     wm.free()
+
+
+@pytest.mark.parametrize("kind", ["q4_0", "q8_0"])
+def test_gemv_wide_row_kernel_on_every_launch_it_supports(ops, oracle, kind):
+    """option gemv_wide 2 sends every quantised single-row Linear without a LayerNorm or a fused argmax through the
+    wide-row kernel: widths of one partial round, whole and partial tiles of 1..4 rounds, fewer rows than wavefronts
+    and many more, several input rows, every prologue and epilogue it carries."""
+    from caten_amd import _lib
+    from caten_amd.llm import Tensor
+    lib = _lib.load()
+    tol = dict(rtol=2e-4, atol=2e-4)
+    _lib.check(lib.cthip_set_option(b"gemv_wide", 2))
+    try:
+        for rows, cols, m in [(5, 64, 1), (70, 96, 2), (1000, 2048, 1), (777, 2080, 3), (2304, 768, 1), (640, 4096, 1),
+                              (5000, 5504, 1), (300, 6144, 1), (9, 8192, 7), (16500, 1024, 1)]:
+            print(f"case: wide-row kernel {kind} ({rows},{cols}) m {m}", flush=True)
+            rng = np.random.default_rng(rows * 3 + cols)
+            w = rng.normal(0, 0.02, (rows, cols)).astype(np.float32)
+            w[:, ::61] += 0.05
+            x = rng.normal(0.1, 1, (m, cols)).astype(np.float32)
+            b = rng.normal(0, 0.02, rows).astype(np.float32)
+            r = rng.normal(0, 1, (m, rows)).astype(np.float32)
+            g = rng.normal(1, 0.02, cols).astype(np.float32)
+            t = Tensor.from_f32(w, kind)
+            wd = oracle.dequant(kind, t.raw, w.size).reshape(rows, cols)
+            wm = ops.WeightMatrix(kind, t.raw, rows, cols)
+            xs, rs = (x[0], r[0]) if m == 1 else (x, r)
+            close(ops.linear(xs, wm), oracle.linear(xs, wd), **tol)
+            close(ops.linear(xs, wm, bias=b, residual=rs, act="gelu"), oracle.gelu_tanh(oracle.linear(xs, wd, b)) + rs, **tol)
+            close(ops.linear(xs, wm, residual=rs, prologue="rmsnorm", norm_g=g), oracle.linear(oracle.rmsnorm(xs, g), wd) + rs, **tol)
+            close(ops.linear(xs, wm, bias=b, prologue="rmsnorm"), oracle.linear(oracle.rmsnorm(xs), wd, b), **tol)
+            xu = rng.normal(0, 1, (m, 2 * cols)).astype(np.float32)
+            sw = (oracle.silu(xu[:, :cols]) * xu[:, cols:]).astype(np.float32)
+            xus, sws = (xu[0], sw[0]) if m == 1 else (xu, sw)
+            close(ops.linear(xus, wm, bias=b, prologue="swiglu"), oracle.linear(sws, wd, b), **tol)
+            # a LayerNorm in front keeps the register-resident kernels
+            close(ops.linear(xs, wm, prologue="layernorm", norm_g=g), oracle.linear(oracle.layernorm(xs, g), wd), **tol)
+            wm.free()
+    finally:
+        _lib.check(lib.cthip_set_option(b"gemv_wide", 1))
 
 
 def test_linear_batched_rows(ops, oracle):

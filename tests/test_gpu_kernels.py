@@ -364,6 +364,8 @@ def test_gemv_wide_row_kernel_on_every_launch_it_supports(ops, oracle, kind):
             w = rng.normal(0, 0.02, (rows, cols)).astype(np.float32)
             w[:, ::61] += 0.05
             x = rng.normal(0.1, 1, (m, cols)).astype(np.float32)
+            x[:, 32:64] = 0.0      # a chunk of zeros
+            x[:, 5] = 30.0         # a large input among small ones
             b = rng.normal(0, 0.02, rows).astype(np.float32)
             r = rng.normal(0, 1, (m, rows)).astype(np.float32)
             g = rng.normal(1, 0.02, cols).astype(np.float32)

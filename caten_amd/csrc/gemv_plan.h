@@ -196,9 +196,10 @@ struct GemvWidePlan {
 constexpr size_t kGemvWideMaxLdsBytes = 150 * 1024;
 inline GemvWidePlan gemv_wide_plan(int type, long long rows, long long cols, int compute_units) {
   GemvWidePlan p;
-  if (type != CTHIP_Q8_0 && type != CTHIP_Q4_0) return p;
-  if (rows <= 0 || rows > 0x7fffffff || cols < 64 || cols % 32 || cols > 0x7fffffff) return p;
+  if (type != CTHIP_Q8_0 && type != CTHIP_Q4_0 && type != CTHIP_F16 && type != CTHIP_F32) return p;
   const int xpc = gemv_xpc(type);
+  const bool quant = type == CTHIP_Q8_0 || type == CTHIP_Q4_0;
+  if (rows <= 0 || rows > 0x7fffffff || cols < 64 || cols % (quant ? 32 : xpc) || cols > 0x7fffffff) return p;
   const int nchunks = (int)(cols / xpc);
   p.lds_floats = (size_t)cols + (type == CTHIP_Q4_0 ? (size_t)nchunks : 0) + 16;
   if (p.lds_floats * 4 > kGemvWideMaxLdsBytes) return p;

@@ -1,4 +1,4 @@
-// Single-row Linear for Q8_0 / Q4_0 rows of any width LDS can hold, streamed with the input vector in LDS.
+// Single-row Linear for rows of any width LDS can hold (every weight format), streamed with the input vector in LDS.
 //
 // The register-resident kernels (gemv_kernels.h) give every lane its share of the input vector for the whole
 // launch: 128 floats per lane at 8192 columns of 4-bit weights, which is 304 registers and one wavefront per SIMD
@@ -32,7 +32,7 @@ template <int TYPE, int NC, int RW, bool NT>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4)))
 void k_gemv_wide(GemvArgs a, int tpr) {
   constexpr int XPC = Fmt<TYPE>::XPC, F4 = XPC / 4, PD = 12 / (NC * RW);
-  constexpr bool Q4 = TYPE == CTHIP_Q4_0;
+  constexpr bool Q4 = TYPE == CTHIP_Q4_0, QUANT = TYPE == CTHIP_Q4_0 || TYPE == CTHIP_Q8_0;
   extern __shared__ float wide_lds[];
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int nchunks = a.cols / XPC, n4 = a.cols >> 2;
@@ -63,8 +63,10 @@ void k_gemv_wide(GemvArgs a, int tpr) {
       const int sidx = Q4 ? c : c >> 1;
       wt[p][0][k] = load_chunk<NT>(ok ? qp + (int64_t)row0 * nchunks + c : (const uint4 *)g_gemv_zeros);
       if (RW > 1) wt[p][RW - 1][k] = load_chunk<NT>(ok ? qp + (int64_t)row1 * nchunks + c : (const uint4 *)g_gemv_zeros);
-      st[p][0][k] = *(ok ? a.d + (int64_t)row0 * scales_per_row + sidx : (const unsigned short *)g_gemv_zeros);
-      if (RW > 1) st[p][RW - 1][k] = *(ok ? a.d + (int64_t)row1 * scales_per_row + sidx : (const unsigned short *)g_gemv_zeros);
+      if (QUANT) {
+        st[p][0][k] = *(ok ? a.d + (int64_t)row0 * scales_per_row + sidx : (const unsigned short *)g_gemv_zeros);
+        if (RW > 1) st[p][RW - 1][k] = *(ok ? a.d + (int64_t)row1 * scales_per_row + sidx : (const unsigned short *)g_gemv_zeros);
+      }
     }
     // the rows' bias and residual travel with their tiles: lanes 0, 1 ask for row0's, lanes 2, 3 for row1's
     const int er = (lane & 2) ? row1 : row0;
@@ -140,8 +142,8 @@ void k_gemv_wide(GemvArgs a, int tpr) {
         xl[4 * t] = v.x, xl[4 * t + 1] = v.y, xl[4 * t + 2] = v.z, xl[4 * t + 3] = v.w;
       }
       const float cs = Q4 ? csum[cl] : 0.0f;
-      acc0 += chunk_dot<TYPE>(wt[p][0][k], half_bits_to_float((unsigned short)st[p][0][k]), xl, cs);
-      if (RW > 1) acc1 += chunk_dot<TYPE>(wt[p][RW - 1][k], half_bits_to_float((unsigned short)st[p][RW - 1][k]), xl, cs);
+      acc0 += chunk_dot<TYPE>(wt[p][0][k], QUANT ? half_bits_to_float((unsigned short)st[p][0][k]) : 1.0f, xl, cs);
+      if (RW > 1) acc1 += chunk_dot<TYPE>(wt[p][RW - 1][k], QUANT ? half_bits_to_float((unsigned short)st[p][RW - 1][k]) : 1.0f, xl, cs);
     }
     if (++cs_grp == tpr) {  // (uniform) the pair of rows is complete
       const float s0 = wave_sum(acc0) * rstd, s1 = RW > 1 ? wave_sum(acc1) * rstd : 0.0f;
@@ -194,6 +196,8 @@ int launch_gemv_wide(const WMat *w, GemvArgs a, int m) {
                    : (nt ? k_gemv_wide<T, NC_, 1, true> : k_gemv_wide<T, NC_, 1, false>);
   PICK(CTHIP_Q4_0, 1)
   PICK(CTHIP_Q8_0, 1) PICK(CTHIP_Q8_0, 2) PICK(CTHIP_Q8_0, 3)
+  PICK(CTHIP_F16, 1) PICK(CTHIP_F16, 2) PICK(CTHIP_F16, 3)
+  PICK(CTHIP_F32, 1) PICK(CTHIP_F32, 2) PICK(CTHIP_F32, 3)
 #undef PICK
   if (!fn) return fail(CTHIP_E_STATE, "gemv: no wide-row kernel for %d rounds per tile", p.nc);
   const size_t lds = p.lds_floats * sizeof(float);

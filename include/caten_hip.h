@@ -251,7 +251,7 @@ int cthip_linear(float *y, const void *wmat, const float *x, int m, const float 
  *   decoder session whose weights together exceed three quarters of it; 0 = never; 1 = always.  Results do
  *   not depend on it.  A decoder session picks its kernels when it first runs.
  * "gemv_wide": which single-row Linear launches take the wide-row kernel (input vector staged in LDS instead of
- *   held in registers; Q8_0 / Q4_0 rows of up to 36 000 columns, no LayerNorm prologue, no fused argmax): 0 = none
+ *   held in registers; rows of up to 36 000 columns in any weight format, no LayerNorm prologue, no fused argmax): 0 = none
  *   (rows wider than the register-resident kernels cover go as column slices, one launch each), 1 (default) = the
  *   rows no register-resident kernel covers and those whose register-resident kernel runs one wavefront per SIMD
  *   (4-bit rows past 6144 columns, 8-bit rows past 4096), 2 = every launch it supports.  Results differ between the two kernel

@@ -214,7 +214,9 @@ static void walk_wide(int type, int rows, int cols, int m_rows, int pro, bool bi
   const int XPC = gemv_xpc(type), F4 = XPC / 4, NC = p.nc, RW = p.rw, PD = 12 / (NC * RW), tpr = p.tpr;
   const int nchunks = cols / XPC, n4 = cols >> 2, spr = cols >> 5;
   const long long x_stride = swiglu ? 2ll * cols : cols, y_stride = rows;
-  Region Q = {"quant plane", true, (Q4 ? cols / 2 : (long long)cols) * rows}, D = {"scale plane", true, 2ll * spr * rows};
+  const bool QUANT = Q4 || type == CTHIP_Q8_0;
+  const long long row_bytes = Q4 ? cols / 2 : type == CTHIP_Q8_0 ? cols : type == CTHIP_F16 ? 2ll * cols : 4ll * cols;
+  Region Q = {"quant plane", true, row_bytes * rows}, D = {"scale plane", QUANT, 2ll * spr * rows};
   Region X = {"x", true, 4 * x_stride * m_rows}, NG = {"norm_g", rms && gamma, 4ll * cols}, B = {"bias", bias, 4ll * rows};
   Region R = {"residual", residual, 4 * y_stride * m_rows}, Y = {"y", true, 4 * y_stride * m_rows};
   Region LDS = {"LDS", true, 4ll * (long long)p.lds_floats};
@@ -241,7 +243,7 @@ static void walk_wide(int type, int rows, int cols, int m_rows, int pro, bool bi
             if (c >= nchunks) continue;  // reads the zero block
             for (int row : {row0, row1}) {
               touch(Q, ((long long)row * nchunks + c) * 16, 16, "wide tile");
-              touch(D, 2 * ((long long)row * spr + (Q4 ? c : c >> 1)), 2, "wide scale");
+              if (QUANT) touch(D, 2 * ((long long)row * spr + (Q4 ? c : c >> 1)), 2, "wide scale");
             }
           }
           const int er = (lane & 2) ? row1 : row0;
@@ -418,7 +420,7 @@ int main(int argc, char **argv) {
     }
   }
   // the wide-row kernel on widths around its tile sizes, and rows fewer / more than wavefronts
-  for (int type : {CTHIP_Q8_0, CTHIP_Q4_0})
+  for (int type : {CTHIP_Q8_0, CTHIP_Q4_0, CTHIP_F16, CTHIP_F32})
     for (int cols : {64, 96, 2048, 2080, 4096, 5504, 6144, 8192, 8224, 11008})
       for (int rows : {1, 7, 513, 4100})
         for (int pro : {(int)CTHIP_PRO_NONE, (int)CTHIP_PRO_SWIGLU, (int)CTHIP_PRO_RMSNORM})

@@ -346,9 +346,9 @@ def _wide_rows_case(ops, oracle, kind, rows, cols, m):
     wm.free()
 
 
-@pytest.mark.parametrize("kind", ["q4_0", "q8_0"])
+@pytest.mark.parametrize("kind", ["q4_0", "q8_0", "f16", "f32"])
 def test_gemv_wide_row_kernel_on_every_launch_it_supports(ops, oracle, kind):
-    """option gemv_wide 2 sends every quantised single-row Linear without a LayerNorm or a fused argmax through the
+    """option gemv_wide 2 sends every single-row Linear without a LayerNorm or a fused argmax through the
     wide-row kernel: widths of one partial round, whole and partial tiles of 1..4 rounds, fewer rows than wavefronts
     and many more, several input rows, every prologue and epilogue it carries."""
     from caten_amd import _lib

@@ -4,10 +4,10 @@ reach as the bytes per step grow from 0.13 GB (GPT-2 small, the headline workloa
 round-trip latencies) to tens of GB (a 70B-parameter shape in Q4_0, which one GPU's 288 GB holds).
 
 Shapes: the reference's GPT-2 table (apps/gpt2/gpt2.lisp:36-44) with Q8_0 weights and Llama-shaped models
-(external/llm/layers.lisp; TinyLlama-1.1B is BASELINE's stretch configuration, the larger ones are the public
-Llama-2 shapes) with Q4_0 weights.  Weights are synthetic: ONE layer is drawn and quantised on the host and loaded
-into every layer of the session, so the host work stays small while every layer has its own copy in HBM (a step
-reads every byte of every copy).  One JSON line per model:
+(external/llm/layers.lisp; TinyLlama-1.1B and the public Llama-2 shapes) with Q4_0 weights (--llama-kind q8_0 / f16
+for the other formats).  Weights are synthetic: ONE layer is drawn and quantised on the host and loaded into every
+layer of the session, so the host work stays small while every layer has its own copy in HBM (a step reads every
+byte of every copy).  One JSON line per model:
   {"model", "kind", "weights_GB", "us_per_step", "tokens_per_s", "bytes_per_step", "GBps", "frac", "launches_per_layer"}
 `frac` = algorithmic bytes per step (cthip_decoder_step_bytes) / time / 8 TB/s.
 

@@ -398,7 +398,7 @@ def _run_item(ca, item, arg_values):
 
 
 def test_matmul_item_runs_the_mfma_gemm(oracle):
-    """BASELINE config 1 through the plug-in path: the blueprint of (caten (!relu (!matmul a b))) at 1024^3 is
+    """The 1024^3 matmul configuration through the plug-in path: the blueprint of (caten (!relu (!matmul a b))) at 1024^3 is
     recognised and the launch goes to the MFMA GEMM, not to the rendered thread-per-output kernel; the result is
     the oracle's (rtol 1e-3 / atol 1e-4); with routes switched off the rendered kernel gives the same."""
     import caten_amd as ca

@@ -25,6 +25,9 @@ struct State {
   // option "gemv_wide": which single-row launches take the wide-row kernel (input vector in LDS): 0 = none, 1 = rows
   // no register-resident variant covers or only one that runs a single wavefront per SIMD, 2 = every launch it supports
   int gemv_wide = 1;
+  // option "attn_split": sessions created afterwards share the keys of a head among several workgroups in the decode
+  // attention of the one-launch-per-Linear step (long contexts); 0 = one workgroup per head
+  int attn_split = 1;
   // decoder sessions read these when they first run
   int decoder_graph = 1;  // option "decoder_graph": 0 = the step's launches are issued one by one (kernel tracing)
   int prefill_gemm = 1;   // option "prefill_gemm": 0 = prompts are fed row by row through the decode step
@@ -184,8 +187,15 @@ bool gemv_is_direct(const WMat *w);
 int gemv_rows_per_wave(int type, int64_t cols);
 // out[i] = silu(in[2i]) * in[2i+1], i < n (gate / up columns interleaved)
 int launch_swiglu_pairs(float *out, const float *in, int64_t n);
+// One query row over a long context: `ranges` workgroups per head share the keys (k_attn_cached, SPLIT).  part holds
+// H x ranges x (head_dim + 2) floats, count H zeroed ints (each launch leaves them zeroed again).
+struct AttnSplit {
+  int ranges;
+  float *part;
+  int *count;
+};
 int launch_attn(float *out, const float *q, const float *kc, const float *vc, int S, int start_pos, const int *pos,
-                int max_T, int H, int Hkv, int Dh);
+                int max_T, int H, int Hkv, int Dh, const AttnSplit *split = nullptr);
 int launch_embedding(float *out, const float *W, const float *idx_f, const int *idx_i, int ntok, int vocab, int dim,
                      const float *W2, const int *pos, int max_pos);
 int launch_argmax(int64_t *out, const float *x, int64_t rows, int n, int *tok_out, int *pos, int64_t *history,
@@ -229,7 +239,7 @@ int launch_prologue(float *out, const float *x, int cols, int pro, const float *
 int launch_qkv_split(float *q, float *kc, float *vc, const float *qkv, int S, int start_pos, int H, int Hkv, int Dh,
                      float rope_base);
 int launch_attn_rope_append(float *out, const float *q, float *kc, float *vc, const float *newkv, const int *pos, int H,
-                            int Hkv, int Dh, float base);
+                            int Hkv, int Dh, float base, const AttnSplit *split = nullptr);
 int launch_rope_append(float *kc, float *vc, const float *kv, int Hkv, int Dh, float base, const int *pos);
 int launch_rope(float *out, const float *x, int B, int S, int H, int Dh, float base, int start_pos, const int *pos);
 

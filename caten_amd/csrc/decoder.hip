@@ -82,6 +82,7 @@ struct Decoder {
   float *lm_s = nullptr, *lm_c = nullptr;  // ln_f folded through lm_head
   // activations
   float *x = nullptr, *q = nullptr, *kv_tmp = nullptr, *att = nullptr, *h = nullptr, *logits = nullptr;
+  AttnSplit att_split = {1, nullptr, nullptr};  // the one-launch-per-Linear step: workgroups per head of its attention launch
   // device-resident loop state: [0] = current token, [1] = position
   int *tokpos = nullptr;
   int64_t *token64 = nullptr;
@@ -362,6 +363,17 @@ static int finalize(Decoder *d) {
   TRY(dev_alloc(d, (void **)&d->q, sizeof(float) * D));
   TRY(dev_alloc(d, (void **)&d->kv_tmp, sizeof(float) * 2 * KD));
   TRY(dev_alloc(d, (void **)&d->att, sizeof(float) * D));
+  {
+    // long contexts: the keys of a head shared by as many workgroups as give every compute unit two (at most 16)
+    const int Dh = D / c.n_heads;
+    int ranges = c.max_seq >= 512 ? 2 * state().compute_units / c.n_heads : 1;
+    ranges = ranges < 1 ? 1 : ranges > 16 ? 16 : ranges;
+    if (ranges > 1 && state().attn_split) {
+      TRY(dev_alloc(d, (void **)&d->att_split.part, sizeof(float) * (size_t)c.n_heads * ranges * (Dh + 2)));
+      TRY(dev_alloc(d, (void **)&d->att_split.count, sizeof(int) * (size_t)c.n_heads));  // zero-filled
+      d->att_split.ranges = ranges;
+    }
+  }
   TRY(dev_alloc(d, (void **)&d->h, sizeof(float) * hdim));
   TRY(dev_alloc(d, (void **)&d->logits, sizeof(float) * V));
   TRY(dev_alloc(d, (void **)&d->tokpos, 256));
@@ -751,9 +763,9 @@ static int queue_step(Decoder *d, bool with_head, bool embed) {
     } else if (!gpt2) {
       // q and the new key are rotated inside the attention launch, which also appends k / v at `pos`
       TRY(launch_attn_rope_append(d->att, d->q, L.k_cache, L.v_cache, d->kv_tmp, pos, c.n_heads, c.n_kv_heads, Dh,
-                                  c.rope_base));
+                                  c.rope_base, &d->att_split));
     } else {
-      TRY(launch_attn(d->att, d->q, L.k_cache, L.v_cache, 1, 0, pos, c.max_seq, c.n_heads, c.n_kv_heads, Dh));
+      TRY(launch_attn(d->att, d->q, L.k_cache, L.v_cache, 1, 0, pos, c.max_seq, c.n_heads, c.n_kv_heads, Dh, &d->att_split));
     }
     GemvArgs p = {};
     p.x = d->att;

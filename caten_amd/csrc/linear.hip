@@ -736,6 +736,11 @@ int cthip_set_option(const char *name, int value) {
     state().gemv_stream = value;
     return 0;
   }
+  if (!strcmp(name, "attn_split")) {
+    if (value != 0 && value != 1) return fail(CTHIP_E_BAD_ARG, "cthip_set_option: attn_split is 0 or 1");
+    state().attn_split = value;
+    return 0;
+  }
   if (!strcmp(name, "gemv_wide")) {
     if (value < 0 || value > 2) return fail(CTHIP_E_BAD_ARG, "cthip_set_option: gemv_wide is 0, 1 or 2");
     state().gemv_wide = value;

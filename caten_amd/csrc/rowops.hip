@@ -701,12 +701,21 @@ __global__ __launch_bounds__(256) void k_qkv_split(float *__restrict__ q, float 
 // (positional-encoding.lisp:3-64 at position pos), uses them for key T-1, and the first query head of each
 // kv group stores the rotated key and the value into cache row T-1 -- the rotation and the `!assign` into
 // the cache (layers.lisp:13-33) need no launches of their own.
-template <int DH, bool APPEND>
+//
+// SPLIT (one query row, long contexts): gridDim.z workgroups share a head's keys.  With one workgroup per head a
+// 32-head model reads its cache through 32 compute units (Llama-7B shape at position 1940: 107 us per layer for
+// 64 MB of rows); here the keys are cut into ranges of whole tiles, a workgroup leaves (max, sum, unnormalised
+// output) of its range in `sp_part`, takes a ticket from the head's counter, and the one that draws the last ticket
+// adds the ranges up.  The grid is fixed when the step is captured while the position is device data, so how many
+// ranges are in use is decided here: workgroups past the last range leave at once, and a context of one tile is
+// one range whose workgroup writes the output itself, without a ticket.
+template <int DH, bool APPEND, bool SPLIT>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)))
 void k_attn_cached(float *__restrict__ out, const float *__restrict__ q,
                                                       float *__restrict__ kc, float *__restrict__ vc,
                                                       int start_pos, const int *__restrict__ pos, int H, int Hkv,
-                                                      const float *__restrict__ newkv, float log2_base) {
+                                                      const float *__restrict__ newkv, float log2_base,
+                                                      float *__restrict__ sp_part, int *__restrict__ sp_count) {
   constexpr int LPK = DH / 4;      // lanes per key
   constexpr int KPW = 64 / LPK;    // keys per wavefront per pass
   constexpr int KPT = 4;           // passes held in registers
@@ -714,8 +723,19 @@ void k_attn_cached(float *__restrict__ out, const float *__restrict__ q,
   constexpr int TILE = NW * KPW * KPT;
   __shared__ float part[NW][DH];
   __shared__ float pm[NW], pl[NW];
+  __shared__ int ticket;
   const int h = blockIdx.x, i = blockIdx.y;
   const int T = start_pos + (pos ? pos[0] : 0) + i + 1;
+  // this workgroup's keys [k0, k1): everything, or one of `nranges` ranges of whole tiles
+  int k0 = 0, k1 = T, nranges = 1;
+  if (SPLIT) {
+    const int nz = (int)gridDim.z, tiles = (T + TILE - 1) / TILE;
+    const int per = ((tiles + nz - 1) / nz) * TILE;  // keys per range
+    nranges = (T + per - 1) / per;
+    k0 = (int)blockIdx.z * per;
+    if (k0 >= T) return;  // (uniform) no range for this workgroup
+    k1 = min(T, k0 + per);
+  }
   const int hk = h / (H / Hkv);
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int g = lane / LPK, c = lane % LPK;
@@ -731,7 +751,7 @@ void k_attn_cached(float *__restrict__ out, const float *__restrict__ q,
     q4 = rope4_apply(q4, ra);
     kn = rope4_apply(*(const float4 *)(newkv + hk * DH + 4 * c), ra);
     vn = *(const float4 *)(newkv + KD + hk * DH + 4 * c);
-    if (h % (H / Hkv) == 0 && tid < LPK) {
+    if (h % (H / Hkv) == 0 && tid < LPK && (!SPLIT || blockIdx.z == 0)) {
       ((float4 *)(kc + (int64_t)(T - 1) * KD + hk * DH))[c] = kn;
       ((float4 *)(vc + (int64_t)(T - 1) * KD + hk * DH))[c] = vn;
     }
@@ -770,7 +790,7 @@ void k_attn_cached(float *__restrict__ out, const float *__restrict__ q,
 #pragma unroll
         for (int o = LPK / 2; o > 0; o >>= 1) d += __shfl_xor(d, o, 64);
       }
-      const bool ok = (t0 + (wv * NP + u) * KPW + g) < T;
+      const bool ok = (t0 + (wv * NP + u) * KPW + g) < k1;
       sc[u] = ok ? d * scale : -INFINITY;
       tmax = fmaxf(tmax, sc[u]);
     }
@@ -803,11 +823,11 @@ void k_attn_cached(float *__restrict__ out, const float *__restrict__ q,
     l = l * corr + ps;
     m = m_new;
   };
-  if (T <= TILE) {
-    if (wv * KPT * KPW < T) tile(std::integral_constant<int, KPT>(), 0);  // (uniform per wavefront)
+  if (k1 - k0 <= TILE) {
+    if (k0 + wv * KPT * KPW < k1) tile(std::integral_constant<int, KPT>(), k0);  // (uniform per wavefront)
   } else {
-    for (int t0 = 0; t0 < T; t0 += 2 * TILE) {
-      if (t0 + wv * 2 * KPT * KPW >= T) break;  // nothing left for this wavefront (uniform)
+    for (int t0 = k0; t0 < k1; t0 += 2 * TILE) {
+      if (t0 + wv * 2 * KPT * KPW >= k1) break;  // nothing left for this wavefront (uniform)
       tile(std::integral_constant<int, 2 * KPT>(), t0);
     }
   }
@@ -837,7 +857,42 @@ void k_attn_cached(float *__restrict__ out, const float *__restrict__ q,
       o = fmaf(e, part[w][tid], o);
       L = fmaf(e, pl[w], L);
     }
-    out[((int64_t)i * H + h) * DH + tid] = o / L;
+    if (!SPLIT || nranges == 1) {
+      out[((int64_t)i * H + h) * DH + tid] = o / L;
+    } else {
+      // device-scope stores: written through to memory, no cache to flush (a fence here would write back and
+      // invalidate the whole L2 of the XCD under every other workgroup's key reads: measured 2x slower than no split)
+      float *mine = sp_part + ((int64_t)h * gridDim.z + blockIdx.z) * (DH + 2);
+      __hip_atomic_store(mine + tid, o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (tid == 0) {
+        __hip_atomic_store(mine + DH, M, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(mine + DH + 1, L, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+  }
+  if (SPLIT && nranges > 1) {
+    // a thread's stores have reached memory when the memory counter is back at zero; after the barrier that holds
+    // for the whole workgroup, and only then is its ticket drawn.  The workgroup with the last ticket reads every
+    // range's triple with device-scope loads (which do not look into a cache that could hold an older launch's).
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (tid == 0) ticket = __hip_atomic_fetch_add(sp_count + h, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (ticket != nranges - 1) return;  // (uniform)
+    if (tid < DH) {
+      const float *all = sp_part + (int64_t)h * gridDim.z * (DH + 2);
+      auto ld = [&](int k) { return __hip_atomic_load(all + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+      float M = -INFINITY;
+      for (int r = 0; r < nranges; r++) M = fmaxf(M, ld(r * (DH + 2) + DH));
+      float o = 0.0f, L = 0.0f;
+      for (int r = 0; r < nranges; r++) {
+        const float e = ct_exp(ld(r * (DH + 2) + DH) - M);
+        o = fmaf(e, ld(r * (DH + 2) + tid), o);
+        L = fmaf(e, ld(r * (DH + 2) + DH + 1), L);
+      }
+      out[((int64_t)i * H + h) * DH + tid] = o / L;
+    }
+    if (tid == 0) __hip_atomic_store(sp_count + h, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // the next launch counts again
   }
 }
 
@@ -1324,7 +1379,7 @@ __global__ __launch_bounds__(64 * NW) void k_attn_mfma_bf(float *__restrict__ ou
 }
 
 int launch_attn(float *out, const float *q, const float *kc, const float *vc, int S, int start_pos, const int *pos,
-                int max_T, int H, int Hkv, int Dh) {
+                int max_T, int H, int Hkv, int Dh, const AttnSplit *split) {
   if (S == 0) return 0;
   (void)max_T;
   hipStream_t st = state().stream;
@@ -1361,13 +1416,26 @@ int launch_attn(float *out, const float *q, const float *kc, const float *vc, in
     CTHIP_LAUNCH_CHECK();
     return 0;
   }
-  dim3 grid(H, S), block(1024);
   float *kcw = const_cast<float *>(kc), *vcw = const_cast<float *>(vc);
   const float *nokv = nullptr;
+  float *nop = nullptr;
+  int *noc = nullptr;
+  if (S == 1 && split && split->ranges > 1) {  // one row over a context that may be long: the keys shared by several workgroups
+    dim3 grid(H, 1, split->ranges), block(1024);
+    switch (Dh) {
+      case 32: hipLaunchKernelGGL((k_attn_cached<32, false, true>), grid, block, 0, st, out, q, kcw, vcw, start_pos, pos, H, Hkv, nokv, 0.0f, split->part, split->count); break;
+      case 64: hipLaunchKernelGGL((k_attn_cached<64, false, true>), grid, block, 0, st, out, q, kcw, vcw, start_pos, pos, H, Hkv, nokv, 0.0f, split->part, split->count); break;
+      case 128: hipLaunchKernelGGL((k_attn_cached<128, false, true>), grid, block, 0, st, out, q, kcw, vcw, start_pos, pos, H, Hkv, nokv, 0.0f, split->part, split->count); break;
+      default: return fail(CTHIP_E_UNSUPPORTED, "attention: head_dim %d (supported: 32, 64, 128)", Dh);
+    }
+    CTHIP_LAUNCH_CHECK();
+    return 0;
+  }
+  dim3 grid(H, S), block(1024);
   switch (Dh) {
-    case 32: hipLaunchKernelGGL((k_attn_cached<32, false>), grid, block, 0, st, out, q, kcw, vcw, start_pos, pos, H, Hkv, nokv, 0.0f); break;
-    case 64: hipLaunchKernelGGL((k_attn_cached<64, false>), grid, block, 0, st, out, q, kcw, vcw, start_pos, pos, H, Hkv, nokv, 0.0f); break;
-    case 128: hipLaunchKernelGGL((k_attn_cached<128, false>), grid, block, 0, st, out, q, kcw, vcw, start_pos, pos, H, Hkv, nokv, 0.0f); break;
+    case 32: hipLaunchKernelGGL((k_attn_cached<32, false, false>), grid, block, 0, st, out, q, kcw, vcw, start_pos, pos, H, Hkv, nokv, 0.0f, nop, noc); break;
+    case 64: hipLaunchKernelGGL((k_attn_cached<64, false, false>), grid, block, 0, st, out, q, kcw, vcw, start_pos, pos, H, Hkv, nokv, 0.0f, nop, noc); break;
+    case 128: hipLaunchKernelGGL((k_attn_cached<128, false, false>), grid, block, 0, st, out, q, kcw, vcw, start_pos, pos, H, Hkv, nokv, 0.0f, nop, noc); break;
     default: return fail(CTHIP_E_UNSUPPORTED, "attention: head_dim %d (supported: 32, 64, 128)", Dh);
   }
   CTHIP_LAUNCH_CHECK();
@@ -1376,14 +1444,27 @@ int launch_attn(float *out, const float *q, const float *kc, const float *vc, in
 
 // one decode row of a RoPE model: rotates q and the new key, appends k / v at `pos`, attends (see k_attn_cached)
 int launch_attn_rope_append(float *out, const float *q, float *kc, float *vc, const float *newkv, const int *pos, int H,
-                            int Hkv, int Dh, float base) {
+                            int Hkv, int Dh, float base, const AttnSplit *split) {
   hipStream_t st = state().stream;
-  dim3 grid(H, 1), block(1024);
   const float lb = log2f(base);
+  if (split && split->ranges > 1) {
+    dim3 grid(H, 1, split->ranges), block(1024);
+    switch (Dh) {
+      case 32: hipLaunchKernelGGL((k_attn_cached<32, true, true>), grid, block, 0, st, out, q, kc, vc, 0, pos, H, Hkv, newkv, lb, split->part, split->count); break;
+      case 64: hipLaunchKernelGGL((k_attn_cached<64, true, true>), grid, block, 0, st, out, q, kc, vc, 0, pos, H, Hkv, newkv, lb, split->part, split->count); break;
+      case 128: hipLaunchKernelGGL((k_attn_cached<128, true, true>), grid, block, 0, st, out, q, kc, vc, 0, pos, H, Hkv, newkv, lb, split->part, split->count); break;
+      default: return fail(CTHIP_E_UNSUPPORTED, "attention: head_dim %d (supported: 32, 64, 128)", Dh);
+    }
+    CTHIP_LAUNCH_CHECK();
+    return 0;
+  }
+  dim3 grid(H, 1), block(1024);
+  float *nop = nullptr;
+  int *noc = nullptr;
   switch (Dh) {
-    case 32: hipLaunchKernelGGL((k_attn_cached<32, true>), grid, block, 0, st, out, q, kc, vc, 0, pos, H, Hkv, newkv, lb); break;
-    case 64: hipLaunchKernelGGL((k_attn_cached<64, true>), grid, block, 0, st, out, q, kc, vc, 0, pos, H, Hkv, newkv, lb); break;
-    case 128: hipLaunchKernelGGL((k_attn_cached<128, true>), grid, block, 0, st, out, q, kc, vc, 0, pos, H, Hkv, newkv, lb); break;
+    case 32: hipLaunchKernelGGL((k_attn_cached<32, true, false>), grid, block, 0, st, out, q, kc, vc, 0, pos, H, Hkv, newkv, lb, nop, noc); break;
+    case 64: hipLaunchKernelGGL((k_attn_cached<64, true, false>), grid, block, 0, st, out, q, kc, vc, 0, pos, H, Hkv, newkv, lb, nop, noc); break;
+    case 128: hipLaunchKernelGGL((k_attn_cached<128, true, false>), grid, block, 0, st, out, q, kc, vc, 0, pos, H, Hkv, newkv, lb, nop, noc); break;
     default: return fail(CTHIP_E_UNSUPPORTED, "attention: head_dim %d (supported: 32, 64, 128)", Dh);
   }
   CTHIP_LAUNCH_CHECK();
@@ -1531,7 +1612,7 @@ int cthip_sdpa_cached(float *out, const float *q, const float *k_cache, const fl
   CTHIP_REQUIRE_INIT();
   CTHIP_ARG(S >= 0 && start_pos >= 0 && H > 0 && Hkv > 0 && H % Hkv == 0);
   CTHIP_ARG(S == 0 || (out && q && k_cache && v_cache));
-  return launch_attn(out, q, k_cache, v_cache, S, start_pos, nullptr, start_pos + S, H, Hkv, Dh);
+  return launch_attn(out, q, k_cache, v_cache, S, start_pos, nullptr, start_pos + S, H, Hkv, Dh, nullptr);
 }
 
 }  // extern "C"

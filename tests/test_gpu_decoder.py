@@ -406,3 +406,45 @@ def test_generate_until_stops_on_the_device(name):
     with pytest.raises(HipError):
         model.generate_until(5, cfg["vocab"])
     model.close()
+
+
+@pytest.mark.parametrize("arch,heads,kv_heads,dim,plen", [("llama", 8, 2, 512, 700), ("llama", 4, 4, 512, 1300), ("gpt2", 4, 4, 256, 900),
+                                                          ("llama", 8, 8, 256, 130)])
+def test_decode_attention_with_the_keys_of_a_head_shared_by_workgroups(arch, heads, kv_heads, dim, plen):
+    """One launch per Linear, long contexts: the decode attention cuts a head's keys into ranges of whole tiles, one
+    workgroup each, and the workgroup that draws the last ticket adds the ranges up (option attn_split, on by
+    default).  Same tokens as one workgroup per head, logits inside the fp32 band (the sums are taken in another
+    order), two runs bit-identical (the ranges are added in a fixed order whichever workgroup finishes last);
+    head_dim 64, 128 and 32, grouped-query and plain heads, with the rotation and the append inside the launch and
+    without, contexts of one range and of many."""
+    print(f"case: split decode attention {arch} heads {heads}/{kv_heads} dim {dim} prompt {plen}", flush=True)
+    from caten_amd import _lib, synth, llm
+    lib = _lib.load()
+    if arch == "gpt2":
+        cfg = dict(synth.GPT2_CONFIGS["gpt2-tiny"], n_heads=heads, dim=dim, ffn=4 * dim, max_seq=1536)
+        sd = llm.gpt2_state_dict(synth.gpt2_weights(cfg, seed=17), "q8_0")
+        make = llm.make_gpt2
+    else:
+        cfg = dict(synth.LLAMA_CONFIGS["llama-tiny"], n_heads=heads, n_kv_heads=kv_heads, dim=dim, ffn=2 * dim, max_seq=1536)
+        sd = llm.llama_state_dict(synth.llama_weights(cfg, seed=17), "q8_0")
+        make = llm.make_llama
+    prompt = synth.prompt(cfg["vocab"], plen, seed=17)
+    runs = []
+    try:
+        _lib.check(lib.cthip_set_option(b"decode_fused", 0))
+        for split in (1, 0, 1):
+            _lib.check(lib.cthip_set_option(b"attn_split", split))
+            model = make(cfg, sd)
+            runs.append(llm.gpt2_generate(model, prompt, 24, on_device=False, keep_logits=True))
+            if split:
+                m2 = make(cfg, sd)
+                assert llm.gpt2_generate(m2, prompt, 24, on_device=True) == runs[-1][0]  # inside the step graphs too
+                m2.close()
+            model.close()
+    finally:
+        _lib.check(lib.cthip_set_option(b"decode_fused", 1))
+        _lib.check(lib.cthip_set_option(b"attn_split", 1))
+    assert runs[0][0] == runs[1][0] == runs[2][0]
+    for a, b, c in zip(*[r[1] for r in runs]):
+        close(a, b)
+        assert np.array_equal(a, c)

@@ -5,9 +5,10 @@
 // (measured 3.65 TB/s on a 264 MB matrix), and nothing at all past 8192 columns.  Here a workgroup of eight
 // wavefronts stages the vector once -- with its prologue: SwiGLU, or an RMSNorm folded through the product
 // (gamma * x staged, the row's sum multiplied by rstd at the end) -- and every wavefront streams whole rows: lane l
-// takes chunks l, l + 64, ... of the row, a tile is NC such rounds of two rows requested together, PD = 6 / NC tiles
-// are in flight per wavefront across row boundaries, all requests unconditional (rows past the end repeat the last row and
-// are not stored; chunks past the end of a row read a zero block).  A chunk's 16 / 32 input floats are read from
+// takes chunks l, l + 64, ... of the row, a tile is NC such rounds of RW rows requested together, PD = 12 / (NC RW)
+// tiles are in flight per wavefront across row boundaries (twelve 16-byte requests per lane), all requests
+// unconditional (rows past the end repeat the last row and are not stored; chunks past the end of a row read a zero
+// block).  A chunk's 16 / 32 input floats are read from
 // LDS when its weights have arrived; float4 t of chunk c is stored at position t ^ (c mod 4 or 8) of the chunk, so
 // that the 16-byte reads of neighbouring lanes, 64 or 128 bytes apart, spread over the banks.  4-bit weights need
 // the sum of a chunk's inputs (q - 8 = q minus a constant): one float per chunk, computed once after the staging.

@@ -117,6 +117,11 @@ int launch_kvq_append(void *q, void *d, const float *src, int64_t src_stride, in
 int launch_kvq_dequant(float *dst, const void *q, const void *d, int rows, int KD);
 int launch_attn_q8(float *out, const float *q, const void *kq, const void *kd, const void *vq, const void *vd, int start_pos,
                    const int *pos, int H, int Hkv, int Dh);
+// one decode step over Q8_0 rows: rotation (rope_base > 0), quantisation and append of the new row (newkv: k then v,
+// fp32, unrotated) and the attention in one launch; `split` as for launch_attn
+struct AttnSplit;
+int launch_attn_q8_step(float *out, const float *q, const float *newkv, void *kq, void *kd, void *vq, void *vd, const int *pos,
+                        int H, int Hkv, int Dh, float rope_base, const AttnSplit *split);
 
 // Arguments of one fused Linear launch:
 //   y = act(prologue(x) . W^T + bias) + residual

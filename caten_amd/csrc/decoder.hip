@@ -742,15 +742,10 @@ static int queue_step(Decoder *d, bool with_head, bool embed) {
     }
     TRY(launch_gemv(L.attn, a, 1));
     if (d->kvq) {
-      // the new row is in kv_tmp (k then v): rotate q and k where the model rotates, quantise the row into the
-      // cache at `pos`, attend over the Q8_0 rows
-      if (!gpt2) {
-        TRY(launch_rope(d->q, d->q, 1, 1, c.n_heads, Dh, c.rope_base, 0, pos));
-        TRY(launch_rope(d->kv_tmp, d->kv_tmp, 1, 1, c.n_kv_heads, Dh, c.rope_base, 0, pos));
-      }
-      TRY(launch_kvq_append(L.kq, L.kdq, d->kv_tmp, KD, 1, 0, pos, KD));
-      TRY(launch_kvq_append(L.vq, L.vdq, d->kv_tmp + KD, KD, 1, 0, pos, KD));
-      TRY(launch_attn_q8(d->att, d->q, L.kq, L.kdq, L.vq, L.vdq, 0, pos, c.n_heads, c.n_kv_heads, Dh));
+      // the new row is in kv_tmp (k then v): one launch rotates q and k where the model rotates, quantises the row
+      // into the cache at `pos` and attends over the Q8_0 rows
+      TRY(launch_attn_q8_step(d->att, d->q, d->kv_tmp, L.kq, L.kdq, L.vq, L.vdq, pos, c.n_heads, c.n_kv_heads, Dh,
+                              gpt2 ? 0.0f : c.rope_base, &d->att_split));
     } else if (d->kvp) {
       // the new row is in kv_tmp (k then v): rotate q and k where the model rotates, copy the row into its page,
       // attend over the pages
@@ -1193,7 +1188,7 @@ int cthip_decoder_layer_launches(void *dec) {
   if (d->flow) return 1;  // all layers are ONE launch
   if (d->fused || d->fused_gqa) return 3;  // (GPT-2 shapes: also over a cache of Q8_0 rows)
   if (d->kvp) return d->cfg.arch == CTHIP_ARCH_GPT2 ? 6 : 8;  // + one append (+ two rotations) around the attention launch
-  if (d->kvq) return d->cfg.arch == CTHIP_ARCH_GPT2 ? 7 : 9;  // + two appends (+ two rotations) around the attention launch
+  if (d->kvq) return 5;  // (rotation, quantisation and append of the new row happen inside the attention launch)
   return 5;
 }
 

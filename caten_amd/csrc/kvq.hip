@@ -163,6 +163,235 @@ __global__ __launch_bounds__(256) void k_attn_cached_q8(float *__restrict__ out,
   }
 }
 
+// ---- one decode step over Q8_0 rows in ONE launch ----
+// What a step of a session with such a cache used to queue per layer besides its Linears: rotate q, rotate the new
+// key, quantise and append the key row, the same for the value row, attend.  Here the workgroup does all of it in
+// registers: the head's rotation angles are computed once (one pair per thread, shared through LDS; the pair
+// rotation has the rounding of k_rope), the lane rotates its 16 query elements and its 16 elements of the new key,
+// quantises the new key and value as k_kvq_append does (the planes get the same bits), uses them as key T - 1 and,
+// in the first query head of each key / value head, stores them into the planes.  A head's keys are shared by
+// gridDim.z workgroups as in k_attn_cached's SPLIT form (ranges of whole tiles, device-scope stores of the
+// (max, sum, output) triples, a ticket per range, the last one adds them up in range order).
+template <int DH>
+__global__ __launch_bounds__(256) void k_attn_q8_step(float *__restrict__ out, const float *__restrict__ qv, const float *__restrict__ newkv,
+                                                      signed char *__restrict__ kq, unsigned short *__restrict__ kd,
+                                                      signed char *__restrict__ vq, unsigned short *__restrict__ vd,
+                                                      const int *__restrict__ pos, int H, int Hkv, float log2_base, int rope,
+                                                      float *__restrict__ sp_part, int *__restrict__ sp_count) {
+  constexpr int LPK = DH / 16, KPW = 64 / LPK, KPT = 4, NW = 4, TILE = NW * KPW * KPT;
+  __shared__ float part[NW][DH];
+  __shared__ float pm[NW], pl[NW];
+  __shared__ float ang_s[DH / 2], ang_c[DH / 2];
+  __shared__ int ticket;
+  const int h = blockIdx.x;
+  const int T = pos[0] + 1;
+  int k0 = 0, k1 = T, nranges = 1;
+  {
+    const int nz = (int)gridDim.z, tiles = (T + TILE - 1) / TILE;
+    const int per = ((tiles + nz - 1) / nz) * TILE;  // keys per range
+    nranges = (T + per - 1) / per;
+    k0 = (int)blockIdx.z * per;
+    if (k0 >= T) return;  // (uniform) no range for this workgroup
+    k1 = min(T, k0 + per);
+  }
+  const int group = H / Hkv, hk = h / group;
+  const int KD = Hkv * DH, nb = KD / 32;
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int g = lane / LPK, c = lane % LPK;
+  const int col = hk * DH + 16 * c;  // first of this lane's 16 elements inside a cache row
+  if (rope) {
+    if (tid < DH / 2) {  // theta_i = base^(-2i / DH), as k_rope spells it
+      const float expo = (float)(2 * tid) / (float)DH;
+      const float theta = exp2f(-(expo * (log2_base * 0.6931472f)) * 1.442695f);
+      float sn, cs;
+      sincosf((float)(T - 1) * theta, &sn, &cs);
+      ang_s[tid] = sn;
+      ang_c[tid] = cs;
+    }
+    __syncthreads();
+  }
+  auto load16 = [&](const float *src, float *x) {
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      const float4 v = *(const float4 *)(src + 4 * e);
+      x[4 * e] = v.x, x[4 * e + 1] = v.y, x[4 * e + 2] = v.z, x[4 * e + 3] = v.w;
+    }
+  };
+  auto rotate16 = [&](float *x) {  // pairs 8c .. 8c + 7 of the head
+#pragma unroll
+    for (int t = 0; t < 8; t++) {
+      float o0, o1;
+      rope_pair(x[2 * t], x[2 * t + 1], ang_s[8 * c + t], ang_c[8 * c + t], o0, o1);
+      x[2 * t] = o0, x[2 * t + 1] = o1;
+    }
+  };
+  float qr[16];
+  load16(qv + (int64_t)h * DH + 16 * c, qr);
+  if (rope) rotate16(qr);
+  // the new row of this key / value head: needed by the range that ends at T, and by the one that stores it
+  uint4 knq = make_uint4(0u, 0u, 0u, 0u), vnq = knq;
+  unsigned knd = 0, vnd = 0;
+  const bool has_new = k1 == T, stores = blockIdx.z == 0 && h % group == 0;
+  if (has_new || stores) {  // (uniform)
+    auto quantise = [&](const float *x, uint4 &qv4, unsigned &dv) {  // lanes c and c ^ 1 share a block of 32
+      float amax = 0.0f;
+#pragma unroll
+      for (int e = 0; e < 16; e++) amax = fmaxf(amax, fabsf(x[e]));
+      amax = fmaxf(amax, dpp_f<0xB1>(amax));  // quad_perm [1,0,3,2]
+      const float dd = amax / 127.0f;
+      const float inv = dd != 0.0f ? 1.0f / dd : 0.0f;
+      unsigned w[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+      for (int e = 0; e < 16; e++) {
+        const float t = x[e] * inv;
+        const int r = (int)(t + copysignf(0.5f, t));  // = copysign(floor(|t| + 0.5), t): the conversion truncates
+        w[e >> 2] |= ((unsigned)r & 255u) << (8 * (e & 3));
+      }
+      qv4 = make_uint4(w[0], w[1], w[2], w[3]);
+      dv = __builtin_bit_cast(unsigned short, (_Float16)dd);
+    };
+    float x[16];
+    load16(newkv + col, x);
+    if (rope) rotate16(x);
+    quantise(x, knq, knd);
+    load16(newkv + KD + col, x);
+    quantise(x, vnq, vnd);
+    if (stores && tid < LPK) {  // the `!assign` into the cache row at pos
+      *(uint4 *)(kq + (int64_t)(T - 1) * KD + col) = knq;
+      *(uint4 *)(vq + (int64_t)(T - 1) * KD + col) = vnq;
+      if ((c & 1) == 0) {
+        kd[(int64_t)(T - 1) * nb + (col >> 5)] = (unsigned short)knd;
+        vd[(int64_t)(T - 1) * nb + (col >> 5)] = (unsigned short)vnd;
+      }
+    }
+  }
+  const float scale = 1.0f / sqrtf((float)DH);
+  float m = -INFINITY, l = 0.0f;
+  float acc[16];
+#pragma unroll
+  for (int e = 0; e < 16; e++) acc[e] = 0.0f;
+  auto widen = [](const uint4 w, float *f) {
+    const uint32_t dw[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+      const int v = (int)dw[t];
+      f[4 * t + 0] = (float)(int)(int8_t)v;
+      f[4 * t + 1] = (float)(int)(int8_t)(v >> 8);
+      f[4 * t + 2] = (float)(int)(int8_t)(v >> 16);
+      f[4 * t + 3] = (float)(v >> 24);
+    }
+  };
+  for (int t0 = k0; t0 < k1; t0 += TILE) {
+    if (t0 + wv * KPT * KPW >= k1) break;  // nothing left for this wavefront (uniform)
+    uint4 kr[KPT], vr[KPT];
+    unsigned ks[KPT], vs[KPT];
+#pragma unroll
+    for (int u = 0; u < KPT; u++) {
+      const int j = t0 + (wv * KPT + u) * KPW + g;
+      const int jj = min(j, max(T - 2, 0));  // clamped: masked below; row T - 1 is not in the planes yet
+      kr[u] = *(const uint4 *)(kq + (int64_t)jj * KD + col);
+      vr[u] = *(const uint4 *)(vq + (int64_t)jj * KD + col);
+      ks[u] = kd[(int64_t)jj * nb + (col >> 5)];
+      vs[u] = vd[(int64_t)jj * nb + (col >> 5)];
+      if (j >= T - 1) kr[u] = knq, vr[u] = vnq, ks[u] = knd, vs[u] = vnd;
+    }
+    float sc[KPT];
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < KPT; u++) {
+      float kf[16];
+      widen(kr[u], kf);
+      float dsum = 0.0f;
+#pragma unroll
+      for (int e = 0; e < 16; e++) dsum = fmaf(qr[e], kf[e], dsum);
+      dsum *= half_bits_to_float((unsigned short)ks[u]);
+#pragma unroll
+      for (int o = LPK / 2; o > 0; o >>= 1) dsum += __shfl_xor(dsum, o, 64);
+      const bool ok = (t0 + (wv * KPT + u) * KPW + g) < k1;
+      sc[u] = ok ? dsum * scale : -INFINITY;
+      tmax = fmaxf(tmax, sc[u]);
+    }
+#pragma unroll
+    for (int o = LPK; o < 64; o <<= 1) tmax = fmaxf(tmax, __shfl_xor(tmax, o, 64));
+    const float m_new = fmaxf(m, tmax);   // finite: this wavefront has at least one key here
+    const float corr = ct_exp(m - m_new);  // 0 on its first tile (m = -inf)
+    float ps = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 16; e++) acc[e] *= corr;
+#pragma unroll
+    for (int u = 0; u < KPT; u++) {
+      const float p = ct_exp(sc[u] - m_new);  // exp2(-inf) = 0 for masked keys
+      ps += p;
+      float vf[16];
+      widen(vr[u], vf);
+      const float pv = p * half_bits_to_float((unsigned short)vs[u]);
+#pragma unroll
+      for (int e = 0; e < 16; e++) acc[e] = fmaf(pv, vf[e], acc[e]);
+    }
+#pragma unroll
+    for (int o = LPK; o < 64; o <<= 1) ps += __shfl_xor(ps, o, 64);  // every lane of a key holds the same p
+    l = l * corr + ps;
+    m = m_new;
+  }
+#pragma unroll
+  for (int o = LPK; o < 64; o <<= 1) {
+#pragma unroll
+    for (int e = 0; e < 16; e++) acc[e] += __shfl_xor(acc[e], o, 64);
+  }
+  if (lane < LPK) {
+#pragma unroll
+    for (int e = 0; e < 16; e++) part[wv][16 * lane + e] = acc[e];
+  }
+  if (lane == 0) {
+    pm[wv] = m;
+    pl[wv] = l;
+  }
+  __syncthreads();
+  if (tid < DH) {
+    float M = pm[0];
+#pragma unroll
+    for (int w = 1; w < NW; w++) M = fmaxf(M, pm[w]);
+    float o = 0.0f, L = 0.0f;
+#pragma unroll
+    for (int w = 0; w < NW; w++) {
+      const float e = ct_exp(pm[w] - M);  // wavefronts without keys hold m = -inf: weight 0
+      o = fmaf(e, part[w][tid], o);
+      L = fmaf(e, pl[w], L);
+    }
+    if (nranges == 1) {
+      out[(int64_t)h * DH + tid] = o / L;
+    } else {
+      float *mine = sp_part + ((int64_t)h * gridDim.z + blockIdx.z) * (DH + 2);
+      __hip_atomic_store(mine + tid, o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (tid == 0) {
+        __hip_atomic_store(mine + DH, M, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(mine + DH + 1, L, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+  }
+  if (nranges > 1) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this thread's device-scope stores have reached memory
+    __syncthreads();
+    if (tid == 0) ticket = __hip_atomic_fetch_add(sp_count + h, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (ticket != nranges - 1) return;  // (uniform)
+    if (tid < DH) {
+      const float *all = sp_part + (int64_t)h * gridDim.z * (DH + 2);
+      auto ld = [&](int k) { return __hip_atomic_load(all + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+      float M = -INFINITY;
+      for (int r = 0; r < nranges; r++) M = fmaxf(M, ld(r * (DH + 2) + DH));
+      float o = 0.0f, L = 0.0f;
+      for (int r = 0; r < nranges; r++) {
+        const float e = ct_exp(ld(r * (DH + 2) + DH) - M);
+        o = fmaf(e, ld(r * (DH + 2) + tid), o);
+        L = fmaf(e, ld(r * (DH + 2) + DH + 1), L);
+      }
+      out[(int64_t)h * DH + tid] = o / L;
+    }
+    if (tid == 0) __hip_atomic_store(sp_count + h, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // the next launch counts again
+  }
+}
+
 int launch_kvq_append(void *q, void *d, const float *src, int64_t src_stride, int s, int row0, const int *pos, int KD) {
   if (s <= 0) return 0;
   if (KD % 32) return fail(CTHIP_E_BAD_ARG, "quantised KV cache: rows of %d elements are not whole blocks of 32", KD);
@@ -189,6 +418,28 @@ int launch_attn_q8(float *out, const float *q, const void *kq, const void *kd, c
 #define ATT(DH_)                                                                                                          \
   hipLaunchKernelGGL((k_attn_cached_q8<DH_>), grid, block, 0, st, out, q, (const signed char *)kq, (const unsigned short *)kd, \
                      (const signed char *)vq, (const unsigned short *)vd, start_pos, pos, H, Hkv)
+  switch (Dh) {
+    case 32: ATT(32); break;
+    case 64: ATT(64); break;
+    case 128: ATT(128); break;
+    default: return fail(CTHIP_E_UNSUPPORTED, "quantised KV cache: head_dim %d (supported: 32, 64, 128)", Dh);
+  }
+#undef ATT
+  CTHIP_LAUNCH_CHECK();
+  return 0;
+}
+
+int launch_attn_q8_step(float *out, const float *q, const float *newkv, void *kq, void *kd, void *vq, void *vd, const int *pos,
+                        int H, int Hkv, int Dh, float rope_base, const AttnSplit *split) {
+  if (Hkv <= 0 || H % Hkv) return fail(CTHIP_E_BAD_ARG, "quantised KV cache: %d query heads over %d key / value heads", H, Hkv);
+  const bool shared = split && split->ranges > 1;
+  dim3 grid((unsigned)H, 1, shared ? (unsigned)split->ranges : 1u), block(256);
+  hipStream_t st = state().stream;
+  const int rope = rope_base > 0.0f ? 1 : 0;
+  const float lb = rope ? log2f(rope_base) : 0.0f;
+#define ATT(DH_)                                                                                                                 \
+  hipLaunchKernelGGL((k_attn_q8_step<DH_>), grid, block, 0, st, out, q, newkv, (signed char *)kq, (unsigned short *)kd, (signed char *)vq, \
+                     (unsigned short *)vd, pos, H, Hkv, lb, rope, shared ? split->part : nullptr, shared ? split->count : nullptr)
   switch (Dh) {
     case 32: ATT(32); break;
     case 64: ATT(64); break;

@@ -262,7 +262,7 @@ int cthip_linear(float *y, const void *wmat, const float *x, int m, const float 
  * "kv_cache": how decoder sessions created afterwards keep their KV cache: 0 (default) = fp32 rows, the
  *   reference's dense cache (external/llm/layers.lisp:19-33); 1 = GGUF-Q8_0 rows (blocks of 32 int8 and one fp16
  *   scale per cache row, quantised once when the row is appended): 3.76x fewer cache bytes held and read per
- *   step.  Such a session runs one launch per Linear (GPT-2 shapes: three launches per layer); logits stay within rtol 2e-2 / atol 2e-2 of the fp32
+ *   step.  Such a session runs one launch per Linear + one attention launch (GPT-2 shapes: three launches per layer); logits stay within rtol 2e-2 / atol 2e-2 of the fp32
  *   cache's on the tested models (the band of 8-bit keys and values, not of the fp32 arithmetic around them).
  *   2 = fp32 rows in pages of cthip_kv_page_rows() rows per layer, opened when the position first reaches them
  *   (a session then holds the rows it has used instead of max_seq rows); such a session runs one launch per
@@ -393,8 +393,9 @@ int cthip_decoder_position(const void *dec);
 int64_t cthip_decoder_step_bytes(const void *dec, int t);
 /* Launches per layer of one decode step of this session: 3 (attention + projection and the whole MLP merged,
  * per-XCD accumulators -- taken only when the device passed the load-time checks that XCD ids are 0..7 and that
- * atomics of different workgroups of an XCD meet in its L2), 5 (one launch per Linear + attention), more with a
- * Q8_0 KV cache (the append and, for RoPE models, the rotations are launches of their own).  -1 on error. */
+ * atomics of different workgroups of an XCD meet in its L2), 5 (one launch per Linear + attention; over Q8_0 cache
+ * rows the attention launch also rotates, quantises and appends the new row), more with a paged KV cache (the
+ * append and, for RoPE models, the rotations are launches of their own).  -1 on error. */
 int cthip_decoder_layer_launches(void *dec);
 /* Device pointers into the session, for parity tests: "k_cache.<l>", "v_cache.<l>" (fp32 rows; with a Q8_0
  * cache their dequantised values, in a buffer the next peek overwrites), "logits", "x"; with a Q8_0 cache also

@@ -408,16 +408,18 @@ def test_generate_until_stops_on_the_device(name):
     model.close()
 
 
+@pytest.mark.parametrize("kv", [0, 1])
 @pytest.mark.parametrize("arch,heads,kv_heads,dim,plen", [("llama", 8, 2, 512, 700), ("llama", 4, 4, 512, 1300), ("gpt2", 4, 4, 256, 900),
                                                           ("llama", 8, 8, 256, 130)])
-def test_decode_attention_with_the_keys_of_a_head_shared_by_workgroups(arch, heads, kv_heads, dim, plen):
+def test_decode_attention_with_the_keys_of_a_head_shared_by_workgroups(arch, heads, kv_heads, dim, plen, kv):
     """One launch per Linear, long contexts: the decode attention cuts a head's keys into ranges of whole tiles, one
     workgroup each, and the workgroup that draws the last ticket adds the ranges up (option attn_split, on by
     default).  Same tokens as one workgroup per head, logits inside the fp32 band (the sums are taken in another
     order), two runs bit-identical (the ranges are added in a fixed order whichever workgroup finishes last);
     head_dim 64, 128 and 32, grouped-query and plain heads, with the rotation and the append inside the launch and
-    without, contexts of one range and of many."""
-    print(f"case: split decode attention {arch} heads {heads}/{kv_heads} dim {dim} prompt {plen}", flush=True)
+    without, contexts of one range and of many; over fp32 cache rows (kv 0) and over Q8_0 rows (kv 1: the launch
+    also quantises the new row, and the planes of layer 0 have the same bits either way)."""
+    print(f"case: split decode attention {arch} heads {heads}/{kv_heads} dim {dim} prompt {plen} kv_cache {kv}", flush=True)
     from caten_amd import _lib, synth, llm
     lib = _lib.load()
     if arch == "gpt2":
@@ -429,13 +431,16 @@ def test_decode_attention_with_the_keys_of_a_head_shared_by_workgroups(arch, hea
         sd = llm.llama_state_dict(synth.llama_weights(cfg, seed=17), "q8_0")
         make = llm.make_llama
     prompt = synth.prompt(cfg["vocab"], plen, seed=17)
-    runs = []
+    runs, planes = [], []
     try:
         _lib.check(lib.cthip_set_option(b"decode_fused", 0))
+        _lib.check(lib.cthip_set_option(b"kv_cache", kv))
         for split in (1, 0, 1):
             _lib.check(lib.cthip_set_option(b"attn_split", split))
             model = make(cfg, sd)
             runs.append(llm.gpt2_generate(model, prompt, 24, on_device=False, keep_logits=True))
+            if kv:
+                planes.append(tuple(model.peek(n).view(np.uint8).copy() for n in ("k_cache_q8.0", "k_cache_d.0", "v_cache_q8.0", "v_cache_d.0")))
             if split:
                 m2 = make(cfg, sd)
                 assert llm.gpt2_generate(m2, prompt, 24, on_device=True) == runs[-1][0]  # inside the step graphs too
@@ -444,7 +449,10 @@ def test_decode_attention_with_the_keys_of_a_head_shared_by_workgroups(arch, hea
     finally:
         _lib.check(lib.cthip_set_option(b"decode_fused", 1))
         _lib.check(lib.cthip_set_option(b"attn_split", 1))
+        _lib.check(lib.cthip_set_option(b"kv_cache", 0))
     assert runs[0][0] == runs[1][0] == runs[2][0]
     for a, b, c in zip(*[r[1] for r in runs]):
         close(a, b)
         assert np.array_equal(a, c)
+    for x, y in zip(planes[:1] * 2, planes[1:]):
+        assert all(np.array_equal(p, q) for p, q in zip(x, y))

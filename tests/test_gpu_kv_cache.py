@@ -98,7 +98,7 @@ def test_decoder_with_a_q8_0_cache_stays_in_the_band_of_the_fp32_cache(oracle, a
         _lib.check(lib.cthip_set_option(b"kv_cache", 0))
         _lib.check(lib.cthip_set_option(b"decode_fused", 1))
     (t0, l0, k0, _, n0), (t1, l1, k1, (q1, d1), n1) = runs[0], runs[1]
-    assert n0 == 5 and n1 == (7 if arch == "gpt2" else 9)
+    assert n0 == 5 and n1 == 5  # (the Q8_0 session's attention launch rotates, quantises and appends the new row itself)
     # 8-bit keys and values may turn a near-tie of the greedy choice; from there on the two sessions see other tokens.
     # Everything is compared over the steps that had the same history (at least the prompt and half of the decode).
     same = 0
@@ -243,7 +243,7 @@ def test_three_launch_layer_over_a_q8_0_cache(oracle, name, wtype, plen):
     """GPT-2 shapes keep three launches per layer over Q8_0 cache rows: the attention launch quantises the step's new
     row itself.  Bars: layer 0's planes are the oracle's quantisation of the rows the fp32-cache session of the same
     three-launch layer wrote, bit for bit (decoded rows and batched prompt rows alike); logits inside the 8-bit band of
-    the seven-launch Q8_0 session; two runs bit-identical; the device-resident loop gives the same tokens.  The long
+    the five-launch Q8_0 session; two runs bit-identical; the device-resident loop gives the same tokens.  The long
     prompt makes the decode steps cross the 512 keys one pass of the launch covers."""
     print(f"case: three-launch layer over q8_0 cache {name} {wtype} prompt {plen}", flush=True)
     from caten_amd import _lib, synth, llm
@@ -279,7 +279,7 @@ def test_three_launch_layer_over_a_q8_0_cache(oracle, name, wtype, plen):
         _lib.check(lib.cthip_set_option(b"kv_cache", 0))
         _lib.check(lib.cthip_set_option(b"decode_fused", 1))
     a, b, f, a2 = runs
-    assert (a[2], b[2], f[2]) == (3, 7, 3)
+    assert (a[2], b[2], f[2]) == (3, 5, 3)
     assert a[0] == a2[0] and all(np.array_equal(x, y) for x, y in zip(a[1], a2[1]))
     for (q, d), (q2, d2) in zip(a[4], a2[4]):
         assert np.array_equal(q, q2) and np.array_equal(d, d2)
@@ -290,7 +290,7 @@ def test_three_launch_layer_over_a_q8_0_cache(oracle, name, wtype, plen):
             n += 1
         return n
 
-    # against the seven-launch session over the same kind of cache: a near-tie may turn the greedy choice
+    # against the five-launch session over the same kind of cache: a near-tie may turn the greedy choice
     same = agree(a[0], b[0])
     print("tokens", a[0], b[0], "agree for", same, flush=True)
     assert same >= steps // 2

@@ -113,6 +113,9 @@ int launch_kvp_append(float *const *kpages, float *const *vpages, const float *k
 int launch_kvp_gather(float *dst, const float *const *pages, int rows, int KD);
 int launch_attn_paged(float *out, const float *q, const float *const *kpages, const float *const *vpages, int start_pos,
                       const int *pos, int H, int Hkv, int Dh);
+struct AttnSplit;
+int launch_attn_paged_step(float *out, const float *q, const float *newkv, float *const *kpages, float *const *vpages, const int *pos,
+                           int H, int Hkv, int Dh, float rope_base, const AttnSplit *split);
 int launch_kvq_append(void *q, void *d, const float *src, int64_t src_stride, int s, int row0, const int *pos, int KD);
 int launch_kvq_dequant(float *dst, const void *q, const void *d, int rows, int KD);
 int launch_attn_q8(float *out, const float *q, const void *kq, const void *kd, const void *vq, const void *vd, int start_pos,

@@ -747,14 +747,10 @@ static int queue_step(Decoder *d, bool with_head, bool embed) {
       TRY(launch_attn_q8_step(d->att, d->q, d->kv_tmp, L.kq, L.kdq, L.vq, L.vdq, pos, c.n_heads, c.n_kv_heads, Dh,
                               gpt2 ? 0.0f : c.rope_base, &d->att_split));
     } else if (d->kvp) {
-      // the new row is in kv_tmp (k then v): rotate q and k where the model rotates, copy the row into its page,
-      // attend over the pages
-      if (!gpt2) {
-        TRY(launch_rope(d->q, d->q, 1, 1, c.n_heads, Dh, c.rope_base, 0, pos));
-        TRY(launch_rope(d->kv_tmp, d->kv_tmp, 1, 1, c.n_kv_heads, Dh, c.rope_base, 0, pos));
-      }
-      TRY(launch_kvp_append(L.k_pages, L.v_pages, d->kv_tmp, d->kv_tmp + KD, KD, 1, 0, pos, KD));
-      TRY(launch_attn_paged(d->att, d->q, L.k_pages, L.v_pages, 0, pos, c.n_heads, c.n_kv_heads, Dh));
+      // the new row is in kv_tmp (k then v): one launch rotates q and k where the model rotates, copies the row into
+      // its page and attends over the pages
+      TRY(launch_attn_paged_step(d->att, d->q, d->kv_tmp, L.k_pages, L.v_pages, pos, c.n_heads, c.n_kv_heads, Dh,
+                                 gpt2 ? 0.0f : c.rope_base, &d->att_split));
     } else if (!gpt2) {
       // q and the new key are rotated inside the attention launch, which also appends k / v at `pos`
       TRY(launch_attn_rope_append(d->att, d->q, L.k_cache, L.v_cache, d->kv_tmp, pos, c.n_heads, c.n_kv_heads, Dh,
@@ -1187,9 +1183,7 @@ int cthip_decoder_layer_launches(void *dec) {
   if (rc) return -1;
   if (d->flow) return 1;  // all layers are ONE launch
   if (d->fused || d->fused_gqa) return 3;  // (GPT-2 shapes: also over a cache of Q8_0 rows)
-  if (d->kvp) return d->cfg.arch == CTHIP_ARCH_GPT2 ? 6 : 8;  // + one append (+ two rotations) around the attention launch
-  if (d->kvq) return 5;  // (rotation, quantisation and append of the new row happen inside the attention launch)
-  return 5;
+  return 5;  // (Q8_0 and paged caches too: rotation, quantisation / copy and append of the new row happen inside the attention launch)
 }
 
 int64_t cthip_decoder_step_bytes(const void *dec, int t) {

@@ -44,20 +44,54 @@ __global__ __launch_bounds__(256) void k_kvp_gather(float *__restrict__ dst, con
 // The lane layout of k_attn_cached (rowops.hip): a key row of a head is read by DH/4 adjacent lanes as one float4
 // each, a wavefront holds KPT passes of K and V (all page pointers requested first, then all rows: two memory
 // round trips a tile instead of one), online softmax per wavefront, one meeting in LDS.
-template <int DH>
+//
+// STEP (a session's decode step): the launch also does what k_attn_cached does in its APPEND and SPLIT forms -- the
+// step's new key / value row (newkv: k then v, unrotated) is rotated in registers where the model rotates, used as
+// key T - 1 and copied into its page by the first query head of each key / value head, and the keys of a head are
+// shared by gridDim.z workgroups (ranges of whole tiles, device-scope stores of the (max, sum, output) triples, a
+// ticket per range, the last one adds them up in range order).  The page of row T - 1 was opened by the host before
+// the step was queued.
+template <int DH, bool STEP>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)))
 void k_attn_cached_paged(float *__restrict__ out, const float *__restrict__ q, const float *const *__restrict__ kpages,
-                         const float *const *__restrict__ vpages, int start_pos, const int *__restrict__ pos, int H, int Hkv) {
+                         const float *const *__restrict__ vpages, int start_pos, const int *__restrict__ pos, int H, int Hkv,
+                         const float *__restrict__ newkv, float log2_base, int rope, float *__restrict__ sp_part,
+                         int *__restrict__ sp_count) {
   constexpr int LPK = DH / 4, KPW = 64 / LPK, KPT = 4, NW = 16, TILE = NW * KPW * KPT;
   __shared__ float part[NW][DH];
   __shared__ float pm[NW], pl[NW];
+  __shared__ int ticket;
   const int h = blockIdx.x;
   const int T = start_pos + (pos ? pos[0] : 0) + 1;
+  int k0 = 0, k1 = T, nranges = 1;
+  if (STEP) {
+    const int nz = (int)gridDim.z, tiles = (T + TILE - 1) / TILE;
+    const int per = ((tiles + nz - 1) / nz) * TILE;  // keys per range
+    nranges = (T + per - 1) / per;
+    k0 = (int)blockIdx.z * per;
+    if (k0 >= T) return;  // (uniform) no range for this workgroup
+    k1 = min(T, k0 + per);
+  }
   const int hk = h / (H / Hkv);
   const int KD = Hkv * DH;
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int g = lane / LPK, c = lane % LPK;
-  const float4 q4 = *(const float4 *)(q + (int64_t)h * DH + 4 * c);
+  float4 q4 = *(const float4 *)(q + (int64_t)h * DH + 4 * c);
+  float4 kn = make_float4(0.f, 0.f, 0.f, 0.f), vn = kn;
+  if (STEP) {
+    kn = *(const float4 *)(newkv + hk * DH + 4 * c);
+    vn = *(const float4 *)(newkv + KD + hk * DH + 4 * c);
+    if (rope) {
+      const Rope4 ra = rope4_angles(c, DH, log2_base, T - 1);
+      q4 = rope4_apply(q4, ra);
+      kn = rope4_apply(kn, ra);
+    }
+    if (h % (H / Hkv) == 0 && tid < LPK && blockIdx.z == 0) {  // the `!assign` into the cache row at pos
+      float *kd = const_cast<float *>(kvp_row(kpages, T - 1, KD)), *vd = const_cast<float *>(kvp_row(vpages, T - 1, KD));
+      ((float4 *)(kd + hk * DH))[c] = kn;
+      ((float4 *)(vd + hk * DH))[c] = vn;
+    }
+  }
   const float scale = 1.0f / sqrtf((float)DH);
   float m = -INFINITY, l = 0.0f;
   float acc[4] = {0.f, 0.f, 0.f, 0.f};
@@ -68,7 +102,7 @@ void k_attn_cached_paged(float *__restrict__ out, const float *__restrict__ q, c
 #pragma unroll
     for (int u = 0; u < NP; u++) {
       const int j = t0 + (wv * NP + u) * KPW + g;
-      const int jj = min(j, T - 1);  // clamped: masked below, never a row that has no page yet
+      const int jj = min(j, STEP ? max(T - 2, 0) : T - 1);  // clamped: masked below, never a row that has no page yet; STEP: row T - 1 comes from the registers
       kpg[u] = kpages[jj / kKvPageRows];
       vpg[u] = vpages[jj / kKvPageRows];
       off[u] = (unsigned)(jj % kKvPageRows) * (unsigned)KD + (unsigned)(hk * DH + 4 * c);
@@ -78,6 +112,7 @@ void k_attn_cached_paged(float *__restrict__ out, const float *__restrict__ q, c
     for (int u = 0; u < NP; u++) {
       kr[u] = *(const float4 *)(kpg[u] + off[u]);
       vr[u] = *(const float4 *)(vpg[u] + off[u]);
+      if (STEP && t0 + (wv * NP + u) * KPW + g >= T - 1) kr[u] = kn, vr[u] = vn;
     }
     float sc[NP];
     float tmax = -INFINITY;
@@ -93,7 +128,7 @@ void k_attn_cached_paged(float *__restrict__ out, const float *__restrict__ q, c
 #pragma unroll
         for (int o = LPK / 2; o > 0; o >>= 1) d += __shfl_xor(d, o, 64);
       }
-      const bool ok = (t0 + (wv * NP + u) * KPW + g) < T;
+      const bool ok = (t0 + (wv * NP + u) * KPW + g) < k1;
       sc[u] = ok ? d * scale : -INFINITY;
       tmax = fmaxf(tmax, sc[u]);
     }
@@ -126,11 +161,11 @@ void k_attn_cached_paged(float *__restrict__ out, const float *__restrict__ q, c
     l = l * corr + ps;
     m = m_new;
   };
-  if (T <= TILE) {
-    if (wv * KPT * KPW < T) tile(std::integral_constant<int, KPT>(), 0);  // (uniform per wavefront)
+  if (k1 - k0 <= TILE) {
+    if (k0 + wv * KPT * KPW < k1) tile(std::integral_constant<int, KPT>(), k0);  // (uniform per wavefront)
   } else {
-    for (int t0 = 0; t0 < T; t0 += 2 * TILE) {
-      if (t0 + wv * 2 * KPT * KPW >= T) break;  // nothing left for this wavefront (uniform)
+    for (int t0 = k0; t0 < k1; t0 += 2 * TILE) {
+      if (t0 + wv * 2 * KPT * KPW >= k1) break;  // nothing left for this wavefront (uniform)
       tile(std::integral_constant<int, 2 * KPT>(), t0);
     }
   }
@@ -159,7 +194,37 @@ void k_attn_cached_paged(float *__restrict__ out, const float *__restrict__ q, c
       o = fmaf(e, part[w][tid], o);
       L = fmaf(e, pl[w], L);
     }
-    out[(int64_t)h * DH + tid] = o / L;
+    if (!STEP || nranges == 1) {
+      out[(int64_t)h * DH + tid] = o / L;
+    } else {
+      float *mine = sp_part + ((int64_t)h * gridDim.z + blockIdx.z) * (DH + 2);
+      __hip_atomic_store(mine + tid, o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (tid == 0) {
+        __hip_atomic_store(mine + DH, M, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(mine + DH + 1, L, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+  }
+  if (STEP && nranges > 1) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this thread's device-scope stores have reached memory
+    __syncthreads();
+    if (tid == 0) ticket = __hip_atomic_fetch_add(sp_count + h, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (ticket != nranges - 1) return;  // (uniform)
+    if (tid < DH) {
+      const float *all = sp_part + (int64_t)h * gridDim.z * (DH + 2);
+      auto ld = [&](int k) { return __hip_atomic_load(all + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+      float M = -INFINITY;
+      for (int r = 0; r < nranges; r++) M = fmaxf(M, ld(r * (DH + 2) + DH));
+      float o = 0.0f, L = 0.0f;
+      for (int r = 0; r < nranges; r++) {
+        const float e = ct_exp(ld(r * (DH + 2) + DH) - M);
+        o = fmaf(e, ld(r * (DH + 2) + tid), o);
+        L = fmaf(e, ld(r * (DH + 2) + DH + 1), L);
+      }
+      out[(int64_t)h * DH + tid] = o / L;
+    }
+    if (tid == 0) __hip_atomic_store(sp_count + h, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // the next launch counts again
   }
 }
 
@@ -186,12 +251,42 @@ int launch_attn_paged(float *out, const float *q, const float *const *kpages, co
                       const int *pos, int H, int Hkv, int Dh) {
   dim3 grid(H), block(1024);
   hipStream_t st = state().stream;
+  const float *nokv = nullptr;
+  float *nop = nullptr;
+  int *noc = nullptr;
+#define ATT(DH_) hipLaunchKernelGGL((k_attn_cached_paged<DH_, false>), grid, block, 0, st, out, q, kpages, vpages, start_pos, pos, H, Hkv, nokv, 0.0f, 0, nop, noc)
   switch (Dh) {
-    case 32: hipLaunchKernelGGL((k_attn_cached_paged<32>), grid, block, 0, st, out, q, kpages, vpages, start_pos, pos, H, Hkv); break;
-    case 64: hipLaunchKernelGGL((k_attn_cached_paged<64>), grid, block, 0, st, out, q, kpages, vpages, start_pos, pos, H, Hkv); break;
-    case 128: hipLaunchKernelGGL((k_attn_cached_paged<128>), grid, block, 0, st, out, q, kpages, vpages, start_pos, pos, H, Hkv); break;
+    case 32: ATT(32); break;
+    case 64: ATT(64); break;
+    case 128: ATT(128); break;
     default: return fail(CTHIP_E_UNSUPPORTED, "attention: head_dim %d (supported: 32, 64, 128)", Dh);
   }
+#undef ATT
+  CTHIP_LAUNCH_CHECK();
+  return 0;
+}
+
+// one decode step over a paged cache: rotation (rope_base > 0) and append of the new row (newkv: k then v, fp32,
+// unrotated) and the attention in one launch; `split` as for launch_attn
+int launch_attn_paged_step(float *out, const float *q, const float *newkv, float *const *kpages, float *const *vpages, const int *pos,
+                           int H, int Hkv, int Dh, float rope_base, const AttnSplit *split) {
+  if (Hkv <= 0 || H % Hkv) return fail(CTHIP_E_BAD_ARG, "paged KV cache: %d query heads over %d key / value heads", H, Hkv);
+  const bool shared = split && split->ranges > 1;
+  dim3 grid((unsigned)H, 1, shared ? (unsigned)split->ranges : 1u), block(1024);
+  hipStream_t st = state().stream;
+  const int rope = rope_base > 0.0f ? 1 : 0;
+  const float lb = rope ? log2f(rope_base) : 0.0f;
+#define ATT(DH_)                                                                                                               \
+  hipLaunchKernelGGL((k_attn_cached_paged<DH_, true>), grid, block, 0, st, out, q, (const float *const *)kpages,                  \
+                     (const float *const *)vpages, 0, pos, H, Hkv, newkv, lb, rope, shared ? split->part : nullptr,               \
+                     shared ? split->count : nullptr)
+  switch (Dh) {
+    case 32: ATT(32); break;
+    case 64: ATT(64); break;
+    case 128: ATT(128); break;
+    default: return fail(CTHIP_E_UNSUPPORTED, "attention: head_dim %d (supported: 32, 64, 128)", Dh);
+  }
+#undef ATT
   CTHIP_LAUNCH_CHECK();
   return 0;
 }

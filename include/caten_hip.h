@@ -394,8 +394,8 @@ int64_t cthip_decoder_step_bytes(const void *dec, int t);
 /* Launches per layer of one decode step of this session: 3 (attention + projection and the whole MLP merged,
  * per-XCD accumulators -- taken only when the device passed the load-time checks that XCD ids are 0..7 and that
  * atomics of different workgroups of an XCD meet in its L2), 5 (one launch per Linear + attention; over Q8_0 cache
- * rows the attention launch also rotates, quantises and appends the new row), more with a paged KV cache (the
- * append and, for RoPE models, the rotations are launches of their own).  -1 on error. */
+ * rows and over a paged cache the attention launch also rotates, quantises / copies and appends the new row).
+ * -1 on error. */
 int cthip_decoder_layer_launches(void *dec);
 /* Device pointers into the session, for parity tests: "k_cache.<l>", "v_cache.<l>" (fp32 rows; with a Q8_0
  * cache their dequantised values, in a buffer the next peek overwrites), "logits", "x"; with a Q8_0 cache also

@@ -408,7 +408,7 @@ def test_generate_until_stops_on_the_device(name):
     model.close()
 
 
-@pytest.mark.parametrize("kv", [0, 1])
+@pytest.mark.parametrize("kv", [0, 1, 2])
 @pytest.mark.parametrize("arch,heads,kv_heads,dim,plen", [("llama", 8, 2, 512, 700), ("llama", 4, 4, 512, 1300), ("gpt2", 4, 4, 256, 900),
                                                           ("llama", 8, 8, 256, 130)])
 def test_decode_attention_with_the_keys_of_a_head_shared_by_workgroups(arch, heads, kv_heads, dim, plen, kv):
@@ -418,7 +418,8 @@ def test_decode_attention_with_the_keys_of_a_head_shared_by_workgroups(arch, hea
     order), two runs bit-identical (the ranges are added in a fixed order whichever workgroup finishes last);
     head_dim 64, 128 and 32, grouped-query and plain heads, with the rotation and the append inside the launch and
     without, contexts of one range and of many; over fp32 cache rows (kv 0) and over Q8_0 rows (kv 1: the launch
-    also quantises the new row, and the planes of layer 0 have the same bits either way)."""
+    also quantises the new row, and the planes of layer 0 have the same bits either way) and over fp32 pages (kv 2: the
+    launch also rotates the new row and stores it into its page)."""
     print(f"case: split decode attention {arch} heads {heads}/{kv_heads} dim {dim} prompt {plen} kv_cache {kv}", flush=True)
     from caten_amd import _lib, synth, llm
     lib = _lib.load()
@@ -439,7 +440,7 @@ def test_decode_attention_with_the_keys_of_a_head_shared_by_workgroups(arch, hea
             _lib.check(lib.cthip_set_option(b"attn_split", split))
             model = make(cfg, sd)
             runs.append(llm.gpt2_generate(model, prompt, 24, on_device=False, keep_logits=True))
-            if kv:
+            if kv == 1:
                 planes.append(tuple(model.peek(n).view(np.uint8).copy() for n in ("k_cache_q8.0", "k_cache_d.0", "v_cache_q8.0", "v_cache_d.0")))
             if split:
                 m2 = make(cfg, sd)

@@ -223,7 +223,7 @@ def test_decoder_with_a_paged_cache_equals_the_dense_cache(arch, plen):
         _lib.check(lib.cthip_set_option(b"decode_fused", 1))
     (t0, l0, k0, v0, n0, held0, n_rows), (t2, l2, k2, v2, n2, held2, _) = runs[0], runs[2]
     assert t0 == t2
-    assert n0 == 5 and n2 == (6 if arch == "gpt2" else 8)
+    assert n0 == 5 and n2 == 5  # (the paged session's attention launch rotates and appends the new row itself)
     if arch == "gpt2":
         assert all(np.array_equal(a, b) for a, b in zip(l0, l2))
         assert np.array_equal(k0, k2) and np.array_equal(v0, v2)

@@ -26,7 +26,8 @@ struct State {
   // no register-resident variant covers or only one that runs a single wavefront per SIMD, 2 = every launch it supports
   int gemv_wide = 1;
   // option "attn_split": sessions created afterwards share the keys of a head among several workgroups in the decode
-  // attention of the one-launch-per-Linear step (long contexts); 0 = one workgroup per head
+  // attention of the one-launch-per-Linear step (long contexts): 1 = compute units / heads of them (at most 16),
+  // 2 .. 16 = that many, 0 = one workgroup per head
   int attn_split = 1;
   // decoder sessions read these when they first run
   int decoder_graph = 1;  // option "decoder_graph": 0 = the step's launches are issued one by one (kernel tracing)
@@ -202,6 +203,7 @@ struct AttnSplit {
   float *part;
   int *count;
 };
+constexpr int kAttnSplitMaxRanges = 16;
 int launch_attn(float *out, const float *q, const float *kc, const float *vc, int S, int start_pos, const int *pos,
                 int max_T, int H, int Hkv, int Dh, const AttnSplit *split = nullptr);
 int launch_embedding(float *out, const float *W, const float *idx_f, const int *idx_i, int ntok, int vocab, int dim,
@@ -317,6 +319,35 @@ __device__ __forceinline__ float half_bits_to_float(unsigned short h) {
 // api/high-level-ops.lisp:112-117): exp(x) = exp2(x * 1/ln2); sigmoid = recip(1 + exp2(-x/ln2));
 // tanh(y) = 2*sigmoid(2y) - 1.
 __device__ __forceinline__ float ct_exp(float x) { return exp2f(x * 1.442695f); }
+// The workgroup that drew a head's last ticket adds the ranges' triples up, in range order: `all` holds nranges
+// records of dh unnormalised outputs, the running maximum and the running sum.  The loads are device-scope (they do
+// not look into a cache that could hold an older launch's values) and ALL of them are requested before the first is
+// used, so the merge costs one memory round trip whatever the number of ranges (one load after the other it cost a
+// round trip per range).  Returns output column `col`.
+__device__ __forceinline__ float attn_split_merge(const float *all, int nranges, int dh, int col) {
+  float mv[kAttnSplitMaxRanges], lv[kAttnSplitMaxRanges], ov[kAttnSplitMaxRanges];
+#pragma unroll
+  for (int r = 0; r < kAttnSplitMaxRanges; r++) {
+    const float *t = all + (int64_t)(r < nranges ? r : nranges - 1) * (dh + 2);
+    mv[r] = __hip_atomic_load(t + dh, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    lv[r] = __hip_atomic_load(t + dh + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    ov[r] = __hip_atomic_load(t + col, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  float M = -INFINITY;
+#pragma unroll
+  for (int r = 0; r < kAttnSplitMaxRanges; r++)
+    if (r < nranges) M = fmaxf(M, mv[r]);
+  float o = 0.0f, L = 0.0f;
+#pragma unroll
+  for (int r = 0; r < kAttnSplitMaxRanges; r++) {
+    if (r < nranges) {
+      const float e = ct_exp(mv[r] - M);
+      o = fmaf(e, ov[r], o);
+      L = fmaf(e, lv[r], L);
+    }
+  }
+  return o / L;
+}
 __device__ __forceinline__ float ct_sigmoid(float x) { return 1.0f / (1.0f + exp2f(x * -1.442695f)); }
 __device__ __forceinline__ float ct_tanh(float y) { return 2.0f * ct_sigmoid(2.0f * y) - 1.0f; }
 // GELU(tanh): 0.5 x (1 + tanh(u)) = x sigmoid(2u), u = sqrt(2/pi) (x + 0.044715 x^3) -- the same function without the

@@ -364,10 +364,12 @@ static int finalize(Decoder *d) {
   TRY(dev_alloc(d, (void **)&d->kv_tmp, sizeof(float) * 2 * KD));
   TRY(dev_alloc(d, (void **)&d->att, sizeof(float) * D));
   {
-    // long contexts: the keys of a head shared by as many workgroups as give every compute unit two (at most 16)
+    // long contexts: the keys of a head shared by as many workgroups as give every compute unit one (at most 16):
+    // all of a launch's workgroups are then resident together and ask for their rows at once
     const int Dh = D / c.n_heads;
-    int ranges = c.max_seq >= 512 ? 2 * state().compute_units / c.n_heads : 1;
-    ranges = ranges < 1 ? 1 : ranges > 16 ? 16 : ranges;
+    int ranges = c.max_seq >= 512 ? state().compute_units / c.n_heads : 1;
+    ranges = ranges < 1 ? 1 : ranges > kAttnSplitMaxRanges ? kAttnSplitMaxRanges : ranges;
+    if (state().attn_split > 1) ranges = state().attn_split;  // (a given number of ranges)
     if (ranges > 1 && state().attn_split) {
       TRY(dev_alloc(d, (void **)&d->att_split.part, sizeof(float) * (size_t)c.n_heads * ranges * (Dh + 2)));
       TRY(dev_alloc(d, (void **)&d->att_split.count, sizeof(int) * (size_t)c.n_heads));  // zero-filled

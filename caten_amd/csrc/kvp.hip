@@ -81,21 +81,9 @@ void k_attn_cached_paged(float *__restrict__ out, const float *__restrict__ q, c
   if (STEP) {
     kn = *(const float4 *)(newkv + hk * DH + 4 * c);
     vn = *(const float4 *)(newkv + KD + hk * DH + 4 * c);
-    if (rope) {
-      const Rope4 ra = rope4_angles(c, DH, log2_base, T - 1);
-      q4 = rope4_apply(q4, ra);
-      kn = rope4_apply(kn, ra);
-    }
-    if (h % (H / Hkv) == 0 && tid < LPK && blockIdx.z == 0) {  // the `!assign` into the cache row at pos
-      float *kd = const_cast<float *>(kvp_row(kpages, T - 1, KD)), *vd = const_cast<float *>(kvp_row(vpages, T - 1, KD));
-      ((float4 *)(kd + hk * DH))[c] = kn;
-      ((float4 *)(vd + hk * DH))[c] = vn;
-    }
   }
-  const float scale = 1.0f / sqrtf((float)DH);
-  float m = -INFINITY, l = 0.0f;
-  float acc[4] = {0.f, 0.f, 0.f, 0.f};
-  auto tile = [&](auto np_tag, int t0) {
+  // a tile's rows: the page pointers first, then the rows they address
+  auto request = [&](auto np_tag, int t0, float4 *kr, float4 *vr) {
     constexpr int NP = decltype(np_tag)::value;
     const float *kpg[NP], *vpg[NP];
     unsigned off[NP];
@@ -107,12 +95,37 @@ void k_attn_cached_paged(float *__restrict__ out, const float *__restrict__ q, c
       vpg[u] = vpages[jj / kKvPageRows];
       off[u] = (unsigned)(jj % kKvPageRows) * (unsigned)KD + (unsigned)(hk * DH + 4 * c);
     }
-    float4 kr[NP], vr[NP];
 #pragma unroll
     for (int u = 0; u < NP; u++) {
       kr[u] = *(const float4 *)(kpg[u] + off[u]);
       vr[u] = *(const float4 *)(vpg[u] + off[u]);
-      if (STEP && t0 + (wv * NP + u) * KPW + g >= T - 1) kr[u] = kn, vr[u] = vn;
+    }
+  };
+  // rotation of the query and of the new key, and the new row's store (the `!assign` into the cache row at pos)
+  auto rotate_and_append = [&]() {
+    if (STEP) {
+      if (rope) {
+        const Rope4 ra = rope4_angles(c, DH, log2_base, T - 1);
+        q4 = rope4_apply(q4, ra);
+        kn = rope4_apply(kn, ra);
+      }
+      if (h % (H / Hkv) == 0 && tid < LPK && blockIdx.z == 0) {
+        float *kd = const_cast<float *>(kvp_row(kpages, T - 1, KD)), *vd = const_cast<float *>(kvp_row(vpages, T - 1, KD));
+        ((float4 *)(kd + hk * DH))[c] = kn;
+        ((float4 *)(vd + hk * DH))[c] = vn;
+      }
+    }
+  };
+  const float scale = 1.0f / sqrtf((float)DH);
+  float m = -INFINITY, l = 0.0f;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  auto consume = [&](auto np_tag, int t0, float4 *kr, float4 *vr) {
+    constexpr int NP = decltype(np_tag)::value;
+    if (STEP) {
+#pragma unroll
+      for (int u = 0; u < NP; u++) {
+        if (t0 + (wv * NP + u) * KPW + g >= T - 1) kr[u] = kn, vr[u] = vn;
+      }
     }
     float sc[NP];
     float tmax = -INFINITY;
@@ -161,12 +174,34 @@ void k_attn_cached_paged(float *__restrict__ out, const float *__restrict__ q, c
     l = l * corr + ps;
     m = m_new;
   };
+  // The first tile's rows are asked for as soon as the position is known, before the query is waited for and rotated
+  // (as in k_attn_cached).
   if (k1 - k0 <= TILE) {
-    if (k0 + wv * KPT * KPW < k1) tile(std::integral_constant<int, KPT>(), k0);  // (uniform per wavefront)
+    const bool has_keys = k0 + wv * KPT * KPW < k1;  // (uniform per wavefront)
+    float4 kr[KPT], vr[KPT];
+    if (has_keys) request(std::integral_constant<int, KPT>(), k0, kr, vr);
+    rotate_and_append();
+    if (has_keys) consume(std::integral_constant<int, KPT>(), k0, kr, vr);
   } else {
-    for (int t0 = k0; t0 < k1; t0 += 2 * TILE) {
-      if (t0 + wv * 2 * KPT * KPW >= k1) break;  // nothing left for this wavefront (uniform)
-      tile(std::integral_constant<int, 2 * KPT>(), t0);
+    const bool has_keys = k0 + wv * 2 * KPT * KPW < k1;
+    float4 kr[2 * KPT], vr[2 * KPT];
+    if (has_keys) request(std::integral_constant<int, 2 * KPT>(), k0, kr, vr);
+    rotate_and_append();
+    // (two spellings of one loop: the register allocator keeps each variant of the kernel inside its 128 registers
+    // with one of them only)
+    if (STEP) {
+      for (int t0 = k0; t0 < k1; t0 += 2 * TILE) {
+        if (t0 + wv * 2 * KPT * KPW >= k1) break;  // nothing left for this wavefront (uniform)
+        if (t0 != k0) request(std::integral_constant<int, 2 * KPT>(), t0, kr, vr);
+        consume(std::integral_constant<int, 2 * KPT>(), t0, kr, vr);
+      }
+    } else if (has_keys) {
+      for (int t0 = k0;;) {
+        consume(std::integral_constant<int, 2 * KPT>(), t0, kr, vr);
+        t0 += 2 * TILE;
+        if (t0 + wv * 2 * KPT * KPW >= k1) break;
+        request(std::integral_constant<int, 2 * KPT>(), t0, kr, vr);
+      }
     }
   }
 #pragma unroll
@@ -212,17 +247,7 @@ void k_attn_cached_paged(float *__restrict__ out, const float *__restrict__ q, c
     __syncthreads();
     if (ticket != nranges - 1) return;  // (uniform)
     if (tid < DH) {
-      const float *all = sp_part + (int64_t)h * gridDim.z * (DH + 2);
-      auto ld = [&](int k) { return __hip_atomic_load(all + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
-      float M = -INFINITY;
-      for (int r = 0; r < nranges; r++) M = fmaxf(M, ld(r * (DH + 2) + DH));
-      float o = 0.0f, L = 0.0f;
-      for (int r = 0; r < nranges; r++) {
-        const float e = ct_exp(ld(r * (DH + 2) + DH) - M);
-        o = fmaf(e, ld(r * (DH + 2) + tid), o);
-        L = fmaf(e, ld(r * (DH + 2) + DH + 1), L);
-      }
-      out[(int64_t)h * DH + tid] = o / L;
+      out[(int64_t)h * DH + tid] = attn_split_merge(sp_part + (int64_t)h * gridDim.z * (DH + 2), nranges, DH, tid);
     }
     if (tid == 0) __hip_atomic_store(sp_count + h, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // the next launch counts again
   }
@@ -271,6 +296,7 @@ int launch_attn_paged(float *out, const float *q, const float *const *kpages, co
 int launch_attn_paged_step(float *out, const float *q, const float *newkv, float *const *kpages, float *const *vpages, const int *pos,
                            int H, int Hkv, int Dh, float rope_base, const AttnSplit *split) {
   if (Hkv <= 0 || H % Hkv) return fail(CTHIP_E_BAD_ARG, "paged KV cache: %d query heads over %d key / value heads", H, Hkv);
+  if (split && split->ranges > kAttnSplitMaxRanges) return fail(CTHIP_E_BAD_ARG, "paged KV cache: %d key ranges per head (at most %d)", split->ranges, kAttnSplitMaxRanges);
   const bool shared = split && split->ranges > 1;
   dim3 grid((unsigned)H, 1, shared ? (unsigned)split->ranges : 1u), block(1024);
   hipStream_t st = state().stream;

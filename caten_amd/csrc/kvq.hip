@@ -199,6 +199,22 @@ __global__ __launch_bounds__(256) void k_attn_q8_step(float *__restrict__ out, c
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int g = lane / LPK, c = lane % LPK;
   const int col = hk * DH + 16 * c;  // first of this lane's 16 elements inside a cache row
+  // A tile's rows and scales.  The first tile is asked for as soon as the position is known, before the angles, the
+  // query and the new row are worked on: its round trip to memory runs beside that arithmetic.
+  uint4 kr[KPT], vr[KPT];
+  unsigned ks[KPT], vs[KPT];
+  auto request = [&](int t0) {
+#pragma unroll
+    for (int u = 0; u < KPT; u++) {
+      const int j = t0 + (wv * KPT + u) * KPW + g;
+      const int jj = min(j, max(T - 2, 0));  // clamped: masked below; row T - 1 is not in the planes yet
+      kr[u] = *(const uint4 *)(kq + (int64_t)jj * KD + col);
+      vr[u] = *(const uint4 *)(vq + (int64_t)jj * KD + col);
+      ks[u] = kd[(int64_t)jj * nb + (col >> 5)];
+      vs[u] = vd[(int64_t)jj * nb + (col >> 5)];
+    }
+  };
+  if (k0 + wv * KPT * KPW < k1) request(k0);  // (uniform per wavefront)
   if (rope) {
     if (tid < DH / 2) {  // theta_i = base^(-2i / DH), as k_rope spells it
       const float expo = (float)(2 * tid) / (float)DH;
@@ -283,17 +299,10 @@ __global__ __launch_bounds__(256) void k_attn_q8_step(float *__restrict__ out, c
   };
   for (int t0 = k0; t0 < k1; t0 += TILE) {
     if (t0 + wv * KPT * KPW >= k1) break;  // nothing left for this wavefront (uniform)
-    uint4 kr[KPT], vr[KPT];
-    unsigned ks[KPT], vs[KPT];
+    if (t0 != k0) request(t0);
 #pragma unroll
     for (int u = 0; u < KPT; u++) {
-      const int j = t0 + (wv * KPT + u) * KPW + g;
-      const int jj = min(j, max(T - 2, 0));  // clamped: masked below; row T - 1 is not in the planes yet
-      kr[u] = *(const uint4 *)(kq + (int64_t)jj * KD + col);
-      vr[u] = *(const uint4 *)(vq + (int64_t)jj * KD + col);
-      ks[u] = kd[(int64_t)jj * nb + (col >> 5)];
-      vs[u] = vd[(int64_t)jj * nb + (col >> 5)];
-      if (j >= T - 1) kr[u] = knq, vr[u] = vnq, ks[u] = knd, vs[u] = vnd;
+      if (t0 + (wv * KPT + u) * KPW + g >= T - 1) kr[u] = knq, vr[u] = vnq, ks[u] = knd, vs[u] = vnd;
     }
     float sc[KPT];
     float tmax = -INFINITY;
@@ -376,17 +385,7 @@ __global__ __launch_bounds__(256) void k_attn_q8_step(float *__restrict__ out, c
     __syncthreads();
     if (ticket != nranges - 1) return;  // (uniform)
     if (tid < DH) {
-      const float *all = sp_part + (int64_t)h * gridDim.z * (DH + 2);
-      auto ld = [&](int k) { return __hip_atomic_load(all + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
-      float M = -INFINITY;
-      for (int r = 0; r < nranges; r++) M = fmaxf(M, ld(r * (DH + 2) + DH));
-      float o = 0.0f, L = 0.0f;
-      for (int r = 0; r < nranges; r++) {
-        const float e = ct_exp(ld(r * (DH + 2) + DH) - M);
-        o = fmaf(e, ld(r * (DH + 2) + tid), o);
-        L = fmaf(e, ld(r * (DH + 2) + DH + 1), L);
-      }
-      out[(int64_t)h * DH + tid] = o / L;
+      out[(int64_t)h * DH + tid] = attn_split_merge(sp_part + (int64_t)h * gridDim.z * (DH + 2), nranges, DH, tid);
     }
     if (tid == 0) __hip_atomic_store(sp_count + h, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // the next launch counts again
   }
@@ -432,6 +431,7 @@ int launch_attn_q8(float *out, const float *q, const void *kq, const void *kd, c
 int launch_attn_q8_step(float *out, const float *q, const float *newkv, void *kq, void *kd, void *vq, void *vd, const int *pos,
                         int H, int Hkv, int Dh, float rope_base, const AttnSplit *split) {
   if (Hkv <= 0 || H % Hkv) return fail(CTHIP_E_BAD_ARG, "quantised KV cache: %d query heads over %d key / value heads", H, Hkv);
+  if (split && split->ranges > kAttnSplitMaxRanges) return fail(CTHIP_E_BAD_ARG, "quantised KV cache: %d key ranges per head (at most %d)", split->ranges, kAttnSplitMaxRanges);
   const bool shared = split && split->ranges > 1;
   dim3 grid((unsigned)H, 1, shared ? (unsigned)split->ranges : 1u), block(256);
   hipStream_t st = state().stream;

@@ -737,7 +737,7 @@ int cthip_set_option(const char *name, int value) {
     return 0;
   }
   if (!strcmp(name, "attn_split")) {
-    if (value != 0 && value != 1) return fail(CTHIP_E_BAD_ARG, "cthip_set_option: attn_split is 0 or 1");
+    if (value < 0 || value > kAttnSplitMaxRanges) return fail(CTHIP_E_BAD_ARG, "cthip_set_option: attn_split is 0, 1 or a number of key ranges per head up to %d", kAttnSplitMaxRanges);
     state().attn_split = value;
     return 0;
   }

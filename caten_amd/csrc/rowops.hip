@@ -746,24 +746,14 @@ void k_attn_cached(float *__restrict__ out, const float *__restrict__ q,
   const float scale = 1.0f / sqrtf((float)DH);
   float4 kn = make_float4(0.f, 0.f, 0.f, 0.f), vn = kn;
   if (APPEND) {
-    const int KD = Hkv * DH;
-    const Rope4 ra = rope4_angles(c, DH, log2_base, T - 1);
-    q4 = rope4_apply(q4, ra);
-    kn = rope4_apply(*(const float4 *)(newkv + hk * DH + 4 * c), ra);
-    vn = *(const float4 *)(newkv + KD + hk * DH + 4 * c);
-    if (h % (H / Hkv) == 0 && tid < LPK && (!SPLIT || blockIdx.z == 0)) {
-      ((float4 *)(kc + (int64_t)(T - 1) * KD + hk * DH))[c] = kn;
-      ((float4 *)(vc + (int64_t)(T - 1) * KD + hk * DH))[c] = vn;
-    }
+    kn = *(const float4 *)(newkv + hk * DH + 4 * c);
+    vn = *(const float4 *)(newkv + Hkv * DH + hk * DH + 4 * c);
   }
-  float m = -INFINITY, l = 0.0f;
-  float acc[4] = {0.f, 0.f, 0.f, 0.f};
   // One tile = NP key passes per wavefront, all requested together: wavefront wv owns keys t0 + (wv*NP + u)*KPW + g.
   // Up to TILE keys that is KPT passes; a longer context takes tiles of twice as many passes, so that positions up
   // to twice as far still cost one memory round trip instead of two.
-  auto tile = [&](auto np_tag, int t0) {
+  auto request = [&](auto np_tag, int t0, float4 *kr, float4 *vr) {
     constexpr int NP = decltype(np_tag)::value;
-    float4 kr[NP], vr[NP];
 #pragma unroll
     for (int u = 0; u < NP; u++) {
       const int j = t0 + (wv * NP + u) * KPW + g;
@@ -771,9 +761,33 @@ void k_attn_cached(float *__restrict__ out, const float *__restrict__ q,
       const unsigned jj = (unsigned)min(j, APPEND ? max(T - 2, 0) : T - 1);
       kr[u] = kp[jj * kvs4];
       vr[u] = vp[jj * kvs4];
-      if (APPEND && j >= T - 1) {
-        kr[u] = kn;
-        vr[u] = vn;
+    }
+  };
+  // rotation of the query and of the new key, and the new row's store.  The angles need the position alone and many
+  // registers for a moment: they are worked out before the rows are asked for, the rotation itself afterwards.
+  auto rotate_and_append = [&]() {
+    if (APPEND) {
+      const int KD = Hkv * DH;
+      const Rope4 ra = rope4_angles(c, DH, log2_base, T - 1);
+      q4 = rope4_apply(q4, ra);
+      kn = rope4_apply(kn, ra);
+      if (h % (H / Hkv) == 0 && tid < LPK && (!SPLIT || blockIdx.z == 0)) {
+        ((float4 *)(kc + (int64_t)(T - 1) * KD + hk * DH))[c] = kn;
+        ((float4 *)(vc + (int64_t)(T - 1) * KD + hk * DH))[c] = vn;
+      }
+    }
+  };
+  float m = -INFINITY, l = 0.0f;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  auto consume = [&](auto np_tag, int t0, float4 *kr, float4 *vr) {
+    constexpr int NP = decltype(np_tag)::value;
+    if (APPEND) {
+#pragma unroll
+      for (int u = 0; u < NP; u++) {
+        if (t0 + (wv * NP + u) * KPW + g >= T - 1) {
+          kr[u] = kn;
+          vr[u] = vn;
+        }
       }
     }
     float sc[NP];
@@ -823,12 +837,34 @@ void k_attn_cached(float *__restrict__ out, const float *__restrict__ q,
     l = l * corr + ps;
     m = m_new;
   };
+  // The first tile's rows are asked for as soon as the position is known, BEFORE the query is waited for and rotated:
+  // their round trip to memory runs beside the query's, the new row's and the angles' arithmetic.
   if (k1 - k0 <= TILE) {
-    if (k0 + wv * KPT * KPW < k1) tile(std::integral_constant<int, KPT>(), k0);  // (uniform per wavefront)
+    const bool has_keys = k0 + wv * KPT * KPW < k1;  // (uniform per wavefront)
+    float4 kr[KPT], vr[KPT];
+    if (has_keys) request(std::integral_constant<int, KPT>(), k0, kr, vr);
+    rotate_and_append();
+    if (has_keys) consume(std::integral_constant<int, KPT>(), k0, kr, vr);
   } else {
-    for (int t0 = k0; t0 < k1; t0 += 2 * TILE) {
-      if (t0 + wv * 2 * KPT * KPW >= k1) break;  // nothing left for this wavefront (uniform)
-      tile(std::integral_constant<int, 2 * KPT>(), t0);
+    const bool has_keys = k0 + wv * 2 * KPT * KPW < k1;
+    float4 kr[2 * KPT], vr[2 * KPT];
+    if (has_keys) request(std::integral_constant<int, 2 * KPT>(), k0, kr, vr);
+    rotate_and_append();
+    // (two spellings of one loop: the register allocator keeps each variant of the kernel inside its 128 registers
+    // with one of them only)
+    if (APPEND) {
+      for (int t0 = k0; t0 < k1; t0 += 2 * TILE) {
+        if (t0 + wv * 2 * KPT * KPW >= k1) break;  // nothing left for this wavefront (uniform)
+        if (t0 != k0) request(std::integral_constant<int, 2 * KPT>(), t0, kr, vr);
+        consume(std::integral_constant<int, 2 * KPT>(), t0, kr, vr);
+      }
+    } else if (has_keys) {
+      for (int t0 = k0;;) {
+        consume(std::integral_constant<int, 2 * KPT>(), t0, kr, vr);
+        t0 += 2 * TILE;
+        if (t0 + wv * 2 * KPT * KPW >= k1) break;
+        request(std::integral_constant<int, 2 * KPT>(), t0, kr, vr);
+      }
     }
   }
   // combine the key groups inside the wavefront, then the wavefronts through LDS
@@ -880,17 +916,7 @@ void k_attn_cached(float *__restrict__ out, const float *__restrict__ q,
     __syncthreads();
     if (ticket != nranges - 1) return;  // (uniform)
     if (tid < DH) {
-      const float *all = sp_part + (int64_t)h * gridDim.z * (DH + 2);
-      auto ld = [&](int k) { return __hip_atomic_load(all + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
-      float M = -INFINITY;
-      for (int r = 0; r < nranges; r++) M = fmaxf(M, ld(r * (DH + 2) + DH));
-      float o = 0.0f, L = 0.0f;
-      for (int r = 0; r < nranges; r++) {
-        const float e = ct_exp(ld(r * (DH + 2) + DH) - M);
-        o = fmaf(e, ld(r * (DH + 2) + tid), o);
-        L = fmaf(e, ld(r * (DH + 2) + DH + 1), L);
-      }
-      out[((int64_t)i * H + h) * DH + tid] = o / L;
+      out[((int64_t)i * H + h) * DH + tid] = attn_split_merge(sp_part + (int64_t)h * gridDim.z * (DH + 2), nranges, DH, tid);
     }
     if (tid == 0) __hip_atomic_store(sp_count + h, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // the next launch counts again
   }
@@ -1420,6 +1446,7 @@ int launch_attn(float *out, const float *q, const float *kc, const float *vc, in
   const float *nokv = nullptr;
   float *nop = nullptr;
   int *noc = nullptr;
+  if (split && split->ranges > kAttnSplitMaxRanges) return fail(CTHIP_E_BAD_ARG, "attention: %d key ranges per head (at most %d)", split->ranges, kAttnSplitMaxRanges);
   if (S == 1 && split && split->ranges > 1) {  // one row over a context that may be long: the keys shared by several workgroups
     dim3 grid(H, 1, split->ranges), block(1024);
     switch (Dh) {
@@ -1447,6 +1474,7 @@ int launch_attn_rope_append(float *out, const float *q, float *kc, float *vc, co
                             int Hkv, int Dh, float base, const AttnSplit *split) {
   hipStream_t st = state().stream;
   const float lb = log2f(base);
+  if (split && split->ranges > kAttnSplitMaxRanges) return fail(CTHIP_E_BAD_ARG, "attention: %d key ranges per head (at most %d)", split->ranges, kAttnSplitMaxRanges);
   if (split && split->ranges > 1) {
     dim3 grid(H, 1, split->ranges), block(1024);
     switch (Dh) {

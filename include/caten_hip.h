@@ -257,8 +257,9 @@ int cthip_linear(float *y, const void *wmat, const float *x, int m, const float 
  *   (4-bit rows past 6144 columns, 8-bit rows past 4096), 2 = every launch it supports.  Results differ between the two kernel
  *   families only in summation order.
  * "attn_split": 1 (default) = decoder sessions created afterwards that run one launch per Linear and have
- *   max_seq >= 512 share the keys of a head among up to 16 workgroups in their decode attention (long contexts);
- *   0 = one workgroup per head.  Same tokens; logits differ in summation order only.
+ *   max_seq >= 512 share the keys of a head among (compute units / heads) workgroups, at most 16, in their decode
+ *   attention (long contexts); 2 .. 16 = that many workgroups per head; 0 = one workgroup per head.  Same tokens;
+ *   logits differ in summation order only.
  * "kv_cache": how decoder sessions created afterwards keep their KV cache: 0 (default) = fp32 rows, the
  *   reference's dense cache (external/llm/layers.lisp:19-33); 1 = GGUF-Q8_0 rows (blocks of 32 int8 and one fp16
  *   scale per cache row, quantised once when the row is appended): 3.76x fewer cache bytes held and read per

@@ -436,13 +436,13 @@ def test_decode_attention_with_the_keys_of_a_head_shared_by_workgroups(arch, hea
     try:
         _lib.check(lib.cthip_set_option(b"decode_fused", 0))
         _lib.check(lib.cthip_set_option(b"kv_cache", kv))
-        for split in (1, 0, 1):
+        for split in (1, 0, 1, 3):  # (3: exactly three key ranges per head)
             _lib.check(lib.cthip_set_option(b"attn_split", split))
             model = make(cfg, sd)
             runs.append(llm.gpt2_generate(model, prompt, 24, on_device=False, keep_logits=True))
             if kv == 1:
                 planes.append(tuple(model.peek(n).view(np.uint8).copy() for n in ("k_cache_q8.0", "k_cache_d.0", "v_cache_q8.0", "v_cache_d.0")))
-            if split:
+            if split == 1:
                 m2 = make(cfg, sd)
                 assert llm.gpt2_generate(m2, prompt, 24, on_device=True) == runs[-1][0]  # inside the step graphs too
                 m2.close()
@@ -451,9 +451,10 @@ def test_decode_attention_with_the_keys_of_a_head_shared_by_workgroups(arch, hea
         _lib.check(lib.cthip_set_option(b"decode_fused", 1))
         _lib.check(lib.cthip_set_option(b"attn_split", 1))
         _lib.check(lib.cthip_set_option(b"kv_cache", 0))
-    assert runs[0][0] == runs[1][0] == runs[2][0]
-    for a, b, c in zip(*[r[1] for r in runs]):
+    assert runs[0][0] == runs[1][0] == runs[2][0] == runs[3][0]
+    for a, b, c, d in zip(*[r[1] for r in runs]):
         close(a, b)
+        close(a, d)
         assert np.array_equal(a, c)
-    for x, y in zip(planes[:1] * 2, planes[1:]):
+    for x, y in zip(planes[:1] * 3, planes[1:]):
         assert all(np.array_equal(p, q) for p, q in zip(x, y))

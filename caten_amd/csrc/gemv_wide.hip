@@ -90,15 +90,31 @@ void k_gemv_wide(GemvArgs a, int tpr) {
   const float4 *x4 = (const float4 *)x;
   const float4 *u4 = swiglu ? (const float4 *)(x + a.cols) : (rms && a.norm_g) ? (const float4 *)a.norm_g : x4;
   float s2 = 0.0f;
-  for (int i = tid; i < n4; i += 512) {
-    const float4 v = x4[i], u = u4[i];
-    float4 o = v;
-    if (swiglu) o = make_float4(ct_silu(v.x) * u.x, ct_silu(v.y) * u.y, ct_silu(v.z) * u.z, ct_silu(v.w) * u.w);
-    if (rms) {
-      s2 = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, fmaf(v.w, v.w, s2))));
-      if (a.norm_g) o = make_float4(v.x * u.x, v.y * u.y, v.z * u.z, v.w * u.w);
+  // SB pieces of the vector (and of its partner: SwiGLU's other half, the norm's gamma) are asked for together: a
+  // piece per loop iteration would cost a memory round trip each
+  constexpr int SB = 6;
+  for (int i0 = tid; i0 < n4; i0 += 512 * SB) {
+    float4 vb[SB], ub[SB];
+#pragma unroll
+    for (int b = 0; b < SB; b++) {
+      const int i = min(i0 + 512 * b, n4 - 1);
+      vb[b] = x4[i];
+      ub[b] = u4[i];
     }
-    ((float4 *)xs)[wide_slot<F4>(i)] = o;
+#pragma unroll
+    for (int b = 0; b < SB; b++) {
+      const int i = i0 + 512 * b;
+      if (i < n4) {
+        const float4 v = vb[b], u = ub[b];
+        float4 o = v;
+        if (swiglu) o = make_float4(ct_silu(v.x) * u.x, ct_silu(v.y) * u.y, ct_silu(v.z) * u.z, ct_silu(v.w) * u.w);
+        if (rms) {
+          s2 = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, fmaf(v.w, v.w, s2))));
+          if (a.norm_g) o = make_float4(v.x * u.x, v.y * u.y, v.z * u.z, v.w * u.w);
+        }
+        ((float4 *)xs)[wide_slot<F4>(i)] = o;
+      }
+    }
   }
   if (rms) {
     s2 = wave_sum(s2);

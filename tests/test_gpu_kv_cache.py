@@ -175,13 +175,14 @@ def test_append_and_attention_over_paged_rows(oracle, H, Hkv, Dh):
         assert np.allclose(got, want, rtol=1e-3, atol=1e-4), (T, float(np.max(np.abs(got - want))))
 
 
-@pytest.mark.parametrize("arch,plen", [("gpt2", 3), ("gpt2", 70), ("llama", 3), ("llama", 70)])
+@pytest.mark.parametrize("arch,plen", [("gpt2", 3), ("gpt2", 70), ("llama", 3), ("llama", 70), ("gpt2", 600), ("llama", 600)])
 def test_decoder_with_a_paged_cache_equals_the_dense_cache(arch, plen):
     """A session whose cache lives in pages against one with the dense cache, both with one launch per Linear: a prompt
     fed row by row or as one batch that crosses a page edge, then decode steps across another edge.  Same tokens; for
     the GPT-2 shape the same logits and cache rows bit for bit (the arithmetic is the same); where the model rotates,
-    q and k are rotated by a launch of their own instead of inside the attention launch, so logits are compared inside
-    the fp32 band (rtol 1e-3 / atol 1e-4).  The paged session holds the rows it has reached, not max_seq rows."""
+    logits are compared inside the fp32 band (rtol 1e-3 / atol 1e-4).  The prompts of 600 reach contexts whose keys
+    several workgroups per head share, in both sessions.  The paged session holds the rows it has reached, not
+    max_seq rows."""
     print(f"case: decoder with paged cache {arch} prompt {plen}", flush=True)
     import ctypes as C
     from caten_amd import _lib, synth, llm
@@ -234,7 +235,10 @@ def test_decoder_with_a_paged_cache_equals_the_dense_cache(arch, plen):
     assert not k2[n_rows:].any()  # rows never reached read as zeros, as the dense cache holds them
     # the dense session holds max_seq rows per layer, the paged one three pages (139 or 72 rows reached)
     dense_rows = 2 * cfg["n_layers"] * cfg["max_seq"] * kd * 4
-    assert held0 - held2 > dense_rows // 2, (held0, held2, dense_rows)
+    if n_rows <= 256:
+        assert held0 - held2 > dense_rows // 2, (held0, held2, dense_rows)
+    else:
+        assert held0 > held2, (held0, held2)
 
 
 @pytest.mark.parametrize("name,wtype,plen", [("gpt2-tiny", "q8_0", 3), ("gpt2-tiny", "q4_0", 20), ("gpt2-mini", "q8_0", 5),

@@ -29,6 +29,9 @@ struct State {
   // attention of the one-launch-per-Linear step (long contexts): 1 = compute units / heads of them (at most 16),
   // 2 .. 16 = that many, 0 = one workgroup per head
   int attn_split = 1;
+  // option "attn_long_from": the position from which sessions with a three-launch layer give the attention a launch
+  // of its own (keys shared by several workgroups, then the projection): four launches per layer; 0 = never
+  int attn_long_from = 896;
   // decoder sessions read these when they first run
   int decoder_graph = 1;  // option "decoder_graph": 0 = the step's launches are issued one by one (kernel tracing)
   int prefill_gemm = 1;   // option "prefill_gemm": 0 = prompts are fed row by row through the decode step

@@ -60,6 +60,7 @@ struct DecAttnArgs {
   float *part;               // out: fp32 [H][D], head h's share of the projection
   void *zero;                // cleared here: the MLP accumulators
   int64_t zero_n16;          // ... in 16-byte units
+  const float *att_in;       // null, or the heads' attention outputs [H][Dh] from a launch of its own: projection only
 };
 
 // the same launch over a cache kept as Q8_0 rows (kvq.hip): the step's new key / value row arrives as fp32 (k then v,
@@ -276,6 +277,7 @@ struct GqaAttnArgs {
   void *zero;                // cleared here: the MLP launch's accumulators
   int64_t zero_n16;
   int D, KD;
+  const float *att_in;       // null, or the heads' attention outputs [H][Dh] from a launch of its own: projection only
 };
 
 struct GqaMlpArgs {

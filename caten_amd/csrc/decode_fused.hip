@@ -171,7 +171,7 @@ __global__ __launch_bounds__(256) void k_dec_qkv(DecQkvArgs a) {
 // holds four passes of K and V in registers, per-wavefront online softmax, one meeting in LDS.  The head's
 // slab of the projection (D rows x DH columns, contiguous after the re-layout) does not depend on anything
 // computed here and is requested first, so it arrives while the keys are being processed.
-template <int TYPE, int DH, int JR>
+template <int TYPE, int DH, int JR, bool ATT_IN>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)))
 void k_dec_attn_proj(DecAttnArgs a) {
   constexpr int LPK = DH / 4, KPW = 64 / LPK, KPT = 4, NW = 16, TILE = NW * KPW * KPT;
@@ -197,118 +197,126 @@ void k_dec_attn_proj(DecAttnArgs a) {
     pw[j] = ((const uint4 *)a.pq)[((int64_t)h * D + r) * CPR + pc];
     ps[j] = DecFmt<TYPE>::QUANT ? a.pd[((int64_t)h * D + r) * (DH / 32) + ((pc * XPC) >> 5)] : 0;
   }
-  const int T = a.pos[0] + 1;
-  const unsigned kvs4 = (unsigned)(D / 4);
-  const float4 q4 = *(const float4 *)(a.q + h * DH + 4 * c);
-  const float4 *__restrict__ kp = (const float4 *)(a.kc + h * DH) + c;
-  const float4 *__restrict__ vp = (const float4 *)(a.vc + h * DH) + c;
-  const float scale = 1.0f / sqrtf((float)DH);
   // the accumulators of the MLP launch are cleared here: their last reader (this layer's k_dec_qkv) has finished
-  {
+  auto clear_accumulators = [&]() {
     uint4 *z = (uint4 *)a.zero;
     const uint4 zz = make_uint4(0u, 0u, 0u, 0u);
     const int64_t nthr = (int64_t)H * gridDim.y * 1024;
     for (int64_t k = ((int64_t)blockIdx.y * H + h) * 1024 + tid; k < a.zero_n16; k += nthr) z[k] = zz;
-  }
-  float m = -INFINITY, lsum = 0.0f;
-  float acc[4] = {0.f, 0.f, 0.f, 0.f};
-  // One tile = NP key passes per wavefront, all requested together: wavefront wv owns keys t0 + (wv*NP + u)*KPW + g.
-  // Up to 16*KPW*KPT keys that is KPT passes; a longer context takes tiles of twice as many passes, so that
-  // positions up to twice as far still cost ONE memory round trip instead of two.
-  auto tile = [&](auto np_tag, int t0) {
-    constexpr int NP = decltype(np_tag)::value;
-    float4 kr[NP], vr[NP];
-#pragma unroll
-    for (int u = 0; u < NP; u++) {
-      const int j = t0 + (wv * NP + u) * KPW + g;
-      const unsigned jj = (unsigned)min(j, T - 1);  // clamped: masked below, never outside the cache
-      kr[u] = kp[jj * kvs4];
-      vr[u] = vp[jj * kvs4];
-    }
-    float sc[NP];
-    float tmax = -INFINITY;
-#pragma unroll
-    for (int u = 0; u < NP; u++) {
-      float d = q4.x * kr[u].x;
-      d = fmaf(q4.y, kr[u].y, d);
-      d = fmaf(q4.z, kr[u].z, d);
-      d = fmaf(q4.w, kr[u].w, d);
-      // over the key's 16 lanes: data-parallel-primitive adds, no trip through the LDS crossbar
-      if (LPK == 16) {
-        d = row16_sum(d);
-      } else {
-#pragma unroll
-        for (int o = LPK / 2; o > 0; o >>= 1) d += __shfl_xor(d, o, 64);
-      }
-      const bool ok = (t0 + (wv * NP + u) * KPW + g) < T;
-      sc[u] = ok ? d * scale : -INFINITY;
-      tmax = fmaxf(tmax, sc[u]);
-    }
-    if (LPK == 16) {
-      tmax = groups16_max(tmax);
-    } else {
-#pragma unroll
-      for (int o = LPK; o < 64; o <<= 1) tmax = fmaxf(tmax, __shfl_xor(tmax, o, 64));
-    }
-    const float m_new = fmaxf(m, tmax);
-    const float corr = ct_exp(m - m_new);
-    float psum = 0.0f;
-#pragma unroll
-    for (int k2 = 0; k2 < 4; k2++) acc[k2] *= corr;
-#pragma unroll
-    for (int u = 0; u < NP; u++) {
-      const float p = ct_exp(sc[u] - m_new);
-      psum += p;
-      acc[0] = fmaf(p, vr[u].x, acc[0]);
-      acc[1] = fmaf(p, vr[u].y, acc[1]);
-      acc[2] = fmaf(p, vr[u].z, acc[2]);
-      acc[3] = fmaf(p, vr[u].w, acc[3]);
-    }
-    if (LPK == 16) {
-      psum = groups16_sum(psum);
-    } else {
-#pragma unroll
-      for (int o = LPK; o < 64; o <<= 1) psum += __shfl_xor(psum, o, 64);
-    }
-    lsum = lsum * corr + psum;
-    m = m_new;
   };
-  if (T <= TILE) {
-    if (wv * KPT * KPW < T) tile(std::integral_constant<int, KPT>(), 0);  // (uniform per wavefront)
+  if constexpr (ATT_IN) {
+    clear_accumulators();
+    // the head's attention was computed by a launch of its own (long contexts: its keys shared by several workgroups)
+    if (tid < DH) oh[tid] = a.att_in[h * DH + tid];
+    __syncthreads();
   } else {
-    for (int t0 = 0; t0 < T; t0 += 2 * TILE) {
-      if (t0 + wv * 2 * KPT * KPW >= T) break;  // nothing left for this wavefront (uniform)
-      tile(std::integral_constant<int, 2 * KPT>(), t0);
+    const int T = a.pos[0] + 1;
+    const unsigned kvs4 = (unsigned)(D / 4);
+    const float4 q4 = *(const float4 *)(a.q + h * DH + 4 * c);
+    const float4 *__restrict__ kp = (const float4 *)(a.kc + h * DH) + c;
+    const float4 *__restrict__ vp = (const float4 *)(a.vc + h * DH) + c;
+    const float scale = 1.0f / sqrtf((float)DH);
+    clear_accumulators();
+    float m = -INFINITY, lsum = 0.0f;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    // One tile = NP key passes per wavefront, all requested together: wavefront wv owns keys t0 + (wv*NP + u)*KPW + g.
+    // Up to 16*KPW*KPT keys that is KPT passes; a longer context takes tiles of twice as many passes, so that
+    // positions up to twice as far still cost ONE memory round trip instead of two.
+    auto tile = [&](auto np_tag, int t0) {
+      constexpr int NP = decltype(np_tag)::value;
+      float4 kr[NP], vr[NP];
+  #pragma unroll
+      for (int u = 0; u < NP; u++) {
+        const int j = t0 + (wv * NP + u) * KPW + g;
+        const unsigned jj = (unsigned)min(j, T - 1);  // clamped: masked below, never outside the cache
+        kr[u] = kp[jj * kvs4];
+        vr[u] = vp[jj * kvs4];
+      }
+      float sc[NP];
+      float tmax = -INFINITY;
+  #pragma unroll
+      for (int u = 0; u < NP; u++) {
+        float d = q4.x * kr[u].x;
+        d = fmaf(q4.y, kr[u].y, d);
+        d = fmaf(q4.z, kr[u].z, d);
+        d = fmaf(q4.w, kr[u].w, d);
+        // over the key's 16 lanes: data-parallel-primitive adds, no trip through the LDS crossbar
+        if (LPK == 16) {
+          d = row16_sum(d);
+        } else {
+  #pragma unroll
+          for (int o = LPK / 2; o > 0; o >>= 1) d += __shfl_xor(d, o, 64);
+        }
+        const bool ok = (t0 + (wv * NP + u) * KPW + g) < T;
+        sc[u] = ok ? d * scale : -INFINITY;
+        tmax = fmaxf(tmax, sc[u]);
+      }
+      if (LPK == 16) {
+        tmax = groups16_max(tmax);
+      } else {
+  #pragma unroll
+        for (int o = LPK; o < 64; o <<= 1) tmax = fmaxf(tmax, __shfl_xor(tmax, o, 64));
+      }
+      const float m_new = fmaxf(m, tmax);
+      const float corr = ct_exp(m - m_new);
+      float psum = 0.0f;
+  #pragma unroll
+      for (int k2 = 0; k2 < 4; k2++) acc[k2] *= corr;
+  #pragma unroll
+      for (int u = 0; u < NP; u++) {
+        const float p = ct_exp(sc[u] - m_new);
+        psum += p;
+        acc[0] = fmaf(p, vr[u].x, acc[0]);
+        acc[1] = fmaf(p, vr[u].y, acc[1]);
+        acc[2] = fmaf(p, vr[u].z, acc[2]);
+        acc[3] = fmaf(p, vr[u].w, acc[3]);
+      }
+      if (LPK == 16) {
+        psum = groups16_sum(psum);
+      } else {
+  #pragma unroll
+        for (int o = LPK; o < 64; o <<= 1) psum += __shfl_xor(psum, o, 64);
+      }
+      lsum = lsum * corr + psum;
+      m = m_new;
+    };
+    if (T <= TILE) {
+      if (wv * KPT * KPW < T) tile(std::integral_constant<int, KPT>(), 0);  // (uniform per wavefront)
+    } else {
+      for (int t0 = 0; t0 < T; t0 += 2 * TILE) {
+        if (t0 + wv * 2 * KPT * KPW >= T) break;  // nothing left for this wavefront (uniform)
+        tile(std::integral_constant<int, 2 * KPT>(), t0);
+      }
     }
-  }
-#pragma unroll
-  for (int o = LPK; o < 64; o <<= 1) {
-#pragma unroll
-    for (int k2 = 0; k2 < 4; k2++) acc[k2] += __shfl_xor(acc[k2], o, 64);
-  }
-  if (lane < LPK) {
-#pragma unroll
-    for (int k2 = 0; k2 < 4; k2++) part[wv][4 * lane + k2] = acc[k2];
-  }
-  if (lane == 0) {
-    pm[wv] = m;
-    pl[wv] = lsum;
-  }
-  __syncthreads();
-  if (tid < DH) {
-    float M = pm[0];
-#pragma unroll
-    for (int w = 1; w < NW; w++) M = fmaxf(M, pm[w]);
-    float o = 0.0f, L = 0.0f;
-#pragma unroll
-    for (int w = 0; w < NW; w++) {
-      const float e = ct_exp(pm[w] - M);
-      o = fmaf(e, part[w][tid], o);
-      L = fmaf(e, pl[w], L);
+  #pragma unroll
+    for (int o = LPK; o < 64; o <<= 1) {
+  #pragma unroll
+      for (int k2 = 0; k2 < 4; k2++) acc[k2] += __shfl_xor(acc[k2], o, 64);
     }
-    oh[tid] = o / L;
+    if (lane < LPK) {
+  #pragma unroll
+      for (int k2 = 0; k2 < 4; k2++) part[wv][4 * lane + k2] = acc[k2];
+    }
+    if (lane == 0) {
+      pm[wv] = m;
+      pl[wv] = lsum;
+    }
+    __syncthreads();
+    if (tid < DH) {
+      float M = pm[0];
+  #pragma unroll
+      for (int w = 1; w < NW; w++) M = fmaxf(M, pm[w]);
+      float o = 0.0f, L = 0.0f;
+  #pragma unroll
+      for (int w = 0; w < NW; w++) {
+        const float e = ct_exp(pm[w] - M);
+        o = fmaf(e, part[w][tid], o);
+        L = fmaf(e, pl[w], L);
+      }
+      oh[tid] = o / L;
+    }
+    __syncthreads();
   }
-  __syncthreads();
   // partial projection: row r of the slab times the head's outputs; CPR lanes share a row
   float xr[XPC];
   lds_floats<XPC>(oh + pc * XPC, xr);
@@ -796,12 +804,21 @@ int launch_dec_attn_proj(const DecAttnArgs &a, int type, int H, int D, int repli
   // passes over the slab rows: (D / replicas) rows of 64 / xpc chunks over 1024 threads
   const int rpp = 1024 / (64 / xpc), jr = (D / replicas + rpp - 1) / rpp;
   if (jr > 4) return fail(CTHIP_E_BAD_ARG, "decoder: fused attention launch needs %d passes over its slab", jr);
-#define GO_T(T)                                                                              \
-  switch (jr) {                                                                              \
-    case 1: hipLaunchKernelGGL((k_dec_attn_proj<T, 64, 1>), grid, block, 0, st, a); break;   \
-    case 2: hipLaunchKernelGGL((k_dec_attn_proj<T, 64, 2>), grid, block, 0, st, a); break;   \
-    case 3: hipLaunchKernelGGL((k_dec_attn_proj<T, 64, 3>), grid, block, 0, st, a); break;   \
-    default: hipLaunchKernelGGL((k_dec_attn_proj<T, 64, 4>), grid, block, 0, st, a); break;  \
+#define GO_T(T)                                                                                     \
+  if (a.att_in) {                                                                                   \
+    switch (jr) {                                                                                   \
+      case 1: hipLaunchKernelGGL((k_dec_attn_proj<T, 64, 1, true>), grid, block, 0, st, a); break;  \
+      case 2: hipLaunchKernelGGL((k_dec_attn_proj<T, 64, 2, true>), grid, block, 0, st, a); break;  \
+      case 3: hipLaunchKernelGGL((k_dec_attn_proj<T, 64, 3, true>), grid, block, 0, st, a); break;  \
+      default: hipLaunchKernelGGL((k_dec_attn_proj<T, 64, 4, true>), grid, block, 0, st, a); break; \
+    }                                                                                               \
+  } else {                                                                                          \
+    switch (jr) {                                                                                   \
+      case 1: hipLaunchKernelGGL((k_dec_attn_proj<T, 64, 1, false>), grid, block, 0, st, a); break;  \
+      case 2: hipLaunchKernelGGL((k_dec_attn_proj<T, 64, 2, false>), grid, block, 0, st, a); break;  \
+      case 3: hipLaunchKernelGGL((k_dec_attn_proj<T, 64, 3, false>), grid, block, 0, st, a); break;  \
+      default: hipLaunchKernelGGL((k_dec_attn_proj<T, 64, 4, false>), grid, block, 0, st, a); break; \
+    }                                                                                               \
   }
   DEC_TYPES(GO_T)
 #undef GO_T

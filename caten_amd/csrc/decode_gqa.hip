@@ -188,7 +188,7 @@ __global__ __launch_bounds__(NT) void k_gqa_qkv(GqaQkvArgs a) {
 // Attention as in k_dec_attn_proj; the key / value rows are those of the head's group.  The head's slab of wo
 // (D rows x two Q4_0 blocks) is requested first.  gridDim.y workgroups per head repeat the attention and share
 // the slab's rows.
-template <int JR>
+template <int JR, bool ATT_IN>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4)))
 void k_gqa_attn_proj(GqaAttnArgs a) {
   constexpr int DH = 64, LPK = DH / 4, KPW = 64 / LPK, KPT = 4, NW = 16, TILE = NW * KPW * KPT;
@@ -211,100 +211,106 @@ void k_gqa_attn_proj(GqaAttnArgs a) {
     pw[j] = ((const uint4 *)a.pq)[idx];
     ps[j] = a.pd[idx];
   }
-  const int T = a.pos[0] + 1;
-  const unsigned kvs4 = (unsigned)(KD / 4);
-  const float4 q4 = *(const float4 *)(a.q + h * DH + 4 * c);
-  const float4 *__restrict__ kp = (const float4 *)(a.kc + hk * DH) + c;
-  const float4 *__restrict__ vp = (const float4 *)(a.vc + hk * DH) + c;
-  const float scale = 1.0f / sqrtf((float)DH);
   {  // the MLP launch's accumulators: read last by this layer's qkv launch
     uint4 *z = (uint4 *)a.zero;
     const uint4 zz = make_uint4(0u, 0u, 0u, 0u);
     const int64_t nthr = (int64_t)H * gridDim.y * 1024;
     for (int64_t k = ((int64_t)blockIdx.y * H + h) * 1024 + tid; k < a.zero_n16; k += nthr) z[k] = zz;
   }
-  float m = -INFINITY, lsum = 0.0f;
-  float acc[4] = {0.f, 0.f, 0.f, 0.f};
-  // one tile = NP key passes per wavefront, all requested together (see k_dec_attn_proj): KPT passes up to
-  // 16*KPW*KPT keys, twice as many beyond, so that twice the context still costs one memory round trip
-  auto tile = [&](auto np_tag, int t0) {
-    constexpr int NP = decltype(np_tag)::value;
-    float4 kr[NP], vr[NP];
-#pragma unroll
-    for (int u = 0; u < NP; u++) {
-      const int j = t0 + (wv * NP + u) * KPW + g;
-      const unsigned jj = (unsigned)min(j, T - 1);  // clamped: masked below, never outside the cache
-      kr[u] = kp[jj * kvs4];
-      vr[u] = vp[jj * kvs4];
-    }
-    float sc[NP];
-    float tmax = -INFINITY;
-#pragma unroll
-    for (int u = 0; u < NP; u++) {
-      float d = q4.x * kr[u].x;
-      d = fmaf(q4.y, kr[u].y, d);
-      d = fmaf(q4.z, kr[u].z, d);
-      d = fmaf(q4.w, kr[u].w, d);
-      d = row16_sum(d);
-      const bool ok = (t0 + (wv * NP + u) * KPW + g) < T;
-      sc[u] = ok ? d * scale : -INFINITY;
-      tmax = fmaxf(tmax, sc[u]);
-    }
-    tmax = groups16_max(tmax);  // LPK == 16: one value per group of 16 lanes
-    const float m_new = fmaxf(m, tmax);
-    const float corr = ct_exp(m - m_new);
-    float psum = 0.0f;
-#pragma unroll
-    for (int k2 = 0; k2 < 4; k2++) acc[k2] *= corr;
-#pragma unroll
-    for (int u = 0; u < NP; u++) {
-      const float p = ct_exp(sc[u] - m_new);
-      psum += p;
-      acc[0] = fmaf(p, vr[u].x, acc[0]);
-      acc[1] = fmaf(p, vr[u].y, acc[1]);
-      acc[2] = fmaf(p, vr[u].z, acc[2]);
-      acc[3] = fmaf(p, vr[u].w, acc[3]);
-    }
-    psum = groups16_sum(psum);
-    lsum = lsum * corr + psum;
-    m = m_new;
-  };
-  if (T <= TILE) {
-    if (wv * KPT * KPW < T) tile(std::integral_constant<int, KPT>(), 0);  // (uniform per wavefront)
+  if constexpr (ATT_IN) {
+    // the head's attention was computed by a launch of its own (long contexts: its keys shared by several workgroups)
+    if (tid < DH) oh[tid] = a.att_in[h * DH + tid];
+    __syncthreads();
   } else {
-    for (int t0 = 0; t0 < T; t0 += 2 * TILE) {
-      if (t0 + wv * 2 * KPT * KPW >= T) break;  // nothing left for this wavefront (uniform)
-      tile(std::integral_constant<int, 2 * KPT>(), t0);
+    const int T = a.pos[0] + 1;
+    const unsigned kvs4 = (unsigned)(KD / 4);
+    const float4 q4 = *(const float4 *)(a.q + h * DH + 4 * c);
+    const float4 *__restrict__ kp = (const float4 *)(a.kc + hk * DH) + c;
+    const float4 *__restrict__ vp = (const float4 *)(a.vc + hk * DH) + c;
+    const float scale = 1.0f / sqrtf((float)DH);
+    float m = -INFINITY, lsum = 0.0f;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    // one tile = NP key passes per wavefront, all requested together (see k_dec_attn_proj): KPT passes up to
+    // 16*KPW*KPT keys, twice as many beyond, so that twice the context still costs one memory round trip
+    auto tile = [&](auto np_tag, int t0) {
+      constexpr int NP = decltype(np_tag)::value;
+      float4 kr[NP], vr[NP];
+  #pragma unroll
+      for (int u = 0; u < NP; u++) {
+        const int j = t0 + (wv * NP + u) * KPW + g;
+        const unsigned jj = (unsigned)min(j, T - 1);  // clamped: masked below, never outside the cache
+        kr[u] = kp[jj * kvs4];
+        vr[u] = vp[jj * kvs4];
+      }
+      float sc[NP];
+      float tmax = -INFINITY;
+  #pragma unroll
+      for (int u = 0; u < NP; u++) {
+        float d = q4.x * kr[u].x;
+        d = fmaf(q4.y, kr[u].y, d);
+        d = fmaf(q4.z, kr[u].z, d);
+        d = fmaf(q4.w, kr[u].w, d);
+        d = row16_sum(d);
+        const bool ok = (t0 + (wv * NP + u) * KPW + g) < T;
+        sc[u] = ok ? d * scale : -INFINITY;
+        tmax = fmaxf(tmax, sc[u]);
+      }
+      tmax = groups16_max(tmax);  // LPK == 16: one value per group of 16 lanes
+      const float m_new = fmaxf(m, tmax);
+      const float corr = ct_exp(m - m_new);
+      float psum = 0.0f;
+  #pragma unroll
+      for (int k2 = 0; k2 < 4; k2++) acc[k2] *= corr;
+  #pragma unroll
+      for (int u = 0; u < NP; u++) {
+        const float p = ct_exp(sc[u] - m_new);
+        psum += p;
+        acc[0] = fmaf(p, vr[u].x, acc[0]);
+        acc[1] = fmaf(p, vr[u].y, acc[1]);
+        acc[2] = fmaf(p, vr[u].z, acc[2]);
+        acc[3] = fmaf(p, vr[u].w, acc[3]);
+      }
+      psum = groups16_sum(psum);
+      lsum = lsum * corr + psum;
+      m = m_new;
+    };
+    if (T <= TILE) {
+      if (wv * KPT * KPW < T) tile(std::integral_constant<int, KPT>(), 0);  // (uniform per wavefront)
+    } else {
+      for (int t0 = 0; t0 < T; t0 += 2 * TILE) {
+        if (t0 + wv * 2 * KPT * KPW >= T) break;  // nothing left for this wavefront (uniform)
+        tile(std::integral_constant<int, 2 * KPT>(), t0);
+      }
     }
-  }
-#pragma unroll
-  for (int o = LPK; o < 64; o <<= 1) {
-#pragma unroll
-    for (int k2 = 0; k2 < 4; k2++) acc[k2] += __shfl_xor(acc[k2], o, 64);
-  }
-  if (lane < LPK) {
-#pragma unroll
-    for (int k2 = 0; k2 < 4; k2++) part[wv][4 * lane + k2] = acc[k2];
-  }
-  if (lane == 0) {
-    pm[wv] = m;
-    pl[wv] = lsum;
-  }
-  __syncthreads();
-  if (tid < DH) {
-    float M = pm[0];
-#pragma unroll
-    for (int w = 1; w < NW; w++) M = fmaxf(M, pm[w]);
-    float o = 0.0f, L = 0.0f;
-#pragma unroll
-    for (int w = 0; w < NW; w++) {
-      const float e = ct_exp(pm[w] - M);
-      o = fmaf(e, part[w][tid], o);
-      L = fmaf(e, pl[w], L);
+  #pragma unroll
+    for (int o = LPK; o < 64; o <<= 1) {
+  #pragma unroll
+      for (int k2 = 0; k2 < 4; k2++) acc[k2] += __shfl_xor(acc[k2], o, 64);
     }
-    oh[tid] = o / L;
+    if (lane < LPK) {
+  #pragma unroll
+      for (int k2 = 0; k2 < 4; k2++) part[wv][4 * lane + k2] = acc[k2];
+    }
+    if (lane == 0) {
+      pm[wv] = m;
+      pl[wv] = lsum;
+    }
+    __syncthreads();
+    if (tid < DH) {
+      float M = pm[0];
+  #pragma unroll
+      for (int w = 1; w < NW; w++) M = fmaxf(M, pm[w]);
+      float o = 0.0f, L = 0.0f;
+  #pragma unroll
+      for (int w = 0; w < NW; w++) {
+        const float e = ct_exp(pm[w] - M);
+        o = fmaf(e, part[w][tid], o);
+        L = fmaf(e, pl[w], L);
+      }
+      oh[tid] = o / L;
+    }
+    __syncthreads();
   }
-  __syncthreads();
   float xr[32], xsum = 0.0f;
   {
     float p8[8];
@@ -475,10 +481,19 @@ int launch_gqa_attn_proj(const GqaAttnArgs &a, int H, int HKV, int replicas) {
                 D, H, HKV, replicas);
   dim3 grid(H, replicas), block(1024);
   hipStream_t st = state().stream;
-  switch ((D / replicas + 511) / 512) {
-    case 1: hipLaunchKernelGGL((k_gqa_attn_proj<1>), grid, block, 0, st, a); break;
-    case 2: hipLaunchKernelGGL((k_gqa_attn_proj<2>), grid, block, 0, st, a); break;
-    default: hipLaunchKernelGGL((k_gqa_attn_proj<4>), grid, block, 0, st, a); break;
+  const int jr = (D / replicas + 511) / 512;
+  if (a.att_in) {
+    switch (jr) {
+      case 1: hipLaunchKernelGGL((k_gqa_attn_proj<1, true>), grid, block, 0, st, a); break;
+      case 2: hipLaunchKernelGGL((k_gqa_attn_proj<2, true>), grid, block, 0, st, a); break;
+      default: hipLaunchKernelGGL((k_gqa_attn_proj<4, true>), grid, block, 0, st, a); break;
+    }
+  } else {
+    switch (jr) {
+      case 1: hipLaunchKernelGGL((k_gqa_attn_proj<1, false>), grid, block, 0, st, a); break;
+      case 2: hipLaunchKernelGGL((k_gqa_attn_proj<2, false>), grid, block, 0, st, a); break;
+      default: hipLaunchKernelGGL((k_gqa_attn_proj<4, false>), grid, block, 0, st, a); break;
+    }
   }
   CTHIP_LAUNCH_CHECK();
   return 0;

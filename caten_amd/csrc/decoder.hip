@@ -113,7 +113,11 @@ struct Decoder {
   float *peek_f32 = nullptr;
   // KV cache in pages (kvp.hip)
   bool kvp = false;
-  hipGraphExec_t g_step = nullptr, g_body = nullptr, g_multi = nullptr;
+  // [0]: the step as the session runs it at short contexts; [1]: three-launch layers at long contexts (long_from > 0):
+  // the attention as a launch of its own with a head's keys shared by several workgroups, then the projection
+  hipGraphExec_t g_step[2] = {nullptr, nullptr}, g_body[2] = {nullptr, nullptr}, g_multi[2] = {nullptr, nullptr};
+  int long_from = 0;       // position from which [1] runs; 0 = never
+  bool long_mode = false;  // which of the two queue_step queues
   int64_t weight_bytes = 0, vector_bytes = 0;
   std::vector<void *> owned;  // device blocks to free
 };
@@ -519,20 +523,27 @@ static int finalize(Decoder *d) {
       TRY(cthip_memset(d->pattn, 0, sizeof(long long) * (size_t)kDecXcds * D));
     }
   }
+  // three-launch layers over fp32 cache rows: from this position on the attention is a launch of its own
+  if (!d->flow && ((d->fused && !d->kvq) || d->fused_gqa) && d->att_split.ranges > 1 && state().attn_long_from > 0 &&
+      state().attn_long_from < c.max_seq)
+    d->long_from = state().attn_long_from;
   if (!state().decoder_graph) d->use_graph = false;
   if (d->use_graph) {
     hipStream_t st = state().stream;
     // 0: one step with the head; 1: one step without (prompt rows fed one by one); 2: kStepsPerGraph steps
     // with their heads back to back (the device-resident loop: fewer graph launches per token)
-    for (int pass = 0; pass < 3; pass++) {
+    for (int pass = 0; pass < (d->long_from > 0 ? 6 : 3); pass++) {
+      const int mode = pass / 3;
+      d->long_mode = mode == 1;
       hipGraph_t g = nullptr;
       CTHIP_CHECK(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
       // the device-resident loop (pass 2) only ever follows a head, which leaves the next input in place
-      rc = queue_step(d, pass != 1, pass != 2);
-      for (int k = 1; pass == 2 && k < kStepsPerGraph && !rc; k++) rc = queue_step(d, true, false);
+      rc = queue_step(d, pass % 3 != 1, pass % 3 != 2);
+      for (int k = 1; pass % 3 == 2 && k < kStepsPerGraph && !rc; k++) rc = queue_step(d, true, false);
       hipError_t e = hipStreamEndCapture(st, &g);
       if (rc) {
         if (g) (void)hipGraphDestroy(g);
+        d->long_mode = false;
         return rc;
       }
       if (e != hipSuccess) return fail((int)e, "decoder: hipStreamEndCapture -> %s", hipGetErrorString(e));
@@ -540,8 +551,9 @@ static int finalize(Decoder *d) {
       e = hipGraphInstantiate(&ex, g, nullptr, nullptr, 0);
       (void)hipGraphDestroy(g);
       if (e != hipSuccess) return fail((int)e, "decoder: hipGraphInstantiate -> %s", hipGetErrorString(e));
-      (pass == 0 ? d->g_step : pass == 1 ? d->g_body : d->g_multi) = ex;
+      (pass % 3 == 0 ? d->g_step : pass % 3 == 1 ? d->g_body : d->g_multi)[mode] = ex;
     }
+    d->long_mode = false;
   }
 #undef TRY
   d->finalized = true;
@@ -619,7 +631,13 @@ static int queue_step(Decoder *d, bool with_head, bool embed) {
         a8.zero = aa.zero;
         a8.zero_n16 = aa.zero_n16;
         if (!(skip & 2)) TRY(launch_dec_attn_proj_q8(a8, L.attn->type, c.n_heads, D, replicas));
-      } else if (!(skip & 2)) TRY(launch_dec_attn_proj(aa, L.attn->type, c.n_heads, D, replicas));
+      } else if (!(skip & 2)) {
+        if (d->long_mode) {
+          TRY(launch_attn(d->att, d->q, L.k_cache, L.v_cache, 1, 0, pos, c.max_seq, c.n_heads, c.n_kv_heads, Dh, &d->att_split));
+          aa.att_in = d->att;
+        }
+        TRY(launch_dec_attn_proj(aa, L.attn->type, c.n_heads, D, replicas));
+      }
       DecMlpArgs ma = {};
       ma.st.base = d->x2;
       ma.st.bias = L.proj_b;
@@ -689,6 +707,10 @@ static int queue_step(Decoder *d, bool with_head, bool embed) {
       aa.zero_n16 = acc16;
       aa.D = D;
       aa.KD = KD;
+      if (d->long_mode) {
+        TRY(launch_attn(d->att, d->q, L.k_cache, L.v_cache, 1, 0, pos, c.max_seq, c.n_heads, c.n_kv_heads, Dh, &d->att_split));
+        aa.att_in = d->att;
+      }
       TRY(launch_gqa_attn_proj(aa, c.n_heads, c.n_kv_heads, replicas));
       GqaMlpArgs ma = {};
       ma.st.base = d->x2;
@@ -976,12 +998,17 @@ static int flow_check(Decoder *d) {
               dec_flow_grid(d->cfg.dim, d->cfg.n_heads, d->cfg.ffn));
 }
 
-static int run_step(Decoder *d, bool with_head) {
+// `position`: where the step's row goes (what the host knows of it: never below the device's)
+static int run_step(Decoder *d, bool with_head, int position) {
+  const int mode = d->long_from > 0 && position >= d->long_from ? 1 : 0;
   if (d->use_graph) {
-    CTHIP_CHECK(hipGraphLaunch(with_head ? d->g_step : d->g_body, state().stream));
+    CTHIP_CHECK(hipGraphLaunch((with_head ? d->g_step : d->g_body)[mode], state().stream));
     return 0;
   }
-  return queue_step(d, with_head);
+  d->long_mode = mode == 1;
+  const int rc = queue_step(d, with_head);
+  d->long_mode = false;
+  return rc;
 }
 
 }  // namespace cthip
@@ -1015,9 +1042,11 @@ int cthip_decoder_destroy(void *dec) {
   if (!dec) return 0;
   Decoder *d = (Decoder *)dec;
   if (state().inited) (void)hipStreamSynchronize(state().stream);
-  if (d->g_step) (void)hipGraphExecDestroy(d->g_step);
-  if (d->g_body) (void)hipGraphExecDestroy(d->g_body);
-  if (d->g_multi) (void)hipGraphExecDestroy(d->g_multi);
+  for (int mode = 0; mode < 2; mode++) {
+    if (d->g_step[mode]) (void)hipGraphExecDestroy(d->g_step[mode]);
+    if (d->g_body[mode]) (void)hipGraphExecDestroy(d->g_body[mode]);
+    if (d->g_multi[mode]) (void)hipGraphExecDestroy(d->g_multi[mode]);
+  }
   if (d->ctrl_host) (void)hipHostFree(d->ctrl_host);
   if (d->ctrl_ev) (void)hipEventDestroy(d->ctrl_ev);
   for (auto &kv : d->raw) cthip_free(kv.second.dev);
@@ -1104,7 +1133,7 @@ int cthip_decoder_forward(void *dec, const float *tokens, int s, int n, int64_t 
     for (int i = 0; i < s; i++) {
       int tp[2] = {ids[i], n + i};
       if ((rc = cthip_h2d(d->tokpos, tp, sizeof(tp)))) return rc;
-      if ((rc = run_step(d, i == s - 1))) return rc;
+      if ((rc = run_step(d, i == s - 1, n + i))) return rc;
     }
   }
   if (logits_out && (rc = cthip_d2h(logits_out, d->logits, sizeof(float) * (size_t)c.vocab))) return rc;
@@ -1147,9 +1176,10 @@ static int generate_impl(Decoder *d, int steps, int eos, int64_t *tokens_out, in
     return false;
   };
   if (d->use_graph)
-    for (; i + kStepsPerGraph <= steps && !ended(); i += kStepsPerGraph) CTHIP_CHECK(hipGraphLaunch(d->g_multi, st));
+    for (; i + kStepsPerGraph <= steps && !ended(); i += kStepsPerGraph)
+      CTHIP_CHECK(hipGraphLaunch(d->g_multi[d->long_from > 0 && d->position + i >= d->long_from ? 1 : 0], st));
   for (; i < steps && !ended(); i++)
-    if ((rc = run_step(d, true))) return rc;
+    if ((rc = run_step(d, true, d->position + i))) return rc;
   int n = 0;
   if ((rc = cthip_d2h(&n, d->hist_n, sizeof(int)))) return rc;  // synchronises
   if ((rc = flow_check(d))) return rc;

@@ -741,6 +741,11 @@ int cthip_set_option(const char *name, int value) {
     state().attn_split = value;
     return 0;
   }
+  if (!strcmp(name, "attn_long_from")) {
+    if (value < 0) return fail(CTHIP_E_BAD_ARG, "cthip_set_option: attn_long_from is a position (0 = never)");
+    state().attn_long_from = value;
+    return 0;
+  }
   if (!strcmp(name, "gemv_wide")) {
     if (value < 0 || value > 2) return fail(CTHIP_E_BAD_ARG, "cthip_set_option: gemv_wide is 0, 1 or 2");
     state().gemv_wide = value;

@@ -260,6 +260,10 @@ int cthip_linear(float *y, const void *wmat, const float *x, int m, const float 
  *   max_seq >= 512 share the keys of a head among (compute units / heads) workgroups, at most 16, in their decode
  *   attention (long contexts); 2 .. 16 = that many workgroups per head; 0 = one workgroup per head.  Same tokens;
  *   logits differ in summation order only.
+ * "attn_long_from": a position (default 896; 0 = never).  Decoder sessions created afterwards whose layers run as
+ *   three launches (fp32 cache rows) switch, from this position on, to four launches per layer: the attention as a
+ *   launch of its own with a head's keys shared by several workgroups ("attn_split"), then the projection.  Same
+ *   tokens; logits differ in summation order only.
  * "kv_cache": how decoder sessions created afterwards keep their KV cache: 0 (default) = fp32 rows, the
  *   reference's dense cache (external/llm/layers.lisp:19-33); 1 = GGUF-Q8_0 rows (blocks of 32 int8 and one fp16
  *   scale per cache row, quantised once when the row is appended): 3.76x fewer cache bytes held and read per
@@ -392,11 +396,11 @@ int cthip_decoder_position(const void *dec);
 /* Bytes of HBM one decode step must read at position t (weights + norms/biases + KV rows at their stored
  * size: 4 bytes per element, 1.0625 with option "kv_cache" 1). */
 int64_t cthip_decoder_step_bytes(const void *dec, int t);
-/* Launches per layer of one decode step of this session: 3 (attention + projection and the whole MLP merged,
+/* Launches per layer of one decode step of this session at short contexts: 3 (attention + projection and the whole MLP merged,
  * per-XCD accumulators -- taken only when the device passed the load-time checks that XCD ids are 0..7 and that
  * atomics of different workgroups of an XCD meet in its L2), 5 (one launch per Linear + attention; over Q8_0 cache
  * rows and over a paged cache the attention launch also rotates, quantises / copies and appends the new row).
- * -1 on error. */
+ * A session of 3 runs 4 from position "attn_long_from" on.  -1 on error. */
 int cthip_decoder_layer_launches(void *dec);
 /* Device pointers into the session, for parity tests: "k_cache.<l>", "v_cache.<l>" (fp32 rows; with a Q8_0
  * cache their dequantised values, in a buffer the next peek overwrites), "logits", "x"; with a Q8_0 cache also

@@ -164,6 +164,52 @@ def test_three_launch_layer_equals_five_launch_layer(name, plen, kind):
         assert np.array_equal(a, c)
 
 
+@pytest.mark.parametrize("arch,plen", [("gpt2", 40), ("gpt2", 700), ("llama", 40), ("llama", 600)])
+def test_three_launch_layer_with_the_attention_as_a_launch_of_its_own(arch, plen):
+    """Long contexts of the three-launch layers (option attn_long_from, a position): from there on the attention is a
+    launch of its own in which several workgroups share a head's keys, and the projection launch takes its outputs
+    instead of repeating the attention in every workgroup of the head -- four launches per layer.  Same greedy tokens
+    as three launches throughout (attn_long_from 0) and logits inside the fp32 band (the keys are added in another
+    order); two runs bit-identical; the threshold crossed in the middle of a generation (prompt 40, from position 64)
+    and far behind it (prompts of 600 / 700); the host-driven loop and the device-resident loop (graphs of one and of
+    eight steps, picked per launch by the position the host knows)."""
+    print(f"case: three-launch layer, attention as its own launch from position 64, {arch} prompt {plen}", flush=True)
+    from caten_amd import _lib, synth, llm
+    lib = _lib.load()
+    if arch == "gpt2":
+        cfg = dict(synth.GPT2_CONFIGS["gpt2-mini"], max_seq=1024)
+        sd = llm.gpt2_state_dict(synth.gpt2_weights(cfg, seed=29), "q8_0")
+        make = llm.make_gpt2
+    else:
+        cfg = dict(synth.LLAMA_CONFIGS["llama-1.1b"], n_layers=2, max_seq=1024, vocab=2000)
+        sd = llm.llama_state_dict(synth.llama_weights(cfg, seed=29), "q4_0")
+        make = llm.make_llama
+    prompt = synth.prompt(cfg["vocab"], plen, seed=29)
+    steps = 40
+    runs = []
+    try:
+        for long_from in (64, 0, 64):
+            _lib.check(lib.cthip_set_option(b"attn_long_from", long_from))
+            model = make(cfg, sd)
+            assert lib.cthip_decoder_layer_launches(model.handle) == 3  # (what the session runs at short contexts)
+            runs.append(llm.gpt2_generate(model, prompt, steps, on_device=False, keep_logits=True))
+            model.close()
+            if long_from:
+                model = make(cfg, sd)
+                assert llm.gpt2_generate(model, prompt, steps, on_device=True) == runs[-1][0]
+                model.close()
+    finally:
+        _lib.check(lib.cthip_set_option(b"attn_long_from", 896))
+    assert runs[0][0] == runs[1][0] == runs[2][0]
+    for a, b, c in zip(*[r[1] for r in runs]):
+        close(a, b)
+        assert np.array_equal(a, c)
+    # (the other launch sequence did run: where a head's keys are cut into several ranges the low bits differ; a
+    # context of one tile is one range, added up in the order of the three-launch layer)
+    if plen >= 600:
+        assert any(not np.array_equal(a, b) for a, b in zip(runs[0][1][-8:], runs[1][1][-8:]))
+
+
 @pytest.mark.parametrize("plen", [3, 40])
 def test_three_launch_grouped_query_layer_equals_five_launch_layer(plen):
     """The same for RMSNorm / RoPE / grouped-query / SwiGLU layers with Q4_0 weights at the width the three-launch

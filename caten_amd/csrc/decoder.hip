@@ -523,10 +523,12 @@ static int finalize(Decoder *d) {
       TRY(cthip_memset(d->pattn, 0, sizeof(long long) * (size_t)kDecXcds * D));
     }
   }
-  // three-launch layers over fp32 cache rows: from this position on the attention is a launch of its own
-  if (!d->flow && ((d->fused && !d->kvq) || d->fused_gqa) && d->att_split.ranges > 1 && state().attn_long_from > 0 &&
-      state().attn_long_from < c.max_seq)
-    d->long_from = state().attn_long_from;
+  // three-launch layers: from this position on the attention is a launch of its own (Q8_0 cache rows are a quarter of
+  // the bytes, the repeated attention stays the cheaper one half as far again)
+  if (!d->flow && (d->fused || d->fused_gqa) && d->att_split.ranges > 1 && state().attn_long_from > 0) {
+    const int64_t from = d->kvq ? (int64_t)state().attn_long_from * 3 / 2 : state().attn_long_from;
+    if (from < c.max_seq) d->long_from = (int)from;
+  }
   if (!state().decoder_graph) d->use_graph = false;
   if (d->use_graph) {
     hipStream_t st = state().stream;
@@ -630,7 +632,14 @@ static int queue_step(Decoder *d, bool with_head, bool embed) {
         a8.part = aa.part;
         a8.zero = aa.zero;
         a8.zero_n16 = aa.zero_n16;
-        if (!(skip & 2)) TRY(launch_dec_attn_proj_q8(a8, L.attn->type, c.n_heads, D, replicas));
+        if (skip & 2) {
+        } else if (d->long_mode) {  // rotation (none here), quantisation, append and attention, then the projection
+          TRY(launch_attn_q8_step(d->att, d->q, d->kv_tmp, L.kq, L.kdq, L.vq, L.vdq, pos, c.n_heads, c.n_kv_heads, Dh, 0.0f, &d->att_split));
+          aa.att_in = d->att;
+          TRY(launch_dec_attn_proj(aa, L.attn->type, c.n_heads, D, replicas));
+        } else {
+          TRY(launch_dec_attn_proj_q8(a8, L.attn->type, c.n_heads, D, replicas));
+        }
       } else if (!(skip & 2)) {
         if (d->long_mode) {
           TRY(launch_attn(d->att, d->q, L.k_cache, L.v_cache, 1, 0, pos, c.max_seq, c.n_heads, c.n_kv_heads, Dh, &d->att_split));

@@ -261,7 +261,7 @@ int cthip_linear(float *y, const void *wmat, const float *x, int m, const float 
  *   attention (long contexts); 2 .. 16 = that many workgroups per head; 0 = one workgroup per head.  Same tokens;
  *   logits differ in summation order only.
  * "attn_long_from": a position (default 896; 0 = never).  Decoder sessions created afterwards whose layers run as
- *   three launches (fp32 cache rows) switch, from this position on, to four launches per layer: the attention as a
+ *   three launches switch, from this position on (half as far again over Q8_0 cache rows), to four launches per layer: the attention as a
  *   launch of its own with a head's keys shared by several workgroups ("attn_split"), then the projection.  Same
  *   tokens; logits differ in summation order only.
  * "kv_cache": how decoder sessions created afterwards keep their KV cache: 0 (default) = fp32 rows, the

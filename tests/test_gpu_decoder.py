@@ -164,16 +164,18 @@ def test_three_launch_layer_equals_five_launch_layer(name, plen, kind):
         assert np.array_equal(a, c)
 
 
-@pytest.mark.parametrize("arch,plen", [("gpt2", 40), ("gpt2", 700), ("llama", 40), ("llama", 600)])
-def test_three_launch_layer_with_the_attention_as_a_launch_of_its_own(arch, plen):
+@pytest.mark.parametrize("arch,plen,kv", [("gpt2", 40, 0), ("gpt2", 700, 0), ("llama", 40, 0), ("llama", 600, 0), ("gpt2", 40, 1),
+                                          ("gpt2", 700, 1)])
+def test_three_launch_layer_with_the_attention_as_a_launch_of_its_own(arch, plen, kv):
     """Long contexts of the three-launch layers (option attn_long_from, a position): from there on the attention is a
     launch of its own in which several workgroups share a head's keys, and the projection launch takes its outputs
     instead of repeating the attention in every workgroup of the head -- four launches per layer.  Same greedy tokens
     as three launches throughout (attn_long_from 0) and logits inside the fp32 band (the keys are added in another
     order); two runs bit-identical; the threshold crossed in the middle of a generation (prompt 40, from position 64)
     and far behind it (prompts of 600 / 700); the host-driven loop and the device-resident loop (graphs of one and of
-    eight steps, picked per launch by the position the host knows)."""
-    print(f"case: three-launch layer, attention as its own launch from position 64, {arch} prompt {plen}", flush=True)
+    eight steps, picked per launch by the position the host knows); over fp32 cache rows and, for the GPT-2 shape, over
+    Q8_0 rows (kv 1: the attention launch also quantises and appends the step's row)."""
+    print(f"case: three-launch layer, attention as its own launch from position 64, {arch} prompt {plen} kv_cache {kv}", flush=True)
     from caten_amd import _lib, synth, llm
     lib = _lib.load()
     if arch == "gpt2":
@@ -185,9 +187,10 @@ def test_three_launch_layer_with_the_attention_as_a_launch_of_its_own(arch, plen
         sd = llm.llama_state_dict(synth.llama_weights(cfg, seed=29), "q4_0")
         make = llm.make_llama
     prompt = synth.prompt(cfg["vocab"], plen, seed=29)
-    steps = 40
+    steps = 72  # (over Q8_0 rows the threshold is half as far again: position 96)
     runs = []
     try:
+        _lib.check(lib.cthip_set_option(b"kv_cache", kv))
         for long_from in (64, 0, 64):
             _lib.check(lib.cthip_set_option(b"attn_long_from", long_from))
             model = make(cfg, sd)
@@ -200,6 +203,7 @@ def test_three_launch_layer_with_the_attention_as_a_launch_of_its_own(arch, plen
                 model.close()
     finally:
         _lib.check(lib.cthip_set_option(b"attn_long_from", 896))
+        _lib.check(lib.cthip_set_option(b"kv_cache", 0))
     assert runs[0][0] == runs[1][0] == runs[2][0]
     for a, b, c in zip(*[r[1] for r in runs]):
         close(a, b)

@@ -207,6 +207,16 @@ struct AttnSplit {
   int *count;
 };
 constexpr int kAttnSplitMaxRanges = 16;
+#ifdef __HIPCC__
+// Which head a workgroup of a decode attention launch takes.  Workgroups are dealt to the eight XCDs in turn (XCD =
+// linear workgroup id mod 8, blockIdx.x running fastest).  With H a multiple of 8, head (b mod 8) * (H / 8) + b / 8
+// puts consecutive heads -- the query heads that share a key / value head -- on ONE XCD: the group's cache rows enter
+// one L2 instead of eight (70B shape at position 1940: 11.60 -> 10.96 ms per step).  Heads that share nothing keep
+// the plain order, which spreads an XCD's reads over a cache row (7B shape: 3 % faster than the grouped order).
+__device__ __forceinline__ int attn_head_of_block(int b, int H, int Hkv) {
+  return ((H & 7) || H == Hkv) ? b : (b & 7) * (H >> 3) + (b >> 3);
+}
+#endif
 int launch_attn(float *out, const float *q, const float *kc, const float *vc, int S, int start_pos, const int *pos,
                 int max_T, int H, int Hkv, int Dh, const AttnSplit *split = nullptr);
 int launch_embedding(float *out, const float *W, const float *idx_f, const int *idx_i, int ntok, int vocab, int dim,

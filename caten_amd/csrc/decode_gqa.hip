@@ -195,7 +195,8 @@ void k_gqa_attn_proj(GqaAttnArgs a) {
   __shared__ float part[NW][DH];
   __shared__ float pm[NW], pl[NW];
   __shared__ __align__(16) float oh[DH];
-  const int h = blockIdx.x, H = gridDim.x, D = a.D, KD = a.KD;
+  const int H = gridDim.x, D = a.D, KD = a.KD;
+  const int h = attn_head_of_block(blockIdx.x, H, KD / DH);  // the query heads of a key / value head on one XCD
   const int hk = h / (H / (KD / DH));
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int g = lane / LPK, c = lane % LPK;

@@ -61,7 +61,7 @@ void k_attn_cached_paged(float *__restrict__ out, const float *__restrict__ q, c
   __shared__ float part[NW][DH];
   __shared__ float pm[NW], pl[NW];
   __shared__ int ticket;
-  const int h = blockIdx.x;
+  const int h = attn_head_of_block(blockIdx.x, H, Hkv);
   const int T = start_pos + (pos ? pos[0] : 0) + 1;
   int k0 = 0, k1 = T, nranges = 1;
   if (STEP) {

@@ -183,7 +183,7 @@ __global__ __launch_bounds__(256) void k_attn_q8_step(float *__restrict__ out, c
   __shared__ float pm[NW], pl[NW];
   __shared__ float ang_s[DH / 2], ang_c[DH / 2];
   __shared__ int ticket;
-  const int h = blockIdx.x;
+  const int h = attn_head_of_block(blockIdx.x, H, Hkv);
   const int T = pos[0] + 1;
   int k0 = 0, k1 = T, nranges = 1;
   {

@@ -724,7 +724,7 @@ void k_attn_cached(float *__restrict__ out, const float *__restrict__ q,
   __shared__ float part[NW][DH];
   __shared__ float pm[NW], pl[NW];
   __shared__ int ticket;
-  const int h = blockIdx.x, i = blockIdx.y;
+  const int h = attn_head_of_block(blockIdx.x, H, Hkv), i = blockIdx.y;
   const int T = start_pos + (pos ? pos[0] : 0) + i + 1;
   // this workgroup's keys [k0, k1): everything, or one of `nranges` ranges of whole tiles
   int k0 = 0, k1 = T, nranges = 1;

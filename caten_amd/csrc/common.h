@@ -197,6 +197,9 @@ int wmat_create_impl(WMat **out, int type, const void *raw, int64_t rows, int64_
 bool gemv_is_direct(const WMat *w);
 // rows a wavefront of the register-resident variant for (type, cols) produces per pass; 0 = no such variant
 int gemv_rows_per_wave(int type, int64_t cols);
+// true when the single-row launch over a (rows, cols) matrix whose rows are gate / up rows in turn holds a row pair
+// per wavefront, so that SwiGLU can be its epilogue
+bool gemv_pair_swiglu_ok(int type, int64_t rows, int64_t cols);
 // out[i] = silu(in[2i]) * in[2i+1], i < n (gate / up columns interleaved)
 int launch_swiglu_pairs(float *out, const float *in, int64_t n);
 // One query row over a long context: `ranges` workgroups per head share the keys (k_attn_cached, SPLIT).  part holds

@@ -327,7 +327,7 @@ static int finalize(Decoder *d) {
       TRY(to_f32(d, key(l, "ffn_norm.weight"), D, &L.ln2_g));
       // gate and up rows interleaved when the GEMV variant keeps a row pair in one wavefront: SwiGLU then
       // happens in that launch's epilogue and the down projection reads ffn floats instead of 2 * ffn
-      L.fc_pairs = gemv_rows_per_wave(d->raw.at(key(l, "feed_forward.w1.weight")).type, D) >= 2;
+      L.fc_pairs = gemv_pair_swiglu_ok(d->raw.at(key(l, "feed_forward.w1.weight")).type, 2 * (int64_t)F, D);
       TRY(to_wmat(d, {key(l, "feed_forward.w1.weight"), key(l, "feed_forward.w3.weight")}, 2 * F, D, &L.fc, L.fc_pairs));
       TRY(to_wmat(d, {key(l, "feed_forward.w2.weight")}, D, F, &L.fc2));
     }

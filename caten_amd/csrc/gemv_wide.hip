@@ -167,8 +167,12 @@ void k_gemv_wide(GemvArgs a, int tpr) {
       const int row0 = RW * cs_pair;
       const float b0 = a.bias ? __shfl(row_epi, 0, 64) : 0.0f, r0 = a.residual ? __shfl(row_epi, 1, 64) : 0.0f;
       const float b1 = a.bias ? __shfl(row_epi, 2, 64) : 0.0f, r1 = a.residual ? __shfl(row_epi, 3, 64) : 0.0f;
-      if (lane == 0) gemv_store(a, m, row0, s0, posv, b0, r0);
-      if (RW > 1 && lane == 1 && row0 + 1 < a.rows) gemv_store(a, m, row0 + 1, s1, posv, b1, r1);
+      if (RW > 1 && a.pair_swiglu) {  // the pair is a (gate, up) row pair: SwiGLU here, one output per pair
+        if (lane == 0) a.y[(int64_t)m * a.y_stride + (row0 >> 1)] = ct_silu(s0 + b0) * (s1 + b1);
+      } else {
+        if (lane == 0) gemv_store(a, m, row0, s0, posv, b0, r0);
+        if (RW > 1 && lane == 1 && row0 + 1 < a.rows) gemv_store(a, m, row0 + 1, s1, posv, b1, r1);
+      }
       acc0 = acc1 = 0.0f;
       cs_grp = 0;
       cs_pair += total_waves;
@@ -190,8 +194,11 @@ void k_gemv_wide(GemvArgs a, int tpr) {
 // true when the launch is one this kernel runs: quantised rows that LDS holds, no LayerNorm, no fused argmax, no
 // paired epilogue
 bool gemv_wide_supported(const WMat *w, const GemvArgs &a) {
-  if (a.pro == CTHIP_PRO_LAYERNORM || a.fold_s || a.am_val || a.pair_swiglu) return false;
-  return gemv_wide_plan(w->type, w->rows, w->cols, state().compute_units).ok;
+  if (a.pro == CTHIP_PRO_LAYERNORM || a.fold_s || a.am_val) return false;
+  const GemvWidePlan p = gemv_wide_plan(w->type, w->rows, w->cols, state().compute_units);
+  // the paired SwiGLU epilogue: a wavefront must hold a (gate, up) row pair, outputs plain
+  if (a.pair_swiglu && (p.rw != 2 || (w->rows & 1) || a.residual || a.act != CTHIP_ACT_NONE || (a.split1 > 0 && a.split1 != (int)w->rows))) return false;
+  return p.ok;
 }
 
 int launch_gemv_wide(const WMat *w, GemvArgs a, int m) {

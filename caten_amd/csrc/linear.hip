@@ -366,6 +366,30 @@ bool gemv_is_direct(const WMat *w) {
   return pick_variant(w->type, (int)w->cols) != nullptr || gemv_slices(w->type, (long long)w->cols, &width) > 0 ||
          gemv_wide_plan(w->type, w->rows, w->cols, state().compute_units).ok;
 }
+// true when a single-row launch over a (rows, cols) matrix of gate / up rows in turn can apply SwiGLU in its epilogue:
+// the launch it will be holds a row pair per wavefront (the routing of launch_gemv, repeated)
+// The wide-row kernel takes the rows no variant covers, and those whose variant holds so much of the input vector
+// per lane (128 floats: 4-bit rows past 6144 columns, 8-bit rows past 4096) that it needs more than 256 registers
+// and runs one wavefront per SIMD (Llama-70B shape, 8192-wide 4-bit rows: 12.3 -> 11.8 ms per step; narrower
+// rows are faster from registers: 7B / 13B shapes 1.83 / 2.96 ms against 2.02 / 3.29 with every launch here).
+// (a wavefront there takes whole rows: with few rows it leaves compute units idle -- GPT-2 large's 1280 x 5120
+// projection is slower there, GPT-2 XL's 1600 x 6400, whose variant needs 366 registers, faster)
+static bool gemv_prefers_wide(const GemvVariant *v, int type, int64_t rows) {
+  const bool heavy = v && ((type == CTHIP_Q4_0 && v->KC >= 4 && rows >= 1024) ||
+                           (type == CTHIP_Q8_0 && (v->KC >= 8 ? rows >= 1024 : v->KC >= 6 && rows >= 4096)));
+  const int opt = state().gemv_wide;
+  return opt && (!v || heavy || opt >= 2);
+}
+bool gemv_pair_swiglu_ok(int type, int64_t rows, int64_t cols) {
+  if (rows <= 0 || (rows & 1) || cols <= 0 || cols > 0x7fffffff) return false;
+  const GemvVariant *v = pick_variant(type, (int)cols);
+  const State &s = state();
+  if (gemv_prefers_wide(v, type, rows)) {
+    const GemvWidePlan p = gemv_wide_plan(type, rows, cols, s.compute_units);
+    if (p.ok) return p.rw == 2;
+  }
+  return v && v->G <= 32;
+}
 int gemv_rows_per_wave(int type, int64_t cols) {
   const GemvVariant *v = cols <= 0x7fffffff ? pick_variant(type, (int)cols) : nullptr;
   return v ? 64 / v->G : 0;
@@ -450,17 +474,9 @@ int launch_gemv(const WMat *w, GemvArgs a, int m) {
   if (a.split1 <= 0) a.split1 = a.split2 = a.rows;
   if (a.am_val && m != 1) return fail(CTHIP_E_BAD_ARG, "gemv: the fused argmax needs m == 1");
   const GemvVariant *v = pick_variant(w->type, a.cols);
+  if (gemv_prefers_wide(v, w->type, a.rows) && gemv_wide_supported(w, a)) return launch_gemv_wide(w, a, m);
   if (a.pair_swiglu && (!v || v->G > 32 || (a.rows & 1) || a.am_val || a.residual || a.split1 != a.rows))
     return fail(CTHIP_E_UNSUPPORTED, "gemv: the paired SwiGLU epilogue needs two rows per wavefront and plain outputs");
-  // The wide-row kernel takes the rows no variant covers, and those whose variant holds so much of the input vector
-  // per lane (128 floats: 4-bit rows past 6144 columns, 8-bit rows past 4096) that it needs more than 256 registers
-  // and runs one wavefront per SIMD (Llama-70B shape, 8192-wide 4-bit rows: 12.3 -> 11.8 ms per step; narrower
-  // rows are faster from registers: 7B / 13B shapes 1.83 / 2.96 ms against 2.02 / 3.29 with every launch here).
-  // (a wavefront here takes whole rows: with few rows it leaves compute units idle -- GPT-2 large's 1280 x 5120
-  // projection is slower here, GPT-2 XL's 1600 x 6400, whose variant needs 366 registers, faster)
-  const bool heavy = v && ((w->type == CTHIP_Q4_0 && v->KC >= 4 && a.rows >= 1024) ||
-                           (w->type == CTHIP_Q8_0 && (v->KC >= 8 ? a.rows >= 1024 : v->KC >= 6 && a.rows >= 4096)));
-  if (s.gemv_wide && (!v || heavy || s.gemv_wide >= 2) && gemv_wide_supported(w, a)) return launch_gemv_wide(w, a, m);
   if (v) return launch_variant(v, w, a, m);
   // wider than any variant: column slices, when nothing in the launch needs the whole row at once (a norm of the
   // input, an activation of the sum, an argmax) and the output is one plain vector per input row

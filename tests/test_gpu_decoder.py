@@ -164,6 +164,41 @@ def test_three_launch_layer_equals_five_launch_layer(name, plen, kind):
         assert np.array_equal(a, c)
 
 
+@pytest.mark.parametrize("kind", ["q4_0", "q8_0", "f16"])
+def test_llama_swiglu_in_the_epilogue_of_the_wide_row_gate_up_launch(oracle, kind):
+    """A model whose gate|up launch runs on the wide-row kernel with a (gate, up) row pair per wavefront (8192 rows
+    of gate and up in turn; option gemv_wide 2 sends every launch it supports there) applies SwiGLU in that launch's
+    epilogue, and the down projection stages one vector instead of two.  Same tokens as the CPU decoder and as the
+    session whose launches take the register-resident kernels; logits inside the fp32 band of both."""
+    print(f"case: SwiGLU in the epilogue of the wide-row gate|up launch, {kind}", flush=True)
+    from caten_amd import _lib, synth, llm
+    lib = _lib.load()
+    cfg = dict(synth.LLAMA_CONFIGS["llama-tiny"], ffn=4096, max_seq=64)
+    w = synth.llama_weights(cfg, seed=31)
+    sd = llm.llama_state_dict(w, kind)
+    prompt = synth.prompt(cfg["vocab"], 9, seed=31)
+    runs = []
+    try:
+        for wide in (2, 1):
+            _lib.check(lib.cthip_set_option(b"gemv_wide", wide))
+            model = llm.make_llama(cfg, sd)
+            runs.append(llm.gpt2_generate(model, prompt, 12, on_device=False, keep_logits=True))
+            model.close()
+            model = llm.make_llama(cfg, sd)
+            assert llm.gpt2_generate(model, prompt, 12, on_device=True) == runs[-1][0]
+            model.close()
+    finally:
+        _lib.check(lib.cthip_set_option(b"gemv_wide", 1))
+    assert runs[0][0] == runs[1][0]
+    for a, b in zip(runs[0][1], runs[1][1]):
+        close(a, b)
+    ref = oracle.Llama(cfg, _dequantised(oracle, w, synth.LLAMA_LINEAR_KEYS + ("lm_head",), kind))
+    want_tokens, want_logits = ref.generate(prompt, 12, keep_logits=True)
+    assert runs[0][0] == want_tokens
+    for g, r in zip(runs[0][1], want_logits):
+        close(g, r)
+
+
 @pytest.mark.parametrize("arch,plen,kv", [("gpt2", 40, 0), ("gpt2", 700, 0), ("llama", 40, 0), ("llama", 600, 0), ("gpt2", 40, 1),
                                           ("gpt2", 700, 1)])
 def test_three_launch_layer_with_the_attention_as_a_launch_of_its_own(arch, plen, kv):

@@ -380,14 +380,20 @@ __device__ __forceinline__ void gemv_ring(const GemvArgs &a, float *xs_lds, floa
   float epi_t[PD];
 #pragma unroll
   for (int p = 0; p < PD; p++) epi_t[p] = 0.0f;
-  const int own = wave < nrq ? wave : nrq - 1;  // what a slot without a tile requests: lines this wavefront fetches anyway
+  // Which tile ring slot p holds first.  Plain: wave + p * total_waves.  With one row per wavefront and the paired
+  // SwiGLU epilogue a wavefront takes (gate, up) row pairs: slots 2k and 2k + 1 hold rows 2 (wave + k * total_waves)
+  // and the one after it; a slot's next tile is PD * total_waves further on either way.
+  const bool pair1 = RPW == 1 && PD >= 2 && a.pair_swiglu;
+  const int first = pair1 ? 2 * wave : wave;
+  auto slot_off = [&](int p) { return pair1 ? (p >> 1) * 2 * total_waves + (p & 1) : p * total_waves; };
+  const int own = first < nrq ? first : nrq - 1;  // what a slot without a tile requests: lines this wavefront fetches anyway
   // Only the first tile goes out before the staged input is picked up: requests are issued in program order and
   // a compute unit accepts them no faster than earlier ones are answered, so the whole ring in front of the
   // staging code would hold that code back until most of the ring had arrived.
   constexpr int PRE = 1;
 #pragma unroll
   for (int p = 0; p < PRE; p++) {
-    const int rq = wave + p * total_waves;
+    const int rq = first + slot_off(p);
     request(rq < nrq ? rq : own, wt[p], st[p], epi_t[p]);
   }
 
@@ -496,7 +502,7 @@ __device__ __forceinline__ void gemv_ring(const GemvArgs &a, float *xs_lds, floa
   }
 #pragma unroll
   for (int p = PRE; p < PD; p++) {
-    const int rq = wave + p * total_waves;
+    const int rq = first + slot_off(p);
     request(rq < nrq ? rq : own, wt[p], st[p], epi_t[p]);
   }
   if (folded && !coop) {
@@ -553,6 +559,7 @@ __device__ __forceinline__ void gemv_ring(const GemvArgs &a, float *xs_lds, floa
   // ---- (4) stream the rows: slot p of the ring holds tile base + p * total_waves ----
   float best_v = -INFINITY;
   int best_i = 0x7fffffff;
+  float held_gate = 0.0f;
   auto consume = [&](int p, int rq) {
     float acc = 0.0f;
 #pragma unroll
@@ -567,7 +574,14 @@ __device__ __forceinline__ void gemv_ring(const GemvArgs &a, float *xs_lds, floa
     const float fs = (EPI && a.fold_s) ? dpp_f<0x102>(epi_t[p]) : 0.0f;       // row_shl:2
     if (folded) acc = rstd * (acc - mu * fs);
     const int row = rq * RPW + g;
-    if (RPW >= 2 && a.pair_swiglu) {
+    if (RPW == 1 && PD >= 2 && a.pair_swiglu) {
+      // SwiGLU across the (gate, up) row pair held by two neighbouring ring slots of this wavefront
+      if (p & 1) {
+        if (l == 0 && row < a.rows) a.y[(int64_t)m * a.y_stride + (row >> 1)] = ct_silu(held_gate) * (acc + bias);
+      } else {
+        held_gate = acc + bias;
+      }
+    } else if (RPW >= 2 && a.pair_swiglu) {
       // SwiGLU across the (gate, up) row pair held by neighbouring lane groups
       const float mine = acc + bias;
       const float other = __shfl_xor(mine, G & 63, 64);
@@ -578,11 +592,11 @@ __device__ __forceinline__ void gemv_ring(const GemvArgs &a, float *xs_lds, floa
     }
   };
   const int stride = PD * total_waves;
-  int base = wave;
+  int base = first;
   for (; base + stride < nrq; base += stride) {  // every slot holds a tile; slot 0 has a successor
 #pragma unroll
     for (int p = 0; p < PD; p++) {
-      const int rq = base + p * total_waves;
+      const int rq = base + slot_off(p);
       consume(p, rq);
       const int nxt = rq + stride;
       request(nxt < nrq ? nxt : rq, wt[p], st[p], epi_t[p]);
@@ -590,7 +604,7 @@ __device__ __forceinline__ void gemv_ring(const GemvArgs &a, float *xs_lds, floa
   }
 #pragma unroll
   for (int p = 0; p < PD; p++) {
-    const int rq = base + p * total_waves;
+    const int rq = base + slot_off(p);
     if (rq < nrq) consume(p, rq);  // wavefront-uniform
   }
   if (a.am_val) gemv_argmax_tail(a, wave, lane, best_v, best_i);

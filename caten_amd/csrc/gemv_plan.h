@@ -24,6 +24,8 @@ namespace cthip {
 // lane in registers) keep two tiles, which leaves room for a second wavefront per SIMD
 #define PD_OF_T(T, KC) (KC >= 12 ? 1 : (KC >= 6 || ((T) == CTHIP_Q4_0 && KC >= 3)) ? 2 : 4)
 
+// tiles a wavefront of the looping kernel keeps in flight
+inline int gemv_ring_depth(int type, int KC) { return PD_OF_T(type, KC); }
 struct GemvShape {
   int type, G, KC;
 };

@@ -388,7 +388,11 @@ bool gemv_pair_swiglu_ok(int type, int64_t rows, int64_t cols) {
     const GemvWidePlan p = gemv_wide_plan(type, rows, cols, s.compute_units);
     if (p.ok) return p.rw == 2;
   }
-  return v && v->G <= 32;
+  if (!v) return false;
+  if (v->G <= 32) return true;  // two rows and more per wavefront: the pair sits in neighbouring lane groups
+  // one row per wavefront: the pair sits in neighbouring slots of the ring, which a looping launch with an even ring
+  // has (enough rows for every wavefront to loop at any occupancy)
+  return (gemv_ring_depth(type, v->KC) & 1) == 0 && rows >= 32ll * s.compute_units;
 }
 int gemv_rows_per_wave(int type, int64_t cols) {
   const GemvVariant *v = cols <= 0x7fffffff ? pick_variant(type, (int)cols) : nullptr;
@@ -440,6 +444,9 @@ static int launch_variant(const GemvVariant *v, const WMat *w, GemvArgs a, int m
       p = gemv_plan(in);
     }
     if (p.error) return fail(CTHIP_E_UNSUPPORTED, "gemv: (%d, %d): %s", a.rows, a.cols, p.error);
+    // the paired SwiGLU epilogue with one row per wavefront: the pair sits in two neighbouring slots of the ring
+    if (a.pair_swiglu && v->G > 32 && (p.kernel == GEMV_K_SMALL || (gemv_ring_depth(w->type, v->KC) & 1)))
+      return fail(CTHIP_E_UNSUPPORTED, "gemv: the paired SwiGLU epilogue over (%d, %d) needs a looping launch with an even ring", a.rows, a.cols);
     a.stage_x = p.stage ? 1 : 0;
     if (p.unfold) {
       a.fold_s = nullptr;
@@ -475,8 +482,8 @@ int launch_gemv(const WMat *w, GemvArgs a, int m) {
   if (a.am_val && m != 1) return fail(CTHIP_E_BAD_ARG, "gemv: the fused argmax needs m == 1");
   const GemvVariant *v = pick_variant(w->type, a.cols);
   if (gemv_prefers_wide(v, w->type, a.rows) && gemv_wide_supported(w, a)) return launch_gemv_wide(w, a, m);
-  if (a.pair_swiglu && (!v || v->G > 32 || (a.rows & 1) || a.am_val || a.residual || a.split1 != a.rows))
-    return fail(CTHIP_E_UNSUPPORTED, "gemv: the paired SwiGLU epilogue needs two rows per wavefront and plain outputs");
+  if (a.pair_swiglu && (!v || (a.rows & 1) || a.am_val || a.residual || a.split1 != a.rows))
+    return fail(CTHIP_E_UNSUPPORTED, "gemv: the paired SwiGLU epilogue needs a register-resident launch and plain outputs");
   if (v) return launch_variant(v, w, a, m);
   // wider than any variant: column slices, when nothing in the launch needs the whole row at once (a norm of the
   // input, an activation of the sum, an argmax) and the output is one plain vector per input row

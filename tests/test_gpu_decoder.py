@@ -164,12 +164,14 @@ def test_three_launch_layer_equals_five_launch_layer(name, plen, kind):
         assert np.array_equal(a, c)
 
 
-@pytest.mark.parametrize("kind", ["q4_0", "q8_0", "f16"])
-def test_llama_swiglu_in_the_epilogue_of_the_wide_row_gate_up_launch(oracle, kind):
-    """A model whose gate|up launch runs on the wide-row kernel with a (gate, up) row pair per wavefront (8192 rows
-    of gate and up in turn; option gemv_wide 2 sends every launch it supports there) applies SwiGLU in that launch's
-    epilogue, and the down projection stages one vector instead of two.  Same tokens as the CPU decoder and as the
-    session whose launches take the register-resident kernels; logits inside the fp32 band of both."""
+@pytest.mark.parametrize("kind", ["q4_0", "q8_0", "f16", "f32"])
+def test_llama_swiglu_in_the_epilogue_of_the_gate_up_launch(oracle, kind):
+    """A model whose gate|up launch holds (gate, up) row pairs applies SwiGLU in that launch's epilogue, and the down
+    projection stages one vector instead of two.  8192 rows of gate and up in turn: on the wide-row kernel (option
+    gemv_wide 2 sends every launch it supports there) a wavefront streams the two rows together; on the
+    register-resident kernels the pair sits in neighbouring lane groups (Q8_0 / Q4_0 at this width) or, with one row
+    per wavefront (fp16 / fp32 at this width), in neighbouring slots of the wavefront's ring.  Same tokens as the
+    CPU decoder either way; logits inside the fp32 band of it and of each other."""
     print(f"case: SwiGLU in the epilogue of the wide-row gate|up launch, {kind}", flush=True)
     from caten_amd import _lib, synth, llm
     lib = _lib.load()

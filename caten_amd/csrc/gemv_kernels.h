@@ -272,7 +272,7 @@ __device__ __forceinline__ uint4 load_chunk(const uint4 *src) {
 // PD - 1 tiles requested after it; (ii) the input side (vector, gamma or the gate's partner) is
 // requested BEFORE the weight ring: loads return in order, so a vector requested behind four tiles
 // would hold back the first product until all four had arrived.
-template <int TYPE, int G, int KC, int PD, bool NT, bool EPI, bool DIRECT>
+template <int TYPE, int G, int KC, int PD, bool NT, bool EPI, bool DIRECT, bool PAIR1>
 __device__ __forceinline__ void gemv_ring(const GemvArgs &a, float *xs_lds, float *red) {
   constexpr int XPC = Fmt<TYPE>::XPC;
   constexpr int RPW = 64 / G;
@@ -383,7 +383,9 @@ __device__ __forceinline__ void gemv_ring(const GemvArgs &a, float *xs_lds, floa
   // Which tile ring slot p holds first.  Plain: wave + p * total_waves.  With one row per wavefront and the paired
   // SwiGLU epilogue a wavefront takes (gate, up) row pairs: slots 2k and 2k + 1 hold rows 2 (wave + k * total_waves)
   // and the one after it; a slot's next tile is PD * total_waves further on either way.
-  const bool pair1 = RPW == 1 && PD >= 2 && a.pair_swiglu;
+  // (PAIR1 is its own instantiation: the others keep the plain order as constants)
+  constexpr bool pair1 = PAIR1;
+  static_assert(!PAIR1 || (RPW == 1 && PD >= 2 && PD % 2 == 0 && !EPI && !DIRECT), "row pairs in ring slots: one row per wavefront, an even ring");
   const int first = pair1 ? 2 * wave : wave;
   auto slot_off = [&](int p) { return pair1 ? (p >> 1) * 2 * total_waves + (p & 1) : p * total_waves; };
   const int own = first < nrq ? first : nrq - 1;  // what a slot without a tile requests: lines this wavefront fetches anyway
@@ -574,7 +576,7 @@ __device__ __forceinline__ void gemv_ring(const GemvArgs &a, float *xs_lds, floa
     const float fs = (EPI && a.fold_s) ? dpp_f<0x102>(epi_t[p]) : 0.0f;       // row_shl:2
     if (folded) acc = rstd * (acc - mu * fs);
     const int row = rq * RPW + g;
-    if (RPW == 1 && PD >= 2 && a.pair_swiglu) {
+    if (PAIR1) {
       // SwiGLU across the (gate, up) row pair held by two neighbouring ring slots of this wavefront
       if (p & 1) {
         if (l == 0 && row < a.rows) a.y[(int64_t)m * a.y_stride + (row >> 1)] = ct_silu(held_gate) * (acc + bias);
@@ -615,7 +617,7 @@ __device__ __forceinline__ void gemv_ring(const GemvArgs &a, float *xs_lds, floa
 // NT: the weights are requested with the non-temporal hint.  A model whose weights exceed the 256 MB Infinity
 // Cache streams all of them from HBM every step whatever the hint; without it the stream also evicts the
 // vectors, fold terms and KV rows that the step does reuse.
-template <int TYPE, int G, int KC, int PD, bool NT, bool EPI = false, bool DIRECT = false>
+template <int TYPE, int G, int KC, int PD, bool NT, bool EPI = false, bool DIRECT = false, bool PAIR1 = false>
 __global__ __launch_bounds__(256) void k_gemv(GemvArgs a) {
   constexpr int XPC = Fmt<TYPE>::XPC;
   constexpr int RPW = 64 / G;  // rows per wavefront per iteration
@@ -666,7 +668,7 @@ __global__ __launch_bounds__(256) void k_gemv(GemvArgs a) {
   };
 
   if constexpr (PD > 1) {
-    gemv_ring<TYPE, G, KC, PD, NT, EPI, DIRECT>(a, xs_lds, red);
+    gemv_ring<TYPE, G, KC, PD, NT, EPI, DIRECT, PAIR1>(a, xs_lds, red);
     return;
   }
   // Everything this wavefront needs from memory is requested before any arithmetic so the
@@ -793,12 +795,19 @@ struct GemvVariant {
   gemv_fn fn_epi[2];   // the same with per-row epilogue operands (bias, residual, fold term) travelling in the ring
   gemv_fn fn_direct[2];  // looping, no epilogue operands, a LayerNorm applied to the staged input
   gemv_fn fn_small[2]; // one tile per wavefront: latency-bound launches
+  gemv_fn fn_pair[2];  // looping, one row per wavefront, (gate, up) row pairs in neighbouring ring slots with SwiGLU as the epilogue; null where the shape has none
 };
+template <int T, int G, int KC, bool NT>
+constexpr gemv_fn gemv_pair_fn() {
+  if constexpr (G == 64 && PD_OF_T(T, KC) >= 2 && PD_OF_T(T, KC) % 2 == 0) return k_gemv<T, G, KC, PD_OF_T(T, KC), NT, false, false, true>;
+  else return nullptr;
+}
 #define V(T, G, KC)                                                                           \
   {T, G, KC, {k_gemv<T, G, KC, PD_OF_T(T, KC), false>, k_gemv<T, G, KC, PD_OF_T(T, KC), true>},         \
    {k_gemv<T, G, KC, PD_OF_T(T, KC), false, PD_OF_T(T, KC) != 1>, k_gemv<T, G, KC, PD_OF_T(T, KC), true, PD_OF_T(T, KC) != 1>}, \
    {k_gemv<T, G, KC, PD_OF_T(T, KC), false, false, PD_OF_T(T, KC) != 1>, k_gemv<T, G, KC, PD_OF_T(T, KC), true, false, PD_OF_T(T, KC) != 1>}, \
-   {k_gemv<T, G, KC, 1, false>, k_gemv<T, G, KC, 1, true>}},
+   {k_gemv<T, G, KC, 1, false>, k_gemv<T, G, KC, 1, true>},                                              \
+   {gemv_pair_fn<T, G, KC, false>(), gemv_pair_fn<T, G, KC, true>()}},
 // defined in gemv_q8.hip, gemv_q4.hip, gemv_f32.hip, gemv_f16.hip
 extern const GemvVariant kGemvQ8[], kGemvQ4[], kGemvF32[], kGemvF16[];
 extern const int kGemvQ8Count, kGemvQ4Count, kGemvF32Count, kGemvF16Count;

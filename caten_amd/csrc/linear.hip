@@ -445,8 +445,9 @@ static int launch_variant(const GemvVariant *v, const WMat *w, GemvArgs a, int m
     }
     if (p.error) return fail(CTHIP_E_UNSUPPORTED, "gemv: (%d, %d): %s", a.rows, a.cols, p.error);
     // the paired SwiGLU epilogue with one row per wavefront: the pair sits in two neighbouring slots of the ring
-    if (a.pair_swiglu && v->G > 32 && (p.kernel == GEMV_K_SMALL || (gemv_ring_depth(w->type, v->KC) & 1)))
-      return fail(CTHIP_E_UNSUPPORTED, "gemv: the paired SwiGLU epilogue over (%d, %d) needs a looping launch with an even ring", a.rows, a.cols);
+    const bool pair1 = a.pair_swiglu && v->G > 32;
+    if (pair1 && (p.kernel != GEMV_K_LOOP || !v->fn_pair[0]))
+      return fail(CTHIP_E_UNSUPPORTED, "gemv: the paired SwiGLU epilogue over (%d, %d) needs a looping launch with an even ring and no per-row operands", a.rows, a.cols);
     a.stage_x = p.stage ? 1 : 0;
     if (p.unfold) {
       a.fold_s = nullptr;
@@ -458,7 +459,7 @@ static int launch_variant(const GemvVariant *v, const WMat *w, GemvArgs a, int m
     // the looping kernel with per-row operands in its ring dereferences one of them unconditionally
     if (p.kernel == GEMV_K_LOOP_EPI && !a.bias && !a.residual && !a.fold_s)
       return fail(CTHIP_E_STATE, "gemv: a launch with epilogue operands in its ring has none");
-    const gemv_fn fn = p.kernel == GEMV_K_SMALL ? v->fn_small[nt] : p.kernel == GEMV_K_LOOP_EPI ? v->fn_epi[nt]
+    const gemv_fn fn = pair1 ? v->fn_pair[nt] : p.kernel == GEMV_K_SMALL ? v->fn_small[nt] : p.kernel == GEMV_K_LOOP_EPI ? v->fn_epi[nt]
                      : p.kernel == GEMV_K_LOOP_DIRECT ? v->fn_direct[nt] : v->fn[nt];
     hipLaunchKernelGGL(fn, dim3(p.grid_x, p.grid_y), dim3(p.block), p.lds, s.stream, a);
     CTHIP_LAUNCH_CHECK();
